@@ -1,0 +1,70 @@
+"""Build libhk355.so (the C-ABI library) from hipkittens_amd/csrc/*.hip with hipcc for gfx950.
+
+Each .hip file is compiled to an object in parallel and the objects are linked
+into one shared library that sits next to this file, so that it travels with the
+source tree.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC = PKG_DIR / "csrc"
+BUILD_DIR = PKG_DIR / "csrc" / "build"
+LIB_PATH = PKG_DIR / "libhk355.so"
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++20",
+    "-fPIC",
+    "-Wno-unused-command-line-argument",
+    "-Wno-inline-asm",
+    # packed-fp32 VALU forms are kept out of all device code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; cannot build libhk355.so")
+    return exe
+
+
+def _compile_one(src: Path, extra: list[str]) -> Path:
+    obj = BUILD_DIR / (src.stem + ".o")
+    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", str(src), "-o", str(obj)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src.name}:\n{res.stdout}\n{res.stderr}")
+    return obj
+
+
+def build(verbose: bool = True, extra_flags: list[str] | None = None, jobs: int = 8) -> Path:
+    """Compile every csrc/*.hip and link libhk355.so. Always recompiles."""
+    extra = list(extra_flags or [])
+    BUILD_DIR.mkdir(parents=True, exist_ok=True)
+    sources = sorted(CSRC.glob("*.hip"))
+    if not sources:
+        raise RuntimeError(f"no .hip sources under {CSRC}")
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(lambda s: _compile_one(s, extra), sources))
+    tmp = LIB_PATH.with_suffix(".so.tmp")
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
+    os.replace(tmp, LIB_PATH)
+    if verbose:
+        print(f"built {LIB_PATH} from {len(sources)} sources", file=sys.stderr)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()

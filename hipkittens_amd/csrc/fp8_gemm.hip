@@ -1,0 +1,276 @@
+// FP8 e4m3 GEMM for gfx950: C[M,N] = bf16(alpha * A[M,K] * B[N,K]^T), fp32 accumulate.
+//
+// Replaces the reference's kernels/gemm/fp8fp32 executables (4-wave / 8-wave
+// schedules, kernels/gemm/fp8fp32/README.md:3-21); helper layer studied:
+// kernels/gemm/fp8fp32/FP8_4wave/utils.cpp:23-174.
+//
+// Tile kernel: one workgroup owns a 256x256 tile of C and walks K in steps of 128.
+// A and B tiles (256 rows x 128 bytes each) are fetched with direct global->LDS
+// loads into a two-stage ring of swizzled LDS tiles; each wave reads its operand
+// fragments with ds_read_b128 and issues v_mfma_f32_16x16x128_f8f6f4.
+// The MFMA is issued with the operand roles swapped (B rows as the "A" operand) so
+// that a lane's 4 accumulator values are 4 consecutive columns of one C row, and
+// the B tile's rows are permuted on their way into LDS so that two neighbouring
+// MFMA tiles give a lane 8 consecutive columns = one 16-byte bf16 store.
+#include "hk_device.h"
+#include "../../include/hk355.h"
+
+namespace hk {
+
+constexpr int BM = 256, BN = 256, BK = 128;
+constexpr int kTileBytes = BM * BK;           // one operand tile in LDS (32 KiB)
+constexpr int kStageBytes = 2 * kTileBytes;   // A tile + B tile
+constexpr int kLdsBytes = 2 * kStageBytes;    // two stages (128 KiB)
+
+// Position of LDS row R of the B tile inside the tile's 256 columns of C:
+// within each group of 32 rows, row 16*t + r (t = MFMA tile parity, r = operand
+// row) holds column 8*(r/4) + 4*t + r%4.
+__device__ __forceinline__ int b_row_to_col(int R) {
+    const int r = R & 15, t = (R >> 4) & 1;
+    return (R & ~31) | ((r >> 2) << 3) | (t << 2) | (r & 3);
+}
+
+template <int WM, int WN, bool EDGE>
+__global__ __launch_bounds__(WM * WN * 64) void fp8_gemm_tile_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n) {
+    constexpr int NW = WM * WN;
+    constexpr int TM = BM / WM, TN = BN / WN;  // per-wave tile of C
+    constexpr int MT = TM / 16, NT = TN / 16;  // MFMA tiles per wave
+    constexpr int NDMA = kTileBytes / (NW * 1024);  // loads per wave per operand per K-step
+    static_assert(NT % 2 == 0, "column pairs");
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+
+    const int lane = lane_id();
+    const int w = wave_id();
+    const int wm = w / WN, wn = w % WN;
+
+    int pm, pn;
+    {
+        const int num_wg = tiles_m * tiles_n;
+        const int id = xcd_chunk_order(blockIdx.x, num_wg, kCuPerXcd);
+        grouped_raster(id, tiles_m, tiles_n, 8, pm, pn);
+    }
+    const int row0 = pm * BM, col0 = pn * BN;
+
+    // ---- global -> LDS addressing -------------------------------------------------
+    const uint8_t* a_base = A + (size_t)row0 * K;
+    const uint8_t* b_base = B + (size_t)col0 * K;
+    const int a_rows = min(M - row0, BM), b_rows = min(N - col0, BN);
+    const v4i srd_a = make_srd(a_base, (uint32_t)a_rows * (uint32_t)K);
+    const v4i srd_b = make_srd(b_base, (uint32_t)b_rows * (uint32_t)K);
+
+    // Load i of this wave fills LDS rows 8*(i*NW + w) .. +8 of the tile; lane l lands
+    // in row +l/8, physical chunk l%8, and therefore fetches logical chunk
+    // swz(row, l%8) (the swizzle is an involution).
+    uint32_t voff_a[EDGE ? NDMA : 1], voff_b[EDGE ? NDMA : 1];
+    {
+#pragma unroll
+        for (int i = 0; i < (EDGE ? NDMA : 1); ++i) {
+            const int R = 8 * (i * NW + w) + (lane >> 3);
+            const uint32_t c = swz_chunk(R, lane & 7);
+            int ra = R, rb = b_row_to_col(R);
+            if (EDGE) {
+                ra = min(ra, a_rows - 1);
+                rb = min(rb, b_rows - 1);
+            }
+            voff_a[i] = (uint32_t)ra * (uint32_t)K + c * 16u;
+            voff_b[i] = (uint32_t)rb * (uint32_t)K + c * 16u;
+        }
+    }
+    const uint32_t dma_row_stride = to_sgpr((uint32_t)(8 * NW) * (uint32_t)K);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+    const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
+
+    auto issue_tile = [&](int stage, int kt) {
+        const uint32_t k0 = (uint32_t)kt * BK;
+        const uint32_t dst = lds_wave + (uint32_t)stage * kStageBytes;
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) {
+            if (EDGE)
+                dma16(srd_a, dst + i * NW * 1024, voff_a[i], k0);
+            else
+                dma16(srd_a, dst + i * NW * 1024, voff_a[0], k0 + i * dma_row_stride);
+        }
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) {
+            if (EDGE)
+                dma16(srd_b, dst + kTileBytes + i * NW * 1024, voff_b[i], k0);
+            else
+                dma16(srd_b, dst + kTileBytes + i * NW * 1024, voff_b[0], k0 + i * dma_row_stride);
+        }
+    };
+
+    // ---- LDS -> register addressing -----------------------------------------------
+    const uint32_t r = lane & 15, g = lane >> 4;
+    const uint32_t rd_lo = r * 128u + swz_chunk(r, g) * 16u;
+    const uint32_t rd_hi = r * 128u + swz_chunk(r, g + 4) * 16u;
+    uint32_t a_lo = lds0 + wm * (TM * BK) + rd_lo, a_hi = lds0 + wm * (TM * BK) + rd_hi;
+    uint32_t b_lo = lds0 + kTileBytes + wn * (TN * BK) + rd_lo;
+    uint32_t b_hi = lds0 + kTileBytes + wn * (TN * BK) + rd_hi;
+
+    v4f acc[MT][NT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    const int nk = K / BK;
+    issue_tile(0, 0);
+    for (int kt = 0; kt < nk; ++kt) {
+        wait_vmcnt<0>();
+        block_barrier();
+        if (kt + 1 < nk) issue_tile((kt + 1) & 1, kt + 1);
+
+        v8i bf[NT];
+#pragma unroll
+        for (int n = 0; n < NT; ++n) bf[n] = lds_frag(b_lo, b_hi, n * 16 * BK);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const v8i af = lds_frag(a_lo, a_hi, m * 16 * BK);
+#pragma unroll
+            for (int n = 0; n < NT; ++n) acc[m][n] = mfma_fp8_16x16x128(bf[n], af, acc[m][n]);
+        }
+        a_lo ^= kStageBytes; a_hi ^= kStageBytes;
+        b_lo ^= kStageBytes; b_hi ^= kStageBytes;
+    }
+
+    // ---- epilogue: alpha, bf16 (RNE), 16-byte stores --------------------------------
+    // acc[m][2p], acc[m][2p+1] hold, for C row row0 + wm*TM + 16m + lane%16, the 8
+    // columns col0 + wn*TN + 32p + 8*(lane/16) .. +8.
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int row = row0 + wm * TM + 16 * m + (int)r;
+#pragma unroll
+        for (int p = 0; p < NT / 2; ++p) {
+            const int col = col0 + wn * TN + 32 * p + 8 * (int)g;
+            const v4f x = acc[m][2 * p] * alpha, y = acc[m][2 * p + 1] * alpha;
+            if (!EDGE) {
+                v4i out;
+                out.x = pack_bf16(x.x, x.y); out.y = pack_bf16(x.z, x.w);
+                out.z = pack_bf16(y.x, y.y); out.w = pack_bf16(y.z, y.w);
+                *(v4i*)(C + (size_t)row * N + col) = out;
+            } else if (row < M) {
+                const float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
+                if (col + 8 <= N && (N & 7) == 0) {
+                    v4i out;
+                    out.x = pack_bf16(v[0], v[1]); out.y = pack_bf16(v[2], v[3]);
+                    out.z = pack_bf16(v[4], v[5]); out.w = pack_bf16(v[6], v[7]);
+                    *(v4i*)(C + (size_t)row * N + col) = out;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (col + j < N)
+                            C[(size_t)row * N + col + j] = (uint16_t)(pack_bf16(v[j], 0.f) & 0xffffu);
+                }
+            }
+        }
+    }
+}
+
+// Portable kernel for any M, N and K % 16 == 0: 4 waves, each a 32x32 patch of a 64x64
+// tile, operands fetched straight from global memory into MFMA fragments with
+// per-lane masking (rows past the edge and 16-byte chunks past K read as zero).
+__global__ __launch_bounds__(256) void fp8_gemm_portable_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, float alpha) {
+    const int lane = lane_id(), w = wave_id();
+    const int r = lane & 15, g = lane >> 4;
+    const int row0 = blockIdx.y * 64 + (w >> 1) * 32;
+    const int col0 = blockIdx.x * 64 + (w & 1) * 32;
+    v4f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    auto frag = [&](const uint8_t* base, int row, int rows, int k0) {
+        v4i lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+        if (row < rows) {
+            const uint8_t* p = base + (size_t)row * K + k0 + 32 * g;
+            if (k0 + 32 * g < K) lo = *(const v4i*)p;
+            if (k0 + 32 * g + 16 < K) hi = *(const v4i*)(p + 16);
+        }
+        return (v8i)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+
+    for (int k0 = 0; k0 < K; k0 += 128) {
+        v8i af[2], bf[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            af[i] = frag(A, row0 + 16 * i + r, M, k0);
+            bf[i] = frag(B, col0 + 16 * i + r, N, k0);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) acc[i][j] = mfma_fp8_16x16x128(bf[j], af[i], acc[i][j]);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int row = row0 + 16 * i + r;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const v4f x = acc[i][j] * alpha;
+            const float v[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int col = col0 + 16 * j + 4 * g + e;
+                if (row < M && col < N)
+                    C[(size_t)row * N + col] = (uint16_t)(pack_bf16(v[e], 0.f) & 0xffffu);
+            }
+        }
+    }
+}
+
+template <int WM, int WN, bool EDGE>
+static int launch_tile(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
+                       hipStream_t stream) {
+    auto kern = fp8_gemm_tile_kernel<WM, WN, EDGE>;
+    static bool configured = false;  // attribute is per function; set once per process
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kLdsBytes) != hipSuccess)
+            return HK_ERR_LAUNCH;
+        configured = true;
+    }
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(WM * WN * 64), kLdsBytes, stream,
+                       (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
+                       tiles_n);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
+}  // namespace hk
+
+extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M, int N, int K,
+                                   float scale_a, float scale_b, int variant, void* stream) {
+    using namespace hk;
+    if (!A || !B || !C) return HK_ERR_NULL_POINTER;
+    if (M <= 0 || N <= 0 || K <= 0 || (K % 16) != 0) return HK_ERR_BAD_SHAPE;
+    if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    if (variant < 0 || variant > 2) return HK_ERR_UNSUPPORTED;
+    if (variant != 0 && ((K % BK) != 0 || (long long)K * BM >= (1ll << 31))) return HK_ERR_BAD_SHAPE;
+    const float alpha = scale_a * scale_b;
+    hipStream_t s = (hipStream_t)stream;
+    if (variant == 0) {
+        if ((long long)((M + 63) / 64) > 65535) return HK_ERR_BAD_SHAPE;
+        dim3 grid((N + 63) / 64, (M + 63) / 64);
+        hipLaunchKernelGGL(fp8_gemm_portable_kernel, grid, dim3(256), 0, s, (const uint8_t*)A,
+                           (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha);
+        return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+    }
+    const bool edge = (M % BM) != 0 || (N % BN) != 0;
+    if (variant == 1)
+        return edge ? launch_tile<2, 4, true>(A, B, C, M, N, K, alpha, s)
+                    : launch_tile<2, 4, false>(A, B, C, M, N, K, alpha, s);
+    return edge ? launch_tile<2, 2, true>(A, B, C, M, N, K, alpha, s)
+                : launch_tile<2, 2, false>(A, B, C, M, N, K, alpha, s);
+}
+
+extern "C" int hk_fp8_gemm(const void* A, const void* B, void* C, int M, int N, int K,
+                           float scale_a, float scale_b, void* stream) {
+    const bool tile_ok = K > 0 && (K % hk::BK) == 0 && (long long)K * hk::BM < (1ll << 31) &&
+                         M >= 64 && N >= 64;
+    return hk_fp8_gemm_variant(A, B, C, M, N, K, scale_a, scale_b, tile_ok ? 2 : 0, stream);
+}

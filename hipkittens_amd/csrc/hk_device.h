@@ -1,0 +1,122 @@
+// Device-side building blocks shared by the gfx950 kernels: buffer descriptors,
+// direct global->LDS loads, the LDS tile swizzle, MFMA wrappers, bf16 packing and
+// the XCD-aware workgroup order.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hk {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) const v4i lds_v4i_t;
+
+constexpr int kWave = 64;
+constexpr int kNumXcd = 8;
+constexpr int kCuPerXcd = 32;
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+// Wave index as a scalar (SGPR) value.
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
+__device__ __forceinline__ uint32_t to_sgpr(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
+
+// Raw (unstrided, unswizzled) buffer descriptor over [base, base+bytes).
+// Plays the role of make_srsrc in the reference
+// (include/ops/warp/memory/util/util.cuh:72-88).
+__device__ __forceinline__ v4i make_srd(const void* base, uint32_t bytes) {
+    uint64_t p = (uint64_t)base;
+    v4i s;
+    s.x = to_sgpr((uint32_t)p);
+    s.y = to_sgpr((uint32_t)(p >> 32) & 0xffffu);
+    s.z = to_sgpr(bytes);
+    s.w = 0x00020000;
+    return s;
+}
+
+// One `buffer_load_dwordx4 ... lds`: every lane fetches 16 bytes from
+// srd.base + voff + soff and the wave's 1024 bytes land contiguously in LDS at
+// lds_base + 16*lane. lds_base and soff must be wave-uniform.
+// Written as inline asm so that the compiler's LDS-DMA alias tracking does not
+// force vmcnt(0) in front of every later LDS read; completion is awaited
+// explicitly with wait_vmcnt<N>().
+__device__ __forceinline__ void dma16(v4i srd, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dwordx4 %1, %2, %3 offen lds"
+        :
+        : "s"(lds_base), "v"(voff), "s"(srd), "s"(soff)
+        : "memory", "m0");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ void block_barrier() { __builtin_amdgcn_s_barrier(); }
+
+// LDS tile layout for K-contiguous operand tiles with 128-byte rows: the 16-byte
+// chunk index is XORed with bits [1..3] of the row. With lane l of an MFMA
+// operand read touching row l%16 and chunk l/16 this is free of bank conflicts
+// for ds_read_b128 (formula as in kernels/gemm/fp8fp32/FP8_4wave/utils.cpp:123-128).
+__device__ __forceinline__ uint32_t swz_chunk(uint32_t row, uint32_t chunk) {
+    return chunk ^ ((row >> 1) & 7u);
+}
+
+// 16x128 (fp8) / 16x256 (fp4) MFMA operand fragment: lane l holds row l%16 and the
+// two 16-byte chunks l/16 and 4 + l/16 of the 128-byte row. The K order this
+// induces is the same for both operands, so the contraction is unchanged, and each
+// 16-byte half is one whole 32-element block when the row holds fp4.
+__device__ __forceinline__ v8i lds_frag(uint32_t addr_lo, uint32_t addr_hi, int imm) {
+    v4i lo = *(lds_v4i_t*)(uintptr_t)(addr_lo + imm);
+    v4i hi = *(lds_v4i_t*)(uintptr_t)(addr_hi + imm);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// D(16x16, fp32) += A(16x128, e4m3) * B(16x128, e4m3)^T. Lane l supplies row l%16,
+// K-block l/16 of each operand and receives D[4*(l/16)+j][l%16] in element j.
+// Same instruction as the reference's mfma1616128
+// (include/ops/warp/register/tile/mma.cuh:112-125).
+__device__ __forceinline__ v4f mfma_fp8_16x16x128(v8i a, v8i b, v4f c) {
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+// Two fp32 -> packed bf16 (round to nearest even); `lo` goes to bits [15:0].
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    v2f f = {lo, hi};
+    v2bf h = __builtin_convertvector(f, v2bf);
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+// Workgroup order. Hardware hands consecutive workgroup ids to the 8 XCDs round
+// robin. `xcd_chunk_order` regroups ids so that each XCD (own L2) owns runs of
+// `chunk` consecutive logical ids (cf. chiplet_transform_chunked,
+// include/common/util.cuh:78-101); `grouped_raster` then walks the tile grid in
+// column-major groups of `group_m` tile rows so that a run of `chunk` ids is a
+// compact 2-D patch of C sharing A/B panels in that L2.
+__device__ __forceinline__ int xcd_chunk_order(int wg, int num_wg, int chunk) {
+    const int span = kNumXcd * chunk;
+    const int full = (num_wg / span) * span;
+    if (wg >= full) return wg;
+    const int xcd = wg % kNumXcd;
+    const int local = wg / kNumXcd;
+    return (local / chunk) * span + xcd * chunk + (local % chunk);
+}
+
+__device__ __forceinline__ void grouped_raster(int id, int tiles_m, int tiles_n, int group_m,
+                                               int& pm, int& pn) {
+    const int per_group = group_m * tiles_n;
+    const int group = id / per_group;
+    const int first_m = group * group_m;
+    const int gsize = min(tiles_m - first_m, group_m);
+    const int in_group = id - group * per_group;
+    pm = first_m + in_group % gsize;
+    pn = in_group / gsize;
+}
+
+}  // namespace hk

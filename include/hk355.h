@@ -1,0 +1,64 @@
+/*
+ * hk355 — C ABI of the MI355X (gfx950) quantized-contraction library.
+ *
+ * Every entry point:
+ *   - takes plain device pointers owned by the caller (inputs and outputs are
+ *     caller-allocated, as in the reference's pybind11 boundary, which only
+ *     reads data_ptr()/shape: include/pyutils/pyutils.cuh:14-47, :66-71);
+ *   - is asynchronous on `stream` (a hipStream_t passed as void*; NULL = the
+ *     null stream, which is what the reference's bindings launch on:
+ *     kernels/gemm/bf16fp32/mi325x/256_256_64_16.cpp:24-32, :227-231);
+ *   - returns HK_OK or a negative hk_status; it never aborts and never throws.
+ *     Argument errors are detected on the host before anything is launched.
+ */
+#ifndef HK355_H
+#define HK355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum hk_status {
+    HK_OK = 0,
+    HK_ERR_NULL_POINTER = -1, /* a required pointer is NULL                      */
+    HK_ERR_BAD_SHAPE = -2,    /* a dimension is <= 0 or violates a divisibility  */
+    HK_ERR_BAD_ALIGNMENT = -3,/* a pointer is not 16-byte aligned                */
+    HK_ERR_WORKSPACE = -4,    /* workspace missing or too small                  */
+    HK_ERR_LAUNCH = -5,       /* HIP reported an error at launch                 */
+    HK_ERR_UNSUPPORTED = -6   /* valid but not implemented for these parameters  */
+} hk_status;
+
+/* Human-readable name of a status code (static storage). */
+const char* hk_status_string(int status);
+
+/* Library version, e.g. 100 = 0.1.0 (no reference counterpart). */
+int hk_version(void);
+
+/*
+ * FP8 e4m3 (OCP e4m3fn) GEMM:  C[M,N] = bf16( (scale_a*scale_b) * sum_k A[m,k]*B[n,k] ).
+ * A is [M,K] row-major, B is [N,K] row-major ("column-major B"), both 1 byte per
+ * element; fp32 accumulation; C is [M,N] row-major bf16, rounded to nearest even.
+ * Replaces the reference's FP8 GEMM executable (kernels/gemm/fp8fp32/README.md:7-21;
+ * math = mma_ABt, include/ops/warp/register/tile/mma.cuh:382-422 with the fp8
+ * MFMA of :112-125) behind the dispatch_micro(A, B, C) convention of
+ * kernels/gemm/bf16fp32/mi350x/test_python.py:80-82. The reference applies no
+ * scale; scale_a = scale_b = 1 reproduces it.
+ * Requirements: M,N,K > 0; K % 16 == 0; A, B, C 16-byte aligned.
+ */
+int hk_fp8_gemm(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
+                int M, int N, int K, float scale_a, float scale_b, void* stream);
+
+/* Same contract, forced onto one kernel variant (for tests and tuning):
+ * 0 = portable tile kernel (any shape), 1 = 256x256x128 8-wave, 2 = 256x256x128 4-wave.
+ * Variants 1,2 need K % 128 == 0. */
+int hk_fp8_gemm_variant(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
+                        int M, int N, int K, float scale_a, float scale_b,
+                        int variant, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HK355_H */
