@@ -30,6 +30,43 @@ __device__ __forceinline__ int b_row_to_col(int R) {
     return (R & ~31) | ((r >> 2) << 3) | (t << 2) | (r & 3);
 }
 
+// Epilogue of the tile kernels: alpha, bf16 (RNE), 16-byte stores.
+// acc[m][2p], acc[m][2p+1] hold, for C row `row_base + 16m + lane%16`, the 8 columns
+// `col_base + 32p + 8*(lane/16) .. +8` (see b_row_to_col).
+template <int MT, int NT, bool EDGE>
+__device__ __forceinline__ void store_c_tile(const v4f (&acc)[MT][NT], uint16_t* __restrict__ C,
+                                             int M, int N, int row_base, int col_base, float alpha) {
+    const int r = lane_id() & 15, g = lane_id() >> 4;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int row = row_base + 16 * m + r;
+#pragma unroll
+        for (int p = 0; p < NT / 2; ++p) {
+            const int col = col_base + 32 * p + 8 * g;
+            const v4f x = acc[m][2 * p] * alpha, y = acc[m][2 * p + 1] * alpha;
+            if (!EDGE) {
+                v4i out;
+                out.x = pack_bf16(x.x, x.y); out.y = pack_bf16(x.z, x.w);
+                out.z = pack_bf16(y.x, y.y); out.w = pack_bf16(y.z, y.w);
+                *(v4i*)(C + (size_t)row * N + col) = out;
+            } else if (row < M) {
+                const float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
+                if (col + 8 <= N && (N & 7) == 0) {
+                    v4i out;
+                    out.x = pack_bf16(v[0], v[1]); out.y = pack_bf16(v[2], v[3]);
+                    out.z = pack_bf16(v[4], v[5]); out.w = pack_bf16(v[6], v[7]);
+                    *(v4i*)(C + (size_t)row * N + col) = out;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (col + j < N)
+                            C[(size_t)row * N + col + j] = (uint16_t)(pack_bf16(v[j], 0.f) & 0xffffu);
+                }
+            }
+        }
+    }
+}
+
 template <int WM, int WN, bool EDGE>
 __global__ __launch_bounds__(WM * WN * 64) void fp8_gemm_tile_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
@@ -135,37 +172,165 @@ __global__ __launch_bounds__(WM * WN * 64) void fp8_gemm_tile_kernel(
         b_lo ^= kStageBytes; b_hi ^= kStageBytes;
     }
 
-    // ---- epilogue: alpha, bf16 (RNE), 16-byte stores --------------------------------
-    // acc[m][2p], acc[m][2p+1] hold, for C row row0 + wm*TM + 16m + lane%16, the 8
-    // columns col0 + wn*TN + 32p + 8*(lane/16) .. +8.
+    store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
+}
+
+// ---------------------------------------------------------------------------------------
+// 4-wave interleaved kernel: one wave per SIMD, each owning a 128x128 patch of the 256x256
+// tile (8x8 MFMA tiles, 256 accumulator registers). Every LDS read, global->LDS load and
+// MFMA has a fixed place in the instruction stream (one MFMA per "slot", memory operations
+// attached to slots) so that operand fragments for the next MFMA group and the next K-step
+// are in flight while the matrix pipe works:
+//   groups 0..PG   : MFMAs with A fragment m; LDS read of A fragment m+3 (4 rotating buffers)
+//   after group PG : all reads of this stage are issued -> wait for the next tile's loads,
+//                    one barrier, then refill this stage with tile kt+2
+//   groups PG+1..7 : MFMAs; LDS reads of the next K-step's B fragments and first A fragments.
+// Schedule idea after the reference's 4-wave kernel (kernels/gemm/fp8fp32/README.md:3-5,
+// per-instruction helpers in FP8_4wave/utils.cpp:44-52, 131-137, 150-161).
+template <bool EDGE>
+__global__ __launch_bounds__(256) void fp8_gemm_4wave_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n) {
+    constexpr int NW = 4, TM = 128, TN = 128, MT = 8, NT = 8;
+    constexpr int NDMA = kTileBytes / (NW * 1024);  // 8 loads per wave per operand per K-step
+    constexpr int PG = 4;                            // barrier sits after MFMA group PG
+    constexpr int AD = 3;                            // A fragments are read AD groups ahead
+    static_assert(PG == 4 && AD == 3 && MT == 8, "slot plan below is written for these");
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+
+    const int lane = lane_id();
+    const int w = wave_id();
+    const int wm = w >> 1, wn = w & 1;
+
+    int pm, pn;
+    {
+        const int id = xcd_chunk_order(blockIdx.x, tiles_m * tiles_n, kCuPerXcd);
+        grouped_raster(id, tiles_m, tiles_n, 8, pm, pn);
+    }
+    const int row0 = pm * BM, col0 = pn * BN;
+
+    const int a_rows = min(M - row0, BM), b_rows = min(N - col0, BN);
+    const v4i srd_a = make_srd(A + (size_t)row0 * K, (uint32_t)a_rows * (uint32_t)K);
+    const v4i srd_b = make_srd(B + (size_t)col0 * K, (uint32_t)b_rows * (uint32_t)K);
+
+    uint32_t voff_a[EDGE ? NDMA : 1], voff_b[EDGE ? NDMA : 1];
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
-        const int row = row0 + wm * TM + 16 * m + (int)r;
+    for (int i = 0; i < (EDGE ? NDMA : 1); ++i) {
+        const int R = 8 * (i * NW + w) + (lane >> 3);
+        const uint32_t c = swz_chunk(R, lane & 7);
+        int ra = R, rb = b_row_to_col(R);
+        if (EDGE) {
+            ra = min(ra, a_rows - 1);
+            rb = min(rb, b_rows - 1);
+        }
+        voff_a[i] = (uint32_t)ra * (uint32_t)K + c * 16u;
+        voff_b[i] = (uint32_t)rb * (uint32_t)K + c * 16u;
+    }
+    const uint32_t dma_row_stride = to_sgpr((uint32_t)(8 * NW) * (uint32_t)K);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+    const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
+
+    // One global->LDS load: operand op (0 = A, 1 = B), load index i, into `stage`.
+    auto dma_one = [&](int op, int i, int stage, uint32_t k0, v4i srd) {
+        const uint32_t dst = lds_wave + (uint32_t)stage * kStageBytes + op * kTileBytes + i * NW * 1024;
+        if (EDGE)
+            dma16(srd, dst, op ? voff_b[i] : voff_a[i], k0);
+        else
+            dma16(srd, dst, op ? voff_b[0] : voff_a[0], k0 + i * dma_row_stride);
+    };
+
+    const uint32_t r = lane & 15, g = lane >> 4;
+    const uint32_t rd_lo = r * 128u + swz_chunk(r, g) * 16u;
+    const uint32_t rd_hi = r * 128u + swz_chunk(r, g + 4) * 16u;
+    uint32_t a_lo[2], a_hi[2], b_lo[2], b_hi[2];
 #pragma unroll
-        for (int p = 0; p < NT / 2; ++p) {
-            const int col = col0 + wn * TN + 32 * p + 8 * (int)g;
-            const v4f x = acc[m][2 * p] * alpha, y = acc[m][2 * p + 1] * alpha;
-            if (!EDGE) {
-                v4i out;
-                out.x = pack_bf16(x.x, x.y); out.y = pack_bf16(x.z, x.w);
-                out.z = pack_bf16(y.x, y.y); out.w = pack_bf16(y.z, y.w);
-                *(v4i*)(C + (size_t)row * N + col) = out;
-            } else if (row < M) {
-                const float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
-                if (col + 8 <= N && (N & 7) == 0) {
-                    v4i out;
-                    out.x = pack_bf16(v[0], v[1]); out.y = pack_bf16(v[2], v[3]);
-                    out.z = pack_bf16(v[4], v[5]); out.w = pack_bf16(v[6], v[7]);
-                    *(v4i*)(C + (size_t)row * N + col) = out;
+    for (int st = 0; st < 2; ++st) {
+        a_lo[st] = lds0 + st * kStageBytes + wm * (TM * BK) + rd_lo;
+        a_hi[st] = lds0 + st * kStageBytes + wm * (TM * BK) + rd_hi;
+        b_lo[st] = lds0 + st * kStageBytes + kTileBytes + wn * (TN * BK) + rd_lo;
+        b_hi[st] = lds0 + st * kStageBytes + kTileBytes + wn * (TN * BK) + rd_hi;
+    }
+
+    v4f acc[MT][NT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
+    v8i bf[2][NT];  // B fragments of the current / next K-step
+    v8i af[4];      // rotating A fragments
+
+    const int nk = K / BK;
+
+    // ---- prologue: tile 0 (and 1) in flight, first fragments in registers -----------------
+#pragma unroll
+    for (int i = 0; i < NDMA; ++i) dma_one(0, i, 0, 0, srd_a);
+#pragma unroll
+    for (int i = 0; i < NDMA; ++i) dma_one(1, i, 0, 0, srd_b);
+    wait_vmcnt<0>();
+    block_barrier();
+    if (nk > 1) {
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) dma_one(0, i, 1, BK, srd_a);
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) dma_one(1, i, 1, BK, srd_b);
+    }
+#pragma unroll
+    for (int n = 0; n < NT; ++n) bf[0][n] = lds_frag(b_lo[0], b_hi[0], n * 16 * BK);
+#pragma unroll
+    for (int m = 0; m < AD; ++m) af[m] = lds_frag(a_lo[0], a_hi[0], m * 16 * BK);
+
+    // One K-step with stage/parity P. Every step runs the same code: the last step's
+    // prefetch reads return stale LDS contents that are never used, and refills past the
+    // end of K are issued against a zero-sized buffer (out of range for every lane, no
+    // memory traffic), so that no step needs a differently scheduled body.
+    auto step = [&]<int P>(int kt) {
+        const uint32_t k2 = (uint32_t)(kt + 2) * BK;
+        v4i sa = srd_a, sb = srd_b;
+        if (kt + 2 >= nk) { sa.z = 0; sb.z = 0; }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+#pragma unroll
+            for (int n = 0; n < NT; ++n) {
+                mfma_fp8_16x16x128_acc(acc[m][n], bf[P][n], af[m & 3]);
+                if (m <= PG) {
+                    // A fragment m+AD, early in the group
+                    if (n == 0) af[(m + AD) & 3] = lds_frag(a_lo[P], a_hi[P], (m + AD) * 16 * BK);
                 } else {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j)
-                        if (col + j < N)
-                            C[(size_t)row * N + col + j] = (uint16_t)(pack_bf16(v[j], 0.f) & 0xffffu);
+                    const int j = (m - PG - 1) * NT + n;  // slot index after the barrier
+                    if (j < NT) {
+                        bf[P ^ 1][j] = lds_frag(b_lo[P ^ 1], b_hi[P ^ 1], j * 16 * BK);
+                    } else if (j == NT || j == NT + 1) {
+                        // buffers 0 and 1 were last used by groups PG and PG+1
+                        af[j - NT] = lds_frag(a_lo[P ^ 1], a_hi[P ^ 1], (j - NT) * 16 * BK);
+                    } else if (j == 2 * NT) {
+                        // buffer 2 is in use until group PG+2 has been issued
+                        af[2] = lds_frag(a_lo[P ^ 1], a_hi[P ^ 1], 2 * 16 * BK);
+                    }
+                    if (j < 2 * NDMA) dma_one(j / NDMA, j % NDMA, P, k2, j / NDMA ? sb : sa);
                 }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (m == PG) {
+                // every read of stage P by this wave has been issued; once they have returned
+                // and the next tile has landed for all waves, stage P may be refilled
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                wait_vmcnt<0>();
+                block_barrier();
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
+    };
+
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+        step.template operator()<0>(kt);
+        step.template operator()<1>(kt + 1);
     }
+    if (kt < nk) step.template operator()<0>(kt);
+    wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
+    mfma_drain();
+
+    store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
 }
 
 // Portable kernel for any M, N and K % 16 == 0: 4 waves, each a 32x32 patch of a 64x64
@@ -241,6 +406,24 @@ static int launch_tile(const void* A, const void* B, void* C, int M, int N, int 
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
+template <bool EDGE>
+static int launch_4wave(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
+                        hipStream_t stream) {
+    auto kern = fp8_gemm_4wave_kernel<EDGE>;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kLdsBytes) != hipSuccess)
+            return HK_ERR_LAUNCH;
+        configured = true;
+    }
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), kLdsBytes, stream,
+                       (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
+                       tiles_n);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
 }  // namespace hk
 
 extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M, int N, int K,
@@ -249,7 +432,7 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 16) != 0) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < 0 || variant > 2) return HK_ERR_UNSUPPORTED;
+    if (variant < 0 || variant > 3) return HK_ERR_UNSUPPORTED;
     if (variant != 0 && ((K % BK) != 0 || (long long)K * BM >= (1ll << 31))) return HK_ERR_BAD_SHAPE;
     const float alpha = scale_a * scale_b;
     hipStream_t s = (hipStream_t)stream;
@@ -264,8 +447,11 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
     if (variant == 1)
         return edge ? launch_tile<2, 4, true>(A, B, C, M, N, K, alpha, s)
                     : launch_tile<2, 4, false>(A, B, C, M, N, K, alpha, s);
-    return edge ? launch_tile<2, 2, true>(A, B, C, M, N, K, alpha, s)
-                : launch_tile<2, 2, false>(A, B, C, M, N, K, alpha, s);
+    if (variant == 3)
+        return edge ? launch_tile<2, 2, true>(A, B, C, M, N, K, alpha, s)
+                    : launch_tile<2, 2, false>(A, B, C, M, N, K, alpha, s);
+    return edge ? launch_4wave<true>(A, B, C, M, N, K, alpha, s)
+                : launch_4wave<false>(A, B, C, M, N, K, alpha, s);
 }
 
 extern "C" int hk_fp8_gemm(const void* A, const void* B, void* C, int M, int N, int K,

@@ -86,6 +86,18 @@ __device__ __forceinline__ v4f mfma_fp8_16x16x128(v8i a, v8i b, v4f c) {
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
 }
 
+// Same MFMA with the accumulator tied in place in an accumulation register (AGPR).
+// Used by the hand-scheduled kernels, where the register allocator must not move
+// accumulators between register files. The compiler does not see the instruction's
+// hazards: accumulators may be read by other instructions only after
+// mfma_drain() (the operands here come from LDS reads, which need no extra spacing).
+__device__ __forceinline__ void mfma_fp8_16x16x128_acc(v4f& acc, const v8i& a, const v8i& b) {
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+// Wait states between the last MFMA and the first read of its result by a
+// non-MFMA instruction (the longest case on this ISA is 18 cycles for a 16-pass MFMA).
+__device__ __forceinline__ void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 7" ::: "memory"); }
+
 // Two fp32 -> packed bf16 (round to nearest even); `lo` goes to bits [15:0].
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     v2f f = {lo, hi};

@@ -52,8 +52,9 @@ int hk_fp8_gemm(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
                 int M, int N, int K, float scale_a, float scale_b, void* stream);
 
 /* Same contract, forced onto one kernel variant (for tests and tuning):
- * 0 = portable tile kernel (any shape), 1 = 256x256x128 8-wave, 2 = 256x256x128 4-wave.
- * Variants 1,2 need K % 128 == 0. */
+ * 0 = portable kernel (any shape), 1 = 256x256x128 tile, 8 waves, 2 = 256x256x128 tile,
+ * 4 waves, hand-interleaved schedule, 3 = 256x256x128 tile, 4 waves, plain loop.
+ * Variants 1-3 need K % 128 == 0. */
 int hk_fp8_gemm_variant(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
                         int M, int N, int K, float scale_a, float scale_b,
                         int variant, void* stream);
