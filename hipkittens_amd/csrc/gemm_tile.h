@@ -1,0 +1,58 @@
+// Pieces shared by the 256x256 tile GEMM kernels (FP8 and MXFP4): tile geometry, the
+// column permutation of the B tile and the bf16 epilogue.
+#pragma once
+#include "hk_device.h"
+
+namespace hk {
+
+constexpr int BM = 256, BN = 256, BK = 128;
+constexpr int kTileBytes = BM * BK;           // one operand tile in LDS (32 KiB)
+constexpr int kStageBytes = 2 * kTileBytes;   // A tile + B tile
+constexpr int kLdsBytes = 2 * kStageBytes;    // two stages (128 KiB)
+
+// Position of LDS row R of the B tile inside the tile's 256 columns of C:
+// within each group of 32 rows, row 16*t + r (t = MFMA tile parity, r = operand
+// row) holds column 8*(r/4) + 4*t + r%4.
+__device__ __forceinline__ int b_row_to_col(int R) {
+    const int r = R & 15, t = (R >> 4) & 1;
+    return (R & ~31) | ((r >> 2) << 3) | (t << 2) | (r & 3);
+}
+
+// Epilogue of the tile kernels: alpha, bf16 (RNE), 16-byte stores.
+// acc[m][2p], acc[m][2p+1] hold, for C row `row_base + 16m + lane%16`, the 8 columns
+// `col_base + 32p + 8*(lane/16) .. +8` (see b_row_to_col).
+template <int MT, int NT, bool EDGE>
+__device__ __forceinline__ void store_c_tile(const v4f (&acc)[MT][NT], uint16_t* __restrict__ C,
+                                             int M, int N, int row_base, int col_base, float alpha) {
+    const int r = lane_id() & 15, g = lane_id() >> 4;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int row = row_base + 16 * m + r;
+#pragma unroll
+        for (int p = 0; p < NT / 2; ++p) {
+            const int col = col_base + 32 * p + 8 * g;
+            const v4f x = acc[m][2 * p] * alpha, y = acc[m][2 * p + 1] * alpha;
+            if (!EDGE) {
+                v4i out;
+                out.x = pack_bf16(x.x, x.y); out.y = pack_bf16(x.z, x.w);
+                out.z = pack_bf16(y.x, y.y); out.w = pack_bf16(y.z, y.w);
+                *(v4i*)(C + (size_t)row * N + col) = out;
+            } else if (row < M) {
+                const float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
+                if (col + 8 <= N && (N & 7) == 0) {
+                    v4i out;
+                    out.x = pack_bf16(v[0], v[1]); out.y = pack_bf16(v[2], v[3]);
+                    out.z = pack_bf16(v[4], v[5]); out.w = pack_bf16(v[6], v[7]);
+                    *(v4i*)(C + (size_t)row * N + col) = out;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (col + j < N)
+                            C[(size_t)row * N + col + j] = (uint16_t)(pack_bf16(v[j], 0.f) & 0xffffu);
+                }
+            }
+        }
+    }
+}
+
+}  // namespace hk

@@ -1,0 +1,376 @@
+// MXFP4 GEMM for gfx950: C[M,N] = bf16( sum_k A[m,k] * B[n,k] ), A and B in OCP MX format:
+// e2m1 elements packed two per byte (even k in the low nibble) and one e8m0 scale per 32
+// consecutive k (scales row-major [rows, K/32]); fp32 accumulation.
+//
+// No counterpart in the reference (it has no MXFP4 code); built on the same skeleton as the
+// FP8 kernel (kernels/gemm/fp8fp32 in the reference) with the block scales applied inside
+// the MFMA: v_mfma_scale_f32_16x16x128_f8f6f4 with cbsz = blgp = 4 (e2m1 operands) takes, per
+// lane, one e8m0 byte for the lane's own 32-element K-block of each operand, which is exactly
+// one MX block.
+//
+// Tile kernel: 256x256 tile of C, K-step 256 elements = 128 bytes per operand row, so the LDS
+// tile layout, swizzle and read pattern are those of the FP8 kernel; the two 16-byte halves a
+// lane reads per fragment row are MX blocks g and 4+g of the K-step and feed two MFMAs. The
+// 8 scale bytes per row and K-step travel through LDS next to the tiles (4-byte direct loads)
+// and are read back with one ds_read_b64 per fragment; a per-lane shift moves byte g into the
+// position the MFMA reads.
+#include "gemm_tile.h"
+#include "../../include/hk355.h"
+
+namespace hk {
+
+typedef __attribute__((address_space(3))) const v2i lds_v2i_t;
+
+constexpr int kScaleTileBytes = BM * 8;                // 8 scale bytes per row and K-step
+constexpr int kScaleStageBytes = 2 * kScaleTileBytes;  // A + B
+constexpr int kScaleBase = kLdsBytes;                  // scales sit behind the operand stages
+constexpr int kLdsBytesFp4 = kLdsBytes + 2 * kScaleStageBytes;
+
+struct Frag4 {
+    v4i lo, hi;  // MX blocks g and 4+g of this lane's row
+};
+
+__device__ __forceinline__ Frag4 lds_frag4(uint32_t addr_lo, uint32_t addr_hi, int imm) {
+    Frag4 f;
+    f.lo = *(lds_v4i_t*)(uintptr_t)(addr_lo + imm);
+    f.hi = *(lds_v4i_t*)(uintptr_t)(addr_hi + imm);
+    return f;
+}
+
+// 4-byte direct global->LDS load (64 lanes -> 256 contiguous LDS bytes).
+__device__ __forceinline__ void dma4(v4i srd, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dword %1, %2, %3 offen lds"
+        :
+        : "s"(lds_base), "v"(voff), "s"(srd), "s"(soff)
+        : "memory", "m0");
+}
+
+// acc(16x16) += X(16x128 e2m1, scale sx) * Y(16x128 e2m1, scale sy)^T, accumulator tied in
+// an AGPR; sx / sy carry the lane's e8m0 byte in bits [7:0].
+__device__ __forceinline__ void mfma_fp4_acc(v4f& acc, const v4i& x, const v4i& y, int sx, int sy) {
+    asm volatile(
+        "v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+        : "+a"(acc)
+        : "v"(x), "v"(y), "v"(sx), "v"(sy));
+}
+
+__device__ __forceinline__ v4f mfma_fp4(v4i x, v4i y, v4f c, int sx, int sy) {
+    v8i x8 = __builtin_shufflevector(x, x, 0, 1, 2, 3, 0, 1, 2, 3);
+    v8i y8 = __builtin_shufflevector(y, y, 0, 1, 2, 3, 0, 1, 2, 3);
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x8, y8, c, 4, 4, 0, sx, 0, sy);
+}
+
+template <bool EDGE>
+__global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
+    const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int tiles_m,
+    int tiles_n) {
+    constexpr int NW = 4, TM = 128, TN = 128, MT = 8, NT = 8;
+    constexpr int NDMA = kTileBytes / (NW * 1024);
+    constexpr int PG = 4, AD = 3;
+    static_assert(PG == 4 && AD == 3 && MT == 8, "slot plan below is written for these");
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+
+    const int lane = lane_id();
+    const int w = wave_id();
+    const int wm = w >> 1, wn = w & 1;
+    const int Kb = K >> 1;   // operand row pitch in bytes
+    const int Ks = K >> 5;   // scale row pitch in bytes
+
+    int pm, pn;
+    {
+        const int id = xcd_chunk_order(blockIdx.x, tiles_m * tiles_n, kCuPerXcd);
+        grouped_raster(id, tiles_m, tiles_n, 8, pm, pn);
+    }
+    const int row0 = pm * BM, col0 = pn * BN;
+    const int a_rows = min(M - row0, BM), b_rows = min(N - col0, BN);
+    const v4i srd_a = make_srd(A + (size_t)row0 * Kb, (uint32_t)a_rows * (uint32_t)Kb);
+    const v4i srd_b = make_srd(B + (size_t)col0 * Kb, (uint32_t)b_rows * (uint32_t)Kb);
+    const v4i srd_sa = make_srd(SA + (size_t)row0 * Ks, (uint32_t)a_rows * (uint32_t)Ks);
+    const v4i srd_sb = make_srd(SB + (size_t)col0 * Ks, (uint32_t)b_rows * (uint32_t)Ks);
+
+    // operand tiles: as in the FP8 kernel
+    uint32_t voff_a[EDGE ? NDMA : 1], voff_b[EDGE ? NDMA : 1];
+#pragma unroll
+    for (int i = 0; i < (EDGE ? NDMA : 1); ++i) {
+        const int R = 8 * (i * NW + w) + (lane >> 3);
+        const uint32_t c = swz_chunk(R, lane & 7);
+        int ra = R, rb = b_row_to_col(R);
+        if (EDGE) {
+            ra = min(ra, a_rows - 1);
+            rb = min(rb, b_rows - 1);
+        }
+        voff_a[i] = (uint32_t)ra * (uint32_t)Kb + c * 16u;
+        voff_b[i] = (uint32_t)rb * (uint32_t)Kb + c * 16u;
+    }
+    // scale tiles: load q (0..7) covers LDS rows 32q..32q+31, lane l -> row +l/2, dword l%2;
+    // this wave issues q = 2w and 2w+1 for each operand.
+    uint32_t voff_sa[2], voff_sb[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int R = 32 * (2 * w + j) + (lane >> 1);
+        int ra = R, rb = b_row_to_col(R);
+        if (EDGE) {
+            ra = min(ra, a_rows - 1);
+            rb = min(rb, b_rows - 1);
+        }
+        voff_sa[j] = (uint32_t)ra * (uint32_t)Ks + (lane & 1) * 4u;
+        voff_sb[j] = (uint32_t)rb * (uint32_t)Ks + (lane & 1) * 4u;
+    }
+    const uint32_t dma_row_stride = to_sgpr((uint32_t)(8 * NW) * (uint32_t)Kb);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+    const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
+    const uint32_t lds_scale_wave = to_sgpr(lds0 + kScaleBase + (uint32_t)w * 512u);
+
+    auto dma_one = [&](int op, int i, int stage, uint32_t k0, v4i srd) {
+        const uint32_t dst = lds_wave + (uint32_t)stage * kStageBytes + op * kTileBytes + i * NW * 1024;
+        if (EDGE)
+            dma16(srd, dst, op ? voff_b[i] : voff_a[i], k0);
+        else
+            dma16(srd, dst, op ? voff_b[0] : voff_a[0], k0 + i * dma_row_stride);
+    };
+    // j = 0..3: (operand j/2, load j%2) of this wave's scale loads for K-step kt into `stage`
+    auto dma_scale = [&](int j, int stage, uint32_t kt, v4i srd) {
+        const int op = j >> 1, h = j & 1;
+        const uint32_t dst = lds_scale_wave + (uint32_t)stage * kScaleStageBytes + op * kScaleTileBytes + h * 256;
+        dma4(srd, dst, op ? voff_sb[h] : voff_sa[h], kt * 8u);
+    };
+
+    const uint32_t r = lane & 15, g = lane >> 4;
+    const uint32_t rd_lo = r * 128u + swz_chunk(r, g) * 16u;
+    const uint32_t rd_hi = r * 128u + swz_chunk(r, g + 4) * 16u;
+    uint32_t a_lo[2], a_hi[2], b_lo[2], b_hi[2];
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+        a_lo[st] = lds0 + st * kStageBytes + wm * (TM * BK) + rd_lo;
+        a_hi[st] = lds0 + st * kStageBytes + wm * (TM * BK) + rd_hi;
+        b_lo[st] = lds0 + st * kStageBytes + kTileBytes + wn * (TN * BK) + rd_lo;
+        b_hi[st] = lds0 + st * kStageBytes + kTileBytes + wn * (TN * BK) + rd_hi;
+    }
+    // scales of fragment f, stage st: base + st*kScaleStageBytes + f*128
+    uint32_t sa_rd = lds0 + kScaleBase + (wm * TM + r) * 8u;
+    uint32_t sb_rd = lds0 + kScaleBase + kScaleTileBytes + (wn * TN + r) * 8u;
+    asm volatile("" : "+v"(sa_rd), "+v"(sb_rd));  // keep the large base in the register, offsets in immediates
+    const uint32_t sh = 8u * g;  // byte g of each scale dword belongs to this lane
+    auto rd_scale = [&](uint32_t base, int stage, int f) -> v2i {
+        return *(lds_v2i_t*)(uintptr_t)(base + stage * kScaleStageBytes + f * 128);
+    };
+    auto shift_scale = [&](v2i& s) {
+        s.x = (int)((uint32_t)s.x >> sh);
+        s.y = (int)((uint32_t)s.y >> sh);
+    };
+
+    v4f acc[MT][NT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
+    Frag4 bf[2][NT], af[4];
+    v2i bs[2][NT], as[4];
+
+    const int nk = K / 256;
+
+    // ---- prologue ----------------------------------------------------------------------
+#pragma unroll
+    for (int i = 0; i < NDMA; ++i) dma_one(0, i, 0, 0, srd_a);
+#pragma unroll
+    for (int i = 0; i < NDMA; ++i) dma_one(1, i, 0, 0, srd_b);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dma_scale(j, 0, 0, j >> 1 ? srd_sb : srd_sa);
+    wait_vmcnt<0>();
+    block_barrier();
+    if (nk > 1) {
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) dma_one(0, i, 1, BK, srd_a);
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) dma_one(1, i, 1, BK, srd_b);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dma_scale(j, 1, 1, j >> 1 ? srd_sb : srd_sa);
+    }
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+        bf[0][n] = lds_frag4(b_lo[0], b_hi[0], n * 16 * BK);
+        bs[0][n] = rd_scale(sb_rd, 0, n);
+    }
+#pragma unroll
+    for (int m = 0; m < AD; ++m) {
+        af[m] = lds_frag4(a_lo[0], a_hi[0], m * 16 * BK);
+        as[m] = rd_scale(sa_rd, 0, m);
+    }
+#pragma unroll
+    for (int n = 0; n < NT; ++n) shift_scale(bs[0][n]);
+    shift_scale(as[0]);  // as[1], as[2] are shifted inside the first step (groups 0 and 1)
+
+    // One K-step (see the FP8 4-wave kernel for the slot plan). Scale handling: the raw
+    // 8 bytes of a fragment are read together with the fragment; the shift that exposes
+    // this lane's byte is placed well after the read (B: group 7; A fragment f: group f-1).
+    auto step = [&]<int P>(int kt) {
+        const uint32_t k2 = (uint32_t)(kt + 2) * BK;
+        v4i sa = srd_a, sb = srd_b, ssa = srd_sa, ssb = srd_sb;
+        if (kt + 2 >= nk) { sa.z = 0; sb.z = 0; ssa.z = 0; ssb.z = 0; }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            // first the 8 MFMAs on the low K-half (MX block g), then the 8 on the high half
+            // (block 4+g): the two MFMAs into one accumulator are 8 issue slots apart
+#pragma unroll
+            for (int n = 0; n < NT; ++n) {
+                mfma_fp4_acc(acc[m][n], bf[P][n].lo, af[m & 3].lo, bs[P][n].x, as[m & 3].x);
+                if (m <= PG) {
+                    if (n == 0) {
+                        af[(m + AD) & 3] = lds_frag4(a_lo[P], a_hi[P], (m + AD) * 16 * BK);
+                        as[(m + AD) & 3] = rd_scale(sa_rd, P, m + AD);
+                    }
+                } else {
+                    const int j = (m - PG - 1) * NT + n;
+                    if (j < NT) {
+                        bf[P ^ 1][j] = lds_frag4(b_lo[P ^ 1], b_hi[P ^ 1], j * 16 * BK);
+                        bs[P ^ 1][j] = rd_scale(sb_rd, P ^ 1, j);
+                    } else if (j == NT || j == NT + 1) {
+                        af[j - NT] = lds_frag4(a_lo[P ^ 1], a_hi[P ^ 1], (j - NT) * 16 * BK);
+                        as[j - NT] = rd_scale(sa_rd, P ^ 1, j - NT);
+                    } else if (j == 2 * NT) {
+                        af[2] = lds_frag4(a_lo[P ^ 1], a_hi[P ^ 1], 2 * 16 * BK);
+                        as[2] = rd_scale(sa_rd, P ^ 1, 2);
+                    }
+                    if (j < 2 * NDMA) dma_one(j / NDMA, j % NDMA, P, k2, j / NDMA ? sb : sa);
+                    else if (j < 2 * NDMA + 4) dma_scale(j - 2 * NDMA, P, kt + 2, (j - 2 * NDMA) >> 1 ? ssb : ssa);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int n = 0; n < NT; ++n) {
+                mfma_fp4_acc(acc[m][n], bf[P][n].hi, af[m & 3].hi, bs[P][n].y, as[m & 3].y);
+                if (m == MT - 1) shift_scale(bs[P ^ 1][n]);
+                // scale of A fragment m+1 (next step's fragment 0 when m == 7)
+                if (n == 4) shift_scale(as[(m + 1) & 3]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (m == PG) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                wait_vmcnt<0>();
+                block_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+        step.template operator()<0>(kt);
+        step.template operator()<1>(kt + 1);
+    }
+    if (kt < nk) step.template operator()<0>(kt);
+    wait_vmcnt<0>();
+    mfma_drain();
+
+    store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, 1.0f);
+}
+
+// Portable kernel for any M, N and K % 32 == 0: operands and scales straight from global
+// memory, K-step 128 elements (lane group g holds MX block g of the step).
+__global__ __launch_bounds__(256) void mxfp4_gemm_portable_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
+    const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K) {
+    const int lane = lane_id(), w = wave_id();
+    const int r = lane & 15, g = lane >> 4;
+    const int row0 = blockIdx.y * 64 + (w >> 1) * 32;
+    const int col0 = blockIdx.x * 64 + (w & 1) * 32;
+    const int Kb = K >> 1, Ks = K >> 5;
+    v4f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    for (int k0 = 0; k0 < K; k0 += 128) {
+        v4i af[2], bf[2];
+        int as[2], bs[2];
+        const int kk = k0 + 32 * g;  // first element of this lane's block
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int ra = row0 + 16 * i + r, rb = col0 + 16 * i + r;
+            af[i] = v4i{0, 0, 0, 0}; bf[i] = v4i{0, 0, 0, 0};
+            as[i] = 127; bs[i] = 127;
+            if (ra < M && kk < K) {
+                af[i] = *(const v4i*)(A + (size_t)ra * Kb + (kk >> 1));
+                as[i] = SA[(size_t)ra * Ks + (kk >> 5)];
+            }
+            if (rb < N && kk < K) {
+                bf[i] = *(const v4i*)(B + (size_t)rb * Kb + (kk >> 1));
+                bs[i] = SB[(size_t)rb * Ks + (kk >> 5)];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) acc[i][j] = mfma_fp4(bf[j], af[i], acc[i][j], bs[j], as[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int row = row0 + 16 * i + r;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const float v[4] = {acc[i][j].x, acc[i][j].y, acc[i][j].z, acc[i][j].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int col = col0 + 16 * j + 4 * g + e;
+                if (row < M && col < N)
+                    C[(size_t)row * N + col] = (uint16_t)(pack_bf16(v[e], 0.f) & 0xffffu);
+            }
+        }
+    }
+}
+
+template <bool EDGE>
+static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, const void* SB, void* C,
+                              int M, int N, int K, hipStream_t stream) {
+    auto kern = mxfp4_gemm_4wave_kernel<EDGE>;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kLdsBytesFp4) != hipSuccess)
+            return HK_ERR_LAUNCH;
+        configured = true;
+    }
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), kLdsBytesFp4, stream,
+                       (const uint8_t*)A, (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB,
+                       (uint16_t*)C, M, N, K, tiles_m, tiles_n);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
+}  // namespace hk
+
+extern "C" int hk_mxfp4_gemm_variant(const void* A, const void* A_scales, const void* B,
+                                     const void* B_scales, void* C, int M, int N, int K, int variant,
+                                     void* stream) {
+    using namespace hk;
+    if (!A || !A_scales || !B || !B_scales || !C) return HK_ERR_NULL_POINTER;
+    if (M <= 0 || N <= 0 || K <= 0 || (K % 32) != 0) return HK_ERR_BAD_SHAPE;
+    if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    if (variant < 0 || variant > 1) return HK_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    if (variant == 0) {
+        if ((M + 63) / 64 > 65535) return HK_ERR_BAD_SHAPE;
+        dim3 grid((N + 63) / 64, (M + 63) / 64);
+        hipLaunchKernelGGL(mxfp4_gemm_portable_kernel, grid, dim3(256), 0, s, (const uint8_t*)A,
+                           (const uint8_t*)A_scales, (const uint8_t*)B, (const uint8_t*)B_scales,
+                           (uint16_t*)C, M, N, K);
+        return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+    }
+    if ((K % 256) != 0 || (long long)(K / 2) * BM >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
+    if (((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) return HK_ERR_BAD_ALIGNMENT;
+    const bool edge = (M % BM) != 0 || (N % BN) != 0;
+    return edge ? launch_mxfp4_4wave<true>(A, A_scales, B, B_scales, C, M, N, K, s)
+                : launch_mxfp4_4wave<false>(A, A_scales, B, B_scales, C, M, N, K, s);
+}
+
+extern "C" int hk_mxfp4_gemm(const void* A, const void* A_scales, const void* B, const void* B_scales,
+                             void* C, int M, int N, int K, void* stream) {
+    const bool tile_ok = K > 0 && (K % 256) == 0 && M >= 64 && N >= 64 &&
+                         ((((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) == 0);
+    return hk_mxfp4_gemm_variant(A, A_scales, B, B_scales, C, M, N, K, tile_ok ? 1 : 0, stream);
+}

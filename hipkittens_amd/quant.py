@@ -22,3 +22,26 @@ def quantize_fp8_per_tensor(x: torch.Tensor):
     amax = xf.abs().max()
     scale = torch.where(amax > 0, amax / E4M3_MAX, torch.ones_like(amax)).to(torch.float32)
     return to_e4m3_saturating(xf / scale), float(scale)
+
+
+def quantize_mxfp4(x: torch.Tensor):
+    """OCP MX (v1.0) quantization along the last dim in blocks of 32: shared exponent
+    e = floor(log2(amax)) - 2 stored as e8m0 byte e + 127, elements e2m1(x / 2^e) (round to
+    nearest even, saturating at 6). Returns (packed uint8 [..., K/2] with the even k in the low
+    nibble, scales uint8 [..., K/32])."""
+    K = x.shape[-1]
+    if K % 32:
+        raise RuntimeError("quantize_mxfp4: last dimension must be a multiple of 32")
+    xb = x.float().reshape(*x.shape[:-1], K // 32, 32)
+    amax = xb.abs().amax(dim=-1)
+    _, ex = torch.frexp(amax)
+    e = (ex - 3).clamp(-127, 127)
+    e = torch.where(amax > 0, e, torch.zeros_like(e))
+    scaled = torch.ldexp(xb, (-e).unsqueeze(-1))
+    a = scaled.abs().clamp(max=6.0)
+    code = torch.where(a < 2.0, torch.round(a * 2.0),
+                       torch.where(a < 4.0, 4.0 + torch.round(a - 2.0), 6.0 + torch.round((a - 4.0) * 0.5)))
+    code = code.to(torch.uint8) | (torch.signbit(scaled).to(torch.uint8) << 3)
+    code = code.reshape(*x.shape[:-1], K)
+    packed = code[..., 0::2] | (code[..., 1::2] << 4)
+    return packed.contiguous(), (e + 127).to(torch.uint8).contiguous()

@@ -64,3 +64,35 @@ def dispatch_fp8_gemm(A, B, C, scale_a: float = 1.0, scale_b: float = 1.0, varia
 def dispatch_micro(A, B, C) -> None:
     """The reference's GEMM entry point name: C = A @ B.T with unit scales."""
     dispatch_fp8_gemm(A, B, C, 1.0, 1.0)
+
+
+_U8 = (torch.uint8,)
+_FP4 = tuple(d for d in (torch.uint8, getattr(torch, "float4_e2m1fn_x2", None)) if d is not None)
+_E8M0 = tuple(d for d in (torch.uint8, getattr(torch, "float8_e8m0fnu", None)) if d is not None)
+
+
+def dispatch_mxfp4_gemm(A, A_scales, B, B_scales, C, variant: int = -1) -> None:
+    """C[M,N] (bf16) = dequant(A) @ dequant(B).T for MXFP4 operands: A [M,K/2] packed e2m1
+    (low nibble = even k), A_scales [M,K/32] e8m0, B [N,K/2], B_scales [N,K/32]."""
+    _check_tensor(A, "A", _FP4, 2)
+    _check_tensor(B, "B", _FP4, 2)
+    _check_tensor(A_scales, "A_scales", _E8M0, 2)
+    _check_tensor(B_scales, "B_scales", _E8M0, 2)
+    _check_tensor(C, "C", (torch.bfloat16,), 2)
+    M, Kh = A.shape
+    N, Kh2 = B.shape
+    K = 2 * Kh
+    if Kh2 != Kh or K % 32 != 0 or tuple(A_scales.shape) != (M, K // 32) or \
+            tuple(B_scales.shape) != (N, K // 32) or tuple(C.shape) != (M, N):
+        raise RuntimeError(
+            f"shape mismatch: A {tuple(A.shape)}, A_scales {tuple(A_scales.shape)}, B {tuple(B.shape)}, "
+            f"B_scales {tuple(B_scales.shape)}, C {tuple(C.shape)}")
+    if len({t.device for t in (A, A_scales, B, B_scales, C)}) != 1:
+        raise RuntimeError("all tensors must be on the same device")
+    lib = _lib.load_library()
+    args = (A.data_ptr(), A_scales.data_ptr(), B.data_ptr(), B_scales.data_ptr(), C.data_ptr(), M, N, K)
+    if variant < 0:
+        st = lib.hk_mxfp4_gemm(*args, _stream(A))
+    else:
+        st = lib.hk_mxfp4_gemm_variant(*args, int(variant), _stream(A))
+    _lib.check(st, "dispatch_mxfp4_gemm")

@@ -59,6 +59,23 @@ int hk_fp8_gemm_variant(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
                         int M, int N, int K, float scale_a, float scale_b,
                         int variant, void* stream);
 
+/*
+ * MXFP4 GEMM (OCP Microscaling v1.0): C[M,N] = bf16( sum_k a[m,k] * b[n,k] ) with
+ *   a[m,k] = e2m1(A[m, k/2] nibble k%2; low nibble = even k) * 2^(A_scales[m, k/32] - 127)
+ * and b likewise. A is [M, K/2] bytes, A_scales [M, K/32] e8m0 bytes, B [N, K/2], B_scales
+ * [N, K/32], all row-major; fp32 accumulation, C [M,N] bf16 (RNE).
+ * No counterpart in the reference (it has no MXFP4 code); same calling convention as
+ * hk_fp8_gemm. Requirements: M,N,K > 0; K % 32 == 0; A, B, C 16-byte aligned.
+ */
+int hk_mxfp4_gemm(const void* A_e2m1, const void* A_scales_e8m0, const void* B_e2m1,
+                  const void* B_scales_e8m0, void* C_bf16, int M, int N, int K, void* stream);
+
+/* Same contract on a chosen kernel: 0 = portable kernel (any shape), 1 = 256x256x256 tile
+ * kernel (needs K % 256 == 0 and 4-byte aligned scale pointers). */
+int hk_mxfp4_gemm_variant(const void* A_e2m1, const void* A_scales_e8m0, const void* B_e2m1,
+                          const void* B_scales_e8m0, void* C_bf16, int M, int N, int K,
+                          int variant, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,114 @@
+"""MXFP4 GEMM: HIP path (through the C ABI) against the CPU oracle (dequantize + fp32 matmul).
+
+Tolerance: relative Frobenius error <= 1e-2 on the bf16 output (north-star bound). The MFMA
+applies the e8m0 block scales exactly (powers of two) and accumulates in fp32, so only
+accumulation order and the final bf16 rounding differ from the oracle (~2e-3 observed).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import formats as F
+from oracle import gemm as G
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def _run(hk, a, sa, b, sb, variant=-1):
+    dev = torch.device("cuda:0")
+    t = [torch.from_numpy(x).to(dev) for x in (a, sa, b, sb)]
+    C = torch.full((a.shape[0], b.shape[0]), float("nan"), dtype=torch.bfloat16, device=dev)
+    hk.tk_kernel.dispatch_mxfp4_gemm(t[0], t[1], t[2], t[3], C, variant=variant)
+    torch.cuda.synchronize()
+    return C.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def _rand_mx(rng, rows, K, spread=True):
+    x = rng.standard_normal((rows, K)).astype(np.float32)
+    if spread:  # different magnitudes per block so that the scales matter
+        x *= np.exp2(rng.integers(-6, 7, size=(rows, K // 32))).repeat(32, axis=1).astype(np.float32)
+    return F.quantize_mxfp4(x)
+
+
+SHAPES = [(256, 256, 256), (256, 256, 512), (512, 768, 1024), (1024, 1024, 2048)]
+RAGGED = [(300, 200, 256), (257, 255, 512), (64, 72, 768), (1000, 520, 512)]
+
+
+@pytest.mark.parametrize("variant", [0, 1, -1])
+@pytest.mark.parametrize("shape", SHAPES + RAGGED)
+def test_mxfp4_gemm_matches_oracle(hk, shape, variant):
+    M, N, K = shape
+    print(f"mxfp4_gemm shape={shape} variant={variant}", flush=True)
+    rng = np.random.default_rng(99 + M + N + K)
+    (a, sa), (b, sb) = _rand_mx(rng, M, K), _rand_mx(rng, N, K)
+    out = F.bf16_to_f32(_run(hk, a, sa, b, sb, variant))
+    ref = G.mxfp4_gemm(a, sa, b, sb)
+    assert np.isfinite(out).all()
+    err = G.rel_fro_error(out, ref)
+    assert err <= TOL, (shape, variant, err)
+    assert err <= 5e-3
+
+
+@pytest.mark.parametrize("variant", [0, -1])
+def test_mxfp4_gemm_k_not_multiple_of_256(hk, variant):
+    M, N, K = 96, 80, 160
+    rng = np.random.default_rng(7)
+    (a, sa), (b, sb) = _rand_mx(rng, M, K), _rand_mx(rng, N, K)
+    out = F.bf16_to_f32(_run(hk, a, sa, b, sb, variant))
+    assert G.rel_fro_error(out, G.mxfp4_gemm(a, sa, b, sb)) <= 5e-3
+
+
+def test_mxfp4_gemm_tile_kernel_rejects_k_tail(hk):
+    rng = np.random.default_rng(7)
+    (a, sa), (b, sb) = _rand_mx(rng, 64, 160), _rand_mx(rng, 64, 160)
+    with pytest.raises(RuntimeError):
+        _run(hk, a, sa, b, sb, 1)
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+def test_mxfp4_gemm_exact_small_integers(hk, variant):
+    """Elements in {-2,-1,0,1,2} with power-of-two block scales: every product and partial sum
+    is exact in fp32, so the result must equal the exact value rounded once to bf16."""
+    M, N, K = 256, 512, 512
+    rng = np.random.default_rng(21)
+    codes = np.array([0, 2, 4, 10, 12], dtype=np.uint8)  # e2m1 codes of 0, 1, 2, -1, -2
+
+    def make(rows):
+        c = codes[rng.integers(0, 5, size=(rows, K))]
+        packed = (c[:, 0::2] | (c[:, 1::2] << 4)).astype(np.uint8)
+        scales = rng.integers(125, 130, size=(rows, K // 32)).astype(np.uint8)
+        return packed, scales
+
+    (a, sa), (b, sb) = make(M), make(N)
+    out = _run(hk, a, sa, b, sb, variant)
+    exact = F.dequantize_mxfp4(a, sa).astype(np.float64) @ F.dequantize_mxfp4(b, sb).astype(np.float64).T
+    assert np.array_equal(out, F.bf16_round(exact.astype(np.float32)))
+
+
+def test_mxfp4_gemm_scale_byte_positions(hk):
+    """One nonzero block per row pair: catches a scale applied to the wrong 32-block."""
+    M = N = 256
+    K = 512
+    a = np.zeros((M, K // 2), np.uint8); b = np.zeros((N, K // 2), np.uint8)
+    sa = np.full((M, K // 32), 127, np.uint8); sb = np.full((N, K // 32), 127, np.uint8)
+    rng = np.random.default_rng(2)
+    blk_a = rng.integers(0, K // 32, size=M)
+    for i in range(M):
+        a[i, blk_a[i] * 16:(blk_a[i] + 1) * 16] = 0x22  # all ones in that block
+        sa[i, :] = rng.integers(120, 134, size=K // 32)
+    b[:] = 0x22
+    sb[:] = rng.integers(120, 134, size=(N, K // 32))
+    out = _run(hk, a, sa, b, sb, 1)
+    exact = F.dequantize_mxfp4(a, sa).astype(np.float64) @ F.dequantize_mxfp4(b, sb).astype(np.float64).T
+    assert np.array_equal(out, F.bf16_round(exact.astype(np.float32)))
+
+
+def test_mxfp4_gemm_device_quantizer_matches_oracle(hk):
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((128, 256)) * np.exp2(rng.integers(-20, 20, size=(128, 1)))).astype(np.float32)
+    x[3, :32] = 0.0
+    p, s = hk.quant.quantize_mxfp4(torch.from_numpy(x).to(dev))
+    po, so = F.quantize_mxfp4(x)
+    assert np.array_equal(p.cpu().numpy(), po) and np.array_equal(s.cpu().numpy(), so)
