@@ -30,6 +30,13 @@ HIPCC_FLAGS = [
 ]
 
 
+# Files whose arithmetic is specified operation by operation (bit-exact against the CPU oracle)
+# are built without fused multiply-add contraction.
+PER_FILE_FLAGS = {
+    "moe_routing.hip": ["-ffp-contract=off"],
+}
+
+
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -39,7 +46,7 @@ def _hipcc() -> str:
 
 def _compile_one(src: Path, extra: list[str]) -> Path:
     obj = BUILD_DIR / (src.stem + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", str(src), "-o", str(obj)]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *PER_FILE_FLAGS.get(src.name, []), *extra, "-c", str(src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src.name}:\n{res.stdout}\n{res.stderr}")

@@ -1,0 +1,359 @@
+// MoE routing for gfx950: top-k selection (softmax and group-limited sigmoid) and the stable
+// counting sort of (token, choice) slots by expert. All bandwidth / latency bound; one wave per
+// token, wavefront shuffles and ballots, coalesced HBM access.
+//
+// The reference has no MoE code (no counterpart to cite). Integer outputs are specified to be
+// bit-exact against the CPU oracle: ties go to the lower expert id, the sort is stable, and the
+// sigmoid used for selection is a fixed sequence of correctly rounded fp32 operations.
+#include "hk_device.h"
+#include "../../include/hk355.h"
+
+// This file must be compiled with -ffp-contract=off (hipkittens_amd/build.py does): the routing
+// arithmetic is specified as separately rounded fp32 operations, and HIP's __fmul_rn / __fadd_rn
+// are plain operators that the compiler would otherwise fuse into FMAs.
+
+namespace hk {
+
+// ---------------------------------------------------------------------------------- helpers
+// Monotonic key: larger float -> larger key; -0.0 and +0.0 compare equal.
+__device__ __forceinline__ uint32_t float_key(float x) {
+    uint32_t u = __float_as_uint(x);
+    if (x == 0.0f) u = 0;
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+// (key, expert id) packed so that max() picks the larger key and, on ties, the lower id.
+__device__ __forceinline__ uint64_t pack_choice(float x, int id) {
+    return ((uint64_t)float_key(x) << 32) | (uint32_t)(0x7fffffff - id);
+}
+__device__ __forceinline__ int choice_id(uint64_t c) { return 0x7fffffff - (int)(uint32_t)c; }
+
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const uint64_t o = __shfl_xor(v, off, 64);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+__device__ __forceinline__ float wave_sum_f32_ordered(float v, int k, int lane) {
+    // sum of lanes 0..k-1 in lane order (k <= 64), the same order the oracle uses
+    float tot = 0.f;
+    for (int j = 0; j < k; ++j) tot = __fadd_rn(tot, __shfl(v, j, 64));
+    return tot;
+}
+
+// exp(x) for x in [-87, 0] and the sigmoid built on it: fixed fp32 operation sequence, no
+// contraction, so that CPU and GPU agree bit for bit.
+__device__ __forceinline__ float exp_neg_f32(float x) {
+    x = fmaxf(x, -87.0f);
+    const float n = rintf(__fmul_rn(x, 1.4426950408889634f));
+    float r = __fsub_rn(x, __fmul_rn(n, 0.693145751953125f));
+    r = __fsub_rn(r, __fmul_rn(n, 1.4286068203094172e-06f));
+    float p = 1.0f / 720;
+    p = __fadd_rn(__fmul_rn(p, r), 1.0f / 120);
+    p = __fadd_rn(__fmul_rn(p, r), 1.0f / 24);
+    p = __fadd_rn(__fmul_rn(p, r), 1.0f / 6);
+    p = __fadd_rn(__fmul_rn(p, r), 0.5f);
+    p = __fadd_rn(__fmul_rn(p, r), 1.0f);
+    p = __fadd_rn(__fmul_rn(p, r), 1.0f);
+    return ldexpf(p, (int)n);
+}
+__device__ __forceinline__ float sigmoid_f32(float x) {
+    const float e = exp_neg_f32(-fabsf(x));
+    const float d = __fadd_rn(1.0f, e);
+    return x >= 0.f ? __fdiv_rn(1.0f, d) : __fdiv_rn(e, d);
+}
+
+constexpr int kMaxPerLane = 8;  // experts per lane: E <= 512
+
+// ------------------------------------------------------------------------- top-k softmax
+// One wave per token. ids[t, j] = j-th largest logit (ties -> lower id); w = softmax over the k
+// selected logits.
+__global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const float* __restrict__ logits, int T,
+                                                               int E, int k, int32_t* __restrict__ ids,
+                                                               float* __restrict__ w) {
+    const int lane = lane_id();
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= T) return;
+    const float* row = logits + (size_t)t * E;
+    uint64_t cand[kMaxPerLane];
+    const int per = (E + 63) / 64;
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+        const int e = i * 64 + lane;  // coalesced
+        cand[i] = (i < per && e < E) ? pack_choice(row[e], e) : 0ull;
+    }
+    float my_logit = 0.f, top_logit = 0.f;
+    int my_id = 0;
+    for (int j = 0; j < k; ++j) {
+        uint64_t best = 0;
+#pragma unroll
+        for (int i = 0; i < kMaxPerLane; ++i) best = cand[i] > best ? cand[i] : best;
+        best = wave_max_u64(best);
+        const int id = choice_id(best);
+#pragma unroll
+        for (int i = 0; i < kMaxPerLane; ++i)
+            if (cand[i] == best) cand[i] = 0ull;  // ids are unique, only the owner matches
+        const float v = row[id];
+        if (j == 0) top_logit = v;
+        if (lane == j) { my_logit = v; my_id = id; }
+    }
+    const float ex = lane < k ? expf(my_logit - top_logit) : 0.f;
+    float tot = ex;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) tot += __shfl_xor(tot, off, 64);
+    if (lane < k) {
+        ids[(size_t)t * k + lane] = my_id;
+        w[(size_t)t * k + lane] = ex / tot;
+    }
+}
+
+// ------------------------------------------------------------- group-limited sigmoid top-k
+__global__ __launch_bounds__(256) void moe_topk_grouped_sigmoid_kernel(
+    const float* __restrict__ logits, const float* __restrict__ bias, int T, int E, int k, int n_group,
+    int topk_group, float routed_scale, int32_t* __restrict__ ids, float* __restrict__ w) {
+    const int lane = lane_id();
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= T) return;
+    const float* row = logits + (size_t)t * E;
+    const int gs = E / n_group;
+    const int per = (E + 63) / 64;
+    float s[kMaxPerLane], c[kMaxPerLane];
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+        const int e = i * 64 + lane;
+        s[i] = 0.f; c[i] = 0.f;
+        if (i < per && e < E) {
+            s[i] = sigmoid_f32(row[e]);
+            c[i] = bias ? __fadd_rn(s[i], bias[e]) : s[i];
+        }
+    }
+    // group scores: sum of the two largest c in each group. Lane g (< n_group) ends up owning
+    // group g's score.
+    float gscore = -INFINITY;
+    for (int grp = 0; grp < n_group; ++grp) {
+        uint64_t best1 = 0, best2 = 0;
+#pragma unroll
+        for (int i = 0; i < kMaxPerLane; ++i) {
+            const int e = i * 64 + lane;
+            if (i < per && e < E && e / gs == grp) {
+                const uint64_t p = pack_choice(c[i], e);
+                if (p > best1) { best2 = best1; best1 = p; } else if (p > best2) best2 = p;
+            }
+        }
+        const uint64_t m1 = wave_max_u64(best1);
+        const uint64_t mine = (best1 == m1) ? best2 : best1;  // runner-up candidates
+        const uint64_t m2 = wave_max_u64(mine);
+        // recover the two values from their owners
+        float v1 = 0.f, v2 = 0.f;
+        const int id1 = choice_id(m1), id2 = choice_id(m2);
+#pragma unroll
+        for (int i = 0; i < kMaxPerLane; ++i) {
+            const int e = i * 64 + lane;
+            if (i < per && e == id1) v1 = c[i];
+            if (i < per && e == id2) v2 = c[i];
+        }
+        v1 = __shfl(v1, id1 & 63, 64);
+        v2 = __shfl(v2, id2 & 63, 64);
+        const float sc = gs >= 2 ? __fadd_rn(v1, v2) : v1;
+        if (lane == grp) gscore = sc;
+    }
+    // keep the topk_group best groups (ties -> lower group id)
+    uint64_t gc = lane < n_group ? pack_choice(gscore, lane) : 0ull;
+    uint64_t keep_mask = 0;
+    for (int j = 0; j < topk_group; ++j) {
+        const uint64_t b = wave_max_u64(gc);
+        if (gc == b) gc = 0ull;
+        keep_mask |= 1ull << choice_id(b);
+    }
+    // top-k of c among the kept groups
+    uint64_t cand[kMaxPerLane];
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+        const int e = i * 64 + lane;
+        const bool ok = i < per && e < E && ((keep_mask >> (e / gs)) & 1ull);
+        cand[i] = ok ? pack_choice(c[i], e) : 0ull;
+    }
+    float my_s = 0.f;
+    int my_id = 0;
+    for (int j = 0; j < k; ++j) {
+        uint64_t best = 0;
+#pragma unroll
+        for (int i = 0; i < kMaxPerLane; ++i) best = cand[i] > best ? cand[i] : best;
+        best = wave_max_u64(best);
+        const int id = choice_id(best);
+        float sv = 0.f;
+#pragma unroll
+        for (int i = 0; i < kMaxPerLane; ++i)
+            if (cand[i] == best) { cand[i] = 0ull; sv = s[i]; }
+        sv = __shfl(sv, id & 63, 64);
+        if (lane == j) { my_s = sv; my_id = id; }
+    }
+    const float tot = wave_sum_f32_ordered(my_s, k, lane);
+    if (lane < k) {
+        ids[(size_t)t * k + lane] = my_id;
+        w[(size_t)t * k + lane] = __fmul_rn(__fdiv_rn(my_s, tot), routed_scale);
+    }
+}
+
+// --------------------------------------------------------------------------------- sort
+// Stable counting sort of S = T*k slots by expert id, three launches:
+//   count   : per-chunk histogram (chunk = 1024 consecutive slots) -> ws[chunk][E]
+//   scan    : ws[chunk][e] := first output position of chunk's slots of expert e;
+//             expert_offsets[0..E]
+//   scatter : position of a slot = ws[chunk][e] + number of earlier slots of e in the chunk
+// The within-chunk rank comes from wave ballots in slot order, never from atomics' arrival
+// order, so the result is deterministic and stable.
+constexpr int kSortChunk = 1024;
+constexpr int kSortMaxE = 512;
+
+__global__ __launch_bounds__(256) void moe_sort_count_kernel(const int32_t* __restrict__ ids, int S,
+                                                             int E, int32_t* __restrict__ ws) {
+    __shared__ int cnt[kSortMaxE];
+    for (int e = threadIdx.x; e < E; e += 256) cnt[e] = 0;
+    __syncthreads();
+    const int base = blockIdx.x * kSortChunk;
+#pragma unroll
+    for (int i = 0; i < kSortChunk / 256; ++i) {
+        const int sidx = base + i * 256 + threadIdx.x;
+        if (sidx < S) atomicAdd(&cnt[ids[sidx]], 1);
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += 256) ws[(size_t)blockIdx.x * E + e] = cnt[e];
+}
+
+__global__ __launch_bounds__(512) void moe_sort_scan_kernel(int32_t* __restrict__ ws, int nchunks, int E,
+                                                             int32_t* __restrict__ expert_offsets) {
+    __shared__ int total[kSortMaxE];
+    __shared__ int start[kSortMaxE + 1];
+    const int e = threadIdx.x;
+    int run = 0;
+    if (e < E) {
+        for (int c = 0; c < nchunks; ++c) {
+            const int v = ws[(size_t)c * E + e];
+            ws[(size_t)c * E + e] = run;
+            run += v;
+        }
+        total[e] = run;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int acc = 0;
+        for (int i = 0; i < E; ++i) { start[i] = acc; acc += total[i]; }
+        start[E] = acc;
+    }
+    __syncthreads();
+    if (e < E) {
+        const int st = start[e];
+        expert_offsets[e] = st;
+        for (int c = 0; c < nchunks; ++c) ws[(size_t)c * E + e] += st;
+    }
+    if (e == 0) expert_offsets[E] = start[E];
+}
+
+__global__ __launch_bounds__(256) void moe_sort_scatter_kernel(const int32_t* __restrict__ ids, int S, int E,
+                                                               const int32_t* __restrict__ ws,
+                                                               int32_t* __restrict__ sorted_slots,
+                                                               int32_t* __restrict__ slot_to_pos) {
+    // 16 rounds of 64 consecutive slots per chunk: wave w takes rounds 4w..4w+3
+    __shared__ int round_cnt[16][kSortMaxE];  // later: exclusive prefix over rounds
+    const int lane = lane_id(), wv = threadIdx.x >> 6;
+    const int base = blockIdx.x * kSortChunk;
+    for (int i = threadIdx.x; i < 16 * E; i += 256) round_cnt[i / E][i % E] = 0;
+    __syncthreads();
+    int my_e[4], my_rank[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int rnd = wv * 4 + q;
+        const int sidx = base + rnd * 64 + lane;
+        const int e = sidx < S ? ids[sidx] : -1;
+        my_e[q] = e;
+        // stable rank among equal ids inside this round of 64
+        uint64_t todo = __ballot(e >= 0);
+        int rank = 0;
+        while (todo) {
+            const int leader = __ffsll((unsigned long long)todo) - 1;
+            const int e0 = __shfl(e, leader, 64);
+            const uint64_t same = __ballot(e == e0);
+            if (e == e0) {
+                rank = __popcll(same & ((1ull << lane) - 1ull));
+                if (lane == leader) round_cnt[rnd][e0] = __popcll(same);
+            }
+            todo &= ~same;
+        }
+        my_rank[q] = rank;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += 256) {
+        int run = ws[(size_t)blockIdx.x * E + e];
+#pragma unroll
+        for (int rnd = 0; rnd < 16; ++rnd) {
+            const int v = round_cnt[rnd][e];
+            round_cnt[rnd][e] = run;
+            run += v;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int rnd = wv * 4 + q;
+        const int sidx = base + rnd * 64 + lane;
+        if (my_e[q] >= 0) {
+            const int pos = round_cnt[rnd][my_e[q]] + my_rank[q];
+            sorted_slots[pos] = sidx;
+            if (slot_to_pos) slot_to_pos[sidx] = pos;
+        }
+    }
+}
+
+}  // namespace hk
+
+extern "C" int hk_moe_topk_softmax(const float* logits, int T, int E, int k, int32_t* ids, float* w,
+                                   void* stream) {
+    using namespace hk;
+    if (!logits || !ids || !w) return HK_ERR_NULL_POINTER;
+    if (T <= 0 || E <= 0 || k <= 0 || k > E || k > 64 || E > 64 * kMaxPerLane) return HK_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(moe_topk_softmax_kernel, dim3((T + 3) / 4), dim3(256), 0, (hipStream_t)stream,
+                       logits, T, E, k, ids, w);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
+extern "C" int hk_moe_topk_grouped_sigmoid(const float* logits, const float* bias_or_null, int T, int E,
+                                           int k, int n_group, int topk_group, float routed_scale,
+                                           int32_t* ids, float* w, void* stream) {
+    using namespace hk;
+    if (!logits || !ids || !w) return HK_ERR_NULL_POINTER;
+    if (T <= 0 || E <= 0 || k <= 0 || k > 64 || E > 64 * kMaxPerLane || n_group <= 0 || n_group > 64 ||
+        (E % n_group) != 0 || topk_group <= 0 || topk_group > n_group ||
+        k > topk_group * (E / n_group))
+        return HK_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(moe_topk_grouped_sigmoid_kernel, dim3((T + 3) / 4), dim3(256), 0,
+                       (hipStream_t)stream, logits, bias_or_null, T, E, k, n_group, topk_group,
+                       routed_scale, ids, w);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
+extern "C" size_t hk_moe_sort_workspace_bytes(int T, int k, int E) {
+    if (T <= 0 || k <= 0 || E <= 0) return 0;
+    const size_t S = (size_t)T * k;
+    const size_t nchunks = (S + hk::kSortChunk - 1) / hk::kSortChunk;
+    return nchunks * (size_t)E * sizeof(int32_t);
+}
+
+extern "C" int hk_moe_sort(const int32_t* ids, int T, int k, int E, int32_t* sorted_slots,
+                           int32_t* expert_offsets, int32_t* slot_to_pos_or_null, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+    using namespace hk;
+    if (!ids || !sorted_slots || !expert_offsets) return HK_ERR_NULL_POINTER;
+    if (T <= 0 || k <= 0 || E <= 0 || E > kSortMaxE || (long long)T * k >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
+    if (!workspace || workspace_bytes < hk_moe_sort_workspace_bytes(T, k, E)) return HK_ERR_WORKSPACE;
+    const int S = T * k;
+    const int nchunks = (S + kSortChunk - 1) / kSortChunk;
+    hipStream_t s = (hipStream_t)stream;
+    int32_t* ws = (int32_t*)workspace;
+    hipLaunchKernelGGL(moe_sort_count_kernel, dim3(nchunks), dim3(256), 0, s, ids, S, E, ws);
+    hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(1), dim3(512), 0, s, ws, nchunks, E, expert_offsets);
+    hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(nchunks), dim3(256), 0, s, ids, S, E,
+                       (const int32_t*)ws, sorted_slots, slot_to_pos_or_null);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}

@@ -96,3 +96,63 @@ def dispatch_mxfp4_gemm(A, A_scales, B, B_scales, C, variant: int = -1) -> None:
     else:
         st = lib.hk_mxfp4_gemm_variant(*args, int(variant), _stream(A))
     _lib.check(st, "dispatch_mxfp4_gemm")
+
+
+# ------------------------------------------------------------------------------ MoE routing
+_F32 = (torch.float32,)
+_I32 = (torch.int32,)
+
+
+def dispatch_moe_topk_softmax(logits, ids, weights) -> None:
+    """logits [T,E] fp32 -> ids [T,k] int32, weights [T,k] fp32 (k from the output shape)."""
+    _check_tensor(logits, "logits", _F32, 2)
+    _check_tensor(ids, "ids", _I32, 2)
+    _check_tensor(weights, "weights", _F32, 2)
+    T, E = logits.shape
+    if ids.shape[0] != T or tuple(weights.shape) != tuple(ids.shape):
+        raise RuntimeError("shape mismatch between logits, ids and weights")
+    st = _lib.load_library().hk_moe_topk_softmax(logits.data_ptr(), T, E, ids.shape[1], ids.data_ptr(),
+                                                 weights.data_ptr(), _stream(logits))
+    _lib.check(st, "dispatch_moe_topk_softmax")
+
+
+def dispatch_moe_topk_grouped_sigmoid(logits, bias, ids, weights, n_group: int, topk_group: int,
+                                      routed_scale: float = 1.0) -> None:
+    """Group-limited sigmoid routing; `bias` [E] fp32 or None."""
+    _check_tensor(logits, "logits", _F32, 2)
+    if bias is not None:
+        _check_tensor(bias, "bias", _F32, 1)
+    _check_tensor(ids, "ids", _I32, 2)
+    _check_tensor(weights, "weights", _F32, 2)
+    T, E = logits.shape
+    if ids.shape[0] != T or tuple(weights.shape) != tuple(ids.shape) or (bias is not None and bias.shape[0] != E):
+        raise RuntimeError("shape mismatch between logits, bias, ids and weights")
+    st = _lib.load_library().hk_moe_topk_grouped_sigmoid(
+        logits.data_ptr(), bias.data_ptr() if bias is not None else None, T, E, ids.shape[1],
+        int(n_group), int(topk_group), float(routed_scale), ids.data_ptr(), weights.data_ptr(),
+        _stream(logits))
+    _lib.check(st, "dispatch_moe_topk_grouped_sigmoid")
+
+
+def moe_sort_workspace_bytes(T: int, k: int, E: int) -> int:
+    return int(_lib.load_library().hk_moe_sort_workspace_bytes(T, k, E))
+
+
+def dispatch_moe_sort(ids, sorted_slots, expert_offsets, slot_to_pos, workspace) -> None:
+    """ids [T,k] int32 -> sorted_slots [T*k], expert_offsets [E+1], slot_to_pos [T*k] or None;
+    `workspace` is a uint8/int32 tensor of at least moe_sort_workspace_bytes(T, k, E) bytes."""
+    _check_tensor(ids, "ids", _I32, 2)
+    _check_tensor(sorted_slots, "sorted_slots", _I32, 1)
+    _check_tensor(expert_offsets, "expert_offsets", _I32, 1)
+    if slot_to_pos is not None:
+        _check_tensor(slot_to_pos, "slot_to_pos", _I32, 1)
+    _check_tensor(workspace, "workspace", (torch.uint8, torch.int32), 1)
+    T, k = ids.shape
+    E = expert_offsets.shape[0] - 1
+    if sorted_slots.shape[0] != T * k or (slot_to_pos is not None and slot_to_pos.shape[0] != T * k) or E <= 0:
+        raise RuntimeError("shape mismatch between ids, sorted_slots, expert_offsets and slot_to_pos")
+    st = _lib.load_library().hk_moe_sort(
+        ids.data_ptr(), T, k, E, sorted_slots.data_ptr(), expert_offsets.data_ptr(),
+        slot_to_pos.data_ptr() if slot_to_pos is not None else None, workspace.data_ptr(),
+        workspace.numel() * workspace.element_size(), _stream(ids))
+    _lib.check(st, "dispatch_moe_sort")

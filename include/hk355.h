@@ -76,6 +76,36 @@ int hk_mxfp4_gemm_variant(const void* A_e2m1, const void* A_scales_e8m0, const v
                           const void* B_scales_e8m0, void* C_bf16, int M, int N, int K,
                           int variant, void* stream);
 
+/* ------------------------------------------------------------------ MoE routing
+ * The reference has no MoE code; these entry points have no counterpart in it. They follow
+ * the same conventions as the GEMMs (caller-owned device buffers, asynchronous, status code).
+ * Integer outputs are deterministic: ties go to the lower expert id and the sort is stable.
+ */
+
+/* Top-k softmax routing. logits [T,E] fp32 -> ids [T,k] int32 (descending logit order) and
+ * w [T,k] fp32 = softmax over the k selected logits. Requirements: k <= 64, E <= 512. */
+int hk_moe_topk_softmax(const float* logits, int T, int E, int k, int32_t* ids, float* w,
+                        void* stream);
+
+/* Group-limited sigmoid routing (DeepSeek-V3 style). s = sigmoid(logit); selection score
+ * c = s + bias (bias [E] may be NULL); experts form n_group contiguous groups; a group's score
+ * is the sum of its two largest c; the topk_group best groups are kept; ids = top-k of c within
+ * kept groups; w = s[ids] / sum(s[ids]) * routed_scale.
+ * Requirements: E % n_group == 0, n_group <= 64, k <= topk_group * (E / n_group). */
+int hk_moe_topk_grouped_sigmoid(const float* logits, const float* bias_or_null, int T, int E,
+                                int k, int n_group, int topk_group, float routed_scale,
+                                int32_t* ids, float* w, void* stream);
+
+/* Stable sort of the T*k (token, choice) slots by expert id.
+ * sorted_slots [T*k]: slot indices t*k+j ordered by expert, ascending slot index inside an
+ * expert; expert_offsets [E+1]: exclusive prefix sum of per-expert counts; slot_to_pos [T*k]
+ * (optional): position of each slot in sorted_slots. workspace: hk_moe_sort_workspace_bytes().
+ * Requirements: E <= 512. */
+size_t hk_moe_sort_workspace_bytes(int T, int k, int E);
+int hk_moe_sort(const int32_t* ids, int T, int k, int E, int32_t* sorted_slots,
+                int32_t* expert_offsets, int32_t* slot_to_pos_or_null, void* workspace,
+                size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,81 @@
+"""CPU-only checks of the C-ABI boundary: the library loads, exports every symbol declared in
+include/hk355.h, and rejects bad arguments with the documented status codes before anything
+touches a GPU. The Python shim's checks mirror the reference's binding
+(include/pyutils/pyutils.cuh:14-47: Tensor, contiguous, not on the CPU) and raise RuntimeError."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import hipkittens_amd as hk
+from hipkittens_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "hk355.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = hk.load_library()
+    names = _declared_symbols()
+    assert "hk_fp8_gemm" in names and "hk_mxfp4_gemm" in names and "hk_moe_sort" in names
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/hk355.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert lib.hk_version() >= 100
+    assert lib.hk_status_string(0) == b"ok" and lib.hk_status_string(-2) == b"bad shape"
+
+
+def test_c_entry_points_reject_bad_arguments_without_a_gpu():
+    lib = hk.load_library()
+    buf = ctypes.create_string_buffer(4096 + 64)
+    p = (ctypes.addressof(buf) + 63) & ~63  # aligned host pointer; never dereferenced on this path
+    assert lib.hk_fp8_gemm(None, p, p, 256, 256, 256, 1.0, 1.0, None) == -1
+    assert lib.hk_fp8_gemm(p, p, p, 0, 256, 256, 1.0, 1.0, None) == -2
+    assert lib.hk_fp8_gemm(p, p, p, 256, 256, 250, 1.0, 1.0, None) == -2      # K % 16
+    assert lib.hk_fp8_gemm(p + 1, p, p, 256, 256, 256, 1.0, 1.0, None) == -3
+    assert lib.hk_fp8_gemm_variant(p, p, p, 256, 256, 272, 1.0, 1.0, 2, None) == -2  # K % 128 for tile kernels
+    assert lib.hk_fp8_gemm_variant(p, p, p, 256, 256, 256, 1.0, 1.0, 9, None) == -6
+    assert lib.hk_mxfp4_gemm(p, None, p, p, p, 64, 64, 64, None) == -1
+    assert lib.hk_mxfp4_gemm(p, p, p, p, p, 64, 64, 48, None) == -2           # K % 32
+    assert lib.hk_mxfp4_gemm_variant(p, p, p, p, p, 64, 64, 64, 1, None) == -2  # K % 256 for the tile kernel
+    assert lib.hk_moe_topk_softmax(p, 4, 1024, 2, p, p, None) == -2           # E > 512
+    assert lib.hk_moe_topk_softmax(p, 4, 16, 17, p, p, None) == -2            # k > E
+    assert lib.hk_moe_topk_grouped_sigmoid(p, None, 4, 30, 2, 4, 2, 1.0, p, p, None) == -2
+    assert lib.hk_moe_sort(p, 4, 2, 8, p, p, None, None, 0, None) == -4       # no workspace
+    assert lib.hk_moe_sort(p, 4, 2, 8, p, p, None, p, 4, None) == -4          # workspace too small
+    assert lib.hk_moe_sort_workspace_bytes(4096, 4, 128) == 16 * 128 * 4
+
+
+def test_python_boundary_rejects_like_the_reference():
+    A = torch.zeros((256, 256), dtype=torch.uint8)
+    C = torch.zeros((256, 256), dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        hk.tk_kernel.dispatch_fp8_gemm(A, A, C)                 # CPU tensors
+    with pytest.raises(RuntimeError, match="contiguous"):
+        hk.tk_kernel.dispatch_fp8_gemm(A.t(), A, C)
+    with pytest.raises(RuntimeError, match="Tensor"):
+        hk.tk_kernel.dispatch_fp8_gemm([1, 2], A, C)
+    with pytest.raises(RuntimeError, match="GPU"):
+        hk.tk_kernel.dispatch_micro(A, A, C)
+
+
+def test_device_independent_quantizers_match_oracle_on_cpu():
+    import numpy as np
+
+    from oracle import formats as F
+
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal((64, 256)) * np.exp2(rng.integers(-10, 10, size=(64, 1)))).astype(np.float32)
+    p, s = hk.quant.quantize_mxfp4(torch.from_numpy(x))
+    po, so = F.quantize_mxfp4(x)
+    assert np.array_equal(p.numpy(), po) and np.array_equal(s.numpy(), so)
+    q, sc = hk.quant.quantize_fp8_per_tensor(torch.from_numpy(x))
+    qo, sco = F.quantize_e4m3_per_tensor(x)
+    assert np.float32(sc) == sco and np.array_equal(q.view(torch.uint8).numpy(), qo)

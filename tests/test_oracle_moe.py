@@ -1,0 +1,128 @@
+"""Pin the MoE oracle (CPU only): brute force on small inputs, library routines, invariants."""
+import math
+
+import numpy as np
+import torch
+
+from oracle import formats as F
+from oracle import moe as O
+
+
+def test_sigmoid_f32_close_to_libm_and_monotone():
+    x = np.linspace(-30, 30, 20001).astype(np.float32)
+    s = O.sigmoid_f32(x)
+    ref = 1.0 / (1.0 + np.exp(-x.astype(np.float64)))
+    assert np.max(np.abs(s - ref) / ref) < 5e-7
+    assert np.all(np.diff(s) >= 0)
+    assert O.sigmoid_f32(np.array([0.0], np.float32))[0] == 0.5
+
+
+def test_topk_softmax_brute_force():
+    rng = np.random.default_rng(0)
+    logits = rng.standard_normal((37, 16)).astype(np.float32)
+    logits[3, 5] = logits[3, 2]          # exact tie -> lower id first
+    logits[4, :] = 0.25                   # all equal -> ids 0..k-1
+    ids, w = O.topk_softmax(logits, 4)
+    for t in range(logits.shape[0]):
+        order = sorted(range(16), key=lambda e: (-float(logits[t, e]), e))[:4]
+        assert list(ids[t]) == order
+        ex = [math.exp(float(logits[t, e]) - float(logits[t, order[0]])) for e in order]
+        assert np.allclose(w[t], np.array(ex) / sum(ex), rtol=1e-6)
+    assert list(ids[4]) == [0, 1, 2, 3]
+    assert list(ids[3]).index(2) < list(ids[3]).index(5) if 5 in ids[3] and 2 in ids[3] else True
+    # library cross-check: torch.topk values agree
+    tv, _ = torch.topk(torch.from_numpy(logits), 4, dim=-1)
+    assert np.array_equal(np.take_along_axis(logits, ids, axis=-1), tv.numpy())
+
+
+def test_grouped_sigmoid_brute_force():
+    rng = np.random.default_rng(1)
+    T, E, G, KG, K = 29, 32, 8, 3, 6
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    bias = (rng.standard_normal(E) * 0.1).astype(np.float32)
+    for b in (None, bias):
+        ids, w = O.topk_grouped_sigmoid(logits, b, K, G, KG, routed_scale=2.5)
+        s = O.sigmoid_f32(logits)
+        c = s if b is None else (s + b[None, :]).astype(np.float32)
+        gs = E // G
+        for t in range(T):
+            gscore = []
+            for g in range(G):
+                v = sorted((float(x) for x in c[t, g * gs:(g + 1) * gs]), reverse=True)
+                gscore.append(float(np.float32(np.float32(v[0]) + np.float32(v[1]))))
+            keep = sorted(range(G), key=lambda g: (-gscore[g], g))[:KG]
+            cand = [e for e in range(E) if e // gs in keep]
+            want = sorted(cand, key=lambda e: (-float(c[t, e]), e))[:K]
+            assert list(ids[t]) == want
+            sel = s[t, want]
+            tot = np.float32(0)
+            for v in sel:
+                tot = np.float32(tot + v)
+            assert np.array_equal(w[t], (sel / tot).astype(np.float32) * np.float32(2.5))
+            assert abs(float(w[t].sum()) - 2.5) < 1e-5
+
+
+def test_moe_sort_invariants_and_library():
+    rng = np.random.default_rng(2)
+    T, k, E = 257, 4, 16
+    ids = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    order, offs, inv = O.moe_sort(ids, E)
+    flat = ids.reshape(-1)
+    assert sorted(order.tolist()) == list(range(T * k))
+    assert offs[0] == 0 and offs[-1] == T * k and np.all(np.diff(offs) >= 0)
+    for e in range(E):
+        seg = order[offs[e]:offs[e + 1]]
+        assert np.all(flat[seg] == e) and np.all(np.diff(seg) > 0)
+    assert np.array_equal(order[inv], np.arange(T * k))
+    ts = torch.sort(torch.from_numpy(flat.astype(np.int64)), stable=True).indices.numpy()
+    assert np.array_equal(order, ts.astype(np.int32))
+    # an expert nobody chose gets an empty range
+    ids2 = np.zeros((5, 1), dtype=np.int32)
+    _, offs2, _ = O.moe_sort(ids2, 3)
+    assert list(offs2) == [0, 5, 5, 5]
+
+
+def test_moe_mxfp4_forward_single_expert_reduces_to_two_gemms():
+    """E = 1, k = 1, w = 1: the MoE is quantize -> GEMM -> SiLU-mul -> quantize -> GEMM."""
+    rng = np.random.default_rng(3)
+    T, H, I = 8, 64, 32
+    x = F.bf16_to_f32(F.bf16_round(rng.standard_normal((T, H)).astype(np.float32)))
+    w13 = (rng.standard_normal((1, 2 * I, H)) * 0.2).astype(np.float32)
+    w2 = (rng.standard_normal((1, H, I)) * 0.2).astype(np.float32)
+    w13p, w13s = F.quantize_mxfp4(w13)
+    w2p, w2s = F.quantize_mxfp4(w2)
+    ids = np.zeros((T, 1), dtype=np.int32)
+    w = np.ones((T, 1), dtype=np.float32)
+    y, _ = O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s)
+    xd = F.dequantize_mxfp4(*F.quantize_mxfp4(x))
+    gu = xd @ F.dequantize_mxfp4(w13p[0], w13s[0]).T
+    g, u = gu[:, :I].astype(np.float64), gu[:, I:]
+    h = (g / (1 + np.exp(-g)) * u).astype(np.float32)
+    hd = F.dequantize_mxfp4(*F.quantize_mxfp4(h))
+    o = hd @ F.dequantize_mxfp4(w2p[0], w2s[0]).T
+    want = F.bf16_round(F.bf16_to_f32(F.bf16_round(o)))
+    assert np.array_equal(y, want)
+
+
+def test_moe_mxfp4_forward_brute_force_tiny():
+    """T=8, E=4, k=2, H=64, I=32: loop over tokens and choices instead of experts."""
+    rng = np.random.default_rng(4)
+    T, E, k, H, I = 8, 4, 2, 64, 32
+    x = F.bf16_to_f32(F.bf16_round(rng.standard_normal((T, H)).astype(np.float32)))
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    ids, w = O.topk_softmax(logits, k)
+    w13p, w13s = F.quantize_mxfp4((rng.standard_normal((E, 2 * I, H)) * 0.2).astype(np.float32))
+    w2p, w2s = F.quantize_mxfp4((rng.standard_normal((E, H, I)) * 0.2).astype(np.float32))
+    y, _ = O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s)
+    xd = F.dequantize_mxfp4(*F.quantize_mxfp4(x))
+    want = np.zeros((T, H), dtype=np.float32)
+    for j in range(k):
+        for t in range(T):
+            e = ids[t, j]
+            gu = xd[t:t + 1] @ F.dequantize_mxfp4(w13p[e], w13s[e]).T
+            h = (O.silu(gu[:, :I]) * gu[:, I:]).astype(np.float32)
+            hd = F.dequantize_mxfp4(*F.quantize_mxfp4(h))
+            o = F.bf16_to_f32(F.bf16_round(hd @ F.dequantize_mxfp4(w2p[e], w2s[e]).T))
+            want[t] += w[t, j] * o[0]
+    got = F.bf16_to_f32(y)
+    assert np.allclose(got, F.bf16_to_f32(F.bf16_round(want)), rtol=2e-2, atol=1e-6)
