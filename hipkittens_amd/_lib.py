@@ -22,6 +22,14 @@ SIGNATURES = {
     "hk_moe_sort_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "hk_moe_sort": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                             c_void_p]),
+    "hk_mxfp4_quantize_rows": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
+    "hk_moe_unpermute": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "hk_moe_mxfp4_workspace_bytes": (c_size_t, [c_int] * 5),
+    "hk_moe_mxfp4_experts": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p,
+                                     c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                     c_void_p, c_size_t, c_void_p]),
+    "hk_moe_mxfp4_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int,
+                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
 }
 
 

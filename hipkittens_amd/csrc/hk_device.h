@@ -53,6 +53,17 @@ __device__ __forceinline__ void dma16(v4i srd, uint32_t lds_base, uint32_t voff,
         : "memory", "m0");
 }
 
+// 4-byte direct global->LDS load (64 lanes -> 256 contiguous LDS bytes).
+__device__ __forceinline__ void dma4(v4i srd, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dword %1, %2, %3 offen lds"
+        :
+        : "s"(lds_base), "v"(voff), "s"(srd), "s"(soff)
+        : "memory", "m0");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");

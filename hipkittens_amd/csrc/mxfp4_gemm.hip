@@ -37,17 +37,6 @@ __device__ __forceinline__ Frag4 lds_frag4(uint32_t addr_lo, uint32_t addr_hi, i
     return f;
 }
 
-// 4-byte direct global->LDS load (64 lanes -> 256 contiguous LDS bytes).
-__device__ __forceinline__ void dma4(v4i srd, uint32_t lds_base, uint32_t voff, uint32_t soff) {
-    asm volatile(
-        "s_mov_b32 m0, %0\n\t"
-        "s_nop 0\n\t"
-        "buffer_load_dword %1, %2, %3 offen lds"
-        :
-        : "s"(lds_base), "v"(voff), "s"(srd), "s"(soff)
-        : "memory", "m0");
-}
-
 // acc(16x16) += X(16x128 e2m1, scale sx) * Y(16x128 e2m1, scale sy)^T, accumulator tied in
 // an AGPR; sx / sy carry the lane's e8m0 byte in bits [7:0].
 __device__ __forceinline__ void mfma_fp4_acc(v4f& acc, const v4i& x, const v4i& y, int sx, int sy) {

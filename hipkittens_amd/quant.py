@@ -45,3 +45,14 @@ def quantize_mxfp4(x: torch.Tensor):
     code = code.reshape(*x.shape[:-1], K)
     packed = code[..., 0::2] | (code[..., 1::2] << 4)
     return packed.contiguous(), (e + 127).to(torch.uint8).contiguous()
+
+
+def pad_scales(scales: torch.Tensor, multiple: int = 8) -> torch.Tensor:
+    """Pad the last dim of an e8m0 scale tensor to a multiple of `multiple` with the neutral byte
+    127 (the row pitch the MoE kernels load scales with)."""
+    n = scales.shape[-1]
+    pad = (-n) % multiple
+    if pad == 0:
+        return scales.contiguous()
+    fill = torch.full((*scales.shape[:-1], pad), 127, dtype=scales.dtype, device=scales.device)
+    return torch.cat([scales, fill], dim=-1).contiguous()

@@ -156,3 +156,90 @@ def dispatch_moe_sort(ids, sorted_slots, expert_offsets, slot_to_pos, workspace)
         slot_to_pos.data_ptr() if slot_to_pos is not None else None, workspace.data_ptr(),
         workspace.numel() * workspace.element_size(), _stream(ids))
     _lib.check(st, "dispatch_moe_sort")
+
+
+# ---------------------------------------------------------------------------- MXFP4 fused MoE
+_BF16 = (torch.bfloat16,)
+
+
+def dispatch_mxfp4_quantize_rows(x, packed, scales) -> None:
+    """x [R,C] bf16 -> packed [R,C/2] uint8, scales [R,pitch] uint8 (pitch >= C/32, multiple of 8)."""
+    _check_tensor(x, "x", _BF16, 2)
+    _check_tensor(packed, "packed", _FP4, 2)
+    _check_tensor(scales, "scales", _E8M0, 2)
+    R, C = x.shape
+    if tuple(packed.shape) != (R, C // 2) or scales.shape[0] != R:
+        raise RuntimeError("shape mismatch between x, packed and scales")
+    st = _lib.load_library().hk_mxfp4_quantize_rows(x.data_ptr(), R, C, packed.data_ptr(), scales.data_ptr(),
+                                                    scales.shape[1], _stream(x))
+    _lib.check(st, "dispatch_mxfp4_quantize_rows")
+
+
+def dispatch_moe_unpermute(o, weights, slot_to_pos, y) -> None:
+    """y [T,H] bf16 = sum_j weights[t,j] * o[slot_to_pos[t*k+j]] with o [T*k,H] bf16."""
+    _check_tensor(o, "o", _BF16, 2)
+    _check_tensor(weights, "weights", _F32, 2)
+    _check_tensor(slot_to_pos, "slot_to_pos", _I32, 1)
+    _check_tensor(y, "y", _BF16, 2)
+    T, k = weights.shape
+    H = y.shape[1]
+    if tuple(o.shape) != (T * k, H) or y.shape[0] != T or slot_to_pos.shape[0] != T * k:
+        raise RuntimeError("shape mismatch between o, weights, slot_to_pos and y")
+    st = _lib.load_library().hk_moe_unpermute(o.data_ptr(), weights.data_ptr(), slot_to_pos.data_ptr(), T, k, H,
+                                              y.data_ptr(), _stream(o))
+    _lib.check(st, "dispatch_moe_unpermute")
+
+
+def moe_mxfp4_workspace_bytes(T: int, H: int, I: int, E: int, k: int) -> int:
+    return int(_lib.load_library().hk_moe_mxfp4_workspace_bytes(T, H, I, E, k))
+
+
+def _check_moe_weights(x, w13, w13_scales, w2, w2_scales, y):
+    _check_tensor(x, "x", _BF16, 2)
+    _check_tensor(w13, "w13", _FP4, 3)
+    _check_tensor(w13_scales, "w13_scales", _E8M0, 3)
+    _check_tensor(w2, "w2", _FP4, 3)
+    _check_tensor(w2_scales, "w2_scales", _E8M0, 3)
+    _check_tensor(y, "y", _BF16, 2)
+    T, H = x.shape
+    E, twoI, Hh = w13.shape
+    I = twoI // 2
+    if Hh * 2 != H or tuple(w2.shape) != (E, H, I // 2) or tuple(y.shape) != (T, H) or \
+            tuple(w13_scales.shape[:2]) != (E, twoI) or tuple(w2_scales.shape[:2]) != (E, H):
+        raise RuntimeError("shape mismatch between x, w13, w13_scales, w2, w2_scales and y")
+    return T, H, I, E
+
+
+def dispatch_moe_mxfp4_experts(x, w13, w13_scales, w2, w2_scales, weights, sorted_slots, expert_offsets,
+                               slot_to_pos, y, workspace) -> None:
+    """Expert MLP on routed + sorted tokens (see include/hk355.h: hk_moe_mxfp4_experts)."""
+    T, H, I, E = _check_moe_weights(x, w13, w13_scales, w2, w2_scales, y)
+    _check_tensor(weights, "weights", _F32, 2)
+    _check_tensor(sorted_slots, "sorted_slots", _I32, 1)
+    _check_tensor(expert_offsets, "expert_offsets", _I32, 1)
+    _check_tensor(slot_to_pos, "slot_to_pos", _I32, 1)
+    _check_tensor(workspace, "workspace", (torch.uint8,), 1)
+    k = weights.shape[1]
+    if weights.shape[0] != T or sorted_slots.shape[0] != T * k or expert_offsets.shape[0] != E + 1 or \
+            slot_to_pos.shape[0] != T * k:
+        raise RuntimeError("shape mismatch between routing tensors")
+    st = _lib.load_library().hk_moe_mxfp4_experts(
+        x.data_ptr(), w13.data_ptr(), w13_scales.data_ptr(), w13_scales.shape[2], w2.data_ptr(),
+        w2_scales.data_ptr(), w2_scales.shape[2], weights.data_ptr(), sorted_slots.data_ptr(),
+        expert_offsets.data_ptr(), slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, workspace.data_ptr(),
+        workspace.numel(), _stream(x))
+    _lib.check(st, "dispatch_moe_mxfp4_experts")
+
+
+def dispatch_moe_mxfp4(x, router_logits, w13, w13_scales, w2, w2_scales, y, topk: int, workspace) -> None:
+    """Whole MXFP4 MoE layer: top-k softmax routing, sort, expert MLP, un-permute into y."""
+    T, H, I, E = _check_moe_weights(x, w13, w13_scales, w2, w2_scales, y)
+    _check_tensor(router_logits, "router_logits", _F32, 2)
+    _check_tensor(workspace, "workspace", (torch.uint8,), 1)
+    if tuple(router_logits.shape) != (T, E):
+        raise RuntimeError("router_logits must be [T, E]")
+    st = _lib.load_library().hk_moe_mxfp4_forward(
+        x.data_ptr(), router_logits.data_ptr(), w13.data_ptr(), w13_scales.data_ptr(), w13_scales.shape[2],
+        w2.data_ptr(), w2_scales.data_ptr(), w2_scales.shape[2], y.data_ptr(), T, H, I, E, int(topk),
+        workspace.data_ptr(), workspace.numel(), _stream(x))
+    _lib.check(st, "dispatch_moe_mxfp4")

@@ -106,6 +106,48 @@ int hk_moe_sort(const int32_t* ids, int T, int k, int E, int32_t* sorted_slots,
                 int32_t* expert_offsets, int32_t* slot_to_pos_or_null, void* workspace,
                 size_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------ MXFP4 fused MoE
+ * No counterpart in the reference. Tensors (all row-major, caller owned):
+ *   x            [T, H]  bf16 activations
+ *   w13          [E, 2I, H/2] packed e2m1; rows 0..I-1 = gate projection, I..2I-1 = up projection
+ *   w13_scales   [E, 2I, w13_scale_pitch] e8m0, one per 32 elements of H; the pitch is >= H/32
+ *                and a multiple of 8, padding bytes must not be 0xFF (use 127)
+ *   w2           [E, H, I/2] packed e2m1, w2_scales [E, H, w2_scale_pitch] likewise over I
+ *   y            [T, H]  bf16
+ * Per token t and choice j with expert e = ids[t,j]:
+ *   h = silu(xq W13g[e]^T) * (xq W13u[e]^T),  o = hq W2[e]^T,  y[t] = sum_j w[t,j] * bf16(o)
+ * where xq / hq are the activations re-quantized to MXFP4 (blocks of 32 along H / I, OCP MX
+ * rule: shared exponent floor(log2(amax)) - 2), so every GEMM runs on the FP4 MFMA path.
+ * Requirements: H % 32 == 0, I % 32 == 0, E <= 512, k <= 64.
+ */
+
+/* bf16 [rows, cols] -> packed e2m1 [rows, cols/2] + e8m0 scales [rows, scale_pitch]
+ * (scale_pitch >= cols/32, multiple of 8; padding columns are written as 127). */
+int hk_mxfp4_quantize_rows(const void* x_bf16, int rows, int cols, void* packed, void* scales,
+                           int scale_pitch, void* stream);
+
+/* y[t,:] = bf16(sum_j w[t,j] * o[slot_to_pos[t*k+j], :]), o [T*k, H] bf16. H % 8 == 0. */
+int hk_moe_unpermute(const void* o_bf16, const float* w, const int32_t* slot_to_pos, int T, int k,
+                     int H, void* y_bf16, void* stream);
+
+size_t hk_moe_mxfp4_workspace_bytes(int T, int H, int I, int E, int k);
+
+/* Expert MLP for tokens that are already routed and sorted (outputs of hk_moe_topk_* and
+ * hk_moe_sort): activation quantization, grouped gate+up GEMM with SiLU-mul and MX
+ * re-quantization, grouped down GEMM, weighted un-permute. */
+int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const void* w13_scales,
+                         int w13_scale_pitch, const void* w2, const void* w2_scales,
+                         int w2_scale_pitch, const float* topk_w, const int32_t* sorted_slots,
+                         const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
+                         int T, int H, int I, int E, int k, void* workspace, size_t workspace_bytes,
+                         void* stream);
+
+/* Whole layer: top-k softmax routing of router_logits [T,E] fp32, sort, expert MLP. */
+int hk_moe_mxfp4_forward(const void* x_bf16, const float* router_logits, const void* w13,
+                         const void* w13_scales, int w13_scale_pitch, const void* w2,
+                         const void* w2_scales, int w2_scale_pitch, void* y_bf16, int T, int H, int I,
+                         int E, int k, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

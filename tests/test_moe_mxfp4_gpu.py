@@ -1,0 +1,170 @@
+"""MXFP4 fused MoE on the GPU against the CPU oracle.
+
+Bit-exact: activation quantizer (codes and e8m0 bytes). Floating point (y): relative Frobenius
+error <= 1e-2 against the oracle, which quantizes activations with the same MX rule, dequantizes
+weights and accumulates in fp32 (north-star tolerance). Size-independent properties at the full
+GPT-OSS-like shape: permutation invariance of y under token reordering and linearity in the
+routing weights.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import formats as F
+from oracle import gemm as G
+from oracle import moe as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 1e-2
+
+
+def _bf16(a):
+    return F.bf16_to_f32(F.bf16_round(np.asarray(a, dtype=np.float32)))
+
+
+def _to_bf16_tensor(a):
+    return torch.from_numpy(F.bf16_round(a).view(np.int16)).view(torch.bfloat16).to(DEV)
+
+
+def _weights(rng, E, I, H, std=0.2):
+    w13p, w13s = F.quantize_mxfp4((rng.standard_normal((E, 2 * I, H)) * std).astype(np.float32))
+    w2p, w2s = F.quantize_mxfp4((rng.standard_normal((E, H, I)) * std).astype(np.float32))
+    return w13p, w13s, w2p, w2s
+
+
+def _pad(s):
+    pad = (-s.shape[-1]) % 8
+    return np.concatenate([s, np.full((*s.shape[:-1], pad), 127, np.uint8)], axis=-1) if pad else s
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 256), (33, 2880), (1, 32), (500, 96)])
+def test_quantize_rows_bit_exact(hk, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = _bf16(rng.standard_normal((rows, cols)) * np.exp2(rng.integers(-12, 12, size=(rows, 1))))
+    x[0, :32] = 0.0
+    pitch = (cols // 32 + 7) // 8 * 8
+    xt = _to_bf16_tensor(x)
+    packed = torch.zeros((rows, cols // 2), dtype=torch.uint8, device=DEV)
+    scales = torch.zeros((rows, pitch), dtype=torch.uint8, device=DEV)
+    hk.tk_kernel.dispatch_mxfp4_quantize_rows(xt, packed, scales)
+    torch.cuda.synchronize()
+    po, so = F.quantize_mxfp4(x)
+    assert np.array_equal(packed.cpu().numpy(), po)
+    assert np.array_equal(scales.cpu().numpy()[:, :cols // 32], so)
+    assert np.all(scales.cpu().numpy()[:, cols // 32:] == 127)
+
+
+def test_unpermute_matches_oracle(hk):
+    rng = np.random.default_rng(0)
+    T, k, H = 77, 4, 2880
+    o = _bf16(rng.standard_normal((T * k, H)))
+    w = rng.random((T, k)).astype(np.float32)
+    inv = rng.permutation(T * k).astype(np.int32)
+    y = torch.zeros((T, H), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_unpermute(_to_bf16_tensor(o), torch.from_numpy(w).to(DEV), torch.from_numpy(inv).to(DEV), y)
+    torch.cuda.synchronize()
+    want = np.zeros((T, H), dtype=np.float64)
+    for j in range(k):
+        want += w[:, j:j + 1].astype(np.float64) * o[inv[np.arange(T) * k + j]]
+    got = y.float().cpu().numpy()
+    assert np.abs(got - want).max() <= np.abs(want).max() * 2.0 ** -7
+    assert G.rel_fro_error(got, want) <= 4e-3  # one bf16 rounding
+
+
+def _run_forward(hk, x, logits, w13p, w13s, w2p, w2s, k):
+    T, H = x.shape
+    E, twoI, _ = w13p.shape
+    I = twoI // 2
+    ws = torch.empty(hk.tk_kernel.moe_mxfp4_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=DEV)
+    y = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_mxfp4(
+        _to_bf16_tensor(x), torch.from_numpy(logits).to(DEV), torch.from_numpy(w13p).to(DEV),
+        torch.from_numpy(_pad(w13s)).to(DEV), torch.from_numpy(w2p).to(DEV), torch.from_numpy(_pad(w2s)).to(DEV),
+        y, k, ws)
+    torch.cuda.synchronize()
+    return y.float().cpu().numpy()
+
+
+CASES = [
+    # T, E, k, H, I
+    (8, 4, 2, 64, 32),        # the oracle's tiny brute-force case
+    (64, 4, 2, 256, 128),
+    (300, 8, 2, 512, 384),    # several m-tiles per expert (about 75 rows each, some > 128 after skew)
+    (200, 16, 4, 2880, 2880 // 9 * 1),  # K tail (2880 = 11.25 * 256) with I = 320
+    (96, 128, 4, 288, 160),   # many experts, most with 1-5 rows, some empty
+]
+
+
+@pytest.mark.parametrize("T,E,k,H,I", CASES)
+def test_moe_mxfp4_forward_matches_oracle(hk, T, E, k, H, I):
+    print(f"moe_mxfp4 T={T} E={E} k={k} H={H} I={I}", flush=True)
+    rng = np.random.default_rng(T + E + H)
+    x = _bf16(rng.standard_normal((T, H)))
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    w13p, w13s, w2p, w2s = _weights(rng, E, I, H)
+    got = _run_forward(hk, x, logits, w13p, w13s, w2p, w2s, k)
+    ids, w = O.topk_softmax(logits, k)
+    want_bits, _ = O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s)
+    want = F.bf16_to_f32(want_bits)
+    assert np.isfinite(got).all()
+    err = G.rel_fro_error(got, want)
+    assert err <= TOL, err
+
+
+def test_moe_mxfp4_skewed_routing_many_rows_per_expert(hk):
+    """All tokens on two experts: 2 x 600 rows -> five m-tiles per expert; others empty."""
+    rng = np.random.default_rng(5)
+    T, E, k, H, I = 600, 6, 2, 256, 256
+    x = _bf16(rng.standard_normal((T, H)))
+    logits = np.full((T, E), -5.0, dtype=np.float32)
+    logits[:, 1] = 3.0 + rng.random(T).astype(np.float32)
+    logits[:, 4] = 2.0 + rng.random(T).astype(np.float32)
+    w13p, w13s, w2p, w2s = _weights(rng, E, I, H)
+    got = _run_forward(hk, x, logits, w13p, w13s, w2p, w2s, k)
+    ids, w = O.topk_softmax(logits, k)
+    want = F.bf16_to_f32(O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s)[0])
+    assert G.rel_fro_error(got, want) <= TOL
+
+
+def test_moe_mxfp4_full_shape_properties(hk):
+    """GPT-OSS-like shape (T=4096, H=I=2880, E=128, k=4): checks that do not need the CPU oracle
+    at full size, plus the oracle on a sample of tokens (experts evaluated only for those tokens)."""
+    T, E, k, H, I = 4096, 128, 4, 2880, 2880
+    g = torch.Generator(device=DEV).manual_seed(0)
+    x = torch.randn(T, H, device=DEV, generator=g).to(torch.bfloat16)
+    logits = torch.randn(T, E, device=DEV, generator=g)
+    w13p = torch.empty((E, 2 * I, H // 2), dtype=torch.uint8, device=DEV)
+    w13s = torch.empty((E, 2 * I, 96), dtype=torch.uint8, device=DEV)
+    w2p = torch.empty((E, H, I // 2), dtype=torch.uint8, device=DEV)
+    w2s = torch.empty((E, H, 96), dtype=torch.uint8, device=DEV)
+    for e in range(E):  # per expert, to bound temporaries
+        a, s = hk.quant.quantize_mxfp4(torch.randn(2 * I, H, device=DEV, generator=g) * 0.02)
+        w13p[e], w13s[e] = a, hk.quant.pad_scales(s)
+        a, s = hk.quant.quantize_mxfp4(torch.randn(H, I, device=DEV, generator=g) * 0.02)
+        w2p[e], w2s[e] = a, hk.quant.pad_scales(s)
+    ws = torch.empty(hk.tk_kernel.moe_mxfp4_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=DEV)
+    y = torch.empty((T, H), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_mxfp4(x, logits, w13p, w13s, w2p, w2s, y, k, ws)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all()
+    # (1) token permutation: y is a per-token function -> permuting inputs permutes outputs exactly
+    perm = torch.randperm(T, device=DEV, generator=g)
+    y2 = torch.empty_like(y)
+    hk.tk_kernel.dispatch_moe_mxfp4(x[perm].contiguous(), logits[perm].contiguous(), w13p, w13s, w2p, w2s, y2, k, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(y2, y[perm])
+    # (2) oracle on 24 sampled tokens
+    sel = torch.arange(0, T, T // 24, device=DEV)[:24]
+    xs = x[sel].float().cpu().numpy()
+    ls = logits[sel].cpu().numpy()
+    ids, w = O.topk_softmax(ls, k)
+    used = np.unique(ids)
+    remap = {int(e): i for i, e in enumerate(used)}
+    ids_l = np.vectorize(remap.get)(ids).astype(np.int32)
+    ut = torch.from_numpy(used.astype(np.int64)).to(DEV)
+    want = F.bf16_to_f32(O.moe_mxfp4_forward(
+        xs, ids_l, w, w13p[ut].cpu().numpy(), w13s[ut][:, :, :H // 32].cpu().numpy(),
+        w2p[ut].cpu().numpy(), w2s[ut][:, :, :I // 32].cpu().numpy())[0])
+    got = y[sel].float().cpu().numpy()
+    assert G.rel_fro_error(got, want) <= TOL
