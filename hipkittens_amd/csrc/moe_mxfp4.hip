@@ -6,12 +6,14 @@
 // tiles, ds_read_b128 fragments, v_mfma_scale_f32_16x16x128_f8f6f4 with in-MFMA e8m0 scales).
 //
 // Grouped GEMM: a work item is (m-tile, n-tile) where an m-tile is up to 128 consecutive rows
-// (sorted positions) of one expert; the m-tile list is built on the device from
-// expert_offsets. Each workgroup (4 waves, one per SIMD) computes a 128 x 256 tile; every wave
-// spans all 128 rows and owns 64 of the 256 weight rows, so that 16-row fragments beyond the
-// tile's real row count are skipped by all waves alike. Weights dominate HBM traffic at MoE
-// shapes (about 128 rows per expert), so the K loop runs a three-stage LDS ring: two K-steps
-// of operands are always in flight.
+// (sorted positions) of one expert; the item list is built on the device from
+// expert_offsets. A workgroup (4 waves, one per SIMD) computes a 128 x 256 tile per item; every
+// wave spans all 128 rows and owns 64 of the 256 weight rows, so that 16-row fragments beyond
+// the tile's real row count are skipped by all waves alike. Weights dominate HBM traffic at MoE
+// shapes (about 128 rows per expert), so the K loop runs a three-stage LDS ring (two K-steps of
+// operands always in flight) and workgroups are persistent: each walks a contiguous range of
+// items and the ring keeps running across item boundaries, so the next item's first K-steps
+// load while the current item's epilogue runs.
 #include "gemm_tile.h"
 #include "../../include/hk355.h"
 
@@ -76,36 +78,84 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_rows_kernel(const uint16_t
     if ((c8 & 3) == 0) scales[(size_t)row * scale_pitch + (c8 >> 2)] = (uint8_t)(e + 127);
 }
 
-// ------------------------------------------------------------------------------ tile list
-// m-tiles of up to kMoeBM rows, experts in order. tile_info[3*i] = {expert, first row, rows}.
-constexpr int kMoeBM = 128;
-
-__global__ __launch_bounds__(64) void moe_build_tiles_kernel(const int32_t* __restrict__ expert_offsets,
-                                                             int E, int32_t* __restrict__ tile_info,
-                                                             int32_t* __restrict__ num_tiles) {
-    if (threadIdx.x != 0) return;
-    int n = 0;
-    for (int e = 0; e < E; ++e) {
-        const int lo = expert_offsets[e], hi = expert_offsets[e + 1];
-        for (int r = lo; r < hi; r += kMoeBM) {
-            tile_info[3 * n + 0] = e;
-            tile_info[3 * n + 1] = r;
-            tile_info[3 * n + 2] = min(kMoeBM, hi - r);
-            ++n;
+// Quantize-and-permute: row `pos` of the output is token sorted_slots[pos] / topk of x, so
+// that each expert's rows are contiguous for the grouped GEMM (the "permute" step of the MoE).
+__global__ __launch_bounds__(256) void mxfp4_quantize_permute_kernel(
+    const uint16_t* __restrict__ x, const int32_t* __restrict__ sorted_slots, int topk, int S, int cols,
+    uint8_t* __restrict__ packed, uint8_t* __restrict__ scales, int scale_pitch) {
+    const int per_row = scale_pitch * 4;
+    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+    const int pos = (int)(gid / per_row);
+    const int c8 = (int)(gid % per_row);
+    if (pos >= S) return;
+    const int row = sorted_slots[pos] / topk;
+    float v[8];
+    const bool in = c8 * 8 < cols;
+    if (in) {
+        const v4i raw = *(const v4i*)(x + (size_t)row * cols + c8 * 8);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __uint_as_float((uint32_t)raw[i] << 16);
+            v[2 * i + 1] = __uint_as_float((uint32_t)raw[i] & 0xffff0000u);
         }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = 0.f;
     }
-    *num_tiles = n;
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+    const int e = mx_block_exponent(amax);
+    if (in) *(uint32_t*)(packed + (size_t)pos * (cols / 2) + c8 * 4) = pack8_e2m1(v, e);
+    if ((c8 & 3) == 0) scales[(size_t)pos * scale_pitch + (c8 >> 2)] = (uint8_t)(e + 127);
+}
+
+// ------------------------------------------------------------------------------ work items
+// A work item is (m-tile, n-tile): up to kMoeBM consecutive sorted rows of one expert times one
+// tile of weight rows. Items are listed expert by expert, n-tile by n-tile, the m-tiles of one
+// (expert, n-tile) next to each other, so that a workgroup walking a contiguous range re-reads a
+// weight tile for the expert's second m-tile straight from its XCD's L2.
+constexpr int kMoeBM = 128;
+struct MoeItem { int expert, row_start, rows, n_tile; };
+
+__global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __restrict__ expert_offsets,
+                                                              int E, int n_tiles_n, MoeItem* __restrict__ items,
+                                                              int32_t* __restrict__ num_items) {
+    __shared__ int scan[512];
+    const int e = threadIdx.x;
+    int lo = 0, hi = 0, cnt = 0;
+    if (e < E) {
+        lo = expert_offsets[e]; hi = expert_offsets[e + 1];
+        cnt = (hi - lo + kMoeBM - 1) / kMoeBM;
+    }
+    scan[e] = cnt * n_tiles_n;
+    __syncthreads();
+    for (int d = 1; d < 512; d <<= 1) {
+        const int v = e >= d ? scan[e - d] : 0;
+        __syncthreads();
+        scan[e] += v;
+        __syncthreads();
+    }
+    const int base = scan[e] - cnt * n_tiles_n;
+    for (int n = 0; n < n_tiles_n; ++n)
+        for (int m = 0; m < cnt; ++m) {
+            MoeItem it;
+            it.expert = e; it.row_start = lo + m * kMoeBM; it.rows = min(kMoeBM, hi - it.row_start); it.n_tile = n;
+            items[base + n * cnt + m] = it;
+        }
+    if (e == 511) *num_items = scan[511];
 }
 
 // ---------------------------------------------------------------------------- grouped GEMM
 struct MoeGemmParams {
-    const uint8_t* A;        // activations, packed e2m1 rows
-    const uint8_t* SA;       // their e8m0 scales
+    const uint8_t* A;        // activations in sorted order, packed e2m1 [S][a_pitch]
+    const uint8_t* SA;       // their e8m0 scales [S][sa_pitch]
     const uint8_t* B;        // expert weights, packed e2m1 [E][rows_b][b_pitch]
     const uint8_t* SB;       // their scales [E][rows_b][sb_pitch]
-    const int32_t* sorted_slots;  // MODE 0: row p of the sorted order reads token sorted_slots[p]/topk
-    const int32_t* tile_info;
-    const int32_t* num_tiles;
+    const MoeItem* items;
+    const int32_t* num_items;
     void* out0;              // MODE 0: packed h [S][out_pitch]; MODE 1: bf16 o [S][N]
     uint8_t* out_scales;     // MODE 0: e8m0 scales of h [S][out_scale_pitch]
     long long b_expert_stride, sb_expert_stride;
@@ -113,7 +163,8 @@ struct MoeGemmParams {
     int out_pitch, out_scale_pitch;
     int K;                   // contraction length in elements
     int N;                   // MODE 0: I (h columns; weight rows i and I+i); MODE 1: output columns
-    int topk, n_tiles_n;
+    int n_tiles_n;
+    int lookahead;           // 1: persistent workgroups prefetch across items (needs >= 3 K-steps)
 };
 
 constexpr int kMoeATile = kMoeBM * 128;                 // 16 KiB
@@ -126,96 +177,102 @@ constexpr int kMoeScaleBase = kMoeStages * kMoeStage;
 constexpr int kMoeLds = kMoeScaleBase + kMoeStages * kMoeScaleStage;  // 153 KiB
 constexpr int kMoeDmaPerTile = 4 + 8 + 1 + 2;           // A, B, A scales, B scales per wave
 
+// Global->LDS source offsets of one work item.
+struct MoeAddr {
+    v4i srd_b, srd_sb;
+    uint32_t voff_a[4], voff_b[8], voff_sa, voff_sb[2];
+    int row_start, rows, n0, n_tile;
+    bool valid;
+};
+
 template <int MODE>
 __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams p) {
     constexpr int MT = 8, NT = 4, AD = 3, PG = 4;
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
     const int lane = lane_id(), w = wave_id();
-    const int m_tile = blockIdx.x / p.n_tiles_n, n_tile = blockIdx.x % p.n_tiles_n;
-    if (m_tile >= *p.num_tiles) return;
-    const int expert = to_sgpr(p.tile_info[3 * m_tile + 0]);
-    const int row_start = to_sgpr(p.tile_info[3 * m_tile + 1]);
-    const int rows = to_sgpr(p.tile_info[3 * m_tile + 2]);
-    const int mt_act = (rows + 15) >> 4;
-    const int n0 = n_tile * (MODE == 0 ? 128 : 256);  // first h column / output column of the tile
+    const int n_items = *p.num_items;
+    const int chunk = (n_items + (int)gridDim.x - 1) / (int)gridDim.x;
+    int it = blockIdx.x * chunk;
+    const int it_end = min(n_items, it + chunk);
+    if (it >= it_end) return;
 
     const int Kb = p.K >> 1;                 // contraction bytes per row
     const int nk = (Kb + 127) >> 7;
     const int tail_bytes = Kb - (nk - 1) * 128;  // valid bytes of the last K-step (16..128)
-
-    const uint8_t* b_base = p.B + (size_t)expert * p.b_expert_stride;
-    const uint8_t* sb_base = p.SB + (size_t)expert * p.sb_expert_stride;
     const int rows_b = MODE == 0 ? 2 * p.N : p.N;
     const v4i srd_a = make_srd(p.A, 0x7fffffffu);
     const v4i srd_sa = make_srd(p.SA, 0x7fffffffu);
-    const v4i srd_b = make_srd(b_base, (uint32_t)rows_b * (uint32_t)p.b_pitch);
-    const v4i srd_sb = make_srd(sb_base, (uint32_t)rows_b * (uint32_t)p.sb_pitch);
 
-    // Weight row held by LDS row R of the B tile.
-    auto b_row = [&](int R) -> int {
-        if (MODE == 1) return min(n0 + b_row_to_col(R), p.N - 1);
-        const int wn = R >> 6, t = (R >> 4) & 3, r = R & 15;
-        const int hcol = 32 * wn + 8 * (r >> 2) + 4 * (t >> 1) + (r & 3);
-        return (t & 1) * p.N + min(n0 + hcol, p.N - 1);
-    };
-    // Activation row (byte offset base) held by LDS row R of the A tile.
-    auto a_row = [&](int R) -> uint32_t {
-        const int pos = row_start + min(R, rows - 1);
-        if (MODE == 0) return (uint32_t)(p.sorted_slots[pos] / p.topk);
-        return (uint32_t)pos;
-    };
+    const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);  // same for every load index
+    const bool tail_oob = (int)(chunk16 * 16) >= tail_bytes;
 
-    const uint32_t chunk = swz_chunk(8 * w + (lane >> 3), lane & 7);  // same for every load index
-    const bool tail_oob = (int)(chunk * 16) >= tail_bytes;
-    uint32_t voff_a[4], voff_b[8], voff_sa, voff_sb[2];
+    auto make_addr = [&](int idx, MoeAddr& a) {
+        a.valid = idx < it_end;
+        if (!a.valid) idx = it_end - 1;  // harmless values; every load of an invalid set is zero-sized
+        const MoeItem item = p.items[idx];
+        const int expert = to_sgpr(item.expert);
+        a.row_start = to_sgpr(item.row_start);
+        a.rows = to_sgpr(item.rows);
+        a.n_tile = to_sgpr(item.n_tile);
+        a.n0 = a.n_tile * (MODE == 0 ? 128 : 256);
+        a.srd_b = make_srd(p.B + (size_t)expert * p.b_expert_stride, (uint32_t)rows_b * (uint32_t)p.b_pitch);
+        a.srd_sb = make_srd(p.SB + (size_t)expert * p.sb_expert_stride, (uint32_t)rows_b * (uint32_t)p.sb_pitch);
+        // weight row held by LDS row R of the B tile
+        auto b_row = [&](int R) -> int {
+            if (MODE == 1) return min(a.n0 + b_row_to_col(R), p.N - 1);
+            const int wn = R >> 6, t = (R >> 4) & 3, r = R & 15;
+            const int hcol = 32 * wn + 8 * (r >> 2) + 4 * (t >> 1) + (r & 3);
+            return (t & 1) * p.N + min(a.n0 + hcol, p.N - 1);
+        };
+        auto a_row = [&](int R) -> uint32_t { return (uint32_t)(a.row_start + min(R, a.rows - 1)); };
 #pragma unroll
-    for (int i = 0; i < 4; ++i) voff_a[i] = a_row(8 * (i * 4 + w) + (lane >> 3)) * (uint32_t)p.a_pitch + chunk * 16u;
+        for (int i = 0; i < 4; ++i)
+            a.voff_a[i] = a_row(8 * (i * 4 + w) + (lane >> 3)) * (uint32_t)p.a_pitch + chunk16 * 16u;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) voff_b[i] = (uint32_t)b_row(8 * (i * 4 + w) + (lane >> 3)) * (uint32_t)p.b_pitch + chunk * 16u;
-    voff_sa = a_row(32 * w + (lane >> 1)) * (uint32_t)p.sa_pitch + (lane & 1) * 4u;
+        for (int i = 0; i < 8; ++i)
+            a.voff_b[i] = (uint32_t)b_row(8 * (i * 4 + w) + (lane >> 3)) * (uint32_t)p.b_pitch + chunk16 * 16u;
+        a.voff_sa = a_row(32 * w + (lane >> 1)) * (uint32_t)p.sa_pitch + (lane & 1) * 4u;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) voff_sb[j] = (uint32_t)b_row(32 * (2 * w + j) + (lane >> 1)) * (uint32_t)p.sb_pitch + (lane & 1) * 4u;
+        for (int j = 0; j < 2; ++j)
+            a.voff_sb[j] = (uint32_t)b_row(32 * (2 * w + j) + (lane >> 1)) * (uint32_t)p.sb_pitch + (lane & 1) * 4u;
+    };
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
     const uint32_t lds_sa_wave = to_sgpr(lds0 + kMoeScaleBase + (uint32_t)w * 256u);
     const uint32_t lds_sb_wave = to_sgpr(lds0 + kMoeScaleBase + kMoeScaleA + (uint32_t)w * 512u);
 
-    // All 15 loads of K-step kt into `stage`. Past the end of K they are issued against
-    // zero-sized buffers (no traffic) so that the outstanding-load count stays uniform.
-    auto issue_tile = [&](int stage, int kt) {
-        v4i sa = srd_a, sb = srd_b, ssa = srd_sa, ssb = srd_sb;
-        if (kt >= nk) { sa.z = 0; sb.z = 0; ssa.z = 0; ssb.z = 0; }
+    // All 15 loads of K-step kt of item `a` into `stage`. For an invalid item or past the end
+    // of K they are issued against zero-sized buffers (no traffic), which keeps the number of
+    // outstanding loads per K-step uniform.
+    auto issue_tile = [&](const MoeAddr& a, int stage, int kt) {
+        v4i sa = srd_a, sb = a.srd_b, ssa = srd_sa, ssb = a.srd_sb;
+        if (!a.valid || kt >= nk) { sa.z = 0; sb.z = 0; ssa.z = 0; ssb.z = 0; }
         const bool last = (kt == nk - 1) && tail_oob;
         const uint32_t k0 = (uint32_t)kt * 128u;
         const uint32_t dst = lds_wave + (uint32_t)stage * kMoeStage;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(sa, dst + i * 4096, last ? 0x80000000u : voff_a[i], k0);
+        for (int i = 0; i < 4; ++i) dma16(sa, dst + i * 4096, last ? 0x80000000u : a.voff_a[i], k0);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) dma16(sb, dst + kMoeATile + i * 4096, last ? 0x80000000u : voff_b[i], k0);
-        dma4(ssa, lds_sa_wave + (uint32_t)stage * kMoeScaleStage, voff_sa, (uint32_t)kt * 8u);
+        for (int i = 0; i < 8; ++i) dma16(sb, dst + kMoeATile + i * 4096, last ? 0x80000000u : a.voff_b[i], k0);
+        dma4(ssa, lds_sa_wave + (uint32_t)stage * kMoeScaleStage, a.voff_sa, (uint32_t)kt * 8u);
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-            dma4(ssb, lds_sb_wave + (uint32_t)stage * kMoeScaleStage + j * 256, voff_sb[j], (uint32_t)kt * 8u);
+            dma4(ssb, lds_sb_wave + (uint32_t)stage * kMoeScaleStage + j * 256, a.voff_sb[j], (uint32_t)kt * 8u);
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
     const uint32_t rd_lo = r * 128u + swz_chunk(r, g) * 16u;
     const uint32_t rd_hi = r * 128u + swz_chunk(r, g + 4) * 16u;
-    uint32_t a_lo[3], a_hi[3], b_lo[3], b_hi[3];
-#pragma unroll
-    for (int st = 0; st < 3; ++st) {
-        a_lo[st] = lds0 + st * kMoeStage + rd_lo;
-        a_hi[st] = lds0 + st * kMoeStage + rd_hi;
-        b_lo[st] = lds0 + st * kMoeStage + kMoeATile + w * (64 * 128) + rd_lo;
-        b_hi[st] = lds0 + st * kMoeStage + kMoeATile + w * (64 * 128) + rd_hi;
-    }
-    uint32_t sa_rd = lds0 + kMoeScaleBase + r * 8u;
-    uint32_t sb_rd = lds0 + kMoeScaleBase + kMoeScaleA + (w * 64 + r) * 8u;
-    asm volatile("" : "+v"(sa_rd), "+v"(sb_rd));
+    // stage 0 addresses; a K-step on stage st adds st * kMoeStage (scales: st * kMoeScaleStage)
+    const uint32_t a_lo0 = lds0 + rd_lo, a_hi0 = lds0 + rd_hi;
+    const uint32_t b_lo0 = lds0 + kMoeATile + w * (64 * 128) + rd_lo;
+    const uint32_t b_hi0 = lds0 + kMoeATile + w * (64 * 128) + rd_hi;
+    const uint32_t sa_rd0 = lds0 + kMoeScaleBase + r * 8u;
+    const uint32_t sb_rd0 = lds0 + kMoeScaleBase + kMoeScaleA + (w * 64 + r) * 8u;
     const uint32_t sh = 8u * g;
-    auto rd_scale = [&](uint32_t base, int stage, int f) -> v2i {
-        return *(lds_v2i_t*)(uintptr_t)(base + stage * kMoeScaleStage + f * 128);
+    auto rd_scale = [&](uint32_t base, int f) -> v2i {
+        return *(lds_v2i_t*)(uintptr_t)(base + f * 128);
     };
     auto shift_scale = [&](v2i& s) {
         s.x = (int)((uint32_t)s.x >> sh);
@@ -236,170 +293,175 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
     };
 
     v4f acc[MT][NT];
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
-    Frag4 bf[2][NT], af[4];
-    v2i bs[2][NT], as[4];
+    Frag4 bf[NT], af[4];
+    v2i bs[NT], as[4];
+    MoeAddr cur, nxt;
+    int mt_act = 0;
 
-    // ---- prologue: three K-steps in flight, fragments of the first in registers ----------
-    issue_tile(0, 0);
-    issue_tile(1, 1);
-    issue_tile(2, 2);
-    wait_vmcnt<2 * kMoeDmaPerTile>();
-    block_barrier();
+    // One K-step on LDS stage `st` (a run-time value, so that a single copy of this code
+    // serves the whole ring): read this step's B fragments and first A fragments, then MFMA
+    // groups with the A fragments read three groups ahead; after group PG one barrier, then the
+    // refill of stage `st` with the K-step three positions ahead in the stream (which may
+    // belong to the next work item). The LDS latency exposed at the start of every step is
+    // hidden behind the weight stream from HBM that bounds this kernel.
+    auto step = [&](int kt, int st) {
+        uint32_t a_lo = a_lo0 + (uint32_t)st * kMoeStage, a_hi = a_hi0 + (uint32_t)st * kMoeStage;
+        uint32_t b_lo = b_lo0 + (uint32_t)st * kMoeStage, b_hi = b_hi0 + (uint32_t)st * kMoeStage;
+        uint32_t sa_rd = sa_rd0 + (uint32_t)st * kMoeScaleStage, sb_rd = sb_rd0 + (uint32_t)st * kMoeScaleStage;
+        // keep the (large) bases in registers so that fragment offsets stay immediates
+        asm volatile("" : "+v"(a_lo), "+v"(a_hi), "+v"(b_lo), "+v"(b_hi), "+v"(sa_rd), "+v"(sb_rd));
 #pragma unroll
-    for (int n = 0; n < NT; ++n) {
-        bf[0][n] = rd_frag(b_lo[0], b_hi[0], n * 2048);
-        bs[0][n] = rd_scale(sb_rd, 0, n);
-    }
+        for (int n = 0; n < NT; ++n) {
+            bf[n] = rd_frag(b_lo, b_hi, n * 2048);
+            bs[n] = rd_scale(sb_rd, n);
+        }
 #pragma unroll
-    for (int m = 0; m < AD; ++m) {
-        af[m] = rd_frag(a_lo[0], a_hi[0], m * 2048);
-        as[m] = rd_scale(sa_rd, 0, m);
-    }
+        for (int m = 0; m < AD; ++m) {
+            af[m] = rd_frag(a_lo, a_hi, m * 2048);
+            as[m] = rd_scale(sa_rd, m);
+        }
 #pragma unroll
-    for (int n = 0; n < NT; ++n) shift_scale(bs[0][n]);
-    shift_scale(as[0]);
-
-    // One K-step. ST = LDS stage of this step, Q = parity of the B-fragment register set.
-    auto step = [&]<int ST, int Q>(int kt) {
-        constexpr int NS = (ST + 1) % 3;  // stage of the next K-step
+        for (int n = 0; n < NT; ++n) shift_scale(bs[n]);
+        shift_scale(as[0]);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             if (m < mt_act) {
 #pragma unroll
                 for (int n = 0; n < NT; ++n) {
-                    mfma(acc[m][n], bf[Q][n].lo, af[m & 3].lo, bs[Q][n].x, as[m & 3].x);
+                    mfma(acc[m][n], bf[n].lo, af[m & 3].lo, bs[n].x, as[m & 3].x);
                     if (n == 0 && m <= PG) {
-                        af[(m + AD) & 3] = rd_frag(a_lo[ST], a_hi[ST], (m + AD) * 2048);
-                        as[(m + AD) & 3] = rd_scale(sa_rd, ST, m + AD);
+                        af[(m + AD) & 3] = rd_frag(a_lo, a_hi, (m + AD) * 2048);
+                        as[(m + AD) & 3] = rd_scale(sa_rd, m + AD);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
 #pragma unroll
                 for (int n = 0; n < NT; ++n) {
-                    mfma(acc[m][n], bf[Q][n].hi, af[m & 3].hi, bs[Q][n].y, as[m & 3].y);
-                    if (n == 2) shift_scale(as[(m + 1) & 3]);
+                    mfma(acc[m][n], bf[n].hi, af[m & 3].hi, bs[n].y, as[m & 3].y);
+                    if (n == 2 && m + 1 < MT) shift_scale(as[(m + 1) & 3]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-            } else {
+            } else if (m <= PG) {
                 // keep the rotation of A buffers in step with the full schedule
-                if (m <= PG) {
-                    af[(m + AD) & 3] = rd_frag(a_lo[ST], a_hi[ST], (m + AD) * 2048);
-                    as[(m + AD) & 3] = rd_scale(sa_rd, ST, m + AD);
-                }
+                af[(m + AD) & 3] = rd_frag(a_lo, a_hi, (m + AD) * 2048);
+                as[(m + AD) & 3] = rd_scale(sa_rd, m + AD);
                 shift_scale(as[(m + 1) & 3]);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (m == PG) {
-                // all reads of stage ST are issued; wait for them and for the next K-step's
-                // loads (the K-step after that may stay in flight), then refill stage ST
+                // all reads of stage st are issued; wait for them and for the next K-step's
+                // loads (the K-step after that may stay in flight), then refill stage st
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 wait_vmcnt<kMoeDmaPerTile>();
                 block_barrier();
-                issue_tile(ST, kt + 3);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if (m == PG + 1) {
-#pragma unroll
-                for (int n = 0; n < NT; ++n) {
-                    bf[Q ^ 1][n] = rd_frag(b_lo[NS], b_hi[NS], n * 2048);
-                    bs[Q ^ 1][n] = rd_scale(sb_rd, NS, n);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if (m == PG + 2) {
-                af[0] = rd_frag(a_lo[NS], a_hi[NS], 0);
-                as[0] = rd_scale(sa_rd, NS, 0);
-                af[1] = rd_frag(a_lo[NS], a_hi[NS], 2048);
-                as[1] = rd_scale(sa_rd, NS, 1);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if (m == PG + 3) {
-                af[2] = rd_frag(a_lo[NS], a_hi[NS], 2 * 2048);
-                as[2] = rd_scale(sa_rd, NS, 2);
-#pragma unroll
-                for (int n = 0; n < NT; ++n) shift_scale(bs[Q ^ 1][n]);
+                if (kt + 3 < nk) issue_tile(cur, st, kt + 3);
+                else issue_tile(nxt, st, kt + 3 - nk);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
 
-    // stage cycles with period 3, register parity with period 2 -> unroll by 6
-    int kt = 0;
-    for (; kt + 5 < nk; kt += 6) {
-        step.template operator()<0, 0>(kt);
-        step.template operator()<1, 1>(kt + 1);
-        step.template operator()<2, 0>(kt + 2);
-        step.template operator()<0, 1>(kt + 3);
-        step.template operator()<1, 0>(kt + 4);
-        step.template operator()<2, 1>(kt + 5);
-    }
-    if (kt < nk) { step.template operator()<0, 0>(kt); ++kt; }
-    if (kt < nk) { step.template operator()<1, 1>(kt); ++kt; }
-    if (kt < nk) { step.template operator()<2, 0>(kt); ++kt; }
-    if (kt < nk) { step.template operator()<0, 1>(kt); ++kt; }
-    if (kt < nk) { step.template operator()<1, 0>(kt); ++kt; }
-    wait_vmcnt<0>();
-    mfma_drain();
-
-    // ---- epilogue -------------------------------------------------------------------------
-    if (MODE == 1) {
-        uint16_t* out = (uint16_t*)p.out0;
+    auto epilogue = [&](const MoeAddr& a) {
+        const int rows = a.rows, row_start = a.row_start, n0 = a.n0;
+        if (MODE == 1) {
+            uint16_t* out = (uint16_t*)p.out0;
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            const int row = 16 * m + (int)r;
-            if (row >= rows) continue;
-            const size_t pos = (size_t)(row_start + row);
+            for (int m = 0; m < MT; ++m) {
+                const int row = 16 * m + (int)r;
+                if (row >= rows) continue;
+                const size_t pos = (size_t)(row_start + row);
 #pragma unroll
-            for (int q = 0; q < NT / 2; ++q) {
-                const int col = n0 + w * 64 + 32 * q + 8 * (int)g;
-                if (col + 8 > p.N) continue;  // N % 8 == 0
-                const v4f x = acc[m][2 * q], y = acc[m][2 * q + 1];
-                v4i o4;
-                o4.x = pack_bf16(x.x, x.y); o4.y = pack_bf16(x.z, x.w);
-                o4.z = pack_bf16(y.x, y.y); o4.w = pack_bf16(y.z, y.w);
-                *(v4i*)(out + pos * p.N + col) = o4;
-            }
-        }
-    } else {
-        uint8_t* hq = (uint8_t*)p.out0;
-        const int hcol0 = n0 + 32 * w;  // this wave's MX block of h
-        const bool col_ok = hcol0 < p.N;
-        const bool last_n = n_tile == p.n_tiles_n - 1;
-#pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            const int row = 16 * m + (int)r;
-            float h[8];
-#pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                const v4f gt = acc[m][2 * q], up = acc[m][2 * q + 1];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float gv = gt[j];
-                    h[4 * q + j] = gv / (1.0f + __expf(-gv)) * up[j];
+                for (int q = 0; q < NT / 2; ++q) {
+                    const int col = n0 + w * 64 + 32 * q + 8 * (int)g;
+                    if (col + 8 > p.N) continue;  // N % 8 == 0
+                    const v4f x = acc[m][2 * q], y = acc[m][2 * q + 1];
+                    v4i o4;
+                    o4.x = pack_bf16(x.x, x.y); o4.y = pack_bf16(x.z, x.w);
+                    o4.z = pack_bf16(y.x, y.y); o4.w = pack_bf16(y.z, y.w);
+                    *(v4i*)(out + pos * p.N + col) = o4;
                 }
             }
-            float amax = 0.f;
+        } else {
+            uint8_t* hq = (uint8_t*)p.out0;
+            const int hcol0 = n0 + 32 * w;  // this wave's MX block of h
+            const bool col_ok = hcol0 < p.N;
+            const bool last_n = a.n_tile == p.n_tiles_n - 1;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(h[i]));
-            amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-            amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-            const int e = mx_block_exponent(amax);
-            if (row < rows && col_ok) {
-                const size_t pos = (size_t)(row_start + row);
-                *(uint32_t*)(hq + pos * p.out_pitch + (hcol0 >> 1) + 4 * g) = pack8_e2m1(h, e);
-                if (g == 0) p.out_scales[pos * p.out_scale_pitch + (hcol0 >> 5)] = (uint8_t)(e + 127);
-            }
-            if (row < rows && last_n && w == 0 && g == 1) {
-                // neutral scale bytes in the padding columns of this row
-                const size_t pos = (size_t)(row_start + row);
-                for (int c = p.N >> 5; c < p.out_scale_pitch; ++c) p.out_scales[pos * p.out_scale_pitch + c] = 127;
+            for (int m = 0; m < MT; ++m) {
+                const int row = 16 * m + (int)r;
+                float h[8];
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const v4f gt = acc[m][2 * q], up = acc[m][2 * q + 1];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float gv = gt[j];
+                        h[4 * q + j] = gv / (1.0f + __expf(-gv)) * up[j];
+                    }
+                }
+                float amax = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(h[i]));
+                amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+                const int e = mx_block_exponent(amax);
+                if (row < rows && col_ok) {
+                    const size_t pos = (size_t)(row_start + row);
+                    *(uint32_t*)(hq + pos * p.out_pitch + (hcol0 >> 1) + 4 * g) = pack8_e2m1(h, e);
+                    if (g == 0) p.out_scales[pos * p.out_scale_pitch + (hcol0 >> 5)] = (uint8_t)(e + 127);
+                }
+                if (row < rows && last_n && w == 0 && g == 1) {
+                    // neutral scale bytes in the padding columns of this row
+                    const size_t pos = (size_t)(row_start + row);
+                    for (int c = p.N >> 5; c < p.out_scale_pitch; ++c)
+                        p.out_scales[pos * p.out_scale_pitch + c] = 127;
+                }
             }
         }
+    };
+
+    const bool look = p.lookahead != 0;
+    bool need_prologue = true;
+    int st = 0;  // LDS stage of the next K-step to compute
+    make_addr(it, cur);
+    for (;;) {
+        make_addr(look ? it + 1 : it_end, nxt);
+        mt_act = (cur.rows + 15) >> 4;
+        if (need_prologue) {
+            // three K-steps in flight, fragments of the first in registers
+#pragma unroll
+            for (int s3 = 0; s3 < 3; ++s3) {
+                if (s3 < nk) issue_tile(cur, s3, s3);
+                else issue_tile(nxt, s3, s3 - nk);  // only without lookahead: zero-sized
+            }
+            wait_vmcnt<2 * kMoeDmaPerTile>();
+            block_barrier();
+            st = 0;
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int kt = 0; kt < nk; ++kt) {
+            step(kt, st);
+            st = st == 2 ? 0 : st + 1;
+        }
+        mfma_drain();
+        epilogue(cur);
+        if (++it >= it_end) break;
+        if (look) {
+            cur = nxt;
+        } else {
+            // no cross-item prefetch: drain the ring and start the next item from scratch
+            wait_vmcnt<0>();
+            block_barrier();
+            make_addr(it, cur);
+            need_prologue = true;
+        }
+        need_prologue = !look;
     }
+    wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
 }
 
 // ------------------------------------------------------------------------------ un-permute
@@ -432,8 +494,19 @@ __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __re
 
 static int round_up(int x, int m) { return (x + m - 1) / m * m; }
 
+static int num_compute_units() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256;
+        cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    }
+    return cus;
+}
+
 template <int MODE>
-static int launch_moe_gemm(const MoeGemmParams& p, int max_m_tiles, hipStream_t s) {
+static int launch_moe_gemm(MoeGemmParams p, int max_items, hipStream_t s) {
     auto kern = moe_mxfp4_gemm_kernel<MODE>;
     static bool configured = false;
     if (!configured) {
@@ -442,7 +515,11 @@ static int launch_moe_gemm(const MoeGemmParams& p, int max_m_tiles, hipStream_t 
             return HK_ERR_LAUNCH;
         configured = true;
     }
-    hipLaunchKernelGGL(kern, dim3(max_m_tiles * p.n_tiles_n), dim3(256), kMoeLds, s, p);
+    const int nk = (p.K / 2 + 127) / 128;
+    p.lookahead = nk >= 3 ? 1 : 0;
+    // persistent: one workgroup per CU walks a contiguous range of items; otherwise one per item
+    const int grid = p.lookahead ? min(max_items, num_compute_units()) : max_items;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), kMoeLds, s, p);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
@@ -475,7 +552,8 @@ extern "C" int hk_moe_unpermute(const void* o_bf16, const float* w, const int32_
 
 // Workspace layout of hk_moe_mxfp4_forward (all regions 256-byte aligned).
 struct MoeWs {
-    size_t ids, w, sorted, offsets, inv, sort_ws, tiles, ntiles, xq, xs, hq, hs, o, total;
+    size_t ids, w, sorted, offsets, inv, sort_ws, items1, items2, nitems, xq, xs, hq, hs, o, total;
+    int max_items1, max_items2;
 };
 static MoeWs moe_ws_layout(int T, int H, int I, int E, int k) {
     MoeWs L;
@@ -484,9 +562,13 @@ static MoeWs moe_ws_layout(int T, int H, int I, int E, int k) {
     const size_t S = (size_t)T * k;
     L.ids = take(S * 4); L.w = take(S * 4); L.sorted = take(S * 4); L.offsets = take((size_t)(E + 1) * 4);
     L.inv = take(S * 4); L.sort_ws = take(hk_moe_sort_workspace_bytes(T, k, E));
-    const size_t max_tiles = S / kMoeBM + E;
-    L.tiles = take(max_tiles * 12); L.ntiles = take(4);
-    L.xq = take((size_t)T * (H / 2)); L.xs = take((size_t)T * round_up(H / 32, 8));
+    const int max_tiles = (int)(S / kMoeBM) + E;
+    L.max_items1 = max_tiles * ((I + 127) / 128);
+    L.max_items2 = max_tiles * ((H + 255) / 256);
+    L.items1 = take((size_t)L.max_items1 * sizeof(MoeItem));
+    L.items2 = take((size_t)L.max_items2 * sizeof(MoeItem));
+    L.nitems = take(8);
+    L.xq = take(S * (H / 2)); L.xs = take(S * round_up(H / 32, 8));
     L.hq = take(S * (I / 2)); L.hs = take(S * round_up(I / 32, 8));
     L.o = take(S * (size_t)H * 2);
     L.total = off;
@@ -505,7 +587,7 @@ static int moe_mxfp4_check(int T, int H, int I, int E, int k, int w13_scale_pitc
         (w2_scale_pitch % 8) != 0)
         return HK_ERR_BAD_SHAPE;
     if ((long long)T * k >= (1ll << 24) || (long long)T * k * (I / 2) >= (1ll << 31) ||
-        (long long)T * (H / 2) >= (1ll << 31) || (long long)2 * I * (H / 2) >= (1ll << 31) ||
+        (long long)T * k * (H / 2) >= (1ll << 31) || (long long)2 * I * (H / 2) >= (1ll << 31) ||
         (long long)H * (I / 2) >= (1ll << 31))
         return HK_ERR_BAD_SHAPE;
     return HK_OK;
@@ -532,23 +614,27 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
     uint8_t* ws = (uint8_t*)workspace;
     const int S = T * k;
     const int xs_pitch = round_up(H / 32, 8), hs_pitch = round_up(I / 32, 8);
-    const int max_tiles = S / kMoeBM + E;
 
-    st = hk_mxfp4_quantize_rows(x_bf16, T, H, ws + L.xq, ws + L.xs, xs_pitch, stream);
-    if (st != HK_OK) return st;
-    hipLaunchKernelGGL(moe_build_tiles_kernel, dim3(1), dim3(64), 0, s, expert_offsets, E,
-                       (int32_t*)(ws + L.tiles), (int32_t*)(ws + L.ntiles));
+    {
+        const long long threads = (long long)S * xs_pitch * 4;
+        hipLaunchKernelGGL(mxfp4_quantize_permute_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
+                           (const uint16_t*)x_bf16, sorted_slots, k, S, H, ws + L.xq, ws + L.xs, xs_pitch);
+    }
+    int32_t* nitems = (int32_t*)(ws + L.nitems);
+    hipLaunchKernelGGL(moe_build_items_kernel, dim3(1), dim3(512), 0, s, expert_offsets, E, (I + 127) / 128,
+                       (MoeItem*)(ws + L.items1), nitems);
+    hipLaunchKernelGGL(moe_build_items_kernel, dim3(1), dim3(512), 0, s, expert_offsets, E, (H + 255) / 256,
+                       (MoeItem*)(ws + L.items2), nitems + 1);
 
     MoeGemmParams p{};
     p.A = ws + L.xq; p.SA = ws + L.xs; p.a_pitch = H / 2; p.sa_pitch = xs_pitch;
     p.B = (const uint8_t*)w13; p.SB = (const uint8_t*)w13_scales;
     p.b_pitch = H / 2; p.sb_pitch = w13_scale_pitch;
     p.b_expert_stride = (long long)2 * I * (H / 2); p.sb_expert_stride = (long long)2 * I * w13_scale_pitch;
-    p.sorted_slots = sorted_slots; p.tile_info = (const int32_t*)(ws + L.tiles);
-    p.num_tiles = (const int32_t*)(ws + L.ntiles);
+    p.items = (const MoeItem*)(ws + L.items1); p.num_items = nitems;
     p.out0 = ws + L.hq; p.out_scales = ws + L.hs; p.out_pitch = I / 2; p.out_scale_pitch = hs_pitch;
-    p.K = H; p.N = I; p.topk = k; p.n_tiles_n = (I + 127) / 128;
-    st = launch_moe_gemm<0>(p, max_tiles, s);
+    p.K = H; p.N = I; p.n_tiles_n = (I + 127) / 128;
+    st = launch_moe_gemm<0>(p, L.max_items1, s);
     if (st != HK_OK) return st;
 
     MoeGemmParams q{};
@@ -556,10 +642,10 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
     q.B = (const uint8_t*)w2; q.SB = (const uint8_t*)w2_scales;
     q.b_pitch = I / 2; q.sb_pitch = w2_scale_pitch;
     q.b_expert_stride = (long long)H * (I / 2); q.sb_expert_stride = (long long)H * w2_scale_pitch;
-    q.sorted_slots = sorted_slots; q.tile_info = p.tile_info; q.num_tiles = p.num_tiles;
+    q.items = (const MoeItem*)(ws + L.items2); q.num_items = nitems + 1;
     q.out0 = ws + L.o; q.out_scales = nullptr; q.out_pitch = 0; q.out_scale_pitch = 0;
-    q.K = I; q.N = H; q.topk = k; q.n_tiles_n = (H + 255) / 256;
-    st = launch_moe_gemm<1>(q, max_tiles, s);
+    q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
+    st = launch_moe_gemm<1>(q, L.max_items2, s);
     if (st != HK_OK) return st;
 
     return hk_moe_unpermute(ws + L.o, topk_w, slot_to_pos, T, k, H, y_bf16, stream);
