@@ -64,9 +64,33 @@ __device__ __forceinline__ void dma4(v4i srd, uint32_t lds_base, uint32_t voff, 
         : "memory", "m0");
 }
 
+// dma16 restricted to the lanes set in `mask` (lane l still lands at lds_base + 16*l).
+__device__ __forceinline__ void dma16_lanes(v4i srd, uint32_t lds_base, uint32_t voff, uint32_t soff,
+                                            uint64_t mask) {
+    uint64_t saved;
+    asm volatile(
+        "s_mov_b64 %0, exec\n\t"
+        "s_mov_b64 exec, %5\n\t"
+        "s_mov_b32 m0, %1\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dwordx4 %2, %3, %4 offen lds\n\t"
+        "s_mov_b64 exec, %0"
+        : "=&s"(saved)
+        : "s"(lds_base), "v"(voff), "s"(srd), "s"(soff), "s"(mask)
+        : "memory", "m0");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Fixes the position of everything around it: memory operations may not be moved across the
+// empty asm (compiler fence) and the machine scheduler may not move anything across the
+// scheduling barrier. Used between the slots of the hand-interleaved schedules.
+__device__ __forceinline__ void slot_fence() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
 }
 
 __device__ __forceinline__ void block_barrier() { __builtin_amdgcn_s_barrier(); }
@@ -95,6 +119,30 @@ __device__ __forceinline__ v8i lds_frag(uint32_t addr_lo, uint32_t addr_hi, int 
 // (include/ops/warp/register/tile/mma.cuh:112-125).
 __device__ __forceinline__ v4f mfma_fp8_16x16x128(v8i a, v8i b, v4f c) {
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+// D(16x16, fp32) += X(16x128 e2m1, scale sx) * Y(16x128 e2m1, scale sy)^T: the FP4 form of the
+// same instruction (cbsz = blgp = 4). Each lane holds 32 elements (16 bytes) of its row's K-block
+// l/16 and supplies the e8m0 scale of exactly that block in bits [7:0] of sx / sy. The builtin
+// takes 8-dword operands of which the FP4 form reads the first four; the duplicate shuffle costs
+// no instructions.
+__device__ __forceinline__ v4f mfma_fp4(v4i x, v4i y, v4f c, int sx, int sy) {
+    v8i x8 = __builtin_shufflevector(x, x, 0, 1, 2, 3, 0, 1, 2, 3);
+    v8i y8 = __builtin_shufflevector(y, y, 0, 1, 2, 3, 0, 1, 2, 3);
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x8, y8, c, 4, 4, 0, sx, 0, sy);
+}
+
+// Uniform 16-byte read through the scalar cache (s_load_dwordx4); `p` must be wave-uniform and
+// point to data written before this kernel started.
+__device__ __forceinline__ v4i scalar_load_x4(const void* p) {
+    v4i r;
+    asm volatile("s_load_dwordx4 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r) : "s"(p) : "memory");
+    return r;
+}
+__device__ __forceinline__ int scalar_load_x1(const void* p) {
+    int r;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r) : "s"(p) : "memory");
+    return r;
 }
 
 // Same MFMA with the accumulator tied in place in an accumulation register (AGPR).

@@ -5,15 +5,14 @@
 // interleaved FP8/MXFP4 kernels of this library (LDS-direct loads into swizzled 128-byte-row
 // tiles, ds_read_b128 fragments, v_mfma_scale_f32_16x16x128_f8f6f4 with in-MFMA e8m0 scales).
 //
-// Grouped GEMM: a work item is (m-tile, n-tile) where an m-tile is up to 128 consecutive rows
-// (sorted positions) of one expert; the item list is built on the device from
-// expert_offsets. A workgroup (4 waves, one per SIMD) computes a 128 x 256 tile per item; every
-// wave spans all 128 rows and owns 64 of the 256 weight rows, so that 16-row fragments beyond
-// the tile's real row count are skipped by all waves alike. Weights dominate HBM traffic at MoE
-// shapes (about 128 rows per expert), so the K loop runs a three-stage LDS ring (two K-steps of
-// operands always in flight) and workgroups are persistent: each walks a contiguous range of
-// items and the ring keeps running across item boundaries, so the next item's first K-steps
-// load while the current item's epilogue runs.
+// Grouped GEMM: a work item is (m-tile, n-tile) where an m-tile is up to 256 consecutive rows
+// (sorted positions) of one expert, so that at MoE shapes (100-300 rows per expert) an expert's
+// weight tile is streamed from HBM once; the item list is built on the device from
+// expert_offsets. A workgroup (4 waves, one per SIMD) computes a 256 x 256 tile per item; every
+// wave spans all 256 rows and owns 64 of the 256 weight rows. Weights dominate HBM traffic, so
+// workgroups are persistent: each walks a contiguous range of items and the two-stage LDS ring
+// keeps running across item boundaries, so the next item's first K-steps load while the
+// current item's epilogue runs.
 #include "gemm_tile.h"
 #include "../../include/hk355.h"
 
@@ -78,20 +77,26 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_rows_kernel(const uint16_t
     if ((c8 & 3) == 0) scales[(size_t)row * scale_pitch + (c8 >> 2)] = (uint8_t)(e + 127);
 }
 
-// Quantize-and-permute: row `pos` of the output is token sorted_slots[pos] / topk of x, so
-// that each expert's rows are contiguous for the grouped GEMM (the "permute" step of the MoE).
+// Activation layout inside the MoE ("K-step-major tiles"): for a matrix of S rows the bytes of
+// K-step kt (256 elements = 128 bytes per row, zero-padded past K) of all rows are contiguous,
+//   data   [nk][S][128] bytes,   scales [nk][S][8] e8m0 bytes (padding = 127),
+// so that the A tile of a work item (consecutive rows) and its scale tile are single contiguous,
+// 128-byte aligned runs for the global->LDS loads.
+//
+// Quantize-and-permute: row `pos` of the output is token sorted_slots[pos] / topk of x, so that
+// each expert's rows are contiguous for the grouped GEMM (the "permute" step of the MoE).
 __global__ __launch_bounds__(256) void mxfp4_quantize_permute_kernel(
     const uint16_t* __restrict__ x, const int32_t* __restrict__ sorted_slots, int topk, int S, int cols,
-    uint8_t* __restrict__ packed, uint8_t* __restrict__ scales, int scale_pitch) {
-    const int per_row = scale_pitch * 4;
+    uint8_t* __restrict__ tiled, uint8_t* __restrict__ tiled_scales) {
+    const int nk = (cols / 2 + 127) >> 7;
+    const int per_row = nk * 32;  // threads per row: one per 8 elements of the padded row
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
     const int pos = (int)(gid / per_row);
     const int c8 = (int)(gid % per_row);
     if (pos >= S) return;
     const int row = sorted_slots[pos] / topk;
     float v[8];
-    const bool in = c8 * 8 < cols;
-    if (in) {
+    if (c8 * 8 < cols) {
         const v4i raw = *(const v4i*)(x + (size_t)row * cols + c8 * 8);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -108,8 +113,71 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_permute_kernel(
     amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
     amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
     const int e = mx_block_exponent(amax);
-    if (in) *(uint32_t*)(packed + (size_t)pos * (cols / 2) + c8 * 4) = pack8_e2m1(v, e);
-    if ((c8 & 3) == 0) scales[(size_t)pos * scale_pitch + (c8 >> 2)] = (uint8_t)(e + 127);
+    const size_t tile_row = (size_t)(c8 >> 5) * S + pos;  // (kt, pos)
+    *(uint32_t*)(tiled + tile_row * 128 + (c8 & 31) * 4) = pack8_e2m1(v, e);
+    if ((c8 & 3) == 0) tiled_scales[tile_row * 8 + ((c8 >> 2) & 7)] = (uint8_t)(e + 127);
+}
+
+// Zero / neutral padding of the last K-step of a tiled activation matrix whose K is not a
+// multiple of 256 (the part the producing GEMM epilogue never writes).
+__global__ __launch_bounds__(256) void moe_pad_tiled_kernel(uint8_t* __restrict__ tiled,
+                                                            uint8_t* __restrict__ tiled_scales, int S, int K) {
+    const int Kb = K >> 1, nk = (Kb + 127) >> 7;
+    const int valid = Kb - (nk - 1) * 128;  // valid bytes of the last K-step, a multiple of 16
+    const int pos = blockIdx.x * 8 + (threadIdx.x >> 5);
+    const int c = threadIdx.x & 31;  // 4-byte column
+    if (pos >= S) return;
+    const size_t tile_row = (size_t)(nk - 1) * S + pos;
+    if (c * 4 >= valid) *(uint32_t*)(tiled + tile_row * 128 + c * 4) = 0u;
+    if (c < 8 && c * 16 >= valid) tiled_scales[tile_row * 8 + c] = 127;
+}
+
+// ---------------------------------------------------------------------- weight pre-shuffle
+// Row of the expert's weight matrix held by LDS row R (0..255) of the B tile of n-tile `n_tile`.
+// mode 0 (gate+up, N = I): each wave's 64 rows alternate 16 gate rows / 16 up rows of the same 16
+// h columns, permuted so that a lane ends up with 8 consecutive h columns; mode 1 (down, N = H):
+// b_row_to_col permutation (8 consecutive output columns per lane).
+__device__ __forceinline__ int moe_b_row(int mode, int R, int n_tile, int N) {
+    if (mode == 1) return min(n_tile * 256 + b_row_to_col(R), N - 1);
+    const int wn = R >> 6, t = (R >> 4) & 3, r = R & 15;
+    const int hcol = 32 * wn + 8 * (r >> 2) + 4 * (t >> 1) + (r & 3);
+    return (t & 1) * N + min(n_tile * 128 + hcol, N - 1);
+}
+
+// Pre-shuffled weight layout: for every expert, n-tile and K-step one contiguous 32 KiB block
+// holding the 256 x 128-byte B tile exactly as it sits in LDS (row permutation and chunk
+// swizzle applied, K zero-padded to whole K-steps), followed in a second array by the 2 KiB
+// scale tile (256 rows x 8 bytes, padding = 127). The grouped GEMM then streams weights from
+// HBM in long contiguous bursts instead of 128-byte pieces a row pitch apart.
+//   out_w [E][n_tiles][nk][256][128] bytes, out_s [E][n_tiles][nk][256][8] bytes.
+__global__ __launch_bounds__(256) void moe_preshuffle_kernel(const uint8_t* __restrict__ w,
+                                                             const uint8_t* __restrict__ sc, int E, int N,
+                                                             int K, int scale_pitch, int mode, int n_tiles,
+                                                             uint8_t* __restrict__ out_w,
+                                                             uint8_t* __restrict__ out_s) {
+    const int Kb = K >> 1, nk = (Kb + 127) >> 7;
+    const int rows_b = mode == 0 ? 2 * N : N;
+    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;  // one 16-byte chunk each
+    const long long total = (long long)E * n_tiles * nk * 2048;
+    if (gid >= total) return;
+    const int pc = (int)(gid & 7), R = (int)((gid >> 3) & 255);
+    long long rest = gid >> 11;
+    const int kt = (int)(rest % nk); rest /= nk;
+    const int nt = (int)(rest % n_tiles);
+    const int e = (int)(rest / n_tiles);
+    const int row = moe_b_row(mode, R, nt, N);
+    const int c = pc ^ ((R >> 1) & 7);
+    const int kb = kt * 128 + c * 16;
+    v4i val = {0, 0, 0, 0};
+    if (kb < Kb) val = *(const v4i*)(w + ((size_t)e * rows_b + row) * Kb + kb);
+    *(v4i*)(out_w + gid * 16) = val;
+    if (pc == 0) {
+        // this thread also moves the row's 8 scale bytes of the K-step
+        uint8_t* dst = out_s + (gid >> 3) * 8;
+        const uint8_t* src = sc + ((size_t)e * rows_b + row) * scale_pitch + kt * 8;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) dst[b] = (kt * 8 + b < (K >> 5)) ? src[b] : (uint8_t)127;
+    }
 }
 
 // ------------------------------------------------------------------------------ work items
@@ -117,7 +185,7 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_permute_kernel(
 // tile of weight rows. Items are listed expert by expert, n-tile by n-tile, the m-tiles of one
 // (expert, n-tile) next to each other, so that a workgroup walking a contiguous range re-reads a
 // weight tile for the expert's second m-tile straight from its XCD's L2.
-constexpr int kMoeBM = 128;
+constexpr int kMoeBM = 256;
 struct MoeItem { int expert, row_start, rows, n_tile; };
 
 __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __restrict__ expert_offsets,
@@ -150,47 +218,50 @@ __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __r
 
 // ---------------------------------------------------------------------------- grouped GEMM
 struct MoeGemmParams {
-    const uint8_t* A;        // activations in sorted order, packed e2m1 [S][a_pitch]
-    const uint8_t* SA;       // their e8m0 scales [S][sa_pitch]
+    const uint8_t* A;        // activations in sorted order, K-step-major tiles [nk][S][128]
+    const uint8_t* SA;       // their e8m0 scales [nk][S][8]
     const uint8_t* B;        // expert weights, packed e2m1 [E][rows_b][b_pitch]
     const uint8_t* SB;       // their scales [E][rows_b][sb_pitch]
     const MoeItem* items;
     const int32_t* num_items;
-    void* out0;              // MODE 0: packed h [S][out_pitch]; MODE 1: bf16 o [S][N]
-    uint8_t* out_scales;     // MODE 0: e8m0 scales of h [S][out_scale_pitch]
+    void* out0;              // MODE 0: packed h as K-step-major tiles [nk2][S][128]; MODE 1: bf16 o [S][N]
+    uint8_t* out_scales;     // MODE 0: e8m0 scales of h [nk2][S][8]
     long long b_expert_stride, sb_expert_stride;
-    int a_pitch, sa_pitch, b_pitch, sb_pitch;
-    int out_pitch, out_scale_pitch;
+    int b_pitch, sb_pitch;   // plain weight layout only
+    int S;                   // rows of the activation matrices (T * topk)
     int K;                   // contraction length in elements
     int N;                   // MODE 0: I (h columns; weight rows i and I+i); MODE 1: output columns
     int n_tiles_n;
-    int lookahead;           // 1: persistent workgroups prefetch across items (needs >= 3 K-steps)
+#if defined(HK_EXP_TIMING)
+    void* out_scales_dbg;
+#endif
+    int lookahead;           // 1: persistent workgroups prefetch across items (needs >= 2 K-steps)
+    int shuffled;            // 1: B / SB are in the pre-shuffled tile layout (see moe_preshuffle_kernel)
 };
 
-constexpr int kMoeATile = kMoeBM * 128;                 // 16 KiB
+constexpr int kMoeATile = kMoeBM * 128;                 // 32 KiB
 constexpr int kMoeBTile = 256 * 128;                    // 32 KiB
-constexpr int kMoeStage = kMoeATile + kMoeBTile;        // 48 KiB
-constexpr int kMoeStages = 3;
+constexpr int kMoeStage = kMoeATile + kMoeBTile;        // 64 KiB
+constexpr int kMoeStages = 2;
 constexpr int kMoeScaleA = kMoeBM * 8, kMoeScaleB = 256 * 8;
-constexpr int kMoeScaleStage = kMoeScaleA + kMoeScaleB; // 3 KiB
+constexpr int kMoeScaleStage = kMoeScaleA + kMoeScaleB; // 4 KiB
 constexpr int kMoeScaleBase = kMoeStages * kMoeStage;
-constexpr int kMoeLds = kMoeScaleBase + kMoeStages * kMoeScaleStage;  // 153 KiB
-constexpr int kMoeDmaPerTile = 4 + 8 + 1 + 2;           // A, B, A scales, B scales per wave
+constexpr int kMoeLds = kMoeScaleBase + kMoeStages * kMoeScaleStage;  // 136 KiB
 
 // Global->LDS source offsets of one work item.
 struct MoeAddr {
     v4i srd_b, srd_sb;
-    uint32_t voff_a[4], voff_b[8], voff_sa, voff_sb[2];
+    uint32_t voff_b[8], voff_sb[2];  // pre-shuffled weights use voff_b[0], voff_sb[0] only
     int row_start, rows, n0, n_tile;
     bool valid;
 };
 
-template <int MODE>
+template <int MODE, bool SHUF>
 __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams p) {
-    constexpr int MT = 8, NT = 4, AD = 3, PG = 4;
+    constexpr int MT = kMoeBM / 16, NT = 4, AD = 3, PG = MT - 1 - AD;
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
     const int lane = lane_id(), w = wave_id();
-    const int n_items = *p.num_items;
+    const int n_items = scalar_load_x1(p.num_items);
     const int chunk = (n_items + (int)gridDim.x - 1) / (int)gridDim.x;
     int it = blockIdx.x * chunk;
     const int it_end = min(n_items, it + chunk);
@@ -200,8 +271,10 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
     const int nk = (Kb + 127) >> 7;
     const int tail_bytes = Kb - (nk - 1) * 128;  // valid bytes of the last K-step (16..128)
     const int rows_b = MODE == 0 ? 2 * p.N : p.N;
-    const v4i srd_a = make_srd(p.A, 0x7fffffffu);
-    const v4i srd_sa = make_srd(p.SA, 0x7fffffffu);
+    // loads per wave and K-step: A tile, B tile, A scales, B scales
+    constexpr int kDma = 8 + 8 + 1 + (SHUF ? 1 : 2);
+    const v4i srd_a = make_srd(p.A, (uint32_t)nk * (uint32_t)p.S * 128u);
+    const v4i srd_sa = make_srd(p.SA, (uint32_t)nk * (uint32_t)p.S * 8u);
 
     const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);  // same for every load index
     const bool tail_oob = (int)(chunk16 * 16) >= tail_bytes;
@@ -209,56 +282,90 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
     auto make_addr = [&](int idx, MoeAddr& a) {
         a.valid = idx < it_end;
         if (!a.valid) idx = it_end - 1;  // harmless values; every load of an invalid set is zero-sized
-        const MoeItem item = p.items[idx];
-        const int expert = to_sgpr(item.expert);
-        a.row_start = to_sgpr(item.row_start);
-        a.rows = to_sgpr(item.rows);
-        a.n_tile = to_sgpr(item.n_tile);
+        const v4i item = scalar_load_x4(p.items + idx);  // {expert, row_start, rows, n_tile}
+        const int expert = item.x;
+        a.row_start = item.y;
+        a.rows = item.z;
+        a.n_tile = item.w;
         a.n0 = a.n_tile * (MODE == 0 ? 128 : 256);
-        a.srd_b = make_srd(p.B + (size_t)expert * p.b_expert_stride, (uint32_t)rows_b * (uint32_t)p.b_pitch);
-        a.srd_sb = make_srd(p.SB + (size_t)expert * p.sb_expert_stride, (uint32_t)rows_b * (uint32_t)p.sb_pitch);
-        // weight row held by LDS row R of the B tile
-        auto b_row = [&](int R) -> int {
-            if (MODE == 1) return min(a.n0 + b_row_to_col(R), p.N - 1);
-            const int wn = R >> 6, t = (R >> 4) & 3, r = R & 15;
-            const int hcol = 32 * wn + 8 * (r >> 2) + 4 * (t >> 1) + (r & 3);
-            return (t & 1) * p.N + min(a.n0 + hcol, p.N - 1);
-        };
-        auto a_row = [&](int R) -> uint32_t { return (uint32_t)(a.row_start + min(R, a.rows - 1)); };
+        if (SHUF) {
+            // one contiguous run of nk tiles per (expert, n-tile)
+            a.srd_b = make_srd(p.B + (size_t)expert * p.b_expert_stride + (size_t)a.n_tile * nk * kMoeBTile,
+                               (uint32_t)nk * kMoeBTile);
+            a.srd_sb = make_srd(p.SB + (size_t)expert * p.sb_expert_stride + (size_t)a.n_tile * nk * kMoeScaleB,
+                                (uint32_t)nk * kMoeScaleB);
+        } else {
+            a.srd_b = make_srd(p.B + (size_t)expert * p.b_expert_stride, (uint32_t)rows_b * (uint32_t)p.b_pitch);
+            a.srd_sb = make_srd(p.SB + (size_t)expert * p.sb_expert_stride, (uint32_t)rows_b * (uint32_t)p.sb_pitch);
+        }
+        auto b_row = [&](int R) -> int { return moe_b_row(MODE, R, a.n_tile, p.N); };
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            a.voff_a[i] = a_row(8 * (i * 4 + w) + (lane >> 3)) * (uint32_t)p.a_pitch + chunk16 * 16u;
+        for (int i = 0; i < (SHUF ? 1 : 8); ++i)
+            a.voff_b[i] = SHUF ? (uint32_t)(w * 1024 + lane * 16)
+                               : (uint32_t)b_row(8 * (i * 4 + w) + (lane >> 3)) * (uint32_t)p.b_pitch + chunk16 * 16u;
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            a.voff_b[i] = (uint32_t)b_row(8 * (i * 4 + w) + (lane >> 3)) * (uint32_t)p.b_pitch + chunk16 * 16u;
-        a.voff_sa = a_row(32 * w + (lane >> 1)) * (uint32_t)p.sa_pitch + (lane & 1) * 4u;
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-            a.voff_sb[j] = (uint32_t)b_row(32 * (2 * w + j) + (lane >> 1)) * (uint32_t)p.sb_pitch + (lane & 1) * 4u;
+        for (int j = 0; j < (SHUF ? 1 : 2); ++j)
+            a.voff_sb[j] = SHUF ? (uint32_t)(w * 512 + lane * 16)
+                                : (uint32_t)b_row(32 * (2 * w + j) + (lane >> 1)) * (uint32_t)p.sb_pitch + (lane & 1) * 4u;
     };
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-    const uint32_t lds_sa_wave = to_sgpr(lds0 + kMoeScaleBase + (uint32_t)w * 256u);
+    const uint32_t lds_sa_wave = to_sgpr(lds0 + kMoeScaleBase + (uint32_t)w * 512u);
     const uint32_t lds_sb_wave = to_sgpr(lds0 + kMoeScaleBase + kMoeScaleA + (uint32_t)w * 512u);
 
-    // All 15 loads of K-step kt of item `a` into `stage`. For an invalid item or past the end
-    // of K they are issued against zero-sized buffers (no traffic), which keeps the number of
+#if defined(HK_EXP_TIMING)
+    long long* tlog = (long long*)p.out_scales_dbg;
+    int tcount = 0;
+#define HK_T(tag) do { if (tlog && blockIdx.x == 3 && threadIdx.x == 0 && tcount < 4000) { tlog[tcount++] = ((long long)(tag) << 48) | (__builtin_readcyclecounter() & 0xffffffffffffll); } } while (0)
+#else
+#define HK_T(tag) do {} while (0)
+#endif
+    // A-side offsets do not depend on the work item: LDS row R of the A tile is row
+    // row_start + R of the K-step's contiguous [S][128] block (rows past the tile's count are
+    // other rows of the matrix, or out of range = zero, and their results are never stored).
+    uint32_t voff_a[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) voff_a[i] = (uint32_t)(8 * (i * 4 + w) + (lane >> 3)) * 128u + chunk16 * 16u;
+    const uint32_t voff_sa = (uint32_t)(w * 512 + lane * 16);  // 32 lanes x 16 bytes = 64 rows of scales
+
+    // All loads of K-step kt of item `a` into `stage`. For an invalid item or past the end of K
+    // they are issued against zero-sized buffers (no traffic), which keeps the number of
     // outstanding loads per K-step uniform.
     auto issue_tile = [&](const MoeAddr& a, int stage, int kt) {
         v4i sa = srd_a, sb = a.srd_b, ssa = srd_sa, ssb = a.srd_sb;
         if (!a.valid || kt >= nk) { sa.z = 0; sb.z = 0; ssa.z = 0; ssb.z = 0; }
-        const bool last = (kt == nk - 1) && tail_oob;
-        const uint32_t k0 = (uint32_t)kt * 128u;
+#if defined(HK_EXP_NOA)
+        sa.z = 0; ssa.z = 0;
+#endif
+#if defined(HK_EXP_NOB)
+        sb.z = 0; ssb.z = 0;
+#endif
+        const uint32_t row_base = (uint32_t)kt * (uint32_t)p.S + (uint32_t)a.row_start;
         const uint32_t dst = lds_wave + (uint32_t)stage * kMoeStage;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(sa, dst + i * 4096, last ? 0x80000000u : a.voff_a[i], k0);
+        for (int i = 0; i < 8; ++i) dma16(sa, dst + i * 4096, voff_a[i], row_base * 128u);
+        HK_T(10);
+        if (SHUF) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) dma16(sb, dst + kMoeATile + i * 4096, last ? 0x80000000u : a.voff_b[i], k0);
-        dma4(ssa, lds_sa_wave + (uint32_t)stage * kMoeScaleStage, a.voff_sa, (uint32_t)kt * 8u);
+            for (int i = 0; i < 8; ++i)
+                dma16(sb, dst + kMoeATile + i * 4096, a.voff_b[0], (uint32_t)kt * kMoeBTile + i * 4096);
+        } else {
+            const bool last = (kt == nk - 1) && tail_oob;  // 16-byte chunks past the end of K read as zero
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-            dma4(ssb, lds_sb_wave + (uint32_t)stage * kMoeScaleStage + j * 256, a.voff_sb[j], (uint32_t)kt * 8u);
+            for (int i = 0; i < 8; ++i)
+                dma16(sb, dst + kMoeATile + i * 4096, last ? 0x80000000u : a.voff_b[i], (uint32_t)kt * 128u);
+        }
+        HK_T(11);
+        dma16_lanes(ssa, lds_sa_wave + (uint32_t)stage * kMoeScaleStage, voff_sa, row_base * 8u, 0xffffffffull);
+        if (SHUF) {
+            dma16_lanes(ssb, lds_sb_wave + (uint32_t)stage * kMoeScaleStage, a.voff_sb[0],
+                        (uint32_t)kt * kMoeScaleB, 0xffffffffull);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                dma4(ssb, lds_sb_wave + (uint32_t)stage * kMoeScaleStage + j * 256, a.voff_sb[j], (uint32_t)kt * 8u);
+        }
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
@@ -285,7 +392,12 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
         f.hi = *(lds_v4i_t*)(uintptr_t)(hi + imm);
         return f;
     };
+    // Inline asm so that the MFMA keeps its place between the LDS reads of the schedule (a
+    // builtin call is free to sink below them); the 256 accumulator registers live in AGPRs.
     auto mfma = [&](v4f& acc, const v4i& x, const v4i& y, int sx, int sy) {
+#if defined(HK_EXP_NOMFMA)
+        return;
+#endif
         asm volatile(
             "v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"
             : "+a"(acc)
@@ -296,15 +408,15 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
     Frag4 bf[NT], af[4];
     v2i bs[NT], as[4];
     MoeAddr cur, nxt;
-    int mt_act = 0;
 
     // One K-step on LDS stage `st` (a run-time value, so that a single copy of this code
     // serves the whole ring): read this step's B fragments and first A fragments, then MFMA
     // groups with the A fragments read three groups ahead; after group PG one barrier, then the
-    // refill of stage `st` with the K-step three positions ahead in the stream (which may
+    // refill of stage `st` with the K-step two positions ahead in the stream (which may
     // belong to the next work item). The LDS latency exposed at the start of every step is
     // hidden behind the weight stream from HBM that bounds this kernel.
     auto step = [&](int kt, int st) {
+        HK_T(1);
         uint32_t a_lo = a_lo0 + (uint32_t)st * kMoeStage, a_hi = a_hi0 + (uint32_t)st * kMoeStage;
         uint32_t b_lo = b_lo0 + (uint32_t)st * kMoeStage, b_hi = b_hi0 + (uint32_t)st * kMoeStage;
         uint32_t sa_rd = sa_rd0 + (uint32_t)st * kMoeScaleStage, sb_rd = sb_rd0 + (uint32_t)st * kMoeScaleStage;
@@ -323,41 +435,43 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
 #pragma unroll
         for (int n = 0; n < NT; ++n) shift_scale(bs[n]);
         shift_scale(as[0]);
-        __builtin_amdgcn_sched_barrier(0);
+        slot_fence();
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-            if (m < mt_act) {
+            // All MT groups always run, also for tiles with fewer than 128 real rows: the rows
+            // beyond the tile's count are clamped duplicates whose results are not stored. A
+            // branch around a group would make the accumulators live across control flow (and
+            // cost register copies every K-step), and the MFMA time of a full step is still
+            // below the time its weight tile needs to arrive from HBM.
 #pragma unroll
-                for (int n = 0; n < NT; ++n) {
-                    mfma(acc[m][n], bf[n].lo, af[m & 3].lo, bs[n].x, as[m & 3].x);
-                    if (n == 0 && m <= PG) {
-                        af[(m + AD) & 3] = rd_frag(a_lo, a_hi, (m + AD) * 2048);
-                        as[(m + AD) & 3] = rd_scale(sa_rd, m + AD);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
+            for (int n = 0; n < NT; ++n) {
+                mfma(acc[m][n], bf[n].lo, af[m & 3].lo, bs[n].x, as[m & 3].x);
+                if (n == 0 && m <= PG) {
+                    af[(m + AD) & 3] = rd_frag(a_lo, a_hi, (m + AD) * 2048);
+                    as[(m + AD) & 3] = rd_scale(sa_rd, m + AD);
                 }
+                slot_fence();
+            }
 #pragma unroll
-                for (int n = 0; n < NT; ++n) {
-                    mfma(acc[m][n], bf[n].hi, af[m & 3].hi, bs[n].y, as[m & 3].y);
-                    if (n == 2 && m + 1 < MT) shift_scale(as[(m + 1) & 3]);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            } else if (m <= PG) {
-                // keep the rotation of A buffers in step with the full schedule
-                af[(m + AD) & 3] = rd_frag(a_lo, a_hi, (m + AD) * 2048);
-                as[(m + AD) & 3] = rd_scale(sa_rd, m + AD);
-                shift_scale(as[(m + 1) & 3]);
-                __builtin_amdgcn_sched_barrier(0);
+            for (int n = 0; n < NT; ++n) {
+                mfma(acc[m][n], bf[n].hi, af[m & 3].hi, bs[n].y, as[m & 3].y);
+                if (n == 2 && m + 1 < MT) shift_scale(as[(m + 1) & 3]);
+                slot_fence();
             }
             if (m == PG) {
                 // all reads of stage st are issued; wait for them and for the next K-step's
-                // loads (the K-step after that may stay in flight), then refill stage st
+                // loads (issued one K-step ago), then refill stage st with the K-step after that
+                HK_T(2);
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                wait_vmcnt<kMoeDmaPerTile>();
+                HK_T(3);
+                wait_vmcnt<0>();
+                HK_T(4);
                 block_barrier();
-                if (kt + 3 < nk) issue_tile(cur, st, kt + 3);
-                else issue_tile(nxt, st, kt + 3 - nk);
-                __builtin_amdgcn_sched_barrier(0);
+                HK_T(5);
+                if (kt + 2 < nk) issue_tile(cur, st, kt + 2);
+                else issue_tile(nxt, st, kt + 2 - nk);
+                HK_T(6);
+                slot_fence();
             }
         }
     };
@@ -383,10 +497,13 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
                 }
             }
         } else {
+            // h goes out as K-step-major tiles for the down GEMM: column c of row pos lives in
+            // K-step c / 256 at byte (c % 256) / 2; this wave's 32 columns are one MX block.
             uint8_t* hq = (uint8_t*)p.out0;
-            const int hcol0 = n0 + 32 * w;  // this wave's MX block of h
+            const int hcol0 = n0 + 32 * w;
             const bool col_ok = hcol0 < p.N;
-            const bool last_n = a.n_tile == p.n_tiles_n - 1;
+            const size_t kt2 = (size_t)(hcol0 >> 8);
+            const int byte0 = ((hcol0 & 255) >> 1) + 4 * (int)g, blk = (hcol0 & 255) >> 5;
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 const int row = 16 * m + (int)r;
@@ -407,15 +524,9 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
                 amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
                 const int e = mx_block_exponent(amax);
                 if (row < rows && col_ok) {
-                    const size_t pos = (size_t)(row_start + row);
-                    *(uint32_t*)(hq + pos * p.out_pitch + (hcol0 >> 1) + 4 * g) = pack8_e2m1(h, e);
-                    if (g == 0) p.out_scales[pos * p.out_scale_pitch + (hcol0 >> 5)] = (uint8_t)(e + 127);
-                }
-                if (row < rows && last_n && w == 0 && g == 1) {
-                    // neutral scale bytes in the padding columns of this row
-                    const size_t pos = (size_t)(row_start + row);
-                    for (int c = p.N >> 5; c < p.out_scale_pitch; ++c)
-                        p.out_scales[pos * p.out_scale_pitch + c] = 127;
+                    const size_t tile_row = kt2 * p.S + (size_t)(row_start + row);
+                    *(uint32_t*)(hq + tile_row * 128 + byte0) = pack8_e2m1(h, e);
+                    if (g == 0) p.out_scales[tile_row * 8 + blk] = (uint8_t)(e + 127);
                 }
             }
         }
@@ -427,15 +538,14 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
     make_addr(it, cur);
     for (;;) {
         make_addr(look ? it + 1 : it_end, nxt);
-        mt_act = (cur.rows + 15) >> 4;
         if (need_prologue) {
-            // three K-steps in flight, fragments of the first in registers
+            // two K-steps in flight
 #pragma unroll
-            for (int s3 = 0; s3 < 3; ++s3) {
+            for (int s3 = 0; s3 < 2; ++s3) {
                 if (s3 < nk) issue_tile(cur, s3, s3);
                 else issue_tile(nxt, s3, s3 - nk);  // only without lookahead: zero-sized
             }
-            wait_vmcnt<2 * kMoeDmaPerTile>();
+            wait_vmcnt<kDma>();
             block_barrier();
             st = 0;
         }
@@ -445,10 +555,12 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
             for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
         for (int kt = 0; kt < nk; ++kt) {
             step(kt, st);
-            st = st == 2 ? 0 : st + 1;
+            st ^= 1;
         }
+        HK_T(7);
         mfma_drain();
         epilogue(cur);
+        HK_T(8);
         if (++it >= it_end) break;
         if (look) {
             cur = nxt;
@@ -505,9 +617,9 @@ static int num_compute_units() {
     return cus;
 }
 
-template <int MODE>
+template <int MODE, bool SHUF>
 static int launch_moe_gemm(MoeGemmParams p, int max_items, hipStream_t s) {
-    auto kern = moe_mxfp4_gemm_kernel<MODE>;
+    auto kern = moe_mxfp4_gemm_kernel<MODE, SHUF>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMoeLds) !=
@@ -516,7 +628,7 @@ static int launch_moe_gemm(MoeGemmParams p, int max_items, hipStream_t s) {
         configured = true;
     }
     const int nk = (p.K / 2 + 127) / 128;
-    p.lookahead = nk >= 3 ? 1 : 0;
+    p.lookahead = nk >= 2 ? 1 : 0;
     // persistent: one workgroup per CU walks a contiguous range of items; otherwise one per item
     const int grid = p.lookahead ? min(max_items, num_compute_units()) : max_items;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), kMoeLds, s, p);
@@ -550,6 +662,31 @@ extern "C" int hk_moe_unpermute(const void* o_bf16, const float* w, const int32_
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
+extern "C" int hk_moe_mxfp4_preshuffle_bytes(int E, int N, int K, int mode, size_t* w_bytes, size_t* s_bytes) {
+    if (!w_bytes || !s_bytes) return HK_ERR_NULL_POINTER;
+    if (E <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || (mode != 0 && mode != 1)) return HK_ERR_BAD_SHAPE;
+    const size_t n_tiles = mode == 0 ? (N + 127) / 128 : (N + 255) / 256;
+    const size_t nk = (K / 2 + 127) / 128;
+    *w_bytes = (size_t)E * n_tiles * nk * kMoeBTile;
+    *s_bytes = (size_t)E * n_tiles * nk * kMoeScaleB;
+    return HK_OK;
+}
+
+extern "C" int hk_moe_mxfp4_preshuffle(const void* w, const void* scales, int scale_pitch, int E, int N, int K,
+                                       int mode, void* out_w, void* out_s, void* stream) {
+    if (!w || !scales || !out_w || !out_s) return HK_ERR_NULL_POINTER;
+    if (E <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || scale_pitch < K / 32 || (mode != 0 && mode != 1))
+        return HK_ERR_BAD_SHAPE;
+    if (((uintptr_t)w | (uintptr_t)out_w) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    const int n_tiles = mode == 0 ? (N + 127) / 128 : (N + 255) / 256;
+    const long long total = (long long)E * n_tiles * ((K / 2 + 127) / 128) * 2048;
+    if ((total + 255) / 256 >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(moe_preshuffle_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, (const uint8_t*)w, (const uint8_t*)scales, E, N, K, scale_pitch, mode,
+                       n_tiles, (uint8_t*)out_w, (uint8_t*)out_s);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
 // Workspace layout of hk_moe_mxfp4_forward (all regions 256-byte aligned).
 struct MoeWs {
     size_t ids, w, sorted, offsets, inv, sort_ws, items1, items2, nitems, xq, xs, hq, hs, o, total;
@@ -568,8 +705,9 @@ static MoeWs moe_ws_layout(int T, int H, int I, int E, int k) {
     L.items1 = take((size_t)L.max_items1 * sizeof(MoeItem));
     L.items2 = take((size_t)L.max_items2 * sizeof(MoeItem));
     L.nitems = take(8);
-    L.xq = take(S * (H / 2)); L.xs = take(S * round_up(H / 32, 8));
-    L.hq = take(S * (I / 2)); L.hs = take(S * round_up(I / 32, 8));
+    const size_t nk1 = (H / 2 + 127) / 128, nk2 = (I / 2 + 127) / 128;  // K-step-major activation tiles
+    L.xq = take(nk1 * S * 128); L.xs = take(nk1 * S * 8);
+    L.hq = take(nk2 * S * 128); L.hs = take(nk2 * S * 8);
     L.o = take(S * (size_t)H * 2);
     L.total = off;
     return L;
@@ -586,8 +724,8 @@ static int moe_mxfp4_check(int T, int H, int I, int E, int k, int w13_scale_pitc
     if (w13_scale_pitch < H / 32 || (w13_scale_pitch % 8) != 0 || w2_scale_pitch < I / 32 ||
         (w2_scale_pitch % 8) != 0)
         return HK_ERR_BAD_SHAPE;
-    if ((long long)T * k >= (1ll << 24) || (long long)T * k * (I / 2) >= (1ll << 31) ||
-        (long long)T * k * (H / 2) >= (1ll << 31) || (long long)2 * I * (H / 2) >= (1ll << 31) ||
+    if ((long long)T * k >= (1ll << 24) || (long long)T * k * (((I / 2 + 127) / 128) * 128) >= (1ll << 31) ||
+        (long long)T * k * (((H / 2 + 127) / 128) * 128) >= (1ll << 31) || (long long)2 * I * (H / 2) >= (1ll << 31) ||
         (long long)H * (I / 2) >= (1ll << 31))
         return HK_ERR_BAD_SHAPE;
     return HK_OK;
@@ -598,12 +736,14 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
                                     int w13_scale_pitch, const void* w2, const void* w2_scales,
                                     int w2_scale_pitch, const float* topk_w, const int32_t* sorted_slots,
                                     const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
-                                    int T, int H, int I, int E, int k, void* workspace, size_t workspace_bytes,
-                                    void* stream) {
+                                    int T, int H, int I, int E, int k, int weight_layout, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
     if (!x_bf16 || !w13 || !w13_scales || !w2 || !w2_scales || !topk_w || !sorted_slots || !expert_offsets ||
         !slot_to_pos || !y_bf16)
         return HK_ERR_NULL_POINTER;
-    int st = moe_mxfp4_check(T, H, I, E, k, w13_scale_pitch, w2_scale_pitch);
+    if (weight_layout != 0 && weight_layout != 1) return HK_ERR_UNSUPPORTED;
+    int st = moe_mxfp4_check(T, H, I, E, k, weight_layout ? round_up(H / 32, 8) : w13_scale_pitch,
+                             weight_layout ? round_up(I / 32, 8) : w2_scale_pitch);
     if (st != HK_OK) return st;
     const MoeWs L = moe_ws_layout(T, H, I, E, k);
     if (!workspace || workspace_bytes < L.total) return HK_ERR_WORKSPACE;
@@ -613,12 +753,13 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
     hipStream_t s = (hipStream_t)stream;
     uint8_t* ws = (uint8_t*)workspace;
     const int S = T * k;
-    const int xs_pitch = round_up(H / 32, 8), hs_pitch = round_up(I / 32, 8);
 
     {
-        const long long threads = (long long)S * xs_pitch * 4;
+        const long long threads = (long long)S * ((H / 2 + 127) / 128) * 32;
         hipLaunchKernelGGL(mxfp4_quantize_permute_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
-                           (const uint16_t*)x_bf16, sorted_slots, k, S, H, ws + L.xq, ws + L.xs, xs_pitch);
+                           (const uint16_t*)x_bf16, sorted_slots, k, S, H, ws + L.xq, ws + L.xs);
+        if (I % 256)
+            hipLaunchKernelGGL(moe_pad_tiled_kernel, dim3((S + 7) / 8), dim3(256), 0, s, ws + L.hq, ws + L.hs, S, I);
     }
     int32_t* nitems = (int32_t*)(ws + L.nitems);
     hipLaunchKernelGGL(moe_build_items_kernel, dim3(1), dim3(512), 0, s, expert_offsets, E, (I + 127) / 128,
@@ -627,25 +768,39 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
                        (MoeItem*)(ws + L.items2), nitems + 1);
 
     MoeGemmParams p{};
-    p.A = ws + L.xq; p.SA = ws + L.xs; p.a_pitch = H / 2; p.sa_pitch = xs_pitch;
+    p.A = ws + L.xq; p.SA = ws + L.xs; p.S = S;
     p.B = (const uint8_t*)w13; p.SB = (const uint8_t*)w13_scales;
     p.b_pitch = H / 2; p.sb_pitch = w13_scale_pitch;
     p.b_expert_stride = (long long)2 * I * (H / 2); p.sb_expert_stride = (long long)2 * I * w13_scale_pitch;
+    if (weight_layout) {
+        const long long tiles = (long long)((I + 127) / 128) * ((H / 2 + 127) / 128);
+        p.b_expert_stride = tiles * kMoeBTile; p.sb_expert_stride = tiles * kMoeScaleB;
+    }
+    p.shuffled = weight_layout;
     p.items = (const MoeItem*)(ws + L.items1); p.num_items = nitems;
-    p.out0 = ws + L.hq; p.out_scales = ws + L.hs; p.out_pitch = I / 2; p.out_scale_pitch = hs_pitch;
+    p.out0 = ws + L.hq; p.out_scales = ws + L.hs;
     p.K = H; p.N = I; p.n_tiles_n = (I + 127) / 128;
-    st = launch_moe_gemm<0>(p, L.max_items1, s);
+    st = weight_layout ? launch_moe_gemm<0, true>(p, L.max_items1, s) : launch_moe_gemm<0, false>(p, L.max_items1, s);
     if (st != HK_OK) return st;
 
     MoeGemmParams q{};
-    q.A = ws + L.hq; q.SA = ws + L.hs; q.a_pitch = I / 2; q.sa_pitch = hs_pitch;
+    q.A = ws + L.hq; q.SA = ws + L.hs; q.S = S;
     q.B = (const uint8_t*)w2; q.SB = (const uint8_t*)w2_scales;
     q.b_pitch = I / 2; q.sb_pitch = w2_scale_pitch;
     q.b_expert_stride = (long long)H * (I / 2); q.sb_expert_stride = (long long)H * w2_scale_pitch;
+    if (weight_layout) {
+        const long long tiles = (long long)((H + 255) / 256) * ((I / 2 + 127) / 128);
+        q.b_expert_stride = tiles * kMoeBTile; q.sb_expert_stride = tiles * kMoeScaleB;
+    }
+    q.shuffled = weight_layout;
     q.items = (const MoeItem*)(ws + L.items2); q.num_items = nitems + 1;
-    q.out0 = ws + L.o; q.out_scales = nullptr; q.out_pitch = 0; q.out_scale_pitch = 0;
+    q.out0 = ws + L.o; q.out_scales = nullptr;
     q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
-    st = launch_moe_gemm<1>(q, L.max_items2, s);
+#if defined(HK_EXP_TIMING)
+    q.out_scales_dbg = ws + L.xq;  // debug only: xq is dead once the first GEMM has run
+    p.out_scales_dbg = ws + L.o;  // debug only: o is not written before the second GEMM
+#endif
+    st = weight_layout ? launch_moe_gemm<1, true>(q, L.max_items2, s) : launch_moe_gemm<1, false>(q, L.max_items2, s);
     if (st != HK_OK) return st;
 
     return hk_moe_unpermute(ws + L.o, topk_w, slot_to_pos, T, k, H, y_bf16, stream);
@@ -654,9 +809,12 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
 extern "C" int hk_moe_mxfp4_forward(const void* x_bf16, const float* router_logits, const void* w13,
                                     const void* w13_scales, int w13_scale_pitch, const void* w2,
                                     const void* w2_scales, int w2_scale_pitch, void* y_bf16, int T, int H, int I,
-                                    int E, int k, void* workspace, size_t workspace_bytes, void* stream) {
+                                    int E, int k, int weight_layout, void* workspace, size_t workspace_bytes,
+                                    void* stream) {
     if (!router_logits) return HK_ERR_NULL_POINTER;
-    int st = moe_mxfp4_check(T, H, I, E, k, w13_scale_pitch, w2_scale_pitch);
+    if (weight_layout != 0 && weight_layout != 1) return HK_ERR_UNSUPPORTED;
+    int st = moe_mxfp4_check(T, H, I, E, k, weight_layout ? round_up(H / 32, 8) : w13_scale_pitch,
+                             weight_layout ? round_up(I / 32, 8) : w2_scale_pitch);
     if (st != HK_OK) return st;
     const MoeWs L = moe_ws_layout(T, H, I, E, k);
     if (!workspace || workspace_bytes < L.total) return HK_ERR_WORKSPACE;
@@ -669,5 +827,5 @@ extern "C" int hk_moe_mxfp4_forward(const void* x_bf16, const float* router_logi
     return hk_moe_mxfp4_experts(x_bf16, w13, w13_scales, w13_scale_pitch, w2, w2_scales, w2_scale_pitch,
                                 (const float*)(ws + L.w), (const int32_t*)(ws + L.sorted),
                                 (const int32_t*)(ws + L.offsets), (const int32_t*)(ws + L.inv), y_bf16, T, H, I, E,
-                                k, workspace, workspace_bytes, stream);
+                                k, weight_layout, workspace, workspace_bytes, stream);
 }

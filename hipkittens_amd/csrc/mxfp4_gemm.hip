@@ -46,12 +46,6 @@ __device__ __forceinline__ void mfma_fp4_acc(v4f& acc, const v4i& x, const v4i& 
         : "v"(x), "v"(y), "v"(sx), "v"(sy));
 }
 
-__device__ __forceinline__ v4f mfma_fp4(v4i x, v4i y, v4f c, int sx, int sy) {
-    v8i x8 = __builtin_shufflevector(x, x, 0, 1, 2, 3, 0, 1, 2, 3);
-    v8i y8 = __builtin_shufflevector(y, y, 0, 1, 2, 3, 0, 1, 2, 3);
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x8, y8, c, 4, 4, 0, sx, 0, sy);
-}
-
 template <bool EDGE>
 __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,

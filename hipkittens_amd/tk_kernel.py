@@ -194,6 +194,61 @@ def moe_mxfp4_workspace_bytes(T: int, H: int, I: int, E: int, k: int) -> int:
     return int(_lib.load_library().hk_moe_mxfp4_workspace_bytes(T, H, I, E, k))
 
 
+class MoeMxfp4ShuffledWeights:
+    """Expert weights in the pre-shuffled tile layout (hk_moe_mxfp4_preshuffle): built once,
+    offline, from the plain [E, rows, K/2] + [E, rows, K/32] tensors."""
+
+    def __init__(self, w13, w13_scales, w2, w2_scales, E: int, H: int, I: int):
+        self.w13, self.w13_scales, self.w2, self.w2_scales = w13, w13_scales, w2, w2_scales
+        self.E, self.H, self.I = E, H, I
+
+    @staticmethod
+    def _shuffle(w, scales, N: int, K: int, mode: int):
+        lib = _lib.load_library()
+        E = w.shape[0]
+        import ctypes
+        wb, sb = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        _lib.check(lib.hk_moe_mxfp4_preshuffle_bytes(E, N, K, mode, ctypes.byref(wb), ctypes.byref(sb)),
+                   "moe_mxfp4_preshuffle_bytes")
+        out_w = torch.empty(wb.value, dtype=torch.uint8, device=w.device)
+        out_s = torch.empty(sb.value, dtype=torch.uint8, device=w.device)
+        st = lib.hk_moe_mxfp4_preshuffle(w.data_ptr(), scales.data_ptr(), scales.shape[2], E, N, K, mode,
+                                         out_w.data_ptr(), out_s.data_ptr(), _stream(w))
+        _lib.check(st, "moe_mxfp4_preshuffle")
+        return out_w, out_s
+
+    @classmethod
+    def from_plain(cls, w13, w13_scales, w2, w2_scales):
+        _check_tensor(w13, "w13", _FP4, 3)
+        _check_tensor(w13_scales, "w13_scales", _E8M0, 3)
+        _check_tensor(w2, "w2", _FP4, 3)
+        _check_tensor(w2_scales, "w2_scales", _E8M0, 3)
+        E, twoI, Hh = w13.shape
+        H, I = 2 * Hh, twoI // 2
+        if tuple(w2.shape) != (E, H, I // 2) or tuple(w13_scales.shape[:2]) != (E, twoI) or \
+                tuple(w2_scales.shape[:2]) != (E, H) or w13_scales.shape[2] < H // 32 or w2_scales.shape[2] < I // 32:
+            raise RuntimeError("shape mismatch between w13, w13_scales, w2 and w2_scales")
+        a, sa = cls._shuffle(w13, w13_scales, I, H, 0)
+        b, sb = cls._shuffle(w2, w2_scales, H, I, 1)
+        return cls(a, sa, b, sb, E, H, I)
+
+
+def _moe_weight_args(x, weights_or_w13, w13_scales, w2, w2_scales, y):
+    """-> (T, H, I, E, layout, w13_ptr, s13_ptr, s13_pitch, w2_ptr, s2_ptr, s2_pitch)"""
+    _check_tensor(x, "x", _BF16, 2)
+    _check_tensor(y, "y", _BF16, 2)
+    T, H = x.shape
+    if isinstance(weights_or_w13, MoeMxfp4ShuffledWeights):
+        W = weights_or_w13
+        if W.H != H or tuple(y.shape) != (T, H):
+            raise RuntimeError("shape mismatch between x, y and the shuffled weights")
+        return (T, H, W.I, W.E, 1, W.w13.data_ptr(), W.w13_scales.data_ptr(), 0, W.w2.data_ptr(),
+                W.w2_scales.data_ptr(), 0)
+    T, H, I, E = _check_moe_weights(x, weights_or_w13, w13_scales, w2, w2_scales, y)
+    return (T, H, I, E, 0, weights_or_w13.data_ptr(), w13_scales.data_ptr(), w13_scales.shape[2], w2.data_ptr(),
+            w2_scales.data_ptr(), w2_scales.shape[2])
+
+
 def _check_moe_weights(x, w13, w13_scales, w2, w2_scales, y):
     _check_tensor(x, "x", _BF16, 2)
     _check_tensor(w13, "w13", _FP4, 3)
@@ -212,8 +267,9 @@ def _check_moe_weights(x, w13, w13_scales, w2, w2_scales, y):
 
 def dispatch_moe_mxfp4_experts(x, w13, w13_scales, w2, w2_scales, weights, sorted_slots, expert_offsets,
                                slot_to_pos, y, workspace) -> None:
-    """Expert MLP on routed + sorted tokens (see include/hk355.h: hk_moe_mxfp4_experts)."""
-    T, H, I, E = _check_moe_weights(x, w13, w13_scales, w2, w2_scales, y)
+    """Expert MLP on routed + sorted tokens (see include/hk355.h: hk_moe_mxfp4_experts). `w13` may be
+    a MoeMxfp4ShuffledWeights, in which case w13_scales, w2 and w2_scales are ignored (pass None)."""
+    T, H, I, E, layout, pw13, ps13, pitch13, pw2, ps2, pitch2 = _moe_weight_args(x, w13, w13_scales, w2, w2_scales, y)
     _check_tensor(weights, "weights", _F32, 2)
     _check_tensor(sorted_slots, "sorted_slots", _I32, 1)
     _check_tensor(expert_offsets, "expert_offsets", _I32, 1)
@@ -224,22 +280,21 @@ def dispatch_moe_mxfp4_experts(x, w13, w13_scales, w2, w2_scales, weights, sorte
             slot_to_pos.shape[0] != T * k:
         raise RuntimeError("shape mismatch between routing tensors")
     st = _lib.load_library().hk_moe_mxfp4_experts(
-        x.data_ptr(), w13.data_ptr(), w13_scales.data_ptr(), w13_scales.shape[2], w2.data_ptr(),
-        w2_scales.data_ptr(), w2_scales.shape[2], weights.data_ptr(), sorted_slots.data_ptr(),
-        expert_offsets.data_ptr(), slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, workspace.data_ptr(),
-        workspace.numel(), _stream(x))
+        x.data_ptr(), pw13, ps13, pitch13, pw2, ps2, pitch2, weights.data_ptr(), sorted_slots.data_ptr(),
+        expert_offsets.data_ptr(), slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, layout,
+        workspace.data_ptr(), workspace.numel(), _stream(x))
     _lib.check(st, "dispatch_moe_mxfp4_experts")
 
 
 def dispatch_moe_mxfp4(x, router_logits, w13, w13_scales, w2, w2_scales, y, topk: int, workspace) -> None:
-    """Whole MXFP4 MoE layer: top-k softmax routing, sort, expert MLP, un-permute into y."""
-    T, H, I, E = _check_moe_weights(x, w13, w13_scales, w2, w2_scales, y)
+    """Whole MXFP4 MoE layer: top-k softmax routing, sort, expert MLP, un-permute into y. `w13` may be
+    a MoeMxfp4ShuffledWeights (then pass None for w13_scales, w2, w2_scales)."""
+    T, H, I, E, layout, pw13, ps13, pitch13, pw2, ps2, pitch2 = _moe_weight_args(x, w13, w13_scales, w2, w2_scales, y)
     _check_tensor(router_logits, "router_logits", _F32, 2)
     _check_tensor(workspace, "workspace", (torch.uint8,), 1)
     if tuple(router_logits.shape) != (T, E):
         raise RuntimeError("router_logits must be [T, E]")
     st = _lib.load_library().hk_moe_mxfp4_forward(
-        x.data_ptr(), router_logits.data_ptr(), w13.data_ptr(), w13_scales.data_ptr(), w13_scales.shape[2],
-        w2.data_ptr(), w2_scales.data_ptr(), w2_scales.shape[2], y.data_ptr(), T, H, I, E, int(topk),
-        workspace.data_ptr(), workspace.numel(), _stream(x))
+        x.data_ptr(), router_logits.data_ptr(), pw13, ps13, pitch13, pw2, ps2, pitch2, y.data_ptr(), T, H, I, E,
+        int(topk), layout, workspace.data_ptr(), workspace.numel(), _stream(x))
     _lib.check(st, "dispatch_moe_mxfp4")

@@ -132,21 +132,33 @@ int hk_moe_unpermute(const void* o_bf16, const float* w, const int32_t* slot_to_
 
 size_t hk_moe_mxfp4_workspace_bytes(int T, int H, int I, int E, int k);
 
+/* Offline weight pre-shuffle (weight_layout = 1 below). For every expert, n-tile and K-step the
+ * 256 x 128-byte weight tile is stored contiguously in the order the kernel keeps it in LDS
+ * (K zero-padded to whole 256-element steps), scales likewise as 256 x 8-byte tiles, so that the
+ * GEMMs stream weights from HBM in 32 KiB bursts. mode 0: gate+up matrix [E, 2N, K/2] with N = I,
+ * K = H; mode 1: down matrix [E, N, K/2] with N = H, K = I. scales [E, rows, scale_pitch]. */
+int hk_moe_mxfp4_preshuffle_bytes(int E, int N, int K, int mode, size_t* w_bytes, size_t* s_bytes);
+int hk_moe_mxfp4_preshuffle(const void* w, const void* scales, int scale_pitch, int E, int N, int K,
+                            int mode, void* out_w, void* out_s, void* stream);
+
 /* Expert MLP for tokens that are already routed and sorted (outputs of hk_moe_topk_* and
  * hk_moe_sort): activation quantization, grouped gate+up GEMM with SiLU-mul and MX
- * re-quantization, grouped down GEMM, weighted un-permute. */
+ * re-quantization, grouped down GEMM, weighted un-permute. weight_layout 0: w13 / w2 and their
+ * scales in the plain row-major layout above; 1: outputs of hk_moe_mxfp4_preshuffle (the scale
+ * pitch arguments are then ignored). Both layouts give bit-identical results. */
 int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const void* w13_scales,
                          int w13_scale_pitch, const void* w2, const void* w2_scales,
                          int w2_scale_pitch, const float* topk_w, const int32_t* sorted_slots,
                          const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
-                         int T, int H, int I, int E, int k, void* workspace, size_t workspace_bytes,
-                         void* stream);
+                         int T, int H, int I, int E, int k, int weight_layout, void* workspace,
+                         size_t workspace_bytes, void* stream);
 
 /* Whole layer: top-k softmax routing of router_logits [T,E] fp32, sort, expert MLP. */
 int hk_moe_mxfp4_forward(const void* x_bf16, const float* router_logits, const void* w13,
                          const void* w13_scales, int w13_scale_pitch, const void* w2,
                          const void* w2_scales, int w2_scale_pitch, void* y_bf16, int T, int H, int I,
-                         int E, int k, void* workspace, size_t workspace_bytes, void* stream);
+                         int E, int k, int weight_layout, void* workspace, size_t workspace_bytes,
+                         void* stream);
 
 #ifdef __cplusplus
 }

@@ -73,16 +73,22 @@ def test_unpermute_matches_oracle(hk):
 
 
 def _run_forward(hk, x, logits, w13p, w13s, w2p, w2s, k):
+    """Runs the layer with plain and with pre-shuffled weights; both must agree bit for bit."""
     T, H = x.shape
     E, twoI, _ = w13p.shape
     I = twoI // 2
     ws = torch.empty(hk.tk_kernel.moe_mxfp4_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=DEV)
     y = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
-    hk.tk_kernel.dispatch_moe_mxfp4(
-        _to_bf16_tensor(x), torch.from_numpy(logits).to(DEV), torch.from_numpy(w13p).to(DEV),
-        torch.from_numpy(_pad(w13s)).to(DEV), torch.from_numpy(w2p).to(DEV), torch.from_numpy(_pad(w2s)).to(DEV),
-        y, k, ws)
+    tw = [torch.from_numpy(w13p).to(DEV), torch.from_numpy(_pad(w13s)).to(DEV), torch.from_numpy(w2p).to(DEV),
+          torch.from_numpy(_pad(w2s)).to(DEV)]
+    xt, lt = _to_bf16_tensor(x), torch.from_numpy(logits).to(DEV)
+    hk.tk_kernel.dispatch_moe_mxfp4(xt, lt, tw[0], tw[1], tw[2], tw[3], y, k, ws)
     torch.cuda.synchronize()
+    shuf = hk.tk_kernel.MoeMxfp4ShuffledWeights.from_plain(*tw)
+    y2 = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_mxfp4(xt, lt, shuf, None, None, None, y2, k, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16)), "plain and pre-shuffled weights disagree"
     return y.float().cpu().numpy()
 
 
@@ -148,6 +154,11 @@ def test_moe_mxfp4_full_shape_properties(hk):
     hk.tk_kernel.dispatch_moe_mxfp4(x, logits, w13p, w13s, w2p, w2s, y, k, ws)
     torch.cuda.synchronize()
     assert torch.isfinite(y.float()).all()
+    shuf = hk.tk_kernel.MoeMxfp4ShuffledWeights.from_plain(w13p, w13s, w2p, w2s)
+    y3 = torch.empty_like(y)
+    hk.tk_kernel.dispatch_moe_mxfp4(x, logits, shuf, None, None, None, y3, k, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(y3, y)  # pre-shuffled weight layout: identical arithmetic
     # (1) token permutation: y is a per-token function -> permuting inputs permutes outputs exactly
     perm = torch.randperm(T, device=DEV, generator=g)
     y2 = torch.empty_like(y)
