@@ -232,10 +232,7 @@ struct MoeGemmParams {
     int K;                   // contraction length in elements
     int N;                   // MODE 0: I (h columns; weight rows i and I+i); MODE 1: output columns
     int n_tiles_n;
-#if defined(HK_EXP_TIMING)
-    void* out_scales_dbg;
-#endif
-    int lookahead;           // 1: persistent workgroups prefetch across items (needs >= 2 K-steps)
+    int lookahead;           // 1: the load stream runs ahead across work-item boundaries
     int shuffled;            // 1: B / SB are in the pre-shuffled tile layout (see moe_preshuffle_kernel)
 };
 
@@ -251,20 +248,35 @@ constexpr int kMoeLds = kMoeScaleBase + kMoeStages * kMoeScaleStage;  // 136 KiB
 // Global->LDS source offsets of one work item.
 struct MoeAddr {
     v4i srd_b, srd_sb;
-    uint32_t voff_b[8], voff_sb[2];  // pre-shuffled weights use voff_b[0], voff_sb[0] only
+    uint32_t voff_b[4], voff_sb;  // pre-shuffled weights use voff_b[0] only
     int row_start, rows, n0, n_tile;
     bool valid;
 };
 
+// 8 waves (two per SIMD), wave (wm, wn) = (w / 4, w % 4) owns the 16-row fragments 2m + wm
+// (m = 0..7: even or odd fragments, so that both waves of a SIMD have work whatever the tile's
+// row count) x weight rows [64 wn, +64) of the 256 x 256 tile. The K loop is deliberately simple - wait for the K-step's
+// operands, one barrier, start the loads of the next K-step into the other LDS stage, compute -
+// because the two waves of a SIMD cover for each other: while one is held up issuing loads or
+// waiting for LDS, the other feeds the matrix pipe (a single wave per SIMD cannot issue the
+// 16-cycle FP4 MFMA back to back, nor issue loads and MFMAs at the same time).
 template <int MODE, bool SHUF>
-__global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams p) {
-    constexpr int MT = kMoeBM / 16, NT = 4, AD = 3, PG = MT - 1 - AD;
+__global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams p) {
+    constexpr int NW = 8, MT = 8, NT = 4;
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
     const int lane = lane_id(), w = wave_id();
+    const int wm = w >> 2, wn = w & 3;
+    // Item assignment. Workgroup ids go round robin over the 8 XCDs; each XCD takes a contiguous
+    // range of the item list and its workgroups walk that range with a stride equal to their
+    // number, so that at any time the CUs of one XCD work on consecutive items = the same
+    // expert's rows with neighbouring n-tiles, and share that expert's activation tile in the
+    // XCD's L2 (each weight tile is needed exactly once anyway).
     const int n_items = scalar_load_x1(p.num_items);
-    const int chunk = (n_items + (int)gridDim.x - 1) / (int)gridDim.x;
-    int it = blockIdx.x * chunk;
-    const int it_end = min(n_items, it + chunk);
+    const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+    const int it_stride = ((int)gridDim.x - xcd + kNumXcd - 1) / kNumXcd;  // workgroups on this XCD
+    const int per_xcd = (n_items + kNumXcd - 1) / kNumXcd;
+    int it = xcd * per_xcd + slot;
+    const int it_end = min(n_items, (xcd + 1) * per_xcd);
     if (it >= it_end) return;
 
     const int Kb = p.K >> 1;                 // contraction bytes per row
@@ -272,11 +284,13 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
     const int tail_bytes = Kb - (nk - 1) * 128;  // valid bytes of the last K-step (16..128)
     const int rows_b = MODE == 0 ? 2 * p.N : p.N;
     // loads per wave and K-step: A tile, B tile, A scales, B scales
-    constexpr int kDma = 8 + 8 + 1 + (SHUF ? 1 : 2);
+    constexpr int kDma = 4 + 4 + 1 + 1;
     const v4i srd_a = make_srd(p.A, (uint32_t)nk * (uint32_t)p.S * 128u);
     const v4i srd_sa = make_srd(p.SA, (uint32_t)nk * (uint32_t)p.S * 8u);
 
-    const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);  // same for every load index
+    // Load i of this wave fills LDS rows 8*(i*NW + w) .. +8 of a tile; lane l lands in row +l/8,
+    // physical chunk l%8 and fetches logical chunk swz(row, l%8), the same for every i.
+    const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);
     const bool tail_oob = (int)(chunk16 * 16) >= tail_bytes;
 
     auto make_addr = [&](int idx, MoeAddr& a) {
@@ -300,34 +314,24 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
         }
         auto b_row = [&](int R) -> int { return moe_b_row(MODE, R, a.n_tile, p.N); };
 #pragma unroll
-        for (int i = 0; i < (SHUF ? 1 : 8); ++i)
+        for (int i = 0; i < (SHUF ? 1 : 4); ++i)
             a.voff_b[i] = SHUF ? (uint32_t)(w * 1024 + lane * 16)
-                               : (uint32_t)b_row(8 * (i * 4 + w) + (lane >> 3)) * (uint32_t)p.b_pitch + chunk16 * 16u;
-#pragma unroll
-        for (int j = 0; j < (SHUF ? 1 : 2); ++j)
-            a.voff_sb[j] = SHUF ? (uint32_t)(w * 512 + lane * 16)
-                                : (uint32_t)b_row(32 * (2 * w + j) + (lane >> 1)) * (uint32_t)p.sb_pitch + (lane & 1) * 4u;
+                               : (uint32_t)b_row(8 * (i * NW + w) + (lane >> 3)) * (uint32_t)p.b_pitch + chunk16 * 16u;
+        a.voff_sb = SHUF ? (uint32_t)(w * 256 + lane * 16)
+                         : (uint32_t)b_row(32 * w + (lane >> 1)) * (uint32_t)p.sb_pitch + (lane & 1) * 4u;
     };
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-    const uint32_t lds_sa_wave = to_sgpr(lds0 + kMoeScaleBase + (uint32_t)w * 512u);
-    const uint32_t lds_sb_wave = to_sgpr(lds0 + kMoeScaleBase + kMoeScaleA + (uint32_t)w * 512u);
+    const uint32_t lds_s_wave = to_sgpr(lds0 + kMoeScaleBase + (uint32_t)w * 256u);
 
-#if defined(HK_EXP_TIMING)
-    long long* tlog = (long long*)p.out_scales_dbg;
-    int tcount = 0;
-#define HK_T(tag) do { if (tlog && blockIdx.x == 3 && threadIdx.x == 0 && tcount < 4000) { tlog[tcount++] = ((long long)(tag) << 48) | (__builtin_readcyclecounter() & 0xffffffffffffll); } } while (0)
-#else
-#define HK_T(tag) do {} while (0)
-#endif
     // A-side offsets do not depend on the work item: LDS row R of the A tile is row
     // row_start + R of the K-step's contiguous [S][128] block (rows past the tile's count are
     // other rows of the matrix, or out of range = zero, and their results are never stored).
-    uint32_t voff_a[8];
+    uint32_t voff_a[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) voff_a[i] = (uint32_t)(8 * (i * 4 + w) + (lane >> 3)) * 128u + chunk16 * 16u;
-    const uint32_t voff_sa = (uint32_t)(w * 512 + lane * 16);  // 32 lanes x 16 bytes = 64 rows of scales
+    for (int i = 0; i < 4; ++i) voff_a[i] = (uint32_t)(8 * (i * NW + w) + (lane >> 3)) * 128u + chunk16 * 16u;
+    const uint32_t voff_sa = (uint32_t)(w * 256 + lane * 16);  // 16 lanes x 16 bytes = 32 rows of scales
 
     // All loads of K-step kt of item `a` into `stage`. For an invalid item or past the end of K
     // they are issued against zero-sized buffers (no traffic), which keeps the number of
@@ -335,56 +339,36 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
     auto issue_tile = [&](const MoeAddr& a, int stage, int kt) {
         v4i sa = srd_a, sb = a.srd_b, ssa = srd_sa, ssb = a.srd_sb;
         if (!a.valid || kt >= nk) { sa.z = 0; sb.z = 0; ssa.z = 0; ssb.z = 0; }
-#if defined(HK_EXP_NOA)
-        sa.z = 0; ssa.z = 0;
-#endif
-#if defined(HK_EXP_NOB)
-        sb.z = 0; ssb.z = 0;
-#endif
         const uint32_t row_base = (uint32_t)kt * (uint32_t)p.S + (uint32_t)a.row_start;
         const uint32_t dst = lds_wave + (uint32_t)stage * kMoeStage;
+        const uint32_t sdst = lds_s_wave + (uint32_t)stage * kMoeScaleStage;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) dma16(sa, dst + i * 4096, voff_a[i], row_base * 128u);
-        HK_T(10);
+        for (int i = 0; i < 4; ++i) dma16(sa, dst + i * NW * 1024, voff_a[i], row_base * 128u);
         if (SHUF) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                dma16(sb, dst + kMoeATile + i * 4096, a.voff_b[0], (uint32_t)kt * kMoeBTile + i * 4096);
+            for (int i = 0; i < 4; ++i)
+                dma16(sb, dst + kMoeATile + i * NW * 1024, a.voff_b[0], (uint32_t)kt * kMoeBTile + i * NW * 1024);
         } else {
             const bool last = (kt == nk - 1) && tail_oob;  // 16-byte chunks past the end of K read as zero
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                dma16(sb, dst + kMoeATile + i * 4096, last ? 0x80000000u : a.voff_b[i], (uint32_t)kt * 128u);
+            for (int i = 0; i < 4; ++i)
+                dma16(sb, dst + kMoeATile + i * NW * 1024, last ? 0x80000000u : a.voff_b[i], (uint32_t)kt * 128u);
         }
-        HK_T(11);
-        dma16_lanes(ssa, lds_sa_wave + (uint32_t)stage * kMoeScaleStage, voff_sa, row_base * 8u, 0xffffffffull);
-        if (SHUF) {
-            dma16_lanes(ssb, lds_sb_wave + (uint32_t)stage * kMoeScaleStage, a.voff_sb[0],
-                        (uint32_t)kt * kMoeScaleB, 0xffffffffull);
-        } else {
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-                dma4(ssb, lds_sb_wave + (uint32_t)stage * kMoeScaleStage + j * 256, a.voff_sb[j], (uint32_t)kt * 8u);
-        }
+        dma16_lanes(ssa, sdst, voff_sa, row_base * 8u, 0xffffull);
+        if (SHUF) dma16_lanes(ssb, sdst + kMoeScaleA, a.voff_sb, (uint32_t)kt * kMoeScaleB, 0xffffull);
+        else dma4(ssb, sdst + kMoeScaleA, a.voff_sb, (uint32_t)kt * 8u);
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
     const uint32_t rd_lo = r * 128u + swz_chunk(r, g) * 16u;
     const uint32_t rd_hi = r * 128u + swz_chunk(r, g + 4) * 16u;
     // stage 0 addresses; a K-step on stage st adds st * kMoeStage (scales: st * kMoeScaleStage)
-    const uint32_t a_lo0 = lds0 + rd_lo, a_hi0 = lds0 + rd_hi;
-    const uint32_t b_lo0 = lds0 + kMoeATile + w * (64 * 128) + rd_lo;
-    const uint32_t b_hi0 = lds0 + kMoeATile + w * (64 * 128) + rd_hi;
-    const uint32_t sa_rd0 = lds0 + kMoeScaleBase + r * 8u;
-    const uint32_t sb_rd0 = lds0 + kMoeScaleBase + kMoeScaleA + (w * 64 + r) * 8u;
-    const uint32_t sh = 8u * g;
-    auto rd_scale = [&](uint32_t base, int f) -> v2i {
-        return *(lds_v2i_t*)(uintptr_t)(base + f * 128);
-    };
-    auto shift_scale = [&](v2i& s) {
-        s.x = (int)((uint32_t)s.x >> sh);
-        s.y = (int)((uint32_t)s.y >> sh);
-    };
+    const uint32_t a_lo0 = lds0 + wm * 2048 + rd_lo, a_hi0 = lds0 + wm * 2048 + rd_hi;
+    const uint32_t b_lo0 = lds0 + kMoeATile + wn * (64 * 128) + rd_lo;
+    const uint32_t b_hi0 = lds0 + kMoeATile + wn * (64 * 128) + rd_hi;
+    const uint32_t sa_rd0 = lds0 + kMoeScaleBase + (wm * 16 + r) * 8u;
+    const uint32_t sb_rd0 = lds0 + kMoeScaleBase + kMoeScaleA + (wn * 64 + r) * 8u;
+    const uint32_t sh = 8u * g;  // byte g of each scale dword belongs to this lane
     struct Frag4 { v4i lo, hi; };
     auto rd_frag = [&](uint32_t lo, uint32_t hi, int imm) -> Frag4 {
         Frag4 f;
@@ -392,86 +376,40 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
         f.hi = *(lds_v4i_t*)(uintptr_t)(hi + imm);
         return f;
     };
-    // Inline asm so that the MFMA keeps its place between the LDS reads of the schedule (a
-    // builtin call is free to sink below them); the 256 accumulator registers live in AGPRs.
-    auto mfma = [&](v4f& acc, const v4i& x, const v4i& y, int sx, int sy) {
-#if defined(HK_EXP_NOMFMA)
-        return;
-#endif
-        asm volatile(
-            "v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"
-            : "+a"(acc)
-            : "v"(x), "v"(y), "v"(sx), "v"(sy));
+    auto rd_scale = [&](uint32_t base, int f) -> v2i {
+        v2i s = *(lds_v2i_t*)(uintptr_t)(base + f * 128);
+        s.x = (int)((uint32_t)s.x >> sh);
+        s.y = (int)((uint32_t)s.y >> sh);
+        return s;
     };
 
     v4f acc[MT][NT];
-    Frag4 bf[NT], af[4];
-    v2i bs[NT], as[4];
     MoeAddr cur, nxt;
 
-    // One K-step on LDS stage `st` (a run-time value, so that a single copy of this code
-    // serves the whole ring): read this step's B fragments and first A fragments, then MFMA
-    // groups with the A fragments read three groups ahead; after group PG one barrier, then the
-    // refill of stage `st` with the K-step two positions ahead in the stream (which may
-    // belong to the next work item). The LDS latency exposed at the start of every step is
-    // hidden behind the weight stream from HBM that bounds this kernel.
-    auto step = [&](int kt, int st) {
-        HK_T(1);
+    // MFMAs of one K-step on LDS stage st. Fragments past the tile's row count are skipped (the
+    // condition is uniform for the wave).
+    auto compute = [&](int st, int rows) {
         uint32_t a_lo = a_lo0 + (uint32_t)st * kMoeStage, a_hi = a_hi0 + (uint32_t)st * kMoeStage;
         uint32_t b_lo = b_lo0 + (uint32_t)st * kMoeStage, b_hi = b_hi0 + (uint32_t)st * kMoeStage;
         uint32_t sa_rd = sa_rd0 + (uint32_t)st * kMoeScaleStage, sb_rd = sb_rd0 + (uint32_t)st * kMoeScaleStage;
         // keep the (large) bases in registers so that fragment offsets stay immediates
         asm volatile("" : "+v"(a_lo), "+v"(a_hi), "+v"(b_lo), "+v"(b_hi), "+v"(sa_rd), "+v"(sb_rd));
+        Frag4 bf[NT];
+        v2i bs[NT];
 #pragma unroll
         for (int n = 0; n < NT; ++n) {
             bf[n] = rd_frag(b_lo, b_hi, n * 2048);
             bs[n] = rd_scale(sb_rd, n);
         }
 #pragma unroll
-        for (int m = 0; m < AD; ++m) {
-            af[m] = rd_frag(a_lo, a_hi, m * 2048);
-            as[m] = rd_scale(sa_rd, m);
-        }
-#pragma unroll
-        for (int n = 0; n < NT; ++n) shift_scale(bs[n]);
-        shift_scale(as[0]);
-        slot_fence();
-#pragma unroll
         for (int m = 0; m < MT; ++m) {
-            // All MT groups always run, also for tiles with fewer than 128 real rows: the rows
-            // beyond the tile's count are clamped duplicates whose results are not stored. A
-            // branch around a group would make the accumulators live across control flow (and
-            // cost register copies every K-step), and the MFMA time of a full step is still
-            // below the time its weight tile needs to arrive from HBM.
+            if (16 * (2 * m + wm) < rows) {
+                const Frag4 af = rd_frag(a_lo, a_hi, m * 4096);
+                const v2i as = rd_scale(sa_rd, 2 * m);
 #pragma unroll
-            for (int n = 0; n < NT; ++n) {
-                mfma(acc[m][n], bf[n].lo, af[m & 3].lo, bs[n].x, as[m & 3].x);
-                if (n == 0 && m <= PG) {
-                    af[(m + AD) & 3] = rd_frag(a_lo, a_hi, (m + AD) * 2048);
-                    as[(m + AD) & 3] = rd_scale(sa_rd, m + AD);
-                }
-                slot_fence();
-            }
+                for (int n = 0; n < NT; ++n) acc[m][n] = mfma_fp4(bf[n].lo, af.lo, acc[m][n], bs[n].x, as.x);
 #pragma unroll
-            for (int n = 0; n < NT; ++n) {
-                mfma(acc[m][n], bf[n].hi, af[m & 3].hi, bs[n].y, as[m & 3].y);
-                if (n == 2 && m + 1 < MT) shift_scale(as[(m + 1) & 3]);
-                slot_fence();
-            }
-            if (m == PG) {
-                // all reads of stage st are issued; wait for them and for the next K-step's
-                // loads (issued one K-step ago), then refill stage st with the K-step after that
-                HK_T(2);
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                HK_T(3);
-                wait_vmcnt<0>();
-                HK_T(4);
-                block_barrier();
-                HK_T(5);
-                if (kt + 2 < nk) issue_tile(cur, st, kt + 2);
-                else issue_tile(nxt, st, kt + 2 - nk);
-                HK_T(6);
-                slot_fence();
+                for (int n = 0; n < NT; ++n) acc[m][n] = mfma_fp4(bf[n].hi, af.hi, acc[m][n], bs[n].y, as.y);
             }
         }
     };
@@ -482,12 +420,12 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
             uint16_t* out = (uint16_t*)p.out0;
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
-                const int row = 16 * m + (int)r;
+                const int row = 16 * (2 * m + wm) + (int)r;
                 if (row >= rows) continue;
                 const size_t pos = (size_t)(row_start + row);
 #pragma unroll
                 for (int q = 0; q < NT / 2; ++q) {
-                    const int col = n0 + w * 64 + 32 * q + 8 * (int)g;
+                    const int col = n0 + wn * 64 + 32 * q + 8 * (int)g;
                     if (col + 8 > p.N) continue;  // N % 8 == 0
                     const v4f x = acc[m][2 * q], y = acc[m][2 * q + 1];
                     v4i o4;
@@ -500,13 +438,14 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
             // h goes out as K-step-major tiles for the down GEMM: column c of row pos lives in
             // K-step c / 256 at byte (c % 256) / 2; this wave's 32 columns are one MX block.
             uint8_t* hq = (uint8_t*)p.out0;
-            const int hcol0 = n0 + 32 * w;
+            const int hcol0 = n0 + 32 * wn;
             const bool col_ok = hcol0 < p.N;
             const size_t kt2 = (size_t)(hcol0 >> 8);
             const int byte0 = ((hcol0 & 255) >> 1) + 4 * (int)g, blk = (hcol0 & 255) >> 5;
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
-                const int row = 16 * m + (int)r;
+                const int row = 16 * (2 * m + wm) + (int)r;
+                if (16 * (2 * m + wm) >= rows) continue;  // uniform: the whole fragment is padding
                 float h[8];
 #pragma unroll
                 for (int q = 0; q < 2; ++q) {
@@ -532,46 +471,50 @@ __global__ __launch_bounds__(256) void moe_mxfp4_gemm_kernel(const MoeGemmParams
         }
     };
 
+    // Stream of K-steps over this workgroup's items; the loads of stream position s+1 are in
+    // flight while position s is computed, across item boundaries when `lookahead` is set.
+#if defined(HK_EXP_TIMING)
+    long long* tlog = (MODE == 1) ? (long long*)p.out_scales : nullptr;
+    int tcount = 0;
+#define HK_T(tag) do { if (tlog && blockIdx.x == 3 && (threadIdx.x == 0 || threadIdx.x == 256) && tcount < 1900) { tlog[(threadIdx.x >> 8) * 2000 + tcount++] = ((long long)(tag) << 48) | (__builtin_readcyclecounter() & 0xffffffffffffll); } } while (0)
+#else
+#define HK_T(tag) do {} while (0)
+#endif
     const bool look = p.lookahead != 0;
-    bool need_prologue = true;
-    int st = 0;  // LDS stage of the next K-step to compute
+    int st = 0;
     make_addr(it, cur);
+    issue_tile(cur, 0, 0);
     for (;;) {
-        make_addr(look ? it + 1 : it_end, nxt);
-        if (need_prologue) {
-            // two K-steps in flight
-#pragma unroll
-            for (int s3 = 0; s3 < 2; ++s3) {
-                if (s3 < nk) issue_tile(cur, s3, s3);
-                else issue_tile(nxt, s3, s3 - nk);  // only without lookahead: zero-sized
-            }
-            wait_vmcnt<kDma>();
-            block_barrier();
-            st = 0;
-        }
+        make_addr(look ? it + it_stride : it_end, nxt);
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
             for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
         for (int kt = 0; kt < nk; ++kt) {
-            step(kt, st);
+            HK_T(1);
+            wait_vmcnt<0>();   // this wave's part of K-step kt has landed
+            HK_T(2);
+            block_barrier();   // ... everyone's; and everyone is done reading the other stage
+            HK_T(3);
+            if (kt + 1 < nk) issue_tile(cur, st ^ 1, kt + 1);
+            else issue_tile(nxt, st ^ 1, 0);
+            HK_T(4);
+            compute(st, cur.rows);
             st ^= 1;
         }
-        HK_T(7);
-        mfma_drain();
+        HK_T(5);
         epilogue(cur);
-        HK_T(8);
-        if (++it >= it_end) break;
+        HK_T(6);
+        it += it_stride;
+        if (it >= it_end) break;
         if (look) {
             cur = nxt;
         } else {
-            // no cross-item prefetch: drain the ring and start the next item from scratch
+            make_addr(it, cur);
             wait_vmcnt<0>();
             block_barrier();
-            make_addr(it, cur);
-            need_prologue = true;
+            issue_tile(cur, st, 0);
         }
-        need_prologue = !look;
     }
     wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
 }
@@ -627,11 +570,10 @@ static int launch_moe_gemm(MoeGemmParams p, int max_items, hipStream_t s) {
             return HK_ERR_LAUNCH;
         configured = true;
     }
-    const int nk = (p.K / 2 + 127) / 128;
-    p.lookahead = nk >= 2 ? 1 : 0;
+    p.lookahead = 1;
     // persistent: one workgroup per CU walks a contiguous range of items; otherwise one per item
     const int grid = p.lookahead ? min(max_items, num_compute_units()) : max_items;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), kMoeLds, s, p);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kMoeLds, s, p);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
@@ -795,11 +737,10 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
     q.shuffled = weight_layout;
     q.items = (const MoeItem*)(ws + L.items2); q.num_items = nitems + 1;
     q.out0 = ws + L.o; q.out_scales = nullptr;
-    q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
 #if defined(HK_EXP_TIMING)
-    q.out_scales_dbg = ws + L.xq;  // debug only: xq is dead once the first GEMM has run
-    p.out_scales_dbg = ws + L.o;  // debug only: o is not written before the second GEMM
+    q.out_scales = ws + L.xq;  // debug only: timestamps go where the (dead) quantized x was
 #endif
+    q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
     st = weight_layout ? launch_moe_gemm<1, true>(q, L.max_items2, s) : launch_moe_gemm<1, false>(q, L.max_items2, s);
     if (st != HK_OK) return st;
 
