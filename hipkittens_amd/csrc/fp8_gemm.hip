@@ -234,15 +234,8 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_kernel(
     // end of K are issued against a zero-sized buffer (out of range for every lane, no
     // memory traffic), so that no step needs a differently scheduled body.
     auto step = [&]<int P>(int kt) {
-#if defined(HK_EXP_SAMEK)
-        const uint32_t k2 = 0;
-#else
         const uint32_t k2 = (uint32_t)(kt + 2) * BK;
-#endif
         v4i sa = srd_a, sb = srd_b;
-#if defined(HK_EXP_NODMA)
-        sa.z = 0; sb.z = 0;
-#endif
         if (kt + 2 >= nk) { sa.z = 0; sb.z = 0; }
 #pragma unroll
         for (int m = 0; m < MT; ++m) {

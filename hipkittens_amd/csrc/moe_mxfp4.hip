@@ -5,14 +5,14 @@
 // interleaved FP8/MXFP4 kernels of this library (LDS-direct loads into swizzled 128-byte-row
 // tiles, ds_read_b128 fragments, v_mfma_scale_f32_16x16x128_f8f6f4 with in-MFMA e8m0 scales).
 //
-// Grouped GEMM: a work item is (m-tile, n-tile) where an m-tile is up to 256 consecutive rows
-// (sorted positions) of one expert, so that at MoE shapes (100-300 rows per expert) an expert's
-// weight tile is streamed from HBM once; the item list is built on the device from
-// expert_offsets. A workgroup (4 waves, one per SIMD) computes a 256 x 256 tile per item; every
-// wave spans all 256 rows and owns 64 of the 256 weight rows. Weights dominate HBM traffic, so
-// workgroups are persistent: each walks a contiguous range of items and the two-stage LDS ring
-// keeps running across item boundaries, so the next item's first K-steps load while the
-// current item's epilogue runs.
+// Grouped GEMM: a work item is (m-tile, n-tile) where an m-tile is up to 128 consecutive rows
+// (sorted positions) of one expert; the item list is built on the device from expert_offsets.
+// A workgroup (8 waves, two per SIMD) computes a 128 x 256 tile per item. Weights dominate HBM
+// traffic, so workgroups are persistent and the LDS ring (three stages, two K-steps of operands
+// in flight) keeps running across item boundaries: the next item's first K-steps load while
+// the current item's epilogue runs. Items that share an expert run at the same time on the CUs
+// of one XCD, so activation tiles, and the weight tile needed again by an expert's second
+// m-tile, come out of that XCD's L2 and every weight byte leaves HBM once.
 #include "gemm_tile.h"
 #include "../../include/hk355.h"
 
@@ -185,7 +185,7 @@ __global__ __launch_bounds__(256) void moe_preshuffle_kernel(const uint8_t* __re
 // tile of weight rows. Items are listed expert by expert, n-tile by n-tile, the m-tiles of one
 // (expert, n-tile) next to each other, so that a workgroup walking a contiguous range re-reads a
 // weight tile for the expert's second m-tile straight from its XCD's L2.
-constexpr int kMoeBM = 256;
+constexpr int kMoeBM = 128;
 struct MoeItem { int expert, row_start, rows, n_tile; };
 
 __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __restrict__ expert_offsets,
@@ -232,18 +232,17 @@ struct MoeGemmParams {
     int K;                   // contraction length in elements
     int N;                   // MODE 0: I (h columns; weight rows i and I+i); MODE 1: output columns
     int n_tiles_n;
-    int lookahead;           // 1: the load stream runs ahead across work-item boundaries
     int shuffled;            // 1: B / SB are in the pre-shuffled tile layout (see moe_preshuffle_kernel)
 };
 
-constexpr int kMoeATile = kMoeBM * 128;                 // 32 KiB
+constexpr int kMoeATile = kMoeBM * 128;                 // 16 KiB
 constexpr int kMoeBTile = 256 * 128;                    // 32 KiB
 constexpr int kMoeStage = kMoeATile + kMoeBTile;        // 64 KiB
-constexpr int kMoeStages = 2;
+constexpr int kMoeStages = 3;
 constexpr int kMoeScaleA = kMoeBM * 8, kMoeScaleB = 256 * 8;
 constexpr int kMoeScaleStage = kMoeScaleA + kMoeScaleB; // 4 KiB
 constexpr int kMoeScaleBase = kMoeStages * kMoeStage;
-constexpr int kMoeLds = kMoeScaleBase + kMoeStages * kMoeScaleStage;  // 136 KiB
+constexpr int kMoeLds = kMoeScaleBase + kMoeStages * kMoeScaleStage;  // 153 KiB
 
 // Global->LDS source offsets of one work item.
 struct MoeAddr {
@@ -262,7 +261,8 @@ struct MoeAddr {
 // 16-cycle FP4 MFMA back to back, nor issue loads and MFMAs at the same time).
 template <int MODE, bool SHUF>
 __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams p) {
-    constexpr int NW = 8, MT = 8, NT = 4;
+    constexpr int NW = 8, MT = kMoeBM / 32, NT = 4;   // MT fragments of 16 rows per wave
+    constexpr int NA = kMoeBM / 64;                  // A-tile loads per wave and K-step
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
     const int lane = lane_id(), w = wave_id();
     const int wm = w >> 2, wn = w & 3;
@@ -284,7 +284,9 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
     const int tail_bytes = Kb - (nk - 1) * 128;  // valid bytes of the last K-step (16..128)
     const int rows_b = MODE == 0 ? 2 * p.N : p.N;
     // loads per wave and K-step: A tile, B tile, A scales, B scales
-    constexpr int kDma = 4 + 4 + 1 + 1;
+    // (with pre-shuffled weights each wave loads one scale piece: waves 0-3 a quarter of the
+    // B scales, waves 4-7 a quarter of the A scales)
+    constexpr int kDma = NA + 4 + (SHUF ? 1 : 2);
     const v4i srd_a = make_srd(p.A, (uint32_t)nk * (uint32_t)p.S * 128u);
     const v4i srd_sa = make_srd(p.SA, (uint32_t)nk * (uint32_t)p.S * 8u);
 
@@ -317,21 +319,27 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
         for (int i = 0; i < (SHUF ? 1 : 4); ++i)
             a.voff_b[i] = SHUF ? (uint32_t)(w * 1024 + lane * 16)
                                : (uint32_t)b_row(8 * (i * NW + w) + (lane >> 3)) * (uint32_t)p.b_pitch + chunk16 * 16u;
-        a.voff_sb = SHUF ? (uint32_t)(w * 256 + lane * 16)
+        a.voff_sb = SHUF ? (uint32_t)((w & 3) * 512 + lane * 16)
                          : (uint32_t)b_row(32 * w + (lane >> 1)) * (uint32_t)p.sb_pitch + (lane & 1) * 4u;
     };
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-    const uint32_t lds_s_wave = to_sgpr(lds0 + kMoeScaleBase + (uint32_t)w * 256u);
+    // scale pieces per wave: plain weights - A scales of kMoeBM/8 rows and B scales of 32 rows for
+    // every wave; pre-shuffled - B scales of 64 rows (waves 0-3) or A scales of kMoeBM/4 rows (4-7)
+    const uint32_t sa_bytes = SHUF ? kMoeBM * 2 : kMoeBM;  // A-scale bytes per loading wave
+    const uint32_t lds_sa_wave = to_sgpr(lds0 + kMoeScaleBase + (uint32_t)(SHUF ? (w & 3) : w) * sa_bytes);
+    const uint32_t lds_sb_wave = to_sgpr(lds0 + kMoeScaleBase + kMoeScaleA + (uint32_t)(SHUF ? (w & 3) * 512 : w * 256));
 
     // A-side offsets do not depend on the work item: LDS row R of the A tile is row
     // row_start + R of the K-step's contiguous [S][128] block (rows past the tile's count are
     // other rows of the matrix, or out of range = zero, and their results are never stored).
-    uint32_t voff_a[4];
+    uint32_t voff_a[NA];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) voff_a[i] = (uint32_t)(8 * (i * NW + w) + (lane >> 3)) * 128u + chunk16 * 16u;
-    const uint32_t voff_sa = (uint32_t)(w * 256 + lane * 16);  // 16 lanes x 16 bytes = 32 rows of scales
+    for (int i = 0; i < NA; ++i) voff_a[i] = (uint32_t)(8 * (i * NW + w) + (lane >> 3)) * 128u + chunk16 * 16u;
+    // scales of kMoeBM / 8 rows per wave: kMoeBM / 16 lanes x 16 bytes
+    const uint32_t voff_sa = (uint32_t)((SHUF ? (w & 3) : w) * sa_bytes + lane * 16);
+    constexpr uint64_t kSaMask = (1ull << ((SHUF ? kMoeBM * 2 : kMoeBM) / 16)) - 1ull;
 
     // All loads of K-step kt of item `a` into `stage`. For an invalid item or past the end of K
     // they are issued against zero-sized buffers (no traffic), which keeps the number of
@@ -341,9 +349,10 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
         if (!a.valid || kt >= nk) { sa.z = 0; sb.z = 0; ssa.z = 0; ssb.z = 0; }
         const uint32_t row_base = (uint32_t)kt * (uint32_t)p.S + (uint32_t)a.row_start;
         const uint32_t dst = lds_wave + (uint32_t)stage * kMoeStage;
-        const uint32_t sdst = lds_s_wave + (uint32_t)stage * kMoeScaleStage;
+        const uint32_t sadst = lds_sa_wave + (uint32_t)stage * kMoeScaleStage;
+        const uint32_t sbdst = lds_sb_wave + (uint32_t)stage * kMoeScaleStage;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(sa, dst + i * NW * 1024, voff_a[i], row_base * 128u);
+        for (int i = 0; i < NA; ++i) dma16(sa, dst + i * NW * 1024, voff_a[i], row_base * 128u);
         if (SHUF) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -354,9 +363,13 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
             for (int i = 0; i < 4; ++i)
                 dma16(sb, dst + kMoeATile + i * NW * 1024, last ? 0x80000000u : a.voff_b[i], (uint32_t)kt * 128u);
         }
-        dma16_lanes(ssa, sdst, voff_sa, row_base * 8u, 0xffffull);
-        if (SHUF) dma16_lanes(ssb, sdst + kMoeScaleA, a.voff_sb, (uint32_t)kt * kMoeScaleB, 0xffffull);
-        else dma4(ssb, sdst + kMoeScaleA, a.voff_sb, (uint32_t)kt * 8u);
+        if (SHUF) {
+            if (w < 4) dma16_lanes(ssb, sbdst, a.voff_sb, (uint32_t)kt * kMoeScaleB, 0xffffffffull);
+            else dma16_lanes(ssa, sadst, voff_sa, row_base * 8u, kSaMask);
+        } else {
+            dma16_lanes(ssa, sadst, voff_sa, row_base * 8u, kSaMask);
+            dma4(ssb, sbdst, a.voff_sb, (uint32_t)kt * 8u);
+        }
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
@@ -385,6 +398,14 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
 
     v4f acc[MT][NT];
     MoeAddr cur, nxt;
+    // Inline asm (not the builtin) so that the MFMAs keep their place relative to the loads that
+    // are issued before / after them: a builtin call is free to sink below the asm statements.
+    auto mfma = [&](v4f& c, const v4i& x, const v4i& y, int sx, int sy) {
+        asm volatile(
+            "v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+            : "+v"(c)
+            : "v"(x), "v"(y), "v"(sx), "v"(sy));
+    };
 
     // MFMAs of one K-step on LDS stage st. Fragments past the tile's row count are skipped (the
     // condition is uniform for the wave).
@@ -407,9 +428,9 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
                 const Frag4 af = rd_frag(a_lo, a_hi, m * 4096);
                 const v2i as = rd_scale(sa_rd, 2 * m);
 #pragma unroll
-                for (int n = 0; n < NT; ++n) acc[m][n] = mfma_fp4(bf[n].lo, af.lo, acc[m][n], bs[n].x, as.x);
+                for (int n = 0; n < NT; ++n) mfma(acc[m][n], bf[n].lo, af.lo, bs[n].x, as.x);
 #pragma unroll
-                for (int n = 0; n < NT; ++n) acc[m][n] = mfma_fp4(bf[n].hi, af.hi, acc[m][n], bs[n].y, as.y);
+                for (int n = 0; n < NT; ++n) mfma(acc[m][n], bf[n].hi, af.hi, bs[n].y, as.y);
             }
         }
     };
@@ -471,50 +492,46 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
         }
     };
 
-    // Stream of K-steps over this workgroup's items; the loads of stream position s+1 are in
-    // flight while position s is computed, across item boundaries when `lookahead` is set.
-#if defined(HK_EXP_TIMING)
-    long long* tlog = (MODE == 1) ? (long long*)p.out_scales : nullptr;
-    int tcount = 0;
-#define HK_T(tag) do { if (tlog && blockIdx.x == 3 && (threadIdx.x == 0 || threadIdx.x == 256) && tcount < 1900) { tlog[(threadIdx.x >> 8) * 2000 + tcount++] = ((long long)(tag) << 48) | (__builtin_readcyclecounter() & 0xffffffffffffll); } } while (0)
-#else
-#define HK_T(tag) do {} while (0)
-#endif
-    const bool look = p.lookahead != 0;
-    int st = 0;
+    // Stream of K-steps over this workgroup's items through a ring of three LDS stages: the
+    // loads of the next two stream positions are in flight while one position is computed,
+    // across item boundaries (one position ahead only when an item has a single K-step).
+    const int depth = nk >= 2 ? 2 : 1;
+    int st = 0;  // stage of the stream position being computed
     make_addr(it, cur);
     issue_tile(cur, 0, 0);
+    if (depth == 2) issue_tile(cur, 1, 1);
     for (;;) {
-        make_addr(look ? it + it_stride : it_end, nxt);
+        make_addr(it + it_stride, nxt);
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
             for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
         for (int kt = 0; kt < nk; ++kt) {
-            HK_T(1);
-            wait_vmcnt<0>();   // this wave's part of K-step kt has landed
-            HK_T(2);
-            block_barrier();   // ... everyone's; and everyone is done reading the other stage
-            HK_T(3);
-            if (kt + 1 < nk) issue_tile(cur, st ^ 1, kt + 1);
-            else issue_tile(nxt, st ^ 1, 0);
-            HK_T(4);
+            // this wave's part of the current position has landed (younger positions may fly)
+            if (depth == 2) wait_vmcnt<kDma>(); else wait_vmcnt<0>();
+            block_barrier();   // ... everyone's; and everyone is done with the previous position
+            const int ahead = kt + depth;
+            int stage_ahead = st + depth;
+            if (stage_ahead >= 3) stage_ahead -= 3;
+            // The texture-address unit needs about as long to take a K-step's loads as the
+            // matrix pipes need for its MFMAs: the first wave of each SIMD issues its loads
+            // before computing, the second one after, so that the two overlap.
+            if (wm == 0) {
+                if (ahead < nk) issue_tile(cur, stage_ahead, ahead);
+                else issue_tile(nxt, stage_ahead, ahead - nk);
+            }
             compute(st, cur.rows);
-            st ^= 1;
+            if (wm == 1) {
+                if (ahead < nk) issue_tile(cur, stage_ahead, ahead);
+                else issue_tile(nxt, stage_ahead, ahead - nk);
+            }
+            st = st == 2 ? 0 : st + 1;
         }
-        HK_T(5);
+        mfma_drain();
         epilogue(cur);
-        HK_T(6);
         it += it_stride;
         if (it >= it_end) break;
-        if (look) {
-            cur = nxt;
-        } else {
-            make_addr(it, cur);
-            wait_vmcnt<0>();
-            block_barrier();
-            issue_tile(cur, st, 0);
-        }
+        cur = nxt;
     }
     wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
 }
@@ -570,9 +587,8 @@ static int launch_moe_gemm(MoeGemmParams p, int max_items, hipStream_t s) {
             return HK_ERR_LAUNCH;
         configured = true;
     }
-    p.lookahead = 1;
-    // persistent: one workgroup per CU walks a contiguous range of items; otherwise one per item
-    const int grid = p.lookahead ? min(max_items, num_compute_units()) : max_items;
+    // persistent: one workgroup per CU, each walking its share of the item list
+    const int grid = min(max_items, num_compute_units());
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kMoeLds, s, p);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
@@ -737,9 +753,6 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
     q.shuffled = weight_layout;
     q.items = (const MoeItem*)(ws + L.items2); q.num_items = nitems + 1;
     q.out0 = ws + L.o; q.out_scales = nullptr;
-#if defined(HK_EXP_TIMING)
-    q.out_scales = ws + L.xq;  // debug only: timestamps go where the (dead) quantized x was
-#endif
     q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
     st = weight_layout ? launch_moe_gemm<1, true>(q, L.max_items2, s) : launch_moe_gemm<1, false>(q, L.max_items2, s);
     if (st != HK_OK) return st;
