@@ -1,0 +1,32 @@
+// Pieces shared by the MoE kernels (MXFP4 and FP8 block-scaled): work items, the mapping of
+// weight rows to LDS rows of the B tile, and host helpers implemented in moe_mxfp4.hip.
+#pragma once
+#include "gemm_tile.h"
+
+namespace hk {
+
+// Row of the expert's weight matrix held by LDS row R (0..255) of the B tile of n-tile `n_tile`.
+// mode 0 (gate+up, N = I): each wave's 64 rows alternate 16 gate rows / 16 up rows of the same 16
+// h columns, permuted so that a lane ends up with 8 consecutive h columns; mode 1 (down, N = H):
+// b_row_to_col permutation (8 consecutive output columns per lane).
+__device__ __forceinline__ int moe_b_row(int mode, int R, int n_tile, int N) {
+    if (mode == 1) return min(n_tile * 256 + b_row_to_col(R), N - 1);
+    const int wn = R >> 6, t = (R >> 4) & 3, r = R & 15;
+    const int hcol = 32 * wn + 8 * (r >> 2) + 4 * (t >> 1) + (r & 3);
+    return (t & 1) * N + min(n_tile * 128 + hcol, N - 1);
+}
+
+// Work items. A work item is (m-tile, n-tile): up to kMoeBM consecutive sorted rows of one expert
+// times one tile of weight rows. Items are listed expert by expert, n-tile by n-tile, the m-tiles
+// of one (expert, n-tile) next to each other.
+constexpr int kMoeBM = 128;
+struct MoeItem { int expert, row_start, rows, n_tile; };
+
+inline int moe_round_up(int x, int m) { return (x + m - 1) / m * m; }
+// Number of CUs of the current device (cached).
+int moe_num_compute_units();
+// items[] / *num_items from expert_offsets [E+1] for GEMMs with n_tiles_n tiles of weight rows.
+void moe_launch_build_items(const int32_t* expert_offsets, int E, int n_tiles_n, MoeItem* items,
+                            int32_t* num_items, hipStream_t s);
+
+}  // namespace hk

@@ -13,7 +13,7 @@
 // the current item's epilogue runs. Items that share an expert run at the same time on the CUs
 // of one XCD, so activation tiles, and the weight tile needed again by an expert's second
 // m-tile, come out of that XCD's L2 and every weight byte leaves HBM once.
-#include "gemm_tile.h"
+#include "moe_common.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -133,17 +133,6 @@ __global__ __launch_bounds__(256) void moe_pad_tiled_kernel(uint8_t* __restrict_
 }
 
 // ---------------------------------------------------------------------- weight pre-shuffle
-// Row of the expert's weight matrix held by LDS row R (0..255) of the B tile of n-tile `n_tile`.
-// mode 0 (gate+up, N = I): each wave's 64 rows alternate 16 gate rows / 16 up rows of the same 16
-// h columns, permuted so that a lane ends up with 8 consecutive h columns; mode 1 (down, N = H):
-// b_row_to_col permutation (8 consecutive output columns per lane).
-__device__ __forceinline__ int moe_b_row(int mode, int R, int n_tile, int N) {
-    if (mode == 1) return min(n_tile * 256 + b_row_to_col(R), N - 1);
-    const int wn = R >> 6, t = (R >> 4) & 3, r = R & 15;
-    const int hcol = 32 * wn + 8 * (r >> 2) + 4 * (t >> 1) + (r & 3);
-    return (t & 1) * N + min(n_tile * 128 + hcol, N - 1);
-}
-
 // Pre-shuffled weight layout: for every expert, n-tile and K-step one contiguous 32 KiB block
 // holding the 256 x 128-byte B tile exactly as it sits in LDS (row permutation and chunk
 // swizzle applied, K zero-padded to whole K-steps), followed in a second array by the 2 KiB
@@ -179,14 +168,6 @@ __global__ __launch_bounds__(256) void moe_preshuffle_kernel(const uint8_t* __re
         for (int b = 0; b < 8; ++b) dst[b] = (kt * 8 + b < (K >> 5)) ? src[b] : (uint8_t)127;
     }
 }
-
-// ------------------------------------------------------------------------------ work items
-// A work item is (m-tile, n-tile): up to kMoeBM consecutive sorted rows of one expert times one
-// tile of weight rows. Items are listed expert by expert, n-tile by n-tile, the m-tiles of one
-// (expert, n-tile) next to each other, so that a workgroup walking a contiguous range re-reads a
-// weight tile for the expert's second m-tile straight from its XCD's L2.
-constexpr int kMoeBM = 128;
-struct MoeItem { int expert, row_start, rows, n_tile; };
 
 __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __restrict__ expert_offsets,
                                                               int E, int n_tiles_n, MoeItem* __restrict__ items,
@@ -564,9 +545,7 @@ __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __re
     }
 }
 
-static int round_up(int x, int m) { return (x + m - 1) / m * m; }
-
-static int num_compute_units() {
+int moe_num_compute_units() {
     static int cus = 0;
     if (cus == 0) {
         int dev = 0;
@@ -575,6 +554,12 @@ static int num_compute_units() {
         cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     }
     return cus;
+}
+
+void moe_launch_build_items(const int32_t* expert_offsets, int E, int n_tiles_n, MoeItem* items,
+                            int32_t* num_items, hipStream_t s) {
+    hipLaunchKernelGGL(moe_build_items_kernel, dim3(1), dim3(512), 0, s, expert_offsets, E, n_tiles_n, items,
+                       num_items);
 }
 
 template <int MODE, bool SHUF>
@@ -588,7 +573,7 @@ static int launch_moe_gemm(MoeGemmParams p, int max_items, hipStream_t s) {
         configured = true;
     }
     // persistent: one workgroup per CU, each walking its share of the item list
-    const int grid = min(max_items, num_compute_units());
+    const int grid = min(max_items, moe_num_compute_units());
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kMoeLds, s, p);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
@@ -700,8 +685,8 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
         !slot_to_pos || !y_bf16)
         return HK_ERR_NULL_POINTER;
     if (weight_layout != 0 && weight_layout != 1) return HK_ERR_UNSUPPORTED;
-    int st = moe_mxfp4_check(T, H, I, E, k, weight_layout ? round_up(H / 32, 8) : w13_scale_pitch,
-                             weight_layout ? round_up(I / 32, 8) : w2_scale_pitch);
+    int st = moe_mxfp4_check(T, H, I, E, k, weight_layout ? moe_round_up(H / 32, 8) : w13_scale_pitch,
+                             weight_layout ? moe_round_up(I / 32, 8) : w2_scale_pitch);
     if (st != HK_OK) return st;
     const MoeWs L = moe_ws_layout(T, H, I, E, k);
     if (!workspace || workspace_bytes < L.total) return HK_ERR_WORKSPACE;
@@ -720,10 +705,10 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
             hipLaunchKernelGGL(moe_pad_tiled_kernel, dim3((S + 7) / 8), dim3(256), 0, s, ws + L.hq, ws + L.hs, S, I);
     }
     int32_t* nitems = (int32_t*)(ws + L.nitems);
-    hipLaunchKernelGGL(moe_build_items_kernel, dim3(1), dim3(512), 0, s, expert_offsets, E, (I + 127) / 128,
-                       (MoeItem*)(ws + L.items1), nitems);
-    hipLaunchKernelGGL(moe_build_items_kernel, dim3(1), dim3(512), 0, s, expert_offsets, E, (H + 255) / 256,
-                       (MoeItem*)(ws + L.items2), nitems + 1);
+    moe_launch_build_items(expert_offsets, E, (I + 127) / 128,
+                       (MoeItem*)(ws + L.items1), nitems, s);
+    moe_launch_build_items(expert_offsets, E, (H + 255) / 256,
+                       (MoeItem*)(ws + L.items2), nitems + 1, s);
 
     MoeGemmParams p{};
     p.A = ws + L.xq; p.SA = ws + L.xs; p.S = S;
@@ -767,8 +752,8 @@ extern "C" int hk_moe_mxfp4_forward(const void* x_bf16, const float* router_logi
                                     void* stream) {
     if (!router_logits) return HK_ERR_NULL_POINTER;
     if (weight_layout != 0 && weight_layout != 1) return HK_ERR_UNSUPPORTED;
-    int st = moe_mxfp4_check(T, H, I, E, k, weight_layout ? round_up(H / 32, 8) : w13_scale_pitch,
-                             weight_layout ? round_up(I / 32, 8) : w2_scale_pitch);
+    int st = moe_mxfp4_check(T, H, I, E, k, weight_layout ? moe_round_up(H / 32, 8) : w13_scale_pitch,
+                             weight_layout ? moe_round_up(I / 32, 8) : w2_scale_pitch);
     if (st != HK_OK) return st;
     const MoeWs L = moe_ws_layout(T, H, I, E, k);
     if (!workspace || workspace_bytes < L.total) return HK_ERR_WORKSPACE;

@@ -20,7 +20,9 @@ def quantize_fp8_per_tensor(x: torch.Tensor):
     """(e4m3 tensor, fp32 scale) with scale = amax/448 so that x ~= q.float() * scale."""
     xf = x.float()
     amax = xf.abs().max()
-    scale = torch.where(amax > 0, amax / E4M3_MAX, torch.ones_like(amax)).to(torch.float32)
+    # tensor / tensor: a correctly rounded division on every device (dividing by a Python scalar
+    # may be turned into a multiplication by the reciprocal)
+    scale = torch.where(amax > 0, amax / torch.full_like(amax, E4M3_MAX), torch.ones_like(amax)).to(torch.float32)
     return to_e4m3_saturating(xf / scale), float(scale)
 
 
@@ -56,3 +58,18 @@ def pad_scales(scales: torch.Tensor, multiple: int = 8) -> torch.Tensor:
         return scales.contiguous()
     fill = torch.full((*scales.shape[:-1], pad), 127, dtype=scales.dtype, device=scales.device)
     return torch.cat([scales, fill], dim=-1).contiguous()
+
+
+def quantize_fp8_blocks(x: torch.Tensor, block_rows: int, block_cols: int):
+    """e4m3 with one fp32 scale per block_rows x block_cols block of the last two dims
+    (1 x 128 for activations, 128 x 128 for weights): scale = amax/448 (1 for an all-zero block).
+    Both dims must be multiples of the block. Returns (e4m3 tensor, fp32 scales [..., R/br, C/bc])."""
+    R, C = x.shape[-2:]
+    if R % block_rows or C % block_cols:
+        raise RuntimeError("quantize_fp8_blocks: dims must be multiples of the block")
+    lead = x.shape[:-2]
+    xb = x.float().reshape(*lead, R // block_rows, block_rows, C // block_cols, block_cols)
+    amax = xb.abs().amax(dim=(-3, -1))
+    s = torch.where(amax > 0, amax / torch.full_like(amax, E4M3_MAX), torch.ones_like(amax))
+    q = (xb / s[..., :, None, :, None]).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
+    return q.reshape(*lead, R, C).contiguous(), s.contiguous()

@@ -298,3 +298,77 @@ def dispatch_moe_mxfp4(x, router_logits, w13, w13_scales, w2, w2_scales, y, topk
         x.data_ptr(), router_logits.data_ptr(), pw13, ps13, pitch13, pw2, ps2, pitch2, y.data_ptr(), T, H, I, E,
         int(topk), layout, workspace.data_ptr(), workspace.numel(), _stream(x))
     _lib.check(st, "dispatch_moe_mxfp4")
+
+
+# --------------------------------------------------------------------- FP8 block-scaled MoE
+def dispatch_fp8_quantize_rows_1x128(x, q, scales) -> None:
+    """x [R,C] bf16 -> q [R,C] e4m3, scales [R,C/128] fp32 (1 x 128 blocks, scale = amax/448)."""
+    _check_tensor(x, "x", _BF16, 2)
+    _check_tensor(q, "q", _FP8, 2)
+    _check_tensor(scales, "scales", _F32, 2)
+    R, C = x.shape
+    if tuple(q.shape) != (R, C) or tuple(scales.shape) != (R, C // 128):
+        raise RuntimeError("shape mismatch between x, q and scales")
+    st = _lib.load_library().hk_fp8_quantize_rows_1x128(x.data_ptr(), R, C, q.data_ptr(), scales.data_ptr(),
+                                                        _stream(x))
+    _lib.check(st, "dispatch_fp8_quantize_rows_1x128")
+
+
+def moe_fp8blk_workspace_bytes(T: int, H: int, I: int, E: int, k: int) -> int:
+    return int(_lib.load_library().hk_moe_fp8blk_workspace_bytes(T, H, I, E, k))
+
+
+def _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y):
+    _check_tensor(x, "x", _FP8, 2)
+    _check_tensor(x_scales, "x_scales", _F32, 2)
+    _check_tensor(w13, "w13", _FP8, 3)
+    _check_tensor(w13_scales, "w13_scales", _F32, 3)
+    _check_tensor(w2, "w2", _FP8, 3)
+    _check_tensor(w2_scales, "w2_scales", _F32, 3)
+    _check_tensor(y, "y", _BF16, 2)
+    T, H = x.shape
+    E, twoI, H2 = w13.shape
+    I = twoI // 2
+    if H2 != H or H % 128 or I % 128 or tuple(w2.shape) != (E, H, I) or tuple(y.shape) != (T, H) or \
+            tuple(x_scales.shape) != (T, H // 128) or tuple(w13_scales.shape) != (E, twoI // 128, H // 128) or \
+            tuple(w2_scales.shape) != (E, H // 128, I // 128):
+        raise RuntimeError("shape mismatch between x, x_scales, w13, w13_scales, w2, w2_scales and y")
+    return T, H, I, E
+
+
+def dispatch_moe_fp8blk_experts(x, x_scales, w13, w13_scales, w2, w2_scales, weights, sorted_slots,
+                                expert_offsets, slot_to_pos, y, workspace) -> None:
+    """FP8 block-scaled expert MLP on routed + sorted tokens (include/hk355.h: hk_moe_fp8blk_experts)."""
+    T, H, I, E = _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y)
+    _check_tensor(weights, "weights", _F32, 2)
+    _check_tensor(sorted_slots, "sorted_slots", _I32, 1)
+    _check_tensor(expert_offsets, "expert_offsets", _I32, 1)
+    _check_tensor(slot_to_pos, "slot_to_pos", _I32, 1)
+    _check_tensor(workspace, "workspace", (torch.uint8,), 1)
+    k = weights.shape[1]
+    if weights.shape[0] != T or sorted_slots.shape[0] != T * k or expert_offsets.shape[0] != E + 1 or \
+            slot_to_pos.shape[0] != T * k:
+        raise RuntimeError("shape mismatch between routing tensors")
+    st = _lib.load_library().hk_moe_fp8blk_experts(
+        x.data_ptr(), x_scales.data_ptr(), w13.data_ptr(), w13_scales.data_ptr(), w2.data_ptr(),
+        w2_scales.data_ptr(), weights.data_ptr(), sorted_slots.data_ptr(), expert_offsets.data_ptr(),
+        slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, workspace.data_ptr(), workspace.numel(), _stream(x))
+    _lib.check(st, "dispatch_moe_fp8blk_experts")
+
+
+def dispatch_moe_fp8blk(x, x_scales, router_logits, router_bias, w13, w13_scales, w2, w2_scales, y, topk: int,
+                        n_group: int, topk_group: int, routed_scale: float, workspace) -> None:
+    """Whole FP8 block-scaled MoE layer with group-limited sigmoid routing."""
+    T, H, I, E = _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y)
+    _check_tensor(router_logits, "router_logits", _F32, 2)
+    if router_bias is not None:
+        _check_tensor(router_bias, "router_bias", _F32, 1)
+    _check_tensor(workspace, "workspace", (torch.uint8,), 1)
+    if tuple(router_logits.shape) != (T, E):
+        raise RuntimeError("router_logits must be [T, E]")
+    st = _lib.load_library().hk_moe_fp8blk_forward(
+        x.data_ptr(), x_scales.data_ptr(), router_logits.data_ptr(),
+        router_bias.data_ptr() if router_bias is not None else None, int(n_group), int(topk_group),
+        float(routed_scale), w13.data_ptr(), w13_scales.data_ptr(), w2.data_ptr(), w2_scales.data_ptr(),
+        y.data_ptr(), T, H, I, E, int(topk), workspace.data_ptr(), workspace.numel(), _stream(x))
+    _lib.check(st, "dispatch_moe_fp8blk")

@@ -160,6 +160,39 @@ int hk_moe_mxfp4_forward(const void* x_bf16, const float* router_logits, const v
                          int E, int k, int weight_layout, void* workspace, size_t workspace_bytes,
                          void* stream);
 
+/* ------------------------------------------------------------- FP8 block-scaled fused MoE
+ * No counterpart in the reference. DeepSeek-V3 style quantization:
+ *   x          [T, H] e4m3, x_scales [T, H/128] fp32 (one scale per 1 x 128 block: x ~ q * s)
+ *   w13        [E, 2I, H] e4m3 (rows 0..I-1 gate, I..2I-1 up), w13_scales [E, 2I/128, H/128] fp32
+ *   w2         [E, H, I] e4m3, w2_scales [E, H/128, I/128] fp32 (one scale per 128 x 128 block)
+ *   y          [T, H] bf16
+ * h = silu(x W13g^T) * (x W13u^T) is re-quantized to e4m3 with 1 x 128 scales (scale = amax/448),
+ * o = h W2^T, y[t] = sum_j w[t,j] * bf16(o). Requirements: H % 128 == 0, I % 128 == 0,
+ * E <= 512, k <= 64.
+ */
+
+/* bf16 [rows, cols] -> e4m3 [rows, cols] + fp32 scales [rows, cols/128], scale = amax/448
+ * (1 for an all-zero block), elements round to nearest even, saturating. cols % 128 == 0. */
+int hk_fp8_quantize_rows_1x128(const void* x_bf16, int rows, int cols, void* q_e4m3, float* scales,
+                               void* stream);
+
+size_t hk_moe_fp8blk_workspace_bytes(int T, int H, int I, int E, int k);
+
+/* Expert MLP for routed and sorted tokens (outputs of hk_moe_topk_* and hk_moe_sort). */
+int hk_moe_fp8blk_experts(const void* x_e4m3, const float* x_scales, const void* w13,
+                          const float* w13_scales, const void* w2, const float* w2_scales,
+                          const float* topk_w, const int32_t* sorted_slots,
+                          const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
+                          int T, int H, int I, int E, int k, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
+/* Whole layer with group-limited sigmoid routing (see hk_moe_topk_grouped_sigmoid). */
+int hk_moe_fp8blk_forward(const void* x_e4m3, const float* x_scales, const float* router_logits,
+                          const float* router_bias_or_null, int n_group, int topk_group,
+                          float routed_scale, const void* w13, const float* w13_scales, const void* w2,
+                          const float* w2_scales, void* y_bf16, int T, int H, int I, int E, int k,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

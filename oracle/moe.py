@@ -151,3 +151,34 @@ def moe_mxfp4_forward(x_bf16_as_f32, ids, w, w13_packed, w13_scales, w2_packed, 
         y += w[:, j:j + 1].astype(np.float32) * o_bf[inv[np.arange(T) * k + j]]
     return F.bf16_round(y), {"order": order, "offs": offs, "inv": inv, "xq": xq, "xs": xs,
                              "hq": hq, "hs": hs, "o": o}
+
+
+def moe_fp8blk_forward(x_codes, x_scales, ids, w, w13_codes, w13_scales, w2_codes, w2_scales):
+    """Reference forward of the FP8 block-scaled MoE. x_codes [T,H] e4m3 codes with 1x128 scales
+    [T,H/128]; w13_codes [E,2I,H] with 128x128 scales [E,2I/128,H/128]; w2_codes [E,H,I] with
+    [E,H/128,I/128]. h is re-quantized with 1x128 blocks exactly like the kernel. Returns y as
+    bf16 bits [T,H]."""
+    T, H = x_codes.shape
+    E, twoI, _ = w13_codes.shape
+    I = twoI // 2
+    k = ids.shape[1]
+    order, offs, inv = moe_sort(ids, E)
+    xd = F.dequantize_e4m3_blocks(x_codes, x_scales, 1, 128)
+    S = T * k
+    o = np.zeros((S, H), dtype=np.float32)
+    for e in range(E):
+        lo, hi = offs[e], offs[e + 1]
+        if hi == lo:
+            continue
+        tok = order[lo:hi] // k
+        w13 = F.dequantize_e4m3_blocks(w13_codes[e], w13_scales[e], 128, 128)
+        gu = xd[tok] @ w13.T
+        h = (silu(gu[:, :I]) * gu[:, I:]).astype(np.float32)
+        q, s = F.quantize_e4m3_blocks(h, 1, 128)
+        w2 = F.dequantize_e4m3_blocks(w2_codes[e], w2_scales[e], 128, 128)
+        o[lo:hi] = F.dequantize_e4m3_blocks(q, s, 1, 128) @ w2.T
+    o_bf = F.bf16_to_f32(F.bf16_round(o))
+    y = np.zeros((T, H), dtype=np.float32)
+    for j in range(k):
+        y += w[:, j:j + 1].astype(np.float32) * o_bf[inv[np.arange(T) * k + j]]
+    return F.bf16_round(y)

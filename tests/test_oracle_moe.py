@@ -126,3 +126,31 @@ def test_moe_mxfp4_forward_brute_force_tiny():
             want[t] += w[t, j] * o[0]
     got = F.bf16_to_f32(y)
     assert np.allclose(got, F.bf16_to_f32(F.bf16_round(want)), rtol=2e-2, atol=1e-6)
+
+
+def test_moe_fp8blk_forward_single_expert_reduces_to_two_gemms():
+    """E = 1, k = 1, w = 1: dequantize -> GEMM -> SiLU-mul -> 1x128 re-quantize -> GEMM, written out
+    here with explicit per-block scale products instead of dequantized matrices."""
+    rng = np.random.default_rng(5)
+    T, H, I = 6, 256, 128
+    xq, xs = F.quantize_e4m3_blocks(rng.standard_normal((T, H)).astype(np.float32), 1, 128)
+    w13q, w13s = F.quantize_e4m3_blocks((rng.standard_normal((2 * I, H)) * 0.2).astype(np.float32), 128, 128)
+    w2q, w2s = F.quantize_e4m3_blocks((rng.standard_normal((H, I)) * 0.2).astype(np.float32), 128, 128)
+    ids = np.zeros((T, 1), dtype=np.int32)
+    w = np.ones((T, 1), dtype=np.float32)
+    y = O.moe_fp8blk_forward(xq, xs, ids, w, w13q[None], w13s[None], w2q[None], w2s[None])
+    xv, wv = F.e4m3_decode(xq).astype(np.float64), F.e4m3_decode(w13q).astype(np.float64)
+    gu = np.zeros((T, 2 * I))
+    for kb in range(H // 128):
+        part = xv[:, kb * 128:(kb + 1) * 128] @ wv[:, kb * 128:(kb + 1) * 128].T
+        gu += part * xs[:, kb:kb + 1].astype(np.float64) * np.repeat(w13s[:, kb], 128)[None, :]
+    g, u = gu[:, :I], gu[:, I:]
+    h = (g / (1 + np.exp(-g)) * u).astype(np.float32)
+    hq, hs = F.quantize_e4m3_blocks(h, 1, 128)
+    o = (F.e4m3_decode(hq).astype(np.float64) * hs.astype(np.float64)) @ \
+        (F.e4m3_decode(w2q).astype(np.float64) * np.repeat(np.repeat(w2s, 128, 0), 128, 1)).T
+    want = F.bf16_to_f32(F.bf16_round(F.bf16_to_f32(F.bf16_round(o.astype(np.float32)))))
+    got = F.bf16_to_f32(y)
+    # h may land on a different e4m3 code where fp32 and fp64 accumulation differ by an ulp
+    assert np.allclose(got, want, rtol=3e-2, atol=1e-3)
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) < 5e-3
