@@ -193,6 +193,13 @@ int hk_moe_fp8blk_forward(const void* x_e4m3, const float* x_scales, const float
                           const float* w2_scales, void* y_bf16, int T, int H, int I, int E, int k,
                           void* workspace, size_t workspace_bytes, void* stream);
 
+/* Calibration probe (no counterpart in the reference): runs `blocks` workgroups of 8 waves, each
+ * wave `iters` x 32 register-only 16x16x128 MFMAs (fp8 if fp4 == 0, else fp4) on operand bits
+ * taken from `pattern` (16384 device ints); `sink` receives blocks*512 floats. The caller times
+ * the launch; flops = blocks * 8 * iters * 32 * 65536. Gives the power-limited MFMA ceiling for a
+ * given operand bit distribution. */
+int hk_probe_mfma_rate(const void* pattern, void* sink, int blocks, int iters, int fp4, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
