@@ -197,11 +197,11 @@ __global__ __launch_bounds__(256) void moe_topk_grouped_sigmoid_kernel(
 }
 
 // --------------------------------------------------------------------------------- sort
-// Stable counting sort of S = T*k slots by expert id, three launches:
+// Stable counting sort of S = T*k slots by expert id, four launches:
 //   count   : per-chunk histogram (chunk = 1024 consecutive slots) -> ws[chunk][E]
-//   scan    : ws[chunk][e] := first output position of chunk's slots of expert e;
-//             expert_offsets[0..E]
-//   scatter : position of a slot = ws[chunk][e] + number of earlier slots of e in the chunk
+//   scan    : ws[chunk][e] := slots of expert e in earlier chunks (one workgroup per expert);
+//   offsets : expert_offsets[0..E] from the per-expert totals
+//   scatter : position of a slot = expert_offsets[e] + ws[chunk][e] + earlier slots of e in the chunk
 // The within-chunk rank comes from wave ballots in slot order, never from atomics' arrival
 // order, so the result is deterministic and stable.
 constexpr int kSortChunk = 1024;
@@ -222,37 +222,52 @@ __global__ __launch_bounds__(256) void moe_sort_count_kernel(const int32_t* __re
     for (int e = threadIdx.x; e < E; e += 256) ws[(size_t)blockIdx.x * E + e] = cnt[e];
 }
 
-__global__ __launch_bounds__(512) void moe_sort_scan_kernel(int32_t* __restrict__ ws, int nchunks, int E,
-                                                             int32_t* __restrict__ expert_offsets) {
-    __shared__ int total[kSortMaxE];
-    __shared__ int start[kSortMaxE + 1];
-    const int e = threadIdx.x;
-    int run = 0;
-    if (e < E) {
-        for (int c = 0; c < nchunks; ++c) {
-            const int v = ws[(size_t)c * E + e];
-            ws[(size_t)c * E + e] = run;
-            run += v;
+// One workgroup per expert: exclusive prefix of that expert's per-chunk counts over the chunks
+// (ws[chunk][e] := number of slots of e in earlier chunks) and the expert's total.
+__global__ __launch_bounds__(256) void moe_sort_scan_kernel(int32_t* __restrict__ ws, int nchunks, int E,
+                                                            int32_t* __restrict__ totals) {
+    __shared__ int part[256];
+    const int e = blockIdx.x, t = threadIdx.x;
+    int carry = 0;
+    for (int c0 = 0; c0 < nchunks; c0 += 256) {
+        const int c = c0 + t;
+        const int v = c < nchunks ? ws[(size_t)c * E + e] : 0;
+        part[t] = v;
+        __syncthreads();
+        for (int d = 1; d < 256; d <<= 1) {
+            const int u = t >= d ? part[t - d] : 0;
+            __syncthreads();
+            part[t] += u;
+            __syncthreads();
         }
-        total[e] = run;
+        if (c < nchunks) ws[(size_t)c * E + e] = carry + part[t] - v;
+        carry += part[255];
+        __syncthreads();
     }
+    if (t == 0) totals[e] = carry;
+}
+
+// expert_offsets[0..E] = exclusive prefix sum of the per-expert totals.
+__global__ __launch_bounds__(512) void moe_sort_offsets_kernel(const int32_t* __restrict__ totals, int E,
+                                                               int32_t* __restrict__ expert_offsets) {
+    __shared__ int scan[512];
+    const int e = threadIdx.x;
+    const int v = e < E ? totals[e] : 0;
+    scan[e] = v;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int acc = 0;
-        for (int i = 0; i < E; ++i) { start[i] = acc; acc += total[i]; }
-        start[E] = acc;
+    for (int d = 1; d < 512; d <<= 1) {
+        const int u = e >= d ? scan[e - d] : 0;
+        __syncthreads();
+        scan[e] += u;
+        __syncthreads();
     }
-    __syncthreads();
-    if (e < E) {
-        const int st = start[e];
-        expert_offsets[e] = st;
-        for (int c = 0; c < nchunks; ++c) ws[(size_t)c * E + e] += st;
-    }
-    if (e == 0) expert_offsets[E] = start[E];
+    if (e < E) expert_offsets[e] = scan[e] - v;
+    if (e == 511) expert_offsets[E] = scan[511];
 }
 
 __global__ __launch_bounds__(256) void moe_sort_scatter_kernel(const int32_t* __restrict__ ids, int S, int E,
                                                                const int32_t* __restrict__ ws,
+                                                               const int32_t* __restrict__ expert_offsets,
                                                                int32_t* __restrict__ sorted_slots,
                                                                int32_t* __restrict__ slot_to_pos) {
     // 16 rounds of 64 consecutive slots per chunk: wave w takes rounds 4w..4w+3
@@ -285,7 +300,7 @@ __global__ __launch_bounds__(256) void moe_sort_scatter_kernel(const int32_t* __
     }
     __syncthreads();
     for (int e = threadIdx.x; e < E; e += 256) {
-        int run = ws[(size_t)blockIdx.x * E + e];
+        int run = expert_offsets[e] + ws[(size_t)blockIdx.x * E + e];
 #pragma unroll
         for (int rnd = 0; rnd < 16; ++rnd) {
             const int v = round_cnt[rnd][e];
@@ -337,7 +352,7 @@ extern "C" size_t hk_moe_sort_workspace_bytes(int T, int k, int E) {
     if (T <= 0 || k <= 0 || E <= 0) return 0;
     const size_t S = (size_t)T * k;
     const size_t nchunks = (S + hk::kSortChunk - 1) / hk::kSortChunk;
-    return nchunks * (size_t)E * sizeof(int32_t);
+    return (nchunks + 1) * (size_t)E * sizeof(int32_t);  // per-chunk counts + per-expert totals
 }
 
 extern "C" int hk_moe_sort(const int32_t* ids, int T, int k, int E, int32_t* sorted_slots,
@@ -352,8 +367,10 @@ extern "C" int hk_moe_sort(const int32_t* ids, int T, int k, int E, int32_t* sor
     hipStream_t s = (hipStream_t)stream;
     int32_t* ws = (int32_t*)workspace;
     hipLaunchKernelGGL(moe_sort_count_kernel, dim3(nchunks), dim3(256), 0, s, ids, S, E, ws);
-    hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(1), dim3(512), 0, s, ws, nchunks, E, expert_offsets);
+    int32_t* totals = ws + (size_t)nchunks * E;
+    hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(E), dim3(256), 0, s, ws, nchunks, E, totals);
+    hipLaunchKernelGGL(moe_sort_offsets_kernel, dim3(1), dim3(512), 0, s, (const int32_t*)totals, E, expert_offsets);
     hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(nchunks), dim3(256), 0, s, ids, S, E,
-                       (const int32_t*)ws, sorted_slots, slot_to_pos_or_null);
+                       (const int32_t*)ws, (const int32_t*)expert_offsets, sorted_slots, slot_to_pos_or_null);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }

@@ -50,7 +50,7 @@ def test_c_entry_points_reject_bad_arguments_without_a_gpu():
     assert lib.hk_moe_topk_grouped_sigmoid(p, None, 4, 30, 2, 4, 2, 1.0, p, p, None) == -2
     assert lib.hk_moe_sort(p, 4, 2, 8, p, p, None, None, 0, None) == -4       # no workspace
     assert lib.hk_moe_sort(p, 4, 2, 8, p, p, None, p, 4, None) == -4          # workspace too small
-    assert lib.hk_moe_sort_workspace_bytes(4096, 4, 128) == 16 * 128 * 4
+    assert lib.hk_moe_sort_workspace_bytes(4096, 4, 128) == 17 * 128 * 4
 
 
 def test_python_boundary_rejects_like_the_reference():
