@@ -67,21 +67,24 @@ __device__ __forceinline__ float sigmoid_f32(float x) {
 constexpr int kMaxPerLane = 8;  // experts per lane: E <= 512
 
 // ------------------------------------------------------------------------- top-k softmax
-// One wave per token. ids[t, j] = j-th largest logit (ties -> lower id); w = softmax over the k
-// selected logits.
+// LPT lanes per token (64 / LPT tokens per wave): LPT = 16 when E <= 128 and k <= 16, so that a
+// wave's loads cover four token rows, else one wave per token. ids[t, j] = j-th largest logit
+// (ties -> lower id); w = softmax over the k selected logits.
+template <int LPT>
 __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const float* __restrict__ logits, int T,
                                                                int E, int k, int32_t* __restrict__ ids,
                                                                float* __restrict__ w) {
-    const int lane = lane_id();
-    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (t >= T) return;
-    const float* row = logits + (size_t)t * E;
+    constexpr int TPW = 64 / LPT;  // tokens per wave
+    const int lane = lane_id(), sub = lane % LPT;
+    const int t = (blockIdx.x * 4 + (threadIdx.x >> 6)) * TPW + lane / LPT;
+    const bool live = t < T;
+    const float* row = logits + (size_t)(live ? t : 0) * E;
     uint64_t cand[kMaxPerLane];
-    const int per = (E + 63) / 64;
+    const int per = (E + LPT - 1) / LPT;
 #pragma unroll
     for (int i = 0; i < kMaxPerLane; ++i) {
-        const int e = i * 64 + lane;  // coalesced
-        cand[i] = (i < per && e < E) ? pack_choice(row[e], e) : 0ull;
+        const int e = i * LPT + sub;  // coalesced within the token's row
+        cand[i] = (live && i < per && e < E) ? pack_choice(row[e], e) : 0ull;
     }
     float my_logit = 0.f, top_logit = 0.f;
     int my_id = 0;
@@ -89,22 +92,26 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const float* __re
         uint64_t best = 0;
 #pragma unroll
         for (int i = 0; i < kMaxPerLane; ++i) best = cand[i] > best ? cand[i] : best;
-        best = wave_max_u64(best);
-        const int id = choice_id(best);
+#pragma unroll
+        for (int off = LPT / 2; off >= 1; off >>= 1) {
+            const uint64_t o = __shfl_xor(best, off, 64);
+            best = o > best ? o : best;
+        }
+        const int id = live ? choice_id(best) : 0;
 #pragma unroll
         for (int i = 0; i < kMaxPerLane; ++i)
             if (cand[i] == best) cand[i] = 0ull;  // ids are unique, only the owner matches
         const float v = row[id];
         if (j == 0) top_logit = v;
-        if (lane == j) { my_logit = v; my_id = id; }
+        if (sub == j) { my_logit = v; my_id = id; }
     }
-    const float ex = lane < k ? expf(my_logit - top_logit) : 0.f;
+    const float ex = sub < k ? expf(my_logit - top_logit) : 0.f;
     float tot = ex;
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) tot += __shfl_xor(tot, off, 64);
-    if (lane < k) {
-        ids[(size_t)t * k + lane] = my_id;
-        w[(size_t)t * k + lane] = ex / tot;
+    for (int off = LPT / 2; off >= 1; off >>= 1) tot += __shfl_xor(tot, off, 64);
+    if (live && sub < k) {
+        ids[(size_t)t * k + sub] = my_id;
+        w[(size_t)t * k + sub] = ex / tot;
     }
 }
 
@@ -328,8 +335,12 @@ extern "C" int hk_moe_topk_softmax(const float* logits, int T, int E, int k, int
     using namespace hk;
     if (!logits || !ids || !w) return HK_ERR_NULL_POINTER;
     if (T <= 0 || E <= 0 || k <= 0 || k > E || k > 64 || E > 64 * kMaxPerLane) return HK_ERR_BAD_SHAPE;
-    hipLaunchKernelGGL(moe_topk_softmax_kernel, dim3((T + 3) / 4), dim3(256), 0, (hipStream_t)stream,
-                       logits, T, E, k, ids, w);
+    if (E <= 128 && k <= 16)
+        hipLaunchKernelGGL(moe_topk_softmax_kernel<16>, dim3((T + 15) / 16), dim3(256), 0, (hipStream_t)stream,
+                           logits, T, E, k, ids, w);
+    else
+        hipLaunchKernelGGL(moe_topk_softmax_kernel<64>, dim3((T + 3) / 4), dim3(256), 0, (hipStream_t)stream,
+                           logits, T, E, k, ids, w);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
