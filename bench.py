@@ -7,6 +7,7 @@ Protocol follows the reference's harness (kernels/gemm/bf16fp32/mi350x/test_pyth
 79-101: 500 warm-up and 100 timed launches, flops = 2*M*N*K).
 
   python bench.py [--gpus 1] [--steps 100] [--warmup 500] [--only-headline] [--no-cpu-baseline]
+  python bench.py --traffic-calibration     (a 1 GiB copy + the headline GEMM, for counter runs)
 
 `roofline` is measured with HIP events on the launch stream around the timed region.
 `cpu_baseline` times the CPU counterpart (PyTorch-CPU dequantize + fp32 matmul) on the host cores.
@@ -28,6 +29,10 @@ sys.path.insert(0, ROOT)
 PEAK_FP8 = 5033.0     # MI355X dense FP8 MFMA peak, TFLOP/s (256 CU x 2.4 GHz x 8192 flop/clk/CU)
 PEAK_FP4 = 10066.0    # dense MXFP4
 PEAK_HBM = 8000.0     # GB/s
+# HBM-side bytes per 8192^3 launch of the headline kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter
+# runs of `bench.py --traffic-calibration`, each scaled by the same counter's reading for a 1 GiB copy
+# (factors 2.0 and 1.0): 805.8 MB read + 137.3 MB written (profiles/fp8_gemm_4wave_ring_kernel_8192.md).
+TRAFFIC_FP8_8192 = 943.1e6
 
 
 def _timeit(torch, fn, warmup, iters):
@@ -183,6 +188,7 @@ def main() -> int:
     ap.add_argument("--size", type=int, default=8192)
     ap.add_argument("--only-headline", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-calibration", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (--gpus 1); "
@@ -199,6 +205,20 @@ def main() -> int:
     hk.load_library()  # raises if libhk355.so has not been built
     dev = torch.device("cuda:0")
     n = args.size
+
+    if args.traffic_calibration:
+        # For the HBM-traffic counters: a plain copy of known size (1 GiB read + 1 GiB written per
+        # launch) next to the headline GEMM, nothing else, so that the FETCH_SIZE / WRITE_SIZE
+        # readings of the GEMM can be scaled by what the same counters read for the copy.
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        bench_fp8(torch, hk, n, 5, 5, dev)
+        torch.cuda.synchronize()
+        print(json.dumps({"traffic_calibration": {"copy_bytes_read": 1 << 30, "copy_bytes_written": 1 << 30,
+                                                  "copy_launches": 5, "gemm_launches": 10, "n": n}}))
+        return 0
 
     head = bench_fp8(torch, hk, n, args.warmup, args.steps, dev, keep=True)
     tflops = 2.0 * n ** 3 / (head["wall_ms"] * 1e-3) / 1e12
@@ -249,7 +269,8 @@ def main() -> int:
         "pct_of_fp8_peak": round(100.0 * tflops / PEAK_FP8, 2),
         "rel_fro_err_vs_oracle": rel,
         "roofline": {"bound": "mfma", "achieved": round(head["tflops"], 2), "peak": PEAK_FP8, "unit": "TFLOP/s",
-                     "frac": round(head["tflops"] / PEAK_FP8, 4), "traffic": None,
+                     "frac": round(head["tflops"] / PEAK_FP8, 4),
+                     "traffic": TRAFFIC_FP8_8192 if n == 8192 else None,
                      "kernel_ms": round(head["kernel_ms"], 5)},
         "cpu_baseline": cpu,
         "extra": extra,
