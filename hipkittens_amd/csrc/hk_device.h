@@ -145,6 +145,20 @@ __device__ __forceinline__ int scalar_load_x1(const void* p) {
     return r;
 }
 
+// Global stores the compiler does not see. On this ISA loads and stores share one counter but
+// complete out of order with respect to each other, so a compiler that sees both kinds pending
+// waits for all of them (vmcnt(0)) before the first use of any loaded register; kernels that
+// keep register loads in flight across an epilogue issue the epilogue's stores through these.
+__device__ __forceinline__ void store_global_b128(void* p, v4i v) {
+    asm volatile("global_store_dwordx4 %0, %1, off" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void store_global_b32(void* p, uint32_t v) {
+    asm volatile("global_store_dword %0, %1, off" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void store_global_b8(void* p, uint32_t v) {
+    asm volatile("global_store_byte %0, %1, off" ::"v"(p), "v"(v) : "memory");
+}
+
 // Same MFMA with the accumulator tied in place in an accumulation register (AGPR).
 // Used by the hand-scheduled kernels, where the register allocator must not move
 // accumulators between register files. The compiler does not see the instruction's

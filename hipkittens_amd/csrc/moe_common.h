@@ -25,8 +25,9 @@ struct MoeItem { int expert, row_start, rows, n_tile; };
 inline int moe_round_up(int x, int m) { return (x + m - 1) / m * m; }
 // Number of CUs of the current device (cached).
 int moe_num_compute_units();
-// items[] / *num_items from expert_offsets [E+1] for GEMMs with n_tiles_n tiles of weight rows.
-void moe_launch_build_items(const int32_t* expert_offsets, int E, int n_tiles_n, MoeItem* items,
-                            int32_t* num_items, hipStream_t s);
+// Item lists of the two grouped GEMMs of a layer from expert_offsets [E+1]: items1 / num_items[0]
+// for n_tiles_n1 tiles of weight rows, items2 / num_items[1] for n_tiles_n2 (one launch).
+void moe_launch_build_items(const int32_t* expert_offsets, int E, int n_tiles_n1, MoeItem* items1,
+                            int n_tiles_n2, MoeItem* items2, int32_t* num_items, hipStream_t s);
 
 }  // namespace hk

@@ -28,19 +28,24 @@ __device__ __forceinline__ int mx_block_exponent(float amax) {
     const int e = (int)((__float_as_uint(amax) >> 23) & 0xffu) - 127 - 2;
     return max(-127, min(127, e));
 }
-// e2m1 code of v * 2^-e: round to nearest, ties to the even code, saturating at 6.
-__device__ __forceinline__ uint32_t e2m1_code(float v, int e) {
-    const float a = fabsf(ldexpf(v, -e));
-    uint32_t c = (a > 0.25f) + (a >= 0.75f) + (a > 1.25f) + (a >= 1.75f) + (a > 2.5f) + (a >= 3.5f) +
-                 (a > 5.0f);
-    if (a != a) c = 7;  // NaN saturates like the oracle
-    return c | ((__float_as_uint(v) >> 31) << 3);
-}
+// Eight values times 2^-e as packed e2m1 codes (round to nearest, ties to the even code,
+// saturating at 6; element i in nibble i). v_cvt_scalef32_pk_fp4_f32 divides by the power-of-two
+// scale and rounds exactly like that, NaN and infinities included (checked against the compare
+// chain of the CPU oracle over all bf16 inputs, the ties and their neighbours, e = -127..127).
 __device__ __forceinline__ uint32_t pack8_e2m1(const float (&v)[8], int e) {
+    // 2^e as a float; 2^-127 is the denormal 0x00400000
+    const float scale = __uint_as_float(e > -127 ? (uint32_t)(e + 127) << 23 : 0x00400000u);
     uint32_t out = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) out |= e2m1_code(v[i], e) << (4 * i);
+    out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[0], v[1], scale, 0);
+    out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[2], v[3], scale, 1);
+    out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[4], v[5], scale, 2);
+    out = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(out, v[6], v[7], scale, 3);
     return out;
+}
+// SiLU(g) * u of the gate+up epilogue: g / (1 + exp(-g)) with the hardware exp2 and reciprocal
+// (about 1 ulp each; both grouped GEMM kernels use this same sequence).
+__device__ __forceinline__ float silu_mul(float g, float u) {
+    return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
 }
 
 // x [rows, cols] bf16 -> packed e2m1 [rows, cols/2] + e8m0 scales [rows, scale_pitch] (columns
@@ -85,15 +90,26 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_rows_kernel(const uint16_t
 //
 // Quantize-and-permute: row `pos` of the output is token sorted_slots[pos] / topk of x, so that
 // each expert's rows are contiguous for the grouped GEMM (the "permute" step of the MoE).
+// The same launch pads the second tiled matrix of the layer (h, contraction length K2): the part
+// of its last K-step past K2 that the producing GEMM epilogue never writes is set to zero data
+// and neutral scales (nothing to do when K2 is a multiple of 256).
 __global__ __launch_bounds__(256) void mxfp4_quantize_permute_kernel(
     const uint16_t* __restrict__ x, const int32_t* __restrict__ sorted_slots, int topk, int S, int cols,
-    uint8_t* __restrict__ tiled, uint8_t* __restrict__ tiled_scales) {
+    uint8_t* __restrict__ tiled, uint8_t* __restrict__ tiled_scales, uint8_t* __restrict__ tiled2,
+    uint8_t* __restrict__ tiled2_scales, int K2) {
     const int nk = (cols / 2 + 127) >> 7;
     const int per_row = nk * 32;  // threads per row: one per 8 elements of the padded row
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
     const int pos = (int)(gid / per_row);
     const int c8 = (int)(gid % per_row);
     if (pos >= S) return;
+    if (c8 < 32 && (K2 & 255)) {
+        const int Kb2 = K2 >> 1, nk2 = (Kb2 + 127) >> 7;
+        const int valid = Kb2 - (nk2 - 1) * 128;  // valid bytes of the last K-step, a multiple of 16
+        const size_t tile_row2 = (size_t)(nk2 - 1) * S + pos;
+        if (c8 * 4 >= valid) *(uint32_t*)(tiled2 + tile_row2 * 128 + c8 * 4) = 0u;
+        if (c8 < 8 && c8 * 16 >= valid) tiled2_scales[tile_row2 * 8 + c8] = 127;
+    }
     const int row = sorted_slots[pos] / topk;
     float v[8];
     if (c8 * 8 < cols) {
@@ -118,27 +134,16 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_permute_kernel(
     if ((c8 & 3) == 0) tiled_scales[tile_row * 8 + ((c8 >> 2) & 7)] = (uint8_t)(e + 127);
 }
 
-// Zero / neutral padding of the last K-step of a tiled activation matrix whose K is not a
-// multiple of 256 (the part the producing GEMM epilogue never writes).
-__global__ __launch_bounds__(256) void moe_pad_tiled_kernel(uint8_t* __restrict__ tiled,
-                                                            uint8_t* __restrict__ tiled_scales, int S, int K) {
-    const int Kb = K >> 1, nk = (Kb + 127) >> 7;
-    const int valid = Kb - (nk - 1) * 128;  // valid bytes of the last K-step, a multiple of 16
-    const int pos = blockIdx.x * 8 + (threadIdx.x >> 5);
-    const int c = threadIdx.x & 31;  // 4-byte column
-    if (pos >= S) return;
-    const size_t tile_row = (size_t)(nk - 1) * S + pos;
-    if (c * 4 >= valid) *(uint32_t*)(tiled + tile_row * 128 + c * 4) = 0u;
-    if (c < 8 && c * 16 >= valid) tiled_scales[tile_row * 8 + c] = 127;
-}
-
 // ---------------------------------------------------------------------- weight pre-shuffle
-// Pre-shuffled weight layout: for every expert, n-tile and K-step one contiguous 32 KiB block
-// holding the 256 x 128-byte B tile exactly as it sits in LDS (row permutation and chunk
-// swizzle applied, K zero-padded to whole K-steps), followed in a second array by the 2 KiB
-// scale tile (256 rows x 8 bytes, padding = 127). The grouped GEMM then streams weights from
-// HBM in long contiguous bursts instead of 128-byte pieces a row pitch apart.
-//   out_w [E][n_tiles][nk][256][128] bytes, out_s [E][n_tiles][nk][256][8] bytes.
+// Pre-shuffled weight layout, made for moe_mxfp4_stream_kernel: weights go from HBM straight
+// into MFMA operand registers, so for every (expert, n-tile of 256 tile rows, K-step of 256
+// elements) one contiguous 32 KiB block holds, wave by wave (wave wn = tile rows [64 wn, +64)),
+// the wave's eight B fragments f = 2 * nfrag + half as 1 KiB pieces in lane order: lane l's 16
+// bytes are tile row 64 wn + 16 nfrag + l % 16 (moe_b_row gives the weight row), K bytes
+// 128 kt + 64 half + 16 (l / 16) .. +16, zero past the end of K. A second array holds the
+// scales the same way, 8 bytes per lane: byte 4 half + nfrag is the e8m0 scale of that row's
+// 32-element block 8 kt + 4 half + l / 16 (127 past the end of K).
+//   out_w [E][n_tiles][nk][4][8][64][16] bytes, out_s [E][n_tiles][nk][4][64][8] bytes.
 __global__ __launch_bounds__(256) void moe_preshuffle_kernel(const uint8_t* __restrict__ w,
                                                              const uint8_t* __restrict__ sc, int E, int N,
                                                              int K, int scale_pitch, int mode, int n_tiles,
@@ -149,30 +154,38 @@ __global__ __launch_bounds__(256) void moe_preshuffle_kernel(const uint8_t* __re
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;  // one 16-byte chunk each
     const long long total = (long long)E * n_tiles * nk * 2048;
     if (gid >= total) return;
-    const int pc = (int)(gid & 7), R = (int)((gid >> 3) & 255);
+    const int l = (int)(gid & 63), f = (int)((gid >> 6) & 7), wn = (int)((gid >> 9) & 3);
     long long rest = gid >> 11;
     const int kt = (int)(rest % nk); rest /= nk;
     const int nt = (int)(rest % n_tiles);
     const int e = (int)(rest / n_tiles);
-    const int row = moe_b_row(mode, R, nt, N);
-    const int c = pc ^ ((R >> 1) & 7);
-    const int kb = kt * 128 + c * 16;
+    const int row = moe_b_row(mode, 64 * wn + 16 * (f >> 1) + (l & 15), nt, N);
+    const int kb = kt * 128 + 64 * (f & 1) + 16 * (l >> 4);
     v4i val = {0, 0, 0, 0};
     if (kb < Kb) val = *(const v4i*)(w + ((size_t)e * rows_b + row) * Kb + kb);
     *(v4i*)(out_w + gid * 16) = val;
-    if (pc == 0) {
-        // this thread also moves the row's 8 scale bytes of the K-step
-        uint8_t* dst = out_s + (gid >> 3) * 8;
-        const uint8_t* src = sc + ((size_t)e * rows_b + row) * scale_pitch + kt * 8;
+    if (f == 0) {
+        // this thread also writes the lane's 8 scale bytes of the K-step
+        uint8_t* dst = out_s + ((gid >> 11) * 4 + wn) * 512 + l * 8;
 #pragma unroll
-        for (int b = 0; b < 8; ++b) dst[b] = (kt * 8 + b < (K >> 5)) ? src[b] : (uint8_t)127;
+        for (int b = 0; b < 8; ++b) {
+            const int rw = moe_b_row(mode, 64 * wn + 16 * (b & 3) + (l & 15), nt, N);
+            const int blk = kt * 8 + 4 * (b >> 2) + (l >> 4);
+            dst[b] = blk < (K >> 5) ? sc[((size_t)e * rows_b + rw) * scale_pitch + blk] : (uint8_t)127;
+        }
     }
 }
 
+// Item lists of both grouped GEMMs of a layer in one launch: workgroup 0 builds the list for
+// n_tiles[0] tiles of weight rows into items[0], workgroup 1 the one for n_tiles[1].
+struct MoeBuildItems { MoeItem* items[2]; int n_tiles[2]; };
 __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __restrict__ expert_offsets,
-                                                              int E, int n_tiles_n, MoeItem* __restrict__ items,
+                                                              int E, MoeBuildItems b,
                                                               int32_t* __restrict__ num_items) {
     __shared__ int scan[512];
+    const int which = blockIdx.x;
+    const int n_tiles_n = b.n_tiles[which];
+    MoeItem* __restrict__ items = b.items[which];
     const int e = threadIdx.x;
     int lo = 0, hi = 0, cnt = 0;
     if (e < E) {
@@ -194,7 +207,7 @@ __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __r
             it.expert = e; it.row_start = lo + m * kMoeBM; it.rows = min(kMoeBM, hi - it.row_start); it.n_tile = n;
             items[base + n * cnt + m] = it;
         }
-    if (e == 511) *num_items = scan[511];
+    if (e == 511) num_items[which] = scan[511];
 }
 
 // ---------------------------------------------------------------------------- grouped GEMM
@@ -455,7 +468,7 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const float gv = gt[j];
-                        h[4 * q + j] = gv / (1.0f + __expf(-gv)) * up[j];
+                        h[4 * q + j] = silu_mul(gv, up[j]);
                     }
                 }
                 float amax = 0.f;
@@ -517,6 +530,259 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
     wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
 }
 
+// ------------------------------------------------------- grouped GEMM, pre-shuffled weights
+// Weight-streaming variant for the pre-shuffled layout. At MoE shapes the grouped GEMMs are
+// bound by reading every expert's weights once from HBM, so the kernel is built around keeping
+// as many weight bytes in flight per CU as the register file allows:
+//   * weights never touch LDS: the pre-shuffled layout stores, for every (expert, n-tile, K-step,
+//     wave), the wave's eight MFMA B fragments as eight contiguous 1 KiB pieces (lane l's 16
+//     bytes at 16*l), and each wave loads them straight into registers two K-steps ahead of
+//     their use (a ring of four half-K-step register sets);
+//   * their e8m0 scales come the same way (8 bytes per lane and K-step);
+//   * only the activation tile (shared by the four waves, re-read from L2) goes through LDS, in
+//     a ring of four 17 KiB stages filled by direct global->LDS loads three K-steps ahead.
+// Workgroups have 4 waves, wave wn owning weight rows [64 wn, +64) of the 256-row tile and all
+// 128 activation rows; two workgroups share a CU (68 KiB of LDS and 256 registers per lane
+// each) and cover each other's barrier and issue stalls. The K-step stream runs across item
+// boundaries. Results are bit-identical to moe_mxfp4_gemm_kernel (same accumulation order).
+constexpr int kStStages = 4;
+constexpr int kStStage = kMoeATile + kMoeScaleA;   // 16 KiB tile + 1 KiB scales
+constexpr int kStLds = kStStages * kStStage;       // 68 KiB
+
+template <int MODE>
+__global__ __launch_bounds__(256, 2) void moe_mxfp4_stream_kernel(const MoeGemmParams p) {
+    constexpr int MT = kMoeBM / 16, NT = 4;
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    const int lane = lane_id(), w = wave_id();
+    const int n_items = scalar_load_x1(p.num_items);
+    const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+    const int it_stride = ((int)gridDim.x - xcd + kNumXcd - 1) / kNumXcd;  // workgroups on this XCD
+    const int per_xcd = (n_items + kNumXcd - 1) / kNumXcd;
+    const int it0 = xcd * per_xcd + slot;
+    const int it_end = min(n_items, (xcd + 1) * per_xcd);
+    if (it0 >= it_end) return;
+
+    const int Kb = p.K >> 1;
+    const int nk = (Kb + 127) >> 7;
+    const v4i srd_a = make_srd(p.A, (uint32_t)nk * (uint32_t)p.S * 128u);
+    const v4i srd_sa = make_srd(p.SA, (uint32_t)nk * (uint32_t)p.S * 8u);
+
+    // ---- cursors over the stream of (item, K-step) positions of this workgroup ---------------
+    struct Cursor { int it, kt, expert, row_start, rows, n_tile; bool valid; };
+    auto load_item = [&](Cursor& c) __attribute__((always_inline)) {
+        c.valid = c.it < it_end;
+        const v4i item = scalar_load_x4(p.items + (c.valid ? c.it : it_end - 1));
+        c.expert = item.x; c.row_start = item.y; c.rows = item.z; c.n_tile = item.w;
+    };
+    auto advance = [&](Cursor& c) __attribute__((always_inline)) {
+        if (++c.kt == nk) { c.kt = 0; c.it += it_stride; load_item(c); }
+    };
+    Cursor cc{it0, 0}, ca{it0, 0}, cb{it0, 0};  // compute, activation fetch, weight fetch
+    load_item(cc);
+    ca = cc; cb = cc;
+
+    // ---- activation tile: global -> LDS -------------------------------------------------------
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+    const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
+    const uint32_t lds_sa_wave = to_sgpr(lds0 + kMoeATile + (uint32_t)w * 256u);
+    const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);
+    uint32_t voff_a[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) voff_a[i] = (uint32_t)(8 * (i * 4 + w) + (lane >> 3)) * 128u + chunk16 * 16u;
+    const uint32_t voff_sa = (uint32_t)(w * 256 + lane * 16);
+    // 5 loads: the wave's quarter of the tile (rows 8(4i + w) .. +8) and of its scales (32 rows)
+    auto issue_a = [&](const Cursor& c, int stage) __attribute__((always_inline)) {
+        v4i sa = srd_a, ssa = srd_sa;
+        if (!c.valid) { sa.z = 0; ssa.z = 0; }
+        const uint32_t row_base = (uint32_t)c.kt * (uint32_t)p.S + (uint32_t)c.row_start;
+        const uint32_t dst = lds_wave + (uint32_t)stage * kStStage;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dma16(sa, dst + i * 4096, voff_a[i], row_base * 128u);
+        dma16_lanes(ssa, lds_sa_wave + (uint32_t)stage * kStStage, voff_sa, row_base * 8u, 0xffffull);
+    };
+
+    // ---- weights: global -> registers -----------------------------------------------------------
+    // pre-shuffled layout (moe_preshuffle_kernel): [expert][n-tile][K-step][wave][fragment][lane][16]
+    const int voff_b = lane * 16, voff_sb = lane * 8;  // scales: dword 0 first K half, dword 1 second
+    auto rsrc_b = [&](const Cursor& c) __attribute__((always_inline)) {
+        const uint8_t* base = p.B + (size_t)c.expert * p.b_expert_stride + (size_t)c.n_tile * nk * kMoeBTile;
+        return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, c.valid ? nk * kMoeBTile : 0, 0x00020000);
+    };
+    auto rsrc_sb = [&](const Cursor& c) __attribute__((always_inline)) {
+        const uint8_t* base = p.SB + (size_t)c.expert * p.sb_expert_stride + (size_t)c.n_tile * nk * kMoeScaleB;
+        return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, c.valid ? nk * kMoeScaleB : 0, 0x00020000);
+    };
+    v4i bw[2][2][NT];  // [K-step parity][K half][fragment]
+    int bsc[2][2];     // [K-step parity][K half]: the lane's scale bytes of fragments 0..3
+    auto load_b_half = [&](const Cursor& c, v4i (&dst)[NT], int half) {
+        const __amdgpu_buffer_rsrc_t rs = rsrc_b(c);
+        const int soff = c.kt * kMoeBTile + w * 8192 + half * 1024;
+#pragma unroll
+        for (int n = 0; n < NT; ++n) dst[n] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_b, soff + n * 2048, 0);
+    };
+    auto load_b_scales = [&](const Cursor& c, int& dst, int half) __attribute__((always_inline)) {
+        dst = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sb(c), voff_sb, c.kt * kMoeScaleB + w * 512 + half * 4, 0);
+    };
+
+    // ---- LDS -> registers (activation fragments) ------------------------------------------------
+    const uint32_t r = lane & 15, g = lane >> 4;
+    const uint32_t rd_half[2] = {lds0 + r * 128u + swz_chunk(r, g) * 16u, lds0 + r * 128u + swz_chunk(r, g + 4) * 16u};
+    const uint32_t sa_rd0 = lds0 + kMoeATile + r * 8u;
+    const uint32_t sh = 8u * g;  // byte g of each scale dword belongs to this lane
+
+    v4f acc[MT][NT];
+    auto zero_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
+    };
+    auto mfma = [&](v4f& c, const v4i& x, const v4i& y, int sx, int sy) __attribute__((always_inline)) {
+        asm volatile(
+            "v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+            : "+v"(c)
+            : "v"(x), "v"(y), "v"(sx), "v"(sy));
+    };
+    // MFMAs of one K half (128 of the K-step's 256 elements) on LDS stage st
+    auto compute_half = [&](int st, int half, int rows, const v4i (&bfr)[NT], int bscale) {
+        uint32_t a_rd = rd_half[half] + (uint32_t)st * kStStage;
+        uint32_t sa_rd = sa_rd0 + (uint32_t)st * kStStage + 4u * half;
+        asm volatile("" : "+v"(a_rd), "+v"(sa_rd));  // keep the bases in registers, offsets as immediates
+        int bs[NT];
+#pragma unroll
+        for (int n = 0; n < NT; ++n) bs[n] = (int)((uint32_t)bscale >> (8 * n));
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            if (16 * m < rows) {
+                const v4i af = *(lds_v4i_t*)(uintptr_t)(a_rd + m * 2048);
+                const int as = (int)(*(__attribute__((address_space(3))) const uint32_t*)(uintptr_t)(sa_rd + m * 128) >> sh);
+#pragma unroll
+                for (int n = 0; n < NT; ++n) mfma(acc[m][n], bfr[n], af, bs[n], as);
+            }
+        }
+    };
+
+    auto epilogue = [&](const Cursor& c) __attribute__((always_inline)) {
+        const int rows = c.rows, row_start = c.row_start;
+        const int n0 = c.n_tile * (MODE == 0 ? 128 : 256);
+        if (MODE == 1) {
+            uint16_t* out = (uint16_t*)p.out0;
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const int row = 16 * m + (int)r;
+                if (row >= rows) continue;
+                const size_t pos = (size_t)(row_start + row);
+#pragma unroll
+                for (int q = 0; q < NT / 2; ++q) {
+                    const int col = n0 + w * 64 + 32 * q + 8 * (int)g;
+                    if (col + 8 > p.N) continue;  // N % 8 == 0
+                    const v4f x = acc[m][2 * q], y = acc[m][2 * q + 1];
+                    v4i o4;
+                    o4.x = pack_bf16(x.x, x.y); o4.y = pack_bf16(x.z, x.w);
+                    o4.z = pack_bf16(y.x, y.y); o4.w = pack_bf16(y.z, y.w);
+                    store_global_b128(out + pos * p.N + col, o4);
+                }
+            }
+        } else {
+            // see moe_mxfp4_gemm_kernel: this wave's 32 h columns are one MX block
+            uint8_t* hq = (uint8_t*)p.out0;
+            const int hcol0 = n0 + 32 * w;
+            const bool col_ok = hcol0 < p.N;
+            const size_t kt2 = (size_t)(hcol0 >> 8);
+            const int byte0 = ((hcol0 & 255) >> 1) + 4 * (int)g, blk = (hcol0 & 255) >> 5;
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const int row = 16 * m + (int)r;
+                if (16 * m >= rows) continue;  // uniform: the whole fragment is padding
+                float h[8];
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const v4f gt = acc[m][2 * q], up = acc[m][2 * q + 1];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float gv = gt[j];
+                        h[4 * q + j] = silu_mul(gv, up[j]);
+                    }
+                }
+                float amax = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(h[i]));
+                amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+                const int e = mx_block_exponent(amax);
+                if (row < rows && col_ok) {
+                    const size_t tile_row = kt2 * p.S + (size_t)(row_start + row);
+                    store_global_b32(hq + tile_row * 128 + byte0, pack8_e2m1(h, e));
+                    if (g == 0) store_global_b8(p.out_scales + tile_row * 8 + blk, (uint32_t)(e + 127));
+                }
+            }
+        }
+    };
+
+    // ---- prologue: positions 0..2 of the activation ring, positions 0 and 1 of the weights ----
+    issue_a(ca, 0); advance(ca);
+    issue_a(ca, 1); advance(ca);
+    issue_a(ca, 2); advance(ca);
+    // (scales first in every half set: they are the first thing a pass needs, and the wait the
+    // compiler derives for them then allows every younger load to stay in flight)
+    __builtin_amdgcn_sched_barrier(0);
+    auto load_b_set = [&]<int P>() __attribute__((always_inline)) {
+        load_b_scales(cb, bsc[P][0], 0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_b_half(cb, bw[P][0], 0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_b_scales(cb, bsc[P][1], 1);
+        __builtin_amdgcn_sched_barrier(0);
+        load_b_half(cb, bw[P][1], 1);
+        __builtin_amdgcn_sched_barrier(0);
+        advance(cb);
+    };
+    load_b_set.template operator()<0>();
+    load_b_set.template operator()<1>();
+    zero_acc();
+
+    // One stream position with register-set parity P on LDS stage st. In program order a wave
+    // issues per position: 5 activation loads (position +3) and twice 1 scale load + 4 weight loads
+    // (position +2), each half into the registers the MFMAs before it have just finished with.
+    // When a position starts, the 10 weight loads of position +1 and the 5 activation loads of
+    // position +2 may still be in flight: everything older - this position's weights and its
+    // activation tile - has landed after vmcnt(15).
+    auto step = [&]<int P>(int st) __attribute__((always_inline)) {
+        wait_vmcnt<15>();
+        block_barrier();  // everyone's part of this position's tile has landed; stage st-1 is free
+        issue_a(ca, (st + 3) & 3); advance(ca);
+        const int rows = cc.valid ? cc.rows : 0;  // past the end of the stream: no MFMAs, empty loads
+        compute_half(st, 0, rows, bw[P][0], bsc[P][0]);
+        __builtin_amdgcn_sched_barrier(0);  // the refill of a register set follows its last use
+        load_b_scales(cb, bsc[P][0], 0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_b_half(cb, bw[P][0], 0);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_half(st, 1, rows, bw[P][1], bsc[P][1]);
+        __builtin_amdgcn_sched_barrier(0);
+        load_b_scales(cb, bsc[P][1], 1);
+        __builtin_amdgcn_sched_barrier(0);
+        load_b_half(cb, bw[P][1], 1);
+        advance(cb);
+        __builtin_amdgcn_sched_barrier(0);
+        if (cc.valid && cc.kt == nk - 1) {
+            mfma_drain();
+            epilogue(cc);
+            zero_acc();
+        }
+        advance(cc);
+    };
+    // Two positions per trip (the register sets alternate); the second one may lie past the end
+    // of the stream, where it degenerates to its barrier and empty loads. No exit between the
+    // two: a second way into the loop head would make the compiler merge two load histories
+    // and wait for the more recent one.
+    for (int st = 0; cc.valid; st ^= 2) {
+        step.template operator()<0>(st);
+        step.template operator()<1>(st + 1);
+    }
+    wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
+}
+
 // ------------------------------------------------------------------------------ un-permute
 // y[t, :] = bf16( sum_j w[t, j] * o[slot_to_pos[t*k + j], :] ), fp32 accumulation in choice order.
 __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __restrict__ o,
@@ -556,10 +822,28 @@ int moe_num_compute_units() {
     return cus;
 }
 
-void moe_launch_build_items(const int32_t* expert_offsets, int E, int n_tiles_n, MoeItem* items,
-                            int32_t* num_items, hipStream_t s) {
-    hipLaunchKernelGGL(moe_build_items_kernel, dim3(1), dim3(512), 0, s, expert_offsets, E, n_tiles_n, items,
-                       num_items);
+void moe_launch_build_items(const int32_t* expert_offsets, int E, int n_tiles_n1, MoeItem* items1,
+                            int n_tiles_n2, MoeItem* items2, int32_t* num_items, hipStream_t s) {
+    MoeBuildItems b;
+    b.items[0] = items1; b.items[1] = items2;
+    b.n_tiles[0] = n_tiles_n1; b.n_tiles[1] = n_tiles_n2;
+    hipLaunchKernelGGL(moe_build_items_kernel, dim3(2), dim3(512), 0, s, expert_offsets, E, b, num_items);
+}
+
+template <int MODE>
+static int launch_moe_stream(MoeGemmParams p, int max_items, hipStream_t s) {
+    auto kern = moe_mxfp4_stream_kernel<MODE>;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kStLds) !=
+            hipSuccess)
+            return HK_ERR_LAUNCH;
+        configured = true;
+    }
+    // persistent: two workgroups per CU, each walking its share of the item list
+    const int grid = min(max_items, 2 * moe_num_compute_units());
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), kStLds, s, p);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
 template <int MODE, bool SHUF>
@@ -700,15 +984,12 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
     {
         const long long threads = (long long)S * ((H / 2 + 127) / 128) * 32;
         hipLaunchKernelGGL(mxfp4_quantize_permute_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
-                           (const uint16_t*)x_bf16, sorted_slots, k, S, H, ws + L.xq, ws + L.xs);
-        if (I % 256)
-            hipLaunchKernelGGL(moe_pad_tiled_kernel, dim3((S + 7) / 8), dim3(256), 0, s, ws + L.hq, ws + L.hs, S, I);
+                           (const uint16_t*)x_bf16, sorted_slots, k, S, H, ws + L.xq, ws + L.xs, ws + L.hq,
+                           ws + L.hs, I);
     }
     int32_t* nitems = (int32_t*)(ws + L.nitems);
-    moe_launch_build_items(expert_offsets, E, (I + 127) / 128,
-                       (MoeItem*)(ws + L.items1), nitems, s);
-    moe_launch_build_items(expert_offsets, E, (H + 255) / 256,
-                       (MoeItem*)(ws + L.items2), nitems + 1, s);
+    moe_launch_build_items(expert_offsets, E, (I + 127) / 128, (MoeItem*)(ws + L.items1), (H + 255) / 256,
+                           (MoeItem*)(ws + L.items2), nitems, s);
 
     MoeGemmParams p{};
     p.A = ws + L.xq; p.SA = ws + L.xs; p.S = S;
@@ -723,7 +1004,7 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
     p.items = (const MoeItem*)(ws + L.items1); p.num_items = nitems;
     p.out0 = ws + L.hq; p.out_scales = ws + L.hs;
     p.K = H; p.N = I; p.n_tiles_n = (I + 127) / 128;
-    st = weight_layout ? launch_moe_gemm<0, true>(p, L.max_items1, s) : launch_moe_gemm<0, false>(p, L.max_items1, s);
+    st = weight_layout ? launch_moe_stream<0>(p, L.max_items1, s) : launch_moe_gemm<0, false>(p, L.max_items1, s);
     if (st != HK_OK) return st;
 
     MoeGemmParams q{};
@@ -739,7 +1020,7 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
     q.items = (const MoeItem*)(ws + L.items2); q.num_items = nitems + 1;
     q.out0 = ws + L.o; q.out_scales = nullptr;
     q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
-    st = weight_layout ? launch_moe_gemm<1, true>(q, L.max_items2, s) : launch_moe_gemm<1, false>(q, L.max_items2, s);
+    st = weight_layout ? launch_moe_stream<1>(q, L.max_items2, s) : launch_moe_gemm<1, false>(q, L.max_items2, s);
     if (st != HK_OK) return st;
 
     return hk_moe_unpermute(ws + L.o, topk_w, slot_to_pos, T, k, H, y_bf16, stream);

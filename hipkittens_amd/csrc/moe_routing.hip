@@ -272,6 +272,36 @@ __global__ __launch_bounds__(512) void moe_sort_offsets_kernel(const int32_t* __
     if (e == 511) expert_offsets[E] = scan[511];
 }
 
+// Both steps above in one workgroup when there are few chunks: thread e walks expert e's
+// per-chunk counts, then the workgroup scans the totals.
+constexpr int kSortFusedChunks = 64;
+__global__ __launch_bounds__(512) void moe_sort_scan_offsets_kernel(int32_t* __restrict__ ws, int nchunks, int E,
+                                                                    int32_t* __restrict__ expert_offsets) {
+    __shared__ int scan[512];
+    const int e = threadIdx.x;
+    int total = 0;
+    if (e < E) {
+        int v[kSortFusedChunks];
+#pragma unroll
+        for (int c = 0; c < kSortFusedChunks; ++c) v[c] = c < nchunks ? ws[(size_t)c * E + e] : 0;
+#pragma unroll
+        for (int c = 0; c < kSortFusedChunks; ++c) {
+            if (c < nchunks) ws[(size_t)c * E + e] = total;
+            total += v[c];
+        }
+    }
+    scan[e] = total;
+    __syncthreads();
+    for (int d = 1; d < 512; d <<= 1) {
+        const int u = e >= d ? scan[e - d] : 0;
+        __syncthreads();
+        scan[e] += u;
+        __syncthreads();
+    }
+    if (e < E) expert_offsets[e] = scan[e] - total;
+    if (e == 511) expert_offsets[E] = scan[511];
+}
+
 __global__ __launch_bounds__(256) void moe_sort_scatter_kernel(const int32_t* __restrict__ ids, int S, int E,
                                                                const int32_t* __restrict__ ws,
                                                                const int32_t* __restrict__ expert_offsets,
@@ -281,6 +311,7 @@ __global__ __launch_bounds__(256) void moe_sort_scatter_kernel(const int32_t* __
     __shared__ int round_cnt[16][kSortMaxE];  // later: exclusive prefix over rounds
     const int lane = lane_id(), wv = threadIdx.x >> 6;
     const int base = blockIdx.x * kSortChunk;
+    const int id_bits = E > 1 ? 32 - __clz(E - 1) : 0;
     for (int i = threadIdx.x; i < 16 * E; i += 256) round_cnt[i / E][i % E] = 0;
     __syncthreads();
     int my_e[4], my_rank[4];
@@ -290,18 +321,18 @@ __global__ __launch_bounds__(256) void moe_sort_scatter_kernel(const int32_t* __
         const int sidx = base + rnd * 64 + lane;
         const int e = sidx < S ? ids[sidx] : -1;
         my_e[q] = e;
-        // stable rank among equal ids inside this round of 64
-        uint64_t todo = __ballot(e >= 0);
+        // lanes of this round holding the same id, from one ballot per id bit; the stable rank
+        // among equal ids is the number of such lanes below this one
+        uint64_t same = __ballot(e >= 0);
+        for (int b = 0; b < id_bits; ++b) {
+            const bool bit = (e >> b) & 1;
+            const uint64_t m = __ballot(bit);
+            same &= bit ? m : ~m;
+        }
         int rank = 0;
-        while (todo) {
-            const int leader = __ffsll((unsigned long long)todo) - 1;
-            const int e0 = __shfl(e, leader, 64);
-            const uint64_t same = __ballot(e == e0);
-            if (e == e0) {
-                rank = __popcll(same & ((1ull << lane) - 1ull));
-                if (lane == leader) round_cnt[rnd][e0] = __popcll(same);
-            }
-            todo &= ~same;
+        if (e >= 0) {
+            rank = __popcll(same & ((1ull << lane) - 1ull));
+            if (rank == 0) round_cnt[rnd][e] = __popcll(same);
         }
         my_rank[q] = rank;
     }
@@ -378,9 +409,14 @@ extern "C" int hk_moe_sort(const int32_t* ids, int T, int k, int E, int32_t* sor
     hipStream_t s = (hipStream_t)stream;
     int32_t* ws = (int32_t*)workspace;
     hipLaunchKernelGGL(moe_sort_count_kernel, dim3(nchunks), dim3(256), 0, s, ids, S, E, ws);
-    int32_t* totals = ws + (size_t)nchunks * E;
-    hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(E), dim3(256), 0, s, ws, nchunks, E, totals);
-    hipLaunchKernelGGL(moe_sort_offsets_kernel, dim3(1), dim3(512), 0, s, (const int32_t*)totals, E, expert_offsets);
+    if (nchunks <= kSortFusedChunks) {
+        hipLaunchKernelGGL(moe_sort_scan_offsets_kernel, dim3(1), dim3(512), 0, s, ws, nchunks, E, expert_offsets);
+    } else {
+        int32_t* totals = ws + (size_t)nchunks * E;
+        hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(E), dim3(256), 0, s, ws, nchunks, E, totals);
+        hipLaunchKernelGGL(moe_sort_offsets_kernel, dim3(1), dim3(512), 0, s, (const int32_t*)totals, E,
+                           expert_offsets);
+    }
     hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(nchunks), dim3(256), 0, s, ids, S, E,
                        (const int32_t*)ws, (const int32_t*)expert_offsets, sorted_slots, slot_to_pos_or_null);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
