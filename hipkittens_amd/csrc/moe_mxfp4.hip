@@ -93,27 +93,27 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_rows_kernel(const uint16_t
 // The same launch pads the second tiled matrix of the layer (h, contraction length K2): the part
 // of its last K-step past K2 that the producing GEMM epilogue never writes is set to zero data
 // and neutral scales (nothing to do when K2 is a multiple of 256).
-__global__ __launch_bounds__(256) void mxfp4_quantize_permute_kernel(
+// Launch: 128 threads = 4 K-steps x 32 threads (8 elements each); grid (S, ceil(nk / 4)).
+__global__ __launch_bounds__(128) void mxfp4_quantize_permute_kernel(
     const uint16_t* __restrict__ x, const int32_t* __restrict__ sorted_slots, int topk, int S, int cols,
     uint8_t* __restrict__ tiled, uint8_t* __restrict__ tiled_scales, uint8_t* __restrict__ tiled2,
     uint8_t* __restrict__ tiled2_scales, int K2) {
     const int nk = (cols / 2 + 127) >> 7;
-    const int per_row = nk * 32;  // threads per row: one per 8 elements of the padded row
-    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
-    const int pos = (int)(gid / per_row);
-    const int c8 = (int)(gid % per_row);
-    if (pos >= S) return;
-    if (c8 < 32 && (K2 & 255)) {
+    const int pos = blockIdx.x;
+    const int kt = blockIdx.y * 4 + (threadIdx.x >> 5), c = threadIdx.x & 31;  // K-step, 4-byte column
+    if (blockIdx.y == 0 && threadIdx.x < 32 && (K2 & 255)) {
         const int Kb2 = K2 >> 1, nk2 = (Kb2 + 127) >> 7;
         const int valid = Kb2 - (nk2 - 1) * 128;  // valid bytes of the last K-step, a multiple of 16
         const size_t tile_row2 = (size_t)(nk2 - 1) * S + pos;
-        if (c8 * 4 >= valid) *(uint32_t*)(tiled2 + tile_row2 * 128 + c8 * 4) = 0u;
-        if (c8 < 8 && c8 * 16 >= valid) tiled2_scales[tile_row2 * 8 + c8] = 127;
+        if (c * 4 >= valid) *(uint32_t*)(tiled2 + tile_row2 * 128 + c * 4) = 0u;
+        if (c < 8 && c * 16 >= valid) tiled2_scales[tile_row2 * 8 + c] = 127;
     }
+    if (kt >= nk) return;
     const int row = sorted_slots[pos] / topk;
+    const int col = kt * 256 + c * 8;
     float v[8];
-    if (c8 * 8 < cols) {
-        const v4i raw = *(const v4i*)(x + (size_t)row * cols + c8 * 8);
+    if (col < cols) {
+        const v4i raw = *(const v4i*)(x + (size_t)row * cols + col);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             v[2 * i] = __uint_as_float((uint32_t)raw[i] << 16);
@@ -129,9 +129,9 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_permute_kernel(
     amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
     amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
     const int e = mx_block_exponent(amax);
-    const size_t tile_row = (size_t)(c8 >> 5) * S + pos;  // (kt, pos)
-    *(uint32_t*)(tiled + tile_row * 128 + (c8 & 31) * 4) = pack8_e2m1(v, e);
-    if ((c8 & 3) == 0) tiled_scales[tile_row * 8 + ((c8 >> 2) & 7)] = (uint8_t)(e + 127);
+    const size_t tile_row = (size_t)kt * S + pos;
+    *(uint32_t*)(tiled + tile_row * 128 + c * 4) = pack8_e2m1(v, e);
+    if ((c & 3) == 0) tiled_scales[tile_row * 8 + (c >> 2)] = (uint8_t)(e + 127);
 }
 
 // ---------------------------------------------------------------------- weight pre-shuffle
@@ -604,24 +604,39 @@ __global__ __launch_bounds__(256, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
     // ---- weights: global -> registers -----------------------------------------------------------
     // pre-shuffled layout (moe_preshuffle_kernel): [expert][n-tile][K-step][wave][fragment][lane][16]
     const int voff_b = lane * 16, voff_sb = lane * 8;  // scales: dword 0 first K half, dword 1 second
-    auto rsrc_b = [&](const Cursor& c) __attribute__((always_inline)) {
-        const uint8_t* base = p.B + (size_t)c.expert * p.b_expert_stride + (size_t)c.n_tile * nk * kMoeBTile;
-        return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, c.valid ? nk * kMoeBTile : 0, 0x00020000);
+    // The loads are inline asm: the compiler takes the registers as written at once and never
+    // waits for them itself; every use is preceded by one of the vmcnt waits below followed by
+    // `landed`, which makes the compiler see a new value there (so that nothing it derives from
+    // these registers can be placed before the wait).
+    auto srd_b = [&](const Cursor& c) __attribute__((always_inline)) {
+        return make_srd(p.B + (size_t)c.expert * p.b_expert_stride + (size_t)c.n_tile * nk * kMoeBTile,
+                        c.valid ? (uint32_t)nk * kMoeBTile : 0u);
     };
-    auto rsrc_sb = [&](const Cursor& c) __attribute__((always_inline)) {
-        const uint8_t* base = p.SB + (size_t)c.expert * p.sb_expert_stride + (size_t)c.n_tile * nk * kMoeScaleB;
-        return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, c.valid ? nk * kMoeScaleB : 0, 0x00020000);
+    auto srd_sb = [&](const Cursor& c) __attribute__((always_inline)) {
+        return make_srd(p.SB + (size_t)c.expert * p.sb_expert_stride + (size_t)c.n_tile * nk * kMoeScaleB,
+                        c.valid ? (uint32_t)nk * kMoeScaleB : 0u);
     };
     v4i bw[2][2][NT];  // [K-step parity][K half][fragment]
     int bsc[2][2];     // [K-step parity][K half]: the lane's scale bytes of fragments 0..3
-    auto load_b_half = [&](const Cursor& c, v4i (&dst)[NT], int half) {
-        const __amdgpu_buffer_rsrc_t rs = rsrc_b(c);
-        const int soff = c.kt * kMoeBTile + w * 8192 + half * 1024;
+    // 1 scale load + 4 fragment loads of one K half of the weight fetch position
+    auto load_b_half = [&](const Cursor& c, v4i (&dst)[NT], int& dst_scale, int half) __attribute__((always_inline)) {
+        const v4i rs = srd_b(c), rss = srd_sb(c);
+        const uint32_t soff = (uint32_t)c.kt * kMoeBTile + (uint32_t)w * 8192u + (uint32_t)half * 1024u;
+        asm volatile("buffer_load_dword %0, %1, %2, %3 offen"
+                     : "=v"(dst_scale)
+                     : "v"(voff_sb), "s"(rss), "s"((uint32_t)c.kt * kMoeScaleB + (uint32_t)w * 512u + (uint32_t)half * 4u)
+                     : "memory");
 #pragma unroll
-        for (int n = 0; n < NT; ++n) dst[n] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_b, soff + n * 2048, 0);
+        for (int n = 0; n < NT; ++n)
+            asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"
+                         : "=v"(dst[n])
+                         : "v"(voff_b), "s"(rs), "s"(soff + n * 2048u)
+                         : "memory");
     };
-    auto load_b_scales = [&](const Cursor& c, int& dst, int half) __attribute__((always_inline)) {
-        dst = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sb(c), voff_sb, c.kt * kMoeScaleB + w * 512 + half * 4, 0);
+    auto landed = [&](v4i (&x)[NT], int& sc) __attribute__((always_inline)) {
+#pragma unroll
+        for (int n = 0; n < NT; ++n) asm volatile("" : "+v"(x[n]));
+        asm volatile("" : "+v"(sc));
     };
 
     // ---- LDS -> registers (activation fragments) ------------------------------------------------
@@ -643,22 +658,41 @@ __global__ __launch_bounds__(256, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
             : "+v"(c)
             : "v"(x), "v"(y), "v"(sx), "v"(sy));
     };
-    // MFMAs of one K half (128 of the K-step's 256 elements) on LDS stage st
-    auto compute_half = [&](int st, int half, int rows, const v4i (&bfr)[NT], int bscale) {
+    // MFMAs of one K half (128 of the K-step's 256 elements) on LDS stage st. Activation fragment
+    // m + 2 is read from LDS before the MFMAs of fragment m are issued; fragments past the tile's
+    // row count are skipped (the conditions are uniform and nested).
+    auto compute_half = [&](int st, int half, int rows, const v4i (&bfr)[NT], int bscale)
+                            __attribute__((always_inline)) {
         uint32_t a_rd = rd_half[half] + (uint32_t)st * kStStage;
         uint32_t sa_rd = sa_rd0 + (uint32_t)st * kStStage + 4u * half;
         asm volatile("" : "+v"(a_rd), "+v"(sa_rd));  // keep the bases in registers, offsets as immediates
         int bs[NT];
 #pragma unroll
         for (int n = 0; n < NT; ++n) bs[n] = (int)((uint32_t)bscale >> (8 * n));
+        const int mt = (rows + 15) >> 4;
+        v4i af[3];
+        uint32_t as[3];
+        auto rd = [&](int m) __attribute__((always_inline)) {
+            af[m % 3] = *(lds_v4i_t*)(uintptr_t)(a_rd + m * 2048);
+            as[m % 3] = *(__attribute__((address_space(3))) const uint32_t*)(uintptr_t)(sa_rd + m * 128);
+        };
+        // nested conditions (fragment m is reached only through fragment m - 1), so that every
+        // block has one way in and the compiler's LDS wait counts stay exact
+        auto frag = [&]<int M>(auto&& self) __attribute__((always_inline)) {
+            if constexpr (M < MT) {
+                if (M < mt) {
+                    if (M + 2 < MT) rd(M + 2);  // rows past the tile's count are readable, never used
+                    const int sa = (int)(as[M % 3] >> sh);
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            if (16 * m < rows) {
-                const v4i af = *(lds_v4i_t*)(uintptr_t)(a_rd + m * 2048);
-                const int as = (int)(*(__attribute__((address_space(3))) const uint32_t*)(uintptr_t)(sa_rd + m * 128) >> sh);
-#pragma unroll
-                for (int n = 0; n < NT; ++n) mfma(acc[m][n], bfr[n], af, bs[n], as);
+                    for (int n = 0; n < NT; ++n) mfma(acc[M][n], bfr[n], af[M % 3], bs[n], sa);
+                    self.template operator()<M + 1>(self);
+                }
             }
+        };
+        if (mt > 0) {
+            rd(0);
+            rd(1);
+            frag.template operator()<0>(frag);
         }
     };
 
@@ -719,57 +753,49 @@ __global__ __launch_bounds__(256, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
         }
     };
 
-    // ---- prologue: positions 0..2 of the activation ring, positions 0 and 1 of the weights ----
+    // ---- prologue: positions 0..2 of the activation ring, positions 0 and 1 of the weights,
+    // in the order the K loop issues them (5 activation loads between two weight sets), so that
+    // the same load counts hold from the first position on
     issue_a(ca, 0); advance(ca);
     issue_a(ca, 1); advance(ca);
+    load_b_half(cb, bw[0][0], bsc[0][0], 0); load_b_half(cb, bw[0][1], bsc[0][1], 1); advance(cb);
     issue_a(ca, 2); advance(ca);
-    // (scales first in every half set: they are the first thing a pass needs, and the wait the
-    // compiler derives for them then allows every younger load to stay in flight)
-    __builtin_amdgcn_sched_barrier(0);
-    auto load_b_set = [&]<int P>() __attribute__((always_inline)) {
-        load_b_scales(cb, bsc[P][0], 0);
-        __builtin_amdgcn_sched_barrier(0);
-        load_b_half(cb, bw[P][0], 0);
-        __builtin_amdgcn_sched_barrier(0);
-        load_b_scales(cb, bsc[P][1], 1);
-        __builtin_amdgcn_sched_barrier(0);
-        load_b_half(cb, bw[P][1], 1);
-        __builtin_amdgcn_sched_barrier(0);
-        advance(cb);
-    };
-    load_b_set.template operator()<0>();
-    load_b_set.template operator()<1>();
+    load_b_half(cb, bw[1][0], bsc[1][0], 0); load_b_half(cb, bw[1][1], bsc[1][1], 1); advance(cb);
     zero_acc();
 
     // One stream position with register-set parity P on LDS stage st. In program order a wave
-    // issues per position: 5 activation loads (position +3) and twice 1 scale load + 4 weight loads
-    // (position +2), each half into the registers the MFMAs before it have just finished with.
-    // When a position starts, the 10 weight loads of position +1 and the 5 activation loads of
-    // position +2 may still be in flight: everything older - this position's weights and its
-    // activation tile - has landed after vmcnt(15).
+    // issues per position: 5 activation loads (position +3), then after each K half 1 scale load
+    // + 4 weight loads (position +2) into the registers that half's MFMAs have just finished
+    // with. Loads return in order, so counting the loads issued after the ones needed gives:
+    //   first K half:  its weights were followed by 5 (second half) + 15 (previous position)  -> vmcnt(20)
+    //   second K half: by 15 (previous position) + 5 + 5 (this position so far)                -> vmcnt(25)
+    // and the activation tile of the position is older than both. Stores share the counter and
+    // complete out of order, so behind an epilogue's stores those counts would wait for far more
+    // than needed: the position that ends an item first waits until everything the next position
+    // needs has landed (all but the 15 loads it issued itself), then stores, and the next
+    // position runs without waiting.
+    bool after_stores = false;
     auto step = [&]<int P>(int st) __attribute__((always_inline)) {
-        wait_vmcnt<15>();
+        const bool last = cc.valid && cc.kt == nk - 1;
+        if (!after_stores) wait_vmcnt<20>();
         block_barrier();  // everyone's part of this position's tile has landed; stage st-1 is free
         issue_a(ca, (st + 3) & 3); advance(ca);
+        landed(bw[P][0], bsc[P][0]);
         const int rows = cc.valid ? cc.rows : 0;  // past the end of the stream: no MFMAs, empty loads
         compute_half(st, 0, rows, bw[P][0], bsc[P][0]);
-        __builtin_amdgcn_sched_barrier(0);  // the refill of a register set follows its last use
-        load_b_scales(cb, bsc[P][0], 0);
-        __builtin_amdgcn_sched_barrier(0);
-        load_b_half(cb, bw[P][0], 0);
-        __builtin_amdgcn_sched_barrier(0);
+        load_b_half(cb, bw[P][0], bsc[P][0], 0);
+        if (!after_stores) wait_vmcnt<25>();
+        landed(bw[P][1], bsc[P][1]);
         compute_half(st, 1, rows, bw[P][1], bsc[P][1]);
-        __builtin_amdgcn_sched_barrier(0);
-        load_b_scales(cb, bsc[P][1], 1);
-        __builtin_amdgcn_sched_barrier(0);
-        load_b_half(cb, bw[P][1], 1);
+        load_b_half(cb, bw[P][1], bsc[P][1], 1);
         advance(cb);
-        __builtin_amdgcn_sched_barrier(0);
-        if (cc.valid && cc.kt == nk - 1) {
+        if (last) {
+            wait_vmcnt<15>();
             mfma_drain();
             epilogue(cc);
             zero_acc();
         }
+        after_stores = last;
         advance(cc);
     };
     // Two positions per trip (the register sets alternate); the second one may lie past the end
@@ -982,8 +1008,8 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
     const int S = T * k;
 
     {
-        const long long threads = (long long)S * ((H / 2 + 127) / 128) * 32;
-        hipLaunchKernelGGL(mxfp4_quantize_permute_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
+        const int nk1 = (H / 2 + 127) / 128;
+        hipLaunchKernelGGL(mxfp4_quantize_permute_kernel, dim3(S, (nk1 + 3) / 4), dim3(128), 0, s,
                            (const uint16_t*)x_bf16, sorted_slots, k, S, H, ws + L.xq, ws + L.xs, ws + L.hq,
                            ws + L.hs, I);
     }
