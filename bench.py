@@ -119,18 +119,13 @@ def bench_moe_fp8blk(torch, hk, warmup, iters, dev):
         w2q[e], w2s[e] = hk.quant.quantize_fp8_blocks(torch.randn(H, I, device=dev, generator=g) * 0.02, 128, 128)
     ws = torch.empty(hk.tk_kernel.moe_fp8blk_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=dev)
     y = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
-    compulsory = w13q.numel() + w2q.numel() + T * H + T * H * 2
-    # weights in the pre-shuffled layout (an offline, once-per-checkpoint step; the plain copies are dropped)
-    W = hk.tk_kernel.MoeFp8blkShuffledWeights.from_plain(w13q, w13s, w2q, w2s)
-    torch.cuda.synchronize()
-    del w13q, w2q
-    torch.cuda.empty_cache()
-    _, kern = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_fp8blk(xq, xs, logits, None, W, None, None, None, y,
+    _, kern = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_fp8blk(xq, xs, logits, None, w13q, w13s, w2q, w2s, y,
                                                                       k, G, KG, 1.0, ws), warmup, iters)
     flop = 2.0 * T * k * (H * 2 * I + I * H)
     tf = flop / (kern * 1e-3) / 1e12
+    compulsory = w13q.numel() + w2q.numel() + T * H + T * H * 2
     return {"workload": "moe_fp8blk T=8192 H=7168 I=2048 E=256 top-8 sigmoid (8 groups / top-4), e4m3 with "
-                        "1x128 / 128x128 fp32 scales, pre-shuffled weights",
+                        "1x128 / 128x128 fp32 scales",
             "ms": round(kern, 5), "tflops": round(tf, 1), "frac_of_fp8_peak": round(tf / PEAK_FP8, 4),
             "compulsory_GB": round(compulsory / 1e9, 3),
             "frac_of_hbm_roofline": round(compulsory / (kern * 1e-3) / 1e9 / PEAK_HBM, 4)}

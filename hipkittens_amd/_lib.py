@@ -37,12 +37,10 @@ SIGNATURES = {
                                         c_void_p]),
     "hk_fp8_quantize_rows_1x128": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "hk_moe_fp8blk_workspace_bytes": (c_size_t, [c_int] * 5),
-    "hk_moe_fp8blk_preshuffle_bytes": (c_int, [c_int, c_int, c_int, c_int, ctypes.POINTER(c_size_t)]),
-    "hk_moe_fp8blk_preshuffle": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
-    "hk_moe_fp8blk_experts": (c_int, [c_void_p] * 11 + [c_int] * 6 + [c_void_p, c_size_t, c_void_p]),
+    "hk_moe_fp8blk_experts": (c_int, [c_void_p] * 11 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p]),
     "hk_moe_fp8blk_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p,
                                       c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                      c_int, c_void_p, c_size_t, c_void_p]),
+                                      c_void_p, c_size_t, c_void_p]),
     "hk_probe_mfma_rate": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
 }
 

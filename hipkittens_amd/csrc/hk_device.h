@@ -152,9 +152,6 @@ __device__ __forceinline__ int scalar_load_x1(const void* p) {
 __device__ __forceinline__ void store_global_b128(void* p, v4i v) {
     asm volatile("global_store_dwordx4 %0, %1, off" ::"v"(p), "v"(v) : "memory");
 }
-__device__ __forceinline__ void store_global_b64(void* p, v2i v) {
-    asm volatile("global_store_dwordx2 %0, %1, off" ::"v"(p), "v"(v) : "memory");
-}
 __device__ __forceinline__ void store_global_b32(void* p, uint32_t v) {
     asm volatile("global_store_dword %0, %1, off" ::"v"(p), "v"(v) : "memory");
 }

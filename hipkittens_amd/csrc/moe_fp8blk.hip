@@ -336,299 +336,6 @@ static int launch_fp8blk_gemm(const MoeFp8Params& p, int max_items, hipStream_t 
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
-// ------------------------------------------------------- grouped GEMM, pre-shuffled weights
-// Pre-shuffled weight layout: for every (expert, n-tile of 256 tile rows, K-step of 128) one
-// contiguous 32 KiB block; inside it, wave by wave (wave wn = tile rows [64 wn, +64)), the wave's
-// four MFMA B fragments, each as two 1 KiB pieces in lane order: lane l's 16 bytes of piece
-// `part` are tile row 64 wn + 16 f + l % 16 (moe_b_row gives the weight row), K bytes
-// 128 kt + 64 part + 16 (l / 16) .. +16. Scales stay in their plain [E][rows/128][K/128] layout.
-//   out_w [E][n_tiles][nk][4][4][2][64][16] bytes
-__global__ __launch_bounds__(256) void moe_fp8blk_preshuffle_kernel(const uint8_t* __restrict__ w, int E, int N,
-                                                                    int K, int mode, int n_tiles,
-                                                                    uint8_t* __restrict__ out_w) {
-    const int nk = K >> 7;
-    const int rows_b = mode == 0 ? 2 * N : N;
-    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;  // one 16-byte chunk each
-    const long long total = (long long)E * n_tiles * nk * 2048;
-    if (gid >= total) return;
-    const int l = (int)(gid & 63), part = (int)((gid >> 6) & 1), f = (int)((gid >> 7) & 3), wn = (int)((gid >> 9) & 3);
-    long long rest = gid >> 11;
-    const int kt = (int)(rest % nk); rest /= nk;
-    const int nt = (int)(rest % n_tiles);
-    const int e = (int)(rest / n_tiles);
-    const int row = moe_b_row(mode, 64 * wn + 16 * f + (l & 15), nt, N);
-    const int kb = kt * 128 + 64 * part + 16 * (l >> 4);
-    *(v4i*)(out_w + gid * 16) = *(const v4i*)(w + ((size_t)e * rows_b + row) * K + kb);
-}
-
-// Weight-streaming variant of moe_fp8blk_gemm_kernel for the pre-shuffled layout; same design as
-// moe_mxfp4_stream_kernel (moe_mxfp4.hip): 4-wave workgroups, two per CU, wave wn owns weight
-// rows [64 wn, +64) x all 128 activation rows; weights go from HBM straight into MFMA operand
-// registers two K-steps ahead (a ring of four half-K-step register sets, here the two halves of
-// a K-step are its fragment pairs 0,1 and 2,3), only the activation tile passes through a
-// four-stage LDS ring. The weights' 128 x 128 block scales ride the same stream as broadcast
-// dword loads. Every vector-memory operation is inline asm and counted by hand (see the MXFP4
-// kernel for the wait scheme). Results are bit-identical to moe_fp8blk_gemm_kernel.
-// Meant for shapes with few rows per expert, where reading the weights once is what counts; with
-// hundreds of rows per expert the LDS-staged kernel above overlaps its MFMA work better.
-constexpr int kFsStages = 4;
-constexpr int kFsStage = kF8ATile + 1024;            // 16 KiB tile + 512 B of row scales (1 KiB slot)
-constexpr int kFsXch = kFsStages * kFsStage;         // epilogue exchange: kMoeBM x 4 floats
-constexpr int kFsLds = kFsXch + kMoeBM * 16;         // 70 KiB
-
-template <int MODE>
-__global__ __launch_bounds__(256, 2) void moe_fp8blk_stream_kernel(const MoeFp8Params p) {
-    constexpr int MT = kMoeBM / 16, NT = 4;
-    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
-    const int lane = lane_id(), w = wave_id();
-    const int n_items = scalar_load_x1(p.num_items);
-    const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
-    const int it_stride = ((int)gridDim.x - xcd + kNumXcd - 1) / kNumXcd;
-    const int per_xcd = (n_items + kNumXcd - 1) / kNumXcd;
-    const int it0 = xcd * per_xcd + slot;
-    const int it_end = min(n_items, (xcd + 1) * per_xcd);
-    if (it0 >= it_end) return;
-
-    const int nk = p.K >> 7;
-    const v4i srd_a = make_srd(p.A, (uint32_t)nk * (uint32_t)p.S * 128u);
-    const v4i srd_sa = make_srd(p.SA, (uint32_t)nk * (uint32_t)p.S * 4u);
-
-    struct Cursor { int it, kt, expert, row_start, rows, n_tile; bool valid; };
-    auto load_item = [&](Cursor& c) __attribute__((always_inline)) {
-        c.valid = c.it < it_end;
-        const v4i item = scalar_load_x4(p.items + (c.valid ? c.it : it_end - 1));
-        c.expert = item.x; c.row_start = item.y; c.rows = item.z; c.n_tile = item.w;
-    };
-    auto advance = [&](Cursor& c) __attribute__((always_inline)) {
-        if (++c.kt == nk) { c.kt = 0; c.it += it_stride; load_item(c); }
-    };
-    Cursor cc{it0, 0}, ca{it0, 0}, cb{it0, 0};  // compute, activation fetch, weight fetch
-    load_item(cc);
-    ca = cc; cb = cc;
-
-    // ---- activation tile: global -> LDS ---------------------------------------------------------
-    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
-    const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-    const uint32_t lds_sa_wave = to_sgpr(lds0 + kF8ATile + (uint32_t)w * 128u);
-    const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);
-    uint32_t voff_a[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) voff_a[i] = (uint32_t)(8 * (i * 4 + w) + (lane >> 3)) * 128u + chunk16 * 16u;
-    const uint32_t voff_sa = (uint32_t)(w * 128 + lane * 16);
-    // 5 loads: the wave's quarter of the tile (rows 8(4i + w) .. +8) and of its row scales (32 rows)
-    auto issue_a = [&](const Cursor& c, int stage) __attribute__((always_inline)) {
-        v4i sa = srd_a, ssa = srd_sa;
-        if (!c.valid) { sa.z = 0; ssa.z = 0; }
-        const uint32_t row_base = (uint32_t)c.kt * (uint32_t)p.S + (uint32_t)c.row_start;
-        const uint32_t dst = lds_wave + (uint32_t)stage * kFsStage;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(sa, dst + i * 4096, voff_a[i], row_base * 128u);
-        dma16_lanes(ssa, lds_sa_wave + (uint32_t)stage * kFsStage, voff_sa, row_base * 4u, 0xffull);
-    };
-
-    // ---- weights and their block scales: global -> registers -------------------------------------
-    const uint32_t voff_b = lane * 16;
-    auto srd_b = [&](const Cursor& c) __attribute__((always_inline)) {
-        return make_srd(p.B + (size_t)c.expert * p.b_expert_stride + (size_t)c.n_tile * nk * kF8BTile,
-                        c.valid ? (uint32_t)nk * kF8BTile : 0u);
-    };
-    // scale rows of the wave's fragments: MODE 0 gate block n_tile and up block I/128 + n_tile
-    // (even fragments are gate rows, odd ones up rows); MODE 1 the 128-row block of the wave's 64 rows
-    auto srd_s = [&](const Cursor& c, int which) __attribute__((always_inline)) {
-        const float* sb = p.SB + (size_t)c.expert * p.sb_expert_stride;
-        int blk;
-        if (MODE == 0) blk = which ? p.N / 128 + c.n_tile : c.n_tile;
-        else blk = min(2 * c.n_tile + (w >> 1), p.N / 128 - 1);
-        return make_srd(sb + (size_t)blk * nk, c.valid ? (uint32_t)nk * 4u : 0u);
-    };
-    v4i bw[2][2][4];   // [K-step parity][fragment pair][fragment of the pair x 16-byte piece]
-    float wsc[2][2];   // [K-step parity][gate / up] block scales of the fetched K-step
-    auto load_b_half = [&](const Cursor& c, v4i (&dst)[4], int half) __attribute__((always_inline)) {
-        const v4i rs = srd_b(c);
-        const uint32_t soff = (uint32_t)c.kt * kF8BTile + (uint32_t)w * 8192u + (uint32_t)half * 4096u;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"
-                         : "=v"(dst[j])
-                         : "v"(voff_b), "s"(rs), "s"(soff + j * 1024u)
-                         : "memory");
-    };
-    auto load_b_scales = [&](const Cursor& c, float (&dst)[2]) __attribute__((always_inline)) {
-        const uint32_t zero = 0;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const v4i rs = srd_s(c, i);
-            asm volatile("buffer_load_dword %0, %1, %2, %3 offen"
-                         : "=v"(dst[i])
-                         : "v"(zero), "s"(rs), "s"((uint32_t)c.kt * 4u)
-                         : "memory");
-        }
-    };
-    auto landed = [&](v4i (&x)[4]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(x[j]));
-    };
-
-    // ---- LDS -> registers (activation fragments) ------------------------------------------------
-    const uint32_t r = lane & 15, g = lane >> 4;
-    const uint32_t rd_lo = lds0 + r * 128u + swz_chunk(r, g) * 16u;
-    const uint32_t rd_hi = lds0 + r * 128u + swz_chunk(r, g + 4) * 16u;
-    const uint32_t sa_rd0 = lds0 + kF8ATile + r * 4u;
-
-    v4f acc[MT][NT];
-    auto zero_acc = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int m = 0; m < MT; ++m)
-#pragma unroll
-            for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
-    };
-    // fragment pair `half` (a gate and an up fragment in MODE 0) against all activation fragments
-    auto compute_half = [&](int st, int half, int rows, const v4i (&bfr)[4], float ws0, float ws1)
-                            __attribute__((always_inline)) {
-        uint32_t a_lo = rd_lo + (uint32_t)st * kFsStage, a_hi = rd_hi + (uint32_t)st * kFsStage;
-        uint32_t sa_rd = sa_rd0 + (uint32_t)st * kFsStage;
-        asm volatile("" : "+v"(a_lo), "+v"(a_hi), "+v"(sa_rd));
-        const v8i b0 = __builtin_shufflevector(bfr[0], bfr[1], 0, 1, 2, 3, 4, 5, 6, 7);
-        const v8i b1 = __builtin_shufflevector(bfr[2], bfr[3], 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            if (16 * m < rows) {
-                const v8i af = lds_frag(a_lo, a_hi, m * 2048);
-                const float xs = *(lds_f32_t*)(uintptr_t)(sa_rd + m * 64);
-                const float s0 = xs * ws0, s1 = xs * ws1;
-                const v4f p0 = mfma_fp8_16x16x128(b0, af, v4f{0.f, 0.f, 0.f, 0.f});
-                const v4f p1 = mfma_fp8_16x16x128(b1, af, v4f{0.f, 0.f, 0.f, 0.f});
-                acc[m][2 * half] += p0 * s0;
-                acc[m][2 * half + 1] += p1 * s1;
-            }
-        }
-    };
-
-    auto epilogue = [&](const Cursor& c) __attribute__((always_inline)) {
-        const int rows = c.rows, row_start = c.row_start;
-        const int n0 = c.n_tile * (MODE == 0 ? 128 : 256);
-        if (MODE == 1) {
-            uint16_t* out = (uint16_t*)p.out0;
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                const int row = 16 * m + (int)r;
-                if (row >= rows) continue;
-                const size_t pos = (size_t)(row_start + row);
-#pragma unroll
-                for (int q = 0; q < NT / 2; ++q) {
-                    const int col = n0 + w * 64 + 32 * q + 8 * (int)g;
-                    if (col + 8 > p.N) continue;
-                    const v4f x = acc[m][2 * q], y = acc[m][2 * q + 1];
-                    v4i o4;
-                    o4.x = pack_bf16(x.x, x.y); o4.y = pack_bf16(x.z, x.w);
-                    o4.z = pack_bf16(y.x, y.y); o4.w = pack_bf16(y.z, y.w);
-                    store_global_b128(out + pos * p.N + col, o4);
-                }
-            }
-        } else {
-            // see moe_fp8blk_gemm_kernel: the tile's 128 h columns are one 1 x 128 block, the row
-            // maxima of the four waves are combined through LDS
-            uint8_t* hq = (uint8_t*)p.out0;
-            float h[MT][8];
-            const uint32_t xch = lds0 + kFsXch;
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-#pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    const v4f gt = acc[m][2 * q], up = acc[m][2 * q + 1];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const float gv = gt[j];
-                        h[m][4 * q + j] = gv / (1.0f + __expf(-gv)) * up[j];
-                    }
-                }
-                float amax = 0.f;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(h[m][i]));
-                amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-                const int row = 16 * m + (int)r;
-                if (g == 0) *(lds_f32_mut_t*)(uintptr_t)(xch + (row * 4 + w) * 4) = amax;
-            }
-            __syncthreads();
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                const int row = 16 * m + (int)r;
-                const v4f am = *(lds_v4f_t*)(uintptr_t)(xch + row * 16);
-                const float s = e4m3_block_scale(fmaxf(fmaxf(am.x, am.y), fmaxf(am.z, am.w)));
-                if (row < rows) {
-                    const size_t tile_row = (size_t)c.n_tile * p.S + (size_t)(row_start + row);
-                    store_global_b64(hq + tile_row * 128 + 32 * w + 8 * g, quant8_e4m3(h[m], s));
-                    if (w == 0 && g == 0) store_global_b32(p.out_scales + tile_row, __float_as_uint(s));
-                }
-            }
-        }
-    };
-
-    // ---- prologue, in the order the K loop issues its loads -------------------------------------
-    issue_a(ca, 0); advance(ca);
-    issue_a(ca, 1); advance(ca);
-    load_b_scales(cb, wsc[0]); load_b_half(cb, bw[0][0], 0); load_b_half(cb, bw[0][1], 1); advance(cb);
-    issue_a(ca, 2); advance(ca);
-    load_b_scales(cb, wsc[1]); load_b_half(cb, bw[1][0], 0); load_b_half(cb, bw[1][1], 1); advance(cb);
-    zero_acc();
-
-    // One stream position. Loads per wave and position, in program order: 5 activation loads
-    // (position +3), then 2 scale loads + 4 weight loads after the first fragment pair and 4 weight
-    // loads after the second (position +2). Counting the loads issued after the ones needed:
-    //   first pair:  4 (second pair) + 15 (previous position)           -> vmcnt(19)
-    //   second pair: 15 (previous position) + 5 + 6 (this position)      -> vmcnt(26)
-    // A position that ends an item waits for everything but its own 15 loads before it stores
-    // (stores share the counter and complete out of order), and the position after it does not wait.
-    bool after_stores = false;
-    auto step = [&]<int P>(int st) __attribute__((always_inline)) {
-        const bool last = cc.valid && cc.kt == nk - 1;
-        if (!after_stores) wait_vmcnt<19>();
-        block_barrier();
-        issue_a(ca, (st + 3) & 3); advance(ca);
-        landed(bw[P][0]);
-        asm volatile("" : "+v"(wsc[P][0]), "+v"(wsc[P][1]));
-        // copies: the scale registers are refilled before the second pair has used them
-        float ws0 = wsc[P][0], ws1 = MODE == 0 ? wsc[P][1] : wsc[P][0];
-        asm volatile("" : "+v"(ws0), "+v"(ws1));
-        const int rows = cc.valid ? cc.rows : 0;
-        compute_half(st, 0, rows, bw[P][0], ws0, ws1);
-        load_b_scales(cb, wsc[P]);
-        load_b_half(cb, bw[P][0], 0);
-        if (!after_stores) wait_vmcnt<26>();
-        landed(bw[P][1]);
-        compute_half(st, 1, rows, bw[P][1], ws0, ws1);
-        load_b_half(cb, bw[P][1], 1);
-        advance(cb);
-        if (last) {
-            wait_vmcnt<15>();
-            epilogue(cc);
-            zero_acc();
-        }
-        after_stores = last;
-        advance(cc);
-    };
-    for (int st = 0; cc.valid; st ^= 2) {
-        step.template operator()<0>(st);
-        step.template operator()<1>(st + 1);
-    }
-    wait_vmcnt<0>();
-}
-
-template <int MODE>
-static int launch_fp8blk_stream(const MoeFp8Params& p, int max_items, hipStream_t s) {
-    auto kern = moe_fp8blk_stream_kernel<MODE>;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kFsLds) != hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
-    const int grid = min(max_items, 2 * moe_num_compute_units());
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), kFsLds, s, p);
-    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
-}
-
 struct Fp8Ws {
     size_t ids, w, sorted, offsets, inv, sort_ws, items1, items2, nitems, xq, xs, hq, hs, o, total;
     int max_items1, max_items2;
@@ -682,37 +389,14 @@ extern "C" size_t hk_moe_fp8blk_workspace_bytes(int T, int H, int I, int E, int 
     return fp8_ws_layout(T, H, I, E, k).total;
 }
 
-extern "C" int hk_moe_fp8blk_preshuffle_bytes(int E, int N, int K, int mode, size_t* w_bytes) {
-    if (!w_bytes) return HK_ERR_NULL_POINTER;
-    if (E <= 0 || N <= 0 || K <= 0 || (K % 128) != 0 || (N % 128) != 0 || (mode != 0 && mode != 1))
-        return HK_ERR_BAD_SHAPE;
-    const size_t n_tiles = mode == 0 ? N / 128 : (N + 255) / 256;
-    *w_bytes = (size_t)E * n_tiles * (K / 128) * kF8BTile;
-    return HK_OK;
-}
-
-extern "C" int hk_moe_fp8blk_preshuffle(const void* w, int E, int N, int K, int mode, void* out_w, void* stream) {
-    if (!w || !out_w) return HK_ERR_NULL_POINTER;
-    if (E <= 0 || N <= 0 || K <= 0 || (K % 128) != 0 || (N % 128) != 0 || (mode != 0 && mode != 1))
-        return HK_ERR_BAD_SHAPE;
-    if (((uintptr_t)w | (uintptr_t)out_w) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    const int n_tiles = mode == 0 ? N / 128 : (N + 255) / 256;
-    const long long total = (long long)E * n_tiles * (K / 128) * 2048;
-    if ((total + 255) / 256 >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
-    hipLaunchKernelGGL(moe_fp8blk_preshuffle_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)stream, (const uint8_t*)w, E, N, K, mode, n_tiles, (uint8_t*)out_w);
-    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
-}
-
 extern "C" int hk_moe_fp8blk_experts(const void* x_e4m3, const float* x_scales, const void* w13,
                                      const float* w13_scales, const void* w2, const float* w2_scales,
                                      const float* topk_w, const int32_t* sorted_slots, const int32_t* expert_offsets,
                                      const int32_t* slot_to_pos, void* y_bf16, int T, int H, int I, int E, int k,
-                                     int weight_layout, void* workspace, size_t workspace_bytes, void* stream) {
+                                     void* workspace, size_t workspace_bytes, void* stream) {
     if (!x_e4m3 || !x_scales || !w13 || !w13_scales || !w2 || !w2_scales || !topk_w || !sorted_slots ||
         !expert_offsets || !slot_to_pos || !y_bf16)
         return HK_ERR_NULL_POINTER;
-    if (weight_layout != 0 && weight_layout != 1) return HK_ERR_UNSUPPORTED;
     int st = fp8blk_check(T, H, I, E, k);
     if (st != HK_OK) return st;
     const Fp8Ws L = fp8_ws_layout(T, H, I, E, k);
@@ -738,8 +422,7 @@ extern "C" int hk_moe_fp8blk_experts(const void* x_e4m3, const float* x_scales, 
     p.items = (const MoeItem*)(ws + L.items1); p.num_items = nitems;
     p.out0 = ws + L.hq; p.out_scales = (float*)(ws + L.hs);
     p.K = H; p.N = I; p.n_tiles_n = I / 128;
-    if (weight_layout) p.b_expert_stride = (long long)(I / 128) * (H / 128) * kF8BTile;
-    st = weight_layout ? launch_fp8blk_stream<0>(p, L.max_items1, s) : launch_fp8blk_gemm<0>(p, L.max_items1, s);
+    st = launch_fp8blk_gemm<0>(p, L.max_items1, s);
     if (st != HK_OK) return st;
 
     MoeFp8Params q{};
@@ -749,8 +432,7 @@ extern "C" int hk_moe_fp8blk_experts(const void* x_e4m3, const float* x_scales, 
     q.items = (const MoeItem*)(ws + L.items2); q.num_items = nitems + 1;
     q.out0 = ws + L.o; q.out_scales = nullptr;
     q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
-    if (weight_layout) q.b_expert_stride = (long long)((H + 255) / 256) * (I / 128) * kF8BTile;
-    st = weight_layout ? launch_fp8blk_stream<1>(q, L.max_items2, s) : launch_fp8blk_gemm<1>(q, L.max_items2, s);
+    st = launch_fp8blk_gemm<1>(q, L.max_items2, s);
     if (st != HK_OK) return st;
     return hk_moe_unpermute(ws + L.o, topk_w, slot_to_pos, T, k, H, y_bf16, stream);
 }
@@ -759,7 +441,7 @@ extern "C" int hk_moe_fp8blk_forward(const void* x_e4m3, const float* x_scales, 
                                      const float* router_bias_or_null, int n_group, int topk_group,
                                      float routed_scale, const void* w13, const float* w13_scales, const void* w2,
                                      const float* w2_scales, void* y_bf16, int T, int H, int I, int E, int k,
-                                     int weight_layout, void* workspace, size_t workspace_bytes, void* stream) {
+                                     void* workspace, size_t workspace_bytes, void* stream) {
     if (!router_logits) return HK_ERR_NULL_POINTER;
     int st = fp8blk_check(T, H, I, E, k);
     if (st != HK_OK) return st;
@@ -774,6 +456,6 @@ extern "C" int hk_moe_fp8blk_forward(const void* x_e4m3, const float* x_scales, 
     if (st != HK_OK) return st;
     return hk_moe_fp8blk_experts(x_e4m3, x_scales, w13, w13_scales, w2, w2_scales, (const float*)(ws + L.w),
                                  (const int32_t*)(ws + L.sorted), (const int32_t*)(ws + L.offsets),
-                                 (const int32_t*)(ws + L.inv), y_bf16, T, H, I, E, k, weight_layout, workspace,
-                                 workspace_bytes, stream);
+                                 (const int32_t*)(ws + L.inv), y_bf16, T, H, I, E, k, workspace, workspace_bytes,
+                                 stream);
 }

@@ -318,56 +318,9 @@ def moe_fp8blk_workspace_bytes(T: int, H: int, I: int, E: int, k: int) -> int:
     return int(_lib.load_library().hk_moe_fp8blk_workspace_bytes(T, H, I, E, k))
 
 
-class MoeFp8blkShuffledWeights:
-    """FP8 block-scaled expert weights in the pre-shuffled layout (hk_moe_fp8blk_preshuffle): built
-    once, offline, from the plain [E, rows, K] e4m3 tensors; the fp32 block scales stay as they are."""
-
-    def __init__(self, w13, w13_scales, w2, w2_scales, E: int, H: int, I: int):
-        self.w13, self.w13_scales, self.w2, self.w2_scales = w13, w13_scales, w2, w2_scales
-        self.E, self.H, self.I = E, H, I
-
-    @staticmethod
-    def _shuffle(w, N: int, K: int, mode: int):
-        import ctypes
-        lib = _lib.load_library()
-        E = w.shape[0]
-        wb = ctypes.c_size_t(0)
-        _lib.check(lib.hk_moe_fp8blk_preshuffle_bytes(E, N, K, mode, ctypes.byref(wb)), "moe_fp8blk_preshuffle_bytes")
-        out_w = torch.empty(wb.value, dtype=torch.uint8, device=w.device)
-        _lib.check(lib.hk_moe_fp8blk_preshuffle(w.data_ptr(), E, N, K, mode, out_w.data_ptr(), _stream(w)),
-                   "moe_fp8blk_preshuffle")
-        return out_w
-
-    @classmethod
-    def from_plain(cls, w13, w13_scales, w2, w2_scales):
-        _check_tensor(w13, "w13", _FP8, 3)
-        _check_tensor(w13_scales, "w13_scales", _F32, 3)
-        _check_tensor(w2, "w2", _FP8, 3)
-        _check_tensor(w2_scales, "w2_scales", _F32, 3)
-        E, twoI, H = w13.shape
-        I = twoI // 2
-        if H % 128 or I % 128 or tuple(w2.shape) != (E, H, I) or \
-                tuple(w13_scales.shape) != (E, twoI // 128, H // 128) or tuple(w2_scales.shape) != (E, H // 128, I // 128):
-            raise RuntimeError("shape mismatch between w13, w13_scales, w2 and w2_scales")
-        return cls(cls._shuffle(w13, I, H, 0), w13_scales, cls._shuffle(w2, H, I, 1), w2_scales, E, H, I)
-
-
-def _fp8blk_weights(w13, w13_scales, w2, w2_scales):
-    """-> (layout, w13, w13_scales, w2, w2_scales) with the tensors of a shuffled-weights object unpacked"""
-    if isinstance(w13, MoeFp8blkShuffledWeights):
-        return 1, w13.w13, w13.w13_scales, w13.w2, w13.w2_scales, w13
-    return 0, w13, w13_scales, w2, w2_scales, None
-
-
-def _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y, shuffled=None):
+def _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y):
     _check_tensor(x, "x", _FP8, 2)
     _check_tensor(x_scales, "x_scales", _F32, 2)
-    if shuffled is not None:
-        _check_tensor(y, "y", _BF16, 2)
-        T, H = x.shape
-        if H != shuffled.H or tuple(y.shape) != (T, H) or tuple(x_scales.shape) != (T, H // 128):
-            raise RuntimeError("shape mismatch between x, x_scales, the shuffled weights and y")
-        return T, H, shuffled.I, shuffled.E
     _check_tensor(w13, "w13", _FP8, 3)
     _check_tensor(w13_scales, "w13_scales", _F32, 3)
     _check_tensor(w2, "w2", _FP8, 3)
@@ -385,10 +338,8 @@ def _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y, shuffled=None)
 
 def dispatch_moe_fp8blk_experts(x, x_scales, w13, w13_scales, w2, w2_scales, weights, sorted_slots,
                                 expert_offsets, slot_to_pos, y, workspace) -> None:
-    """FP8 block-scaled expert MLP on routed + sorted tokens (include/hk355.h: hk_moe_fp8blk_experts).
-    `w13` may be a MoeFp8blkShuffledWeights (then w13_scales, w2 and w2_scales are ignored)."""
-    layout, w13, w13_scales, w2, w2_scales, shuf = _fp8blk_weights(w13, w13_scales, w2, w2_scales)
-    T, H, I, E = _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y, shuf)
+    """FP8 block-scaled expert MLP on routed + sorted tokens (include/hk355.h: hk_moe_fp8blk_experts)."""
+    T, H, I, E = _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y)
     _check_tensor(weights, "weights", _F32, 2)
     _check_tensor(sorted_slots, "sorted_slots", _I32, 1)
     _check_tensor(expert_offsets, "expert_offsets", _I32, 1)
@@ -401,17 +352,14 @@ def dispatch_moe_fp8blk_experts(x, x_scales, w13, w13_scales, w2, w2_scales, wei
     st = _lib.load_library().hk_moe_fp8blk_experts(
         x.data_ptr(), x_scales.data_ptr(), w13.data_ptr(), w13_scales.data_ptr(), w2.data_ptr(),
         w2_scales.data_ptr(), weights.data_ptr(), sorted_slots.data_ptr(), expert_offsets.data_ptr(),
-        slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, layout, workspace.data_ptr(), workspace.numel(),
-        _stream(x))
+        slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, workspace.data_ptr(), workspace.numel(), _stream(x))
     _lib.check(st, "dispatch_moe_fp8blk_experts")
 
 
 def dispatch_moe_fp8blk(x, x_scales, router_logits, router_bias, w13, w13_scales, w2, w2_scales, y, topk: int,
                         n_group: int, topk_group: int, routed_scale: float, workspace) -> None:
-    """Whole FP8 block-scaled MoE layer with group-limited sigmoid routing. `w13` may be a
-    MoeFp8blkShuffledWeights (then w13_scales, w2 and w2_scales are ignored)."""
-    layout, w13, w13_scales, w2, w2_scales, shuf = _fp8blk_weights(w13, w13_scales, w2, w2_scales)
-    T, H, I, E = _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y, shuf)
+    """Whole FP8 block-scaled MoE layer with group-limited sigmoid routing."""
+    T, H, I, E = _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y)
     _check_tensor(router_logits, "router_logits", _F32, 2)
     if router_bias is not None:
         _check_tensor(router_bias, "router_bias", _F32, 1)
@@ -422,5 +370,5 @@ def dispatch_moe_fp8blk(x, x_scales, router_logits, router_bias, w13, w13_scales
         x.data_ptr(), x_scales.data_ptr(), router_logits.data_ptr(),
         router_bias.data_ptr() if router_bias is not None else None, int(n_group), int(topk_group),
         float(routed_scale), w13.data_ptr(), w13_scales.data_ptr(), w2.data_ptr(), w2_scales.data_ptr(),
-        y.data_ptr(), T, H, I, E, int(topk), layout, workspace.data_ptr(), workspace.numel(), _stream(x))
+        y.data_ptr(), T, H, I, E, int(topk), workspace.data_ptr(), workspace.numel(), _stream(x))
     _lib.check(st, "dispatch_moe_fp8blk")

@@ -179,30 +179,20 @@ int hk_fp8_quantize_rows_1x128(const void* x_bf16, int rows, int cols, void* q_e
 
 size_t hk_moe_fp8blk_workspace_bytes(int T, int H, int I, int E, int k);
 
-/* Offline weight pre-shuffle (no counterpart in the reference): rewrites one expert weight tensor
- * [E, rows, K] e4m3 (mode 0: w13 with N = I, rows = 2I; mode 1: w2 with N = H, rows = H) into the
- * layout the weight-streaming grouped GEMM loads straight into MFMA operand registers
- * (one contiguous 32 KiB block per expert, 256-row tile and 128-wide K-step). The block scales
- * keep their plain layout. `*w_bytes` receives the size of the shuffled tensor. */
-int hk_moe_fp8blk_preshuffle_bytes(int E, int N, int K, int mode, size_t* w_bytes);
-int hk_moe_fp8blk_preshuffle(const void* w, int E, int N, int K, int mode, void* out_w, void* stream);
-
-/* Expert MLP for routed and sorted tokens (outputs of hk_moe_topk_* and hk_moe_sort).
- * weight_layout 0: w13 / w2 plain as described above; 1: both pre-shuffled with
- * hk_moe_fp8blk_preshuffle (same results, bit for bit). */
+/* Expert MLP for routed and sorted tokens (outputs of hk_moe_topk_* and hk_moe_sort). */
 int hk_moe_fp8blk_experts(const void* x_e4m3, const float* x_scales, const void* w13,
                           const float* w13_scales, const void* w2, const float* w2_scales,
                           const float* topk_w, const int32_t* sorted_slots,
                           const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
-                          int T, int H, int I, int E, int k, int weight_layout, void* workspace,
-                          size_t workspace_bytes, void* stream);
+                          int T, int H, int I, int E, int k, void* workspace, size_t workspace_bytes,
+                          void* stream);
 
 /* Whole layer with group-limited sigmoid routing (see hk_moe_topk_grouped_sigmoid). */
 int hk_moe_fp8blk_forward(const void* x_e4m3, const float* x_scales, const float* router_logits,
                           const float* router_bias_or_null, int n_group, int topk_group,
                           float routed_scale, const void* w13, const float* w13_scales, const void* w2,
                           const float* w2_scales, void* y_bf16, int T, int H, int I, int E, int k,
-                          int weight_layout, void* workspace, size_t workspace_bytes, void* stream);
+                          void* workspace, size_t workspace_bytes, void* stream);
 
 /* Calibration probe (no counterpart in the reference): runs `blocks` workgroups of 8 waves, each
  * wave `iters` x 32 register-only 16x16x128 MFMAs (fp8 if fp4 == 0, else fp4) on operand bits
