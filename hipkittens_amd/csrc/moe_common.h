@@ -16,7 +16,8 @@ __device__ __forceinline__ int moe_b_row(int mode, int R, int n_tile, int N) {
     return (t & 1) * N + min(n_tile * 128 + hcol, N - 1);
 }
 
-// Work items. A work item is (m-tile, n-tile): up to kMoeBM consecutive sorted rows of one expert
+// Work items. A work item is (m-tile, n-tile): up to kMoeBM (weight-streaming MXFP4 kernel: 192)
+// consecutive sorted rows of one expert
 // times one tile of weight rows. Items are listed expert by expert, n-tile by n-tile, the m-tiles
 // of one (expert, n-tile) next to each other.
 constexpr int kMoeBM = 128;
@@ -25,9 +26,10 @@ struct MoeItem { int expert, row_start, rows, n_tile; };
 inline int moe_round_up(int x, int m) { return (x + m - 1) / m * m; }
 // Number of CUs of the current device (cached).
 int moe_num_compute_units();
-// Item lists of the two grouped GEMMs of a layer from expert_offsets [E+1]: items1 / num_items[0]
-// for n_tiles_n1 tiles of weight rows, items2 / num_items[1] for n_tiles_n2 (one launch).
-void moe_launch_build_items(const int32_t* expert_offsets, int E, int n_tiles_n1, MoeItem* items1,
+// Item lists of the two grouped GEMMs of a layer from expert_offsets [E+1], m-tiles of up to `bm`
+// rows: items1 / num_items[0] for n_tiles_n1 tiles of weight rows, items2 / num_items[1] for
+// n_tiles_n2 (one launch).
+void moe_launch_build_items(const int32_t* expert_offsets, int E, int bm, int n_tiles_n1, MoeItem* items1,
                             int n_tiles_n2, MoeItem* items2, int32_t* num_items, hipStream_t s);
 
 }  // namespace hk

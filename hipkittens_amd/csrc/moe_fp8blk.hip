@@ -412,7 +412,7 @@ extern "C" int hk_moe_fp8blk_experts(const void* x_e4m3, const float* x_scales, 
                            (const uint8_t*)x_e4m3, x_scales, sorted_slots, k, S, H, ws + L.xq, (float*)(ws + L.xs));
     }
     int32_t* nitems = (int32_t*)(ws + L.nitems);
-    moe_launch_build_items(expert_offsets, E, I / 128, (MoeItem*)(ws + L.items1), (H + 255) / 256,
+    moe_launch_build_items(expert_offsets, E, kMoeBM, I / 128, (MoeItem*)(ws + L.items1), (H + 255) / 256,
                            (MoeItem*)(ws + L.items2), nitems, s);
 
     MoeFp8Params p{};

@@ -135,15 +135,26 @@ __global__ __launch_bounds__(128) void mxfp4_quantize_permute_kernel(
 }
 
 // ---------------------------------------------------------------------- weight pre-shuffle
+// Tile row R (0..255) of n-tile `n_tile` in the pre-shuffled layout -> row of the expert's weight
+// matrix. Wave w of moe_mxfp4_stream_kernel owns tile rows [32 w, +32) = two MFMA fragments.
+// mode 0 (gate+up, N = I): fragment 0 holds the gate rows and fragment 1 the up rows of h columns
+// 128 n_tile + 16 w .. +16, in order; mode 1 (down, N = H): the b_row_to_col permutation, which
+// gives a lane 8 consecutive output columns from its two fragments. Rows past N repeat row N - 1.
+__device__ __forceinline__ int moe_stream_b_row(int mode, int R, int n_tile, int N) {
+    if (mode == 1) return min(n_tile * 256 + b_row_to_col(R), N - 1);
+    const int w = R >> 5, f = (R >> 4) & 1, r = R & 15;
+    return f * N + min(n_tile * 128 + 16 * w + r, N - 1);
+}
+
 // Pre-shuffled weight layout, made for moe_mxfp4_stream_kernel: weights go from HBM straight
 // into MFMA operand registers, so for every (expert, n-tile of 256 tile rows, K-step of 256
-// elements) one contiguous 32 KiB block holds, wave by wave (wave wn = tile rows [64 wn, +64)),
-// the wave's eight B fragments f = 2 * nfrag + half as 1 KiB pieces in lane order: lane l's 16
-// bytes are tile row 64 wn + 16 nfrag + l % 16 (moe_b_row gives the weight row), K bytes
+// elements) one contiguous 32 KiB block holds, wave by wave (wave w = tile rows [32 w, +32)),
+// the wave's four B fragments f = 2 * nfrag + half as 1 KiB pieces in lane order: lane l's 16
+// bytes are tile row 32 w + 16 nfrag + l % 16 (moe_stream_b_row gives the weight row), K bytes
 // 128 kt + 64 half + 16 (l / 16) .. +16, zero past the end of K. A second array holds the
-// scales the same way, 8 bytes per lane: byte 4 half + nfrag is the e8m0 scale of that row's
+// scales the same way, 4 bytes per lane: byte 2 half + nfrag is the e8m0 scale of that row's
 // 32-element block 8 kt + 4 half + l / 16 (127 past the end of K).
-//   out_w [E][n_tiles][nk][4][8][64][16] bytes, out_s [E][n_tiles][nk][4][64][8] bytes.
+//   out_w [E][n_tiles][nk][8][4][64][16] bytes, out_s [E][n_tiles][nk][8][64][4] bytes.
 __global__ __launch_bounds__(256) void moe_preshuffle_kernel(const uint8_t* __restrict__ w,
                                                              const uint8_t* __restrict__ sc, int E, int N,
                                                              int K, int scale_pitch, int mode, int n_tiles,
@@ -154,23 +165,23 @@ __global__ __launch_bounds__(256) void moe_preshuffle_kernel(const uint8_t* __re
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;  // one 16-byte chunk each
     const long long total = (long long)E * n_tiles * nk * 2048;
     if (gid >= total) return;
-    const int l = (int)(gid & 63), f = (int)((gid >> 6) & 7), wn = (int)((gid >> 9) & 3);
+    const int l = (int)(gid & 63), f = (int)((gid >> 6) & 3), wv = (int)((gid >> 8) & 7);
     long long rest = gid >> 11;
     const int kt = (int)(rest % nk); rest /= nk;
     const int nt = (int)(rest % n_tiles);
     const int e = (int)(rest / n_tiles);
-    const int row = moe_b_row(mode, 64 * wn + 16 * (f >> 1) + (l & 15), nt, N);
+    const int row = moe_stream_b_row(mode, 32 * wv + 16 * (f >> 1) + (l & 15), nt, N);
     const int kb = kt * 128 + 64 * (f & 1) + 16 * (l >> 4);
     v4i val = {0, 0, 0, 0};
     if (kb < Kb) val = *(const v4i*)(w + ((size_t)e * rows_b + row) * Kb + kb);
     *(v4i*)(out_w + gid * 16) = val;
     if (f == 0) {
-        // this thread also writes the lane's 8 scale bytes of the K-step
-        uint8_t* dst = out_s + ((gid >> 11) * 4 + wn) * 512 + l * 8;
+        // this thread also writes the lane's 4 scale bytes of the K-step
+        uint8_t* dst = out_s + ((gid >> 11) * 8 + wv) * 256 + l * 4;
 #pragma unroll
-        for (int b = 0; b < 8; ++b) {
-            const int rw = moe_b_row(mode, 64 * wn + 16 * (b & 3) + (l & 15), nt, N);
-            const int blk = kt * 8 + 4 * (b >> 2) + (l >> 4);
+        for (int b = 0; b < 4; ++b) {
+            const int rw = moe_stream_b_row(mode, 32 * wv + 16 * (b & 1) + (l & 15), nt, N);
+            const int blk = kt * 8 + 4 * (b >> 1) + (l >> 4);
             dst[b] = blk < (K >> 5) ? sc[((size_t)e * rows_b + rw) * scale_pitch + blk] : (uint8_t)127;
         }
     }
@@ -178,19 +189,19 @@ __global__ __launch_bounds__(256) void moe_preshuffle_kernel(const uint8_t* __re
 
 // Item lists of both grouped GEMMs of a layer in one launch: workgroup 0 builds the list for
 // n_tiles[0] tiles of weight rows into items[0], workgroup 1 the one for n_tiles[1].
-struct MoeBuildItems { MoeItem* items[2]; int n_tiles[2]; };
+struct MoeBuildItems { MoeItem* items[2]; int n_tiles[2]; int bm; };
 __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __restrict__ expert_offsets,
                                                               int E, MoeBuildItems b,
                                                               int32_t* __restrict__ num_items) {
     __shared__ int scan[512];
     const int which = blockIdx.x;
-    const int n_tiles_n = b.n_tiles[which];
+    const int n_tiles_n = b.n_tiles[which], bm = b.bm;
     MoeItem* __restrict__ items = b.items[which];
     const int e = threadIdx.x;
     int lo = 0, hi = 0, cnt = 0;
     if (e < E) {
         lo = expert_offsets[e]; hi = expert_offsets[e + 1];
-        cnt = (hi - lo + kMoeBM - 1) / kMoeBM;
+        cnt = (hi - lo + bm - 1) / bm;
     }
     scan[e] = cnt * n_tiles_n;
     __syncthreads();
@@ -204,7 +215,7 @@ __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __r
     for (int n = 0; n < n_tiles_n; ++n)
         for (int m = 0; m < cnt; ++m) {
             MoeItem it;
-            it.expert = e; it.row_start = lo + m * kMoeBM; it.rows = min(kMoeBM, hi - it.row_start); it.n_tile = n;
+            it.expert = e; it.row_start = lo + m * bm; it.rows = min(bm, hi - it.row_start); it.n_tile = n;
             items[base + n * cnt + m] = it;
         }
     if (e == 511) num_items[which] = scan[511];
@@ -531,27 +542,36 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
 }
 
 // ------------------------------------------------------- grouped GEMM, pre-shuffled weights
-// Weight-streaming variant for the pre-shuffled layout. At MoE shapes the grouped GEMMs are
+// Weight-streaming grouped GEMM for the pre-shuffled layout. At MoE shapes the grouped GEMMs are
 // bound by reading every expert's weights once from HBM, so the kernel is built around keeping
-// as many weight bytes in flight per CU as the register file allows:
+// as many weight bytes in flight per CU as possible and around reading them once:
 //   * weights never touch LDS: the pre-shuffled layout stores, for every (expert, n-tile, K-step,
-//     wave), the wave's eight MFMA B fragments as eight contiguous 1 KiB pieces (lane l's 16
-//     bytes at 16*l), and each wave loads them straight into registers two K-steps ahead of
-//     their use (a ring of four half-K-step register sets);
-//   * their e8m0 scales come the same way (8 bytes per lane and K-step);
-//   * only the activation tile (shared by the four waves, re-read from L2) goes through LDS, in
-//     a ring of four 17 KiB stages filled by direct global->LDS loads three K-steps ahead.
-// Workgroups have 4 waves, wave wn owning weight rows [64 wn, +64) of the 256-row tile and all
-// 128 activation rows; two workgroups share a CU (68 KiB of LDS and 256 registers per lane
-// each) and cover each other's barrier and issue stalls. The K-step stream runs across item
-// boundaries. Results are bit-identical to moe_mxfp4_gemm_kernel (same accumulation order).
-constexpr int kStStages = 4;
-constexpr int kStStage = kMoeATile + kMoeScaleA;   // 16 KiB tile + 1 KiB scales
-constexpr int kStLds = kStStages * kStStage;       // 68 KiB
+//     wave), the wave's four MFMA B fragments as four contiguous 1 KiB pieces (lane l's 16 bytes
+//     at 16*l), and each wave loads them straight into registers 3.5 K-steps ahead of their use
+//     (a ring of eight half-K-step register sets); their e8m0 scales come the same way;
+//   * a work item covers up to 192 rows of an expert (12 activation fragments), so that an expert
+//     with a few rows more than 128 still needs one pass over its weights;
+//   * only the activation tile (shared by the waves, re-read from L2) goes through LDS, in a ring
+//     of five 25.5 KiB stages filled by direct global->LDS loads four K-steps ahead. Loads return
+//     in order, so the activation tile has to be requested before the weights of the same K-step.
+// One workgroup of 8 waves per CU; wave w owns weight rows [32 w, +32) of the 256-row tile (two
+// fragments) x all rows of the item: 96 accumulator registers. The K-step stream runs across item
+// boundaries. All vector-memory operations are inline asm and counted by hand (the compiler
+// never waits for them): every use of loaded registers is preceded by a vmcnt wait and
+// `landed`, which makes the compiler see a new value there. Results are bit-identical to
+// moe_mxfp4_gemm_kernel (same accumulation order per output element).
+constexpr int kStBM = 192;                              // rows per work item
+constexpr int kStStages = 5;
+constexpr int kStATile = kStBM * 128;                   // 24 KiB
+constexpr int kStStage = kStATile + kStBM * 8;          // + 1.5 KiB of row scales
+constexpr int kStXch = kStStages * kStStage;            // epilogue: row maxima [kStBM][8 waves] floats
+constexpr int kStHTile = kStXch + kStBM * 8 * 4;        // epilogue: packed h tile [kStBM][64 bytes]
+constexpr int kStHScale = kStHTile + kStBM * 64;        // epilogue: h scales [kStBM][4 bytes]
+constexpr int kStLds = kStHScale + kStBM * 4;           // 146.25 KiB
 
 template <int MODE>
-__global__ __launch_bounds__(256, 2) void moe_mxfp4_stream_kernel(const MoeGemmParams p) {
-    constexpr int MT = kMoeBM / 16, NT = 4;
+__global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmParams p) {
+    constexpr int MT = kStBM / 16, NT = 2;
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
     const int lane = lane_id(), w = wave_id();
     const int n_items = scalar_load_x1(p.num_items);
@@ -584,30 +604,32 @@ __global__ __launch_bounds__(256, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
     // ---- activation tile: global -> LDS -------------------------------------------------------
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-    const uint32_t lds_sa_wave = to_sgpr(lds0 + kMoeATile + (uint32_t)w * 256u);
+    const uint32_t lds_sa_wave = to_sgpr(lds0 + kStATile + (uint32_t)w * 192u);
     const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);
-    uint32_t voff_a[4];
+    uint32_t voff_a[3];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) voff_a[i] = (uint32_t)(8 * (i * 4 + w) + (lane >> 3)) * 128u + chunk16 * 16u;
-    const uint32_t voff_sa = (uint32_t)(w * 256 + lane * 16);
-    // 5 loads: the wave's quarter of the tile (rows 8(4i + w) .. +8) and of its scales (32 rows)
+    for (int i = 0; i < 3; ++i) voff_a[i] = (uint32_t)(8 * (i * 8 + w) + (lane >> 3)) * 128u + chunk16 * 16u;
+    const uint32_t voff_sa = (uint32_t)(w * 192 + lane * 16);
+    // 4 loads: rows 8(8i + w) .. +8 of the tile for i = 0..2 (skipped, i.e. issued against an
+    // empty buffer, past the item's last fragment) and the row scales of rows [24 w, +24)
     auto issue_a = [&](const Cursor& c, int stage) __attribute__((always_inline)) {
-        v4i sa = srd_a, ssa = srd_sa;
-        if (!c.valid) { sa.z = 0; ssa.z = 0; }
+        v4i ssa = srd_sa;
+        if (!c.valid) ssa.z = 0;
+        const int rows_up = c.valid ? (c.rows + 15) & ~15 : 0;
         const uint32_t row_base = (uint32_t)c.kt * (uint32_t)p.S + (uint32_t)c.row_start;
         const uint32_t dst = lds_wave + (uint32_t)stage * kStStage;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(sa, dst + i * 4096, voff_a[i], row_base * 128u);
-        dma16_lanes(ssa, lds_sa_wave + (uint32_t)stage * kStStage, voff_sa, row_base * 8u, 0xffffull);
+        for (int i = 0; i < 3; ++i) {
+            v4i sa = srd_a;
+            if (8 * (i * 8 + w) >= rows_up) sa.z = 0;
+            dma16(sa, dst + i * 8192, voff_a[i], row_base * 128u);
+        }
+        dma16_lanes(ssa, lds_sa_wave + (uint32_t)stage * kStStage, voff_sa, row_base * 8u, 0xfffull);
     };
 
     // ---- weights: global -> registers -----------------------------------------------------------
     // pre-shuffled layout (moe_preshuffle_kernel): [expert][n-tile][K-step][wave][fragment][lane][16]
-    const int voff_b = lane * 16, voff_sb = lane * 8;  // scales: dword 0 first K half, dword 1 second
-    // The loads are inline asm: the compiler takes the registers as written at once and never
-    // waits for them itself; every use is preceded by one of the vmcnt waits below followed by
-    // `landed`, which makes the compiler see a new value there (so that nothing it derives from
-    // these registers can be placed before the wait).
+    const uint32_t voff_b = lane * 16, voff_sb = lane * 4;
     auto srd_b = [&](const Cursor& c) __attribute__((always_inline)) {
         return make_srd(p.B + (size_t)c.expert * p.b_expert_stride + (size_t)c.n_tile * nk * kMoeBTile,
                         c.valid ? (uint32_t)nk * kMoeBTile : 0u);
@@ -616,16 +638,11 @@ __global__ __launch_bounds__(256, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
         return make_srd(p.SB + (size_t)c.expert * p.sb_expert_stride + (size_t)c.n_tile * nk * kMoeScaleB,
                         c.valid ? (uint32_t)nk * kMoeScaleB : 0u);
     };
-    v4i bw[2][2][NT];  // [K-step parity][K half][fragment]
-    int bsc[2][2];     // [K-step parity][K half]: the lane's scale bytes of fragments 0..3
-    // 1 scale load + 4 fragment loads of one K half of the weight fetch position
-    auto load_b_half = [&](const Cursor& c, v4i (&dst)[NT], int& dst_scale, int half) __attribute__((always_inline)) {
-        const v4i rs = srd_b(c), rss = srd_sb(c);
-        const uint32_t soff = (uint32_t)c.kt * kMoeBTile + (uint32_t)w * 8192u + (uint32_t)half * 1024u;
-        asm volatile("buffer_load_dword %0, %1, %2, %3 offen"
-                     : "=v"(dst_scale)
-                     : "v"(voff_sb), "s"(rss), "s"((uint32_t)c.kt * kMoeScaleB + (uint32_t)w * 512u + (uint32_t)half * 4u)
-                     : "memory");
+    v4i bw[4][2][NT];  // [K-step mod 4][K half][fragment]
+    int bsc[4];        // [K-step mod 4]: the lane's scale bytes, byte 2 * half + fragment
+    auto load_b_half = [&](const Cursor& c, v4i (&dst)[NT], int half) __attribute__((always_inline)) {
+        const v4i rs = srd_b(c);
+        const uint32_t soff = (uint32_t)c.kt * kMoeBTile + (uint32_t)w * 4096u + (uint32_t)half * 1024u;
 #pragma unroll
         for (int n = 0; n < NT; ++n)
             asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"
@@ -633,16 +650,22 @@ __global__ __launch_bounds__(256, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
                          : "v"(voff_b), "s"(rs), "s"(soff + n * 2048u)
                          : "memory");
     };
-    auto landed = [&](v4i (&x)[NT], int& sc) __attribute__((always_inline)) {
+    auto load_b_scales = [&](const Cursor& c, int& dst) __attribute__((always_inline)) {
+        const v4i rss = srd_sb(c);
+        asm volatile("buffer_load_dword %0, %1, %2, %3 offen"
+                     : "=v"(dst)
+                     : "v"(voff_sb), "s"(rss), "s"((uint32_t)c.kt * kMoeScaleB + (uint32_t)w * 256u)
+                     : "memory");
+    };
+    auto landed = [&](v4i (&x)[NT]) __attribute__((always_inline)) {
 #pragma unroll
         for (int n = 0; n < NT; ++n) asm volatile("" : "+v"(x[n]));
-        asm volatile("" : "+v"(sc));
     };
 
     // ---- LDS -> registers (activation fragments) ------------------------------------------------
     const uint32_t r = lane & 15, g = lane >> 4;
     const uint32_t rd_half[2] = {lds0 + r * 128u + swz_chunk(r, g) * 16u, lds0 + r * 128u + swz_chunk(r, g + 4) * 16u};
-    const uint32_t sa_rd0 = lds0 + kMoeATile + r * 8u;
+    const uint32_t sa_rd0 = lds0 + kStATile + r * 8u;
     const uint32_t sh = 8u * g;  // byte g of each scale dword belongs to this lane
 
     v4f acc[MT][NT];
@@ -668,7 +691,7 @@ __global__ __launch_bounds__(256, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
         asm volatile("" : "+v"(a_rd), "+v"(sa_rd));  // keep the bases in registers, offsets as immediates
         int bs[NT];
 #pragma unroll
-        for (int n = 0; n < NT; ++n) bs[n] = (int)((uint32_t)bscale >> (8 * n));
+        for (int n = 0; n < NT; ++n) bs[n] = (int)((uint32_t)bscale >> (8 * (2 * half + n)));
         const int mt = (rows + 15) >> 4;
         v4i af[3];
         uint32_t as[3];
@@ -698,113 +721,142 @@ __global__ __launch_bounds__(256, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
 
     auto epilogue = [&](const Cursor& c) __attribute__((always_inline)) {
         const int rows = c.rows, row_start = c.row_start;
-        const int n0 = c.n_tile * (MODE == 0 ? 128 : 256);
         if (MODE == 1) {
+            // lane (r, g) holds, for row 16 m + r, the 8 consecutive columns 32 w + 8 g .. +8
             uint16_t* out = (uint16_t*)p.out0;
+            const int col = c.n_tile * 256 + w * 32 + 8 * (int)g;
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 const int row = 16 * m + (int)r;
-                if (row >= rows) continue;
-                const size_t pos = (size_t)(row_start + row);
-#pragma unroll
-                for (int q = 0; q < NT / 2; ++q) {
-                    const int col = n0 + w * 64 + 32 * q + 8 * (int)g;
-                    if (col + 8 > p.N) continue;  // N % 8 == 0
-                    const v4f x = acc[m][2 * q], y = acc[m][2 * q + 1];
-                    v4i o4;
-                    o4.x = pack_bf16(x.x, x.y); o4.y = pack_bf16(x.z, x.w);
-                    o4.z = pack_bf16(y.x, y.y); o4.w = pack_bf16(y.z, y.w);
-                    store_global_b128(out + pos * p.N + col, o4);
-                }
+                if (row >= rows || col + 8 > p.N) continue;  // N % 8 == 0
+                const v4f x = acc[m][0], y = acc[m][1];
+                v4i o4;
+                o4.x = pack_bf16(x.x, x.y); o4.y = pack_bf16(x.z, x.w);
+                o4.z = pack_bf16(y.x, y.y); o4.w = pack_bf16(y.z, y.w);
+                store_global_b128(out + (size_t)(row_start + row) * p.N + col, o4);
             }
         } else {
-            // see moe_mxfp4_gemm_kernel: this wave's 32 h columns are one MX block
-            uint8_t* hq = (uint8_t*)p.out0;
-            const int hcol0 = n0 + 32 * w;
-            const bool col_ok = hcol0 < p.N;
-            const size_t kt2 = (size_t)(hcol0 >> 8);
-            const int byte0 = ((hcol0 & 255) >> 1) + 4 * (int)g, blk = (hcol0 & 255) >> 5;
+            // h = silu(gate) * up: lane (r, g) holds, for row 16 m + r, the h columns
+            // 128 n_tile + 16 w + 4 g .. +4. An MX block of 32 columns spans waves 2u and 2u + 1:
+            // row maxima are exchanged through LDS, the packed tile (64 bytes per row) and its
+            // scales are assembled in LDS and leave with 16-byte stores.
+            typedef __attribute__((address_space(3))) float lds_f32_mut_t;
+            typedef __attribute__((address_space(3))) uint16_t lds_u16_mut_t;
+            typedef __attribute__((address_space(3))) uint8_t lds_u8_mut_t;
+            const int hcol0 = c.n_tile * 128 + 16 * w;  // first of the wave's 16 h columns
+            const bool col_ok = hcol0 < p.N;            // N % 32 == 0: a block is valid as a whole
+            // two groups of six fragments, to keep the number of live h values small
 #pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                const int row = 16 * m + (int)r;
-                if (16 * m >= rows) continue;  // uniform: the whole fragment is padding
-                float h[8];
+            for (int m0 = 0; m0 < MT; m0 += MT / 2) {
+                float h[MT / 2][4];
 #pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    const v4f gt = acc[m][2 * q], up = acc[m][2 * q + 1];
+                for (int mm = 0; mm < MT / 2; ++mm) {
+                    const int m = m0 + mm;
+                    if (16 * m >= rows) continue;  // uniform: the whole fragment is padding
+                    const v4f gt = acc[m][0], up = acc[m][1];
+                    float amax = 0.f;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const float gv = gt[j];
-                        h[4 * q + j] = silu_mul(gv, up[j]);
+                        h[mm][j] = col_ok ? silu_mul(gt[j], up[j]) : 0.f;
+                        amax = fmaxf(amax, fabsf(h[mm][j]));
                     }
+                    amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+                    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+                    if (g == 0) *(lds_f32_mut_t*)(uintptr_t)(lds0 + kStXch + ((16 * m + r) * 8 + w) * 4) = amax;
                 }
-                float amax = 0.f;
+                __syncthreads();
 #pragma unroll
-                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(h[i]));
-                amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-                const int e = mx_block_exponent(amax);
-                if (row < rows && col_ok) {
-                    const size_t tile_row = kt2 * p.S + (size_t)(row_start + row);
-                    store_global_b32(hq + tile_row * 128 + byte0, pack8_e2m1(h, e));
-                    if (g == 0) store_global_b8(p.out_scales + tile_row * 8 + blk, (uint32_t)(e + 127));
+                for (int mm = 0; mm < MT / 2; ++mm) {
+                    const int m = m0 + mm;
+                    if (16 * m >= rows) continue;
+                    const uint32_t row = 16 * m + r;
+                    const v2f am = *(__attribute__((address_space(3))) const v2f*)(uintptr_t)(lds0 + kStXch + (row * 8 + (w & ~1)) * 4);
+                    const int e = mx_block_exponent(fmaxf(am.x, am.y));
+                    const float scale = __uint_as_float(e > -127 ? (uint32_t)(e + 127) << 23 : 0x00400000u);
+                    uint32_t pk = 0;
+                    pk = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(pk, h[mm][0], h[mm][1], scale, 0);
+                    pk = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(pk, h[mm][2], h[mm][3], scale, 1);
+                    *(lds_u16_mut_t*)(uintptr_t)(lds0 + kStHTile + row * 64 + 8 * w + 2 * g) = (uint16_t)pk;
+                    if (g == 0 && (w & 1) == 0)
+                        *(lds_u8_mut_t*)(uintptr_t)(lds0 + kStHScale + row * 4 + (w >> 1)) = col_ok ? (uint8_t)(e + 127) : (uint8_t)127;
                 }
+            }
+            __syncthreads();
+            uint8_t* hq = (uint8_t*)p.out0;
+            const size_t kt2 = (size_t)(c.n_tile >> 1);
+            const int seg = (c.n_tile & 1) * 64;  // the n-tile's 128 columns are half of a K-step row
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const int chunk = (int)threadIdx.x + 512 * q;  // 16-byte chunk of the [kStBM][64] tile
+                const int row = chunk >> 2, part = chunk & 3;
+                if (row < rows) {
+                    const v4i v = *(lds_v4i_t*)(uintptr_t)(lds0 + kStHTile + chunk * 16);
+                    store_global_b128(hq + (kt2 * p.S + (size_t)(row_start + row)) * 128 + seg + part * 16, v);
+                }
+            }
+            if ((int)threadIdx.x < rows) {
+                const uint32_t v = *(__attribute__((address_space(3))) const uint32_t*)(uintptr_t)(lds0 + kStHScale + threadIdx.x * 4);
+                store_global_b32(p.out_scales + (kt2 * p.S + (size_t)(row_start + threadIdx.x)) * 8 + (seg >> 4), v);
             }
         }
     };
 
-    // ---- prologue: positions 0..2 of the activation ring, positions 0 and 1 of the weights,
-    // in the order the K loop issues them (5 activation loads between two weight sets), so that
-    // the same load counts hold from the first position on
-    issue_a(ca, 0); advance(ca);
-    issue_a(ca, 1); advance(ca);
-    load_b_half(cb, bw[0][0], bsc[0][0], 0); load_b_half(cb, bw[0][1], bsc[0][1], 1); advance(cb);
-    issue_a(ca, 2); advance(ca);
-    load_b_half(cb, bw[1][0], bsc[1][0], 0); load_b_half(cb, bw[1][1], bsc[1][1], 1); advance(cb);
+    // ---- prologue: activation positions 0..3 and weight positions 0..3, in the order the K loop
+    // issues them (4 activation loads, then 2 + 3 weight loads per position)
+    auto load_b_set = [&]<int P>() __attribute__((always_inline)) {
+        load_b_half(cb, bw[P][0], 0);
+        load_b_scales(cb, bsc[P]);
+        load_b_half(cb, bw[P][1], 1);
+        advance(cb);
+    };
+    issue_a(ca, 0); advance(ca); load_b_set.template operator()<0>();
+    issue_a(ca, 1); advance(ca); load_b_set.template operator()<1>();
+    issue_a(ca, 2); advance(ca); load_b_set.template operator()<2>();
+    issue_a(ca, 3); advance(ca); load_b_set.template operator()<3>();
     zero_acc();
 
-    // One stream position with register-set parity P on LDS stage st. In program order a wave
-    // issues per position: 5 activation loads (position +3), then after each K half 1 scale load
-    // + 4 weight loads (position +2) into the registers that half's MFMAs have just finished
-    // with. Loads return in order, so counting the loads issued after the ones needed gives:
-    //   first K half:  its weights were followed by 5 (second half) + 15 (previous position)  -> vmcnt(20)
-    //   second K half: by 15 (previous position) + 5 + 5 (this position so far)                -> vmcnt(25)
-    // and the activation tile of the position is older than both. Stores share the counter and
-    // complete out of order, so behind an epilogue's stores those counts would wait for far more
-    // than needed: the position that ends an item first waits until everything the next position
-    // needs has landed (all but the 15 loads it issued itself), then stores, and the next
-    // position runs without waiting.
-    bool after_stores = false;
+    // One stream position on LDS stage st with register set P. In program order a wave issues per
+    // position 9 loads: 4 activation loads (position +4), after the first K half 2 weight loads,
+    // after the second one 1 scale load + 2 weight loads (position +4, into the registers the
+    // MFMAs before them have just finished with). Loads return in order, so counting the loads
+    // issued after the ones needed gives the waits:
+    //   first K half:  scales and weights are followed by 2 + 27 (three positions)   -> vmcnt(29)
+    //   second K half: by 27 + 4 + 2 (this position so far)                          -> vmcnt(33)
+    // and the position's activation tile is older than both. Stores share the counter and
+    // complete out of order, which only makes these waits stricter.
     auto step = [&]<int P>(int st) __attribute__((always_inline)) {
-        const bool last = cc.valid && cc.kt == nk - 1;
-        if (!after_stores) wait_vmcnt<20>();
+        wait_vmcnt<29>();
         block_barrier();  // everyone's part of this position's tile has landed; stage st-1 is free
-        issue_a(ca, (st + 3) & 3); advance(ca);
-        landed(bw[P][0], bsc[P][0]);
+        issue_a(ca, st == 0 ? kStStages - 1 : st - 1); advance(ca);
+        landed(bw[P][0]);
+        asm volatile("" : "+v"(bsc[P]));
+        const int sc = bsc[P];
         const int rows = cc.valid ? cc.rows : 0;  // past the end of the stream: no MFMAs, empty loads
-        compute_half(st, 0, rows, bw[P][0], bsc[P][0]);
-        load_b_half(cb, bw[P][0], bsc[P][0], 0);
-        if (!after_stores) wait_vmcnt<25>();
-        landed(bw[P][1], bsc[P][1]);
-        compute_half(st, 1, rows, bw[P][1], bsc[P][1]);
-        load_b_half(cb, bw[P][1], bsc[P][1], 1);
+        compute_half(st, 0, rows, bw[P][0], sc);
+        load_b_half(cb, bw[P][0], 0);
+        wait_vmcnt<33>();
+        landed(bw[P][1]);
+        compute_half(st, 1, rows, bw[P][1], sc);
+        load_b_scales(cb, bsc[P]);
+        load_b_half(cb, bw[P][1], 1);
         advance(cb);
-        if (last) {
-            wait_vmcnt<15>();
+        if (cc.valid && cc.kt == nk - 1) {
             mfma_drain();
             epilogue(cc);
             zero_acc();
         }
-        after_stores = last;
         advance(cc);
     };
-    // Two positions per trip (the register sets alternate); the second one may lie past the end
-    // of the stream, where it degenerates to its barrier and empty loads. No exit between the
-    // two: a second way into the loop head would make the compiler merge two load histories
-    // and wait for the more recent one.
-    for (int st = 0; cc.valid; st ^= 2) {
-        step.template operator()<0>(st);
-        step.template operator()<1>(st + 1);
+    // Four positions per trip (the register sets rotate); positions past the end of the stream
+    // degenerate to their barrier and empty loads. No exit inside a trip: a second way into the
+    // loop head would hand the compiler two load histories to merge.
+    int st = 0;
+    auto next_stage = [&]() __attribute__((always_inline)) { st = st == kStStages - 1 ? 0 : st + 1; };
+    while (cc.valid) {
+        step.template operator()<0>(st); next_stage();
+        step.template operator()<1>(st); next_stage();
+        step.template operator()<2>(st); next_stage();
+        step.template operator()<3>(st); next_stage();
     }
     wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
 }
@@ -848,9 +900,10 @@ int moe_num_compute_units() {
     return cus;
 }
 
-void moe_launch_build_items(const int32_t* expert_offsets, int E, int n_tiles_n1, MoeItem* items1,
+void moe_launch_build_items(const int32_t* expert_offsets, int E, int bm, int n_tiles_n1, MoeItem* items1,
                             int n_tiles_n2, MoeItem* items2, int32_t* num_items, hipStream_t s) {
     MoeBuildItems b;
+    b.bm = bm;
     b.items[0] = items1; b.items[1] = items2;
     b.n_tiles[0] = n_tiles_n1; b.n_tiles[1] = n_tiles_n2;
     hipLaunchKernelGGL(moe_build_items_kernel, dim3(2), dim3(512), 0, s, expert_offsets, E, b, num_items);
@@ -866,9 +919,9 @@ static int launch_moe_stream(MoeGemmParams p, int max_items, hipStream_t s) {
             return HK_ERR_LAUNCH;
         configured = true;
     }
-    // persistent: two workgroups per CU, each walking its share of the item list
-    const int grid = min(max_items, 2 * moe_num_compute_units());
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), kStLds, s, p);
+    // persistent: one workgroup per CU, each walking its share of the item list
+    const int grid = min(max_items, moe_num_compute_units());
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kStLds, s, p);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
@@ -1014,7 +1067,8 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
                            ws + L.hs, I);
     }
     int32_t* nitems = (int32_t*)(ws + L.nitems);
-    moe_launch_build_items(expert_offsets, E, (I + 127) / 128, (MoeItem*)(ws + L.items1), (H + 255) / 256,
+    moe_launch_build_items(expert_offsets, E, weight_layout ? kStBM : kMoeBM, (I + 127) / 128,
+                           (MoeItem*)(ws + L.items1), (H + 255) / 256,
                            (MoeItem*)(ws + L.items2), nitems, s);
 
     MoeGemmParams p{};
