@@ -5,14 +5,14 @@
 // interleaved FP8/MXFP4 kernels of this library (LDS-direct loads into swizzled 128-byte-row
 // tiles, ds_read_b128 fragments, v_mfma_scale_f32_16x16x128_f8f6f4 with in-MFMA e8m0 scales).
 //
-// Grouped GEMM: a work item is (m-tile, n-tile) where an m-tile is up to 128 consecutive rows
+// Grouped GEMM: a work item is (m-tile, n-tile) where an m-tile is a run of consecutive rows
 // (sorted positions) of one expert; the item list is built on the device from expert_offsets.
-// A workgroup (8 waves, two per SIMD) computes a 128 x 256 tile per item. Weights dominate HBM
-// traffic, so workgroups are persistent and the LDS ring (three stages, two K-steps of operands
-// in flight) keeps running across item boundaries: the next item's first K-steps load while
-// the current item's epilogue runs. Items that share an expert run at the same time on the CUs
-// of one XCD, so activation tiles, and the weight tile needed again by an expert's second
-// m-tile, come out of that XCD's L2 and every weight byte leaves HBM once.
+// Weights dominate HBM traffic, so workgroups are persistent (one per CU) and keep their operand
+// pipelines running across item boundaries. Items that share an expert run at the same time on
+// the CUs of one XCD, so activation tiles come out of that XCD's L2 and every weight byte leaves
+// HBM once. Two kernels: moe_mxfp4_stream_kernel for weights in the pre-shuffled layout (the fast
+// path: weights go straight from HBM into MFMA operand registers, 192-row m-tiles) and
+// moe_mxfp4_gemm_kernel for the plain layout (both operands through an LDS ring, 128-row m-tiles).
 #include "moe_common.h"
 #include "../../include/hk355.h"
 
@@ -237,7 +237,6 @@ struct MoeGemmParams {
     int K;                   // contraction length in elements
     int N;                   // MODE 0: I (h columns; weight rows i and I+i); MODE 1: output columns
     int n_tiles_n;
-    int shuffled;            // 1: B / SB are in the pre-shuffled tile layout (see moe_preshuffle_kernel)
 };
 
 constexpr int kMoeATile = kMoeBM * 128;                 // 16 KiB
@@ -252,7 +251,7 @@ constexpr int kMoeLds = kMoeScaleBase + kMoeStages * kMoeScaleStage;  // 153 KiB
 // Global->LDS source offsets of one work item.
 struct MoeAddr {
     v4i srd_b, srd_sb;
-    uint32_t voff_b[4], voff_sb;  // pre-shuffled weights use voff_b[0] only
+    uint32_t voff_b[4], voff_sb;
     int row_start, rows, n0, n_tile;
     bool valid;
 };
@@ -264,7 +263,7 @@ struct MoeAddr {
 // because the two waves of a SIMD cover for each other: while one is held up issuing loads or
 // waiting for LDS, the other feeds the matrix pipe (a single wave per SIMD cannot issue the
 // 16-cycle FP4 MFMA back to back, nor issue loads and MFMAs at the same time).
-template <int MODE, bool SHUF>
+template <int MODE>
 __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams p) {
     constexpr int NW = 8, MT = kMoeBM / 32, NT = 4;   // MT fragments of 16 rows per wave
     constexpr int NA = kMoeBM / 64;                  // A-tile loads per wave and K-step
@@ -289,9 +288,7 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
     const int tail_bytes = Kb - (nk - 1) * 128;  // valid bytes of the last K-step (16..128)
     const int rows_b = MODE == 0 ? 2 * p.N : p.N;
     // loads per wave and K-step: A tile, B tile, A scales, B scales
-    // (with pre-shuffled weights each wave loads one scale piece: waves 0-3 a quarter of the
-    // B scales, waves 4-7 a quarter of the A scales)
-    constexpr int kDma = NA + 4 + (SHUF ? 1 : 2);
+    constexpr int kDma = NA + 4 + 2;
     const v4i srd_a = make_srd(p.A, (uint32_t)nk * (uint32_t)p.S * 128u);
     const v4i srd_sa = make_srd(p.SA, (uint32_t)nk * (uint32_t)p.S * 8u);
 
@@ -309,32 +306,21 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
         a.rows = item.z;
         a.n_tile = item.w;
         a.n0 = a.n_tile * (MODE == 0 ? 128 : 256);
-        if (SHUF) {
-            // one contiguous run of nk tiles per (expert, n-tile)
-            a.srd_b = make_srd(p.B + (size_t)expert * p.b_expert_stride + (size_t)a.n_tile * nk * kMoeBTile,
-                               (uint32_t)nk * kMoeBTile);
-            a.srd_sb = make_srd(p.SB + (size_t)expert * p.sb_expert_stride + (size_t)a.n_tile * nk * kMoeScaleB,
-                                (uint32_t)nk * kMoeScaleB);
-        } else {
-            a.srd_b = make_srd(p.B + (size_t)expert * p.b_expert_stride, (uint32_t)rows_b * (uint32_t)p.b_pitch);
-            a.srd_sb = make_srd(p.SB + (size_t)expert * p.sb_expert_stride, (uint32_t)rows_b * (uint32_t)p.sb_pitch);
-        }
+        a.srd_b = make_srd(p.B + (size_t)expert * p.b_expert_stride, (uint32_t)rows_b * (uint32_t)p.b_pitch);
+        a.srd_sb = make_srd(p.SB + (size_t)expert * p.sb_expert_stride, (uint32_t)rows_b * (uint32_t)p.sb_pitch);
         auto b_row = [&](int R) -> int { return moe_b_row(MODE, R, a.n_tile, p.N); };
 #pragma unroll
-        for (int i = 0; i < (SHUF ? 1 : 4); ++i)
-            a.voff_b[i] = SHUF ? (uint32_t)(w * 1024 + lane * 16)
-                               : (uint32_t)b_row(8 * (i * NW + w) + (lane >> 3)) * (uint32_t)p.b_pitch + chunk16 * 16u;
-        a.voff_sb = SHUF ? (uint32_t)((w & 3) * 512 + lane * 16)
-                         : (uint32_t)b_row(32 * w + (lane >> 1)) * (uint32_t)p.sb_pitch + (lane & 1) * 4u;
+        for (int i = 0; i < 4; ++i)
+            a.voff_b[i] = (uint32_t)b_row(8 * (i * NW + w) + (lane >> 3)) * (uint32_t)p.b_pitch + chunk16 * 16u;
+        a.voff_sb = (uint32_t)b_row(32 * w + (lane >> 1)) * (uint32_t)p.sb_pitch + (lane & 1) * 4u;
     };
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-    // scale pieces per wave: plain weights - A scales of kMoeBM/8 rows and B scales of 32 rows for
-    // every wave; pre-shuffled - B scales of 64 rows (waves 0-3) or A scales of kMoeBM/4 rows (4-7)
-    const uint32_t sa_bytes = SHUF ? kMoeBM * 2 : kMoeBM;  // A-scale bytes per loading wave
-    const uint32_t lds_sa_wave = to_sgpr(lds0 + kMoeScaleBase + (uint32_t)(SHUF ? (w & 3) : w) * sa_bytes);
-    const uint32_t lds_sb_wave = to_sgpr(lds0 + kMoeScaleBase + kMoeScaleA + (uint32_t)(SHUF ? (w & 3) * 512 : w * 256));
+    // scale pieces per wave: A scales of kMoeBM/8 rows and B scales of 32 rows
+    const uint32_t sa_bytes = kMoeBM;  // A-scale bytes per loading wave
+    const uint32_t lds_sa_wave = to_sgpr(lds0 + kMoeScaleBase + (uint32_t)w * sa_bytes);
+    const uint32_t lds_sb_wave = to_sgpr(lds0 + kMoeScaleBase + kMoeScaleA + (uint32_t)(w * 256));
 
     // A-side offsets do not depend on the work item: LDS row R of the A tile is row
     // row_start + R of the K-step's contiguous [S][128] block (rows past the tile's count are
@@ -343,8 +329,8 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
 #pragma unroll
     for (int i = 0; i < NA; ++i) voff_a[i] = (uint32_t)(8 * (i * NW + w) + (lane >> 3)) * 128u + chunk16 * 16u;
     // scales of kMoeBM / 8 rows per wave: kMoeBM / 16 lanes x 16 bytes
-    const uint32_t voff_sa = (uint32_t)((SHUF ? (w & 3) : w) * sa_bytes + lane * 16);
-    constexpr uint64_t kSaMask = (1ull << ((SHUF ? kMoeBM * 2 : kMoeBM) / 16)) - 1ull;
+    const uint32_t voff_sa = (uint32_t)(w * sa_bytes + lane * 16);
+    constexpr uint64_t kSaMask = (1ull << (kMoeBM / 16)) - 1ull;
 
     // All loads of K-step kt of item `a` into `stage`. For an invalid item or past the end of K
     // they are issued against zero-sized buffers (no traffic), which keeps the number of
@@ -358,23 +344,12 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
         const uint32_t sbdst = lds_sb_wave + (uint32_t)stage * kMoeScaleStage;
 #pragma unroll
         for (int i = 0; i < NA; ++i) dma16(sa, dst + i * NW * 1024, voff_a[i], row_base * 128u);
-        if (SHUF) {
+        const bool last = (kt == nk - 1) && tail_oob;  // 16-byte chunks past the end of K read as zero
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                dma16(sb, dst + kMoeATile + i * NW * 1024, a.voff_b[0], (uint32_t)kt * kMoeBTile + i * NW * 1024);
-        } else {
-            const bool last = (kt == nk - 1) && tail_oob;  // 16-byte chunks past the end of K read as zero
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                dma16(sb, dst + kMoeATile + i * NW * 1024, last ? 0x80000000u : a.voff_b[i], (uint32_t)kt * 128u);
-        }
-        if (SHUF) {
-            if (w < 4) dma16_lanes(ssb, sbdst, a.voff_sb, (uint32_t)kt * kMoeScaleB, 0xffffffffull);
-            else dma16_lanes(ssa, sadst, voff_sa, row_base * 8u, kSaMask);
-        } else {
-            dma16_lanes(ssa, sadst, voff_sa, row_base * 8u, kSaMask);
-            dma4(ssb, sbdst, a.voff_sb, (uint32_t)kt * 8u);
-        }
+        for (int i = 0; i < 4; ++i)
+            dma16(sb, dst + kMoeATile + i * NW * 1024, last ? 0x80000000u : a.voff_b[i], (uint32_t)kt * 128u);
+        dma16_lanes(ssa, sadst, voff_sa, row_base * 8u, kSaMask);
+        dma4(ssb, sbdst, a.voff_sb, (uint32_t)kt * 8u);
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
@@ -925,9 +900,9 @@ static int launch_moe_stream(MoeGemmParams p, int max_items, hipStream_t s) {
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
-template <int MODE, bool SHUF>
+template <int MODE>
 static int launch_moe_gemm(MoeGemmParams p, int max_items, hipStream_t s) {
-    auto kern = moe_mxfp4_gemm_kernel<MODE, SHUF>;
+    auto kern = moe_mxfp4_gemm_kernel<MODE>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMoeLds) !=
@@ -1080,11 +1055,10 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
         const long long tiles = (long long)((I + 127) / 128) * ((H / 2 + 127) / 128);
         p.b_expert_stride = tiles * kMoeBTile; p.sb_expert_stride = tiles * kMoeScaleB;
     }
-    p.shuffled = weight_layout;
     p.items = (const MoeItem*)(ws + L.items1); p.num_items = nitems;
     p.out0 = ws + L.hq; p.out_scales = ws + L.hs;
     p.K = H; p.N = I; p.n_tiles_n = (I + 127) / 128;
-    st = weight_layout ? launch_moe_stream<0>(p, L.max_items1, s) : launch_moe_gemm<0, false>(p, L.max_items1, s);
+    st = weight_layout ? launch_moe_stream<0>(p, L.max_items1, s) : launch_moe_gemm<0>(p, L.max_items1, s);
     if (st != HK_OK) return st;
 
     MoeGemmParams q{};
@@ -1096,11 +1070,10 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
         const long long tiles = (long long)((H + 255) / 256) * ((I / 2 + 127) / 128);
         q.b_expert_stride = tiles * kMoeBTile; q.sb_expert_stride = tiles * kMoeScaleB;
     }
-    q.shuffled = weight_layout;
     q.items = (const MoeItem*)(ws + L.items2); q.num_items = nitems + 1;
     q.out0 = ws + L.o; q.out_scales = nullptr;
     q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
-    st = weight_layout ? launch_moe_stream<1>(q, L.max_items2, s) : launch_moe_gemm<1, false>(q, L.max_items2, s);
+    st = weight_layout ? launch_moe_stream<1>(q, L.max_items2, s) : launch_moe_gemm<1>(q, L.max_items2, s);
     if (st != HK_OK) return st;
 
     return hk_moe_unpermute(ws + L.o, topk_w, slot_to_pos, T, k, H, y_bf16, stream);
