@@ -575,6 +575,18 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
     Cursor cc{it0, 0}, ca{it0, 0}, cb{it0, 0};  // compute, activation fetch, weight fetch
     load_item(cc);
     ca = cc; cb = cc;
+    // buffer descriptors of the weight fetch position's item, rebuilt only when the item changes
+    v4i cb_srd_b, cb_srd_sb;
+    auto cb_descriptors = [&]() __attribute__((always_inline)) {
+        cb_srd_b = make_srd(p.B + (size_t)cb.expert * p.b_expert_stride + (size_t)cb.n_tile * nk * kMoeBTile,
+                            cb.valid ? (uint32_t)nk * kMoeBTile : 0u);
+        cb_srd_sb = make_srd(p.SB + (size_t)cb.expert * p.sb_expert_stride + (size_t)cb.n_tile * nk * kMoeScaleB,
+                             cb.valid ? (uint32_t)nk * kMoeScaleB : 0u);
+    };
+    cb_descriptors();
+    auto advance_cb = [&]() __attribute__((always_inline)) {
+        if (++cb.kt == nk) { cb.kt = 0; cb.it += it_stride; load_item(cb); cb_descriptors(); }
+    };
 
     // ---- activation tile: global -> LDS -------------------------------------------------------
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
@@ -605,18 +617,10 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
     // ---- weights: global -> registers -----------------------------------------------------------
     // pre-shuffled layout (moe_preshuffle_kernel): [expert][n-tile][K-step][wave][fragment][lane][16]
     const uint32_t voff_b = lane * 16, voff_sb = lane * 4;
-    auto srd_b = [&](const Cursor& c) __attribute__((always_inline)) {
-        return make_srd(p.B + (size_t)c.expert * p.b_expert_stride + (size_t)c.n_tile * nk * kMoeBTile,
-                        c.valid ? (uint32_t)nk * kMoeBTile : 0u);
-    };
-    auto srd_sb = [&](const Cursor& c) __attribute__((always_inline)) {
-        return make_srd(p.SB + (size_t)c.expert * p.sb_expert_stride + (size_t)c.n_tile * nk * kMoeScaleB,
-                        c.valid ? (uint32_t)nk * kMoeScaleB : 0u);
-    };
     v4i bw[4][2][NT];  // [K-step mod 4][K half][fragment]
     int bsc[4];        // [K-step mod 4]: the lane's scale bytes, byte 2 * half + fragment
     auto load_b_half = [&](const Cursor& c, v4i (&dst)[NT], int half) __attribute__((always_inline)) {
-        const v4i rs = srd_b(c);
+        const v4i rs = cb_srd_b;
         const uint32_t soff = (uint32_t)c.kt * kMoeBTile + (uint32_t)w * 4096u + (uint32_t)half * 1024u;
 #pragma unroll
         for (int n = 0; n < NT; ++n)
@@ -626,7 +630,7 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
                          : "memory");
     };
     auto load_b_scales = [&](const Cursor& c, int& dst) __attribute__((always_inline)) {
-        const v4i rss = srd_sb(c);
+        const v4i rss = cb_srd_sb;
         asm volatile("buffer_load_dword %0, %1, %2, %3 offen"
                      : "=v"(dst)
                      : "v"(voff_sb), "s"(rss), "s"((uint32_t)c.kt * kMoeScaleB + (uint32_t)w * 256u)
@@ -782,7 +786,7 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
         load_b_half(cb, bw[P][0], 0);
         load_b_scales(cb, bsc[P]);
         load_b_half(cb, bw[P][1], 1);
-        advance(cb);
+        advance_cb();
     };
     issue_a(ca, 0); advance(ca); load_b_set.template operator()<0>();
     issue_a(ca, 1); advance(ca); load_b_set.template operator()<1>();
@@ -814,7 +818,7 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
         compute_half(st, 1, rows, bw[P][1], sc);
         load_b_scales(cb, bsc[P]);
         load_b_half(cb, bw[P][1], 1);
-        advance(cb);
+        advance_cb();
         if (cc.valid && cc.kt == nk - 1) {
             mfma_drain();
             epilogue(cc);
