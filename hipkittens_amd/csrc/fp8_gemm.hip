@@ -451,6 +451,99 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
     store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
 }
 
+// ---------------------------------------------------------------------------------------
+// 128x128-tile kernel for problems with too few 256x256 tiles to occupy the chip (a 1024^3
+// GEMM has 16 of them for 256 CUs): 4 waves, each a 64x64 patch (16 MFMA tiles), three LDS
+// stages of 2 x 16 KiB with two K-steps of loads in flight, plain loop (such problems are
+// bound by launch, prologue and epilogue latency, not by the K loop's schedule). Same tile
+// format, B-row permutation and epilogue as the large-tile kernels.
+constexpr int kSmallTile = 128;
+constexpr int kSmallTileBytes = kSmallTile * BK;          // 16 KiB per operand
+constexpr int kSmallStageBytes = 2 * kSmallTileBytes;
+constexpr int kSmallStages = 3;
+constexpr int kSmallLdsBytes = kSmallStages * kSmallStageBytes;  // 96 KiB
+
+template <bool EDGE>
+__global__ __launch_bounds__(256) void fp8_gemm_tile128_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n) {
+    constexpr int NW = 4, TM = 64, TN = 64, MT = 4, NT = 4;
+    constexpr int NDMA = kSmallTileBytes / (NW * 1024);  // 4 loads per wave per operand per K-step
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    const int lane = lane_id(), w = wave_id();
+    const int wm = w >> 1, wn = w & 1;
+
+    int pm, pn;
+    {
+        const int id = xcd_chunk_order(blockIdx.x, tiles_m * tiles_n, kCuPerXcd);
+        grouped_raster(id, tiles_m, tiles_n, 8, pm, pn);
+    }
+    const int row0 = pm * kSmallTile, col0 = pn * kSmallTile;
+    const int a_rows = min(M - row0, kSmallTile), b_rows = min(N - col0, kSmallTile);
+    const v4i srd_a = make_srd(A + (size_t)row0 * K, (uint32_t)a_rows * (uint32_t)K);
+    const v4i srd_b = make_srd(B + (size_t)col0 * K, (uint32_t)b_rows * (uint32_t)K);
+
+    uint32_t voff_a[NDMA], voff_b[NDMA];
+#pragma unroll
+    for (int i = 0; i < NDMA; ++i) {
+        const int R = 8 * (i * NW + w) + (lane >> 3);
+        const uint32_t c = swz_chunk(R, lane & 7);
+        int ra = R, rb = b_row_to_col(R);
+        if (EDGE) {
+            ra = min(ra, a_rows - 1);
+            rb = min(rb, b_rows - 1);
+        }
+        voff_a[i] = (uint32_t)ra * (uint32_t)K + c * 16u;
+        voff_b[i] = (uint32_t)rb * (uint32_t)K + c * 16u;
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+    const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
+    auto issue_tile = [&](int stage, int kt) {
+        const uint32_t k0 = (uint32_t)kt * BK;
+        const uint32_t dst = lds_wave + (uint32_t)stage * kSmallStageBytes;
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) dma16(srd_a, dst + i * NW * 1024, voff_a[i], k0);
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) dma16(srd_b, dst + kSmallTileBytes + i * NW * 1024, voff_b[i], k0);
+    };
+
+    const uint32_t r = lane & 15, g = lane >> 4;
+    const uint32_t rd_lo = r * 128u + swz_chunk(r, g) * 16u;
+    const uint32_t rd_hi = r * 128u + swz_chunk(r, g + 4) * 16u;
+    const uint32_t a_lo0 = lds0 + wm * (TM * BK) + rd_lo, a_hi0 = lds0 + wm * (TM * BK) + rd_hi;
+    const uint32_t b_lo0 = lds0 + kSmallTileBytes + wn * (TN * BK) + rd_lo;
+    const uint32_t b_hi0 = lds0 + kSmallTileBytes + wn * (TN * BK) + rd_hi;
+
+    v4f acc[MT][NT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    const int nk = K / BK;
+    issue_tile(0, 0);
+    if (nk > 1) issue_tile(1, 1);
+    int st = 0;
+    for (int kt = 0; kt < nk; ++kt) {
+        // this wave's part of K-step kt has landed (the loads of K-step kt + 1 may still fly)
+        if (kt + 1 < nk) wait_vmcnt<2 * NDMA>(); else wait_vmcnt<0>();
+        block_barrier();  // ... everyone's; and everyone is done with the stage of K-step kt - 1
+        if (kt + 2 < nk) issue_tile(st == 0 ? 2 : st - 1, kt + 2);
+        const uint32_t so = (uint32_t)st * kSmallStageBytes;
+        v8i bf[NT];
+#pragma unroll
+        for (int n = 0; n < NT; ++n) bf[n] = lds_frag(b_lo0 + so, b_hi0 + so, n * 16 * BK);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const v8i af = lds_frag(a_lo0 + so, a_hi0 + so, m * 16 * BK);
+#pragma unroll
+            for (int n = 0; n < NT; ++n) acc[m][n] = mfma_fp8_16x16x128(bf[n], af, acc[m][n]);
+        }
+        st = st == 2 ? 0 : st + 1;
+    }
+    store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
+}
+
 // Portable kernel for any M, N and K % 16 == 0: 4 waves, each a 32x32 patch of a 64x64
 // tile, operands fetched straight from global memory into MFMA fragments with
 // per-lane masking (rows past the edge and 16-byte chunks past K read as zero).
@@ -524,6 +617,24 @@ static int launch_tile(const void* A, const void* B, void* C, int M, int N, int 
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
+template <bool EDGE>
+static int launch_tile128(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
+                          hipStream_t stream) {
+    auto kern = fp8_gemm_tile128_kernel<EDGE>;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kSmallLdsBytes) != hipSuccess)
+            return HK_ERR_LAUNCH;
+        configured = true;
+    }
+    const int tiles_m = (M + kSmallTile - 1) / kSmallTile, tiles_n = (N + kSmallTile - 1) / kSmallTile;
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), kSmallLdsBytes, stream,
+                       (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
+                       tiles_n);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
 template <bool EDGE, bool RING>
 static int launch_4wave(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                         hipStream_t stream) {
@@ -551,7 +662,7 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 16) != 0) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < 0 || variant > 4) return HK_ERR_UNSUPPORTED;
+    if (variant < 0 || variant > 5) return HK_ERR_UNSUPPORTED;
     if (variant != 0 && ((K % BK) != 0 || (long long)K * BM >= (1ll << 31))) return HK_ERR_BAD_SHAPE;
     const float alpha = scale_a * scale_b;
     hipStream_t s = (hipStream_t)stream;
@@ -561,6 +672,11 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
         hipLaunchKernelGGL(fp8_gemm_portable_kernel, grid, dim3(256), 0, s, (const uint8_t*)A,
                            (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha);
         return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+    }
+    if (variant == 5) {
+        const bool edge128 = (M % kSmallTile) != 0 || (N % kSmallTile) != 0;
+        return edge128 ? launch_tile128<true>(A, B, C, M, N, K, alpha, s)
+                       : launch_tile128<false>(A, B, C, M, N, K, alpha, s);
     }
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
     if (variant == 1)
@@ -580,5 +696,8 @@ extern "C" int hk_fp8_gemm(const void* A, const void* B, void* C, int M, int N, 
                            float scale_a, float scale_b, void* stream) {
     const bool tile_ok = K > 0 && (K % hk::BK) == 0 && (long long)K * hk::BM < (1ll << 31) &&
                          M >= 64 && N >= 64;
-    return hk_fp8_gemm_variant(A, B, C, M, N, K, scale_a, scale_b, tile_ok ? 4 : 0, stream);
+    // fewer 256x256 tiles than half the CUs of an MI355X: the 128x128-tile kernel spreads the
+    // problem over four times as many workgroups
+    const long long tiles256 = (long long)((M + hk::BM - 1) / hk::BM) * ((N + hk::BN - 1) / hk::BN);
+    return hk_fp8_gemm_variant(A, B, C, M, N, K, scale_a, scale_b, !tile_ok ? 0 : tiles256 < 128 ? 5 : 4, stream);
 }

@@ -41,7 +41,7 @@ _FP8 = (torch.float8_e4m3fn, torch.uint8)
 def dispatch_fp8_gemm(A, B, C, scale_a: float = 1.0, scale_b: float = 1.0, variant: int = -1) -> None:
     """C[M,N] (bf16) = (scale_a*A[M,K]) @ (scale_b*B[N,K]).T, A and B e4m3, fp32 accumulation.
 
-    `variant` -1 lets the library choose; 0..4 force a kernel (see include/hk355.h)."""
+    `variant` -1 lets the library choose; 0..5 force a kernel (see include/hk355.h)."""
     _check_tensor(A, "A", _FP8, 2)
     _check_tensor(B, "B", _FP8, 2)
     _check_tensor(C, "C", (torch.bfloat16,), 2)

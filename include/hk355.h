@@ -55,7 +55,9 @@ int hk_fp8_gemm(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
  * 0 = portable kernel (any shape), 1 = 256x256x128 tile, 8 waves, 2 = 256x256x128 tile,
  * 4 waves, hand-interleaved schedule over two LDS stages, 3 = 256x256x128 tile, 4 waves, plain
  * loop, 4 = 256x256x128 tile, 4 waves, hand-interleaved schedule over a five-slot LDS ring with
- * the loads spread over the whole K-step (what hk_fp8_gemm picks). Variants 1-4 need K % 128 == 0. */
+ * the loads spread over the whole K-step (what hk_fp8_gemm picks when the problem has at least 128
+ * such tiles), 5 = 128x128x128 tile, 4 waves, plain loop (picked for smaller problems).
+ * Variants 1-5 need K % 128 == 0. */
 int hk_fp8_gemm_variant(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
                         int M, int N, int K, float scale_a, float scale_b,
                         int variant, void* stream);

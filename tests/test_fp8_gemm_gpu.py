@@ -35,7 +35,7 @@ SHAPES = [(256, 256, 256), (256, 256, 128), (512, 768, 384), (1024, 1024, 1024),
 RAGGED = [(300, 200, 256), (257, 255, 128), (64, 72, 640), (1000, 1000, 512)]
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 4, -1])
+@pytest.mark.parametrize("variant", [0, 1, 2, 4, 5, -1])
 @pytest.mark.parametrize("shape", SHAPES + RAGGED)
 def test_fp8_gemm_matches_oracle(hk, shape, variant):
     M, N, K = shape
@@ -50,7 +50,7 @@ def test_fp8_gemm_matches_oracle(hk, shape, variant):
     assert err <= 5e-3  # expected level; a layout bug gives O(1)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 4])
+@pytest.mark.parametrize("variant", [0, 1, 2, 4, 5])
 def test_fp8_gemm_portable_k_tail(hk, variant):
     # K % 128 != 0 is only accepted by the portable kernel
     M, N, K = 96, 80, 208
@@ -66,7 +66,7 @@ def test_fp8_gemm_portable_k_tail(hk, variant):
             _run(hk, a, b, 1.0, 1.0, variant)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 4])
+@pytest.mark.parametrize("variant", [0, 1, 2, 4, 5])
 def test_fp8_gemm_identity_is_bit_exact(hk, variant):
     """A = I (K = M): C = bf16(B^T) exactly; every e4m3 value is a bf16 value."""
     n = 256
@@ -81,7 +81,7 @@ def test_fp8_gemm_identity_is_bit_exact(hk, variant):
     assert np.array_equal(F.bf16_to_f32(out), F.bf16_to_f32(expect))
 
 
-@pytest.mark.parametrize("variant", [1, 2, 4])
+@pytest.mark.parametrize("variant", [1, 2, 4, 5])
 def test_fp8_gemm_small_integers_exact(hk, variant):
     """Operands in {-2..2}: all products and partial sums are exact in fp32, so the result is
     order independent and must equal the integer matmul, rounded once to bf16."""
