@@ -28,6 +28,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP8 = 5033.0     # MI355X dense FP8 MFMA peak, TFLOP/s (256 CU x 2.4 GHz x 8192 flop/clk/CU)
 PEAK_FP4 = 10066.0    # dense MXFP4
+PEAK_BF16 = 2516.5    # dense bf16
 PEAK_HBM = 8000.0     # GB/s
 # HBM-side bytes per 8192^3 launch of the headline kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter
 # runs of `bench.py --traffic-calibration`, each scaled by the same counter's reading for a 1 GiB copy
@@ -60,6 +61,18 @@ def bench_fp8(torch, hk, n, warmup, iters, dev, keep=False):
     if keep:
         res.update(A=Aq, B=Bq, C=C, sa=sa, sb=sb)
     return res
+
+
+def bench_bf16(torch, hk, n, warmup, iters, dev):
+    g = torch.Generator(device=dev).manual_seed(0)
+    A = torch.randn(n, n, device=dev, generator=g).to(torch.bfloat16)
+    B = torch.randn(n, n, device=dev, generator=g).to(torch.bfloat16)
+    C = torch.empty(n, n, dtype=torch.bfloat16, device=dev)
+    _, kern = _timeit(torch, lambda: hk.tk_kernel.dispatch_bf16_gemm(A, B, C), warmup, iters)
+    tf = 2.0 * n ** 3 / (kern * 1e-3) / 1e12
+    # reference: 1610.5 TFLOP/s at 8192^3 on MI355X (analysis/bf16_gemm/mi350x/mi355x_bf16_gemm.json)
+    return {"workload": f"bf16_gemm M=N=K={n}", "kernel_ms": round(kern, 5), "tflops": round(tf, 1),
+            "frac_of_bf16_peak": round(tf / PEAK_BF16, 4), "vs_reference_1610.5": round(tf / 1610.5, 4)}
 
 
 def bench_mxfp4(torch, hk, n, warmup, iters, dev):
@@ -239,6 +252,7 @@ def main() -> int:
             str(m): round(bench_fp8(torch, hk, m, 50, 50, dev)["tflops"], 1) for m in (1024, 2048, 4096, 16384)}
         del head["A"], head["B"], head["C"]
         torch.cuda.empty_cache()
+        extra["bf16_gemm"] = bench_bf16(torch, hk, 8192, 50, 50, dev)
         extra["mxfp4_gemm"] = bench_mxfp4(torch, hk, 8192, 50, 50, dev)
         extra["moe_mxfp4"] = bench_moe_mxfp4(torch, hk, quick_w, quick_i, dev)
         torch.cuda.empty_cache()

@@ -18,6 +18,19 @@ __device__ __forceinline__ int b_row_to_col(int R) {
     return (R & ~31) | ((r >> 2) << 3) | (t << 2) | (r & 3);
 }
 
+// The two 16-byte halves of a lane's fragment row (chunks g and g + 4 of the 128-byte row) as
+// separate operands, for kernels whose MFMA consumes 16 bytes per lane: MXFP4 (MX blocks g and
+// 4 + g of a 256-element K-step) and bf16 (elements 8g.. and 32 + 8g.. of a 64-element K-step).
+struct Frag4 {
+    v4i lo, hi;
+};
+__device__ __forceinline__ Frag4 lds_frag4(uint32_t addr_lo, uint32_t addr_hi, int imm) {
+    Frag4 f;
+    f.lo = *(lds_v4i_t*)(uintptr_t)(addr_lo + imm);
+    f.hi = *(lds_v4i_t*)(uintptr_t)(addr_hi + imm);
+    return f;
+}
+
 // Epilogue of the tile kernels: alpha, bf16 (RNE), 16-byte stores.
 // acc[m][2p], acc[m][2p+1] hold, for C row `row_base + 16m + lane%16`, the 8 columns
 // `col_base + 32p + 8*(lane/16) .. +8` (see b_row_to_col).

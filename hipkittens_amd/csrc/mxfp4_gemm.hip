@@ -26,17 +26,6 @@ constexpr int kScaleStageBytes = 2 * kScaleTileBytes;  // A + B
 constexpr int kScaleBase = kLdsBytes;                  // scales sit behind the operand stages
 constexpr int kLdsBytesFp4 = kLdsBytes + 2 * kScaleStageBytes;
 
-struct Frag4 {
-    v4i lo, hi;  // MX blocks g and 4+g of this lane's row
-};
-
-__device__ __forceinline__ Frag4 lds_frag4(uint32_t addr_lo, uint32_t addr_hi, int imm) {
-    Frag4 f;
-    f.lo = *(lds_v4i_t*)(uintptr_t)(addr_lo + imm);
-    f.hi = *(lds_v4i_t*)(uintptr_t)(addr_hi + imm);
-    return f;
-}
-
 // acc(16x16) += X(16x128 e2m1, scale sx) * Y(16x128 e2m1, scale sy)^T, accumulator tied in
 // an AGPR; sx / sy carry the lane's e8m0 byte in bits [7:0].
 __device__ __forceinline__ void mfma_fp4_acc(v4f& acc, const v4i& x, const v4i& y, int sx, int sy) {

@@ -61,9 +61,32 @@ def dispatch_fp8_gemm(A, B, C, scale_a: float = 1.0, scale_b: float = 1.0, varia
     _lib.check(st, "dispatch_fp8_gemm")
 
 
+def dispatch_bf16_gemm(A, B, C, variant: int = -1) -> None:
+    """C[M,N] (bf16) = A[M,K] @ B[N,K].T for bf16 operands, fp32 accumulation
+    (include/hk355.h: hk_bf16_gemm). `variant` -1 lets the library choose; 0 / 1 force a kernel."""
+    _check_tensor(A, "A", _BF16, 2)
+    _check_tensor(B, "B", _BF16, 2)
+    _check_tensor(C, "C", _BF16, 2)
+    M, K = A.shape
+    N = B.shape[0]
+    if B.shape[1] != K or tuple(C.shape) != (M, N):
+        raise RuntimeError(f"shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}, C {tuple(C.shape)}")
+    lib = _lib.load_library()
+    if variant < 0:
+        st = lib.hk_bf16_gemm(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, _stream(A))
+    else:
+        st = lib.hk_bf16_gemm_variant(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, int(variant), _stream(A))
+    _lib.check(st, "dispatch_bf16_gemm")
+
+
 def dispatch_micro(A, B, C) -> None:
-    """The reference's GEMM entry point name: C = A @ B.T with unit scales."""
-    dispatch_fp8_gemm(A, B, C, 1.0, 1.0)
+    """The reference's GEMM entry point name: C = A @ B.T. bf16 operands run the BF16 GEMM (the
+    reference's kernels/gemm/bf16fp32 binding), e4m3 operands the FP8 GEMM with unit scales (its
+    kernels/gemm/fp8fp32 executables)."""
+    if isinstance(A, torch.Tensor) and A.dtype == torch.bfloat16:
+        dispatch_bf16_gemm(A, B, C)
+    else:
+        dispatch_fp8_gemm(A, B, C, 1.0, 1.0)
 
 
 _U8 = (torch.uint8,)

@@ -79,6 +79,21 @@ int hk_mxfp4_gemm_variant(const void* A_e2m1, const void* A_scales_e8m0, const v
                           const void* B_scales_e8m0, void* C_bf16, int M, int N, int K,
                           int variant, void* stream);
 
+/*
+ * BF16 GEMM: C[M,N] = bf16( A[M,K] * B[N,K]^T ), A and B row-major bf16, fp32 accumulation, RNE.
+ * Replaces the reference's flagship kernel behind tk_kernel.dispatch_micro(A, B, C)
+ * (kernels/gemm/bf16fp32/mi350x/test_python.py:80-82, kernel kernels/gemm/bf16fp32/mi350x/, tile
+ * and binding as in kernels/gemm/bf16fp32/mi325x/256_256_64_16.cpp:13-42, 227-237), for any shape
+ * instead of one compiled-in size. Requirements: M,N,K > 0; K % 8 == 0; A, B, C 16-byte aligned.
+ */
+int hk_bf16_gemm(const void* A_bf16, const void* B_bf16, void* C_bf16, int M, int N, int K,
+                 void* stream);
+
+/* Same contract on a chosen kernel: 0 = portable kernel (any shape), 1 = 256x256x64 tile kernel
+ * (the FP8 ring schedule; needs K % 64 == 0). */
+int hk_bf16_gemm_variant(const void* A_bf16, const void* B_bf16, void* C_bf16, int M, int N, int K,
+                         int variant, void* stream);
+
 /* ------------------------------------------------------------------ MoE routing
  * The reference has no MoE code; these entry points have no counterpart in it. They follow
  * the same conventions as the GEMMs (caller-owned device buffers, asynchronous, status code).

@@ -41,6 +41,15 @@ def mxfp4_gemm(a_packed, a_scales, b_packed, b_scales, acc=np.float32) -> np.nda
     return (a @ b.T).astype(np.float32)
 
 
+def bf16_gemm(a_bits, b_bits, acc=np.float32) -> np.ndarray:
+    """fp32 result (not yet rounded to bf16) of A B^T for operands given as bf16 bit patterns
+    (uint16). Follows the reference's check C = A @ B.T
+    (kernels/gemm/bf16fp32/mi350x/test_python.py:17,32)."""
+    a = F.bf16_to_f32(np.asarray(a_bits, dtype=np.uint16)).astype(acc)
+    b = F.bf16_to_f32(np.asarray(b_bits, dtype=np.uint16)).astype(acc)
+    return (a @ b.T).astype(np.float32)
+
+
 def rel_fro_error(out: np.ndarray, ref: np.ndarray) -> float:
     out = np.asarray(out, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)

@@ -146,3 +146,20 @@ def test_reference_random_init_matches_std_mt19937():
     assert a[0, 0] == F.e4m3_encode(np.array([v0], dtype=np.float32))[0]
     assert a.shape == (4, 16) and b.shape == (2, 16)
     assert np.all(np.abs(F.e4m3_decode(a)) <= 1.0)
+
+
+def test_oracle_bf16_gemm_against_torch():
+    """oracle.gemm.bf16_gemm is the fp32 matmul of the bf16 values (torch CPU as the library routine)."""
+    import torch
+    from oracle import gemm as G
+    rng = np.random.default_rng(0)
+    a = F.bf16_round(rng.standard_normal((33, 96)).astype(np.float32))
+    b = F.bf16_round(rng.standard_normal((17, 96)).astype(np.float32))
+    ta = torch.from_numpy(a.view(np.int16)).view(torch.bfloat16).float()
+    tb = torch.from_numpy(b.view(np.int16)).view(torch.bfloat16).float()
+    ref = (ta.double() @ tb.double().t()).numpy()
+    out = G.bf16_gemm(a, b)
+    assert np.abs(out - ref).max() <= 1e-4 * np.abs(ref).max()
+    # identity: exact
+    eye = F.bf16_round(np.eye(96, dtype=np.float32))
+    assert np.array_equal(G.bf16_gemm(eye, b), F.bf16_to_f32(b).T)
