@@ -66,19 +66,22 @@ __global__ __launch_bounds__(256) void bf16_gemm_4wave_ring_kernel(
 
     // One global->LDS load of A (into A slot `slot`) or B (into the B slot at byte offset
     // `slot_off` of the B ring).
-    auto dma_a = [&](int i, int slot, uint32_t k0, v4i srd) {
+    // `vor` is 0, or for the last K-step of a K that is not a multiple of the K-step the lane's
+    // tail_or: bit 31 moves the lanes whose 16-byte chunk lies past the end of the row out of the
+    // buffer's range, and such lanes write zeros to LDS.
+    auto dma_a = [&](int i, int slot, uint32_t k0, v4i srd, uint32_t vor) {
         const uint32_t dst = lds_wave + (uint32_t)slot * kTileBytes + i * NW * 1024;
         if (EDGE)
-            dma16(srd, dst, voff_a[i], k0);
+            dma16(srd, dst, voff_a[i] | vor, k0);
         else
-            dma16(srd, dst, voff_a[0], k0 + i * dma_row_stride);
+            dma16(srd, dst, voff_a[0] | vor, k0 + i * dma_row_stride);
     };
-    auto dma_b = [&](int i, uint32_t slot_off, uint32_t k0, v4i srd) {
+    auto dma_b = [&](int i, uint32_t slot_off, uint32_t k0, v4i srd, uint32_t vor) {
         const uint32_t dst = lds_wave + kBRing + slot_off + i * NW * 1024;
         if (EDGE)
-            dma16(srd, dst, voff_b[i], k0);
+            dma16(srd, dst, voff_b[i] | vor, k0);
         else
-            dma16(srd, dst, voff_b[0], k0 + i * dma_row_stride);
+            dma16(srd, dst, voff_b[0] | vor, k0 + i * dma_row_stride);
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
@@ -101,22 +104,30 @@ __global__ __launch_bounds__(256) void bf16_gemm_4wave_ring_kernel(
     Frag4 bf[2][NT];  // B fragments of the current / next K-step (lo: K 0..31, hi: K 32..63)
     Frag4 af[4];      // rotating A fragments
 
-    const int nk = Kb / BK;
+    const int nk = (Kb + BK - 1) / BK;
+    // the chunk a lane fetches is the same for all of its loads: swz(row, lane % 8) with row bits
+    // [1..3] = 4 w + lane / 16 (mod 8)
+    const uint32_t tail_or =
+        (int)(swz_chunk(8 * w + (lane >> 3), lane & 7) * 16u) >= Kb - (nk - 1) * BK ? 0x80000000u : 0u;
 
     // ---- prologue: tiles 0 and 1 in flight, first fragments in registers ------------------
+    {
+        const uint32_t vor = nk == 1 ? tail_or : 0u;
 #pragma unroll
-    for (int i = 0; i < NDMA; ++i) dma_b(i, 0, 0, srd_b);
+        for (int i = 0; i < NDMA; ++i) dma_b(i, 0, 0, srd_b, vor);
 #pragma unroll
-    for (int i = 0; i < NDMA; ++i) dma_a(i, 0, 0, srd_a);
+        for (int i = 0; i < NDMA; ++i) dma_a(i, 0, 0, srd_a, vor);
+    }
     wait_vmcnt<0>();
     block_barrier();
     {
         v4i sa = srd_a, sb = srd_b;
         if (nk < 2) { sa.z = 0; sb.z = 0; }
+        const uint32_t vor = nk == 2 ? tail_or : 0u;
 #pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma_b(i, kTileBytes, BK, sb);
+        for (int i = 0; i < NDMA; ++i) dma_b(i, kTileBytes, BK, sb, vor);
 #pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma_a(i, 1, BK, sa);
+        for (int i = 0; i < NDMA; ++i) dma_a(i, 1, BK, sa, vor);
     }
 #pragma unroll
     for (int n = 0; n < NT; ++n) bf[0][n] = lds_frag4(b_lo0, b_hi0, n * 16 * BK);
@@ -132,6 +143,7 @@ __global__ __launch_bounds__(256) void bf16_gemm_4wave_ring_kernel(
         const uint32_t k2 = (uint32_t)(kt + 2) * BK;
         v4i sa = srd_a, sb = srd_b;
         if (kt + 2 >= nk) { sa.z = 0; sb.z = 0; }
+        const uint32_t vor = kt + 2 == nk - 1 ? tail_or : 0u;
         const uint32_t bl = b_lo0 + off1, bh = b_hi0 + off1;
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
@@ -141,7 +153,7 @@ __global__ __launch_bounds__(256) void bf16_gemm_4wave_ring_kernel(
                 if (m <= PG) {
                     const int s = m * NT + n;  // 40 slots before the barrier: B loads at 2, 7, .., 37
                     if (n == 0) af[(m + AD) & 3] = lds_frag4(a_lo[P], a_hi[P], (m + AD) * 16 * BK);
-                    if (s % 5 == 2) dma_b(s / 5, off2, k2, sb);
+                    if (s % 5 == 2) dma_b(s / 5, off2, k2, sb, vor);
                 } else {
                     const int j = (m - PG - 1) * NT + n;  // 24 slots after the barrier
                     if (j < NT) {
@@ -151,7 +163,7 @@ __global__ __launch_bounds__(256) void bf16_gemm_4wave_ring_kernel(
                     } else if (j == 2 * NT) {
                         af[2] = lds_frag4(a_lo[P ^ 1], a_hi[P ^ 1], 2 * 16 * BK);
                     }
-                    if (j < 2 * NDMA && (j & 1)) dma_a(j >> 1, P, k2, sa);  // A loads at 1, 3, .., 15
+                    if (j < 2 * NDMA && (j & 1)) dma_a(j >> 1, P, k2, sa, vor);  // A loads at 1, 3, .., 15
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -271,12 +283,12 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
                            (const uint16_t*)B, (uint16_t*)C, M, N, K, 1.0f);
         return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
     }
-    if ((K % 64) != 0 || (long long)2 * K * BM >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
+    if ((long long)2 * K * BM >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
     return edge ? launch_bf16_ring<true>(A, B, C, M, N, K, s) : launch_bf16_ring<false>(A, B, C, M, N, K, s);
 }
 
 extern "C" int hk_bf16_gemm(const void* A, const void* B, void* C, int M, int N, int K, void* stream) {
-    const bool tile_ok = K > 0 && (K % 64) == 0 && (long long)2 * K * hk::BM < (1ll << 31) && M >= 64 && N >= 64;
+    const bool tile_ok = K > 0 && (long long)2 * K * hk::BM < (1ll << 31) && M >= 64 && N >= 64;
     return hk_bf16_gemm_variant(A, B, C, M, N, K, tile_ok ? 1 : 0, stream);
 }

@@ -337,19 +337,22 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
 
     // One global->LDS load of A (into A slot `slot`) or B (into the B slot at byte offset
     // `slot_off` of the B ring).
-    auto dma_a = [&](int i, int slot, uint32_t k0, v4i srd) {
+    // `vor` is 0, or for the last K-step of a K that is not a multiple of the K-step the lane's
+    // tail_or: bit 31 moves the lanes whose 16-byte chunk lies past the end of the row out of the
+    // buffer's range, and such lanes write zeros to LDS.
+    auto dma_a = [&](int i, int slot, uint32_t k0, v4i srd, uint32_t vor) {
         const uint32_t dst = lds_wave + (uint32_t)slot * kTileBytes + i * NW * 1024;
         if (EDGE)
-            dma16(srd, dst, voff_a[i], k0);
+            dma16(srd, dst, voff_a[i] | vor, k0);
         else
-            dma16(srd, dst, voff_a[0], k0 + i * dma_row_stride);
+            dma16(srd, dst, voff_a[0] | vor, k0 + i * dma_row_stride);
     };
-    auto dma_b = [&](int i, uint32_t slot_off, uint32_t k0, v4i srd) {
+    auto dma_b = [&](int i, uint32_t slot_off, uint32_t k0, v4i srd, uint32_t vor) {
         const uint32_t dst = lds_wave + kBRing + slot_off + i * NW * 1024;
         if (EDGE)
-            dma16(srd, dst, voff_b[i], k0);
+            dma16(srd, dst, voff_b[i] | vor, k0);
         else
-            dma16(srd, dst, voff_b[0], k0 + i * dma_row_stride);
+            dma16(srd, dst, voff_b[0] | vor, k0 + i * dma_row_stride);
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
@@ -372,22 +375,30 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
     v8i bf[2][NT];  // B fragments of the current / next K-step
     v8i af[4];      // rotating A fragments
 
-    const int nk = K / BK;
+    const int nk = (K + BK - 1) / BK;
+    // the chunk a lane fetches is the same for all of its loads: swz(row, lane % 8) with row bits
+    // [1..3] = 4 w + lane / 16 (mod 8)
+    const uint32_t tail_or =
+        (int)(swz_chunk(8 * w + (lane >> 3), lane & 7) * 16u) >= K - (nk - 1) * BK ? 0x80000000u : 0u;
 
     // ---- prologue: tiles 0 and 1 in flight, first fragments in registers ------------------
+    {
+        const uint32_t vor = nk == 1 ? tail_or : 0u;
 #pragma unroll
-    for (int i = 0; i < NDMA; ++i) dma_b(i, 0, 0, srd_b);
+        for (int i = 0; i < NDMA; ++i) dma_b(i, 0, 0, srd_b, vor);
 #pragma unroll
-    for (int i = 0; i < NDMA; ++i) dma_a(i, 0, 0, srd_a);
+        for (int i = 0; i < NDMA; ++i) dma_a(i, 0, 0, srd_a, vor);
+    }
     wait_vmcnt<0>();
     block_barrier();
     {
         v4i sa = srd_a, sb = srd_b;
         if (nk < 2) { sa.z = 0; sb.z = 0; }
+        const uint32_t vor = nk == 2 ? tail_or : 0u;
 #pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma_b(i, kTileBytes, BK, sb);
+        for (int i = 0; i < NDMA; ++i) dma_b(i, kTileBytes, BK, sb, vor);
 #pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma_a(i, 1, BK, sa);
+        for (int i = 0; i < NDMA; ++i) dma_a(i, 1, BK, sa, vor);
     }
 #pragma unroll
     for (int n = 0; n < NT; ++n) bf[0][n] = lds_frag(b_lo0, b_hi0, n * 16 * BK);
@@ -403,6 +414,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
         const uint32_t k2 = (uint32_t)(kt + 2) * BK;
         v4i sa = srd_a, sb = srd_b;
         if (kt + 2 >= nk) { sa.z = 0; sb.z = 0; }
+        const uint32_t vor = kt + 2 == nk - 1 ? tail_or : 0u;
         const uint32_t bl = b_lo0 + off1, bh = b_hi0 + off1;
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
@@ -412,7 +424,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
                 if (m <= PG) {
                     const int s = m * NT + n;  // 40 slots before the barrier: B loads at 2, 7, .., 37
                     if (n == 0) af[(m + AD) & 3] = lds_frag(a_lo[P], a_hi[P], (m + AD) * 16 * BK);
-                    if (s % 5 == 2) dma_b(s / 5, off2, k2, sb);
+                    if (s % 5 == 2) dma_b(s / 5, off2, k2, sb, vor);
                 } else {
                     const int j = (m - PG - 1) * NT + n;  // 24 slots after the barrier
                     if (j < NT) {
@@ -422,7 +434,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
                     } else if (j == 2 * NT) {
                         af[2] = lds_frag(a_lo[P ^ 1], a_hi[P ^ 1], 2 * 16 * BK);
                     }
-                    if (j < 2 * NDMA && (j & 1)) dma_a(j >> 1, P, k2, sa);  // A loads at 1, 3, .., 15
+                    if (j < 2 * NDMA && (j & 1)) dma_a(j >> 1, P, k2, sa, vor);  // A loads at 1, 3, .., 15
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -498,13 +510,19 @@ __global__ __launch_bounds__(256) void fp8_gemm_tile128_kernel(
     }
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
+    const int nk = (K + BK - 1) / BK;
+    // last K-step of a K that is not a multiple of 128: lanes whose 16-byte chunk lies past the
+    // end of the row are moved out of the buffer's range (bit 31) and write zeros to LDS
+    const uint32_t tail_or =
+        (int)(swz_chunk(8 * w + (lane >> 3), lane & 7) * 16u) >= K - (nk - 1) * BK ? 0x80000000u : 0u;
     auto issue_tile = [&](int stage, int kt) {
         const uint32_t k0 = (uint32_t)kt * BK;
         const uint32_t dst = lds_wave + (uint32_t)stage * kSmallStageBytes;
+        const uint32_t vor = kt == nk - 1 ? tail_or : 0u;
 #pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma16(srd_a, dst + i * NW * 1024, voff_a[i], k0);
+        for (int i = 0; i < NDMA; ++i) dma16(srd_a, dst + i * NW * 1024, voff_a[i] | vor, k0);
 #pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma16(srd_b, dst + kSmallTileBytes + i * NW * 1024, voff_b[i], k0);
+        for (int i = 0; i < NDMA; ++i) dma16(srd_b, dst + kSmallTileBytes + i * NW * 1024, voff_b[i] | vor, k0);
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
@@ -520,7 +538,6 @@ __global__ __launch_bounds__(256) void fp8_gemm_tile128_kernel(
 #pragma unroll
         for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    const int nk = K / BK;
     issue_tile(0, 0);
     if (nk > 1) issue_tile(1, 1);
     int st = 0;
@@ -663,7 +680,9 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
     if (M <= 0 || N <= 0 || K <= 0 || (K % 16) != 0) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
     if (variant < 0 || variant > 5) return HK_ERR_UNSUPPORTED;
-    if (variant != 0 && ((K % BK) != 0 || (long long)K * BM >= (1ll << 31))) return HK_ERR_BAD_SHAPE;
+    // K tails: the ring kernel (4) and the 128x128-tile kernel (5) take any K % 16 == 0
+    if (variant != 0 && (long long)K * BM >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
+    if (variant >= 1 && variant <= 3 && (K % BK) != 0) return HK_ERR_BAD_SHAPE;
     const float alpha = scale_a * scale_b;
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {
@@ -694,8 +713,7 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
 
 extern "C" int hk_fp8_gemm(const void* A, const void* B, void* C, int M, int N, int K,
                            float scale_a, float scale_b, void* stream) {
-    const bool tile_ok = K > 0 && (K % hk::BK) == 0 && (long long)K * hk::BM < (1ll << 31) &&
-                         M >= 64 && N >= 64;
+    const bool tile_ok = K > 0 && (long long)K * hk::BM < (1ll << 31) && M >= 64 && N >= 64;
     // fewer 256x256 tiles than half the CUs of an MI355X: the 128x128-tile kernel spreads the
     // problem over four times as many workgroups
     const long long tiles256 = (long long)((M + hk::BM - 1) / hk::BM) * ((N + hk::BN - 1) / hk::BN);

@@ -57,7 +57,7 @@ int hk_fp8_gemm(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
  * loop, 4 = 256x256x128 tile, 4 waves, hand-interleaved schedule over a five-slot LDS ring with
  * the loads spread over the whole K-step (what hk_fp8_gemm picks when the problem has at least 128
  * such tiles), 5 = 128x128x128 tile, 4 waves, plain loop (picked for smaller problems).
- * Variants 1-5 need K % 128 == 0. */
+ * Variants 1-3 need K % 128 == 0; 4 and 5 zero-fill the last K-step of any K % 16 == 0. */
 int hk_fp8_gemm_variant(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
                         int M, int N, int K, float scale_a, float scale_b,
                         int variant, void* stream);
@@ -90,7 +90,7 @@ int hk_bf16_gemm(const void* A_bf16, const void* B_bf16, void* C_bf16, int M, in
                  void* stream);
 
 /* Same contract on a chosen kernel: 0 = portable kernel (any shape), 1 = 256x256x64 tile kernel
- * (the FP8 ring schedule; needs K % 64 == 0). */
+ * (the FP8 ring schedule; the last K-step of a K that is not a multiple of 64 is zero-filled). */
 int hk_bf16_gemm_variant(const void* A_bf16, const void* B_bf16, void* C_bf16, int M, int N, int K,
                          int variant, void* stream);
 

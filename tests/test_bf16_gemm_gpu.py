@@ -49,18 +49,17 @@ def test_bf16_gemm_matches_oracle(hk, shape, variant):
     assert err <= 5e-3  # expected level; a layout bug gives O(1)
 
 
-@pytest.mark.parametrize("variant", [0, 1])
-def test_bf16_gemm_k_not_multiple_of_64(hk, variant):
-    M, N, K = 96, 80, 104  # K % 8 == 0 only: portable kernel; the tile kernel refuses
-    rng = np.random.default_rng(11)
+@pytest.mark.parametrize("variant", [0, 1, -1])
+@pytest.mark.parametrize("shape", [(96, 80, 104), (256, 256, 8), (300, 264, 200), (256, 384, 2880)])
+def test_bf16_gemm_k_not_multiple_of_64(hk, shape, variant):
+    """K % 8 == 0 only: the tile kernel zero-fills the last K-step."""
+    M, N, K = shape
+    print(f"bf16_gemm k-tail shape={shape} variant={variant}", flush=True)
+    rng = np.random.default_rng(11 + K)
     a, b = _bits(rng.standard_normal((M, K))), _bits(rng.standard_normal((N, K)))
-    if variant == 0:
-        for v in (0, -1):
-            out = F.bf16_to_f32(_run(hk, a, b, v))
-            assert G.rel_fro_error(out, G.bf16_gemm(a, b)) <= 5e-3
-    else:
-        with pytest.raises(RuntimeError):
-            _run(hk, a, b, variant)
+    out = F.bf16_to_f32(_run(hk, a, b, variant))
+    assert np.isfinite(out).all()
+    assert G.rel_fro_error(out, G.bf16_gemm(a, b)) <= 5e-3
 
 
 @pytest.mark.parametrize("variant", [0, 1])

@@ -50,20 +50,52 @@ def test_fp8_gemm_matches_oracle(hk, shape, variant):
     assert err <= 5e-3  # expected level; a layout bug gives O(1)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 4, 5])
-def test_fp8_gemm_portable_k_tail(hk, variant):
-    # K % 128 != 0 is only accepted by the portable kernel
-    M, N, K = 96, 80, 208
-    rng = np.random.default_rng(7)
+K_TAIL = [(96, 80, 208), (256, 256, 16), (256, 256, 144), (300, 520, 272), (512, 384, 2880), (128, 128, 112)]
+
+
+@pytest.mark.parametrize("variant", [0, 4, 5, -1])
+@pytest.mark.parametrize("shape", K_TAIL)
+def test_fp8_gemm_k_tail(hk, shape, variant):
+    """K % 16 == 0 but K % 128 != 0 (2880 is the hidden size of the MoE models): the ring and
+    128x128-tile kernels zero-fill the last K-step. The buffers are carved out of a larger one
+    filled with NaN codes, so a read past a row's end would show in the result."""
+    M, N, K = shape
+    print(f"fp8_gemm k-tail shape={shape} variant={variant}", flush=True)
+    rng = np.random.default_rng(7 + K)
     (a, sa), (b, sb) = _random_codes(rng, M, K), _random_codes(rng, N, K)
-    if variant == 0:
-        out = F.bf16_to_f32(_run(hk, a, b, float(sa), float(sb), 0))
+    out = F.bf16_to_f32(_run(hk, a, b, float(sa), float(sb), variant))
+    assert np.isfinite(out).all()
+    assert G.rel_fro_error(out, G.fp8_gemm(a, b, sa, sb)) <= 5e-3
+
+
+def test_fp8_gemm_k_tail_last_row_does_not_read_past_the_buffer(hk):
+    """The last row's tail chunks lie past the end of the allocation: with A and B placed at the
+    very end of a NaN-filled pool, a kernel that fetched them would return NaN."""
+    M, N, K = 256, 256, 208
+    rng = np.random.default_rng(99)
+    (a, sa), (b, sb) = _random_codes(rng, M, K), _random_codes(rng, N, K)
+    dev = torch.device("cuda:0")
+    for variant in (4, 5):
+        pool = torch.full((4 * M * K,), 0x7F, dtype=torch.uint8, device=dev)  # e4m3fn NaN code
+        A = pool[M * K:2 * M * K].view(M, K)
+        B = pool[2 * M * K:3 * M * K].view(N, K)
+        A.copy_(torch.from_numpy(a).to(dev))
+        B.copy_(torch.from_numpy(b).to(dev))
+        C = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+        hk.tk_kernel.dispatch_fp8_gemm(A.view(torch.float8_e4m3fn), B.view(torch.float8_e4m3fn), C,
+                                       float(sa), float(sb), variant=variant)
+        torch.cuda.synchronize()
+        out = C.float().cpu().numpy()
+        assert np.isfinite(out).all(), variant
         assert G.rel_fro_error(out, G.fp8_gemm(a, b, sa, sb)) <= 5e-3
-        out = F.bf16_to_f32(_run(hk, a, b, float(sa), float(sb), -1))
-        assert G.rel_fro_error(out, G.fp8_gemm(a, b, sa, sb)) <= 5e-3
-    else:
-        with pytest.raises(RuntimeError):
-            _run(hk, a, b, 1.0, 1.0, variant)
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+def test_fp8_gemm_older_tile_kernels_refuse_k_tail(hk, variant):
+    rng = np.random.default_rng(7)
+    (a, _), (b, _) = _random_codes(rng, 96, 208), _random_codes(rng, 80, 208)
+    with pytest.raises(RuntimeError):
+        _run(hk, a, b, 1.0, 1.0, variant)
 
 
 @pytest.mark.parametrize("variant", [0, 1, 2, 4, 5])
