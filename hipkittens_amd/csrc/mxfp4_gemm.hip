@@ -11,9 +11,12 @@
 // Tile kernel: 256x256 tile of C, K-step 256 elements = 128 bytes per operand row, so the LDS
 // tile layout, swizzle and read pattern are those of the FP8 kernel; the two 16-byte halves a
 // lane reads per fragment row are MX blocks g and 4+g of the K-step and feed two MFMAs. The
-// 8 scale bytes per row and K-step travel through LDS next to the tiles (4-byte direct loads)
-// and are read back with one ds_read_b64 per fragment; a per-lane shift moves byte g into the
-// position the MFMA reads.
+// 8 scale bytes per row and K-step travel through LDS next to the tiles: one 16-byte direct load
+// per row brings the scales of a pair of K-steps (every global->LDS load costs the CU's address
+// unit the same time whatever its width, and that time is taken from the MFMAs, so the scales
+// come in as few loads as possible: 2 per wave and pair of K-steps). They are read back with
+// one ds_read_b64 per fragment and K-step; a per-lane shift moves byte g into the position the
+// MFMA reads.
 #include "gemm_tile.h"
 #include "../../include/hk355.h"
 
@@ -21,7 +24,7 @@ namespace hk {
 
 typedef __attribute__((address_space(3))) const v2i lds_v2i_t;
 
-constexpr int kScaleTileBytes = BM * 8;                // 8 scale bytes per row and K-step
+constexpr int kScaleTileBytes = BM * 16;               // per row: 8 scale bytes for each K-step of a pair
 constexpr int kScaleStageBytes = 2 * kScaleTileBytes;  // A + B
 constexpr int kScaleBase = kLdsBytes;                  // scales sit behind the operand stages
 constexpr int kLdsBytesFp4 = kLdsBytes + 2 * kScaleStageBytes;
@@ -78,24 +81,23 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
         voff_a[i] = (uint32_t)ra * (uint32_t)Kb + c * 16u;
         voff_b[i] = (uint32_t)rb * (uint32_t)Kb + c * 16u;
     }
-    // scale tiles: load q (0..7) covers LDS rows 32q..32q+31, lane l -> row +l/2, dword l%2;
-    // this wave issues q = 2w and 2w+1 for each operand.
-    uint32_t voff_sa[2], voff_sb[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int R = 32 * (2 * w + j) + (lane >> 1);
+    // scale tiles: this wave loads LDS rows 64w..64w+63 of each operand, lane l -> row 64w + l,
+    // 16 bytes = the row's scales of K-steps 2p and 2p+1
+    uint32_t voff_sa, voff_sb;
+    {
+        const int R = 64 * w + lane;
         int ra = R, rb = b_row_to_col(R);
         if (EDGE) {
             ra = min(ra, a_rows - 1);
             rb = min(rb, b_rows - 1);
         }
-        voff_sa[j] = (uint32_t)ra * (uint32_t)Ks + (lane & 1) * 4u;
-        voff_sb[j] = (uint32_t)rb * (uint32_t)Ks + (lane & 1) * 4u;
+        voff_sa = (uint32_t)ra * (uint32_t)Ks;
+        voff_sb = (uint32_t)rb * (uint32_t)Ks;
     }
     const uint32_t dma_row_stride = to_sgpr((uint32_t)(8 * NW) * (uint32_t)Kb);
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-    const uint32_t lds_scale_wave = to_sgpr(lds0 + kScaleBase + (uint32_t)w * 512u);
+    const uint32_t lds_scale_wave = to_sgpr(lds0 + kScaleBase + (uint32_t)w * 1024u);
 
     auto dma_one = [&](int op, int i, int stage, uint32_t k0, v4i srd) {
         const uint32_t dst = lds_wave + (uint32_t)stage * kStageBytes + op * kTileBytes + i * NW * 1024;
@@ -104,11 +106,10 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
         else
             dma16(srd, dst, op ? voff_b[0] : voff_a[0], k0 + i * dma_row_stride);
     };
-    // j = 0..3: (operand j/2, load j%2) of this wave's scale loads for K-step kt into `stage`
-    auto dma_scale = [&](int j, int stage, uint32_t kt, v4i srd) {
-        const int op = j >> 1, h = j & 1;
-        const uint32_t dst = lds_scale_wave + (uint32_t)stage * kScaleStageBytes + op * kScaleTileBytes + h * 256;
-        dma4(srd, dst, op ? voff_sb[h] : voff_sa[h], kt * 8u);
+    // this wave's scale load of operand `op` for the pair of K-steps `pair` (stage pair % 2)
+    auto dma_scale = [&](int op, uint32_t pair, v4i srd) {
+        const uint32_t dst = lds_scale_wave + (pair & 1u) * kScaleStageBytes + op * kScaleTileBytes;
+        dma16(srd, dst, op ? voff_sb : voff_sa, pair * 16u);
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
@@ -122,13 +123,15 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
         b_lo[st] = lds0 + st * kStageBytes + kTileBytes + wn * (TN * BK) + rd_lo;
         b_hi[st] = lds0 + st * kStageBytes + kTileBytes + wn * (TN * BK) + rd_hi;
     }
-    // scales of fragment f, stage st: base + st*kScaleStageBytes + f*128
-    uint32_t sa_rd = lds0 + kScaleBase + (wm * TM + r) * 8u;
-    uint32_t sb_rd = lds0 + kScaleBase + kScaleTileBytes + (wn * TN + r) * 8u;
+    // scales of fragment f, K-step parity p, in the stage of the pair the base points to:
+    // base + f*256 + p*8; sa_rd / sb_rd follow the pair of the running K-step
+    uint32_t sa_rd = lds0 + kScaleBase + (wm * TM + r) * 16u;
+    uint32_t sb_rd = lds0 + kScaleBase + kScaleTileBytes + (wn * TN + r) * 16u;
+    static_assert(kScaleBase % (2 * kScaleStageBytes) == 0, "the pair's stage is toggled with xor");
     asm volatile("" : "+v"(sa_rd), "+v"(sb_rd));  // keep the large base in the register, offsets in immediates
     const uint32_t sh = 8u * g;  // byte g of each scale dword belongs to this lane
-    auto rd_scale = [&](uint32_t base, int stage, int f) -> v2i {
-        return *(lds_v2i_t*)(uintptr_t)(base + stage * kScaleStageBytes + f * 128);
+    auto rd_scale = [&](uint32_t base, int p, int f) -> v2i {
+        return *(lds_v2i_t*)(uintptr_t)(base + f * 256 + p * 8);
     };
     auto shift_scale = [&](v2i& s) {
         s.x = (int)((uint32_t)s.x >> sh);
@@ -150,8 +153,8 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     for (int i = 0; i < NDMA; ++i) dma_one(0, i, 0, 0, srd_a);
 #pragma unroll
     for (int i = 0; i < NDMA; ++i) dma_one(1, i, 0, 0, srd_b);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) dma_scale(j, 0, 0, j >> 1 ? srd_sb : srd_sa);
+    dma_scale(0, 0, srd_sa);
+    dma_scale(1, 0, srd_sb);
     wait_vmcnt<0>();
     block_barrier();
     if (nk > 1) {
@@ -159,8 +162,6 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
         for (int i = 0; i < NDMA; ++i) dma_one(0, i, 1, BK, srd_a);
 #pragma unroll
         for (int i = 0; i < NDMA; ++i) dma_one(1, i, 1, BK, srd_b);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) dma_scale(j, 1, 1, j >> 1 ? srd_sb : srd_sa);
     }
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
@@ -183,6 +184,9 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
         const uint32_t k2 = (uint32_t)(kt + 2) * BK;
         v4i sa = srd_a, sb = srd_b, ssa = srd_sa, ssb = srd_sb;
         if (kt + 2 >= nk) { sa.z = 0; sb.z = 0; ssa.z = 0; ssb.z = 0; }
+        // scales of the next K-step: same pair (P == 0) or the next pair, in the other stage
+        const uint32_t sa_nx = P ? sa_rd ^ kScaleStageBytes : sa_rd;
+        const uint32_t sb_nx = P ? sb_rd ^ kScaleStageBytes : sb_rd;
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             // first the 8 MFMAs on the low K-half (MX block g), then the 8 on the high half
@@ -199,16 +203,18 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
                     const int j = (m - PG - 1) * NT + n;
                     if (j < NT) {
                         bf[P ^ 1][j] = lds_frag4(b_lo[P ^ 1], b_hi[P ^ 1], j * 16 * BK);
-                        bs[P ^ 1][j] = rd_scale(sb_rd, P ^ 1, j);
+                        bs[P ^ 1][j] = rd_scale(sb_nx, P ^ 1, j);
                     } else if (j == NT || j == NT + 1) {
                         af[j - NT] = lds_frag4(a_lo[P ^ 1], a_hi[P ^ 1], (j - NT) * 16 * BK);
-                        as[j - NT] = rd_scale(sa_rd, P ^ 1, j - NT);
+                        as[j - NT] = rd_scale(sa_nx, P ^ 1, j - NT);
                     } else if (j == 2 * NT) {
                         af[2] = lds_frag4(a_lo[P ^ 1], a_hi[P ^ 1], 2 * 16 * BK);
-                        as[2] = rd_scale(sa_rd, P ^ 1, 2);
+                        as[2] = rd_scale(sa_nx, P ^ 1, 2);
                     }
                     if (j < 2 * NDMA) dma_one(j / NDMA, j % NDMA, P, k2, j / NDMA ? sb : sa);
-                    else if (j < 2 * NDMA + 4) dma_scale(j - 2 * NDMA, P, kt + 2, (j - 2 * NDMA) >> 1 ? ssb : ssa);
+                    // the next pair's scales: its stage was last read before this step's barrier
+                    // of the previous odd K-step, and is first read after the next step's barrier
+                    else if (P == 0 && j < 2 * NDMA + 2) dma_scale(j - 2 * NDMA, (uint32_t)(kt >> 1) + 1u, j - 2 * NDMA ? ssb : ssa);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -226,6 +232,10 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
                 block_barrier();
                 __builtin_amdgcn_sched_barrier(0);
             }
+        }
+        if (P) {
+            sa_rd = sa_nx;
+            sb_rd = sb_nx;
         }
     };
 
