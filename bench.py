@@ -111,11 +111,18 @@ def bench_moe_mxfp4(torch, hk, warmup, iters, dev):
     flop = 2.0 * T * k * (H * 2 * I + I * H)
     tf = flop / (kern * 1e-3) / 1e12
     compulsory = wbytes + 2 * T * H * 2  # weights once + x in + y out
+    # the same layer with the GPT-OSS expert epilogues: biases and clamped SwiGLU (the row order of
+    # the source weights was resolved by the pre-shuffle, so the same shuffled weights serve)
+    b13 = torch.randn(E, 2 * I, device=dev, generator=g)
+    b2 = torch.randn(E, H, device=dev, generator=g)
+    _, kern_oai = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_mxfp4(
+        x, logits, W, None, None, None, y, k, ws, bias13=b13, bias2=b2, activation="swiglu_oai"), warmup, iters)
     return {"workload": "moe_mxfp4 T=4096 H=2880 I=2880 E=128 top-4 softmax, MXFP4 activations and weights "
                         "(routing + sort + quantize/permute + 2 grouped GEMMs + un-permute)",
             "ms": round(kern, 5), "tflops": round(tf, 1), "frac_of_mxfp4_peak": round(tf / PEAK_FP4, 4),
             "compulsory_GB": round(compulsory / 1e9, 3),
-            "frac_of_hbm_roofline": round(compulsory / (kern * 1e-3) / 1e9 / PEAK_HBM, 4)}
+            "frac_of_hbm_roofline": round(compulsory / (kern * 1e-3) / 1e9 / PEAK_HBM, 4),
+            "ms_with_biases_and_clamped_swiglu": round(kern_oai, 5)}
 
 
 def bench_moe_fp8blk(torch, hk, warmup, iters, dev):

@@ -9,11 +9,13 @@ namespace hk {
 // mode 0 (gate+up, N = I): each wave's 64 rows alternate 16 gate rows / 16 up rows of the same 16
 // h columns, permuted so that a lane ends up with 8 consecutive h columns; mode 1 (down, N = H):
 // b_row_to_col permutation (8 consecutive output columns per lane).
-__device__ __forceinline__ int moe_b_row(int mode, int R, int n_tile, int N) {
+// `interleaved` (mode 0): the caller's matrix has gate / up of h column c in rows 2c / 2c + 1
+// instead of rows c / N + c.
+__device__ __forceinline__ int moe_b_row(int mode, int R, int n_tile, int N, bool interleaved = false) {
     if (mode == 1) return min(n_tile * 256 + b_row_to_col(R), N - 1);
     const int wn = R >> 6, t = (R >> 4) & 3, r = R & 15;
-    const int hcol = 32 * wn + 8 * (r >> 2) + 4 * (t >> 1) + (r & 3);
-    return (t & 1) * N + min(n_tile * 128 + hcol, N - 1);
+    const int hcol = min(n_tile * 128 + 32 * wn + 8 * (r >> 2) + 4 * (t >> 1) + (r & 3), N - 1);
+    return interleaved ? 2 * hcol + (t & 1) : (t & 1) * N + hcol;
 }
 
 // Work items. A work item is (m-tile, n-tile): up to kMoeBM (weight-streaming MXFP4 kernel: 192)

@@ -47,6 +47,15 @@ __device__ __forceinline__ uint32_t pack8_e2m1(const float (&v)[8], int e) {
 __device__ __forceinline__ float silu_mul(float g, float u) {
     return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
 }
+// Gated activation of the extended epilogues. act 0: SiLU(g) * u; act 1: the clamped SwiGLU of
+// the GPT-OSS experts, (clamp(u, -limit, limit) + 1) * g' * sigmoid(alpha * g') with
+// g' = min(g, limit).
+__device__ __forceinline__ float glu_act(int act, float g, float u, float alpha, float limit) {
+    if (act == 0) return silu_mul(g, u);
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return (u + 1.0f) * (g * __builtin_amdgcn_rcpf(1.0f + __expf(-alpha * g)));
+}
 
 // x [rows, cols] bf16 -> packed e2m1 [rows, cols/2] + e8m0 scales [rows, scale_pitch] (columns
 // >= cols/32 are filled with 127). One thread per 8 elements, 4 threads per MX block.
@@ -140,10 +149,12 @@ __global__ __launch_bounds__(128) void mxfp4_quantize_permute_kernel(
 // mode 0 (gate+up, N = I): fragment 0 holds the gate rows and fragment 1 the up rows of h columns
 // 128 n_tile + 16 w .. +16, in order; mode 1 (down, N = H): the b_row_to_col permutation, which
 // gives a lane 8 consecutive output columns from its two fragments. Rows past N repeat row N - 1.
+// mode 2: as mode 0 for a source matrix with gate / up of h column c in rows 2c / 2c + 1.
 __device__ __forceinline__ int moe_stream_b_row(int mode, int R, int n_tile, int N) {
     if (mode == 1) return min(n_tile * 256 + b_row_to_col(R), N - 1);
     const int w = R >> 5, f = (R >> 4) & 1, r = R & 15;
-    return f * N + min(n_tile * 128 + 16 * w + r, N - 1);
+    const int hcol = min(n_tile * 128 + 16 * w + r, N - 1);
+    return mode == 2 ? 2 * hcol + f : f * N + hcol;
 }
 
 // Pre-shuffled weight layout, made for moe_mxfp4_stream_kernel: weights go from HBM straight
@@ -161,7 +172,7 @@ __global__ __launch_bounds__(256) void moe_preshuffle_kernel(const uint8_t* __re
                                                              uint8_t* __restrict__ out_w,
                                                              uint8_t* __restrict__ out_s) {
     const int Kb = K >> 1, nk = (Kb + 127) >> 7;
-    const int rows_b = mode == 0 ? 2 * N : N;
+    const int rows_b = mode == 1 ? N : 2 * N;
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;  // one 16-byte chunk each
     const long long total = (long long)E * n_tiles * nk * 2048;
     if (gid >= total) return;
@@ -237,6 +248,11 @@ struct MoeGemmParams {
     int K;                   // contraction length in elements
     int N;                   // MODE 0: I (h columns; weight rows i and I+i); MODE 1: output columns
     int n_tiles_n;
+    // extended epilogues (kernels instantiated with EXT) only:
+    const float* bias;       // null or fp32 [E][rows of B] in the caller's row order, added to the GEMM result
+    int act;                 // MODE 0: 0 = SiLU(gate) * up, 1 = clamped SwiGLU (glu_act)
+    float alpha, limit;
+    int interleaved;         // MODE 0: the caller's gate / up rows (and biases) of h column c are 2c / 2c + 1
 };
 
 constexpr int kMoeATile = kMoeBM * 128;                 // 16 KiB
@@ -252,7 +268,7 @@ constexpr int kMoeLds = kMoeScaleBase + kMoeStages * kMoeScaleStage;  // 153 KiB
 struct MoeAddr {
     v4i srd_b, srd_sb;
     uint32_t voff_b[4], voff_sb;
-    int row_start, rows, n0, n_tile;
+    int row_start, rows, n0, n_tile, expert;
     bool valid;
 };
 
@@ -263,7 +279,7 @@ struct MoeAddr {
 // because the two waves of a SIMD cover for each other: while one is held up issuing loads or
 // waiting for LDS, the other feeds the matrix pipe (a single wave per SIMD cannot issue the
 // 16-cycle FP4 MFMA back to back, nor issue loads and MFMAs at the same time).
-template <int MODE>
+template <int MODE, bool EXT>
 __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams p) {
     constexpr int NW = 8, MT = kMoeBM / 32, NT = 4;   // MT fragments of 16 rows per wave
     constexpr int NA = kMoeBM / 64;                  // A-tile loads per wave and K-step
@@ -302,13 +318,14 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
         if (!a.valid) idx = it_end - 1;  // harmless values; every load of an invalid set is zero-sized
         const v4i item = scalar_load_x4(p.items + idx);  // {expert, row_start, rows, n_tile}
         const int expert = item.x;
+        a.expert = expert;
         a.row_start = item.y;
         a.rows = item.z;
         a.n_tile = item.w;
         a.n0 = a.n_tile * (MODE == 0 ? 128 : 256);
         a.srd_b = make_srd(p.B + (size_t)expert * p.b_expert_stride, (uint32_t)rows_b * (uint32_t)p.b_pitch);
         a.srd_sb = make_srd(p.SB + (size_t)expert * p.sb_expert_stride, (uint32_t)rows_b * (uint32_t)p.sb_pitch);
-        auto b_row = [&](int R) -> int { return moe_b_row(MODE, R, a.n_tile, p.N); };
+        auto b_row = [&](int R) -> int { return moe_b_row(MODE, R, a.n_tile, p.N, EXT && p.interleaved); };
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             a.voff_b[i] = (uint32_t)b_row(8 * (i * NW + w) + (lane >> 3)) * (uint32_t)p.b_pitch + chunk16 * 16u;
@@ -428,7 +445,12 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
                 for (int q = 0; q < NT / 2; ++q) {
                     const int col = n0 + wn * 64 + 32 * q + 8 * (int)g;
                     if (col + 8 > p.N) continue;  // N % 8 == 0
-                    const v4f x = acc[m][2 * q], y = acc[m][2 * q + 1];
+                    v4f x = acc[m][2 * q], y = acc[m][2 * q + 1];
+                    if (EXT && p.bias) {
+                        const float* bb = p.bias + (size_t)a.expert * p.N + col;
+                        x += *(const v4f*)bb;
+                        y += *(const v4f*)(bb + 4);
+                    }
                     v4i o4;
                     o4.x = pack_bf16(x.x, x.y); o4.y = pack_bf16(x.z, x.w);
                     o4.z = pack_bf16(y.x, y.y); o4.w = pack_bf16(y.z, y.w);
@@ -443,6 +465,19 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
             const bool col_ok = hcol0 < p.N;
             const size_t kt2 = (size_t)(hcol0 >> 8);
             const int byte0 = ((hcol0 & 255) >> 1) + 4 * (int)g, blk = (hcol0 & 255) >> 5;
+            // extended epilogue: biases of this lane's 8 h columns hcol0 + 8 g .. +8
+            float bg[8], bu[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) bg[i] = bu[i] = 0.f;
+            if (EXT && p.bias && col_ok) {
+                const float* bb = p.bias + (size_t)a.expert * 2 * p.N;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int c = hcol0 + 8 * (int)g + i;
+                    bg[i] = bb[p.interleaved ? 2 * c : c];
+                    bu[i] = bb[p.interleaved ? 2 * c + 1 : p.N + c];
+                }
+            }
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 const int row = 16 * (2 * m + wm) + (int)r;
@@ -454,7 +489,8 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const float gv = gt[j];
-                        h[4 * q + j] = silu_mul(gv, up[j]);
+                        h[4 * q + j] = EXT ? glu_act(p.act, gv + bg[4 * q + j], up[j] + bu[4 * q + j], p.alpha, p.limit)
+                                           : silu_mul(gv, up[j]);
                     }
                 }
                 float amax = 0.f;
@@ -544,7 +580,7 @@ constexpr int kStHTile = kStXch + kStBM * 8 * 4;        // epilogue: packed h ti
 constexpr int kStHScale = kStHTile + kStBM * 64;        // epilogue: h scales [kStBM][4 bytes]
 constexpr int kStLds = kStHScale + kStBM * 4;           // 146.25 KiB
 
-template <int MODE>
+template <int MODE, bool EXT>
 __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmParams p) {
     constexpr int MT = kStBM / 16, NT = 2;
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
@@ -704,11 +740,18 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
             // lane (r, g) holds, for row 16 m + r, the 8 consecutive columns 32 w + 8 g .. +8
             uint16_t* out = (uint16_t*)p.out0;
             const int col = c.n_tile * 256 + w * 32 + 8 * (int)g;
+            v4f b0 = {0.f, 0.f, 0.f, 0.f}, b1 = {0.f, 0.f, 0.f, 0.f};
+            if (EXT && p.bias && col + 8 <= p.N) {
+                const float* bb = p.bias + (size_t)c.expert * p.N + col;
+                b0 = *(const v4f*)bb;
+                b1 = *(const v4f*)(bb + 4);
+            }
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 const int row = 16 * m + (int)r;
                 if (row >= rows || col + 8 > p.N) continue;  // N % 8 == 0
-                const v4f x = acc[m][0], y = acc[m][1];
+                v4f x = acc[m][0], y = acc[m][1];
+                if (EXT) { x += b0; y += b1; }
                 v4i o4;
                 o4.x = pack_bf16(x.x, x.y); o4.y = pack_bf16(x.z, x.w);
                 o4.z = pack_bf16(y.x, y.y); o4.w = pack_bf16(y.z, y.w);
@@ -724,6 +767,17 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
             typedef __attribute__((address_space(3))) uint8_t lds_u8_mut_t;
             const int hcol0 = c.n_tile * 128 + 16 * w;  // first of the wave's 16 h columns
             const bool col_ok = hcol0 < p.N;            // N % 32 == 0: a block is valid as a whole
+            // extended epilogue: biases of this lane's 4 h columns hcol0 + 4 g .. +4
+            float bg[4] = {0.f, 0.f, 0.f, 0.f}, bu[4] = {0.f, 0.f, 0.f, 0.f};
+            if (EXT && p.bias && col_ok) {
+                const float* bb = p.bias + (size_t)c.expert * 2 * p.N;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int hc = hcol0 + 4 * (int)g + j;
+                    bg[j] = bb[p.interleaved ? 2 * hc : hc];
+                    bu[j] = bb[p.interleaved ? 2 * hc + 1 : p.N + hc];
+                }
+            }
             // two groups of six fragments, to keep the number of live h values small
 #pragma unroll
             for (int m0 = 0; m0 < MT; m0 += MT / 2) {
@@ -736,7 +790,8 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
                     float amax = 0.f;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        h[mm][j] = col_ok ? silu_mul(gt[j], up[j]) : 0.f;
+                        if (EXT) h[mm][j] = col_ok ? glu_act(p.act, gt[j] + bg[j], up[j] + bu[j], p.alpha, p.limit) : 0.f;
+                        else h[mm][j] = col_ok ? silu_mul(gt[j], up[j]) : 0.f;
                         amax = fmaxf(amax, fabsf(h[mm][j]));
                     }
                     amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
@@ -888,9 +943,9 @@ void moe_launch_build_items(const int32_t* expert_offsets, int E, int bm, int n_
     hipLaunchKernelGGL(moe_build_items_kernel, dim3(2), dim3(512), 0, s, expert_offsets, E, b, num_items);
 }
 
-template <int MODE>
+template <int MODE, bool EXT>
 static int launch_moe_stream(MoeGemmParams p, int max_items, hipStream_t s) {
-    auto kern = moe_mxfp4_stream_kernel<MODE>;
+    auto kern = moe_mxfp4_stream_kernel<MODE, EXT>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kStLds) !=
@@ -904,9 +959,9 @@ static int launch_moe_stream(MoeGemmParams p, int max_items, hipStream_t s) {
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
-template <int MODE>
+template <int MODE, bool EXT>
 static int launch_moe_gemm(MoeGemmParams p, int max_items, hipStream_t s) {
-    auto kern = moe_mxfp4_gemm_kernel<MODE>;
+    auto kern = moe_mxfp4_gemm_kernel<MODE, EXT>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMoeLds) !=
@@ -949,8 +1004,8 @@ extern "C" int hk_moe_unpermute(const void* o_bf16, const float* w, const int32_
 
 extern "C" int hk_moe_mxfp4_preshuffle_bytes(int E, int N, int K, int mode, size_t* w_bytes, size_t* s_bytes) {
     if (!w_bytes || !s_bytes) return HK_ERR_NULL_POINTER;
-    if (E <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || (mode != 0 && mode != 1)) return HK_ERR_BAD_SHAPE;
-    const size_t n_tiles = mode == 0 ? (N + 127) / 128 : (N + 255) / 256;
+    if (E <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || mode < 0 || mode > 2) return HK_ERR_BAD_SHAPE;
+    const size_t n_tiles = mode != 1 ? (N + 127) / 128 : (N + 255) / 256;
     const size_t nk = (K / 2 + 127) / 128;
     *w_bytes = (size_t)E * n_tiles * nk * kMoeBTile;
     *s_bytes = (size_t)E * n_tiles * nk * kMoeScaleB;
@@ -960,10 +1015,10 @@ extern "C" int hk_moe_mxfp4_preshuffle_bytes(int E, int N, int K, int mode, size
 extern "C" int hk_moe_mxfp4_preshuffle(const void* w, const void* scales, int scale_pitch, int E, int N, int K,
                                        int mode, void* out_w, void* out_s, void* stream) {
     if (!w || !scales || !out_w || !out_s) return HK_ERR_NULL_POINTER;
-    if (E <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || scale_pitch < K / 32 || (mode != 0 && mode != 1))
+    if (E <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || scale_pitch < K / 32 || mode < 0 || mode > 2)
         return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)w | (uintptr_t)out_w) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    const int n_tiles = mode == 0 ? (N + 127) / 128 : (N + 255) / 256;
+    const int n_tiles = mode != 1 ? (N + 127) / 128 : (N + 255) / 256;
     const long long total = (long long)E * n_tiles * ((K / 2 + 127) / 128) * 2048;
     if ((total + 255) / 256 >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
     hipLaunchKernelGGL(moe_preshuffle_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
@@ -1017,12 +1072,18 @@ static int moe_mxfp4_check(int T, int H, int I, int E, int k, int w13_scale_pitc
 }
 
 // Expert MLP on already routed and sorted tokens (steps 3-6 of the forward pass).
-extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const void* w13_scales,
-                                    int w13_scale_pitch, const void* w2, const void* w2_scales,
-                                    int w2_scale_pitch, const float* topk_w, const int32_t* sorted_slots,
-                                    const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
-                                    int T, int H, int I, int E, int k, int weight_layout, void* workspace,
-                                    size_t workspace_bytes, void* stream) {
+extern "C" int hk_moe_mxfp4_experts_ex(const void* x_bf16, const void* w13, const void* w13_scales,
+                                       int w13_scale_pitch, const void* w2, const void* w2_scales,
+                                       int w2_scale_pitch, const float* topk_w, const int32_t* sorted_slots,
+                                       const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
+                                       int T, int H, int I, int E, int k, int weight_layout,
+                                       const float* bias13, const float* bias2, int activation, float alpha,
+                                       float limit, int w13_interleaved, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
+    if (activation != 0 && activation != 1) return HK_ERR_UNSUPPORTED;
+    if (activation == 1 && !(limit > 0.f)) return HK_ERR_BAD_SHAPE;
+    if (((uintptr_t)bias13 | (uintptr_t)bias2) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    const bool ext = bias13 || bias2 || activation != 0 || w13_interleaved;
     if (!x_bf16 || !w13 || !w13_scales || !w2 || !w2_scales || !topk_w || !sorted_slots || !expert_offsets ||
         !slot_to_pos || !y_bf16)
         return HK_ERR_NULL_POINTER;
@@ -1062,7 +1123,11 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
     p.items = (const MoeItem*)(ws + L.items1); p.num_items = nitems;
     p.out0 = ws + L.hq; p.out_scales = ws + L.hs;
     p.K = H; p.N = I; p.n_tiles_n = (I + 127) / 128;
-    st = weight_layout ? launch_moe_stream<0>(p, L.max_items1, s) : launch_moe_gemm<0>(p, L.max_items1, s);
+    p.bias = bias13; p.act = activation; p.alpha = alpha; p.limit = limit; p.interleaved = w13_interleaved != 0;
+    if (ext)
+        st = weight_layout ? launch_moe_stream<0, true>(p, L.max_items1, s) : launch_moe_gemm<0, true>(p, L.max_items1, s);
+    else
+        st = weight_layout ? launch_moe_stream<0, false>(p, L.max_items1, s) : launch_moe_gemm<0, false>(p, L.max_items1, s);
     if (st != HK_OK) return st;
 
     MoeGemmParams q{};
@@ -1077,17 +1142,34 @@ extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const v
     q.items = (const MoeItem*)(ws + L.items2); q.num_items = nitems + 1;
     q.out0 = ws + L.o; q.out_scales = nullptr;
     q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
-    st = weight_layout ? launch_moe_stream<1>(q, L.max_items2, s) : launch_moe_gemm<1>(q, L.max_items2, s);
+    q.bias = bias2;
+    if (bias2)
+        st = weight_layout ? launch_moe_stream<1, true>(q, L.max_items2, s) : launch_moe_gemm<1, true>(q, L.max_items2, s);
+    else
+        st = weight_layout ? launch_moe_stream<1, false>(q, L.max_items2, s) : launch_moe_gemm<1, false>(q, L.max_items2, s);
     if (st != HK_OK) return st;
 
     return hk_moe_unpermute(ws + L.o, topk_w, slot_to_pos, T, k, H, y_bf16, stream);
 }
 
-extern "C" int hk_moe_mxfp4_forward(const void* x_bf16, const float* router_logits, const void* w13,
-                                    const void* w13_scales, int w13_scale_pitch, const void* w2,
-                                    const void* w2_scales, int w2_scale_pitch, void* y_bf16, int T, int H, int I,
-                                    int E, int k, int weight_layout, void* workspace, size_t workspace_bytes,
-                                    void* stream) {
+extern "C" int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const void* w13_scales,
+                                    int w13_scale_pitch, const void* w2, const void* w2_scales,
+                                    int w2_scale_pitch, const float* topk_w, const int32_t* sorted_slots,
+                                    const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
+                                    int T, int H, int I, int E, int k, int weight_layout, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+    return hk_moe_mxfp4_experts_ex(x_bf16, w13, w13_scales, w13_scale_pitch, w2, w2_scales, w2_scale_pitch, topk_w,
+                                   sorted_slots, expert_offsets, slot_to_pos, y_bf16, T, H, I, E, k, weight_layout,
+                                   nullptr, nullptr, 0, 0.f, 0.f, 0, workspace, workspace_bytes, stream);
+}
+
+extern "C" int hk_moe_mxfp4_forward_ex(const void* x_bf16, const float* router_logits, const void* w13,
+                                       const void* w13_scales, int w13_scale_pitch, const void* w2,
+                                       const void* w2_scales, int w2_scale_pitch, void* y_bf16, int T, int H,
+                                       int I, int E, int k, int weight_layout, const float* bias13,
+                                       const float* bias2, int activation, float alpha, float limit,
+                                       int w13_interleaved, void* workspace, size_t workspace_bytes,
+                                       void* stream) {
     if (!router_logits) return HK_ERR_NULL_POINTER;
     if (weight_layout != 0 && weight_layout != 1) return HK_ERR_UNSUPPORTED;
     int st = moe_mxfp4_check(T, H, I, E, k, weight_layout ? moe_round_up(H / 32, 8) : w13_scale_pitch,
@@ -1101,8 +1183,19 @@ extern "C" int hk_moe_mxfp4_forward(const void* x_bf16, const float* router_logi
     st = hk_moe_sort((const int32_t*)(ws + L.ids), T, k, E, (int32_t*)(ws + L.sorted), (int32_t*)(ws + L.offsets),
                      (int32_t*)(ws + L.inv), ws + L.sort_ws, hk_moe_sort_workspace_bytes(T, k, E), stream);
     if (st != HK_OK) return st;
-    return hk_moe_mxfp4_experts(x_bf16, w13, w13_scales, w13_scale_pitch, w2, w2_scales, w2_scale_pitch,
-                                (const float*)(ws + L.w), (const int32_t*)(ws + L.sorted),
-                                (const int32_t*)(ws + L.offsets), (const int32_t*)(ws + L.inv), y_bf16, T, H, I, E,
-                                k, weight_layout, workspace, workspace_bytes, stream);
+    return hk_moe_mxfp4_experts_ex(x_bf16, w13, w13_scales, w13_scale_pitch, w2, w2_scales, w2_scale_pitch,
+                                   (const float*)(ws + L.w), (const int32_t*)(ws + L.sorted),
+                                   (const int32_t*)(ws + L.offsets), (const int32_t*)(ws + L.inv), y_bf16, T, H, I,
+                                   E, k, weight_layout, bias13, bias2, activation, alpha, limit, w13_interleaved,
+                                   workspace, workspace_bytes, stream);
+}
+
+extern "C" int hk_moe_mxfp4_forward(const void* x_bf16, const float* router_logits, const void* w13,
+                                    const void* w13_scales, int w13_scale_pitch, const void* w2,
+                                    const void* w2_scales, int w2_scale_pitch, void* y_bf16, int T, int H, int I,
+                                    int E, int k, int weight_layout, void* workspace, size_t workspace_bytes,
+                                    void* stream) {
+    return hk_moe_mxfp4_forward_ex(x_bf16, router_logits, w13, w13_scales, w13_scale_pitch, w2, w2_scales,
+                                   w2_scale_pitch, y_bf16, T, H, I, E, k, weight_layout, nullptr, nullptr, 0, 0.f,
+                                   0.f, 0, workspace, workspace_bytes, stream);
 }

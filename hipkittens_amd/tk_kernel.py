@@ -221,9 +221,10 @@ class MoeMxfp4ShuffledWeights:
     """Expert weights in the pre-shuffled tile layout (hk_moe_mxfp4_preshuffle): built once,
     offline, from the plain [E, rows, K/2] + [E, rows, K/32] tensors."""
 
-    def __init__(self, w13, w13_scales, w2, w2_scales, E: int, H: int, I: int):
+    def __init__(self, w13, w13_scales, w2, w2_scales, E: int, H: int, I: int, interleaved: bool = False):
         self.w13, self.w13_scales, self.w2, self.w2_scales = w13, w13_scales, w2, w2_scales
         self.E, self.H, self.I = E, H, I
+        self.interleaved = bool(interleaved)  # row order of the source w13 (and of a bias13 given later)
 
     @staticmethod
     def _shuffle(w, scales, N: int, K: int, mode: int):
@@ -241,7 +242,9 @@ class MoeMxfp4ShuffledWeights:
         return out_w, out_s
 
     @classmethod
-    def from_plain(cls, w13, w13_scales, w2, w2_scales):
+    def from_plain(cls, w13, w13_scales, w2, w2_scales, interleaved: bool = False):
+        """`interleaved`: rows 2c / 2c+1 of w13 are gate / up of column c (GPT-OSS checkpoints)
+        instead of rows c / I+c."""
         _check_tensor(w13, "w13", _FP4, 3)
         _check_tensor(w13_scales, "w13_scales", _E8M0, 3)
         _check_tensor(w2, "w2", _FP4, 3)
@@ -251,9 +254,9 @@ class MoeMxfp4ShuffledWeights:
         if tuple(w2.shape) != (E, H, I // 2) or tuple(w13_scales.shape[:2]) != (E, twoI) or \
                 tuple(w2_scales.shape[:2]) != (E, H) or w13_scales.shape[2] < H // 32 or w2_scales.shape[2] < I // 32:
             raise RuntimeError("shape mismatch between w13, w13_scales, w2 and w2_scales")
-        a, sa = cls._shuffle(w13, w13_scales, I, H, 0)
+        a, sa = cls._shuffle(w13, w13_scales, I, H, 2 if interleaved else 0)
         b, sb = cls._shuffle(w2, w2_scales, H, I, 1)
-        return cls(a, sa, b, sb, E, H, I)
+        return cls(a, sa, b, sb, E, H, I, interleaved)
 
 
 def _moe_weight_args(x, weights_or_w13, w13_scales, w2, w2_scales, y):
@@ -288,11 +291,38 @@ def _check_moe_weights(x, w13, w13_scales, w2, w2_scales, y):
     return T, H, I, E
 
 
+_ACTIVATIONS = {"silu": 0, "swiglu_oai": 1}
+
+
+def _moe_ext_args(w13, E, H, I, bias13, bias2, activation, interleaved):
+    """-> (bias13_ptr, bias2_ptr, activation code, interleaved flag) of the extended entry points."""
+    if activation not in _ACTIVATIONS:
+        raise RuntimeError(f"activation must be one of {sorted(_ACTIVATIONS)}")
+    if isinstance(w13, MoeMxfp4ShuffledWeights):
+        if interleaved is not None and bool(interleaved) != w13.interleaved:
+            raise RuntimeError("interleaved does not match the layout the weights were shuffled from")
+        interleaved = w13.interleaved
+    if bias13 is not None:
+        _check_tensor(bias13, "bias13", _F32, 2)
+        if tuple(bias13.shape) != (E, 2 * I):
+            raise RuntimeError("bias13 must be [E, 2I]")
+    if bias2 is not None:
+        _check_tensor(bias2, "bias2", _F32, 2)
+        if tuple(bias2.shape) != (E, H):
+            raise RuntimeError("bias2 must be [E, H]")
+    return (bias13.data_ptr() if bias13 is not None else None, bias2.data_ptr() if bias2 is not None else None,
+            _ACTIVATIONS[activation], 1 if interleaved else 0)
+
+
 def dispatch_moe_mxfp4_experts(x, w13, w13_scales, w2, w2_scales, weights, sorted_slots, expert_offsets,
-                               slot_to_pos, y, workspace) -> None:
-    """Expert MLP on routed + sorted tokens (see include/hk355.h: hk_moe_mxfp4_experts). `w13` may be
-    a MoeMxfp4ShuffledWeights, in which case w13_scales, w2 and w2_scales are ignored (pass None)."""
+                               slot_to_pos, y, workspace, bias13=None, bias2=None, activation: str = "silu",
+                               alpha: float = 1.702, limit: float = 7.0, interleaved=None) -> None:
+    """Expert MLP on routed + sorted tokens (see include/hk355.h: hk_moe_mxfp4_experts_ex). `w13` may be
+    a MoeMxfp4ShuffledWeights, in which case w13_scales, w2 and w2_scales are ignored (pass None).
+    Model-faithful options: bias13 [E, 2I] / bias2 [E, H] fp32, activation "swiglu_oai" (clamped
+    SwiGLU with alpha and limit), interleaved gate / up rows of w13 and bias13."""
     T, H, I, E, layout, pw13, ps13, pitch13, pw2, ps2, pitch2 = _moe_weight_args(x, w13, w13_scales, w2, w2_scales, y)
+    pb13, pb2, act, inter = _moe_ext_args(w13, E, H, I, bias13, bias2, activation, interleaved)
     _check_tensor(weights, "weights", _F32, 2)
     _check_tensor(sorted_slots, "sorted_slots", _I32, 1)
     _check_tensor(expert_offsets, "expert_offsets", _I32, 1)
@@ -302,24 +332,29 @@ def dispatch_moe_mxfp4_experts(x, w13, w13_scales, w2, w2_scales, weights, sorte
     if weights.shape[0] != T or sorted_slots.shape[0] != T * k or expert_offsets.shape[0] != E + 1 or \
             slot_to_pos.shape[0] != T * k:
         raise RuntimeError("shape mismatch between routing tensors")
-    st = _lib.load_library().hk_moe_mxfp4_experts(
+    st = _lib.load_library().hk_moe_mxfp4_experts_ex(
         x.data_ptr(), pw13, ps13, pitch13, pw2, ps2, pitch2, weights.data_ptr(), sorted_slots.data_ptr(),
         expert_offsets.data_ptr(), slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, layout,
-        workspace.data_ptr(), workspace.numel(), _stream(x))
+        pb13, pb2, act, float(alpha), float(limit), inter, workspace.data_ptr(), workspace.numel(), _stream(x))
     _lib.check(st, "dispatch_moe_mxfp4_experts")
 
 
-def dispatch_moe_mxfp4(x, router_logits, w13, w13_scales, w2, w2_scales, y, topk: int, workspace) -> None:
+def dispatch_moe_mxfp4(x, router_logits, w13, w13_scales, w2, w2_scales, y, topk: int, workspace,
+                       bias13=None, bias2=None, activation: str = "silu", alpha: float = 1.702,
+                       limit: float = 7.0, interleaved=None) -> None:
     """Whole MXFP4 MoE layer: top-k softmax routing, sort, expert MLP, un-permute into y. `w13` may be
-    a MoeMxfp4ShuffledWeights (then pass None for w13_scales, w2, w2_scales)."""
+    a MoeMxfp4ShuffledWeights (then pass None for w13_scales, w2, w2_scales). Options as in
+    dispatch_moe_mxfp4_experts."""
     T, H, I, E, layout, pw13, ps13, pitch13, pw2, ps2, pitch2 = _moe_weight_args(x, w13, w13_scales, w2, w2_scales, y)
+    pb13, pb2, act, inter = _moe_ext_args(w13, E, H, I, bias13, bias2, activation, interleaved)
     _check_tensor(router_logits, "router_logits", _F32, 2)
     _check_tensor(workspace, "workspace", (torch.uint8,), 1)
     if tuple(router_logits.shape) != (T, E):
         raise RuntimeError("router_logits must be [T, E]")
-    st = _lib.load_library().hk_moe_mxfp4_forward(
+    st = _lib.load_library().hk_moe_mxfp4_forward_ex(
         x.data_ptr(), router_logits.data_ptr(), pw13, ps13, pitch13, pw2, ps2, pitch2, y.data_ptr(), T, H, I, E,
-        int(topk), layout, workspace.data_ptr(), workspace.numel(), _stream(x))
+        int(topk), layout, pb13, pb2, act, float(alpha), float(limit), inter, workspace.data_ptr(),
+        workspace.numel(), _stream(x))
     _lib.check(st, "dispatch_moe_mxfp4")
 
 

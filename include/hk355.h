@@ -154,7 +154,8 @@ size_t hk_moe_mxfp4_workspace_bytes(int T, int H, int I, int E, int k);
  * 256 x 128-byte weight tile is stored contiguously in the order the kernel keeps it in LDS
  * (K zero-padded to whole 256-element steps), scales likewise as 256 x 8-byte tiles, so that the
  * GEMMs stream weights from HBM in 32 KiB bursts. mode 0: gate+up matrix [E, 2N, K/2] with N = I,
- * K = H; mode 1: down matrix [E, N, K/2] with N = H, K = I. scales [E, rows, scale_pitch]. */
+ * K = H; mode 1: down matrix [E, N, K/2] with N = H, K = I; mode 2: as mode 0 for a source with
+ * interleaved gate / up rows (2c / 2c + 1), same output format. scales [E, rows, scale_pitch]. */
 int hk_moe_mxfp4_preshuffle_bytes(int E, int N, int K, int mode, size_t* w_bytes, size_t* s_bytes);
 int hk_moe_mxfp4_preshuffle(const void* w, const void* scales, int scale_pitch, int E, int N, int K,
                             int mode, void* out_w, void* out_s, void* stream);
@@ -177,6 +178,30 @@ int hk_moe_mxfp4_forward(const void* x_bf16, const float* router_logits, const v
                          const void* w2_scales, int w2_scale_pitch, void* y_bf16, int T, int H, int I,
                          int E, int k, int weight_layout, void* workspace, size_t workspace_bytes,
                          void* stream);
+
+/* Model-faithful variants of the two entry points above (no counterpart in the reference; the
+ * formulas follow the published GPT-OSS model code):
+ *   bias13 [E, 2I] fp32 or NULL: added to the gate+up GEMM result before the activation
+ *   bias2  [E, H]  fp32 or NULL: added to the down GEMM result before the weighted sum
+ *   activation 0: silu(gate) * up; 1: clamped SwiGLU, g = min(gate, limit), u = clamp(up, +-limit),
+ *              h = (u + 1) * g * sigmoid(alpha * g)   (GPT-OSS: alpha 1.702, limit 7)
+ *   w13_interleaved != 0: gate / up of h column c are rows 2c / 2c + 1 of w13, w13_scales and
+ *              bias13 instead of rows c / I + c. With weight_layout 1 the weights must have been
+ *              shuffled with mode 2 (hk_moe_mxfp4_preshuffle), which reads that row order.
+ * With all options off they run the same kernels as the plain entry points. */
+int hk_moe_mxfp4_experts_ex(const void* x_bf16, const void* w13, const void* w13_scales,
+                            int w13_scale_pitch, const void* w2, const void* w2_scales,
+                            int w2_scale_pitch, const float* topk_w, const int32_t* sorted_slots,
+                            const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
+                            int T, int H, int I, int E, int k, int weight_layout, const float* bias13,
+                            const float* bias2, int activation, float alpha, float limit,
+                            int w13_interleaved, void* workspace, size_t workspace_bytes, void* stream);
+int hk_moe_mxfp4_forward_ex(const void* x_bf16, const float* router_logits, const void* w13,
+                            const void* w13_scales, int w13_scale_pitch, const void* w2,
+                            const void* w2_scales, int w2_scale_pitch, void* y_bf16, int T, int H, int I,
+                            int E, int k, int weight_layout, const float* bias13, const float* bias2,
+                            int activation, float alpha, float limit, int w13_interleaved,
+                            void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------- FP8 block-scaled fused MoE
  * No counterpart in the reference. DeepSeek-V3 style quantization:

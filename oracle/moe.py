@@ -118,10 +118,27 @@ def quantize_act_mxfp4(x: np.ndarray):
     return F.quantize_mxfp4(x)
 
 
-def moe_mxfp4_forward(x_bf16_as_f32, ids, w, w13_packed, w13_scales, w2_packed, w2_scales):
+def swiglu_clamped(gate, up, alpha: float, limit: float):
+    """The gated activation of the GPT-OSS experts (published model code: gate clamped from above,
+    up clamped to [-limit, limit], glu = gate * sigmoid(alpha * gate), result (up + 1) * glu).
+    No counterpart in the reference repository; evaluated in float64, rounded once to fp32."""
+    g = np.minimum(np.asarray(gate, dtype=np.float32), np.float32(limit))
+    u = np.clip(np.asarray(up, dtype=np.float32), np.float32(-limit), np.float32(limit))
+    glu = g.astype(np.float64) / (1.0 + np.exp(-float(alpha) * g.astype(np.float64)))
+    return ((u.astype(np.float64) + 1.0) * glu).astype(np.float32)
+
+
+def moe_mxfp4_forward(x_bf16_as_f32, ids, w, w13_packed, w13_scales, w2_packed, w2_scales,
+                      bias13=None, bias2=None, activation: str = "silu", alpha: float = 1.702,
+                      limit: float = 7.0, interleaved: bool = False):
     """Reference forward of the MXFP4 MoE. x [T,H] (bf16 values as fp32); ids/w [T,k];
     w13_packed [E, 2I, H/2], w13_scales [E, 2I, H/32]; w2_packed [E, H, I/2], w2_scales
-    [E, H, I/32]. Returns (y as bf16 bits [T,H], dict of intermediates)."""
+    [E, H, I/32]. Returns (y as bf16 bits [T,H], dict of intermediates).
+
+    Model-faithful options (GPT-OSS): bias13 [E, 2I] / bias2 [E, H] fp32 added to the GEMM
+    results before the activation / before the weighted sum; activation "swiglu_oai" =
+    swiglu_clamped; interleaved: rows 2i / 2i+1 of w13 (and of bias13) are gate / up of column i
+    instead of rows i / I+i."""
     T, H = x_bf16_as_f32.shape
     E, twoI, _ = w13_packed.shape
     I = twoI // 2
@@ -140,11 +157,21 @@ def moe_mxfp4_forward(x_bf16_as_f32, ids, w, w13_packed, w13_scales, w2_packed, 
         tok = order[lo:hi] // k
         w13 = F.dequantize_mxfp4(w13_packed[e], w13_scales[e])
         gu = xd[tok] @ w13.T
-        h = (silu(gu[:, :I]) * gu[:, I:]).astype(np.float32)
+        if bias13 is not None:
+            gu = gu + np.asarray(bias13[e], dtype=np.float32)[None, :]
+        gate, up = (gu[:, 0::2], gu[:, 1::2]) if interleaved else (gu[:, :I], gu[:, I:])
+        if activation == "silu":
+            h = (silu(gate) * up).astype(np.float32)
+        elif activation == "swiglu_oai":
+            h = swiglu_clamped(gate, up, alpha, limit)
+        else:
+            raise ValueError(activation)
         q, s = quantize_act_mxfp4(h)
         hq[lo:hi], hs[lo:hi] = q, s
         w2 = F.dequantize_mxfp4(w2_packed[e], w2_scales[e])
         o[lo:hi] = F.dequantize_mxfp4(q, s) @ w2.T
+        if bias2 is not None:
+            o[lo:hi] += np.asarray(bias2[e], dtype=np.float32)[None, :]
     o_bf = F.bf16_to_f32(F.bf16_round(o))
     y = np.zeros((T, H), dtype=np.float32)
     for j in range(k):

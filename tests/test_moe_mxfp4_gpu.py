@@ -118,6 +118,94 @@ def test_moe_mxfp4_forward_matches_oracle(hk, T, E, k, H, I):
     assert err <= TOL, err
 
 
+def _interleave_rows(a, I):
+    """[E, 2I, ...] with gate rows 0..I-1 / up rows I..2I-1 -> rows 2c / 2c+1 = gate / up of column c."""
+    perm = np.empty(2 * I, dtype=np.int64)
+    perm[0::2], perm[1::2] = np.arange(I), I + np.arange(I)
+    return np.ascontiguousarray(a[:, perm])
+
+
+OPTION_CASES = [
+    # T, E, k, H, I, biases, activation, interleaved
+    (64, 4, 2, 256, 128, True, "swiglu_oai", True),     # everything at once (GPT-OSS experts)
+    (64, 4, 2, 256, 128, True, "silu", False),          # biases alone
+    (64, 4, 2, 256, 128, False, "swiglu_oai", False),   # activation alone
+    (64, 4, 2, 256, 128, False, "silu", True),          # row order alone
+    (300, 8, 2, 512, 384, True, "swiglu_oai", True),    # several m-tiles per expert, ragged tiles
+    (200, 16, 4, 2880, 320, True, "swiglu_oai", True),  # K tail; I not a multiple of 128
+    (96, 128, 4, 288, 160, True, "swiglu_oai", False),  # many experts, some empty
+]
+
+
+@pytest.mark.parametrize("T,E,k,H,I,biases,activation,interleaved", OPTION_CASES)
+def test_moe_mxfp4_model_faithful_options_match_oracle(hk, T, E, k, H, I, biases, activation, interleaved):
+    """Biases, clamped SwiGLU (alpha 1.702, limit 7) and interleaved gate / up rows, with plain and
+    with pre-shuffled weights (bit-identical), against the oracle. Gate values are scaled so that
+    a good part of them reaches the clamp."""
+    print(f"moe_mxfp4 options T={T} E={E} k={k} H={H} I={I} {biases} {activation} {interleaved}", flush=True)
+    rng = np.random.default_rng(T + E + H + 17)
+    x = _bf16(rng.standard_normal((T, H)))
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    w13p, w13s, w2p, w2s = _weights(rng, E, I, H, std=0.35)
+    b13 = (rng.standard_normal((E, 2 * I)) * 2).astype(np.float32) if biases else None
+    b2 = rng.standard_normal((E, H)).astype(np.float32) if biases else None
+    ids, w = O.topk_softmax(logits, k)
+    want_bits, inter = O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s, bias13=b13, bias2=b2,
+                                           activation=activation)
+    want = F.bf16_to_f32(want_bits)
+    if activation == "swiglu_oai":  # the clamp must matter in this test
+        gu = F.dequantize_mxfp4(*F.quantize_mxfp4(x))[:8] @ F.dequantize_mxfp4(w13p[0], w13s[0]).T
+        assert (np.abs(gu) > 7.0).mean() > 0.01
+
+    # device tensors in the caller's row order
+    g13p, g13s, gb13 = w13p, w13s, b13
+    if interleaved:
+        g13p, g13s = _interleave_rows(w13p, I), _interleave_rows(w13s, I)
+        gb13 = _interleave_rows(b13, I) if biases else None
+    tw = [torch.from_numpy(g13p).to(DEV), torch.from_numpy(_pad(g13s)).to(DEV), torch.from_numpy(w2p).to(DEV),
+          torch.from_numpy(_pad(w2s)).to(DEV)]
+    opts = dict(bias13=torch.from_numpy(gb13).to(DEV) if biases else None,
+                bias2=torch.from_numpy(b2).to(DEV) if biases else None, activation=activation,
+                alpha=1.702, limit=7.0)
+    ws = torch.empty(hk.tk_kernel.moe_mxfp4_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=DEV)
+    xt, lt = _to_bf16_tensor(x), torch.from_numpy(logits).to(DEV)
+    y = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_mxfp4(xt, lt, tw[0], tw[1], tw[2], tw[3], y, k, ws, interleaved=interleaved, **opts)
+    torch.cuda.synchronize()
+    shuf = hk.tk_kernel.MoeMxfp4ShuffledWeights.from_plain(*tw, interleaved=interleaved)
+    y2 = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_mxfp4(xt, lt, shuf, None, None, None, y2, k, ws, **opts)
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16)), "plain and pre-shuffled weights disagree"
+    got = y.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    err = G.rel_fro_error(got, want)
+    assert err <= TOL, err
+
+
+def test_moe_mxfp4_options_bad_arguments(hk):
+    T, E, k, H, I = 16, 4, 2, 64, 32
+    rng = np.random.default_rng(0)
+    w13p, w13s, w2p, w2s = _weights(rng, E, I, H)
+    tw = [torch.from_numpy(w13p).to(DEV), torch.from_numpy(_pad(w13s)).to(DEV), torch.from_numpy(w2p).to(DEV),
+          torch.from_numpy(_pad(w2s)).to(DEV)]
+    ws = torch.empty(hk.tk_kernel.moe_mxfp4_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=DEV)
+    x = torch.zeros((T, H), dtype=torch.bfloat16, device=DEV)
+    lt = torch.zeros((T, E), dtype=torch.float32, device=DEV)
+    y = torch.zeros((T, H), dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError):
+        hk.tk_kernel.dispatch_moe_mxfp4(x, lt, *tw, y, k, ws, activation="gelu")
+    with pytest.raises(RuntimeError):
+        hk.tk_kernel.dispatch_moe_mxfp4(x, lt, *tw, y, k, ws, bias13=torch.zeros((E, I), device=DEV))
+    with pytest.raises(RuntimeError):
+        hk.tk_kernel.dispatch_moe_mxfp4(x, lt, *tw, y, k, ws, bias2=torch.zeros((E, H), dtype=torch.float64, device=DEV))
+    with pytest.raises(RuntimeError):
+        hk.tk_kernel.dispatch_moe_mxfp4(x, lt, *tw, y, k, ws, activation="swiglu_oai", limit=0.0)
+    shuf = hk.tk_kernel.MoeMxfp4ShuffledWeights.from_plain(*tw, interleaved=True)
+    with pytest.raises(RuntimeError):
+        hk.tk_kernel.dispatch_moe_mxfp4(x, lt, shuf, None, None, None, y, k, ws, interleaved=False)
+
+
 def test_moe_mxfp4_skewed_routing_many_rows_per_expert(hk):
     """All tokens on two experts: 2 x 600 rows -> five m-tiles per expert; others empty."""
     rng = np.random.default_rng(5)

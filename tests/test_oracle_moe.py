@@ -2,9 +2,11 @@
 import math
 
 import numpy as np
+import pytest
 import torch
 
 from oracle import formats as F
+from oracle import gemm as G
 from oracle import moe as O
 
 
@@ -154,3 +156,72 @@ def test_moe_fp8blk_forward_single_expert_reduces_to_two_gemms():
     # h may land on a different e4m3 code where fp32 and fp64 accumulation differ by an ulp
     assert np.allclose(got, want, rtol=3e-2, atol=1e-3)
     assert np.linalg.norm(got - want) / np.linalg.norm(want) < 5e-3
+
+
+def _tiny_moe(seed=3, T=12, E=3, k=2, H=64, I=32):
+    rng = np.random.default_rng(seed)
+    x = F.bf16_to_f32(F.bf16_round(rng.standard_normal((T, H)).astype(np.float32)))
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    w13p, w13s = F.quantize_mxfp4((rng.standard_normal((E, 2 * I, H)) * 0.3).astype(np.float32))
+    w2p, w2s = F.quantize_mxfp4((rng.standard_normal((E, H, I)) * 0.3).astype(np.float32))
+    ids, w = O.topk_softmax(logits, k)
+    return rng, x, ids, w, w13p, w13s, w2p, w2s
+
+
+def test_swiglu_clamped_against_torch_and_special_cases():
+    """The clamped SwiGLU against the library routines (torch.clamp, torch.sigmoid) written the
+    way the published model code writes it, plus the cases the formula fixes: above the limit
+    the gate saturates, up is clamped on both sides, gate 0 gives 0, and with alpha 1 and no
+    clamping it is silu(gate) * (up + 1)."""
+    rng = np.random.default_rng(0)
+    g = (rng.standard_normal(4096) * 5).astype(np.float32)
+    u = (rng.standard_normal(4096) * 5).astype(np.float32)
+    alpha, limit = 1.702, 7.0
+    tg, tu = torch.from_numpy(g).double(), torch.from_numpy(u).double()
+    tg = tg.clamp(max=limit)
+    tu = tu.clamp(min=-limit, max=limit)
+    want = ((tu + 1) * (tg * torch.sigmoid(tg * alpha))).float().numpy()
+    got = O.swiglu_clamped(g, u, alpha, limit)
+    assert np.allclose(got, want, rtol=1e-6, atol=1e-7)
+    f = np.float32
+    assert O.swiglu_clamped(f(100.0), f(2.0), alpha, limit) == O.swiglu_clamped(f(7.0), f(2.0), alpha, limit)
+    assert O.swiglu_clamped(f(1.0), f(50.0), alpha, limit) == O.swiglu_clamped(f(1.0), f(7.0), alpha, limit)
+    assert O.swiglu_clamped(f(1.0), f(-50.0), alpha, limit) == O.swiglu_clamped(f(1.0), f(-7.0), alpha, limit)
+    assert O.swiglu_clamped(f(0.0), f(3.0), alpha, limit) == 0.0
+    assert O.swiglu_clamped(f(-100.0), f(3.0), alpha, limit) == pytest.approx(0.0, abs=1e-30)
+    assert np.allclose(O.swiglu_clamped(g, u, 1.0, 1e30), O.silu(g) * (u + 1), rtol=1e-6, atol=1e-7)
+
+
+def test_moe_mxfp4_forward_options_reduce_to_the_plain_forward():
+    """Zero biases change nothing; interleaved rows are a pure re-ordering of w13 / bias13; the
+    down bias of a top-1, weight-1 layer is added to the output once; a +1 on the up bias with
+    SiLU is the clamped SwiGLU with alpha 1 and an unreachable limit."""
+    rng, x, ids, w, w13p, w13s, w2p, w2s = _tiny_moe()
+    E, twoI, _ = w13p.shape
+    I, H = twoI // 2, x.shape[1]
+    base, _ = O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s)
+    zero13, zero2 = np.zeros((E, twoI), np.float32), np.zeros((E, H), np.float32)
+    same, _ = O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s, bias13=zero13, bias2=zero2)
+    assert np.array_equal(base, same)
+
+    b13 = rng.standard_normal((E, twoI)).astype(np.float32)
+    b2 = rng.standard_normal((E, H)).astype(np.float32)
+    want, _ = O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s, bias13=b13, bias2=b2, activation="swiglu_oai")
+    perm = np.empty(twoI, dtype=np.int64)      # interleaved row 2c <- gate row c, 2c+1 <- up row I+c
+    perm[0::2], perm[1::2] = np.arange(I), I + np.arange(I)
+    got, _ = O.moe_mxfp4_forward(x, ids, w, w13p[:, perm], w13s[:, perm], w2p, w2s, bias13=b13[:, perm], bias2=b2,
+                                 activation="swiglu_oai", interleaved=True)
+    assert np.array_equal(want, got)
+    assert not np.array_equal(want, base)
+
+    ids1, w1 = ids[:, :1], np.ones((x.shape[0], 1), np.float32)
+    y0 = F.bf16_to_f32(O.moe_mxfp4_forward(x, ids1, w1, w13p, w13s, w2p, w2s)[0])
+    y1 = F.bf16_to_f32(O.moe_mxfp4_forward(x, ids1, w1, w13p, w13s, w2p, w2s, bias2=b2)[0])
+    assert np.allclose(y1 - y0, b2[ids1[:, 0]], atol=2.0 ** -6 * np.maximum(np.abs(y0), np.abs(y1)).max())
+
+    up_plus_one = zero13.copy()
+    up_plus_one[:, I:] = 1.0
+    ya = F.bf16_to_f32(O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s, bias13=up_plus_one)[0])
+    yb = F.bf16_to_f32(O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s, activation="swiglu_oai", alpha=1.0,
+                                           limit=1e30)[0])
+    assert G.rel_fro_error(ya, yb) <= 2e-3  # a last-bit difference in h may flip an MX rounding
