@@ -26,6 +26,8 @@ SIGNATURES = {
                             c_void_p]),
     "hk_mxfp4_quantize_rows": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "hk_moe_unpermute": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "hk_moe_unpermute_add": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p,
+                                     c_void_p]),
     "hk_moe_mxfp4_workspace_bytes": (c_size_t, [c_int] * 5),
     "hk_moe_mxfp4_experts": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
@@ -47,6 +49,10 @@ SIGNATURES = {
     "hk_fp8_quantize_rows_1x128": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "hk_moe_fp8blk_workspace_bytes": (c_size_t, [c_int] * 5),
     "hk_moe_fp8blk_experts": (c_int, [c_void_p] * 11 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p]),
+    "hk_moe_fp8blk_experts_ex": (c_int, [c_void_p] * 11 + [c_int] * 5 + [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hk_moe_fp8blk_forward_ex": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p,
+                                         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                         c_void_p, c_void_p, c_size_t, c_void_p]),
     "hk_moe_fp8blk_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p,
                                       c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                       c_void_p, c_size_t, c_void_p]),

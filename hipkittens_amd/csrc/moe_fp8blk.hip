@@ -389,11 +389,12 @@ extern "C" size_t hk_moe_fp8blk_workspace_bytes(int T, int H, int I, int E, int 
     return fp8_ws_layout(T, H, I, E, k).total;
 }
 
-extern "C" int hk_moe_fp8blk_experts(const void* x_e4m3, const float* x_scales, const void* w13,
-                                     const float* w13_scales, const void* w2, const float* w2_scales,
-                                     const float* topk_w, const int32_t* sorted_slots, const int32_t* expert_offsets,
-                                     const int32_t* slot_to_pos, void* y_bf16, int T, int H, int I, int E, int k,
-                                     void* workspace, size_t workspace_bytes, void* stream) {
+extern "C" int hk_moe_fp8blk_experts_ex(const void* x_e4m3, const float* x_scales, const void* w13,
+                                        const float* w13_scales, const void* w2, const float* w2_scales,
+                                        const float* topk_w, const int32_t* sorted_slots,
+                                        const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
+                                        int T, int H, int I, int E, int k, const void* y_add_bf16_or_null,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
     if (!x_e4m3 || !x_scales || !w13 || !w13_scales || !w2 || !w2_scales || !topk_w || !sorted_slots ||
         !expert_offsets || !slot_to_pos || !y_bf16)
         return HK_ERR_NULL_POINTER;
@@ -434,14 +435,25 @@ extern "C" int hk_moe_fp8blk_experts(const void* x_e4m3, const float* x_scales, 
     q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
     st = launch_fp8blk_gemm<1>(q, L.max_items2, s);
     if (st != HK_OK) return st;
-    return hk_moe_unpermute(ws + L.o, topk_w, slot_to_pos, T, k, H, y_bf16, stream);
+    return hk_moe_unpermute_add(ws + L.o, topk_w, slot_to_pos, T, k, H, y_add_bf16_or_null, y_bf16, stream);
 }
 
-extern "C" int hk_moe_fp8blk_forward(const void* x_e4m3, const float* x_scales, const float* router_logits,
-                                     const float* router_bias_or_null, int n_group, int topk_group,
-                                     float routed_scale, const void* w13, const float* w13_scales, const void* w2,
-                                     const float* w2_scales, void* y_bf16, int T, int H, int I, int E, int k,
+extern "C" int hk_moe_fp8blk_experts(const void* x_e4m3, const float* x_scales, const void* w13,
+                                     const float* w13_scales, const void* w2, const float* w2_scales,
+                                     const float* topk_w, const int32_t* sorted_slots, const int32_t* expert_offsets,
+                                     const int32_t* slot_to_pos, void* y_bf16, int T, int H, int I, int E, int k,
                                      void* workspace, size_t workspace_bytes, void* stream) {
+    return hk_moe_fp8blk_experts_ex(x_e4m3, x_scales, w13, w13_scales, w2, w2_scales, topk_w, sorted_slots,
+                                    expert_offsets, slot_to_pos, y_bf16, T, H, I, E, k, nullptr, workspace,
+                                    workspace_bytes, stream);
+}
+
+extern "C" int hk_moe_fp8blk_forward_ex(const void* x_e4m3, const float* x_scales, const float* router_logits,
+                                        const float* router_bias_or_null, int n_group, int topk_group,
+                                        float routed_scale, const void* w13, const float* w13_scales,
+                                        const void* w2, const float* w2_scales, void* y_bf16, int T, int H, int I,
+                                        int E, int k, const void* y_add_bf16_or_null, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
     if (!router_logits) return HK_ERR_NULL_POINTER;
     int st = fp8blk_check(T, H, I, E, k);
     if (st != HK_OK) return st;
@@ -454,8 +466,18 @@ extern "C" int hk_moe_fp8blk_forward(const void* x_e4m3, const float* x_scales, 
     st = hk_moe_sort((const int32_t*)(ws + L.ids), T, k, E, (int32_t*)(ws + L.sorted), (int32_t*)(ws + L.offsets),
                      (int32_t*)(ws + L.inv), ws + L.sort_ws, hk_moe_sort_workspace_bytes(T, k, E), stream);
     if (st != HK_OK) return st;
-    return hk_moe_fp8blk_experts(x_e4m3, x_scales, w13, w13_scales, w2, w2_scales, (const float*)(ws + L.w),
-                                 (const int32_t*)(ws + L.sorted), (const int32_t*)(ws + L.offsets),
-                                 (const int32_t*)(ws + L.inv), y_bf16, T, H, I, E, k, workspace, workspace_bytes,
-                                 stream);
+    return hk_moe_fp8blk_experts_ex(x_e4m3, x_scales, w13, w13_scales, w2, w2_scales, (const float*)(ws + L.w),
+                                    (const int32_t*)(ws + L.sorted), (const int32_t*)(ws + L.offsets),
+                                    (const int32_t*)(ws + L.inv), y_bf16, T, H, I, E, k, y_add_bf16_or_null,
+                                    workspace, workspace_bytes, stream);
+}
+
+extern "C" int hk_moe_fp8blk_forward(const void* x_e4m3, const float* x_scales, const float* router_logits,
+                                     const float* router_bias_or_null, int n_group, int topk_group,
+                                     float routed_scale, const void* w13, const float* w13_scales, const void* w2,
+                                     const float* w2_scales, void* y_bf16, int T, int H, int I, int E, int k,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+    return hk_moe_fp8blk_forward_ex(x_e4m3, x_scales, router_logits, router_bias_or_null, n_group, topk_group,
+                                    routed_scale, w13, w13_scales, w2, w2_scales, y_bf16, T, H, I, E, k, nullptr,
+                                    workspace, workspace_bytes, stream);
 }

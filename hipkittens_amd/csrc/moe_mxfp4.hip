@@ -896,16 +896,27 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
 }
 
 // ------------------------------------------------------------------------------ un-permute
-// y[t, :] = bf16( sum_j w[t, j] * o[slot_to_pos[t*k + j], :] ), fp32 accumulation in choice order.
+// y[t, :] = bf16( add[t, :] + sum_j w[t, j] * o[slot_to_pos[t*k + j], :] ), fp32 accumulation in
+// choice order starting from add (bf16 [T, H], e.g. a shared expert's output) or from 0 when add
+// is null.
 __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __restrict__ o,
                                                             const float* __restrict__ w,
                                                             const int32_t* __restrict__ slot_to_pos, int T,
-                                                            int k, int H, uint16_t* __restrict__ y) {
+                                                            int k, int H, const uint16_t* __restrict__ add,
+                                                            uint16_t* __restrict__ y) {
     const int t = blockIdx.x;
     for (int c = threadIdx.x; c < H / 8; c += 256) {
         float acc[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+        if (add) {
+            const v4i raw = *(const v4i*)(add + (size_t)t * H + c * 8);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[2 * i] = __uint_as_float((uint32_t)raw[i] << 16);
+                acc[2 * i + 1] = __uint_as_float((uint32_t)raw[i] & 0xffff0000u);
+            }
+        }
         for (int j = 0; j < k; ++j) {
             const int pos = slot_to_pos[(size_t)t * k + j];
             const float wj = w[(size_t)t * k + j];
@@ -992,14 +1003,19 @@ extern "C" int hk_mxfp4_quantize_rows(const void* x_bf16, int rows, int cols, vo
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
-extern "C" int hk_moe_unpermute(const void* o_bf16, const float* w, const int32_t* slot_to_pos, int T, int k,
-                                int H, void* y_bf16, void* stream) {
+extern "C" int hk_moe_unpermute_add(const void* o_bf16, const float* w, const int32_t* slot_to_pos, int T,
+                                    int k, int H, const void* add_bf16_or_null, void* y_bf16, void* stream) {
     if (!o_bf16 || !w || !slot_to_pos || !y_bf16) return HK_ERR_NULL_POINTER;
     if (T <= 0 || k <= 0 || H <= 0 || (H % 8) != 0) return HK_ERR_BAD_SHAPE;
-    if (((uintptr_t)o_bf16 | (uintptr_t)y_bf16) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    if (((uintptr_t)o_bf16 | (uintptr_t)y_bf16 | (uintptr_t)add_bf16_or_null) & 15u) return HK_ERR_BAD_ALIGNMENT;
     hipLaunchKernelGGL(moe_unpermute_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)o_bf16,
-                       w, slot_to_pos, T, k, H, (uint16_t*)y_bf16);
+                       w, slot_to_pos, T, k, H, (const uint16_t*)add_bf16_or_null, (uint16_t*)y_bf16);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
+extern "C" int hk_moe_unpermute(const void* o_bf16, const float* w, const int32_t* slot_to_pos, int T, int k,
+                                int H, void* y_bf16, void* stream) {
+    return hk_moe_unpermute_add(o_bf16, w, slot_to_pos, T, k, H, nullptr, y_bf16, stream);
 }
 
 extern "C" int hk_moe_mxfp4_preshuffle_bytes(int E, int N, int K, int mode, size_t* w_bytes, size_t* s_bytes) {

@@ -198,8 +198,9 @@ def dispatch_mxfp4_quantize_rows(x, packed, scales) -> None:
     _lib.check(st, "dispatch_mxfp4_quantize_rows")
 
 
-def dispatch_moe_unpermute(o, weights, slot_to_pos, y) -> None:
-    """y [T,H] bf16 = sum_j weights[t,j] * o[slot_to_pos[t*k+j]] with o [T*k,H] bf16."""
+def dispatch_moe_unpermute(o, weights, slot_to_pos, y, add=None) -> None:
+    """y [T,H] bf16 = (add [T,H] bf16 if given) + sum_j weights[t,j] * o[slot_to_pos[t*k+j]] with
+    o [T*k,H] bf16."""
     _check_tensor(o, "o", _BF16, 2)
     _check_tensor(weights, "weights", _F32, 2)
     _check_tensor(slot_to_pos, "slot_to_pos", _I32, 1)
@@ -208,8 +209,13 @@ def dispatch_moe_unpermute(o, weights, slot_to_pos, y) -> None:
     H = y.shape[1]
     if tuple(o.shape) != (T * k, H) or y.shape[0] != T or slot_to_pos.shape[0] != T * k:
         raise RuntimeError("shape mismatch between o, weights, slot_to_pos and y")
-    st = _lib.load_library().hk_moe_unpermute(o.data_ptr(), weights.data_ptr(), slot_to_pos.data_ptr(), T, k, H,
-                                              y.data_ptr(), _stream(o))
+    if add is not None:
+        _check_tensor(add, "add", _BF16, 2)
+        if tuple(add.shape) != (T, H):
+            raise RuntimeError("add must be [T, H]")
+    st = _lib.load_library().hk_moe_unpermute_add(o.data_ptr(), weights.data_ptr(), slot_to_pos.data_ptr(), T, k,
+                                                  H, add.data_ptr() if add is not None else None, y.data_ptr(),
+                                                  _stream(o))
     _lib.check(st, "dispatch_moe_unpermute")
 
 
@@ -394,10 +400,21 @@ def _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y):
     return T, H, I, E
 
 
+def _check_y_add(y_add, y):
+    if y_add is None:
+        return None
+    _check_tensor(y_add, "y_add", _BF16, 2)
+    if tuple(y_add.shape) != tuple(y.shape):
+        raise RuntimeError("y_add must have the shape of y")
+    return y_add.data_ptr()
+
+
 def dispatch_moe_fp8blk_experts(x, x_scales, w13, w13_scales, w2, w2_scales, weights, sorted_slots,
-                                expert_offsets, slot_to_pos, y, workspace) -> None:
-    """FP8 block-scaled expert MLP on routed + sorted tokens (include/hk355.h: hk_moe_fp8blk_experts)."""
+                                expert_offsets, slot_to_pos, y, workspace, y_add=None) -> None:
+    """FP8 block-scaled expert MLP on routed + sorted tokens (include/hk355.h: hk_moe_fp8blk_experts_ex).
+    y_add [T,H] bf16: residual added before the output rounding (a shared expert's output)."""
     T, H, I, E = _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y)
+    p_add = _check_y_add(y_add, y)
     _check_tensor(weights, "weights", _F32, 2)
     _check_tensor(sorted_slots, "sorted_slots", _I32, 1)
     _check_tensor(expert_offsets, "expert_offsets", _I32, 1)
@@ -407,26 +424,43 @@ def dispatch_moe_fp8blk_experts(x, x_scales, w13, w13_scales, w2, w2_scales, wei
     if weights.shape[0] != T or sorted_slots.shape[0] != T * k or expert_offsets.shape[0] != E + 1 or \
             slot_to_pos.shape[0] != T * k:
         raise RuntimeError("shape mismatch between routing tensors")
-    st = _lib.load_library().hk_moe_fp8blk_experts(
+    st = _lib.load_library().hk_moe_fp8blk_experts_ex(
         x.data_ptr(), x_scales.data_ptr(), w13.data_ptr(), w13_scales.data_ptr(), w2.data_ptr(),
         w2_scales.data_ptr(), weights.data_ptr(), sorted_slots.data_ptr(), expert_offsets.data_ptr(),
-        slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, workspace.data_ptr(), workspace.numel(), _stream(x))
+        slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, p_add, workspace.data_ptr(), workspace.numel(),
+        _stream(x))
     _lib.check(st, "dispatch_moe_fp8blk_experts")
 
 
+def dispatch_moe_fp8blk_shared_expert(x, x_scales, w13, w13_scales, w2, w2_scales, y, workspace) -> None:
+    """The dense MLP every token passes through (DeepSeek-V3 shared expert): w13 [1, 2I, H],
+    w2 [1, H, I] in the routed experts' format, run as a one-expert layer with identity routing.
+    workspace: moe_fp8blk_workspace_bytes(T, H, I, 1, 1) bytes. Its output is what the routed layer
+    takes as y_add."""
+    T = x.shape[0]
+    ones = torch.ones((T, 1), dtype=torch.float32, device=x.device)
+    ident = torch.arange(T, dtype=torch.int32, device=x.device)
+    offsets = torch.tensor([0, T], dtype=torch.int32, device=x.device)
+    dispatch_moe_fp8blk_experts(x, x_scales, w13, w13_scales, w2, w2_scales, ones, ident, offsets, ident, y,
+                                workspace)
+
+
 def dispatch_moe_fp8blk(x, x_scales, router_logits, router_bias, w13, w13_scales, w2, w2_scales, y, topk: int,
-                        n_group: int, topk_group: int, routed_scale: float, workspace) -> None:
-    """Whole FP8 block-scaled MoE layer with group-limited sigmoid routing."""
+                        n_group: int, topk_group: int, routed_scale: float, workspace, y_add=None) -> None:
+    """Whole FP8 block-scaled MoE layer with group-limited sigmoid routing (router_bias: the
+    selection-only score correction). y_add [T,H] bf16: residual added before the output rounding
+    (dispatch_moe_fp8blk_shared_expert's output)."""
     T, H, I, E = _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y)
+    p_add = _check_y_add(y_add, y)
     _check_tensor(router_logits, "router_logits", _F32, 2)
     if router_bias is not None:
         _check_tensor(router_bias, "router_bias", _F32, 1)
     _check_tensor(workspace, "workspace", (torch.uint8,), 1)
     if tuple(router_logits.shape) != (T, E):
         raise RuntimeError("router_logits must be [T, E]")
-    st = _lib.load_library().hk_moe_fp8blk_forward(
+    st = _lib.load_library().hk_moe_fp8blk_forward_ex(
         x.data_ptr(), x_scales.data_ptr(), router_logits.data_ptr(),
         router_bias.data_ptr() if router_bias is not None else None, int(n_group), int(topk_group),
         float(routed_scale), w13.data_ptr(), w13_scales.data_ptr(), w2.data_ptr(), w2_scales.data_ptr(),
-        y.data_ptr(), T, H, I, E, int(topk), workspace.data_ptr(), workspace.numel(), _stream(x))
+        y.data_ptr(), T, H, I, E, int(topk), p_add, workspace.data_ptr(), workspace.numel(), _stream(x))
     _lib.check(st, "dispatch_moe_fp8blk")

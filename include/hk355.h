@@ -147,6 +147,10 @@ int hk_mxfp4_quantize_rows(const void* x_bf16, int rows, int cols, void* packed,
 /* y[t,:] = bf16(sum_j w[t,j] * o[slot_to_pos[t*k+j], :]), o [T*k, H] bf16. H % 8 == 0. */
 int hk_moe_unpermute(const void* o_bf16, const float* w, const int32_t* slot_to_pos, int T, int k,
                      int H, void* y_bf16, void* stream);
+/* As hk_moe_unpermute with a residual: y[t,:] = bf16(add[t,:] + sum_j ...), add [T, H] bf16 or NULL
+ * (e.g. the output of a shared expert that every token passes through). */
+int hk_moe_unpermute_add(const void* o_bf16, const float* w, const int32_t* slot_to_pos, int T, int k,
+                         int H, const void* add_bf16_or_null, void* y_bf16, void* stream);
 
 size_t hk_moe_mxfp4_workspace_bytes(int T, int H, int I, int E, int k);
 
@@ -235,6 +239,23 @@ int hk_moe_fp8blk_forward(const void* x_e4m3, const float* x_scales, const float
                           float routed_scale, const void* w13, const float* w13_scales, const void* w2,
                           const float* w2_scales, void* y_bf16, int T, int H, int I, int E, int k,
                           void* workspace, size_t workspace_bytes, void* stream);
+
+/* The two entry points above with a residual y_add [T, H] bf16 (or NULL) that is added, in fp32,
+ * to the weighted sum of the routed experts before the single bf16 rounding: the DeepSeek-V3
+ * shared expert. Its output is computed with hk_moe_fp8blk_experts on trivial routing (E = 1,
+ * k = 1, weight 1, identity order), then passed here. y_add may alias y_bf16. */
+int hk_moe_fp8blk_experts_ex(const void* x_e4m3, const float* x_scales, const void* w13,
+                             const float* w13_scales, const void* w2, const float* w2_scales,
+                             const float* topk_w, const int32_t* sorted_slots,
+                             const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
+                             int T, int H, int I, int E, int k, const void* y_add_bf16_or_null,
+                             void* workspace, size_t workspace_bytes, void* stream);
+int hk_moe_fp8blk_forward_ex(const void* x_e4m3, const float* x_scales, const float* router_logits,
+                             const float* router_bias_or_null, int n_group, int topk_group,
+                             float routed_scale, const void* w13, const float* w13_scales,
+                             const void* w2, const float* w2_scales, void* y_bf16, int T, int H, int I,
+                             int E, int k, const void* y_add_bf16_or_null, void* workspace,
+                             size_t workspace_bytes, void* stream);
 
 /* Calibration probe (no counterpart in the reference): runs `blocks` workgroups of 8 waves, each
  * wave `iters` x 32 register-only 16x16x128 MFMAs (fp8 if fp4 == 0, else fp4) on operand bits

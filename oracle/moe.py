@@ -180,11 +180,12 @@ def moe_mxfp4_forward(x_bf16_as_f32, ids, w, w13_packed, w13_scales, w2_packed, 
                              "hq": hq, "hs": hs, "o": o}
 
 
-def moe_fp8blk_forward(x_codes, x_scales, ids, w, w13_codes, w13_scales, w2_codes, w2_scales):
+def moe_fp8blk_forward(x_codes, x_scales, ids, w, w13_codes, w13_scales, w2_codes, w2_scales, y_add=None):
     """Reference forward of the FP8 block-scaled MoE. x_codes [T,H] e4m3 codes with 1x128 scales
     [T,H/128]; w13_codes [E,2I,H] with 128x128 scales [E,2I/128,H/128]; w2_codes [E,H,I] with
     [E,H/128,I/128]. h is re-quantized with 1x128 blocks exactly like the kernel. Returns y as
-    bf16 bits [T,H]."""
+    bf16 bits [T,H]. y_add [T,H] (bf16 values as fp32): residual the weighted sum starts from, e.g.
+    moe_fp8blk_shared_expert's output."""
     T, H = x_codes.shape
     E, twoI, _ = w13_codes.shape
     I = twoI // 2
@@ -205,7 +206,17 @@ def moe_fp8blk_forward(x_codes, x_scales, ids, w, w13_codes, w13_scales, w2_code
         w2 = F.dequantize_e4m3_blocks(w2_codes[e], w2_scales[e], 128, 128)
         o[lo:hi] = F.dequantize_e4m3_blocks(q, s, 1, 128) @ w2.T
     o_bf = F.bf16_to_f32(F.bf16_round(o))
-    y = np.zeros((T, H), dtype=np.float32)
+    y = np.zeros((T, H), dtype=np.float32) if y_add is None else np.array(y_add, dtype=np.float32)
     for j in range(k):
         y += w[:, j:j + 1].astype(np.float32) * o_bf[inv[np.arange(T) * k + j]]
     return F.bf16_round(y)
+
+
+def moe_fp8blk_shared_expert(x_codes, x_scales, w13_codes, w13_scales, w2_codes, w2_scales):
+    """The dense MLP every token passes through (DeepSeek-V3's shared expert): weights shaped
+    [1, 2I, H] / [1, H, I] like one routed expert, every token routed to it with weight 1.
+    Returns bf16 bits [T,H]."""
+    T = x_codes.shape[0]
+    ids = np.zeros((T, 1), dtype=np.int32)
+    return moe_fp8blk_forward(x_codes, x_scales, ids, np.ones((T, 1), np.float32), w13_codes, w13_scales,
+                              w2_codes, w2_scales)

@@ -89,6 +89,55 @@ def test_moe_fp8blk_forward_matches_oracle(hk, T, E, k, G, KG, H, I):
     assert err <= TOL, err
 
 
+@pytest.mark.parametrize("T,E,k,G,KG,H,I,IS", [(64, 8, 2, 4, 2, 256, 128, 256), (200, 32, 8, 8, 4, 1024, 256, 128)])
+def test_moe_fp8blk_with_shared_expert_matches_oracle(hk, T, E, k, G, KG, H, I, IS):
+    """DeepSeek-V3 layer: routed experts (selection-only score bias) + a shared expert of
+    intermediate size IS whose output is the residual of the weighted sum; y_add aliases y."""
+    print(f"moe_fp8blk shared T={T} E={E} k={k} H={H} I={I} IS={IS}", flush=True)
+    rng = np.random.default_rng(T + E + H + I + 1)
+    xq, xs, w13q, w13s, w2q, w2s = _case(rng, T, E, H, I)
+    _, _, s13q, s13s, s2q, s2s = _case(rng, 1, 1, H, IS)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    bias = (rng.standard_normal(E) * 0.05).astype(np.float32)
+    dev = lambda a: torch.from_numpy(a).to(DEV)
+    y = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ws_s = torch.empty(hk.tk_kernel.moe_fp8blk_workspace_bytes(T, H, IS, 1, 1), dtype=torch.uint8, device=DEV)
+    hk.tk_kernel.dispatch_moe_fp8blk_shared_expert(_fp8(xq), dev(xs), _fp8(s13q), dev(s13s), _fp8(s2q), dev(s2s), y, ws_s)
+    torch.cuda.synchronize()
+    shared_want = F.bf16_to_f32(O.moe_fp8blk_shared_expert(xq, xs, s13q, s13s, s2q, s2s))
+    assert GM.rel_fro_error(y.float().cpu().numpy(), shared_want) <= TOL
+    ws = torch.empty(hk.tk_kernel.moe_fp8blk_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=DEV)
+    hk.tk_kernel.dispatch_moe_fp8blk(_fp8(xq), dev(xs), dev(logits), dev(bias), _fp8(w13q), dev(w13s), _fp8(w2q),
+                                     dev(w2s), y, k, G, KG, 2.5, ws, y_add=y)
+    torch.cuda.synchronize()
+    got = y.float().cpu().numpy()
+    ids, w = O.topk_grouped_sigmoid(logits, bias, k, G, KG, 2.5)
+    want = F.bf16_to_f32(O.moe_fp8blk_forward(xq, xs, ids, w, w13q, w13s, w2q, w2s, y_add=shared_want))
+    routed_only = F.bf16_to_f32(O.moe_fp8blk_forward(xq, xs, ids, w, w13q, w13s, w2q, w2s))
+    assert np.isfinite(got).all()
+    assert GM.rel_fro_error(got, want) <= TOL
+    assert GM.rel_fro_error(got, routed_only) > 0.1  # the residual is not a rounding-level effect
+
+
+def test_moe_unpermute_add_is_exact_for_representable_sums(hk):
+    """Small integers: add + sum_j w_j o_j is exact in fp32 and in bf16."""
+    rng = np.random.default_rng(2)
+    T, k, H = 50, 3, 256
+    o = rng.integers(-8, 9, size=(T * k, H)).astype(np.float32)
+    add = rng.integers(-8, 9, size=(T, H)).astype(np.float32)
+    w = rng.integers(1, 4, size=(T, k)).astype(np.float32)
+    inv = rng.permutation(T * k).astype(np.int32)
+    to_bf = lambda a: torch.from_numpy(a).to(DEV).to(torch.bfloat16)
+    y = torch.zeros((T, H), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_unpermute(to_bf(o), torch.from_numpy(w).to(DEV), torch.from_numpy(inv).to(DEV), y,
+                                        add=to_bf(add))
+    torch.cuda.synchronize()
+    want = add.copy()
+    for j in range(k):
+        want += w[:, j:j + 1] * o[inv[np.arange(T) * k + j]]
+    assert np.array_equal(y.float().cpu().numpy(), want)
+
+
 def test_moe_fp8blk_full_width_properties(hk):
     """DeepSeek-V3-like widths (H=7168, I=2048, E=256, k=8, 8 groups / top-4) at a reduced token
     count and expert storage that still fits the test budget: permutation invariance over tokens

@@ -225,3 +225,22 @@ def test_moe_mxfp4_forward_options_reduce_to_the_plain_forward():
     yb = F.bf16_to_f32(O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s, activation="swiglu_oai", alpha=1.0,
                                            limit=1e30)[0])
     assert G.rel_fro_error(ya, yb) <= 2e-3  # a last-bit difference in h may flip an MX rounding
+
+
+def test_moe_fp8blk_shared_expert_and_residual():
+    """The shared expert is the one-expert layer; a zero residual changes nothing; with top-1
+    weight-1 routing onto a copy of the shared expert's weights the layer output is, up to the
+    two bf16 roundings, twice the shared expert's output."""
+    rng = np.random.default_rng(4)
+    T, H, I = 10, 128, 128
+    xq, xs = F.quantize_e4m3_blocks(rng.standard_normal((T, H)).astype(np.float32), 1, 128)
+    w13q, w13s = F.quantize_e4m3_blocks((rng.standard_normal((2 * I, H)) * 0.2).astype(np.float32), 128, 128)
+    w2q, w2s = F.quantize_e4m3_blocks((rng.standard_normal((H, I)) * 0.2).astype(np.float32), 128, 128)
+    w13q, w13s, w2q, w2s = w13q[None], w13s[None], w2q[None], w2s[None]
+    shared = O.moe_fp8blk_shared_expert(xq, xs, w13q, w13s, w2q, w2s)
+    ids, w = np.zeros((T, 1), np.int32), np.ones((T, 1), np.float32)
+    base = O.moe_fp8blk_forward(xq, xs, ids, w, w13q, w13s, w2q, w2s)
+    assert np.array_equal(shared, base)
+    assert np.array_equal(O.moe_fp8blk_forward(xq, xs, ids, w, w13q, w13s, w2q, w2s, y_add=np.zeros((T, H), np.float32)), base)
+    both = F.bf16_to_f32(O.moe_fp8blk_forward(xq, xs, ids, w, w13q, w13s, w2q, w2s, y_add=F.bf16_to_f32(shared)))
+    assert np.array_equal(both, 2 * F.bf16_to_f32(shared))  # doubling is exact in bf16
