@@ -139,6 +139,21 @@ __device__ __forceinline__ v4i scalar_load_x4(const void* p) {
     asm volatile("s_load_dwordx4 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r) : "s"(p) : "memory");
     return r;
 }
+// 16 consecutive floats (four s_load_dwordx4, one wait); same conditions, p 16-byte aligned.
+__device__ __forceinline__ void scalar_load_f16(const float* p, float (&out)[16]) {
+    v4i a, b, c, d;
+    asm volatile(
+        "s_load_dwordx4 %0, %4, 0x0\n\ts_load_dwordx4 %1, %4, 0x10\n\t"
+        "s_load_dwordx4 %2, %4, 0x20\n\ts_load_dwordx4 %3, %4, 0x30\n\ts_waitcnt lgkmcnt(0)"
+        : "=&s"(a), "=&s"(b), "=&s"(c), "=&s"(d) : "s"(p) : "memory");
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        out[i] = __int_as_float(a[i]);
+        out[4 + i] = __int_as_float(b[i]);
+        out[8 + i] = __int_as_float(c[i]);
+        out[12 + i] = __int_as_float(d[i]);
+    }
+}
 __device__ __forceinline__ int scalar_load_x1(const void* p) {
     int r;
     asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r) : "s"(p) : "memory");

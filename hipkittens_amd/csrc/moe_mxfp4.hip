@@ -740,11 +740,21 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
             // lane (r, g) holds, for row 16 m + r, the 8 consecutive columns 32 w + 8 g .. +8
             uint16_t* out = (uint16_t*)p.out0;
             const int col = c.n_tile * 256 + w * 32 + 8 * (int)g;
+            // extended epilogue: the wave's 32 bias values come through the scalar cache (vector
+            // loads here would make the compiler drain the weight prefetch), each lane group picks
+            // its 8. N % 32 == 0: the wave's columns are valid or not as a whole.
             v4f b0 = {0.f, 0.f, 0.f, 0.f}, b1 = {0.f, 0.f, 0.f, 0.f};
-            if (EXT && p.bias && col + 8 <= p.N) {
-                const float* bb = p.bias + (size_t)c.expert * p.N + col;
-                b0 = *(const v4f*)bb;
-                b1 = *(const v4f*)(bb + 4);
+            const int wcol0 = c.n_tile * 256 + w * 32;
+            if (EXT && p.bias && wcol0 < p.N) {
+                float lo[16], hi[16];
+                const float* bb = p.bias + (size_t)c.expert * p.N + wcol0;
+                scalar_load_f16(bb, lo);
+                scalar_load_f16(bb + 16, hi);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    b0[i] = g == 0 ? lo[i] : g == 1 ? lo[8 + i] : g == 2 ? hi[i] : hi[8 + i];
+                    b1[i] = g == 0 ? lo[4 + i] : g == 1 ? lo[12 + i] : g == 2 ? hi[4 + i] : hi[12 + i];
+                }
             }
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
@@ -768,14 +778,22 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
             const int hcol0 = c.n_tile * 128 + 16 * w;  // first of the wave's 16 h columns
             const bool col_ok = hcol0 < p.N;            // N % 32 == 0: a block is valid as a whole
             // extended epilogue: biases of this lane's 4 h columns hcol0 + 4 g .. +4
+            // (through the scalar cache, as above: 16 gate + 16 up values per wave)
             float bg[4] = {0.f, 0.f, 0.f, 0.f}, bu[4] = {0.f, 0.f, 0.f, 0.f};
             if (EXT && p.bias && col_ok) {
                 const float* bb = p.bias + (size_t)c.expert * 2 * p.N;
+                float x0[16], x1[16];   // plain rows: gate / up; interleaved: columns 0-7 / 8-15, gate and up alternating
+                scalar_load_f16(p.interleaved ? bb + 2 * hcol0 : bb + hcol0, x0);
+                scalar_load_f16(p.interleaved ? bb + 2 * hcol0 + 16 : bb + p.N + hcol0, x1);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int hc = hcol0 + 4 * (int)g + j;
-                    bg[j] = bb[p.interleaved ? 2 * hc : hc];
-                    bu[j] = bb[p.interleaved ? 2 * hc + 1 : p.N + hc];
+                    const float pg = g == 0 ? x0[j] : g == 1 ? x0[4 + j] : g == 2 ? x0[8 + j] : x0[12 + j];
+                    const float pu = g == 0 ? x1[j] : g == 1 ? x1[4 + j] : g == 2 ? x1[8 + j] : x1[12 + j];
+                    // interleaved: lane group g's columns 4 g + j sit at floats 8 g + 2 j (+ 1) of the 32
+                    const float ig = g == 0 ? x0[2 * j] : g == 1 ? x0[8 + 2 * j] : g == 2 ? x1[2 * j] : x1[8 + 2 * j];
+                    const float iu = g == 0 ? x0[2 * j + 1] : g == 1 ? x0[9 + 2 * j] : g == 2 ? x1[2 * j + 1] : x1[9 + 2 * j];
+                    bg[j] = p.interleaved ? ig : pg;
+                    bu[j] = p.interleaved ? iu : pu;
                 }
             }
             // two groups of six fragments, to keep the number of live h values small
