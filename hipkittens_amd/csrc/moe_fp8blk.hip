@@ -94,24 +94,12 @@ struct MoeFp8Params {
     int K, N, S, n_tiles_n;
 };
 
-// Item height BM (rows of an expert per work item) and LDS plan. The K-step is bound by LDS read
-// bandwidth (128 B/clk per CU), not by the MFMA pipe: with 128-row items every fragment a wave
-// reads feeds 2 MFMAs, with 192 rows 2.4, with 256 rows 2.7. Activation tiles (L2 resident,
-// shared by the n-tiles of an expert) get two stages. Weight tiles come from HBM, every byte
-// exactly once: BM = 192 leaves room for a three-slot weight ring, so that two weight tiles are
-// in flight (best when experts have few rows and the kernel is a weight stream); BM = 256 only
-// for two slots, one tile in flight (best when experts have about 256 rows or more).
-template <int BM>
-struct F8Geo {
-    static constexpr int kATile = BM * 128;
-    static constexpr int kBTile = 256 * 128;                // 32 KiB
-    static constexpr int kBSlots = BM <= 192 ? 3 : 2;
-    static constexpr int kBBase = 2 * kATile;               // B ring behind the two A stages
-    static constexpr int kScaleBase = kBBase + kBSlots * kBTile;   // A scales: BM floats per A stage
-    static constexpr int kXchBase = kScaleBase + 2 * BM * 4;       // epilogue exchange: BM x 4 floats
-    static constexpr int kLds = kXchBase + BM * 16;
-    static_assert(kLds <= 160 * 1024, "LDS plan");
-};
+constexpr int kF8ATile = kMoeBM * 128;             // 16 KiB
+constexpr int kF8BTile = 256 * 128;                // 32 KiB
+constexpr int kF8Stage = kF8ATile + kF8BTile;      // 48 KiB
+constexpr int kF8ScaleBase = 3 * kF8Stage;         // A scales: 3 stages x kMoeBM floats
+constexpr int kF8XchBase = kF8ScaleBase + 3 * kMoeBM * 4;  // epilogue exchange: kMoeBM x 4 floats
+constexpr int kF8Lds = kF8XchBase + kMoeBM * 16;
 
 // dword global->LDS load restricted to the lanes in `mask` (lane l lands at lds_base + 4*l)
 __device__ __forceinline__ void dma4_lanes(v4i srd, uint32_t lds_base, uint32_t voff, uint32_t soff,
@@ -138,13 +126,10 @@ struct MoeFp8Addr {
     bool valid;
 };
 
-template <int MODE, int BM>
+template <int MODE>
 __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params p) {
-    using Geo = F8Geo<BM>;
-    constexpr int kF8BM = BM, kF8ATile = Geo::kATile, kF8BTile = Geo::kBTile, kF8BBase = Geo::kBBase;
-    constexpr int kF8ScaleBase = Geo::kScaleBase, kF8XchBase = Geo::kXchBase, kBSlots = Geo::kBSlots;
-    constexpr int NW = 8, MT = kF8BM / 32, NT = 4, NA = kF8BM / 64;
-    constexpr int kDmaA = NA + 1, kDmaB = 4, kDma = kDmaA + kDmaB;   // loads per wave and position
+    constexpr int NW = 8, MT = kMoeBM / 32, NT = 4, NA = kMoeBM / 64;
+    constexpr int kDma = NA + 4 + 1;
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
     const int lane = lane_id(), w = wave_id();
     const int wm = w >> 2, wn = w & 3;
@@ -163,7 +148,7 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
     const v4i srd_sa = make_srd(p.SA, (uint32_t)nk * (uint32_t)p.S * 4u);
     const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);
 
-    auto make_addr = [&](int idx, MoeFp8Addr& a) __attribute__((always_inline)) {
+    auto make_addr = [&](int idx, MoeFp8Addr& a) {
         a.valid = idx < it_end;
         if (!a.valid) idx = it_end - 1;
         const v4i item = scalar_load_x4(p.items + idx);
@@ -189,114 +174,69 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-    const uint32_t lds_sa_wave = to_sgpr(lds0 + kF8ScaleBase + (uint32_t)w * (kF8BM / 8) * 4u);
+    const uint32_t lds_sa_wave = to_sgpr(lds0 + kF8ScaleBase + (uint32_t)w * (kMoeBM / 8) * 4u);
     uint32_t voff_a[NA];
 #pragma unroll
     for (int i = 0; i < NA; ++i) voff_a[i] = (uint32_t)(8 * (i * NW + w) + (lane >> 3)) * 128u + chunk16 * 16u;
-    const uint32_t voff_sa = (uint32_t)((w * (kF8BM / 8) + lane) * 4);
-    constexpr uint64_t kSaMask = (1ull << (kF8BM / 8)) - 1ull;
+    const uint32_t voff_sa = (uint32_t)((w * (kMoeBM / 8) + lane) * 4);
+    constexpr uint64_t kSaMask = (1ull << (kMoeBM / 8)) - 1ull;
 
-    // Loads of one stream position, per wave: NA activation pieces + the activation scales into an
-    // A stage, 4 weight pieces into a slot of the B ring. Sources are passed as data (selected
-    // between the running and the next item), never as two copies of the code.
-    struct SrcA { int row_start, rows; bool valid; };
-    struct SrcB { v4i srd_b; uint32_t voff_b[4]; bool valid; };
-    auto issue_a = [&](const SrcA& a, int stage, int kt, int i) __attribute__((always_inline)) {
-        const bool off = !a.valid || kt >= nk;
-        const uint32_t row_base = to_sgpr((uint32_t)kt * (uint32_t)p.S + (uint32_t)a.row_start);
-        if (i < NA) {
-            v4i sa = srd_a;
-            if (off || 64 * i >= a.rows) sa.z = 0;   // piece i holds rows 64 i .. 64 i + 63 of the tile
-            dma16(sa, to_sgpr(lds_wave + (uint32_t)stage * kF8ATile) + i * NW * 1024, voff_a[i], row_base * 128u);
-        } else {
-            v4i ssa = srd_sa;
-            if (off) ssa.z = 0;
-            dma4_lanes(ssa, to_sgpr(lds_sa_wave + (uint32_t)stage * (kF8BM * 4)), voff_sa, row_base * 4u, kSaMask);
-        }
-    };
-    auto issue_b = [&](const SrcB& b, int slot, int kt, int i) __attribute__((always_inline)) {
-        v4i sb = b.srd_b;
-        if (!b.valid || kt >= nk) sb.z = 0;
-        dma16(sb, to_sgpr(lds_wave + kF8BBase + (uint32_t)slot * kF8BTile) + i * NW * 1024, b.voff_b[i],
-              to_sgpr((uint32_t)kt * 128u));
-    };
-    auto src_a = [&](const MoeFp8Addr& a) __attribute__((always_inline)) { return SrcA{a.row_start, a.rows, a.valid}; };
-    auto src_b = [&](const MoeFp8Addr& a) __attribute__((always_inline)) {
-        SrcB b;
-        b.srd_b = a.srd_b; b.valid = a.valid;
+    auto issue_tile = [&](const MoeFp8Addr& a, int stage, int kt) {
+        v4i sa = srd_a, sb = a.srd_b, ssa = srd_sa;
+        if (!a.valid || kt >= nk) { sa.z = 0; sb.z = 0; ssa.z = 0; }
+        const uint32_t row_base = (uint32_t)kt * (uint32_t)p.S + (uint32_t)a.row_start;
+        const uint32_t dst = lds_wave + (uint32_t)stage * kF8Stage;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) b.voff_b[i] = a.voff_b[i];
-        return b;
+        for (int i = 0; i < NA; ++i) dma16(sa, dst + i * NW * 1024, voff_a[i], row_base * 128u);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dma16(sb, dst + kF8ATile + i * NW * 1024, a.voff_b[i], (uint32_t)kt * 128u);
+        dma4_lanes(ssa, lds_sa_wave + (uint32_t)stage * (kMoeBM * 4), voff_sa, row_base * 4u, kSaMask);
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
     const uint32_t rd_lo = r * 128u + swz_chunk(r, g) * 16u;
     const uint32_t rd_hi = r * 128u + swz_chunk(r, g + 4) * 16u;
     const uint32_t a_lo0 = lds0 + wm * 2048 + rd_lo, a_hi0 = lds0 + wm * 2048 + rd_hi;
-    const uint32_t b_lo0 = lds0 + kF8BBase + wn * (64 * 128) + rd_lo;
-    const uint32_t b_hi0 = lds0 + kF8BBase + wn * (64 * 128) + rd_hi;
+    const uint32_t b_lo0 = lds0 + kF8ATile + wn * (64 * 128) + rd_lo;
+    const uint32_t b_hi0 = lds0 + kF8ATile + wn * (64 * 128) + rd_hi;
     const uint32_t sa_rd0 = lds0 + kF8ScaleBase + (wm * 16 + r) * 4u;
 
+    v4f acc[MT][NT];
     MoeFp8Addr cur, nxt;
 
-    // One stream position (one K-step = one 128-wide scale block of an item) on A stage `ast` and
-    // B slot `bsl`, with the loads that ride along spread between the MFMA groups (a burst of
-    // loads right behind the barrier would hold every wave at the address unit for about as
-    // long as the K-step's MFMAs take): first the next position's activations and scales (la,
-    // lkt -> stage ast ^ 1), then the weights `bdepth` positions ahead (lb, lbkt -> slot lbsl).
-    // MTC: fragments per wave that are worked (all MT, or 2 for items of at most 64 rows); rows
-    // past the item's count give results that are never stored, so nothing inside is conditional
-    // (a conditional update of an accumulator costs a second copy of it in registers).
-    auto compute = [&]<int MTC>(v4f (&acc)[MTC][NT], int ast, int bsl, int kt, const SrcA& la, int lkt,
-                                const SrcB& lb, int lbsl, int lbkt) __attribute__((always_inline)) {
-        uint32_t a_lo = a_lo0 + (uint32_t)ast * kF8ATile, a_hi = a_hi0 + (uint32_t)ast * kF8ATile;
-        uint32_t b_lo = b_lo0 + (uint32_t)bsl * kF8BTile, b_hi = b_hi0 + (uint32_t)bsl * kF8BTile;
-        uint32_t sa_rd = sa_rd0 + (uint32_t)ast * (kF8BM * 4);
+    // One K-step (= one 128-wide scale block) on LDS stage st.
+    auto compute = [&](int st, int rows, int kt) {
+        uint32_t a_lo = a_lo0 + (uint32_t)st * kF8Stage, a_hi = a_hi0 + (uint32_t)st * kF8Stage;
+        uint32_t b_lo = b_lo0 + (uint32_t)st * kF8Stage, b_hi = b_hi0 + (uint32_t)st * kF8Stage;
+        uint32_t sa_rd = sa_rd0 + (uint32_t)st * (kMoeBM * 4);
         asm volatile("" : "+v"(a_lo), "+v"(a_hi), "+v"(b_lo), "+v"(b_hi), "+v"(sa_rd));
         const float ws0 = __int_as_float(scalar_load_x1(cur.sb0 + kt));
         const float ws1 = MODE == 0 ? __int_as_float(scalar_load_x1(cur.sb1 + kt)) : ws0;
         v8i bf[NT];
 #pragma unroll
         for (int n = 0; n < NT; ++n) bf[n] = lds_frag(b_lo, b_hi, n * 2048);
-        constexpr int kPer = (kDma + MTC - 1) / MTC;   // loads per fragment slot
-        // the activation fragment and scale of slot m+1 are read while slot m computes
-        v8i af = lds_frag(a_lo, a_hi, 0);
-        float xs = *(lds_f32_t*)(uintptr_t)(sa_rd);
 #pragma unroll
-        for (int m = 0; m < MTC; ++m) {
-            v8i af_next = af;
-            float xs_next = xs;
-            if (m + 1 < MTC) {
-                af_next = lds_frag(a_lo, a_hi, (m + 1) * 4096);
-                xs_next = *(lds_f32_t*)(uintptr_t)(sa_rd + (m + 1) * 128);
+        for (int m = 0; m < MT; ++m) {
+            if (16 * (2 * m + wm) < rows) {
+                const v8i af = lds_frag(a_lo, a_hi, m * 4096);
+                const float xs = *(lds_f32_t*)(uintptr_t)(sa_rd + m * 128);
+                const float s0 = xs * ws0, s1 = xs * ws1;
+#pragma unroll
+                for (int n = 0; n < NT; ++n) {
+                    const v4f part = mfma_fp8_16x16x128(bf[n], af, v4f{0.f, 0.f, 0.f, 0.f});
+                    const float sc = (n & 1) ? s1 : s0;  // MODE 0: odd tiles are up-projection rows
+                    acc[m][n] += part * sc;
+                }
             }
-            const float s0 = xs * ws0, s1 = xs * ws1;
-            // four MFMAs into fresh accumulators, then their scaling FMAs: the first results are
-            // there when the fourth MFMA has been issued, and the second wave of the SIMD feeds
-            // the MFMA pipe meanwhile
-            v4f part[NT];
-#pragma unroll
-            for (int n = 0; n < NT; ++n) part[n] = mfma_fp8_16x16x128(bf[n], af, v4f{0.f, 0.f, 0.f, 0.f});
-#pragma unroll
-            for (int n = 0; n < NT; ++n)   // MODE 0: odd tiles are up-projection rows
-                acc[m][n] += part[n] * ((n & 1) ? s1 : s0);
-#pragma unroll
-            for (int i = m * kPer; i < (m + 1) * kPer && i < kDma; ++i) {
-                if (i < kDmaA) issue_a(la, ast ^ 1, lkt, i);
-                else issue_b(lb, lbsl, lbkt, i - kDmaA);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            af = af_next;
-            xs = xs_next;
         }
     };
 
-    auto epilogue = [&]<int MTC>(const v4f (&acc)[MTC][NT], const MoeFp8Addr& a) __attribute__((always_inline)) {
+    auto epilogue = [&](const MoeFp8Addr& a) {
         const int rows = a.rows, row_start = a.row_start, n0 = a.n0;
         if (MODE == 1) {
             uint16_t* out = (uint16_t*)p.out0;
 #pragma unroll
-            for (int m = 0; m < MTC; ++m) {
+            for (int m = 0; m < MT; ++m) {
                 const int row = 16 * (2 * m + wm) + (int)r;
                 if (row >= rows) continue;
                 const size_t pos = (size_t)(row_start + row);
@@ -316,10 +256,10 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
             // columns are one 1 x 128 quantization block, so the row maxima of the four column
             // waves are combined through LDS.
             uint8_t* hq = (uint8_t*)p.out0;
-            float h[MTC][8];
+            float h[MT][8];
             const uint32_t xch = lds0 + kF8XchBase;
 #pragma unroll
-            for (int m = 0; m < MTC; ++m) {
+            for (int m = 0; m < MT; ++m) {
 #pragma unroll
                 for (int q = 0; q < 2; ++q) {
                     const v4f gt = acc[m][2 * q], up = acc[m][2 * q + 1];
@@ -339,7 +279,7 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
             }
             __syncthreads();
 #pragma unroll
-            for (int m = 0; m < MTC; ++m) {
+            for (int m = 0; m < MT; ++m) {
                 const int row = 16 * (2 * m + wm) + (int)r;
                 const v4f am = *(lds_v4f_t*)(uintptr_t)(xch + row * 16);
                 const float s = e4m3_block_scale(fmaxf(fmaxf(am.x, am.y), fmaxf(am.z, am.w)));
@@ -352,81 +292,47 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
         }
     };
 
-    // Stream of positions (item, K-step) over this workgroup's items. Per position a wave issues,
-    // in this order, the next position's activation loads and the weight loads `bdepth` = 2
-    // positions ahead (1 with a two-slot ring or when an item has a single K-step); loads return in order, so at the top
-    // of a position "at most kDmaB loads outstanding" means its own loads have landed.
-    const int bdepth = (kBSlots == 3 && nk >= 2) ? 2 : 1;
-    int ast = 0, bsl = 0;   // A stage and B slot of the running position
+    const int depth = nk >= 2 ? 2 : 1;
+    int st = 0;
     make_addr(it, cur);
-    make_addr(it + it_stride, nxt);
-    {
-        const SrcA a0 = src_a(cur);
-        const SrcB b0 = src_b(cur), b1 = src_b(nxt);
-#pragma unroll
-        for (int i = 0; i < kDmaA; ++i) issue_a(a0, 0, 0, i);
-#pragma unroll
-        for (int i = 0; i < kDmaB; ++i) issue_b(b0, 0, 0, i);
-        if (bdepth == 2) {
-#pragma unroll
-            for (int i = 0; i < kDmaB; ++i) issue_b(b0, 1, 1, i);
-        }
-    }
+    issue_tile(cur, 0, 0);
+    if (depth == 2) issue_tile(cur, 1, 1);
     for (;;) {
-        const SrcA acur = src_a(cur), anxt = src_a(nxt);
-        const SrcB bcur = src_b(cur), bnxt = src_b(nxt);
-        // the accumulators live inside the path that works the item: all MT fragments per wave,
-        // or 2 for the small remainder items (up to 64 rows)
-        auto work_item = [&]<int MTC>(int ast, int bsl, int& ast_out, int& bsl_out) __attribute__((always_inline)) {
-            v4f acc[MTC][NT];
+        make_addr(it + it_stride, nxt);
 #pragma unroll
-            for (int m = 0; m < MTC; ++m)
+        for (int m = 0; m < MT; ++m)
 #pragma unroll
-                for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
-            for (int kt = 0; kt < nk; ++kt) {
-                if (bdepth == 2) wait_vmcnt<kDmaB>(); else wait_vmcnt<0>();
-                block_barrier();   // everyone's loads; and everyone is done with the previous position
-                const bool a_same = kt + 1 < nk;
-                const SrcA la{a_same ? acur.row_start : anxt.row_start, a_same ? acur.rows : anxt.rows,
-                              a_same ? acur.valid : anxt.valid};
-                const bool b_same = kt + bdepth < nk;
-                SrcB lb;
-                lb.srd_b = b_same ? bcur.srd_b : bnxt.srd_b;
-                lb.valid = b_same ? bcur.valid : bnxt.valid;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) lb.voff_b[i] = b_same ? bcur.voff_b[i] : bnxt.voff_b[i];
-                int lbsl = bsl + bdepth;
-                if (lbsl >= kBSlots) lbsl -= kBSlots;
-                compute.template operator()<MTC>(acc, ast, bsl, kt, la, a_same ? kt + 1 : 0, lb, lbsl,
-                                                 b_same ? kt + bdepth : kt + bdepth - nk);
-                ast ^= 1;
-                bsl = bsl == kBSlots - 1 ? 0 : bsl + 1;
-            }
-            epilogue.template operator()<MTC>(acc, cur);
-            ast_out = ast; bsl_out = bsl;
-        };
-        if (cur.rows > 64) work_item.template operator()<MT>(ast, bsl, ast, bsl);
-        else work_item.template operator()<2>(ast, bsl, ast, bsl);
+            for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int kt = 0; kt < nk; ++kt) {
+            if (depth == 2) wait_vmcnt<kDma>(); else wait_vmcnt<0>();
+            block_barrier();
+            const int ahead = kt + depth;
+            int stage_ahead = st + depth;
+            if (stage_ahead >= 3) stage_ahead -= 3;
+            if (ahead < nk) issue_tile(cur, stage_ahead, ahead);
+            else issue_tile(nxt, stage_ahead, ahead - nk);
+            compute(st, cur.rows, kt);
+            st = st == 2 ? 0 : st + 1;
+        }
+        epilogue(cur);
         it += it_stride;
         if (it >= it_end) break;
         cur = nxt;
-        make_addr(it + it_stride, nxt);
     }
     wait_vmcnt<0>();
 }
 
-template <int MODE, int BM>
+template <int MODE>
 static int launch_fp8blk_gemm(const MoeFp8Params& p, int max_items, hipStream_t s) {
-    auto kern = moe_fp8blk_gemm_kernel<MODE, BM>;
-    constexpr int lds = F8Geo<BM>::kLds;
+    auto kern = moe_fp8blk_gemm_kernel<MODE>;
     static bool configured = false;
     if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kF8Lds) != hipSuccess)
             return HK_ERR_LAUNCH;
         configured = true;
     }
     const int grid = min(max_items, moe_num_compute_units());
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, s, p);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kF8Lds, s, p);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
@@ -507,10 +413,7 @@ extern "C" int hk_moe_fp8blk_experts_ex(const void* x_e4m3, const float* x_scale
                            (const uint8_t*)x_e4m3, x_scales, sorted_slots, k, S, H, ws + L.xq, (float*)(ws + L.xs));
     }
     int32_t* nitems = (int32_t*)(ws + L.nitems);
-    // item height: 256 rows when the experts have about that many rows or more (MFMA/LDS bound), 192
-    // with the deeper weight ring otherwise (weight-stream bound)
-    const bool tall = (long long)T * k >= (long long)200 * E;
-    moe_launch_build_items(expert_offsets, E, tall ? 256 : 192, I / 128, (MoeItem*)(ws + L.items1), (H + 255) / 256,
+    moe_launch_build_items(expert_offsets, E, kMoeBM, I / 128, (MoeItem*)(ws + L.items1), (H + 255) / 256,
                            (MoeItem*)(ws + L.items2), nitems, s);
 
     MoeFp8Params p{};
@@ -520,7 +423,7 @@ extern "C" int hk_moe_fp8blk_experts_ex(const void* x_e4m3, const float* x_scale
     p.items = (const MoeItem*)(ws + L.items1); p.num_items = nitems;
     p.out0 = ws + L.hq; p.out_scales = (float*)(ws + L.hs);
     p.K = H; p.N = I; p.n_tiles_n = I / 128;
-    st = tall ? launch_fp8blk_gemm<0, 256>(p, L.max_items1, s) : launch_fp8blk_gemm<0, 192>(p, L.max_items1, s);
+    st = launch_fp8blk_gemm<0>(p, L.max_items1, s);
     if (st != HK_OK) return st;
 
     MoeFp8Params q{};
@@ -530,7 +433,7 @@ extern "C" int hk_moe_fp8blk_experts_ex(const void* x_e4m3, const float* x_scale
     q.items = (const MoeItem*)(ws + L.items2); q.num_items = nitems + 1;
     q.out0 = ws + L.o; q.out_scales = nullptr;
     q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
-    st = tall ? launch_fp8blk_gemm<1, 256>(q, L.max_items2, s) : launch_fp8blk_gemm<1, 192>(q, L.max_items2, s);
+    st = launch_fp8blk_gemm<1>(q, L.max_items2, s);
     if (st != HK_OK) return st;
     return hk_moe_unpermute_add(ws + L.o, topk_w, slot_to_pos, T, k, H, y_add_bf16_or_null, y_bf16, stream);
 }
