@@ -75,6 +75,25 @@ def bench_bf16(torch, hk, n, warmup, iters, dev):
             "frac_of_bf16_peak": round(tf / PEAK_BF16, 4), "vs_reference_1610.5": round(tf / 1610.5, 4)}
 
 
+def bench_fp8_decode(torch, hk, warmup, iters, dev):
+    """Decode-like shapes (few rows, N = K = 8192): HBM bound, weights read once."""
+    out = []
+    g = torch.Generator(device=dev).manual_seed(0)
+    N = K = 8192
+    B = torch.randn(N, K, device=dev, generator=g).to(torch.float8_e4m3fn)
+    for M in (16, 128):
+        A = torch.randn(M, K, device=dev, generator=g).to(torch.float8_e4m3fn)
+        C = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        ws = torch.empty(max(16, hk.tk_kernel.fp8_gemm_workspace_bytes(M, N, K)), dtype=torch.uint8, device=dev)
+        _, plain = _timeit(torch, lambda: hk.tk_kernel.dispatch_fp8_gemm(A, B, C, 1.0, 1.0), warmup, iters)
+        _, split = _timeit(torch, lambda: hk.tk_kernel.dispatch_fp8_gemm(A, B, C, 1.0, 1.0, workspace=ws), warmup, iters)
+        byts = M * K + N * K + 2 * M * N
+        out.append({"shape": f"M={M} N=K=8192", "us_without_workspace": round(plain * 1e3, 1),
+                    "us_split_k": round(split * 1e3, 1), "GB/s": round(byts / (split * 1e-3) / 1e9, 1),
+                    "frac_of_hbm": round(byts / (split * 1e-3) / 1e9 / PEAK_HBM, 4)})
+    return out
+
+
 def bench_mxfp4(torch, hk, n, warmup, iters, dev):
     g = torch.Generator(device=dev).manual_seed(0)
     A, SA = hk.quant.quantize_mxfp4(torch.randn(n, n, device=dev, generator=g))
@@ -259,6 +278,7 @@ def main() -> int:
             str(m): round(bench_fp8(torch, hk, m, 50, 50, dev)["tflops"], 1) for m in (1024, 2048, 4096, 16384)}
         del head["A"], head["B"], head["C"]
         torch.cuda.empty_cache()
+        extra["fp8_gemm_decode"] = bench_fp8_decode(torch, hk, 50, 50, dev)
         extra["bf16_gemm"] = bench_bf16(torch, hk, 8192, 50, 50, dev)
         extra["mxfp4_gemm"] = bench_mxfp4(torch, hk, 8192, 50, 50, dev)
         extra["moe_mxfp4"] = bench_moe_mxfp4(torch, hk, quick_w, quick_i, dev)

@@ -475,10 +475,14 @@ constexpr int kSmallStageBytes = 2 * kSmallTileBytes;
 constexpr int kSmallStages = 3;
 constexpr int kSmallLdsBytes = kSmallStages * kSmallStageBytes;  // 96 KiB
 
-template <bool EDGE>
+// SPLIT: blockIdx.y selects a range of `kps` K-steps; the tile's fp32 partial sums go to
+// partial[blockIdx.y][M][N] (plain stores; splitk_reduce_kernel adds the ranges in order, so the
+// result does not depend on timing). For problems with few tiles and a long K (decode-like
+// shapes), where a single workgroup per tile walks K one K-step latency at a time.
+template <bool EDGE, bool SPLIT>
 __global__ __launch_bounds__(256) void fp8_gemm_tile128_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, float alpha, int tiles_m, int tiles_n) {
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n, int kps, float* __restrict__ partial) {
     constexpr int NW = 4, TM = 64, TN = 64, MT = 4, NT = 4;
     constexpr int NDMA = kSmallTileBytes / (NW * 1024);  // 4 loads per wave per operand per K-step
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
@@ -515,7 +519,11 @@ __global__ __launch_bounds__(256) void fp8_gemm_tile128_kernel(
     // end of the row are moved out of the buffer's range (bit 31) and write zeros to LDS
     const uint32_t tail_or =
         (int)(swz_chunk(8 * w + (lane >> 3), lane & 7) * 16u) >= K - (nk - 1) * BK ? 0x80000000u : 0u;
-    auto issue_tile = [&](int stage, int kt) {
+    // this workgroup's K-steps: [kt0, kt0 + nkt)
+    const int kt0 = SPLIT ? (int)blockIdx.y * kps : 0;
+    const int nkt = SPLIT ? min(kps, nk - kt0) : nk;
+    auto issue_tile = [&](int stage, int kt_local) {
+        const int kt = kt0 + kt_local;
         const uint32_t k0 = (uint32_t)kt * BK;
         const uint32_t dst = lds_wave + (uint32_t)stage * kSmallStageBytes;
         const uint32_t vor = kt == nk - 1 ? tail_or : 0u;
@@ -539,13 +547,13 @@ __global__ __launch_bounds__(256) void fp8_gemm_tile128_kernel(
         for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
 
     issue_tile(0, 0);
-    if (nk > 1) issue_tile(1, 1);
+    if (nkt > 1) issue_tile(1, 1);
     int st = 0;
-    for (int kt = 0; kt < nk; ++kt) {
+    for (int kt = 0; kt < nkt; ++kt) {
         // this wave's part of K-step kt has landed (the loads of K-step kt + 1 may still fly)
-        if (kt + 1 < nk) wait_vmcnt<2 * NDMA>(); else wait_vmcnt<0>();
+        if (kt + 1 < nkt) wait_vmcnt<2 * NDMA>(); else wait_vmcnt<0>();
         block_barrier();  // ... everyone's; and everyone is done with the stage of K-step kt - 1
-        if (kt + 2 < nk) issue_tile(st == 0 ? 2 : st - 1, kt + 2);
+        if (kt + 2 < nkt) issue_tile(st == 0 ? 2 : st - 1, kt + 2);
         const uint32_t so = (uint32_t)st * kSmallStageBytes;
         v8i bf[NT];
 #pragma unroll
@@ -558,7 +566,52 @@ __global__ __launch_bounds__(256) void fp8_gemm_tile128_kernel(
         }
         st = st == 2 ? 0 : st + 1;
     }
-    store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
+    if (!SPLIT) {
+        store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
+    } else {
+        // fp32 partial sums: lane (r, g) holds, for row 16 m + r, columns 32 p + 8 g .. +8
+        float* out = partial + (size_t)blockIdx.y * M * N;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const int row = row0 + wm * TM + 16 * m + (int)r;
+            if (row >= M) continue;
+#pragma unroll
+            for (int q = 0; q < NT / 2; ++q) {
+                const int col = col0 + wn * TN + 32 * q + 8 * (int)g;
+                float* dst = out + (size_t)row * N + col;
+                if (col + 8 <= N && (N & 3) == 0) {
+                    *(v4f*)dst = acc[m][2 * q];
+                    *(v4f*)(dst + 4) = acc[m][2 * q + 1];
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (col + j < N) dst[j] = j < 4 ? acc[m][2 * q][j] : acc[m][2 * q + 1][j - 4];
+                }
+            }
+        }
+    }
+}
+
+// C = bf16(alpha * sum_s partial[s]) in split order; one thread per 4 columns.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int splits,
+                                                            long long mn, float alpha,
+                                                            uint16_t* __restrict__ C) {
+    const long long i4 = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i4 >= mn) return;
+    if (i4 + 4 <= mn && (mn & 3) == 0) {
+        v4f sum = *(const v4f*)(partial + i4);
+        for (int s2 = 1; s2 < splits; ++s2) sum += *(const v4f*)(partial + (size_t)s2 * mn + i4);
+        sum *= alpha;
+        v2i o;
+        o.x = pack_bf16(sum.x, sum.y); o.y = pack_bf16(sum.z, sum.w);
+        *(v2i*)(C + i4) = o;
+    } else {
+        for (long long i = i4; i < mn && i < i4 + 4; ++i) {
+            float sum = partial[i];
+            for (int s2 = 1; s2 < splits; ++s2) sum += partial[(size_t)s2 * mn + i];
+            C[i] = (uint16_t)(pack_bf16(sum * alpha, 0.f) & 0xffffu);
+        }
+    }
 }
 
 // Portable kernel for any M, N and K % 16 == 0: 4 waves, each a 32x32 patch of a 64x64
@@ -637,7 +690,7 @@ static int launch_tile(const void* A, const void* B, void* C, int M, int N, int 
 template <bool EDGE>
 static int launch_tile128(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                           hipStream_t stream) {
-    auto kern = fp8_gemm_tile128_kernel<EDGE>;
+    auto kern = fp8_gemm_tile128_kernel<EDGE, false>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -648,7 +701,44 @@ static int launch_tile128(const void* A, const void* B, void* C, int M, int N, i
     const int tiles_m = (M + kSmallTile - 1) / kSmallTile, tiles_n = (N + kSmallTile - 1) / kSmallTile;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), kSmallLdsBytes, stream,
                        (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
-                       tiles_n);
+                       tiles_n, 0, (float*)nullptr);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
+// Number of K ranges the split-K path would use: as many as fill the CUs, each at least 4
+// K-steps long, at most 16; 1 = the problem has enough tiles or too short a K.
+static int splitk_ranges(int M, int N, int K) {
+    const long long tiles = (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
+    const int nk = (K + BK - 1) / BK;
+    const int cus = 256;
+    if (tiles * 2 > cus) return 1;
+    long long s = cus / tiles;
+    if (s > nk / 4) s = nk / 4;
+    if (s > 16) s = 16;
+    return s < 2 ? 1 : (int)s;
+}
+
+template <bool EDGE>
+static int launch_tile128_splitk(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
+                                 int splits, float* partial, hipStream_t stream) {
+    auto kern = fp8_gemm_tile128_kernel<EDGE, true>;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kSmallLdsBytes) != hipSuccess)
+            return HK_ERR_LAUNCH;
+        configured = true;
+    }
+    const int tiles_m = (M + kSmallTile - 1) / kSmallTile, tiles_n = (N + kSmallTile - 1) / kSmallTile;
+    const int nk = (K + BK - 1) / BK;
+    const int kps = (nk + splits - 1) / splits;
+    const int used = (nk + kps - 1) / kps;   // ranges that hold at least one K-step
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, used), dim3(256), kSmallLdsBytes, stream,
+                       (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
+                       tiles_n, kps, partial);
+    const long long mn = (long long)M * N;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((mn / 4 + 256) / 256)), dim3(256), 0, stream,
+                       (const float*)partial, used, mn, alpha, (uint16_t*)C);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
@@ -709,6 +799,28 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
                     : launch_4wave<false, true>(A, B, C, M, N, K, alpha, s);
     return edge ? launch_4wave<true, false>(A, B, C, M, N, K, alpha, s)
                 : launch_4wave<false, false>(A, B, C, M, N, K, alpha, s);
+}
+
+extern "C" size_t hk_fp8_gemm_workspace_bytes(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const int s = hk::splitk_ranges(M, N, K);
+    return s < 2 ? 0 : (size_t)s * M * N * sizeof(float);
+}
+
+extern "C" int hk_fp8_gemm_ws(const void* A, const void* B, void* C, int M, int N, int K, float scale_a,
+                              float scale_b, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace hk;
+    if (M <= 0 || N <= 0 || K <= 0) return HK_ERR_BAD_SHAPE;
+    const int splits = splitk_ranges(M, N, K);
+    const bool can_split = splits >= 2 && workspace && workspace_bytes >= (size_t)splits * M * N * sizeof(float) &&
+                           (K % 16) == 0 && (long long)K * BM < (1ll << 31) && (long long)M * N < (1ll << 40);
+    if (!can_split) return hk_fp8_gemm(A, B, C, M, N, K, scale_a, scale_b, stream);
+    if (!A || !B || !C) return HK_ERR_NULL_POINTER;
+    if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)workspace) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    const bool edge = (M % kSmallTile) != 0 || (N % kSmallTile) != 0;
+    const float alpha = scale_a * scale_b;
+    return edge ? launch_tile128_splitk<true>(A, B, C, M, N, K, alpha, splits, (float*)workspace, (hipStream_t)stream)
+                : launch_tile128_splitk<false>(A, B, C, M, N, K, alpha, splits, (float*)workspace, (hipStream_t)stream);
 }
 
 extern "C" int hk_fp8_gemm(const void* A, const void* B, void* C, int M, int N, int K,

@@ -38,10 +38,18 @@ def _stream(t) -> int:
 _FP8 = (torch.float8_e4m3fn, torch.uint8)
 
 
-def dispatch_fp8_gemm(A, B, C, scale_a: float = 1.0, scale_b: float = 1.0, variant: int = -1) -> None:
+def fp8_gemm_workspace_bytes(M: int, N: int, K: int) -> int:
+    """Bytes of workspace with which dispatch_fp8_gemm splits K for this shape (0: it would not)."""
+    return int(_lib.load_library().hk_fp8_gemm_workspace_bytes(int(M), int(N), int(K)))
+
+
+def dispatch_fp8_gemm(A, B, C, scale_a: float = 1.0, scale_b: float = 1.0, variant: int = -1,
+                      workspace=None) -> None:
     """C[M,N] (bf16) = (scale_a*A[M,K]) @ (scale_b*B[N,K]).T, A and B e4m3, fp32 accumulation.
 
-    `variant` -1 lets the library choose; 0..5 force a kernel (see include/hk355.h)."""
+    `variant` -1 lets the library choose; 0..5 force a kernel (see include/hk355.h). `workspace`
+    (uint8, fp8_gemm_workspace_bytes(M, N, K) bytes): lets the library split K for decode-like
+    shapes (hk_fp8_gemm_ws)."""
     _check_tensor(A, "A", _FP8, 2)
     _check_tensor(B, "B", _FP8, 2)
     _check_tensor(C, "C", (torch.bfloat16,), 2)
@@ -52,7 +60,13 @@ def dispatch_fp8_gemm(A, B, C, scale_a: float = 1.0, scale_b: float = 1.0, varia
     if A.device != B.device or A.device != C.device:
         raise RuntimeError("A, B and C must be on the same device")
     lib = _lib.load_library()
-    if variant < 0:
+    if workspace is not None:
+        _check_tensor(workspace, "workspace", (torch.uint8,), 1)
+        if variant >= 0:
+            raise RuntimeError("workspace and a forced variant exclude each other")
+        st = lib.hk_fp8_gemm_ws(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, float(scale_a),
+                                float(scale_b), workspace.data_ptr(), workspace.numel(), _stream(A))
+    elif variant < 0:
         st = lib.hk_fp8_gemm(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K,
                              float(scale_a), float(scale_b), _stream(A))
     else:

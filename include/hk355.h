@@ -51,6 +51,16 @@ int hk_version(void);
 int hk_fp8_gemm(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
                 int M, int N, int K, float scale_a, float scale_b, void* stream);
 
+/* The same GEMM with an optional workspace, for decode-like shapes (few 128x128 tiles of C and a
+ * long K, e.g. M <= 128 with N = K = 8192): the K range is split over several workgroups per
+ * tile, which write fp32 partial sums to the workspace, and a second kernel adds them in a fixed
+ * order (deterministic) and rounds to bf16. hk_fp8_gemm_workspace_bytes returns the bytes this
+ * needs, or 0 when the shape would not be split; with a NULL or too small workspace, or such a
+ * shape, the call is hk_fp8_gemm. No counterpart in the reference (compile-time shapes only). */
+size_t hk_fp8_gemm_workspace_bytes(int M, int N, int K);
+int hk_fp8_gemm_ws(const void* A_e4m3, const void* B_e4m3, void* C_bf16, int M, int N, int K,
+                   float scale_a, float scale_b, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Same contract, forced onto one kernel variant (for tests and tuning):
  * 0 = portable kernel (any shape), 1 = 256x256x128 tile, 8 waves, 2 = 256x256x128 tile,
  * 4 waves, hand-interleaved schedule over two LDS stages, 3 = 256x256x128 tile, 4 waves, plain

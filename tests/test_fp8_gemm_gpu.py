@@ -90,6 +90,51 @@ def test_fp8_gemm_k_tail_last_row_does_not_read_past_the_buffer(hk):
         assert G.rel_fro_error(out, G.fp8_gemm(a, b, sa, sb)) <= 5e-3
 
 
+SPLITK = [(16, 1024, 4096), (64, 512, 8192), (100, 520, 2048), (128, 1024, 2064), (1, 128, 1024), (33, 200, 4096)]
+
+
+@pytest.mark.parametrize("shape", SPLITK)
+def test_fp8_gemm_split_k_matches_oracle(hk, shape):
+    """Decode-like shapes with a workspace: K split over several workgroups per tile, partial sums
+    added in a fixed order. Checked against the oracle and for run-to-run bit identity."""
+    M, N, K = shape
+    print(f"fp8_gemm split-k shape={shape}", flush=True)
+    need = hk.tk_kernel.fp8_gemm_workspace_bytes(M, N, K)
+    assert need > 0, "these shapes are meant to take the split path"
+    rng = np.random.default_rng(3 + M + N + K)
+    (a, sa), (b, sb) = _random_codes(rng, M, K), _random_codes(rng, N, K)
+    dev = torch.device("cuda:0")
+    A = torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
+    B = torch.from_numpy(b).to(dev).view(torch.float8_e4m3fn)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    outs = []
+    for _ in range(2):
+        C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+        ws.fill_(0xFF)  # NaN patterns: every partial sum that is read must have been written
+        hk.tk_kernel.dispatch_fp8_gemm(A, B, C, float(sa), float(sb), workspace=ws)
+        torch.cuda.synchronize()
+        outs.append(C.view(torch.int16).cpu().numpy().view(np.uint16))
+    assert np.array_equal(outs[0], outs[1])
+    out = F.bf16_to_f32(outs[0])
+    assert np.isfinite(out).all()
+    assert G.rel_fro_error(out, G.fp8_gemm(a, b, sa, sb)) <= 5e-3
+
+
+def test_fp8_gemm_workspace_is_optional(hk):
+    # a shape that is not split (enough tiles): zero bytes, and a workspace changes nothing
+    assert hk.tk_kernel.fp8_gemm_workspace_bytes(2048, 2048, 1024) == 0
+    rng = np.random.default_rng(5)
+    (a, sa), (b, sb) = _random_codes(rng, 256, 256), _random_codes(rng, 256, 256)
+    base = _run(hk, a, b, float(sa), float(sb), -1)
+    dev = torch.device("cuda:0")
+    C = torch.zeros((256, 256), dtype=torch.bfloat16, device=dev)
+    hk.tk_kernel.dispatch_fp8_gemm(torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn),
+                                   torch.from_numpy(b).to(dev).view(torch.float8_e4m3fn), C, float(sa), float(sb),
+                                   workspace=torch.empty(16, dtype=torch.uint8, device=dev))
+    torch.cuda.synchronize()
+    assert np.array_equal(C.view(torch.int16).cpu().numpy().view(np.uint16), base)
+
+
 @pytest.mark.parametrize("variant", [1, 2])
 def test_fp8_gemm_older_tile_kernels_refuse_k_tail(hk, variant):
     rng = np.random.default_rng(7)
