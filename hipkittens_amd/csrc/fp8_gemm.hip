@@ -16,6 +16,10 @@
 #include "../../include/hk355.h"
 
 namespace hk {
+int moe_num_compute_units();  // number of CUs of the current device (moe_mxfp4.hip)
+}
+
+namespace hk {
 
 template <int WM, int WN, bool EDGE>
 __global__ __launch_bounds__(WM * WN * 64) void fp8_gemm_tile_kernel(
@@ -710,7 +714,7 @@ static int launch_tile128(const void* A, const void* B, void* C, int M, int N, i
 static int splitk_ranges(int M, int N, int K) {
     const long long tiles = (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
     const int nk = (K + BK - 1) / BK;
-    const int cus = 256;
+    const int cus = moe_num_compute_units();   // 256 when no device can be queried
     if (tiles * 2 > cus) return 1;
     long long s = cus / tiles;
     if (s > nk / 4) s = nk / 4;
