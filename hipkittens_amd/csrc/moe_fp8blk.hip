@@ -4,7 +4,8 @@
 // The reference has no MoE code (no counterpart to cite). Structure as in the MXFP4 MoE of this
 // library (moe_mxfp4.hip): persistent 8-wave workgroups walk a device-built list of (m-tile,
 // n-tile) work items, operands stream through a three-stage LDS ring with direct global->LDS
-// loads, activations live in K-step-major tiles. fp32 block scales cannot ride the MFMA's scale
+// loads. The gate+up GEMM fetches its activation rows from the caller's x by token index (no
+// permuted copy); the intermediate h lives in K-step-major tiles. fp32 block scales cannot ride the MFMA's scale
 // port (e8m0 only), so every K-step of 128 is one unscaled v_mfma_f32_16x16x128_f8f6f4 into a
 // fresh accumulator that a VALU FMA folds into the running sum:
 //     acc += partial * (x_scale[row, kb] * w_scale[col / 128, kb]).
@@ -64,25 +65,8 @@ __global__ __launch_bounds__(256) void fp8_quantize_rows_1x128_kernel(const uint
     if ((c8 & 15) == 0) scales[(size_t)row * (cols / 128) + (c8 >> 4)] = s;
 }
 
-// Permute quantized activations into K-step-major tiles in sorted order: row `pos` of the output
-// is token sorted_slots[pos] / topk. tiled [nk][S][128] bytes, tiled_scales [nk][S] floats.
-__global__ __launch_bounds__(256) void fp8blk_permute_kernel(const uint8_t* __restrict__ xq,
-                                                             const float* __restrict__ xs,
-                                                             const int32_t* __restrict__ sorted_slots, int topk,
-                                                             int S, int cols, uint8_t* __restrict__ tiled,
-                                                             float* __restrict__ tiled_scales) {
-    const int per_row = cols / 16;  // 16-byte chunks
-    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
-    const int pos = (int)(gid / per_row), c = (int)(gid % per_row);
-    if (pos >= S) return;
-    const int row = sorted_slots[pos] / topk;
-    const size_t tile_row = (size_t)(c >> 3) * S + pos;
-    *(v4i*)(tiled + tile_row * 128 + (c & 7) * 16) = *(const v4i*)(xq + (size_t)row * cols + c * 16);
-    if ((c & 7) == 0) tiled_scales[tile_row] = xs[(size_t)row * (cols / 128) + (c >> 3)];
-}
-
 struct MoeFp8Params {
-    const uint8_t* A;      // activations, K-step-major tiles [nk][S][128] e4m3
+    const uint8_t* A;      // activations, K-step-major tiles [nk][S][128] e4m3 (GATHER: see below)
     const float* SA;       // their scales [nk][S]
     const uint8_t* B;      // expert weights [E][rows_b][K] e4m3
     const float* SB;       // their scales [E][rows_b / 128][K / 128]
@@ -92,6 +76,10 @@ struct MoeFp8Params {
     float* out_scales;     // MODE 0: scales of h [I / 128][S]
     long long b_expert_stride, sb_expert_stride;  // bytes / floats
     int K, N, S, n_tiles_n;
+    // GATHER kernels (gate+up GEMM reading the caller's activations in place): A = x [T][K] e4m3,
+    // SA = its scales [T][K / 128]; row `pos` of the sorted order is token sorted_slots[pos] / topk
+    const int32_t* sorted_slots;
+    int topk, T;
 };
 
 constexpr int kF8ATile = kMoeBM * 128;             // 16 KiB
@@ -124,10 +112,15 @@ struct MoeFp8Addr {
     const float* sb1;  // MODE 0: scales of the up-projection row block
     int row_start, rows, n0, n_tile;
     bool valid;
+    uint32_t gvoff_a[kMoeBM / 64], gvoff_sa;  // GATHER: per-lane source offsets of the item's activation rows / scales
 };
 
-template <int MODE>
+// GATHER (MODE 0 only): the activation tile's rows are fetched from the caller's x by token index
+// (one 128-byte line per row and K-step either way), which saves writing and re-reading a
+// permuted copy of x (k times its size).
+template <int MODE, bool GATHER>
 __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params p) {
+    static_assert(!GATHER || MODE == 0, "only the gate+up GEMM reads the caller's activations");
     constexpr int NW = 8, MT = kMoeBM / 32, NT = 4, NA = kMoeBM / 64;
     constexpr int kDma = NA + 4 + 1;
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
@@ -144,11 +137,33 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
 
     const int nk = p.K >> 7;
     const int rows_b = MODE == 0 ? 2 * p.N : p.N;
-    const v4i srd_a = make_srd(p.A, (uint32_t)nk * (uint32_t)p.S * 128u);
-    const v4i srd_sa = make_srd(p.SA, (uint32_t)nk * (uint32_t)p.S * 4u);
+    const v4i srd_a = make_srd(p.A, GATHER ? (uint32_t)p.T * (uint32_t)p.K : (uint32_t)nk * (uint32_t)p.S * 128u);
+    const v4i srd_sa = make_srd(p.SA, GATHER ? (uint32_t)p.T * (uint32_t)nk * 4u : (uint32_t)nk * (uint32_t)p.S * 4u);
     const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);
 
-    auto make_addr = [&](int idx, MoeFp8Addr& a) {
+    // GATHER: sorted slot indices of the activation rows this lane loads for an item (NA tile pieces
+    // and the scale row). They are fetched two items ahead with loads the compiler does not see
+    // (a visible load would make it drain the whole load pipeline with vmcnt(0) before the
+    // first use); the K loop's own waits cover them: they are queued behind the loads of the
+    // item's first two K-steps and complete before the second wait returns.
+    struct SlotIds { uint32_t a[NA]; uint32_t s; };
+    auto issue_ids = [&](int idx, SlotIds& o) __attribute__((always_inline)) {
+        if (idx >= it_end) idx = it_end - 1;
+        const int row_start = scalar_load_x4(p.items + idx).y;
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            const uint32_t off = (uint32_t)min(row_start + 8 * (i * NW + w) + (lane >> 3), p.S - 1) * 4u;
+            asm volatile("global_load_dword %0, %1, %2" : "=v"(o.a[i]) : "v"(off), "s"(p.sorted_slots) : "memory");
+        }
+        const uint32_t off = (uint32_t)min(row_start + w * (kMoeBM / 8) + (lane & (kMoeBM / 8 - 1)), p.S - 1) * 4u;
+        asm volatile("global_load_dword %0, %1, %2" : "=v"(o.s) : "v"(off), "s"(p.sorted_slots) : "memory");
+    };
+    auto landed_ids = [&](SlotIds& o) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NA; ++i) asm volatile("" : "+v"(o.a[i]));
+        asm volatile("" : "+v"(o.s));
+    };
+    auto make_addr = [&](int idx, MoeFp8Addr& a, const SlotIds& ids) __attribute__((always_inline)) {
         a.valid = idx < it_end;
         if (!a.valid) idx = it_end - 1;
         const v4i item = scalar_load_x4(p.items + idx);
@@ -162,6 +177,17 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
         for (int i = 0; i < 4; ++i)
             a.voff_b[i] = (uint32_t)moe_b_row(MODE, 8 * (i * NW + w) + (lane >> 3), a.n_tile, p.N) * (uint32_t)p.K +
                           chunk16 * 16u;
+        if (GATHER) {
+            // rows past the item's count are not fetched at all (bit 31: out of range, LDS gets zeros)
+#pragma unroll
+            for (int i = 0; i < NA; ++i)
+                a.gvoff_a[i] = 8 * (i * NW + w) + (lane >> 3) < a.rows
+                                   ? (ids.a[i] / (uint32_t)p.topk) * (uint32_t)p.K + chunk16 * 16u
+                                   : 0x80000000u;
+            a.gvoff_sa = w * (kMoeBM / 8) + (lane & (kMoeBM / 8 - 1)) < a.rows
+                             ? (ids.s / (uint32_t)p.topk) * (uint32_t)nk * 4u
+                             : 0x80000000u;
+        }
         const float* sb = p.SB + (size_t)expert * p.sb_expert_stride;
         if (MODE == 0) {
             a.sb0 = sb + (size_t)a.n_tile * nk;                    // gate rows n0 .. n0+127
@@ -187,10 +213,19 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
         const uint32_t row_base = (uint32_t)kt * (uint32_t)p.S + (uint32_t)a.row_start;
         const uint32_t dst = lds_wave + (uint32_t)stage * kF8Stage;
 #pragma unroll
-        for (int i = 0; i < NA; ++i) dma16(sa, dst + i * NW * 1024, voff_a[i], row_base * 128u);
+        for (int i = 0; i < NA; ++i) {
+            if (GATHER) {
+                dma16(sa, dst + i * NW * 1024, a.gvoff_a[i], (uint32_t)kt * 128u);
+            } else {
+                v4i sai = sa;   // the piece's 8 rows lie past the item's count: nothing is fetched
+                if (8 * (i * NW + w) >= a.rows) sai.z = 0;
+                dma16(sai, dst + i * NW * 1024, voff_a[i], row_base * 128u);
+            }
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) dma16(sb, dst + kF8ATile + i * NW * 1024, a.voff_b[i], (uint32_t)kt * 128u);
-        dma4_lanes(ssa, lds_sa_wave + (uint32_t)stage * (kMoeBM * 4), voff_sa, row_base * 4u, kSaMask);
+        if (GATHER) dma4_lanes(ssa, lds_sa_wave + (uint32_t)stage * (kMoeBM * 4), a.gvoff_sa, (uint32_t)kt * 4u, kSaMask);
+        else dma4_lanes(ssa, lds_sa_wave + (uint32_t)stage * (kMoeBM * 4), voff_sa, row_base * 4u, kSaMask);
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
@@ -294,11 +329,20 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
 
     const int depth = nk >= 2 ? 2 : 1;
     int st = 0;
-    make_addr(it, cur);
+    SlotIds ids_cur{}, ids_nxt{}, ids_nn{};
+    if (GATHER) {
+        issue_ids(it, ids_cur);
+        issue_ids(it + it_stride, ids_nxt);
+        wait_vmcnt<0>();
+        landed_ids(ids_cur);
+        landed_ids(ids_nxt);
+    }
+    make_addr(it, cur, ids_cur);
     issue_tile(cur, 0, 0);
     if (depth == 2) issue_tile(cur, 1, 1);
     for (;;) {
-        make_addr(it + it_stride, nxt);
+        make_addr(it + it_stride, nxt, ids_nxt);
+        if (GATHER) issue_ids(it + 2 * it_stride, ids_nn);
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
@@ -318,13 +362,18 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
         it += it_stride;
         if (it >= it_end) break;
         cur = nxt;
+        if (GATHER) {   // (asm: the copy must stay behind the K loop's waits)
+#pragma unroll
+            for (int i = 0; i < NA; ++i) asm volatile("v_mov_b32 %0, %1" : "=v"(ids_nxt.a[i]) : "v"(ids_nn.a[i]));
+            asm volatile("v_mov_b32 %0, %1" : "=v"(ids_nxt.s) : "v"(ids_nn.s));
+        }
     }
     wait_vmcnt<0>();
 }
 
-template <int MODE>
+template <int MODE, bool GATHER>
 static int launch_fp8blk_gemm(const MoeFp8Params& p, int max_items, hipStream_t s) {
-    auto kern = moe_fp8blk_gemm_kernel<MODE>;
+    auto kern = moe_fp8blk_gemm_kernel<MODE, GATHER>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kF8Lds) != hipSuccess)
@@ -353,7 +402,7 @@ static Fp8Ws fp8_ws_layout(int T, int H, int I, int E, int k) {
     L.items1 = take((size_t)L.max_items1 * sizeof(MoeItem));
     L.items2 = take((size_t)L.max_items2 * sizeof(MoeItem));
     L.nitems = take(8);
-    L.xq = take(S * (size_t)H); L.xs = take(S * (size_t)(H / 128) * 4);
+    L.xq = L.xs = off;   // (the gate+up GEMM gathers the caller's activations in place: no permuted copy)
     L.hq = take(S * (size_t)I); L.hs = take(S * (size_t)(I / 128) * 4);
     L.o = take(S * (size_t)H * 2);
     L.total = off;
@@ -407,23 +456,19 @@ extern "C" int hk_moe_fp8blk_experts_ex(const void* x_e4m3, const float* x_scale
     hipStream_t s = (hipStream_t)stream;
     uint8_t* ws = (uint8_t*)workspace;
     const int S = T * k;
-    {
-        const long long threads = (long long)S * (H / 16);
-        hipLaunchKernelGGL(fp8blk_permute_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
-                           (const uint8_t*)x_e4m3, x_scales, sorted_slots, k, S, H, ws + L.xq, (float*)(ws + L.xs));
-    }
     int32_t* nitems = (int32_t*)(ws + L.nitems);
     moe_launch_build_items(expert_offsets, E, kMoeBM, I / 128, (MoeItem*)(ws + L.items1), (H + 255) / 256,
                            (MoeItem*)(ws + L.items2), nitems, s);
 
     MoeFp8Params p{};
-    p.A = ws + L.xq; p.SA = (const float*)(ws + L.xs); p.S = S;
+    p.A = (const uint8_t*)x_e4m3; p.SA = x_scales; p.S = S;   // gathered by token index inside the kernel
+    p.sorted_slots = sorted_slots; p.topk = k; p.T = T;
     p.B = (const uint8_t*)w13; p.SB = w13_scales;
     p.b_expert_stride = (long long)2 * I * H; p.sb_expert_stride = (long long)(2 * I / 128) * (H / 128);
     p.items = (const MoeItem*)(ws + L.items1); p.num_items = nitems;
     p.out0 = ws + L.hq; p.out_scales = (float*)(ws + L.hs);
     p.K = H; p.N = I; p.n_tiles_n = I / 128;
-    st = launch_fp8blk_gemm<0>(p, L.max_items1, s);
+    st = launch_fp8blk_gemm<0, true>(p, L.max_items1, s);
     if (st != HK_OK) return st;
 
     MoeFp8Params q{};
@@ -433,7 +478,7 @@ extern "C" int hk_moe_fp8blk_experts_ex(const void* x_e4m3, const float* x_scale
     q.items = (const MoeItem*)(ws + L.items2); q.num_items = nitems + 1;
     q.out0 = ws + L.o; q.out_scales = nullptr;
     q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
-    st = launch_fp8blk_gemm<1>(q, L.max_items2, s);
+    st = launch_fp8blk_gemm<1, false>(q, L.max_items2, s);
     if (st != HK_OK) return st;
     return hk_moe_unpermute_add(ws + L.o, topk_w, slot_to_pos, T, k, H, y_add_bf16_or_null, y_bf16, stream);
 }
