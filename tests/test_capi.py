@@ -51,6 +51,22 @@ def test_c_entry_points_reject_bad_arguments_without_a_gpu():
     assert lib.hk_moe_sort(p, 4, 2, 8, p, p, None, None, 0, None) == -4       # no workspace
     assert lib.hk_moe_sort(p, 4, 2, 8, p, p, None, p, 4, None) == -4          # workspace too small
     assert lib.hk_moe_sort_workspace_bytes(4096, 4, 128) == 17 * 128 * 4
+    # split-K entry point: the same argument checks; the workspace is optional
+    assert lib.hk_fp8_gemm_ws(p, p, p, 0, 256, 256, 1.0, 1.0, None, 0, None) == -2
+    assert lib.hk_fp8_gemm_ws(None, p, p, 16, 4096, 4096, 1.0, 1.0, p, 1 << 40, None) == -1
+    assert lib.hk_fp8_gemm_ws(p, p, p, 16, 4096, 4090, 1.0, 1.0, p, 1 << 40, None) == -2
+    assert lib.hk_fp8_gemm_workspace_bytes(8192, 8192, 8192) == 0
+    assert lib.hk_fp8_gemm_workspace_bytes(16, 8192, 8192) % (16 * 8192 * 4) == 0
+    assert lib.hk_fp8_gemm_workspace_bytes(16, 8192, 8192) > 0
+    assert lib.hk_bf16_gemm(p, p, p, 64, 64, 60, None) == -2                  # K % 8
+    # extended MoE entry points: option checks come before anything touches memory
+    args = (p, p, p, 8, p, p, 8, p, p, p, p, p, 16, 64, 32, 4, 2, 0)
+    assert lib.hk_moe_mxfp4_experts_ex(*args, None, None, 7, 1.702, 7.0, 0, p, 1 << 30, None) == -6   # activation
+    assert lib.hk_moe_mxfp4_experts_ex(*args, None, None, 1, 1.702, 0.0, 0, p, 1 << 30, None) == -2   # limit <= 0
+    assert lib.hk_moe_mxfp4_experts_ex(*args, p + 4, None, 0, 0.0, 0.0, 0, p, 1 << 30, None) == -3    # bias alignment
+    assert lib.hk_moe_mxfp4_experts_ex(*args, None, None, 0, 0.0, 0.0, 0, None, 0, None) == -4        # workspace
+    assert lib.hk_moe_unpermute_add(p, p, p, 4, 2, 60, None, p, None) == -2                            # H % 8
+    assert lib.hk_moe_unpermute_add(p, p, p, 4, 2, 64, p + 2, p, None) == -3
 
 
 def test_python_boundary_rejects_like_the_reference():
