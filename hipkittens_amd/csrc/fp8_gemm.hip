@@ -478,17 +478,23 @@ constexpr int kSmallTileBytes = kSmallTile * BK;          // 16 KiB per operand
 constexpr int kSmallStageBytes = 2 * kSmallTileBytes;
 constexpr int kSmallStages = 3;
 constexpr int kSmallLdsBytes = kSmallStages * kSmallStageBytes;  // 96 KiB
+// the same kernel with 64x64 tiles and four 16 KiB stages (two workgroups per CU): for problems
+// with so few 128x128 tiles that a quarter of the tile is needed to give every CU work
+constexpr int kTinyTile = 64;
+constexpr int kTinyStages = 4;
 
 // SPLIT: blockIdx.y selects a range of `kps` K-steps; the tile's fp32 partial sums go to
 // partial[blockIdx.y][M][N] (plain stores; splitk_reduce_kernel adds the ranges in order, so the
 // result does not depend on timing). For problems with few tiles and a long K (decode-like
 // shapes), where a single workgroup per tile walks K one K-step latency at a time.
-template <bool EDGE, bool SPLIT>
-__global__ __launch_bounds__(256) void fp8_gemm_tile128_kernel(
+template <int TILE, int STAGES, bool EDGE, bool SPLIT>
+__global__ __launch_bounds__(256) void fp8_gemm_small_tile_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
     int M, int N, int K, float alpha, int tiles_m, int tiles_n, int kps, float* __restrict__ partial) {
-    constexpr int NW = 4, TM = 64, TN = 64, MT = 4, NT = 4;
-    constexpr int NDMA = kSmallTileBytes / (NW * 1024);  // 4 loads per wave per operand per K-step
+    constexpr int NW = 4, TM = TILE / 2, TN = TILE / 2, MT = TM / 16, NT = TN / 16;
+    constexpr int kTB = TILE * BK, kSB = 2 * kTB;    // bytes of one operand tile / of one stage
+    constexpr int NDMA = kTB / (NW * 1024);          // loads per wave per operand per K-step
+    static_assert(STAGES >= 3 && STAGES <= 8 && (STAGES - 2) * 2 * NDMA < 64, "vmcnt range");
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
     const int lane = lane_id(), w = wave_id();
     const int wm = w >> 1, wn = w & 1;
@@ -498,8 +504,8 @@ __global__ __launch_bounds__(256) void fp8_gemm_tile128_kernel(
         const int id = xcd_chunk_order(blockIdx.x, tiles_m * tiles_n, kCuPerXcd);
         grouped_raster(id, tiles_m, tiles_n, 8, pm, pn);
     }
-    const int row0 = pm * kSmallTile, col0 = pn * kSmallTile;
-    const int a_rows = min(M - row0, kSmallTile), b_rows = min(N - col0, kSmallTile);
+    const int row0 = pm * TILE, col0 = pn * TILE;
+    const int a_rows = min(M - row0, TILE), b_rows = min(N - col0, TILE);
     const v4i srd_a = make_srd(A + (size_t)row0 * K, (uint32_t)a_rows * (uint32_t)K);
     const v4i srd_b = make_srd(B + (size_t)col0 * K, (uint32_t)b_rows * (uint32_t)K);
 
@@ -529,20 +535,32 @@ __global__ __launch_bounds__(256) void fp8_gemm_tile128_kernel(
     auto issue_tile = [&](int stage, int kt_local) {
         const int kt = kt0 + kt_local;
         const uint32_t k0 = (uint32_t)kt * BK;
-        const uint32_t dst = lds_wave + (uint32_t)stage * kSmallStageBytes;
+        const uint32_t dst = lds_wave + (uint32_t)stage * kSB;
         const uint32_t vor = kt == nk - 1 ? tail_or : 0u;
 #pragma unroll
         for (int i = 0; i < NDMA; ++i) dma16(srd_a, dst + i * NW * 1024, voff_a[i] | vor, k0);
 #pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma16(srd_b, dst + kSmallTileBytes + i * NW * 1024, voff_b[i] | vor, k0);
+        for (int i = 0; i < NDMA; ++i) dma16(srd_b, dst + kTB + i * NW * 1024, voff_b[i] | vor, k0);
+    };
+    // wait until at most `tiles` of the most recently issued K-steps' loads are still in flight
+    auto wait_tiles = [&](int tiles) {
+        switch (tiles) {
+            case 0: wait_vmcnt<0>(); break;
+            case 1: wait_vmcnt<2 * NDMA>(); break;
+            case 2: wait_vmcnt<(STAGES > 3 ? 2 : 1) * 2 * NDMA>(); break;
+            case 3: wait_vmcnt<(STAGES > 4 ? 3 : 1) * 2 * NDMA>(); break;
+            case 4: wait_vmcnt<(STAGES > 5 ? 4 : 1) * 2 * NDMA>(); break;
+            case 5: wait_vmcnt<(STAGES > 6 ? 5 : 1) * 2 * NDMA>(); break;
+            default: wait_vmcnt<(STAGES > 7 ? 6 : 1) * 2 * NDMA>(); break;
+        }
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
     const uint32_t rd_lo = r * 128u + swz_chunk(r, g) * 16u;
     const uint32_t rd_hi = r * 128u + swz_chunk(r, g + 4) * 16u;
     const uint32_t a_lo0 = lds0 + wm * (TM * BK) + rd_lo, a_hi0 = lds0 + wm * (TM * BK) + rd_hi;
-    const uint32_t b_lo0 = lds0 + kSmallTileBytes + wn * (TN * BK) + rd_lo;
-    const uint32_t b_hi0 = lds0 + kSmallTileBytes + wn * (TN * BK) + rd_hi;
+    const uint32_t b_lo0 = lds0 + kTB + wn * (TN * BK) + rd_lo;
+    const uint32_t b_hi0 = lds0 + kTB + wn * (TN * BK) + rd_hi;
 
     v4f acc[MT][NT];
 #pragma unroll
@@ -550,15 +568,17 @@ __global__ __launch_bounds__(256) void fp8_gemm_tile128_kernel(
 #pragma unroll
         for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    issue_tile(0, 0);
-    if (nkt > 1) issue_tile(1, 1);
+    // K-steps kt .. kt + STAGES - 2 are in flight or in LDS while step kt is multiplied
+#pragma unroll
+    for (int p = 0; p < STAGES - 1; ++p)
+        if (p < nkt) issue_tile(p, p);
     int st = 0;
     for (int kt = 0; kt < nkt; ++kt) {
-        // this wave's part of K-step kt has landed (the loads of K-step kt + 1 may still fly)
-        if (kt + 1 < nkt) wait_vmcnt<2 * NDMA>(); else wait_vmcnt<0>();
+        // this wave's part of K-step kt has landed (the loads of the steps behind it may still fly)
+        wait_tiles(min(nkt - 1 - kt, STAGES - 2));
         block_barrier();  // ... everyone's; and everyone is done with the stage of K-step kt - 1
-        if (kt + 2 < nkt) issue_tile(st == 0 ? 2 : st - 1, kt + 2);
-        const uint32_t so = (uint32_t)st * kSmallStageBytes;
+        if (kt + STAGES - 1 < nkt) issue_tile(st == 0 ? STAGES - 1 : st - 1, kt + STAGES - 1);
+        const uint32_t so = (uint32_t)st * kSB;
         v8i bf[NT];
 #pragma unroll
         for (int n = 0; n < NT; ++n) bf[n] = lds_frag(b_lo0 + so, b_hi0 + so, n * 16 * BK);
@@ -568,7 +588,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_tile128_kernel(
 #pragma unroll
             for (int n = 0; n < NT; ++n) acc[m][n] = mfma_fp8_16x16x128(bf[n], af, acc[m][n]);
         }
-        st = st == 2 ? 0 : st + 1;
+        st = st == STAGES - 1 ? 0 : st + 1;
     }
     if (!SPLIT) {
         store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
@@ -691,19 +711,20 @@ static int launch_tile(const void* A, const void* B, void* C, int M, int N, int 
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
-template <bool EDGE>
-static int launch_tile128(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
-                          hipStream_t stream) {
-    auto kern = fp8_gemm_tile128_kernel<EDGE, false>;
+template <int TILE, int STAGES, bool EDGE>
+static int launch_small_tile(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
+                             hipStream_t stream) {
+    auto kern = fp8_gemm_small_tile_kernel<TILE, STAGES, EDGE, false>;
+    constexpr int lds_bytes = STAGES * 2 * TILE * BK;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kSmallLdsBytes) != hipSuccess)
+                                lds_bytes) != hipSuccess)
             return HK_ERR_LAUNCH;
         configured = true;
     }
-    const int tiles_m = (M + kSmallTile - 1) / kSmallTile, tiles_n = (N + kSmallTile - 1) / kSmallTile;
-    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), kSmallLdsBytes, stream,
+    const int tiles_m = (M + TILE - 1) / TILE, tiles_n = (N + TILE - 1) / TILE;
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream,
                        (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
                        tiles_n, 0, (float*)nullptr);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
@@ -715,7 +736,8 @@ static int splitk_ranges(int M, int N, int K) {
     const long long tiles = (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
     const int nk = (K + BK - 1) / BK;
     const int cus = moe_num_compute_units();   // 256 when no device can be queried
-    if (tiles * 2 > cus) return 1;
+    // shorter K: the 64x64-tile kernel without a second launch is as fast or faster
+    if (tiles * 2 > cus || nk < 48) return 1;
     long long s = cus / tiles;
     if (s > nk / 4) s = nk / 4;
     if (s > 16) s = 16;
@@ -725,7 +747,7 @@ static int splitk_ranges(int M, int N, int K) {
 template <bool EDGE>
 static int launch_tile128_splitk(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                                  int splits, float* partial, hipStream_t stream) {
-    auto kern = fp8_gemm_tile128_kernel<EDGE, true>;
+    auto kern = fp8_gemm_small_tile_kernel<kSmallTile, kSmallStages, EDGE, true>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -773,8 +795,8 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 16) != 0) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < 0 || variant > 5) return HK_ERR_UNSUPPORTED;
-    // K tails: the ring kernel (4) and the 128x128-tile kernel (5) take any K % 16 == 0
+    if (variant < 0 || variant > 6) return HK_ERR_UNSUPPORTED;
+    // K tails: the ring kernel (4) and the small-tile kernels (5, 6) take any K % 16 == 0
     if (variant != 0 && (long long)K * BM >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
     if (variant >= 1 && variant <= 3 && (K % BK) != 0) return HK_ERR_BAD_SHAPE;
     const float alpha = scale_a * scale_b;
@@ -788,8 +810,13 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
     }
     if (variant == 5) {
         const bool edge128 = (M % kSmallTile) != 0 || (N % kSmallTile) != 0;
-        return edge128 ? launch_tile128<true>(A, B, C, M, N, K, alpha, s)
-                       : launch_tile128<false>(A, B, C, M, N, K, alpha, s);
+        return edge128 ? launch_small_tile<kSmallTile, kSmallStages, true>(A, B, C, M, N, K, alpha, s)
+                       : launch_small_tile<kSmallTile, kSmallStages, false>(A, B, C, M, N, K, alpha, s);
+    }
+    if (variant == 6) {
+        const bool edge64 = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
+        return edge64 ? launch_small_tile<kTinyTile, kTinyStages, true>(A, B, C, M, N, K, alpha, s)
+                      : launch_small_tile<kTinyTile, kTinyStages, false>(A, B, C, M, N, K, alpha, s);
     }
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
     if (variant == 1)
@@ -829,9 +856,14 @@ extern "C" int hk_fp8_gemm_ws(const void* A, const void* B, void* C, int M, int 
 
 extern "C" int hk_fp8_gemm(const void* A, const void* B, void* C, int M, int N, int K,
                            float scale_a, float scale_b, void* stream) {
-    const bool tile_ok = K > 0 && (long long)K * hk::BM < (1ll << 31) && M >= 64 && N >= 64;
-    // fewer 256x256 tiles than half the CUs of an MI355X: the 128x128-tile kernel spreads the
-    // problem over four times as many workgroups
-    const long long tiles256 = (long long)((M + hk::BM - 1) / hk::BM) * ((N + hk::BN - 1) / hk::BN);
-    return hk_fp8_gemm_variant(A, B, C, M, N, K, scale_a, scale_b, !tile_ok ? 0 : tiles256 < 128 ? 5 : 4, stream);
+    using namespace hk;
+    const bool tile_ok = K > 0 && (long long)K * BM < (1ll << 31) && M >= 16 && N >= 16;
+    // The tile is the largest that still gives every CU of an MI355X work: 256x256 (five-slot ring
+    // kernel) from 128 such tiles on; below that 128x128 tiles, and 64x64 tiles (two workgroups
+    // per CU) when even those number at most 128.
+    const long long tiles256 = (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    const long long tiles128 =
+        (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
+    const int variant = !tile_ok ? 0 : tiles128 <= 128 ? 6 : tiles256 < 128 ? 5 : 4;
+    return hk_fp8_gemm_variant(A, B, C, M, N, K, scale_a, scale_b, variant, stream);
 }

@@ -217,6 +217,9 @@ __device__ __forceinline__ void grouped_raster(int id, int tiles_m, int tiles_n,
     const int in_group = id - group * per_group;
     pm = first_m + in_group % gsize;
     pn = in_group / gsize;
+    // odd groups run right to left: the B panels the previous group used last are the first ones
+    // the next group asks for, while they are still in the memory-side cache
+    if (group & 1) pn = tiles_n - 1 - pn;
 }
 
 }  // namespace hk

@@ -31,7 +31,13 @@ def _check_tensor(t, name: str, dtypes, ndim: int | None = None):
         raise RuntimeError(f"{name}: expected {ndim} dimensions, got {t.dim()}")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t) -> int:
+    """torch's current stream on t's device, as a hipStream_t value."""
+    if _raw_stream is not None:  # the same handle without building a Stream object (saves >1 us per call)
+        return _raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
@@ -47,7 +53,7 @@ def dispatch_fp8_gemm(A, B, C, scale_a: float = 1.0, scale_b: float = 1.0, varia
                       workspace=None) -> None:
     """C[M,N] (bf16) = (scale_a*A[M,K]) @ (scale_b*B[N,K]).T, A and B e4m3, fp32 accumulation.
 
-    `variant` -1 lets the library choose; 0..5 force a kernel (see include/hk355.h). `workspace`
+    `variant` -1 lets the library choose; 0..6 force a kernel (see include/hk355.h). `workspace`
     (uint8, fp8_gemm_workspace_bytes(M, N, K) bytes): lets the library split K for decode-like
     shapes (hk_fp8_gemm_ws)."""
     _check_tensor(A, "A", _FP8, 2)

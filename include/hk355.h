@@ -66,8 +66,10 @@ int hk_fp8_gemm_ws(const void* A_e4m3, const void* B_e4m3, void* C_bf16, int M, 
  * 4 waves, hand-interleaved schedule over two LDS stages, 3 = 256x256x128 tile, 4 waves, plain
  * loop, 4 = 256x256x128 tile, 4 waves, hand-interleaved schedule over a five-slot LDS ring with
  * the loads spread over the whole K-step (what hk_fp8_gemm picks when the problem has at least 128
- * such tiles), 5 = 128x128x128 tile, 4 waves, plain loop (picked for smaller problems).
- * Variants 1-3 need K % 128 == 0; 4 and 5 zero-fill the last K-step of any K % 16 == 0. */
+ * such tiles), 5 = 128x128x128 tile, 4 waves, plain loop over three LDS stages (picked for smaller
+ * problems), 6 = the same loop with 64x64 tiles and four stages, two workgroups per CU (picked
+ * when the problem has at most 128 tiles of 128x128).
+ * Variants 1-3 need K % 128 == 0; 4, 5 and 6 zero-fill the last K-step of any K % 16 == 0. */
 int hk_fp8_gemm_variant(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
                         int M, int N, int K, float scale_a, float scale_b,
                         int variant, void* stream);

@@ -35,7 +35,7 @@ SHAPES = [(256, 256, 256), (256, 256, 128), (512, 768, 384), (1024, 1024, 1024),
 RAGGED = [(300, 200, 256), (257, 255, 128), (64, 72, 640), (1000, 1000, 512)]
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 4, 5, -1])
+@pytest.mark.parametrize("variant", [0, 1, 2, 4, 5, 6, -1])
 @pytest.mark.parametrize("shape", SHAPES + RAGGED)
 def test_fp8_gemm_matches_oracle(hk, shape, variant):
     M, N, K = shape
@@ -53,11 +53,11 @@ def test_fp8_gemm_matches_oracle(hk, shape, variant):
 K_TAIL = [(96, 80, 208), (256, 256, 16), (256, 256, 144), (300, 520, 272), (512, 384, 2880), (128, 128, 112)]
 
 
-@pytest.mark.parametrize("variant", [0, 4, 5, -1])
+@pytest.mark.parametrize("variant", [0, 4, 5, 6, -1])
 @pytest.mark.parametrize("shape", K_TAIL)
 def test_fp8_gemm_k_tail(hk, shape, variant):
     """K % 16 == 0 but K % 128 != 0 (2880 is the hidden size of the MoE models): the ring and
-    128x128-tile kernels zero-fill the last K-step. The buffers are carved out of a larger one
+    128x128- / 64x64-tile kernels zero-fill the last K-step. The buffers are carved out of a larger one
     filled with NaN codes, so a read past a row's end would show in the result."""
     M, N, K = shape
     print(f"fp8_gemm k-tail shape={shape} variant={variant}", flush=True)
@@ -75,7 +75,7 @@ def test_fp8_gemm_k_tail_last_row_does_not_read_past_the_buffer(hk):
     rng = np.random.default_rng(99)
     (a, sa), (b, sb) = _random_codes(rng, M, K), _random_codes(rng, N, K)
     dev = torch.device("cuda:0")
-    for variant in (4, 5):
+    for variant in (4, 5, 6):
         pool = torch.full((4 * M * K,), 0x7F, dtype=torch.uint8, device=dev)  # e4m3fn NaN code
         A = pool[M * K:2 * M * K].view(M, K)
         B = pool[2 * M * K:3 * M * K].view(N, K)
@@ -90,7 +90,7 @@ def test_fp8_gemm_k_tail_last_row_does_not_read_past_the_buffer(hk):
         assert G.rel_fro_error(out, G.fp8_gemm(a, b, sa, sb)) <= 5e-3
 
 
-SPLITK = [(16, 1024, 4096), (64, 512, 8192), (100, 520, 2048), (128, 1024, 2064), (1, 128, 1024), (33, 200, 4096)]
+SPLITK = [(16, 1024, 8192), (64, 512, 8192), (100, 520, 6160), (128, 1024, 6144), (1, 128, 8192), (33, 200, 12288)]
 
 
 @pytest.mark.parametrize("shape", SPLITK)
@@ -121,8 +121,9 @@ def test_fp8_gemm_split_k_matches_oracle(hk, shape):
 
 
 def test_fp8_gemm_workspace_is_optional(hk):
-    # a shape that is not split (enough tiles): zero bytes, and a workspace changes nothing
+    # shapes that are not split (enough tiles, or a short K): zero bytes, and a workspace changes nothing
     assert hk.tk_kernel.fp8_gemm_workspace_bytes(2048, 2048, 1024) == 0
+    assert hk.tk_kernel.fp8_gemm_workspace_bytes(1024, 1024, 1024) == 0
     rng = np.random.default_rng(5)
     (a, sa), (b, sb) = _random_codes(rng, 256, 256), _random_codes(rng, 256, 256)
     base = _run(hk, a, b, float(sa), float(sb), -1)
@@ -143,7 +144,7 @@ def test_fp8_gemm_older_tile_kernels_refuse_k_tail(hk, variant):
         _run(hk, a, b, 1.0, 1.0, variant)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 4, 5])
+@pytest.mark.parametrize("variant", [0, 1, 2, 4, 5, 6])
 def test_fp8_gemm_identity_is_bit_exact(hk, variant):
     """A = I (K = M): C = bf16(B^T) exactly; every e4m3 value is a bf16 value."""
     n = 256
@@ -158,7 +159,7 @@ def test_fp8_gemm_identity_is_bit_exact(hk, variant):
     assert np.array_equal(F.bf16_to_f32(out), F.bf16_to_f32(expect))
 
 
-@pytest.mark.parametrize("variant", [1, 2, 4, 5])
+@pytest.mark.parametrize("variant", [1, 2, 4, 5, 6])
 def test_fp8_gemm_small_integers_exact(hk, variant):
     """Operands in {-2..2}: all products and partial sums are exact in fp32, so the result is
     order independent and must equal the integer matmul, rounded once to bf16."""
