@@ -91,6 +91,59 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_rows_kernel(const uint16_t
     if ((c8 & 3) == 0) scales[(size_t)row * scale_pitch + (c8 >> 2)] = (uint8_t)(e + 127);
 }
 
+// Item lists of the two grouped GEMMs of a layer: list `which` (0 / 1) covers n_tiles[which] tiles
+// of weight rows and goes to items[which], its length to num_items[which]. One workgroup of NT
+// threads per list; thread t owns experts [t * 512 / NT, (t + 1) * 512 / NT). `scan`: NT ints of LDS.
+struct MoeBuildItems { MoeItem* items[2]; int n_tiles[2]; int bm; };
+template <int NT>
+__device__ __forceinline__ void moe_build_items_block(const int32_t* __restrict__ expert_offsets, int E,
+                                                      const MoeBuildItems& b, int which,
+                                                      int32_t* __restrict__ num_items, int* scan) {
+    constexpr int EPT = 512 / NT;
+    const int n_tiles_n = b.n_tiles[which], bm = b.bm;
+    MoeItem* __restrict__ items = b.items[which];
+    const int t = threadIdx.x;
+    int lo[EPT], hi[EPT], cnt[EPT], mine = 0;
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+        const int e = t * EPT + j;
+        lo[j] = hi[j] = cnt[j] = 0;
+        if (e < E) {
+            lo[j] = expert_offsets[e]; hi[j] = expert_offsets[e + 1];
+            cnt[j] = (hi[j] - lo[j] + bm - 1) / bm;
+        }
+        mine += cnt[j] * n_tiles_n;
+    }
+    scan[t] = mine;
+    __syncthreads();
+    for (int d = 1; d < NT; d <<= 1) {
+        const int v = t >= d ? scan[t - d] : 0;
+        __syncthreads();
+        scan[t] += v;
+        __syncthreads();
+    }
+    int base = scan[t] - mine;
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+        for (int n = 0; n < n_tiles_n; ++n)
+            for (int m = 0; m < cnt[j]; ++m) {
+                MoeItem it;
+                it.expert = t * EPT + j; it.row_start = lo[j] + m * bm; it.rows = min(bm, hi[j] - it.row_start);
+                it.n_tile = n;
+                items[base + n * cnt[j] + m] = it;
+            }
+        base += cnt[j] * n_tiles_n;
+    }
+    if (t == NT - 1) num_items[which] = scan[NT - 1];
+}
+
+__global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __restrict__ expert_offsets,
+                                                              int E, MoeBuildItems b,
+                                                              int32_t* __restrict__ num_items) {
+    __shared__ int scan[512];
+    moe_build_items_block<512>(expert_offsets, E, b, blockIdx.x, num_items, scan);
+}
+
 // Activation layout inside the MoE ("K-step-major tiles"): for a matrix of S rows the bytes of
 // K-step kt (256 elements = 128 bytes per row, zero-padded past K) of all rows are contiguous,
 //   data   [nk][S][128] bytes,   scales [nk][S][8] e8m0 bytes (padding = 127),
@@ -102,11 +155,20 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_rows_kernel(const uint16_t
 // The same launch pads the second tiled matrix of the layer (h, contraction length K2): the part
 // of its last K-step past K2 that the producing GEMM epilogue never writes is set to zero data
 // and neutral scales (nothing to do when K2 is a multiple of 256).
-// Launch: 128 threads = 4 K-steps x 32 threads (8 elements each); grid (S, ceil(nk / 4)).
+// Launch: 128 threads = 4 K-steps x 32 threads (8 elements each); grid (S + 2, ceil(nk / 4)).
+// The two workgroups past S (blockIdx.y == 0) build the layer's two work-item lists instead, which
+// need only expert_offsets and so ride along in the shadow of the quantization.
 __global__ __launch_bounds__(128) void mxfp4_quantize_permute_kernel(
     const uint16_t* __restrict__ x, const int32_t* __restrict__ sorted_slots, int topk, int S, int cols,
     uint8_t* __restrict__ tiled, uint8_t* __restrict__ tiled_scales, uint8_t* __restrict__ tiled2,
-    uint8_t* __restrict__ tiled2_scales, int K2) {
+    uint8_t* __restrict__ tiled2_scales, int K2, const int32_t* __restrict__ expert_offsets, int E,
+    MoeBuildItems items, int32_t* __restrict__ num_items) {
+    __shared__ int scan[128];
+    if ((int)blockIdx.x >= S) {
+        if (blockIdx.y == 0)
+            moe_build_items_block<128>(expert_offsets, E, items, (int)blockIdx.x - S, num_items, scan);
+        return;
+    }
     const int nk = (cols / 2 + 127) >> 7;
     const int pos = blockIdx.x;
     const int kt = blockIdx.y * 4 + (threadIdx.x >> 5), c = threadIdx.x & 31;  // K-step, 4-byte column
@@ -196,40 +258,6 @@ __global__ __launch_bounds__(256) void moe_preshuffle_kernel(const uint8_t* __re
             dst[b] = blk < (K >> 5) ? sc[((size_t)e * rows_b + rw) * scale_pitch + blk] : (uint8_t)127;
         }
     }
-}
-
-// Item lists of both grouped GEMMs of a layer in one launch: workgroup 0 builds the list for
-// n_tiles[0] tiles of weight rows into items[0], workgroup 1 the one for n_tiles[1].
-struct MoeBuildItems { MoeItem* items[2]; int n_tiles[2]; int bm; };
-__global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __restrict__ expert_offsets,
-                                                              int E, MoeBuildItems b,
-                                                              int32_t* __restrict__ num_items) {
-    __shared__ int scan[512];
-    const int which = blockIdx.x;
-    const int n_tiles_n = b.n_tiles[which], bm = b.bm;
-    MoeItem* __restrict__ items = b.items[which];
-    const int e = threadIdx.x;
-    int lo = 0, hi = 0, cnt = 0;
-    if (e < E) {
-        lo = expert_offsets[e]; hi = expert_offsets[e + 1];
-        cnt = (hi - lo + bm - 1) / bm;
-    }
-    scan[e] = cnt * n_tiles_n;
-    __syncthreads();
-    for (int d = 1; d < 512; d <<= 1) {
-        const int v = e >= d ? scan[e - d] : 0;
-        __syncthreads();
-        scan[e] += v;
-        __syncthreads();
-    }
-    const int base = scan[e] - cnt * n_tiles_n;
-    for (int n = 0; n < n_tiles_n; ++n)
-        for (int m = 0; m < cnt; ++m) {
-            MoeItem it;
-            it.expert = e; it.row_start = lo + m * bm; it.rows = min(bm, hi - it.row_start); it.n_tile = n;
-            items[base + n * cnt + m] = it;
-        }
-    if (e == 511) num_items[which] = scan[511];
 }
 
 // ---------------------------------------------------------------------------- grouped GEMM
@@ -1134,16 +1162,17 @@ extern "C" int hk_moe_mxfp4_experts_ex(const void* x_bf16, const void* w13, cons
     uint8_t* ws = (uint8_t*)workspace;
     const int S = T * k;
 
+    int32_t* nitems = (int32_t*)(ws + L.nitems);
     {
         const int nk1 = (H / 2 + 127) / 128;
-        hipLaunchKernelGGL(mxfp4_quantize_permute_kernel, dim3(S, (nk1 + 3) / 4), dim3(128), 0, s,
+        MoeBuildItems b;
+        b.bm = weight_layout ? kStBM : kMoeBM;
+        b.items[0] = (MoeItem*)(ws + L.items1); b.items[1] = (MoeItem*)(ws + L.items2);
+        b.n_tiles[0] = (I + 127) / 128; b.n_tiles[1] = (H + 255) / 256;
+        hipLaunchKernelGGL(mxfp4_quantize_permute_kernel, dim3(S + 2, (nk1 + 3) / 4), dim3(128), 0, s,
                            (const uint16_t*)x_bf16, sorted_slots, k, S, H, ws + L.xq, ws + L.xs, ws + L.hq,
-                           ws + L.hs, I);
+                           ws + L.hs, I, expert_offsets, E, b, nitems);
     }
-    int32_t* nitems = (int32_t*)(ws + L.nitems);
-    moe_launch_build_items(expert_offsets, E, weight_layout ? kStBM : kMoeBM, (I + 127) / 128,
-                           (MoeItem*)(ws + L.items1), (H + 255) / 256,
-                           (MoeItem*)(ws + L.items2), nitems, s);
 
     MoeGemmParams p{};
     p.A = ws + L.xq; p.SA = ws + L.xs; p.S = S;

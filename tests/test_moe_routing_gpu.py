@@ -68,7 +68,11 @@ def _sort(hk, ids_np, E):
     return ss.cpu().numpy(), off.cpu().numpy(), inv.cpu().numpy()
 
 
-@pytest.mark.parametrize("T,k,E", [(4096, 4, 128), (8192, 8, 256), (1, 1, 1), (3, 2, 512), (1000, 3, 7), (257, 4, 16)])
+# up to 16384 slots: one workgroup does the whole sort; above: count / scan / scatter launches, with the
+# scan in one workgroup up to 64 chunks of 1024 slots
+@pytest.mark.parametrize("T,k,E", [(4096, 4, 128), (8192, 8, 256), (1, 1, 1), (3, 2, 512), (1000, 3, 7), (257, 4, 16),
+                                   (16384, 1, 512), (16385, 1, 512), (4097, 4, 128), (2048, 8, 3), (65, 1, 2),
+                                   (1023, 16, 300), (40000, 2, 100)])
 def test_moe_sort(hk, T, k, E):
     rng = np.random.default_rng(T * 7 + k)
     ids = np.stack([rng.permutation(E)[:k] if k <= E else rng.integers(0, E, k) for _ in range(T)]).astype(np.int32)
