@@ -683,14 +683,22 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
     const uint32_t voff_b = lane * 16, voff_sb = lane * 4;
     v4i bw[4][2][NT];  // [K-step mod 4][K half][fragment]
     int bsc[4];        // [K-step mod 4]: the lane's scale bytes, byte 2 * half + fragment
+    // Bytes of the last K-step that lie inside K (the layout pads every row to whole K-steps with
+    // zeros): lane l's 16 bytes of half h start at byte 64 h + 16 (l / 16) of the K-step. Lanes
+    // past the end get bit 31 in their offset: outside the buffer, so the load returns the same
+    // zeros without fetching them (K = 2880: 6 % of the weight bytes).
+    const int last_valid = Kb - (nk - 1) * 128;
     auto load_b_half = [&](const Cursor& c, v4i (&dst)[NT], int half) __attribute__((always_inline)) {
         const v4i rs = cb_srd_b;
         const uint32_t soff = (uint32_t)c.kt * kMoeBTile + (uint32_t)w * 4096u + (uint32_t)half * 1024u;
+        // first padded lane * 16 - 1 (uniform); voff_b = 16 l exceeds it exactly in the padded lanes
+        const int thr = c.kt == nk - 1 ? 16 * min(max(last_valid - 64 * half, 0), 64) - 1 : 0x7fffffff;
+        const uint32_t voff = voff_b | ((uint32_t)(thr - (int)voff_b) & 0x80000000u);
 #pragma unroll
         for (int n = 0; n < NT; ++n)
             asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"
                          : "=v"(dst[n])
-                         : "v"(voff_b), "s"(rs), "s"(soff + n * 2048u)
+                         : "v"(voff), "s"(rs), "s"(soff + n * 2048u)
                          : "memory");
     };
     auto load_b_scales = [&](const Cursor& c, int& dst) __attribute__((always_inline)) {
