@@ -101,7 +101,10 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const float* __re
 #pragma unroll
         for (int i = 0; i < kMaxPerLane; ++i)
             if (cand[i] == best) cand[i] = 0ull;  // ids are unique, only the owner matches
-        const float v = row[id];
+        // the logit back from its key (exact; -0 comes back as +0, which the softmax cannot tell apart):
+        // no dependent reload of row[id]
+        const uint32_t key = (uint32_t)(best >> 32);
+        const float v = __uint_as_float((key & 0x80000000u) ? key ^ 0x80000000u : ~key);
         if (j == 0) top_logit = v;
         if (sub == j) { my_logit = v; my_id = id; }
     }
