@@ -149,7 +149,7 @@ def bench_mxfp4(torch, hk, n, warmup, iters, dev):
             "frac_of_mxfp4_peak": round(tf / PEAK_FP4, 4)}
 
 
-def bench_moe_mxfp4(torch, hk, warmup, iters, dev):
+def bench_moe_mxfp4(torch, hk, warmup, iters, dev, graph=True):
     T, E, k, H, I = 4096, 128, 4, 2880, 2880
     g = torch.Generator(device=dev).manual_seed(0)
     x = torch.randn(T, H, device=dev, generator=g).to(torch.bfloat16)
@@ -173,7 +173,7 @@ def bench_moe_mxfp4(torch, hk, warmup, iters, dev):
                       warmup, iters)
     # the layer's nine launches replayed from a HIP graph (no host work or launch gaps between them)
     kern_graph = _timeit_graph(torch, lambda: hk.tk_kernel.dispatch_moe_mxfp4(x, logits, W, None, None, None, y, k, ws),
-                               y, iters)
+                               y, iters) if graph else None
     flop = 2.0 * T * k * (H * 2 * I + I * H)
     tf = flop / (kern * 1e-3) / 1e12
     compulsory = wbytes + 2 * T * H * 2  # weights once + x in + y out
@@ -188,7 +188,7 @@ def bench_moe_mxfp4(torch, hk, warmup, iters, dev):
             "ms": round(kern, 5), "tflops": round(tf, 1), "frac_of_mxfp4_peak": round(tf / PEAK_FP4, 4),
             "compulsory_GB": round(compulsory / 1e9, 3),
             "frac_of_hbm_roofline": round(compulsory / (kern * 1e-3) / 1e9 / PEAK_HBM, 4),
-            "ms_graph_replay": round(kern_graph, 5), "ms_with_biases_and_clamped_swiglu": round(kern_oai, 5)}
+            "ms_graph_replay": round(kern_graph, 5) if graph else None, "ms_with_biases_and_clamped_swiglu": round(kern_oai, 5)}
 
 
 def bench_moe_fp8blk(torch, hk, warmup, iters, dev):
@@ -275,6 +275,7 @@ def main() -> int:
     ap.add_argument("--only-headline", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--traffic-calibration", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph timings (for runs under a profiler)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (--gpus 1); "
@@ -321,7 +322,8 @@ def main() -> int:
     if not args.only_headline:
         quick_w, quick_i = 20, 20
         extra["mfma_fp8_ceiling_tflops_for_this_data"] = round(mfma_ceiling(torch, hk, head["A"], dev), 1)
-        sweep = {m: bench_fp8(torch, hk, m, 50, 50, dev, graph=m <= 4096) for m in (1024, 2048, 4096, 16384)}
+        sweep = {m: bench_fp8(torch, hk, m, 50, 50, dev, graph=m <= 4096 and not args.no_graph)
+                 for m in (1024, 2048, 4096, 16384)}
         # per call through the Python boundary (about 9 us of host time per call bounds the small sizes) ...
         extra["fp8_gemm_sweep_tflops"] = {str(m): round(r["tflops"], 1) for m, r in sweep.items()}
         # ... and the same calls replayed from a HIP graph (GPU time only, like the reference's C++ loop)
@@ -334,7 +336,7 @@ def main() -> int:
         extra["fp8_gemm_decode"] = bench_fp8_decode(torch, hk, 50, 50, dev)
         extra["bf16_gemm"] = bench_bf16(torch, hk, 8192, 50, 50, dev)
         extra["mxfp4_gemm"] = bench_mxfp4(torch, hk, 8192, 50, 50, dev)
-        extra["moe_mxfp4"] = bench_moe_mxfp4(torch, hk, quick_w, quick_i, dev)
+        extra["moe_mxfp4"] = bench_moe_mxfp4(torch, hk, quick_w, quick_i, dev, graph=not args.no_graph)
         torch.cuda.empty_cache()
         extra["moe_fp8blk"] = bench_moe_fp8blk(torch, hk, 5, 10, dev)
         torch.cuda.empty_cache()
