@@ -107,6 +107,31 @@ def bench_fp8_reference_inputs(torch, hk, n, warmup, iters, dev):
             "tflops": round(tf, 1), "vs_reference_3327.46": round(tf / 3327.46, 4) if n == 8192 else None}
 
 
+def bench_library_baselines(torch, n, warmup, iters, dev):
+    """The vendor library on the same box and the same inputs, for reference only (nothing in the
+    product path calls it): hipBLASLt behind torch._scaled_mm for FP8, torch.matmul for bf16. The
+    reference's own table gives hipBLASLt 3233 and torch bf16 1521 TFLOP/s at 8192^3 on its MI355X
+    (analysis/fp8_gemm/mi350x/mi355x_fp8_gemm.json:20-25, analysis/bf16_gemm/mi350x/mi355x_bf16_gemm.json)."""
+    out = {}
+    g = torch.Generator(device=dev).manual_seed(0)
+    a = torch.randn(n, n, device=dev, generator=g)
+    b = torch.randn(n, n, device=dev, generator=g)
+    try:
+        sa, sb = (a.abs().max() / 448).float(), (b.abs().max() / 448).float()
+        A, B = (a / sa).to(torch.float8_e4m3fn), (b / sb).to(torch.float8_e4m3fn)
+        _, ms = _timeit(torch, lambda: torch._scaled_mm(A, B.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16),
+                        warmup, iters)
+        out["hipblaslt_fp8_tflops"] = round(2.0 * n ** 3 / (ms * 1e-3) / 1e12, 1)
+        del A, B
+    except Exception as ex:  # this torch build may not expose the call: the comparison is optional
+        out["hipblaslt_fp8_tflops"] = f"unavailable: {type(ex).__name__}"
+    Ab, Bb = a.to(torch.bfloat16), b.to(torch.bfloat16)
+    del a, b
+    _, ms = _timeit(torch, lambda: torch.matmul(Ab, Bb.t()), warmup, iters)
+    out["torch_bf16_matmul_tflops"] = round(2.0 * n ** 3 / (ms * 1e-3) / 1e12, 1)
+    return out
+
+
 def bench_bf16(torch, hk, n, warmup, iters, dev):
     g = torch.Generator(device=dev).manual_seed(0)
     A = torch.randn(n, n, device=dev, generator=g).to(torch.bfloat16)
@@ -335,6 +360,8 @@ def main() -> int:
         extra["fp8_gemm_reference_inputs"] = bench_fp8_reference_inputs(torch, hk, n, 100, 100, dev)
         extra["fp8_gemm_decode"] = bench_fp8_decode(torch, hk, 50, 50, dev)
         extra["bf16_gemm"] = bench_bf16(torch, hk, 8192, 50, 50, dev)
+        extra["library_on_this_box_8192"] = bench_library_baselines(torch, 8192, 50, 50, dev)
+        torch.cuda.empty_cache()
         extra["mxfp4_gemm"] = bench_mxfp4(torch, hk, 8192, 50, 50, dev)
         extra["moe_mxfp4"] = bench_moe_mxfp4(torch, hk, quick_w, quick_i, dev, graph=not args.no_graph)
         torch.cuda.empty_cache()
