@@ -9,6 +9,7 @@
 // two 16-byte halves a lane reads per fragment row are K elements 8g.. and 32 + 8g.. and feed
 // two v_mfma_f32_16x16x32_bf16 (16 cycles each, together as long as one FP8 MFMA).
 #include "gemm_tile.h"
+#include "gemm_small_tile.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -249,6 +250,45 @@ __global__ __launch_bounds__(256) void bf16_gemm_portable_kernel(
     }
 }
 
+// Small-tile kernels (gemm_small_tile.h) with the bf16 MFMA: the two 16-byte halves of a fragment
+// row are K elements 8g.. and 32 + 8g.. of the 64-element K-step, one v_mfma_f32_16x16x32_bf16 each.
+struct Bf16Mma {
+    typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+    static __device__ __forceinline__ void mma(v4f& acc, const v8i& b, const v8i& a) {
+        const v4i blo = {b[0], b[1], b[2], b[3]}, bhi = {b[4], b[5], b[6], b[7]};
+        const v4i alo = {a[0], a[1], a[2], a[3]}, ahi = {a[4], a[5], a[6], a[7]};
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, blo), __builtin_bit_cast(v8bf, alo),
+                                                      acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, bhi), __builtin_bit_cast(v8bf, ahi),
+                                                      acc, 0, 0, 0);
+    }
+};
+template <int TILE, int STAGES, bool EDGE>
+__global__ __launch_bounds__(256) void bf16_gemm_small_tile_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, int tiles_m, int tiles_n) {
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    gemm_small_tile_body<Bf16Mma, TILE, STAGES, EDGE, false>(smem, A, B, C, M, N, 2 * K, 1.0f, tiles_m, tiles_n, 0,
+                                                             nullptr);
+}
+
+template <int TILE, int STAGES, bool EDGE>
+static int launch_bf16_small_tile(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream) {
+    auto kern = bf16_gemm_small_tile_kernel<TILE, STAGES, EDGE>;
+    constexpr int lds_bytes = STAGES * 2 * TILE * BK;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) !=
+            hipSuccess)
+            return HK_ERR_LAUNCH;
+        configured = true;
+    }
+    const int tiles_m = (M + TILE - 1) / TILE, tiles_n = (N + TILE - 1) / TILE;
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream, (const uint8_t*)A,
+                       (const uint8_t*)B, (uint16_t*)C, M, N, K, tiles_m, tiles_n);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
 template <bool EDGE>
 static int launch_bf16_ring(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream) {
     auto kern = bf16_gemm_4wave_ring_kernel<EDGE>;
@@ -274,7 +314,7 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 8) != 0) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < 0 || variant > 1) return HK_ERR_UNSUPPORTED;
+    if (variant < 0 || variant > 3) return HK_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {
         if ((long long)((M + 63) / 64) > 65535) return HK_ERR_BAD_SHAPE;
@@ -284,11 +324,27 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
         return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
     }
     if ((long long)2 * K * BM >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
+    if (variant == 2) {
+        const bool edge128 = (M % kSmallTile) != 0 || (N % kSmallTile) != 0;
+        return edge128 ? launch_bf16_small_tile<kSmallTile, kSmallStages, true>(A, B, C, M, N, K, s)
+                       : launch_bf16_small_tile<kSmallTile, kSmallStages, false>(A, B, C, M, N, K, s);
+    }
+    if (variant == 3) {
+        const bool edge64 = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
+        return edge64 ? launch_bf16_small_tile<kTinyTile, kTinyStages, true>(A, B, C, M, N, K, s)
+                      : launch_bf16_small_tile<kTinyTile, kTinyStages, false>(A, B, C, M, N, K, s);
+    }
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
     return edge ? launch_bf16_ring<true>(A, B, C, M, N, K, s) : launch_bf16_ring<false>(A, B, C, M, N, K, s);
 }
 
 extern "C" int hk_bf16_gemm(const void* A, const void* B, void* C, int M, int N, int K, void* stream) {
-    const bool tile_ok = K > 0 && (long long)2 * K * hk::BM < (1ll << 31) && M >= 64 && N >= 64;
-    return hk_bf16_gemm_variant(A, B, C, M, N, K, tile_ok ? 1 : 0, stream);
+    using namespace hk;
+    const bool tile_ok = K > 0 && (long long)2 * K * BM < (1ll << 31) && M >= 16 && N >= 16;
+    // the same choice of tile as hk_fp8_gemm: the largest that still gives every CU work
+    const long long tiles256 = (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    const long long tiles128 =
+        (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
+    const int variant = !tile_ok ? 0 : tiles128 <= 128 ? 3 : tiles256 < 128 ? 2 : 1;
+    return hk_bf16_gemm_variant(A, B, C, M, N, K, variant, stream);
 }

@@ -13,6 +13,7 @@
 // the B tile's rows are permuted on their way into LDS so that two neighbouring
 // MFMA tiles give a lane 8 consecutive columns = one 16-byte bf16 store.
 #include "gemm_tile.h"
+#include "gemm_small_tile.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -468,152 +469,19 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
-// 128x128-tile kernel for problems with too few 256x256 tiles to occupy the chip (a 1024^3
-// GEMM has 16 of them for 256 CUs): 4 waves, each a 64x64 patch (16 MFMA tiles), three LDS
-// stages of 2 x 16 KiB with two K-steps of loads in flight, plain loop (such problems are
-// bound by launch, prologue and epilogue latency, not by the K loop's schedule). Same tile
-// format, B-row permutation and epilogue as the large-tile kernels.
-constexpr int kSmallTile = 128;
-constexpr int kSmallTileBytes = kSmallTile * BK;          // 16 KiB per operand
-constexpr int kSmallStageBytes = 2 * kSmallTileBytes;
-constexpr int kSmallStages = 3;
-constexpr int kSmallLdsBytes = kSmallStages * kSmallStageBytes;  // 96 KiB
-// the same kernel with 64x64 tiles and four 16 KiB stages (two workgroups per CU): for problems
-// with so few 128x128 tiles that a quarter of the tile is needed to give every CU work
-constexpr int kTinyTile = 64;
-constexpr int kTinyStages = 4;
-
-// SPLIT: blockIdx.y selects a range of `kps` K-steps; the tile's fp32 partial sums go to
-// partial[blockIdx.y][M][N] (plain stores; splitk_reduce_kernel adds the ranges in order, so the
-// result does not depend on timing). For problems with few tiles and a long K (decode-like
-// shapes), where a single workgroup per tile walks K one K-step latency at a time.
+// Small-tile kernels (gemm_small_tile.h) with the FP8 MFMA.
+struct Fp8Mma {
+    static __device__ __forceinline__ void mma(v4f& acc, const v8i& b, const v8i& a) {
+        acc = mfma_fp8_16x16x128(b, a, acc);
+    }
+};
 template <int TILE, int STAGES, bool EDGE, bool SPLIT>
 __global__ __launch_bounds__(256) void fp8_gemm_small_tile_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
     int M, int N, int K, float alpha, int tiles_m, int tiles_n, int kps, float* __restrict__ partial) {
-    constexpr int NW = 4, TM = TILE / 2, TN = TILE / 2, MT = TM / 16, NT = TN / 16;
-    constexpr int kTB = TILE * BK, kSB = 2 * kTB;    // bytes of one operand tile / of one stage
-    constexpr int NDMA = kTB / (NW * 1024);          // loads per wave per operand per K-step
-    static_assert(STAGES >= 3 && STAGES <= 8 && (STAGES - 2) * 2 * NDMA < 64, "vmcnt range");
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
-    const int lane = lane_id(), w = wave_id();
-    const int wm = w >> 1, wn = w & 1;
-
-    int pm, pn;
-    {
-        const int id = xcd_chunk_order(blockIdx.x, tiles_m * tiles_n, kCuPerXcd);
-        grouped_raster(id, tiles_m, tiles_n, 8, pm, pn);
-    }
-    const int row0 = pm * TILE, col0 = pn * TILE;
-    const int a_rows = min(M - row0, TILE), b_rows = min(N - col0, TILE);
-    const v4i srd_a = make_srd(A + (size_t)row0 * K, (uint32_t)a_rows * (uint32_t)K);
-    const v4i srd_b = make_srd(B + (size_t)col0 * K, (uint32_t)b_rows * (uint32_t)K);
-
-    uint32_t voff_a[NDMA], voff_b[NDMA];
-#pragma unroll
-    for (int i = 0; i < NDMA; ++i) {
-        const int R = 8 * (i * NW + w) + (lane >> 3);
-        const uint32_t c = swz_chunk(R, lane & 7);
-        int ra = R, rb = b_row_to_col(R);
-        if (EDGE) {
-            ra = min(ra, a_rows - 1);
-            rb = min(rb, b_rows - 1);
-        }
-        voff_a[i] = (uint32_t)ra * (uint32_t)K + c * 16u;
-        voff_b[i] = (uint32_t)rb * (uint32_t)K + c * 16u;
-    }
-    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
-    const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-    const int nk = (K + BK - 1) / BK;
-    // last K-step of a K that is not a multiple of 128: lanes whose 16-byte chunk lies past the
-    // end of the row are moved out of the buffer's range (bit 31) and write zeros to LDS
-    const uint32_t tail_or =
-        (int)(swz_chunk(8 * w + (lane >> 3), lane & 7) * 16u) >= K - (nk - 1) * BK ? 0x80000000u : 0u;
-    // this workgroup's K-steps: [kt0, kt0 + nkt)
-    const int kt0 = SPLIT ? (int)blockIdx.y * kps : 0;
-    const int nkt = SPLIT ? min(kps, nk - kt0) : nk;
-    auto issue_tile = [&](int stage, int kt_local) {
-        const int kt = kt0 + kt_local;
-        const uint32_t k0 = (uint32_t)kt * BK;
-        const uint32_t dst = lds_wave + (uint32_t)stage * kSB;
-        const uint32_t vor = kt == nk - 1 ? tail_or : 0u;
-#pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma16(srd_a, dst + i * NW * 1024, voff_a[i] | vor, k0);
-#pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma16(srd_b, dst + kTB + i * NW * 1024, voff_b[i] | vor, k0);
-    };
-    // wait until at most `tiles` of the most recently issued K-steps' loads are still in flight
-    auto wait_tiles = [&](int tiles) {
-        switch (tiles) {
-            case 0: wait_vmcnt<0>(); break;
-            case 1: wait_vmcnt<2 * NDMA>(); break;
-            case 2: wait_vmcnt<(STAGES > 3 ? 2 : 1) * 2 * NDMA>(); break;
-            case 3: wait_vmcnt<(STAGES > 4 ? 3 : 1) * 2 * NDMA>(); break;
-            case 4: wait_vmcnt<(STAGES > 5 ? 4 : 1) * 2 * NDMA>(); break;
-            case 5: wait_vmcnt<(STAGES > 6 ? 5 : 1) * 2 * NDMA>(); break;
-            default: wait_vmcnt<(STAGES > 7 ? 6 : 1) * 2 * NDMA>(); break;
-        }
-    };
-
-    const uint32_t r = lane & 15, g = lane >> 4;
-    const uint32_t rd_lo = r * 128u + swz_chunk(r, g) * 16u;
-    const uint32_t rd_hi = r * 128u + swz_chunk(r, g + 4) * 16u;
-    const uint32_t a_lo0 = lds0 + wm * (TM * BK) + rd_lo, a_hi0 = lds0 + wm * (TM * BK) + rd_hi;
-    const uint32_t b_lo0 = lds0 + kTB + wn * (TN * BK) + rd_lo;
-    const uint32_t b_hi0 = lds0 + kTB + wn * (TN * BK) + rd_hi;
-
-    v4f acc[MT][NT];
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
-
-    // K-steps kt .. kt + STAGES - 2 are in flight or in LDS while step kt is multiplied
-#pragma unroll
-    for (int p = 0; p < STAGES - 1; ++p)
-        if (p < nkt) issue_tile(p, p);
-    int st = 0;
-    for (int kt = 0; kt < nkt; ++kt) {
-        // this wave's part of K-step kt has landed (the loads of the steps behind it may still fly)
-        wait_tiles(min(nkt - 1 - kt, STAGES - 2));
-        block_barrier();  // ... everyone's; and everyone is done with the stage of K-step kt - 1
-        if (kt + STAGES - 1 < nkt) issue_tile(st == 0 ? STAGES - 1 : st - 1, kt + STAGES - 1);
-        const uint32_t so = (uint32_t)st * kSB;
-        v8i bf[NT];
-#pragma unroll
-        for (int n = 0; n < NT; ++n) bf[n] = lds_frag(b_lo0 + so, b_hi0 + so, n * 16 * BK);
-#pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            const v8i af = lds_frag(a_lo0 + so, a_hi0 + so, m * 16 * BK);
-#pragma unroll
-            for (int n = 0; n < NT; ++n) acc[m][n] = mfma_fp8_16x16x128(bf[n], af, acc[m][n]);
-        }
-        st = st == STAGES - 1 ? 0 : st + 1;
-    }
-    if (!SPLIT) {
-        store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
-    } else {
-        // fp32 partial sums: lane (r, g) holds, for row 16 m + r, columns 32 p + 8 g .. +8
-        float* out = partial + (size_t)blockIdx.y * M * N;
-#pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            const int row = row0 + wm * TM + 16 * m + (int)r;
-            if (row >= M) continue;
-#pragma unroll
-            for (int q = 0; q < NT / 2; ++q) {
-                const int col = col0 + wn * TN + 32 * q + 8 * (int)g;
-                float* dst = out + (size_t)row * N + col;
-                if (col + 8 <= N && (N & 3) == 0) {
-                    *(v4f*)dst = acc[m][2 * q];
-                    *(v4f*)(dst + 4) = acc[m][2 * q + 1];
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j)
-                        if (col + j < N) dst[j] = j < 4 ? acc[m][2 * q][j] : acc[m][2 * q + 1][j - 4];
-                }
-            }
-        }
-    }
+    gemm_small_tile_body<Fp8Mma, TILE, STAGES, EDGE, SPLIT>(smem, A, B, C, M, N, K, alpha, tiles_m, tiles_n, kps,
+                                                            partial);
 }
 
 // C = bf16(alpha * sum_s partial[s]) in split order; one thread per 4 columns.

@@ -83,7 +83,7 @@ def dispatch_fp8_gemm(A, B, C, scale_a: float = 1.0, scale_b: float = 1.0, varia
 
 def dispatch_bf16_gemm(A, B, C, variant: int = -1) -> None:
     """C[M,N] (bf16) = A[M,K] @ B[N,K].T for bf16 operands, fp32 accumulation
-    (include/hk355.h: hk_bf16_gemm). `variant` -1 lets the library choose; 0 / 1 force a kernel."""
+    (include/hk355.h: hk_bf16_gemm). `variant` -1 lets the library choose; 0..3 force a kernel."""
     _check_tensor(A, "A", _BF16, 2)
     _check_tensor(B, "B", _BF16, 2)
     _check_tensor(C, "C", _BF16, 2)

@@ -102,7 +102,9 @@ int hk_bf16_gemm(const void* A_bf16, const void* B_bf16, void* C_bf16, int M, in
                  void* stream);
 
 /* Same contract on a chosen kernel: 0 = portable kernel (any shape), 1 = 256x256x64 tile kernel
- * (the FP8 ring schedule; the last K-step of a K that is not a multiple of 64 is zero-filled). */
+ * (the FP8 ring schedule; the last K-step of a K that is not a multiple of 64 is zero-filled),
+ * 2 = 128x128 tiles / three LDS stages, 3 = 64x64 tiles / four stages (the FP8 GEMM's small-tile
+ * kernels with the bf16 MFMA; hk_bf16_gemm picks them by tile count as hk_fp8_gemm does). */
 int hk_bf16_gemm_variant(const void* A_bf16, const void* B_bf16, void* C_bf16, int M, int N, int K,
                          int variant, void* stream);
 
