@@ -41,8 +41,8 @@ __device__ __forceinline__ void mfma_fp4_acc(v4f& acc, const v4i& x, const v4i& 
 template <bool EDGE>
 __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
-    const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int tiles_m,
-    int tiles_n) {
+    const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int sa_pitch,
+    int sb_pitch, int tiles_m, int tiles_n) {
     constexpr int NW = 4, TM = 128, TN = 128, MT = 8, NT = 8;
     constexpr int NDMA = kTileBytes / (NW * 1024);
     constexpr int PG = 4, AD = 3;
@@ -52,8 +52,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     const int lane = lane_id();
     const int w = wave_id();
     const int wm = w >> 1, wn = w & 1;
-    const int Kb = K >> 1;   // operand row pitch in bytes
-    const int Ks = K >> 5;   // scale row pitch in bytes
+    const int Kb = K >> 1;   // operand row pitch in bytes (scale rows: sa_pitch / sb_pitch bytes)
 
     int pm, pn;
     {
@@ -64,8 +63,8 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     const int a_rows = min(M - row0, BM), b_rows = min(N - col0, BN);
     const v4i srd_a = make_srd(A + (size_t)row0 * Kb, (uint32_t)a_rows * (uint32_t)Kb);
     const v4i srd_b = make_srd(B + (size_t)col0 * Kb, (uint32_t)b_rows * (uint32_t)Kb);
-    const v4i srd_sa = make_srd(SA + (size_t)row0 * Ks, (uint32_t)a_rows * (uint32_t)Ks);
-    const v4i srd_sb = make_srd(SB + (size_t)col0 * Ks, (uint32_t)b_rows * (uint32_t)Ks);
+    const v4i srd_sa = make_srd(SA + (size_t)row0 * sa_pitch, (uint32_t)a_rows * (uint32_t)sa_pitch);
+    const v4i srd_sb = make_srd(SB + (size_t)col0 * sb_pitch, (uint32_t)b_rows * (uint32_t)sb_pitch);
 
     // operand tiles: as in the FP8 kernel
     uint32_t voff_a[EDGE ? NDMA : 1], voff_b[EDGE ? NDMA : 1];
@@ -91,20 +90,22 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
             ra = min(ra, a_rows - 1);
             rb = min(rb, b_rows - 1);
         }
-        voff_sa = (uint32_t)ra * (uint32_t)Ks;
-        voff_sb = (uint32_t)rb * (uint32_t)Ks;
+        voff_sa = (uint32_t)ra * (uint32_t)sa_pitch;
+        voff_sb = (uint32_t)rb * (uint32_t)sb_pitch;
     }
     const uint32_t dma_row_stride = to_sgpr((uint32_t)(8 * NW) * (uint32_t)Kb);
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
     const uint32_t lds_scale_wave = to_sgpr(lds0 + kScaleBase + (uint32_t)w * 1024u);
 
-    auto dma_one = [&](int op, int i, int stage, uint32_t k0, v4i srd) {
+    // `vor`: 0, or in the last K-step of a K that is not a multiple of 256 bit 31 for the lanes whose
+    // 16 bytes lie past the end of the row: out of the buffer's range, so zeros land in LDS
+    auto dma_one = [&](int op, int i, int stage, uint32_t k0, v4i srd, uint32_t vor) {
         const uint32_t dst = lds_wave + (uint32_t)stage * kStageBytes + op * kTileBytes + i * NW * 1024;
         if (EDGE)
-            dma16(srd, dst, op ? voff_b[i] : voff_a[i], k0);
+            dma16(srd, dst, (op ? voff_b[i] : voff_a[i]) | vor, k0);
         else
-            dma16(srd, dst, op ? voff_b[0] : voff_a[0], k0 + i * dma_row_stride);
+            dma16(srd, dst, (op ? voff_b[0] : voff_a[0]) | vor, k0 + i * dma_row_stride);
     };
     // this wave's scale load of operand `op` for the pair of K-steps `pair` (stage pair % 2)
     auto dma_scale = [&](int op, uint32_t pair, v4i srd) {
@@ -146,22 +147,25 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     Frag4 bf[2][NT], af[4];
     v2i bs[2][NT], as[4];
 
-    const int nk = K / 256;
+    const int nk = (Kb + BK - 1) / BK;
+    // the chunk a lane fetches is the same for all of its loads (see the FP8 kernel)
+    const uint32_t tail_or =
+        (int)(swz_chunk(8 * w + (lane >> 3), lane & 7) * 16u) >= Kb - (nk - 1) * BK ? 0x80000000u : 0u;
 
     // ---- prologue ----------------------------------------------------------------------
 #pragma unroll
-    for (int i = 0; i < NDMA; ++i) dma_one(0, i, 0, 0, srd_a);
+    for (int i = 0; i < NDMA; ++i) dma_one(0, i, 0, 0, srd_a, nk == 1 ? tail_or : 0u);
 #pragma unroll
-    for (int i = 0; i < NDMA; ++i) dma_one(1, i, 0, 0, srd_b);
+    for (int i = 0; i < NDMA; ++i) dma_one(1, i, 0, 0, srd_b, nk == 1 ? tail_or : 0u);
     dma_scale(0, 0, srd_sa);
     dma_scale(1, 0, srd_sb);
     wait_vmcnt<0>();
     block_barrier();
     if (nk > 1) {
 #pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma_one(0, i, 1, BK, srd_a);
+        for (int i = 0; i < NDMA; ++i) dma_one(0, i, 1, BK, srd_a, nk == 2 ? tail_or : 0u);
 #pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma_one(1, i, 1, BK, srd_b);
+        for (int i = 0; i < NDMA; ++i) dma_one(1, i, 1, BK, srd_b, nk == 2 ? tail_or : 0u);
     }
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
@@ -184,6 +188,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
         const uint32_t k2 = (uint32_t)(kt + 2) * BK;
         v4i sa = srd_a, sb = srd_b, ssa = srd_sa, ssb = srd_sb;
         if (kt + 2 >= nk) { sa.z = 0; sb.z = 0; ssa.z = 0; ssb.z = 0; }
+        const uint32_t vor = kt + 2 == nk - 1 ? tail_or : 0u;
         // scales of the next K-step: same pair (P == 0) or the next pair, in the other stage
         const uint32_t sa_nx = P ? sa_rd ^ kScaleStageBytes : sa_rd;
         const uint32_t sb_nx = P ? sb_rd ^ kScaleStageBytes : sb_rd;
@@ -211,7 +216,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
                         af[2] = lds_frag4(a_lo[P ^ 1], a_hi[P ^ 1], 2 * 16 * BK);
                         as[2] = rd_scale(sa_nx, P ^ 1, 2);
                     }
-                    if (j < 2 * NDMA) dma_one(j / NDMA, j % NDMA, P, k2, j / NDMA ? sb : sa);
+                    if (j < 2 * NDMA) dma_one(j / NDMA, j % NDMA, P, k2, j / NDMA ? sb : sa, vor);
                     // the next pair's scales: its stage was last read before this step's barrier
                     // of the previous odd K-step, and is first read after the next step's barrier
                     else if (P == 0 && j < 2 * NDMA + 2) dma_scale(j - 2 * NDMA, (uint32_t)(kt >> 1) + 1u, j - 2 * NDMA ? ssb : ssa);
@@ -255,12 +260,12 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
 // memory, K-step 128 elements (lane group g holds MX block g of the step).
 __global__ __launch_bounds__(256) void mxfp4_gemm_portable_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
-    const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K) {
+    const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int sa_pitch, int sb_pitch) {
     const int lane = lane_id(), w = wave_id();
     const int r = lane & 15, g = lane >> 4;
     const int row0 = blockIdx.y * 64 + (w >> 1) * 32;
     const int col0 = blockIdx.x * 64 + (w & 1) * 32;
-    const int Kb = K >> 1, Ks = K >> 5;
+    const int Kb = K >> 1;
     v4f acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -278,11 +283,11 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_portable_kernel(
             as[i] = 127; bs[i] = 127;
             if (ra < M && kk < K) {
                 af[i] = *(const v4i*)(A + (size_t)ra * Kb + (kk >> 1));
-                as[i] = SA[(size_t)ra * Ks + (kk >> 5)];
+                as[i] = SA[(size_t)ra * sa_pitch + (kk >> 5)];
             }
             if (rb < N && kk < K) {
                 bf[i] = *(const v4i*)(B + (size_t)rb * Kb + (kk >> 1));
-                bs[i] = SB[(size_t)rb * Ks + (kk >> 5)];
+                bs[i] = SB[(size_t)rb * sb_pitch + (kk >> 5)];
             }
         }
 #pragma unroll
@@ -308,7 +313,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_portable_kernel(
 
 template <bool EDGE>
 static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, const void* SB, void* C,
-                              int M, int N, int K, hipStream_t stream) {
+                              int M, int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
     auto kern = mxfp4_gemm_4wave_kernel<EDGE>;
     static bool configured = false;
     if (!configured) {
@@ -320,39 +325,60 @@ static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, cons
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), kLdsBytesFp4, stream,
                        (const uint8_t*)A, (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB,
-                       (uint16_t*)C, M, N, K, tiles_m, tiles_n);
+                       (uint16_t*)C, M, N, K, sa_pitch, sb_pitch, tiles_m, tiles_n);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
 }  // namespace hk
 
-extern "C" int hk_mxfp4_gemm_variant(const void* A, const void* A_scales, const void* B,
-                                     const void* B_scales, void* C, int M, int N, int K, int variant,
-                                     void* stream) {
+// variant: -1 = choose, 0 = portable kernel, 1 = tile kernel. Scale rows are sa_pitch / sb_pitch bytes
+// apart (>= K / 32).
+static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, const void* B, const void* B_scales,
+                           int sb_pitch, void* C, int M, int N, int K, int variant, void* stream) {
     using namespace hk;
     if (!A || !A_scales || !B || !B_scales || !C) return HK_ERR_NULL_POINTER;
-    if (M <= 0 || N <= 0 || K <= 0 || (K % 32) != 0) return HK_ERR_BAD_SHAPE;
+    if (M <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || sa_pitch < K / 32 || sb_pitch < K / 32)
+        return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < 0 || variant > 1) return HK_ERR_UNSUPPORTED;
+    if (variant < -1 || variant > 1) return HK_ERR_UNSUPPORTED;
+    // the tile kernel fetches a row's scales 16 bytes per lane, two K-steps of 8 bytes at a time:
+    // rows must start 4-byte aligned and hold whole groups of 8 bytes
+    const int groups = (K / 32 + 7) / 8 * 8;
+    const bool pitch_ok = (sa_pitch % 8) == 0 && (sb_pitch % 8) == 0 && sa_pitch >= groups && sb_pitch >= groups &&
+                          ((((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) == 0);
+    const bool size_ok = (long long)(K / 2) * BM < (1ll << 31) && (long long)BM * max(sa_pitch, sb_pitch) < (1ll << 31);
+    if (variant < 0) variant = pitch_ok && size_ok && M >= 64 && N >= 64 ? 1 : 0;
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {
         if ((M + 63) / 64 > 65535) return HK_ERR_BAD_SHAPE;
         dim3 grid((N + 63) / 64, (M + 63) / 64);
         hipLaunchKernelGGL(mxfp4_gemm_portable_kernel, grid, dim3(256), 0, s, (const uint8_t*)A,
                            (const uint8_t*)A_scales, (const uint8_t*)B, (const uint8_t*)B_scales,
-                           (uint16_t*)C, M, N, K);
+                           (uint16_t*)C, M, N, K, sa_pitch, sb_pitch);
         return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
     }
-    if ((K % 256) != 0 || (long long)(K / 2) * BM >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
+    if (!size_ok || (sa_pitch % 8) != 0 || (sb_pitch % 8) != 0 || sa_pitch < groups || sb_pitch < groups)
+        return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) return HK_ERR_BAD_ALIGNMENT;
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
-    return edge ? launch_mxfp4_4wave<true>(A, A_scales, B, B_scales, C, M, N, K, s)
-                : launch_mxfp4_4wave<false>(A, A_scales, B, B_scales, C, M, N, K, s);
+    return edge ? launch_mxfp4_4wave<true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s)
+                : launch_mxfp4_4wave<false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
+}
+
+extern "C" int hk_mxfp4_gemm_variant(const void* A, const void* A_scales, const void* B,
+                                     const void* B_scales, void* C, int M, int N, int K, int variant,
+                                     void* stream) {
+    if (variant < 0) return HK_ERR_UNSUPPORTED;
+    return mxfp4_gemm_impl(A, A_scales, K / 32, B, B_scales, K / 32, C, M, N, K, variant, stream);
 }
 
 extern "C" int hk_mxfp4_gemm(const void* A, const void* A_scales, const void* B, const void* B_scales,
                              void* C, int M, int N, int K, void* stream) {
-    const bool tile_ok = K > 0 && (K % 256) == 0 && M >= 64 && N >= 64 &&
-                         ((((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) == 0);
-    return hk_mxfp4_gemm_variant(A, A_scales, B, B_scales, C, M, N, K, tile_ok ? 1 : 0, stream);
+    return mxfp4_gemm_impl(A, A_scales, K / 32, B, B_scales, K / 32, C, M, N, K, -1, stream);
+}
+
+extern "C" int hk_mxfp4_gemm_pitched(const void* A, const void* A_scales, int a_scale_pitch, const void* B,
+                                     const void* B_scales, int b_scale_pitch, void* C, int M, int N, int K,
+                                     void* stream) {
+    return mxfp4_gemm_impl(A, A_scales, a_scale_pitch, B, B_scales, b_scale_pitch, C, M, N, K, -1, stream);
 }

@@ -116,7 +116,9 @@ _E8M0 = tuple(d for d in (torch.uint8, getattr(torch, "float8_e8m0fnu", None)) i
 
 def dispatch_mxfp4_gemm(A, A_scales, B, B_scales, C, variant: int = -1) -> None:
     """C[M,N] (bf16) = dequant(A) @ dequant(B).T for MXFP4 operands: A [M,K/2] packed e2m1
-    (low nibble = even k), A_scales [M,K/32] e8m0, B [N,K/2], B_scales [N,K/32]."""
+    (low nibble = even k), A_scales [M,K/32] e8m0, B [N,K/2], B_scales [N,K/32]. The scale tensors
+    may be wider than K/32 (padded rows, e.g. quant.pad_scales: any byte but 0xFF in the padding);
+    rows that are a multiple of 8 bytes keep a K that is not a multiple of 256 on the tile kernel."""
     _check_tensor(A, "A", _FP4, 2)
     _check_tensor(B, "B", _FP4, 2)
     _check_tensor(A_scales, "A_scales", _E8M0, 2)
@@ -125,8 +127,8 @@ def dispatch_mxfp4_gemm(A, A_scales, B, B_scales, C, variant: int = -1) -> None:
     M, Kh = A.shape
     N, Kh2 = B.shape
     K = 2 * Kh
-    if Kh2 != Kh or K % 32 != 0 or tuple(A_scales.shape) != (M, K // 32) or \
-            tuple(B_scales.shape) != (N, K // 32) or tuple(C.shape) != (M, N):
+    if Kh2 != Kh or K % 32 != 0 or A_scales.shape[0] != M or A_scales.shape[1] < K // 32 or \
+            B_scales.shape[0] != N or B_scales.shape[1] < K // 32 or tuple(C.shape) != (M, N):
         raise RuntimeError(
             f"shape mismatch: A {tuple(A.shape)}, A_scales {tuple(A_scales.shape)}, B {tuple(B.shape)}, "
             f"B_scales {tuple(B_scales.shape)}, C {tuple(C.shape)}")
@@ -134,7 +136,13 @@ def dispatch_mxfp4_gemm(A, A_scales, B, B_scales, C, variant: int = -1) -> None:
         raise RuntimeError("all tensors must be on the same device")
     lib = _lib.load_library()
     args = (A.data_ptr(), A_scales.data_ptr(), B.data_ptr(), B_scales.data_ptr(), C.data_ptr(), M, N, K)
-    if variant < 0:
+    pa, pb = A_scales.shape[1], B_scales.shape[1]
+    if pa != K // 32 or pb != K // 32:
+        if variant >= 0:
+            raise RuntimeError("padded scale rows and a forced variant exclude each other")
+        st = lib.hk_mxfp4_gemm_pitched(A.data_ptr(), A_scales.data_ptr(), pa, B.data_ptr(), B_scales.data_ptr(), pb,
+                                       C.data_ptr(), M, N, K, _stream(A))
+    elif variant < 0:
         st = lib.hk_mxfp4_gemm(*args, _stream(A))
     else:
         st = lib.hk_mxfp4_gemm_variant(*args, int(variant), _stream(A))

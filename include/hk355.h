@@ -91,6 +91,16 @@ int hk_mxfp4_gemm_variant(const void* A_e2m1, const void* A_scales_e8m0, const v
                           const void* B_scales_e8m0, void* C_bf16, int M, int N, int K,
                           int variant, void* stream);
 
+/* The same GEMM with padded scale rows: row m of A_scales starts at A_scales + m * a_scale_pitch
+ * bytes (pitch >= K / 32), likewise B_scales. With pitches that are multiples of 8 bytes and
+ * 4-byte aligned scale pointers the tile kernel takes any K % 32 == 0 (the hidden size 2880 of
+ * the MoE models: K / 32 = 90 scale bytes in rows of 96); in its last K-step the bytes past the
+ * end of a row are not fetched and count as zeros, so the padding scale bytes only must not be
+ * 0xFF (NaN). Other pitches go to the portable kernel. No counterpart in the reference. */
+int hk_mxfp4_gemm_pitched(const void* A_e2m1, const void* A_scales_e8m0, int a_scale_pitch,
+                          const void* B_e2m1, const void* B_scales_e8m0, int b_scale_pitch,
+                          void* C_bf16, int M, int N, int K, void* stream);
+
 /*
  * BF16 GEMM: C[M,N] = bf16( A[M,K] * B[N,K]^T ), A and B row-major bf16, fp32 accumulation, RNE.
  * Replaces the reference's flagship kernel behind tk_kernel.dispatch_micro(A, B, C)

@@ -112,3 +112,49 @@ def test_mxfp4_gemm_device_quantizer_matches_oracle(hk):
     p, s = hk.quant.quantize_mxfp4(torch.from_numpy(x).to(dev))
     po, so = F.quantize_mxfp4(x)
     assert np.array_equal(p.cpu().numpy(), po) and np.array_equal(s.cpu().numpy(), so)
+
+
+def _pad_rows(rng, s, pitch):
+    """Scale rows widened to `pitch` bytes; the padding holds arbitrary bytes other than 0xFF."""
+    out = rng.integers(0, 255, size=(s.shape[0], pitch), dtype=np.uint8)
+    out[:, :s.shape[1]] = s
+    return out
+
+
+PITCHED = [(256, 256, 2880, 96, 96), (300, 520, 2880, 96, 104), (512, 384, 160, 8, 8), (128, 640, 1056, 40, 40),
+           (256, 256, 512, 24, 16), (200, 264, 96, 8, 16), (96, 80, 2880, 91, 96)]
+
+
+@pytest.mark.parametrize("case", PITCHED)
+def test_mxfp4_gemm_padded_scale_rows_and_k_tails(hk, case):
+    """Scale rows padded to a pitch (a multiple of 8 bytes keeps any K % 32 == 0 on the tile kernel:
+    the last K-step's bytes past the row end are not fetched; the operand buffers sit at the end of
+    a pool filled with 0xFF so that a fetch past the row would show). The last case has a pitch that
+    is not a multiple of 8 and takes the portable kernel."""
+    M, N, K, pa, pb = case
+    print(f"mxfp4_gemm pitched case={case}", flush=True)
+    rng = np.random.default_rng(11 + M + N + K)
+    (a, sa), (b, sb) = _rand_mx(rng, M, K), _rand_mx(rng, N, K)
+    dev = torch.device("cuda:0")
+    pool = torch.full((2 * (a.size + b.size),), 0xFF, dtype=torch.uint8, device=dev)
+    A = pool[pool.numel() - a.size:].view(M, K // 2)
+    B = pool[pool.numel() - a.size - b.size:pool.numel() - a.size].view(N, K // 2)
+    A.copy_(torch.from_numpy(a).to(dev))
+    B.copy_(torch.from_numpy(b).to(dev))
+    SA = torch.from_numpy(_pad_rows(rng, sa, pa)).to(dev)
+    SB = torch.from_numpy(_pad_rows(rng, sb, pb)).to(dev)
+    C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    hk.tk_kernel.dispatch_mxfp4_gemm(A, SA, B, SB, C)
+    torch.cuda.synchronize()
+    out = C.float().cpu().numpy()
+    assert np.isfinite(out).all()
+    assert G.rel_fro_error(out, G.mxfp4_gemm(a, sa, b, sb)) <= 5e-3
+
+
+def test_mxfp4_gemm_padded_rows_equal_dense_rows_bit_for_bit(hk):
+    M, N, K = 512, 768, 1024
+    rng = np.random.default_rng(5)
+    (a, sa), (b, sb) = _rand_mx(rng, M, K), _rand_mx(rng, N, K)
+    dense = _run(hk, a, sa, b, sb)
+    padded = _run(hk, a, _pad_rows(rng, sa, 40), b, _pad_rows(rng, sb, 48))
+    assert np.array_equal(dense, padded)
