@@ -340,7 +340,7 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
 
 extern "C" int hk_bf16_gemm(const void* A, const void* B, void* C, int M, int N, int K, void* stream) {
     using namespace hk;
-    const bool tile_ok = K > 0 && (long long)2 * K * BM < (1ll << 31) && M >= 16 && N >= 16;
+    const bool tile_ok = K > 0 && (long long)2 * K * BM < (1ll << 31);
     // the same choice of tile as hk_fp8_gemm: the largest that still gives every CU work
     const long long tiles256 = (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     const long long tiles128 =

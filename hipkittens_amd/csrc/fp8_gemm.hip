@@ -725,7 +725,7 @@ extern "C" int hk_fp8_gemm_ws(const void* A, const void* B, void* C, int M, int 
 extern "C" int hk_fp8_gemm(const void* A, const void* B, void* C, int M, int N, int K,
                            float scale_a, float scale_b, void* stream) {
     using namespace hk;
-    const bool tile_ok = K > 0 && (long long)K * BM < (1ll << 31) && M >= 16 && N >= 16;
+    const bool tile_ok = K > 0 && (long long)K * BM < (1ll << 31);
     // The tile is the largest that still gives every CU of an MI355X work: 256x256 (five-slot ring
     // kernel) from 128 such tiles on; below that 128x128 tiles, and 64x64 tiles (two workgroups
     // per CU) when even those number at most 128.

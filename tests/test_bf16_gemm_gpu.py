@@ -31,7 +31,7 @@ def _run(hk, a_bits, b_bits, variant=-1):
 
 
 SHAPES = [(256, 256, 64), (256, 256, 128), (256, 256, 192), (512, 768, 1024), (1024, 1024, 2048)]
-RAGGED = [(300, 200, 256), (257, 255, 512), (64, 72, 768), (1000, 520, 320)]
+RAGGED = [(300, 200, 256), (257, 255, 512), (64, 72, 768), (1000, 520, 320), (1, 200, 512), (5, 7, 128)]
 
 
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, -1])

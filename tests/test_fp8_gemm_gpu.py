@@ -32,7 +32,7 @@ def _random_codes(rng, rows, K):
 
 
 SHAPES = [(256, 256, 256), (256, 256, 128), (512, 768, 384), (1024, 1024, 1024), (256, 512, 2048)]
-RAGGED = [(300, 200, 256), (257, 255, 128), (64, 72, 640), (1000, 1000, 512)]
+RAGGED = [(300, 200, 256), (257, 255, 128), (64, 72, 640), (1000, 1000, 512), (1, 200, 512), (5, 7, 256)]
 
 
 @pytest.mark.parametrize("variant", [0, 1, 2, 4, 5, 6, -1])
