@@ -263,18 +263,19 @@ struct Bf16Mma {
                                                       acc, 0, 0, 0);
     }
 };
-template <int TILE, int STAGES, bool EDGE>
+// K: the operands' row length in bytes (2 bytes per element).
+template <int TILE, int STAGES, bool EDGE, bool SPLIT>
 __global__ __launch_bounds__(256) void bf16_gemm_small_tile_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, int tiles_m, int tiles_n) {
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n, int kps, float* __restrict__ partial) {
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
-    gemm_small_tile_body<Bf16Mma, TILE, STAGES, EDGE, false>(smem, A, B, C, M, N, 2 * K, 1.0f, tiles_m, tiles_n, 0,
-                                                             nullptr);
+    gemm_small_tile_body<Bf16Mma, TILE, STAGES, EDGE, SPLIT>(smem, A, B, C, M, N, K, alpha, tiles_m, tiles_n, kps,
+                                                             partial);
 }
 
 template <int TILE, int STAGES, bool EDGE>
 static int launch_bf16_small_tile(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream) {
-    auto kern = bf16_gemm_small_tile_kernel<TILE, STAGES, EDGE>;
+    auto kern = bf16_gemm_small_tile_kernel<TILE, STAGES, EDGE, false>;
     constexpr int lds_bytes = STAGES * 2 * TILE * BK;
     static bool configured = false;
     if (!configured) {
@@ -285,8 +286,16 @@ static int launch_bf16_small_tile(const void* A, const void* B, void* C, int M, 
     }
     const int tiles_m = (M + TILE - 1) / TILE, tiles_n = (N + TILE - 1) / TILE;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream, (const uint8_t*)A,
-                       (const uint8_t*)B, (uint16_t*)C, M, N, K, tiles_m, tiles_n);
+                       (const uint8_t*)B, (uint16_t*)C, M, N, 2 * K, 1.0f, tiles_m, tiles_n, 0, (float*)nullptr);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
+template <bool EDGE>
+static int launch_bf16_splitk(const void* A, const void* B, void* C, int M, int N, int K, int splits, float* partial,
+                              hipStream_t stream) {
+    static bool configured = false;
+    return launch_small_tile_splitk(bf16_gemm_small_tile_kernel<kSmallTile, kSmallStages, EDGE, true>, configured, A,
+                                    B, C, M, N, 2 * K, 1.0f, splits, partial, stream);
 }
 
 template <bool EDGE>
@@ -347,4 +356,25 @@ extern "C" int hk_bf16_gemm(const void* A, const void* B, void* C, int M, int N,
         (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
     const int variant = !tile_ok ? 0 : tiles128 <= 128 ? 3 : tiles256 < 128 ? 2 : 1;
     return hk_bf16_gemm_variant(A, B, C, M, N, K, variant, stream);
+}
+
+extern "C" size_t hk_bf16_gemm_workspace_bytes(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0 || K >= (1 << 30)) return 0;
+    const int s = hk::splitk_ranges(M, N, 2 * K);
+    return s < 2 ? 0 : (size_t)s * M * N * sizeof(float);
+}
+
+extern "C" int hk_bf16_gemm_ws(const void* A, const void* B, void* C, int M, int N, int K, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+    using namespace hk;
+    if (M <= 0 || N <= 0 || K <= 0) return HK_ERR_BAD_SHAPE;
+    const int splits = K < (1 << 30) ? splitk_ranges(M, N, 2 * K) : 1;
+    const bool can_split = splits >= 2 && workspace && workspace_bytes >= (size_t)splits * M * N * sizeof(float) &&
+                           (K % 8) == 0 && (long long)2 * K * BM < (1ll << 31) && (long long)M * N < (1ll << 40);
+    if (!can_split) return hk_bf16_gemm(A, B, C, M, N, K, stream);
+    if (!A || !B || !C) return HK_ERR_NULL_POINTER;
+    if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)workspace) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    const bool edge = (M % kSmallTile) != 0 || (N % kSmallTile) != 0;
+    return edge ? launch_bf16_splitk<true>(A, B, C, M, N, K, splits, (float*)workspace, (hipStream_t)stream)
+                : launch_bf16_splitk<false>(A, B, C, M, N, K, splits, (float*)workspace, (hipStream_t)stream);
 }

@@ -17,7 +17,6 @@
 #include "../../include/hk355.h"
 
 namespace hk {
-int moe_num_compute_units();  // number of CUs of the current device (moe_mxfp4.hip)
 }
 
 namespace hk {
@@ -484,28 +483,6 @@ __global__ __launch_bounds__(256) void fp8_gemm_small_tile_kernel(
                                                             partial);
 }
 
-// C = bf16(alpha * sum_s partial[s]) in split order; one thread per 4 columns.
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int splits,
-                                                            long long mn, float alpha,
-                                                            uint16_t* __restrict__ C) {
-    const long long i4 = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i4 >= mn) return;
-    if (i4 + 4 <= mn && (mn & 3) == 0) {
-        v4f sum = *(const v4f*)(partial + i4);
-        for (int s2 = 1; s2 < splits; ++s2) sum += *(const v4f*)(partial + (size_t)s2 * mn + i4);
-        sum *= alpha;
-        v2i o;
-        o.x = pack_bf16(sum.x, sum.y); o.y = pack_bf16(sum.z, sum.w);
-        *(v2i*)(C + i4) = o;
-    } else {
-        for (long long i = i4; i < mn && i < i4 + 4; ++i) {
-            float sum = partial[i];
-            for (int s2 = 1; s2 < splits; ++s2) sum += partial[(size_t)s2 * mn + i];
-            C[i] = (uint16_t)(pack_bf16(sum * alpha, 0.f) & 0xffffu);
-        }
-    }
-}
-
 // Portable kernel for any M, N and K % 16 == 0: 4 waves, each a 32x32 patch of a 64x64
 // tile, operands fetched straight from global memory into MFMA fragments with
 // per-lane masking (rows past the edge and 16-byte chunks past K read as zero).
@@ -598,42 +575,12 @@ static int launch_small_tile(const void* A, const void* B, void* C, int M, int N
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
-// Number of K ranges the split-K path would use: as many as fill the CUs, each at least 4
-// K-steps long, at most 16; 1 = the problem has enough tiles or too short a K.
-static int splitk_ranges(int M, int N, int K) {
-    const long long tiles = (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
-    const int nk = (K + BK - 1) / BK;
-    const int cus = moe_num_compute_units();   // 256 when no device can be queried
-    // shorter K: the 64x64-tile kernel without a second launch is as fast or faster
-    if (tiles * 2 > cus || nk < 48) return 1;
-    long long s = cus / tiles;
-    if (s > nk / 4) s = nk / 4;
-    if (s > 16) s = 16;
-    return s < 2 ? 1 : (int)s;
-}
-
 template <bool EDGE>
 static int launch_tile128_splitk(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                                  int splits, float* partial, hipStream_t stream) {
-    auto kern = fp8_gemm_small_tile_kernel<kSmallTile, kSmallStages, EDGE, true>;
     static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kSmallLdsBytes) != hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
-    const int tiles_m = (M + kSmallTile - 1) / kSmallTile, tiles_n = (N + kSmallTile - 1) / kSmallTile;
-    const int nk = (K + BK - 1) / BK;
-    const int kps = (nk + splits - 1) / splits;
-    const int used = (nk + kps - 1) / kps;   // ranges that hold at least one K-step
-    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, used), dim3(256), kSmallLdsBytes, stream,
-                       (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
-                       tiles_n, kps, partial);
-    const long long mn = (long long)M * N;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((mn / 4 + 256) / 256)), dim3(256), 0, stream,
-                       (const float*)partial, used, mn, alpha, (uint16_t*)C);
-    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+    return launch_small_tile_splitk(fp8_gemm_small_tile_kernel<kSmallTile, kSmallStages, EDGE, true>, configured, A,
+                                    B, C, M, N, K, alpha, splits, partial, stream);
 }
 
 template <bool EDGE, bool RING>

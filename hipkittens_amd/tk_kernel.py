@@ -81,9 +81,16 @@ def dispatch_fp8_gemm(A, B, C, scale_a: float = 1.0, scale_b: float = 1.0, varia
     _lib.check(st, "dispatch_fp8_gemm")
 
 
-def dispatch_bf16_gemm(A, B, C, variant: int = -1) -> None:
+def bf16_gemm_workspace_bytes(M: int, N: int, K: int) -> int:
+    """Bytes of workspace with which dispatch_bf16_gemm splits K for this shape (0: it would not)."""
+    return int(_lib.load_library().hk_bf16_gemm_workspace_bytes(int(M), int(N), int(K)))
+
+
+def dispatch_bf16_gemm(A, B, C, variant: int = -1, workspace=None) -> None:
     """C[M,N] (bf16) = A[M,K] @ B[N,K].T for bf16 operands, fp32 accumulation
-    (include/hk355.h: hk_bf16_gemm). `variant` -1 lets the library choose; 0..3 force a kernel."""
+    (include/hk355.h: hk_bf16_gemm). `variant` -1 lets the library choose; 0..3 force a kernel.
+    `workspace` (uint8, bf16_gemm_workspace_bytes(M, N, K) bytes): lets the library split K for
+    decode-like shapes (hk_bf16_gemm_ws)."""
     _check_tensor(A, "A", _BF16, 2)
     _check_tensor(B, "B", _BF16, 2)
     _check_tensor(C, "C", _BF16, 2)
@@ -92,7 +99,13 @@ def dispatch_bf16_gemm(A, B, C, variant: int = -1) -> None:
     if B.shape[1] != K or tuple(C.shape) != (M, N):
         raise RuntimeError(f"shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}, C {tuple(C.shape)}")
     lib = _lib.load_library()
-    if variant < 0:
+    if workspace is not None:
+        _check_tensor(workspace, "workspace", (torch.uint8,), 1)
+        if variant >= 0:
+            raise RuntimeError("workspace and a forced variant exclude each other")
+        st = lib.hk_bf16_gemm_ws(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, workspace.data_ptr(),
+                                 workspace.numel(), _stream(A))
+    elif variant < 0:
         st = lib.hk_bf16_gemm(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, _stream(A))
     else:
         st = lib.hk_bf16_gemm_variant(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, int(variant), _stream(A))

@@ -111,6 +111,14 @@ int hk_mxfp4_gemm_pitched(const void* A_e2m1, const void* A_scales_e8m0, int a_s
 int hk_bf16_gemm(const void* A_bf16, const void* B_bf16, void* C_bf16, int M, int N, int K,
                  void* stream);
 
+/* The BF16 GEMM with an optional workspace for decode-like shapes, exactly as hk_fp8_gemm_ws:
+ * few 128x128 tiles and a long K (at least 48 K-steps of 64 elements) are split along K into fp32
+ * partial sums, added in a fixed order. hk_bf16_gemm_workspace_bytes returns 0 for shapes that
+ * would not be split; without a (large enough) workspace the call is hk_bf16_gemm. */
+size_t hk_bf16_gemm_workspace_bytes(int M, int N, int K);
+int hk_bf16_gemm_ws(const void* A_bf16, const void* B_bf16, void* C_bf16, int M, int N, int K,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
 /* Same contract on a chosen kernel: 0 = portable kernel (any shape), 1 = 256x256x64 tile kernel
  * (the FP8 ring schedule; the last K-step of a K that is not a multiple of 64 is zero-filled),
  * 2 = 128x128 tiles / three LDS stages, 3 = 64x64 tiles / four stages (the FP8 GEMM's small-tile

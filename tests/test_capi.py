@@ -59,6 +59,10 @@ def test_c_entry_points_reject_bad_arguments_without_a_gpu():
     assert lib.hk_fp8_gemm_workspace_bytes(16, 8192, 8192) % (16 * 8192 * 4) == 0
     assert lib.hk_fp8_gemm_workspace_bytes(16, 8192, 8192) > 0
     assert lib.hk_bf16_gemm(p, p, p, 64, 64, 60, None) == -2                  # K % 8
+    assert lib.hk_bf16_gemm_ws(p, p, p, 16, 1024, 4092, p, 1 << 40, None) == -2          # K % 8, split path
+    assert lib.hk_bf16_gemm_ws(p, p, p, 0, 256, 256, None, 0, None) == -2
+    assert lib.hk_bf16_gemm_workspace_bytes(8192, 8192, 8192) == 0
+    assert lib.hk_bf16_gemm_workspace_bytes(16, 8192, 4096) == lib.hk_fp8_gemm_workspace_bytes(16, 8192, 8192)
     assert lib.hk_mxfp4_gemm_pitched(p, p, 88, p, p, 96, p, 64, 64, 2880, None) == -2    # pitch < K / 32
     assert lib.hk_mxfp4_gemm_pitched(p, None, 96, p, p, 96, p, 64, 64, 2880, None) == -1
     assert lib.hk_mxfp4_gemm_pitched(p, p, 96, p, p, 96, p, 64, 64, 2872, None) == -2    # K % 32
