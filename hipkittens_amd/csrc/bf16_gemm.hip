@@ -294,7 +294,7 @@ template <bool EDGE>
 static int launch_bf16_splitk(const void* A, const void* B, void* C, int M, int N, int K, int splits, float* partial,
                               hipStream_t stream) {
     static bool configured = false;
-    return launch_small_tile_splitk(bf16_gemm_small_tile_kernel<kSmallTile, kSmallStages, EDGE, true>, configured, A,
+    return launch_small_tile_splitk(bf16_gemm_small_tile_kernel<kTinyTile, kTinyStages, EDGE, true>, configured, A,
                                     B, C, M, N, 2 * K, 1.0f, splits, partial, stream);
 }
 
@@ -374,7 +374,7 @@ extern "C" int hk_bf16_gemm_ws(const void* A, const void* B, void* C, int M, int
     if (!can_split) return hk_bf16_gemm(A, B, C, M, N, K, stream);
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)workspace) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    const bool edge = (M % kSmallTile) != 0 || (N % kSmallTile) != 0;
+    const bool edge = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
     return edge ? launch_bf16_splitk<true>(A, B, C, M, N, K, splits, (float*)workspace, (hipStream_t)stream)
                 : launch_bf16_splitk<false>(A, B, C, M, N, K, splits, (float*)workspace, (hipStream_t)stream);
 }

@@ -579,7 +579,7 @@ template <bool EDGE>
 static int launch_tile128_splitk(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                                  int splits, float* partial, hipStream_t stream) {
     static bool configured = false;
-    return launch_small_tile_splitk(fp8_gemm_small_tile_kernel<kSmallTile, kSmallStages, EDGE, true>, configured, A,
+    return launch_small_tile_splitk(fp8_gemm_small_tile_kernel<kTinyTile, kTinyStages, EDGE, true>, configured, A,
                                     B, C, M, N, K, alpha, splits, partial, stream);
 }
 
@@ -663,7 +663,7 @@ extern "C" int hk_fp8_gemm_ws(const void* A, const void* B, void* C, int M, int 
     if (!can_split) return hk_fp8_gemm(A, B, C, M, N, K, scale_a, scale_b, stream);
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)workspace) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    const bool edge = (M % kSmallTile) != 0 || (N % kSmallTile) != 0;
+    const bool edge = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
     const float alpha = scale_a * scale_b;
     return edge ? launch_tile128_splitk<true>(A, B, C, M, N, K, alpha, splits, (float*)workspace, (hipStream_t)stream)
                 : launch_tile128_splitk<false>(A, B, C, M, N, K, alpha, splits, (float*)workspace, (hipStream_t)stream);

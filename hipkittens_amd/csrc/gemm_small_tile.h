@@ -20,6 +20,7 @@ constexpr int kSmallLdsBytes = kSmallStages * kSmallStageBytes;  // 96 KiB
 // with so few 128x128 tiles that a quarter of the tile is needed to give every CU work
 constexpr int kTinyTile = 64;
 constexpr int kTinyStages = 4;
+constexpr int kTinyLdsBytes = kTinyStages * 2 * kTinyTile * BK;  // 64 KiB
 
 // SPLIT: blockIdx.y selects a range of `kps` K-steps; the tile's fp32 partial sums go to
 // partial[blockIdx.y][M][N] (plain stores; splitk_reduce_kernel adds the ranges in order, so the
@@ -184,18 +185,19 @@ int moe_num_compute_units();  // number of CUs of the current device, cached (mo
 // K-steps long, at most 16; 1 = the problem has enough tiles or too short a K.
 // K: the operands' row length in bytes.
 static inline int splitk_ranges(int M, int N, int K) {
-    const long long tiles = (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
+    // 64x64 tiles, two workgroups per CU
+    const long long tiles = (long long)((M + kTinyTile - 1) / kTinyTile) * ((N + kTinyTile - 1) / kTinyTile);
     const int nk = (K + BK - 1) / BK;
     const int cus = moe_num_compute_units();   // 256 when no device can be queried
     // shorter K: the 64x64-tile kernel without a second launch is as fast or faster
-    if (tiles * 2 > cus || nk < 48) return 1;
-    long long s = cus / tiles;
+    if (tiles > cus || nk < 48) return 1;
+    long long s = 2 * cus / tiles;
     if (s > nk / 4) s = nk / 4;
     if (s > 16) s = 16;
     return s < 2 ? 1 : (int)s;
 }
 
-// Launches `kern` (a small-tile kernel instantiated with SPLIT over 128x128 tiles) on `splits` K ranges
+// Launches `kern` (a small-tile kernel instantiated with SPLIT over 64x64 tiles) on `splits` K ranges
 // and the reduction behind it. K in bytes.
 template <typename Kern>
 static inline int launch_small_tile_splitk(Kern kern, bool& configured, const void* A, const void* B, void* C, int M,
@@ -203,15 +205,15 @@ static inline int launch_small_tile_splitk(Kern kern, bool& configured, const vo
                                            hipStream_t stream) {
     if (!configured) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kSmallLdsBytes) != hipSuccess)
+                                kTinyLdsBytes) != hipSuccess)
             return HK_ERR_LAUNCH;
         configured = true;
     }
-    const int tiles_m = (M + kSmallTile - 1) / kSmallTile, tiles_n = (N + kSmallTile - 1) / kSmallTile;
+    const int tiles_m = (M + kTinyTile - 1) / kTinyTile, tiles_n = (N + kTinyTile - 1) / kTinyTile;
     const int nk = (K + BK - 1) / BK;
     const int kps = (nk + splits - 1) / splits;
     const int used = (nk + kps - 1) / kps;   // ranges that hold at least one K-step
-    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, used), dim3(256), kSmallLdsBytes, stream,
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, used), dim3(256), kTinyLdsBytes, stream,
                        (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
                        tiles_n, kps, partial);
     const long long mn = (long long)M * N;

@@ -51,8 +51,8 @@ int hk_version(void);
 int hk_fp8_gemm(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
                 int M, int N, int K, float scale_a, float scale_b, void* stream);
 
-/* The same GEMM with an optional workspace, for decode-like shapes (few 128x128 tiles of C and a
- * long K, e.g. M <= 128 with N = K = 8192): the K range is split over several workgroups per
+/* The same GEMM with an optional workspace, for decode-like shapes (at most one 64x64 tile of C per
+ * CU and K >= 6144, e.g. M <= 128 with N = K = 8192): the K range is split over several workgroups per
  * tile, which write fp32 partial sums to the workspace, and a second kernel adds them in a fixed
  * order (deterministic) and rounds to bf16. hk_fp8_gemm_workspace_bytes returns the bytes this
  * needs, or 0 when the shape would not be split; with a NULL or too small workspace, or such a
@@ -112,7 +112,7 @@ int hk_bf16_gemm(const void* A_bf16, const void* B_bf16, void* C_bf16, int M, in
                  void* stream);
 
 /* The BF16 GEMM with an optional workspace for decode-like shapes, exactly as hk_fp8_gemm_ws:
- * few 128x128 tiles and a long K (at least 48 K-steps of 64 elements) are split along K into fp32
+ * few 64x64 tiles and a long K (at least 48 K-steps of 64 elements) are split along K into fp32
  * partial sums, added in a fixed order. hk_bf16_gemm_workspace_bytes returns 0 for shapes that
  * would not be split; without a (large enough) workspace the call is hk_bf16_gemm. */
 size_t hk_bf16_gemm_workspace_bytes(int M, int N, int K);
