@@ -253,6 +253,19 @@ def bench_routing(torch, hk, warmup, iters, dev):
     by = T * E * 4 + T * k * 8
     out.append({"kernel": "topk_softmax T=262144 E=128 k=4", "ms": round(ms, 5), "GB/s": round(by / ms / 1e6, 1),
                 "frac_of_hbm": round(by / ms / 1e6 / PEAK_HBM, 4)})
+    # the DeepSeek-V3 router: sigmoid scores + selection bias, 8 groups / top-4 groups, top-8. The fixed,
+    # bit-reproducible fp32 sigmoid (an exact division per expert) makes this kernel VALU bound
+    Tg, Eg, kg = 65536, 256, 8
+    lg = torch.randn(Tg, Eg, device=dev, generator=g)
+    bg = torch.randn(Eg, device=dev, generator=g) * 0.05
+    idg = torch.empty((Tg, kg), dtype=torch.int32, device=dev)
+    wg = torch.empty((Tg, kg), dtype=torch.float32, device=dev)
+    _, ms = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_topk_grouped_sigmoid(lg, bg, idg, wg, 8, 4, 2.5),
+                    warmup, iters)
+    by = Tg * Eg * 4 + Tg * kg * 8
+    out.append({"kernel": "topk_grouped_sigmoid T=65536 E=256 k=8 (8 groups / top-4)", "ms": round(ms, 5),
+                "GB/s": round(by / ms / 1e6, 1), "frac_of_hbm": round(by / ms / 1e6 / PEAK_HBM, 4)})
+    del lg, idg, wg
     ss = torch.empty(T * k, dtype=torch.int32, device=dev)
     off = torch.empty(E + 1, dtype=torch.int32, device=dev)
     inv = torch.empty(T * k, dtype=torch.int32, device=dev)

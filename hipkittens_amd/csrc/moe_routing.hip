@@ -206,6 +206,90 @@ __global__ __launch_bounds__(256) void moe_topk_grouped_sigmoid_kernel(
     }
 }
 
+// The same routing with 16 lanes per token (4 tokens per wave), for E = 16 * PER (PER <= 16) experts
+// whose groups are runs of whole lanes: lane `sub` of a token holds the experts [sub * PER, +PER),
+// a group is LG = (E / n_group) / PER adjacent lanes (a power of two). Reductions then run over
+// 16 lanes and serve four tokens at once; the two best of a group are merged from per-lane pairs.
+// Same operation sequence per value as the kernel above, so the results are bit-identical to it.
+template <int PER>
+__global__ __launch_bounds__(256) void moe_topk_grouped_sigmoid16_kernel(
+    const float* __restrict__ logits, const float* __restrict__ bias, int T, int k, int lg_shift,
+    int topk_group, float routed_scale, int32_t* __restrict__ ids, float* __restrict__ w) {
+    constexpr int E = 16 * PER;
+    const int lane = lane_id(), sub = lane & 15, seg = lane & ~15;
+    const int t = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 4 + (lane >> 4);
+    const bool live = t < T;
+    const float* row = logits + (size_t)(live ? t : 0) * E + sub * PER;
+    const int grp = sub >> lg_shift;   // this lane's group
+    float s[PER];
+    uint64_t cand[PER];
+    uint64_t best1 = 0, best2 = 0;     // the lane's two best (c, id) choices
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = sub * PER + i;
+        s[i] = sigmoid_f32(row[i]);
+        const float c = bias ? __fadd_rn(s[i], bias[e]) : s[i];
+        cand[i] = pack_choice(c, e);
+        if (cand[i] > best1) { best2 = best1; best1 = cand[i]; } else if (cand[i] > best2) best2 = cand[i];
+    }
+    // merge the pairs over the LG lanes of the group: afterwards every lane of a group holds the
+    // group's two best
+    for (int off = 1; off < (1 << lg_shift); off <<= 1) {
+        const uint64_t o1 = __shfl_xor(best1, off, 64), o2 = __shfl_xor(best2, off, 64);
+        const uint64_t hi = best1 > o1 ? best1 : o1, lo = best1 > o1 ? o1 : best1;
+        const uint64_t second = best2 > o2 ? best2 : o2;
+        best1 = hi;
+        best2 = lo > second ? lo : second;
+    }
+    auto key_value = [](uint64_t ch) {
+        const uint32_t key = (uint32_t)(ch >> 32);
+        return __uint_as_float((key & 0x80000000u) ? key ^ 0x80000000u : ~key);
+    };
+    const float gscore = PER << lg_shift >= 2 ? __fadd_rn(key_value(best1), key_value(best2)) : key_value(best1);
+    // keep the topk_group best groups (ties -> lower group id); the lanes of a group carry the same choice
+    uint64_t gc = pack_choice(gscore, grp);
+    bool kept = false;
+    for (int j = 0; j < topk_group; ++j) {
+        uint64_t b = gc;
+#pragma unroll
+        for (int off = 8; off >= 1; off >>= 1) {
+            const uint64_t o = __shfl_xor(b, off, 64);
+            b = o > b ? o : b;
+        }
+        if (gc == b) { gc = 0ull; kept = true; }
+    }
+    if (!kept) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) cand[i] = 0ull;
+    }
+    float my_s = 0.f;
+    int my_id = 0;
+    for (int j = 0; j < k; ++j) {
+        uint64_t best = 0;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) best = cand[i] > best ? cand[i] : best;
+#pragma unroll
+        for (int off = 8; off >= 1; off >>= 1) {
+            const uint64_t o = __shfl_xor(best, off, 64);
+            best = o > best ? o : best;
+        }
+        const int id = choice_id(best);
+        float sv = 0.f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            if (cand[i] == best) { cand[i] = 0ull; sv = s[i]; }
+        sv = __shfl(sv, seg + id / PER, 64);
+        if (sub == j) { my_s = sv; my_id = id; }
+    }
+    // sum of the k selected scores in selection order
+    float tot = 0.f;
+    for (int j = 0; j < k; ++j) tot = __fadd_rn(tot, __shfl(my_s, seg + j, 64));
+    if (live && sub < k) {
+        ids[(size_t)t * k + sub] = my_id;
+        w[(size_t)t * k + sub] = __fmul_rn(__fdiv_rn(my_s, tot), routed_scale);
+    }
+}
+
 // --------------------------------------------------------------------------------- sort
 // Stable counting sort of S = T*k slots by expert id, four launches:
 //   count   : per-chunk histogram (chunk = 1024 consecutive slots) -> ws[chunk][E]
@@ -461,6 +545,24 @@ extern "C" int hk_moe_topk_grouped_sigmoid(const float* logits, const float* bia
         (E % n_group) != 0 || topk_group <= 0 || topk_group > n_group ||
         k > topk_group * (E / n_group))
         return HK_ERR_BAD_SHAPE;
+    // 16 lanes per token when the experts split into 16 equal runs and every group is a
+    // power-of-two number of whole runs
+    const int per = E / 16, gs = E / n_group;
+    const int lanes_per_group = per > 0 && (E % 16) == 0 && (gs % per) == 0 ? gs / per : 0;
+    int lg_shift = -1;
+    for (int q = 0; q <= 4; ++q)
+        if (lanes_per_group == (1 << q)) lg_shift = q;
+    if (lg_shift >= 0 && k <= 16 && (per == 4 || per == 8 || per == 12 || per == 16)) {
+        const dim3 grid((T + 15) / 16), block(256);
+        hipStream_t s = (hipStream_t)stream;
+        switch (per) {
+            case 4: hipLaunchKernelGGL(moe_topk_grouped_sigmoid16_kernel<4>, grid, block, 0, s, logits, bias_or_null, T, k, lg_shift, topk_group, routed_scale, ids, w); break;
+            case 8: hipLaunchKernelGGL(moe_topk_grouped_sigmoid16_kernel<8>, grid, block, 0, s, logits, bias_or_null, T, k, lg_shift, topk_group, routed_scale, ids, w); break;
+            case 12: hipLaunchKernelGGL(moe_topk_grouped_sigmoid16_kernel<12>, grid, block, 0, s, logits, bias_or_null, T, k, lg_shift, topk_group, routed_scale, ids, w); break;
+            default: hipLaunchKernelGGL(moe_topk_grouped_sigmoid16_kernel<16>, grid, block, 0, s, logits, bias_or_null, T, k, lg_shift, topk_group, routed_scale, ids, w); break;
+        }
+        return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+    }
     hipLaunchKernelGGL(moe_topk_grouped_sigmoid_kernel, dim3((T + 3) / 4), dim3(256), 0,
                        (hipStream_t)stream, logits, bias_or_null, T, E, k, n_group, topk_group,
                        routed_scale, ids, w);

@@ -37,7 +37,9 @@ def test_topk_softmax(hk, T, E, k):
 
 @pytest.mark.parametrize("T,E,k,G,KG,use_bias", [(8192, 256, 8, 8, 4, False), (300, 256, 8, 8, 4, True),
                                                  (65, 64, 6, 4, 2, True), (9, 32, 4, 32, 8, False),
-                                                 (17, 128, 8, 1, 1, True)])
+                                                 (17, 128, 8, 1, 1, True), (50, 192, 5, 4, 3, True),
+                                                 (1000, 128, 4, 8, 2, False), (33, 64, 16, 16, 16, True),
+                                                 (21, 96, 3, 3, 2, False)])
 def test_topk_grouped_sigmoid(hk, T, E, k, G, KG, use_bias):
     rng = np.random.default_rng(T + E)
     logits = rng.standard_normal((T, E)).astype(np.float32)
