@@ -94,11 +94,13 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_rows_kernel(const uint16_t
 // Item lists of the two grouped GEMMs of a layer: list `which` (0 / 1) covers n_tiles[which] tiles
 // of weight rows and goes to items[which], its length to num_items[which]. One workgroup of NT
 // threads per list; thread t owns experts [t * 512 / NT, (t + 1) * 512 / NT). `scan`: NT ints of LDS.
+// With nparts > 1 workgroups per list, workgroup `part` writes the n-tiles part, part + nparts, ...
 struct MoeBuildItems { MoeItem* items[2]; int n_tiles[2]; int bm; };
 template <int NT>
 __device__ __forceinline__ void moe_build_items_block(const int32_t* __restrict__ expert_offsets, int E,
                                                       const MoeBuildItems& b, int which,
-                                                      int32_t* __restrict__ num_items, int* scan) {
+                                                      int32_t* __restrict__ num_items, int* scan,
+                                                      int part = 0, int nparts = 1) {
     constexpr int EPT = 512 / NT;
     const int n_tiles_n = b.n_tiles[which], bm = b.bm;
     MoeItem* __restrict__ items = b.items[which];
@@ -125,7 +127,7 @@ __device__ __forceinline__ void moe_build_items_block(const int32_t* __restrict_
     int base = scan[t] - mine;
 #pragma unroll
     for (int j = 0; j < EPT; ++j) {
-        for (int n = 0; n < n_tiles_n; ++n)
+        for (int n = part; n < n_tiles_n; n += nparts)
             for (int m = 0; m < cnt[j]; ++m) {
                 MoeItem it;
                 it.expert = t * EPT + j; it.row_start = lo[j] + m * bm; it.rows = min(bm, hi[j] - it.row_start);
@@ -134,14 +136,14 @@ __device__ __forceinline__ void moe_build_items_block(const int32_t* __restrict_
             }
         base += cnt[j] * n_tiles_n;
     }
-    if (t == NT - 1) num_items[which] = scan[NT - 1];
+    if (t == NT - 1 && part == 0) num_items[which] = scan[NT - 1];
 }
 
 __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __restrict__ expert_offsets,
                                                               int E, MoeBuildItems b,
                                                               int32_t* __restrict__ num_items) {
     __shared__ int scan[512];
-    moe_build_items_block<512>(expert_offsets, E, b, blockIdx.x, num_items, scan);
+    moe_build_items_block<512>(expert_offsets, E, b, blockIdx.x, num_items, scan, blockIdx.y, gridDim.y);
 }
 
 // Activation layout inside the MoE ("K-step-major tiles"): for a matrix of S rows the bytes of
@@ -1005,7 +1007,8 @@ void moe_launch_build_items(const int32_t* expert_offsets, int E, int bm, int n_
     b.bm = bm;
     b.items[0] = items1; b.items[1] = items2;
     b.n_tiles[0] = n_tiles_n1; b.n_tiles[1] = n_tiles_n2;
-    hipLaunchKernelGGL(moe_build_items_kernel, dim3(2), dim3(512), 0, s, expert_offsets, E, b, num_items);
+    // eight workgroups per list share the n-tiles (a thread otherwise writes ~100 items one by one)
+    hipLaunchKernelGGL(moe_build_items_kernel, dim3(2, 8), dim3(512), 0, s, expert_offsets, E, b, num_items);
 }
 
 template <int MODE, bool EXT>
