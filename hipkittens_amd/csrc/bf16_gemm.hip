@@ -253,6 +253,7 @@ __global__ __launch_bounds__(256) void bf16_gemm_portable_kernel(
 // Small-tile kernels (gemm_small_tile.h) with the bf16 MFMA: the two 16-byte halves of a fragment
 // row are K elements 8g.. and 32 + 8g.. of the 64-element K-step, one v_mfma_f32_16x16x32_bf16 each.
 struct Bf16Mma {
+    static constexpr bool kScaled = false;
     typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
     static __device__ __forceinline__ void mma(v4f& acc, const v8i& b, const v8i& a) {
         const v4i blo = {b[0], b[1], b[2], b[3]}, bhi = {b[4], b[5], b[6], b[7]};

@@ -470,6 +470,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
 // ---------------------------------------------------------------------------------------
 // Small-tile kernels (gemm_small_tile.h) with the FP8 MFMA.
 struct Fp8Mma {
+    static constexpr bool kScaled = false;
     static __device__ __forceinline__ void mma(v4f& acc, const v8i& b, const v8i& a) {
         acc = mfma_fp8_16x16x128(b, a, acc);
     }

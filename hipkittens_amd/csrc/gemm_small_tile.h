@@ -28,14 +28,27 @@ constexpr int kTinyLdsBytes = kTinyStages * 2 * kTinyTile * BK;  // 64 KiB
 // shapes), where a single workgroup per tile walks K one K-step latency at a time.
 // MMA: the operand type's MFMA on one 16-row x 128-byte fragment pair, `MMA::mma(acc, b, a)`. K is
 // the operands' row length in BYTES (a multiple of 16); smem: the workgroup's dynamic LDS.
+// MMA::kScaled (MXFP4): every operand row also has e8m0 block scales, 8 bytes per K-step, in rows of
+// sa_pitch / sb_pitch bytes (multiples of 8); `MMA::mma(acc, b, a, sb, sa)` then takes, per fragment,
+// the lane's scale bytes of the K-step's two halves in bits [7:0] of .x / .y.
+struct SmallTileScales { const uint8_t* SA; const uint8_t* SB; int sa_pitch, sb_pitch; };
+template <int TILE, int STAGES>
+constexpr int small_tile_lds_bytes(bool scaled) { return STAGES * 2 * TILE * BK + (scaled ? 4 * 2 * TILE * 16 : 0); }
+
 template <typename MMA, int TILE, int STAGES, bool EDGE, bool SPLIT>
 __device__ __forceinline__ void gemm_small_tile_body(
     uint8_t* smem, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, float alpha, int tiles_m, int tiles_n, int kps, float* __restrict__ partial) {
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n, int kps, float* __restrict__ partial,
+    SmallTileScales sc = SmallTileScales{nullptr, nullptr, 0, 0}) {
     constexpr int NW = 4, TM = TILE / 2, TN = TILE / 2, MT = TM / 16, NT = TN / 16;
     constexpr int kTB = TILE * BK, kSB = 2 * kTB;    // bytes of one operand tile / of one stage
     constexpr int NDMA = kTB / (NW * 1024);          // loads per wave per operand per K-step
-    static_assert(STAGES >= 3 && STAGES <= 8 && (STAGES - 2) * 2 * NDMA < 64, "vmcnt range");
+    constexpr bool kScaled = MMA::kScaled;
+    constexpr int LPT = 2 * NDMA + (kScaled ? 1 : 0);  // loads per wave per K-step
+    // scales: four slots, each the 16 bytes (two K-steps) of the TILE rows of A, then of B
+    constexpr int kScaleSlot = 2 * TILE * 16, kScaleBase = STAGES * kSB;
+    static_assert(STAGES >= 3 && STAGES <= 8 && (STAGES - 2) * LPT < 64, "vmcnt range");
+    static_assert(!kScaled || STAGES <= 5, "four scale slots cover the K-step pairs of at most five stages");
     const int lane = lane_id(), w = wave_id();
     const int wm = w >> 1, wn = w & 1;
 
@@ -72,6 +85,24 @@ __device__ __forceinline__ void gemm_small_tile_body(
     // this workgroup's K-steps: [kt0, kt0 + nkt)
     const int kt0 = SPLIT ? (int)blockIdx.y * kps : 0;
     const int nkt = SPLIT ? min(kps, nk - kt0) : nk;
+    // Scale loads (kScaled): wave w fetches operand w & 1 (0 = A), lane l the 16 bytes of row
+    // 64 (w >> 1) + l (TILE = 128; with TILE = 64 waves 2 and 3 repeat what 0 and 1 fetch), i.e. the
+    // scales of the pair of K-steps kt / 2. Every wave issues one such load with every K-step (on odd
+    // K-steps it repeats the pair's load into the same slot): the same number of loads per K-step in
+    // every wave keeps the counted waits uniform.
+    v4i srd_s = {0, 0, 0, 0};
+    uint32_t voff_s = 0, lds_s = 0;
+    if (kScaled) {
+        const int op = w & 1, srow0 = TILE == 128 ? 64 * (w >> 1) : 0;
+        const int R = srow0 + lane;
+        int rr = op ? b_row_to_col(R) : R;
+        if (EDGE) rr = min(rr, (op ? b_rows : a_rows) - 1);
+        const int pitch = op ? sc.sb_pitch : sc.sa_pitch;
+        srd_s = op ? make_srd(sc.SB + (size_t)col0 * pitch, (uint32_t)b_rows * (uint32_t)pitch)
+                   : make_srd(sc.SA + (size_t)row0 * pitch, (uint32_t)a_rows * (uint32_t)pitch);
+        voff_s = (uint32_t)rr * (uint32_t)pitch;
+        lds_s = to_sgpr(lds0 + kScaleBase + (uint32_t)op * (TILE * 16) + (uint32_t)srow0 * 16u);
+    }
     auto issue_tile = [&](int stage, int kt_local) {
         const int kt = kt0 + kt_local;
         const uint32_t k0 = (uint32_t)kt * BK;
@@ -81,17 +112,18 @@ __device__ __forceinline__ void gemm_small_tile_body(
         for (int i = 0; i < NDMA; ++i) dma16(srd_a, dst + i * NW * 1024, voff_a[i] | vor, k0);
 #pragma unroll
         for (int i = 0; i < NDMA; ++i) dma16(srd_b, dst + kTB + i * NW * 1024, voff_b[i] | vor, k0);
+        if (kScaled) dma16(srd_s, lds_s + (uint32_t)((kt >> 1) & 3) * kScaleSlot, voff_s, (uint32_t)(kt >> 1) * 16u);
     };
     // wait until at most `tiles` of the most recently issued K-steps' loads are still in flight
     auto wait_tiles = [&](int tiles) {
         switch (tiles) {
             case 0: wait_vmcnt<0>(); break;
-            case 1: wait_vmcnt<2 * NDMA>(); break;
-            case 2: wait_vmcnt<(STAGES > 3 ? 2 : 1) * 2 * NDMA>(); break;
-            case 3: wait_vmcnt<(STAGES > 4 ? 3 : 1) * 2 * NDMA>(); break;
-            case 4: wait_vmcnt<(STAGES > 5 ? 4 : 1) * 2 * NDMA>(); break;
-            case 5: wait_vmcnt<(STAGES > 6 ? 5 : 1) * 2 * NDMA>(); break;
-            default: wait_vmcnt<(STAGES > 7 ? 6 : 1) * 2 * NDMA>(); break;
+            case 1: wait_vmcnt<LPT>(); break;
+            case 2: wait_vmcnt<(STAGES > 3 ? 2 : 1) * LPT>(); break;
+            case 3: wait_vmcnt<(STAGES > 4 ? 3 : 1) * LPT>(); break;
+            case 4: wait_vmcnt<(STAGES > 5 ? 4 : 1) * LPT>(); break;
+            case 5: wait_vmcnt<(STAGES > 6 ? 5 : 1) * LPT>(); break;
+            default: wait_vmcnt<(STAGES > 7 ? 6 : 1) * LPT>(); break;
         }
     };
 
@@ -122,11 +154,32 @@ __device__ __forceinline__ void gemm_small_tile_body(
         v8i bf[NT];
 #pragma unroll
         for (int n = 0; n < NT; ++n) bf[n] = lds_frag(b_lo0 + so, b_hi0 + so, n * 16 * BK);
+        if constexpr (kScaled) {
+            // the lane's scale bytes: row 16 f + r of the wave's patch, byte g of each half's dword
+            const int ktg = kt0 + kt;
+            const uint32_t sbase = lds0 + kScaleBase + (uint32_t)((ktg >> 1) & 3) * kScaleSlot + (uint32_t)(ktg & 1) * 8u + r * 16u;
+            const uint32_t sh = 8u * g;
+            v2i bs[NT];
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            const v8i af = lds_frag(a_lo0 + so, a_hi0 + so, m * 16 * BK);
+            for (int n = 0; n < NT; ++n) {
+                bs[n] = *(lds_v2i_t*)(uintptr_t)(sbase + TILE * 16 + (wn * TN + 16 * n) * 16);
+                bs[n].x = (int)((uint32_t)bs[n].x >> sh); bs[n].y = (int)((uint32_t)bs[n].y >> sh);
+            }
 #pragma unroll
-            for (int n = 0; n < NT; ++n) MMA::mma(acc[m][n], bf[n], af);
+            for (int m = 0; m < MT; ++m) {
+                const v8i af = lds_frag(a_lo0 + so, a_hi0 + so, m * 16 * BK);
+                v2i as = *(lds_v2i_t*)(uintptr_t)(sbase + (wm * TM + 16 * m) * 16);
+                as.x = (int)((uint32_t)as.x >> sh); as.y = (int)((uint32_t)as.y >> sh);
+#pragma unroll
+                for (int n = 0; n < NT; ++n) MMA::mma(acc[m][n], bf[n], af, bs[n], as);
+            }
+        } else {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const v8i af = lds_frag(a_lo0 + so, a_hi0 + so, m * 16 * BK);
+#pragma unroll
+                for (int n = 0; n < NT; ++n) MMA::mma(acc[m][n], bf[n], af);
+            }
         }
         st = st == STAGES - 1 ? 0 : st + 1;
     }

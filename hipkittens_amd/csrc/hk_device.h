@@ -14,6 +14,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) const v4i lds_v4i_t;
+typedef __attribute__((address_space(3))) const v2i lds_v2i_t;
 
 constexpr int kWave = 64;
 constexpr int kNumXcd = 8;

@@ -18,11 +18,11 @@
 // one ds_read_b64 per fragment and K-step; a per-lane shift moves byte g into the position the
 // MFMA reads.
 #include "gemm_tile.h"
+#include "gemm_small_tile.h"
 #include "../../include/hk355.h"
 
 namespace hk {
 
-typedef __attribute__((address_space(3))) const v2i lds_v2i_t;
 
 constexpr int kScaleTileBytes = BM * 16;               // per row: 8 scale bytes for each K-step of a pair
 constexpr int kScaleStageBytes = 2 * kScaleTileBytes;  // A + B
@@ -311,6 +311,48 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_portable_kernel(
     }
 }
 
+// Small-tile kernels (gemm_small_tile.h) with the scaled FP4 MFMA, for problems with too few 256x256
+// tiles to occupy the chip: the two 16-byte halves of a fragment row are MX blocks g and 4 + g of
+// the 256-element K-step.
+struct Mxfp4Mma {
+    static constexpr bool kScaled = true;
+    static __device__ __forceinline__ void mma(v4f& acc, const v8i& b, const v8i& a, const v2i& sb, const v2i& sa) {
+        const v4i blo = {b[0], b[1], b[2], b[3]}, bhi = {b[4], b[5], b[6], b[7]};
+        const v4i alo = {a[0], a[1], a[2], a[3]}, ahi = {a[4], a[5], a[6], a[7]};
+        acc = mfma_fp4(blo, alo, acc, sb.x, sa.x);
+        acc = mfma_fp4(bhi, ahi, acc, sb.y, sa.y);
+    }
+};
+// K: the operands' row length in bytes (two elements per byte).
+template <int TILE, int STAGES, bool EDGE>
+__global__ __launch_bounds__(256) void mxfp4_gemm_small_tile_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
+    const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int sa_pitch,
+    int sb_pitch, int tiles_m, int tiles_n) {
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    gemm_small_tile_body<Mxfp4Mma, TILE, STAGES, EDGE, false>(smem, A, B, C, M, N, K, 1.0f, tiles_m, tiles_n, 0,
+                                                              nullptr, SmallTileScales{SA, SB, sa_pitch, sb_pitch});
+}
+
+template <int TILE, int STAGES, bool EDGE>
+static int launch_mxfp4_small_tile(const void* A, const void* SA, const void* B, const void* SB, void* C,
+                                   int M, int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
+    auto kern = mxfp4_gemm_small_tile_kernel<TILE, STAGES, EDGE>;
+    constexpr int lds_bytes = small_tile_lds_bytes<TILE, STAGES>(true);
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) !=
+            hipSuccess)
+            return HK_ERR_LAUNCH;
+        configured = true;
+    }
+    const int tiles_m = (M + TILE - 1) / TILE, tiles_n = (N + TILE - 1) / TILE;
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream, (const uint8_t*)A,
+                       (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB, (uint16_t*)C, M, N, K / 2,
+                       sa_pitch, sb_pitch, tiles_m, tiles_n);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
 template <bool EDGE>
 static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, const void* SB, void* C,
                               int M, int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
@@ -331,8 +373,8 @@ static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, cons
 
 }  // namespace hk
 
-// variant: -1 = choose, 0 = portable kernel, 1 = tile kernel. Scale rows are sa_pitch / sb_pitch bytes
-// apart (>= K / 32).
+// variant: -1 = choose, 0 = portable kernel, 1 = 256x256 tile kernel, 2 / 3 = 128x128 / 64x64 tiles.
+// Scale rows are sa_pitch / sb_pitch bytes apart (>= K / 32).
 static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, const void* B, const void* B_scales,
                            int sb_pitch, void* C, int M, int N, int K, int variant, void* stream) {
     using namespace hk;
@@ -340,14 +382,20 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
     if (M <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || sa_pitch < K / 32 || sb_pitch < K / 32)
         return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < -1 || variant > 1) return HK_ERR_UNSUPPORTED;
+    if (variant < -1 || variant > 3) return HK_ERR_UNSUPPORTED;
     // the tile kernel fetches a row's scales 16 bytes per lane, two K-steps of 8 bytes at a time:
     // rows must start 4-byte aligned and hold whole groups of 8 bytes
     const int groups = (K / 32 + 7) / 8 * 8;
     const bool pitch_ok = (sa_pitch % 8) == 0 && (sb_pitch % 8) == 0 && sa_pitch >= groups && sb_pitch >= groups &&
                           ((((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) == 0);
     const bool size_ok = (long long)(K / 2) * BM < (1ll << 31) && (long long)BM * max(sa_pitch, sb_pitch) < (1ll << 31);
-    if (variant < 0) variant = pitch_ok && size_ok && M >= 64 && N >= 64 ? 1 : 0;
+    if (variant < 0) {
+        // the largest tile that still gives every CU work, as in hk_fp8_gemm
+        const long long tiles256 = (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+        const long long tiles128 =
+            (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
+        variant = !(pitch_ok && size_ok) ? 0 : tiles128 <= 128 ? 3 : tiles256 < 128 ? 2 : 1;
+    }
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {
         if ((M + 63) / 64 > 65535) return HK_ERR_BAD_SHAPE;
@@ -360,6 +408,16 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
     if (!size_ok || (sa_pitch % 8) != 0 || (sb_pitch % 8) != 0 || sa_pitch < groups || sb_pitch < groups)
         return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) return HK_ERR_BAD_ALIGNMENT;
+    if (variant == 2) {
+        const bool e = (M % kSmallTile) != 0 || (N % kSmallTile) != 0;
+        return e ? launch_mxfp4_small_tile<kSmallTile, kSmallStages, true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s)
+                 : launch_mxfp4_small_tile<kSmallTile, kSmallStages, false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
+    }
+    if (variant == 3) {
+        const bool e = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
+        return e ? launch_mxfp4_small_tile<kTinyTile, kTinyStages, true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s)
+                 : launch_mxfp4_small_tile<kTinyTile, kTinyStages, false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
+    }
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
     return edge ? launch_mxfp4_4wave<true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s)
                 : launch_mxfp4_4wave<false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);

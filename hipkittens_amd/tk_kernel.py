@@ -131,7 +131,8 @@ def dispatch_mxfp4_gemm(A, A_scales, B, B_scales, C, variant: int = -1) -> None:
     """C[M,N] (bf16) = dequant(A) @ dequant(B).T for MXFP4 operands: A [M,K/2] packed e2m1
     (low nibble = even k), A_scales [M,K/32] e8m0, B [N,K/2], B_scales [N,K/32]. The scale tensors
     may be wider than K/32 (padded rows, e.g. quant.pad_scales: any byte but 0xFF in the padding);
-    rows that are a multiple of 8 bytes keep a K that is not a multiple of 256 on the tile kernel."""
+    rows that are a multiple of 8 bytes keep a K that is not a multiple of 256 on the tile kernels.
+    `variant` -1 lets the library choose; 0..3 force a kernel (see include/hk355.h)."""
     _check_tensor(A, "A", _FP4, 2)
     _check_tensor(B, "B", _FP4, 2)
     _check_tensor(A_scales, "A_scales", _E8M0, 2)

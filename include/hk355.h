@@ -86,7 +86,9 @@ int hk_mxfp4_gemm(const void* A_e2m1, const void* A_scales_e8m0, const void* B_e
                   const void* B_scales_e8m0, void* C_bf16, int M, int N, int K, void* stream);
 
 /* Same contract on a chosen kernel: 0 = portable kernel (any shape), 1 = 256x256x256 tile
- * kernel (needs K % 256 == 0 and 4-byte aligned scale pointers). */
+ * kernel, 2 = 128x128 tiles / three LDS stages, 3 = 64x64 tiles / four stages (the small-tile
+ * kernels of the FP8 GEMM with the scaled FP4 MFMA; hk_mxfp4_gemm picks by tile count as
+ * hk_fp8_gemm does). 1-3 need K % 256 == 0 (dense scale rows) and 4-byte aligned scale pointers. */
 int hk_mxfp4_gemm_variant(const void* A_e2m1, const void* A_scales_e8m0, const void* B_e2m1,
                           const void* B_scales_e8m0, void* C_bf16, int M, int N, int K,
                           int variant, void* stream);

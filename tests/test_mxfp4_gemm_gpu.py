@@ -32,10 +32,10 @@ def _rand_mx(rng, rows, K, spread=True):
 
 
 SHAPES = [(256, 256, 256), (256, 256, 512), (512, 768, 1024), (1024, 1024, 2048)]
-RAGGED = [(300, 200, 256), (257, 255, 512), (64, 72, 768), (1000, 520, 512)]
+RAGGED = [(300, 200, 256), (257, 255, 512), (64, 72, 768), (1000, 520, 512), (1, 200, 512), (5, 7, 256), (130, 70, 1280)]
 
 
-@pytest.mark.parametrize("variant", [0, 1, -1])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, -1])
 @pytest.mark.parametrize("shape", SHAPES + RAGGED)
 def test_mxfp4_gemm_matches_oracle(hk, shape, variant):
     M, N, K = shape
@@ -121,7 +121,7 @@ def _pad_rows(rng, s, pitch):
     return out
 
 
-PITCHED = [(256, 256, 2880, 96, 96), (300, 520, 2880, 96, 104), (512, 384, 160, 8, 8), (128, 640, 1056, 40, 40),
+PITCHED = [(2048, 2304, 2880, 96, 96), (16, 2880, 2880, 96, 96), (256, 256, 2880, 96, 96), (300, 520, 2880, 96, 104), (512, 384, 160, 8, 8), (128, 640, 1056, 40, 40),
            (256, 256, 512, 24, 16), (200, 264, 96, 8, 16), (96, 80, 2880, 91, 96)]
 
 
