@@ -216,6 +216,38 @@ def bench_moe_mxfp4(torch, hk, warmup, iters, dev, graph=True):
             "ms_graph_replay": round(kern_graph, 5) if graph else None, "ms_with_biases_and_clamped_swiglu": round(kern_oai, 5)}
 
 
+def cpu_baseline_moe_mxfp4(torch, hk, dev):
+    """The CPU oracle's MXFP4 MoE layer (dequantize + fp32 matmuls, expert by expert) timed on a 1/16
+    sample of the workload: 8 of the 128 experts and 256 of the 4096 tokens at the full H = I = 2880,
+    top-4 routing, i.e. the same 128 rows per expert. Weights are quantized on the GPU beforehand;
+    only the oracle's forward pass is timed."""
+    import os
+
+    import numpy as np
+
+    from oracle import formats as F
+    from oracle import moe as OM
+
+    T, E, k, H, I = 256, 8, 4, 2880, 2880
+    g = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn(T, H, device=dev, generator=g).to(torch.bfloat16)
+    logits = torch.randn(T, E, device=dev, generator=g).cpu().numpy()
+    q13 = [hk.quant.quantize_mxfp4(torch.randn(2 * I, H, device=dev, generator=g) * 0.02) for _ in range(E)]
+    q2 = [hk.quant.quantize_mxfp4(torch.randn(H, I, device=dev, generator=g) * 0.02) for _ in range(E)]
+    w13p = np.stack([a.cpu().numpy() for a, _ in q13]); w13s = np.stack([b.cpu().numpy() for _, b in q13])
+    w2p = np.stack([a.cpu().numpy() for a, _ in q2]); w2s = np.stack([b.cpu().numpy() for _, b in q2])
+    xf = F.bf16_to_f32(x.view(torch.int16).cpu().numpy().view(np.uint16))
+    ids, w = OM.topk_softmax(logits, k)
+    best = float("inf")
+    for _ in range(2):
+        t0 = time.perf_counter()
+        OM.moe_mxfp4_forward(xf, ids, w, w13p, w13s, w2p, w2s)
+        best = min(best, time.perf_counter() - t0)
+    flop = 2.0 * T * k * (H * 2 * I + I * H)
+    return {"value": round(flop / best / 1e12, 4), "unit": "TFLOP/s", "cores": os.cpu_count() or 1, "kind": "port",
+            "sample": f"oracle MoE forward on 8 of 128 experts x 256 of 4096 tokens (same rows per expert), best of 2: {best:.2f} s"}
+
+
 def bench_moe_fp8blk(torch, hk, warmup, iters, dev):
     T, E, k, H, I, G, KG = 8192, 256, 8, 7168, 2048, 8, 4
     g = torch.Generator(device=dev).manual_seed(0)
@@ -382,6 +414,8 @@ def main() -> int:
         torch.cuda.empty_cache()
         extra["routing"] = bench_routing(torch, hk, quick_w, quick_i, dev)
 
+    if not args.no_cpu_baseline and not args.only_headline:
+        extra["moe_mxfp4"]["cpu_baseline"] = cpu_baseline_moe_mxfp4(torch, hk, dev)
     cpu = None
     if not args.no_cpu_baseline:
         r = OG.cpu_baseline_fp8_gemm(n, n, n, seed=0, repeats=12)
