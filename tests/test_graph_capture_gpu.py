@@ -109,3 +109,4 @@ def test_moe_fp8blk_layer_in_a_graph(hk):
     _replay_and_compare(lambda: hk.tk_kernel.dispatch_moe_fp8blk(xq, xs, logits, None, w13q, w13s, w2q, w2s, y,
                                                                   k, G, KG, 2.5, ws), [y],
                         scratch_fn=lambda: ws.fill_(0xA5))
+
