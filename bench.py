@@ -392,7 +392,7 @@ def main() -> int:
     if not args.only_headline:
         quick_w, quick_i = 20, 20
         extra["mfma_fp8_ceiling_tflops_for_this_data"] = round(mfma_ceiling(torch, hk, head["A"], dev), 1)
-        sweep = {m: bench_fp8(torch, hk, m, 50, 50, dev, graph=m <= 4096 and not args.no_graph)
+        sweep = {m: bench_fp8(torch, hk, m, 500, 100, dev, graph=m <= 4096 and not args.no_graph)  # the reference's protocol
                  for m in (1024, 2048, 4096, 16384)}
         # per call through the Python boundary (about 9 us of host time per call bounds the small sizes) ...
         extra["fp8_gemm_sweep_tflops"] = {str(m): round(r["tflops"], 1) for m, r in sweep.items()}
@@ -404,10 +404,10 @@ def main() -> int:
         torch.cuda.empty_cache()
         extra["fp8_gemm_reference_inputs"] = bench_fp8_reference_inputs(torch, hk, n, 100, 100, dev)
         extra["fp8_gemm_decode"] = bench_fp8_decode(torch, hk, 50, 50, dev)
-        extra["bf16_gemm"] = bench_bf16(torch, hk, 8192, 50, 50, dev)
-        extra["library_on_this_box_8192"] = bench_library_baselines(torch, 8192, 50, 50, dev)
+        extra["bf16_gemm"] = bench_bf16(torch, hk, 8192, 500, 100, dev)
+        extra["library_on_this_box_8192"] = bench_library_baselines(torch, 8192, 500, 100, dev)
         torch.cuda.empty_cache()
-        extra["mxfp4_gemm"] = bench_mxfp4(torch, hk, 8192, 50, 50, dev)
+        extra["mxfp4_gemm"] = bench_mxfp4(torch, hk, 8192, 500, 100, dev)
         extra["moe_mxfp4"] = bench_moe_mxfp4(torch, hk, quick_w, quick_i, dev, graph=not args.no_graph)
         torch.cuda.empty_cache()
         extra["moe_fp8blk"] = bench_moe_fp8blk(torch, hk, 5, 10, dev)
