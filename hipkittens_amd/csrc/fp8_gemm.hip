@@ -40,7 +40,7 @@ __global__ __launch_bounds__(WM * WN * 64) void fp8_gemm_tile_kernel(
     {
         const int num_wg = tiles_m * tiles_n;
         const int id = xcd_chunk_order(blockIdx.x, num_wg, kCuPerXcd);
-        grouped_raster(id, tiles_m, tiles_n, 8, pm, pn);
+        grouped_raster(id, tiles_m, tiles_n, 4, pm, pn);
     }
     const int row0 = pm * BM, col0 = pn * BN;
 
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_kernel(
     int pm, pn;
     {
         const int id = xcd_chunk_order(blockIdx.x, tiles_m * tiles_n, kCuPerXcd);
-        grouped_raster(id, tiles_m, tiles_n, 8, pm, pn);
+        grouped_raster(id, tiles_m, tiles_n, 4, pm, pn);
     }
     const int row0 = pm * BM, col0 = pn * BN;
 
@@ -314,7 +314,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
     int pm, pn;
     {
         const int id = xcd_chunk_order(blockIdx.x, tiles_m * tiles_n, kCuPerXcd);
-        grouped_raster(id, tiles_m, tiles_n, 8, pm, pn);
+        grouped_raster(id, tiles_m, tiles_n, 4, pm, pn);
     }
     const int row0 = pm * BM, col0 = pn * BN;
 
