@@ -24,7 +24,7 @@ __device__ __forceinline__ void mfma_bf16_16x16x32_acc(v4f& acc, const v4i& x, c
 template <bool EDGE>
 __global__ __launch_bounds__(256) void bf16_gemm_4wave_ring_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, float alpha, int tiles_m, int tiles_n) {
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n, int band_n) {
     const int Kb = 2 * K;  // operand row pitch in bytes; a K-step is 128 bytes = 64 elements
     constexpr int NW = 4, TM = 128, TN = 128, MT = 8, NT = 8;
     constexpr int NDMA = kTileBytes / (NW * 1024);  // 8 loads per wave per operand per K-step
@@ -40,7 +40,7 @@ __global__ __launch_bounds__(256) void bf16_gemm_4wave_ring_kernel(
     int pm, pn;
     {
         const int id = xcd_chunk_order(blockIdx.x, tiles_m * tiles_n, kCuPerXcd);
-        grouped_raster(id, tiles_m, tiles_n, 8, pm, pn);
+        banded_raster(id, tiles_m, tiles_n, band_n < tiles_n ? 4 : 8, band_n, pm, pn);
     }
     const int row0 = pm * BM, col0 = pn * BN;
 
@@ -312,7 +312,8 @@ static int launch_bf16_ring(const void* A, const void* B, void* C, int M, int N,
     }
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream, (const uint8_t*)A,
-                       (const uint8_t*)B, (uint16_t*)C, M, N, K, 1.0f, tiles_m, tiles_n);
+                       (const uint8_t*)B, (uint16_t*)C, M, N, K, 1.0f, tiles_m, tiles_n,
+                       raster_band(((long long)M + N) * K * 2, tiles_n));
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 

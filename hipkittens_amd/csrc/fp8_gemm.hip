@@ -24,7 +24,7 @@ namespace hk {
 template <int WM, int WN, bool EDGE>
 __global__ __launch_bounds__(WM * WN * 64) void fp8_gemm_tile_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, float alpha, int tiles_m, int tiles_n) {
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n, int band_n) {
     constexpr int NW = WM * WN;
     constexpr int TM = BM / WM, TN = BN / WN;  // per-wave tile of C
     constexpr int MT = TM / 16, NT = TN / 16;  // MFMA tiles per wave
@@ -40,7 +40,7 @@ __global__ __launch_bounds__(WM * WN * 64) void fp8_gemm_tile_kernel(
     {
         const int num_wg = tiles_m * tiles_n;
         const int id = xcd_chunk_order(blockIdx.x, num_wg, kCuPerXcd);
-        grouped_raster(id, tiles_m, tiles_n, 4, pm, pn);
+        banded_raster(id, tiles_m, tiles_n, 4, band_n, pm, pn);
     }
     const int row0 = pm * BM, col0 = pn * BN;
 
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(WM * WN * 64) void fp8_gemm_tile_kernel(
 template <bool EDGE>
 __global__ __launch_bounds__(256) void fp8_gemm_4wave_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, float alpha, int tiles_m, int tiles_n) {
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n, int band_n) {
     constexpr int NW = 4, TM = 128, TN = 128, MT = 8, NT = 8;
     constexpr int NDMA = kTileBytes / (NW * 1024);  // 8 loads per wave per operand per K-step
     constexpr int PG = 4;                            // barrier sits after MFMA group PG
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_kernel(
     int pm, pn;
     {
         const int id = xcd_chunk_order(blockIdx.x, tiles_m * tiles_n, kCuPerXcd);
-        grouped_raster(id, tiles_m, tiles_n, 4, pm, pn);
+        banded_raster(id, tiles_m, tiles_n, 4, band_n, pm, pn);
     }
     const int row0 = pm * BM, col0 = pn * BN;
 
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_kernel(
 template <bool EDGE>
 __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, float alpha, int tiles_m, int tiles_n) {
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n, int band_n) {
     constexpr int NW = 4, TM = 128, TN = 128, MT = 8, NT = 8;
     constexpr int NDMA = kTileBytes / (NW * 1024);  // 8 loads per wave per operand per K-step
     constexpr int PG = 4, AD = 3;
@@ -314,7 +314,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
     int pm, pn;
     {
         const int id = xcd_chunk_order(blockIdx.x, tiles_m * tiles_n, kCuPerXcd);
-        grouped_raster(id, tiles_m, tiles_n, 4, pm, pn);
+        banded_raster(id, tiles_m, tiles_n, 4, band_n, pm, pn);
     }
     const int row0 = pm * BM, col0 = pn * BN;
 
@@ -553,7 +553,7 @@ static int launch_tile(const void* A, const void* B, void* C, int M, int N, int 
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(WM * WN * 64), kLdsBytes, stream,
                        (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
-                       tiles_n);
+                       tiles_n, raster_band(((long long)M + N) * K, tiles_n));
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
@@ -599,7 +599,7 @@ static int launch_4wave(const void* A, const void* B, void* C, int M, int N, int
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream,
                        (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
-                       tiles_n);
+                       tiles_n, raster_band(((long long)M + N) * K, tiles_n));
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 

@@ -223,4 +223,18 @@ __device__ __forceinline__ void grouped_raster(int id, int tiles_m, int tiles_n,
     if (group & 1) pn = tiles_n - 1 - pn;
 }
 
+// grouped_raster inside bands of `band_n` tile columns (the last band takes the remainder): a run
+// of 256 ids then covers a squarish 16 x 16 patch of tiles whose B panels stay in the memory-side
+// cache while the band's tile rows stream past, instead of a stripe across all columns.
+__device__ __forceinline__ void banded_raster(int id, int tiles_m, int tiles_n, int group_m, int band_n,
+                                              int& pm, int& pn) {
+    const int bands = max(1, tiles_n / band_n);
+    const int per_band = tiles_m * band_n;
+    const int band = min(id / per_band, bands - 1);
+    const int first_n = band * band_n;
+    const int width = band < bands - 1 ? band_n : tiles_n - first_n;
+    grouped_raster(id - band * per_band, tiles_m, width, group_m, pm, pn);
+    pn += first_n;
+}
+
 }  // namespace hk

@@ -42,7 +42,7 @@ template <bool EDGE>
 __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
     const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int sa_pitch,
-    int sb_pitch, int tiles_m, int tiles_n) {
+    int sb_pitch, int tiles_m, int tiles_n, int band_n) {
     constexpr int NW = 4, TM = 128, TN = 128, MT = 8, NT = 8;
     constexpr int NDMA = kTileBytes / (NW * 1024);
     constexpr int PG = 4, AD = 3;
@@ -57,7 +57,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     int pm, pn;
     {
         const int id = xcd_chunk_order(blockIdx.x, tiles_m * tiles_n, kCuPerXcd);
-        grouped_raster(id, tiles_m, tiles_n, 8, pm, pn);
+        banded_raster(id, tiles_m, tiles_n, band_n < tiles_n ? 4 : 8, band_n, pm, pn);
     }
     const int row0 = pm * BM, col0 = pn * BN;
     const int a_rows = min(M - row0, BM), b_rows = min(N - col0, BN);
@@ -367,7 +367,8 @@ static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, cons
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), kLdsBytesFp4, stream,
                        (const uint8_t*)A, (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB,
-                       (uint16_t*)C, M, N, K, sa_pitch, sb_pitch, tiles_m, tiles_n);
+                       (uint16_t*)C, M, N, K, sa_pitch, sb_pitch, tiles_m, tiles_n,
+                       raster_band(((long long)M + N) * (K / 2), tiles_n));
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
