@@ -341,26 +341,8 @@ __global__ __launch_bounds__(256) void moe_sort_scan_kernel(int32_t* __restrict_
     if (t == 0) totals[e] = carry;
 }
 
-// expert_offsets[0..E] = exclusive prefix sum of the per-expert totals.
-__global__ __launch_bounds__(512) void moe_sort_offsets_kernel(const int32_t* __restrict__ totals, int E,
-                                                               int32_t* __restrict__ expert_offsets) {
-    __shared__ int scan[512];
-    const int e = threadIdx.x;
-    const int v = e < E ? totals[e] : 0;
-    scan[e] = v;
-    __syncthreads();
-    for (int d = 1; d < 512; d <<= 1) {
-        const int u = e >= d ? scan[e - d] : 0;
-        __syncthreads();
-        scan[e] += u;
-        __syncthreads();
-    }
-    if (e < E) expert_offsets[e] = scan[e] - v;
-    if (e == 511) expert_offsets[E] = scan[511];
-}
-
-// Both steps above in one workgroup when there are few chunks: thread e walks expert e's
-// per-chunk counts, then the workgroup scans the totals.
+// The scan above and the exclusive prefix sum of the totals (expert_offsets[0..E]) in one workgroup
+// when there are few chunks: thread e walks expert e's per-chunk counts, then the workgroup scans the totals.
 constexpr int kSortFusedChunks = 64;
 __global__ __launch_bounds__(512) void moe_sort_scan_offsets_kernel(int32_t* __restrict__ ws, int nchunks, int E,
                                                                     int32_t* __restrict__ expert_offsets) {
@@ -458,6 +440,46 @@ __global__ __launch_bounds__(256) void moe_sort_scatter_kernel(const int32_t* __
     sort_scatter_chunk(ids, S, E, chunk, round_cnt,
                        [&](int e) { return expert_offsets[e] + ws[(size_t)chunk * E + e]; }, sorted_slots,
                        slot_to_pos);
+}
+
+// moe_sort_scatter_kernel for many chunks: expert_offsets does not exist yet; every workgroup scans
+// the per-expert totals itself (E <= 512 values, two per thread) and workgroup 0 stores the result,
+// which saves a launch for the prefix sum of the totals.
+__global__ __launch_bounds__(256) void moe_sort_scatter_totals_kernel(const int32_t* __restrict__ ids, int S, int E,
+                                                                      const int32_t* __restrict__ ws,
+                                                                      const int32_t* __restrict__ totals,
+                                                                      int32_t* __restrict__ expert_offsets,
+                                                                      int32_t* __restrict__ sorted_slots,
+                                                                      int32_t* __restrict__ slot_to_pos) {
+    __shared__ int round_cnt[16][kSortMaxE];
+    __shared__ int first[kSortMaxE];
+    __shared__ int wave_tot[4];
+    const int lane = lane_id(), wv = threadIdx.x >> 6, tid = threadIdx.x;
+    const int chunk = blockIdx.x;
+    const int e0 = 2 * tid, e1 = 2 * tid + 1;
+    const int t0 = e0 < E ? totals[e0] : 0, t1 = e1 < E ? totals[e1] : 0;
+    int incl = t0 + t1;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int u = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += u;
+    }
+    if (lane == 63) wave_tot[wv] = incl;
+    __syncthreads();
+    int before = 0;
+#pragma unroll
+    for (int w2 = 0; w2 < 4; ++w2) before += w2 < wv ? wave_tot[w2] : 0;
+    const int x0 = before + incl - t0 - t1, x1 = x0 + t0;
+    if (e0 < E) first[e0] = x0 + ws[(size_t)chunk * E + e0];
+    if (e1 < E) first[e1] = x1 + ws[(size_t)chunk * E + e1];
+    if (chunk == 0) {
+        if (e0 < E) expert_offsets[e0] = x0;
+        if (e1 < E) expert_offsets[e1] = x1;
+        if (e0 == E - 1) expert_offsets[E] = x0 + t0;
+        if (e1 == E - 1) expert_offsets[E] = x1 + t1;
+    }
+    __syncthreads();
+    sort_scatter_chunk(ids, S, E, chunk, round_cnt, [&](int e) { return first[e]; }, sorted_slots, slot_to_pos);
 }
 
 // The whole sort in one launch for S <= 16384 slots (the layer of a few thousand tokens, where
@@ -595,13 +617,14 @@ extern "C" int hk_moe_sort(const int32_t* ids, int T, int k, int E, int32_t* sor
     hipLaunchKernelGGL(moe_sort_count_kernel, dim3(nchunks), dim3(256), 0, s, ids, S, E, ws);
     if (nchunks <= kSortFusedChunks) {
         hipLaunchKernelGGL(moe_sort_scan_offsets_kernel, dim3(1), dim3(512), 0, s, ws, nchunks, E, expert_offsets);
+        hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(nchunks), dim3(256), 0, s, ids, S, E,
+                           (const int32_t*)ws, (const int32_t*)expert_offsets, sorted_slots, slot_to_pos_or_null);
     } else {
         int32_t* totals = ws + (size_t)nchunks * E;
         hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(E), dim3(256), 0, s, ws, nchunks, E, totals);
-        hipLaunchKernelGGL(moe_sort_offsets_kernel, dim3(1), dim3(512), 0, s, (const int32_t*)totals, E,
-                           expert_offsets);
+        hipLaunchKernelGGL(moe_sort_scatter_totals_kernel, dim3(nchunks), dim3(256), 0, s, ids, S, E,
+                           (const int32_t*)ws, (const int32_t*)totals, expert_offsets, sorted_slots,
+                           slot_to_pos_or_null);
     }
-    hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(nchunks), dim3(256), 0, s, ids, S, E,
-                       (const int32_t*)ws, (const int32_t*)expert_offsets, sorted_slots, slot_to_pos_or_null);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
