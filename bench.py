@@ -163,6 +163,24 @@ def bench_fp8_decode(torch, hk, warmup, iters, dev):
     return out
 
 
+def bench_mxfp4_decode(torch, hk, warmup, iters, dev):
+    """MXFP4 decode-like shapes: few rows against a weight matrix that is read once."""
+    out = []
+    g = torch.Generator(device=dev).manual_seed(0)
+    for M, N, K in ((16, 8192, 8192), (16, 4096, 14336)):
+        A, SA = hk.quant.quantize_mxfp4(torch.randn(M, K, device=dev, generator=g))
+        B, SB = hk.quant.quantize_mxfp4(torch.randn(N, K, device=dev, generator=g))
+        C = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        ws = torch.empty(max(16, hk.tk_kernel.mxfp4_gemm_workspace_bytes(M, N, K)), dtype=torch.uint8, device=dev)
+        _, plain = _timeit(torch, lambda: hk.tk_kernel.dispatch_mxfp4_gemm(A, SA, B, SB, C), warmup, iters)
+        _, split = _timeit(torch, lambda: hk.tk_kernel.dispatch_mxfp4_gemm(A, SA, B, SB, C, workspace=ws), warmup, iters)
+        byts = (M + N) * (K // 2 + K // 32) + 2 * M * N
+        out.append({"shape": f"M={M} N={N} K={K}", "us_without_workspace": round(plain * 1e3, 1),
+                    "us_split_k": round(split * 1e3, 1), "GB/s": round(byts / (split * 1e-3) / 1e9, 1),
+                    "frac_of_hbm": round(byts / (split * 1e-3) / 1e9 / PEAK_HBM, 4)})
+    return out
+
+
 def bench_mxfp4(torch, hk, n, warmup, iters, dev):
     g = torch.Generator(device=dev).manual_seed(0)
     A, SA = hk.quant.quantize_mxfp4(torch.randn(n, n, device=dev, generator=g))
@@ -408,6 +426,7 @@ def main() -> int:
         extra["library_on_this_box_8192"] = bench_library_baselines(torch, 8192, 500, 100, dev)
         torch.cuda.empty_cache()
         extra["mxfp4_gemm"] = bench_mxfp4(torch, hk, 8192, 500, 100, dev)
+        extra["mxfp4_gemm_decode"] = bench_mxfp4_decode(torch, hk, 50, 50, dev)
         extra["moe_mxfp4"] = bench_moe_mxfp4(torch, hk, quick_w, quick_i, dev, graph=not args.no_graph)
         torch.cuda.empty_cache()
         extra["moe_fp8blk"] = bench_moe_fp8blk(torch, hk, 5, 10, dev)

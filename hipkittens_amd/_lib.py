@@ -16,6 +16,8 @@ SIGNATURES = {
     "hk_fp8_gemm_variant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_int, c_void_p]),
     "hk_mxfp4_gemm": (c_int, [c_void_p] * 5 + [c_int] * 3 + [c_void_p]),
     "hk_mxfp4_gemm_variant": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_void_p]),
+    "hk_mxfp4_gemm_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "hk_mxfp4_gemm_ws": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p] + [c_int] * 3 + [c_void_p, c_size_t, c_void_p]),
     "hk_mxfp4_gemm_pitched": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p] + [c_int] * 3 + [c_void_p]),
     "hk_bf16_gemm": (c_int, [c_void_p] * 3 + [c_int] * 3 + [c_void_p]),
     "hk_fp8_gemm_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),

@@ -236,14 +236,14 @@ int moe_num_compute_units();  // number of CUs of the current device, cached (mo
 
 // Number of K ranges the split-K path would use: as many as fill the CUs, each at least 4
 // K-steps long, at most 16; 1 = the problem has enough tiles or too short a K.
-// K: the operands' row length in bytes.
-static inline int splitk_ranges(int M, int N, int K) {
+// K: the operands' row length in bytes; min_nk: the shortest K (in K-steps) that is split.
+static inline int splitk_ranges(int M, int N, int K, int min_nk = 48) {
     // 64x64 tiles, two workgroups per CU
     const long long tiles = (long long)((M + kTinyTile - 1) / kTinyTile) * ((N + kTinyTile - 1) / kTinyTile);
     const int nk = (K + BK - 1) / BK;
     const int cus = moe_num_compute_units();   // 256 when no device can be queried
     // shorter K: the 64x64-tile kernel without a second launch is as fast or faster
-    if (tiles > cus || nk < 48) return 1;
+    if (tiles > cus || nk < min_nk) return 1;
     long long s = 2 * cus / tiles;
     if (s > nk / 4) s = nk / 4;
     if (s > 16) s = 16;

@@ -324,14 +324,14 @@ struct Mxfp4Mma {
     }
 };
 // K: the operands' row length in bytes (two elements per byte).
-template <int TILE, int STAGES, bool EDGE>
+template <int TILE, int STAGES, bool EDGE, bool SPLIT = false>
 __global__ __launch_bounds__(256) void mxfp4_gemm_small_tile_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
     const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int sa_pitch,
-    int sb_pitch, int tiles_m, int tiles_n) {
+    int sb_pitch, int tiles_m, int tiles_n, int kps, float* __restrict__ partial) {
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
-    gemm_small_tile_body<Mxfp4Mma, TILE, STAGES, EDGE, false>(smem, A, B, C, M, N, K, 1.0f, tiles_m, tiles_n, 0,
-                                                              nullptr, SmallTileScales{SA, SB, sa_pitch, sb_pitch});
+    gemm_small_tile_body<Mxfp4Mma, TILE, STAGES, EDGE, SPLIT>(smem, A, B, C, M, N, K, 1.0f, tiles_m, tiles_n, kps,
+                                                              partial, SmallTileScales{SA, SB, sa_pitch, sb_pitch});
 }
 
 template <int TILE, int STAGES, bool EDGE>
@@ -349,7 +349,49 @@ static int launch_mxfp4_small_tile(const void* A, const void* SA, const void* B,
     const int tiles_m = (M + TILE - 1) / TILE, tiles_n = (N + TILE - 1) / TILE;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream, (const uint8_t*)A,
                        (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB, (uint16_t*)C, M, N, K / 2,
-                       sa_pitch, sb_pitch, tiles_m, tiles_n);
+                       sa_pitch, sb_pitch, tiles_m, tiles_n, 0, (float*)nullptr);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
+// Split-K over 64x64 tiles for problems with few tiles and a long K (decode shapes): `splits` K ranges of
+// an even number of K-steps each (a range then starts on a pair of K-steps, the unit of a scale load),
+// fp32 partial sums, and the fixed-order reduction behind them. K in elements.
+constexpr int kMxfp4SplitMinSteps = 16;
+// Number of K ranges for the MXFP4 GEMM (1: not split). On top of the common rule: at least four ranges
+// (fewer only occur when the plain kernel already keeps more than half of the CUs busy: measured slower),
+// and the time saved, 0.4 us per K-step taken off a workgroup's K loop, must exceed the second launch
+// (2.5 us) and writing and reading the partial sums at 4 TB/s (M = 128, N = K = 4096: 9.0 us plain,
+// 10.9 us split four ways, so not split; M = 16: 8.6 -> 6.6 us).
+static int mxfp4_splitk_ranges(int M, int N, int K) {
+    const int s = splitk_ranges(M, N, K / 2, kMxfp4SplitMinSteps);
+    if (s < 4) return 1;
+    const int nk = (K / 2 + BK - 1) / BK;
+    const double saved_us = 0.4 * nk * (1.0 - 1.0 / s);
+    const double cost_us = 2.5 + 8.0 * s * (double)M * (double)N / 4e6;
+    return saved_us > cost_us ? s : 1;
+}
+template <bool EDGE>
+static int launch_mxfp4_splitk(const void* A, const void* SA, const void* B, const void* SB, void* C, int M, int N,
+                               int K, int sa_pitch, int sb_pitch, int splits, float* partial, hipStream_t stream) {
+    auto kern = mxfp4_gemm_small_tile_kernel<kTinyTile, kTinyStages, EDGE, true>;
+    constexpr int lds_bytes = small_tile_lds_bytes<kTinyTile, kTinyStages>(true);
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) !=
+            hipSuccess)
+            return HK_ERR_LAUNCH;
+        configured = true;
+    }
+    const int tiles_m = (M + kTinyTile - 1) / kTinyTile, tiles_n = (N + kTinyTile - 1) / kTinyTile;
+    const int nk = (K / 2 + BK - 1) / BK;
+    const int kps = ((nk + splits - 1) / splits + 1) & ~1;
+    const int used = (nk + kps - 1) / kps;   // ranges that hold at least one K-step
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, used), dim3(256), lds_bytes, stream, (const uint8_t*)A,
+                       (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB, (uint16_t*)C, M, N, K / 2,
+                       sa_pitch, sb_pitch, tiles_m, tiles_n, kps, partial);
+    const long long mn = (long long)M * N;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((mn / 4 + 256) / 256)), dim3(256), 0, stream,
+                       (const float*)partial, used, mn, 1.0f, (uint16_t*)C);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
@@ -434,6 +476,38 @@ extern "C" int hk_mxfp4_gemm_variant(const void* A, const void* A_scales, const 
 extern "C" int hk_mxfp4_gemm(const void* A, const void* A_scales, const void* B, const void* B_scales,
                              void* C, int M, int N, int K, void* stream) {
     return mxfp4_gemm_impl(A, A_scales, K / 32, B, B_scales, K / 32, C, M, N, K, -1, stream);
+}
+
+extern "C" size_t hk_mxfp4_gemm_workspace_bytes(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const int s = hk::mxfp4_splitk_ranges(M, N, K);
+    return s < 2 ? 0 : (size_t)s * M * N * sizeof(float);
+}
+
+extern "C" int hk_mxfp4_gemm_ws(const void* A, const void* A_scales, int a_scale_pitch, const void* B,
+                                const void* B_scales, int b_scale_pitch, void* C, int M, int N, int K,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace hk;
+    if (M <= 0 || N <= 0 || K <= 0 || (K % 32) != 0) return HK_ERR_BAD_SHAPE;
+    const int splits = mxfp4_splitk_ranges(M, N, K);
+    const int groups = (K / 32 + 7) / 8 * 8;
+    // what the tile kernels need of the scale rows (see mxfp4_gemm_impl); anything else takes the plain path
+    const bool tile_ok = (a_scale_pitch % 8) == 0 && (b_scale_pitch % 8) == 0 && a_scale_pitch >= groups &&
+                         b_scale_pitch >= groups && A_scales && B_scales &&
+                         ((((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) == 0) &&
+                         (long long)(K / 2) * BM < (1ll << 31) &&
+                         (long long)BM * max(a_scale_pitch, b_scale_pitch) < (1ll << 31);
+    const bool can_split = splits >= 2 && workspace && workspace_bytes >= (size_t)splits * M * N * sizeof(float) &&
+                           tile_ok && (long long)M * N < (1ll << 40);
+    if (!can_split)
+        return mxfp4_gemm_impl(A, A_scales, a_scale_pitch, B, B_scales, b_scale_pitch, C, M, N, K, -1, stream);
+    if (!A || !B || !C) return HK_ERR_NULL_POINTER;
+    if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)workspace) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    const bool edge = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
+    return edge ? launch_mxfp4_splitk<true>(A, A_scales, B, B_scales, C, M, N, K, a_scale_pitch, b_scale_pitch, splits,
+                                            (float*)workspace, (hipStream_t)stream)
+                : launch_mxfp4_splitk<false>(A, A_scales, B, B_scales, C, M, N, K, a_scale_pitch, b_scale_pitch,
+                                             splits, (float*)workspace, (hipStream_t)stream);
 }
 
 extern "C" int hk_mxfp4_gemm_pitched(const void* A, const void* A_scales, int a_scale_pitch, const void* B,

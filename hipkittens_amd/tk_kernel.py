@@ -127,12 +127,19 @@ _FP4 = tuple(d for d in (torch.uint8, getattr(torch, "float4_e2m1fn_x2", None)) 
 _E8M0 = tuple(d for d in (torch.uint8, getattr(torch, "float8_e8m0fnu", None)) if d is not None)
 
 
-def dispatch_mxfp4_gemm(A, A_scales, B, B_scales, C, variant: int = -1) -> None:
+def mxfp4_gemm_workspace_bytes(M: int, N: int, K: int) -> int:
+    """Bytes of workspace with which dispatch_mxfp4_gemm splits K for this shape (0: it would not)."""
+    return int(_lib.load_library().hk_mxfp4_gemm_workspace_bytes(int(M), int(N), int(K)))
+
+
+def dispatch_mxfp4_gemm(A, A_scales, B, B_scales, C, variant: int = -1, workspace=None) -> None:
     """C[M,N] (bf16) = dequant(A) @ dequant(B).T for MXFP4 operands: A [M,K/2] packed e2m1
     (low nibble = even k), A_scales [M,K/32] e8m0, B [N,K/2], B_scales [N,K/32]. The scale tensors
     may be wider than K/32 (padded rows, e.g. quant.pad_scales: any byte but 0xFF in the padding);
     rows that are a multiple of 8 bytes keep a K that is not a multiple of 256 on the tile kernels.
-    `variant` -1 lets the library choose; 0..3 force a kernel (see include/hk355.h)."""
+    `variant` -1 lets the library choose; 0..3 force a kernel (see include/hk355.h).
+    `workspace` (uint8, mxfp4_gemm_workspace_bytes(M, N, K) bytes): lets the library split K for
+    decode-like shapes (hk_mxfp4_gemm_ws)."""
     _check_tensor(A, "A", _FP4, 2)
     _check_tensor(B, "B", _FP4, 2)
     _check_tensor(A_scales, "A_scales", _E8M0, 2)
@@ -151,7 +158,15 @@ def dispatch_mxfp4_gemm(A, A_scales, B, B_scales, C, variant: int = -1) -> None:
     lib = _lib.load_library()
     args = (A.data_ptr(), A_scales.data_ptr(), B.data_ptr(), B_scales.data_ptr(), C.data_ptr(), M, N, K)
     pa, pb = A_scales.shape[1], B_scales.shape[1]
-    if pa != K // 32 or pb != K // 32:
+    if workspace is not None:
+        if variant >= 0:
+            raise RuntimeError("a workspace and a forced variant exclude each other")
+        _check_tensor(workspace, "workspace", (torch.uint8,), 1)
+        if workspace.device != A.device:
+            raise RuntimeError("all tensors must be on the same device")
+        st = lib.hk_mxfp4_gemm_ws(A.data_ptr(), A_scales.data_ptr(), pa, B.data_ptr(), B_scales.data_ptr(), pb,
+                                  C.data_ptr(), M, N, K, workspace.data_ptr(), workspace.numel(), _stream(A))
+    elif pa != K // 32 or pb != K // 32:
         if variant >= 0:
             raise RuntimeError("padded scale rows and a forced variant exclude each other")
         st = lib.hk_mxfp4_gemm_pitched(A.data_ptr(), A_scales.data_ptr(), pa, B.data_ptr(), B_scales.data_ptr(), pb,

@@ -103,6 +103,18 @@ int hk_mxfp4_gemm_pitched(const void* A_e2m1, const void* A_scales_e8m0, int a_s
                           const void* B_e2m1, const void* B_scales_e8m0, int b_scale_pitch,
                           void* C_bf16, int M, int N, int K, void* stream);
 
+/* The MXFP4 GEMM (scale rows with pitches, as hk_mxfp4_gemm_pitched; dense rows: pitch K / 32) with an
+ * optional workspace for decode-like shapes, as hk_fp8_gemm_ws: few 64x64 tiles (at most a quarter of
+ * what fills the GPU) and a K of at least 16 K-steps of 256 elements are split along K into fp32 partial
+ * sums, added in a fixed order, when the shorter K loops save more time than the partial sums cost.
+ * hk_mxfp4_gemm_workspace_bytes returns 0 for shapes that would not be split; without a (large enough,
+ * 16-byte aligned) workspace, or with scale rows the tile kernels do not take, the call is
+ * hk_mxfp4_gemm_pitched. No counterpart in the reference. */
+size_t hk_mxfp4_gemm_workspace_bytes(int M, int N, int K);
+int hk_mxfp4_gemm_ws(const void* A_e2m1, const void* A_scales_e8m0, int a_scale_pitch, const void* B_e2m1,
+                     const void* B_scales_e8m0, int b_scale_pitch, void* C_bf16, int M, int N, int K,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
 /*
  * BF16 GEMM: C[M,N] = bf16( A[M,K] * B[N,K]^T ), A and B row-major bf16, fp32 accumulation, RNE.
  * Replaces the reference's flagship kernel behind tk_kernel.dispatch_micro(A, B, C)

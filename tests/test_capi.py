@@ -66,6 +66,14 @@ def test_c_entry_points_reject_bad_arguments_without_a_gpu():
     assert lib.hk_mxfp4_gemm_pitched(p, p, 88, p, p, 96, p, 64, 64, 2880, None) == -2    # pitch < K / 32
     assert lib.hk_mxfp4_gemm_pitched(p, None, 96, p, p, 96, p, 64, 64, 2880, None) == -1
     assert lib.hk_mxfp4_gemm_pitched(p, p, 96, p, p, 96, p, 64, 64, 2872, None) == -2    # K % 32
+    assert lib.hk_mxfp4_gemm_ws(p, p, 256, p, p, 256, p, 0, 64, 8192, None, 0, None) == -2
+    assert lib.hk_mxfp4_gemm_ws(p, p, 256, p, p, 256, p, 16, 1024, 8176, p, 1 << 40, None) == -2     # K % 32
+    assert lib.hk_mxfp4_gemm_ws(None, p, 256, p, p, 256, p, 16, 1024, 8192, p, 1 << 40, None) == -1  # split path
+    assert lib.hk_mxfp4_gemm_ws(p, p, 256, p, p, 256, p, 16, 1024, 8192, p + 4, 1 << 40, None) == -3
+    assert lib.hk_mxfp4_gemm_ws(p, p, 255, p, p, 256, p, 16, 1024, 8192, p, 1 << 40, None) == -2     # pitch < K / 32
+    assert lib.hk_mxfp4_gemm_workspace_bytes(16, 1024, 8192) % (16 * 1024 * 4) == 0
+    assert lib.hk_mxfp4_gemm_workspace_bytes(16, 1024, 8192) > 0
+    assert lib.hk_mxfp4_gemm_workspace_bytes(8192, 8192, 8192) == 0
     # extended MoE entry points: option checks come before anything touches memory
     args = (p, p, p, 8, p, p, 8, p, p, p, p, p, 16, 64, 32, 4, 2, 0)
     assert lib.hk_moe_mxfp4_experts_ex(*args, None, None, 7, 1.702, 7.0, 0, p, 1 << 30, None) == -6   # activation

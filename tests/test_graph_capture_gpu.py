@@ -56,6 +56,20 @@ def test_fp8_split_k_in_a_graph(hk):
                         scratch_fn=lambda: ws.fill_(0xFF))
 
 
+def test_mxfp4_split_k_in_a_graph(hk):
+    M, N, K = 16, 1024, 8192
+    print("graph mxfp4_gemm split-k", flush=True)
+    g = torch.Generator(device=DEV).manual_seed(5)
+    Ap, As = hk.quant.quantize_mxfp4(torch.randn(M, K, device=DEV, generator=g))
+    Bp, Bs = hk.quant.quantize_mxfp4(torch.randn(N, K, device=DEV, generator=g))
+    C = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    need = hk.tk_kernel.mxfp4_gemm_workspace_bytes(M, N, K)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    _replay_and_compare(lambda: hk.tk_kernel.dispatch_mxfp4_gemm(Ap, As, Bp, Bs, C, workspace=ws), [C],
+                        scratch_fn=lambda: ws.fill_(0xFF))
+
+
 def test_bf16_and_mxfp4_gemm_in_a_graph(hk):
     print("graph bf16 / mxfp4 gemm", flush=True)
     g = torch.Generator(device=DEV).manual_seed(2)

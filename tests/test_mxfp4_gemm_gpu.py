@@ -158,3 +158,41 @@ def test_mxfp4_gemm_padded_rows_equal_dense_rows_bit_for_bit(hk):
     dense = _run(hk, a, sa, b, sb)
     padded = _run(hk, a, _pad_rows(rng, sa, 40), b, _pad_rows(rng, sb, 48))
     assert np.array_equal(dense, padded)
+
+
+SPLITK = [(16, 1024, 8192, 0), (1, 512, 8192, 0), (100, 200, 4128, 136), (128, 1000, 6176, 200), (64, 64, 16384, 0)]
+
+
+@pytest.mark.parametrize("case", SPLITK)
+def test_mxfp4_gemm_split_k_matches_oracle(hk, case):
+    """Decode-like shapes with a workspace: K split over several workgroups per tile (ranges of an even
+    number of K-steps; the last range of two cases ends in a partial K-step), fp32 partial sums added
+    in a fixed order. The workspace starts as NaNs, so a partial sum that is read but was not written
+    would show; with a workspace that is too small the call must give the plain kernel's result."""
+    M, N, K, pitch = case
+    print(f"mxfp4_gemm split-k case={case}", flush=True)
+    need = hk.tk_kernel.mxfp4_gemm_workspace_bytes(M, N, K)
+    assert need > 0, "these shapes are meant to take the split path"
+    assert hk.tk_kernel.mxfp4_gemm_workspace_bytes(1024, 1024, 8192) == 0    # enough tiles
+    assert hk.tk_kernel.mxfp4_gemm_workspace_bytes(16, 2880, 2880) == 0      # K too short
+    assert hk.tk_kernel.mxfp4_gemm_workspace_bytes(128, 4096, 4096) == 0     # partial sums cost more than they save
+    rng = np.random.default_rng(3 + M + N + K)
+    (a, sa), (b, sb) = _rand_mx(rng, M, K), _rand_mx(rng, N, K)
+    ref = G.mxfp4_gemm(a, sa, b, sb)
+    if pitch:
+        sa, sb = _pad_rows(rng, sa, pitch), _pad_rows(rng, sb, pitch)
+    dev = torch.device("cuda:0")
+    t = [torch.from_numpy(x).to(dev) for x in (a, sa, b, sb)]
+    ws = torch.full((need,), 0xFF, dtype=torch.uint8, device=dev)
+    C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    hk.tk_kernel.dispatch_mxfp4_gemm(*t, C, workspace=ws)
+    torch.cuda.synchronize()
+    out = C.float().cpu().numpy()
+    assert np.isfinite(out).all()
+    assert G.rel_fro_error(out, ref) <= 5e-3
+    plain = torch.empty_like(C)
+    hk.tk_kernel.dispatch_mxfp4_gemm(*t, plain)
+    small = torch.empty_like(C)
+    hk.tk_kernel.dispatch_mxfp4_gemm(*t, small, workspace=ws[:need - 16])
+    torch.cuda.synchronize()
+    assert torch.equal(plain.view(torch.int16), small.view(torch.int16))
