@@ -82,12 +82,17 @@ struct MoeFp8Params {
     int topk, T;
 };
 
-constexpr int kF8ATile = kMoeBM * 128;             // 16 KiB
+// Rows of a work item: 160, the most that leaves room for three LDS stages. An expert with up to 320
+// rows then takes two passes over its weights (with 256 +- 16 rows per expert, the DeepSeek-V3 shape at
+// 8192 tokens, 128-row items needed a third pass for half of the experts).
+constexpr int kF8BM = 160;
+constexpr int kF8ATile = kF8BM * 128;              // 20 KiB
 constexpr int kF8BTile = 256 * 128;                // 32 KiB
-constexpr int kF8Stage = kF8ATile + kF8BTile;      // 48 KiB
-constexpr int kF8ScaleBase = 3 * kF8Stage;         // A scales: 3 stages x kMoeBM floats
-constexpr int kF8XchBase = kF8ScaleBase + 3 * kMoeBM * 4;  // epilogue exchange: kMoeBM x 4 floats
-constexpr int kF8Lds = kF8XchBase + kMoeBM * 16;
+constexpr int kF8Stage = kF8ATile + kF8BTile;      // 52 KiB
+constexpr int kF8ScaleBase = 3 * kF8Stage;         // A scales: 3 stages x kF8BM floats
+constexpr int kF8Lds = kF8ScaleBase + 3 * kF8BM * 4;   // 157.9 KiB
+// (the gate+up epilogue's exchange buffer, kF8BM x 4 floats, lies in the stage the K loop used last)
+static_assert(kF8Lds <= 160 * 1024 && kF8BM % 32 == 0 && kF8BM > 128 && kF8BM <= 192, "see the A-tile loads");
 
 // dword global->LDS load restricted to the lanes in `mask` (lane l lands at lds_base + 4*l)
 __device__ __forceinline__ void dma4_lanes(v4i srd, uint32_t lds_base, uint32_t voff, uint32_t soff,
@@ -112,7 +117,7 @@ struct MoeFp8Addr {
     const float* sb1;  // MODE 0: scales of the up-projection row block
     int row_start, rows, n0, n_tile;
     bool valid;
-    uint32_t gvoff_a[kMoeBM / 64], gvoff_sa;  // GATHER: per-lane source offsets of the item's activation rows / scales
+    uint32_t gvoff_a[(kF8BM + 63) / 64], gvoff_sa;  // GATHER: per-lane source offsets of the item's activation rows / scales
 };
 
 // GATHER (MODE 0 only): the activation tile's rows are fetched from the caller's x by token index
@@ -121,7 +126,10 @@ struct MoeFp8Addr {
 template <int MODE, bool GATHER>
 __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params p) {
     static_assert(!GATHER || MODE == 0, "only the gate+up GEMM reads the caller's activations");
-    constexpr int NW = 8, MT = kMoeBM / 32, NT = 4, NA = kMoeBM / 64;
+    // The A tile is loaded in NA = 3 pieces of 64 rows (8 per wave); of the third piece only rows 128..159
+    // exist: waves 4..7 fetch what waves 0..3 fetch (same bytes to the same place), which keeps the number
+    // of loads per wave uniform for the counted waits.
+    constexpr int NW = 8, MT = kF8BM / 32, NT = 4, NA = (kF8BM + 63) / 64, SR = kF8BM / 8;
     constexpr int kDma = NA + 4 + 1;
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
     const int lane = lane_id(), w = wave_id();
@@ -139,7 +147,10 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
     const int rows_b = MODE == 0 ? 2 * p.N : p.N;
     const v4i srd_a = make_srd(p.A, GATHER ? (uint32_t)p.T * (uint32_t)p.K : (uint32_t)nk * (uint32_t)p.S * 128u);
     const v4i srd_sa = make_srd(p.SA, GATHER ? (uint32_t)p.T * (uint32_t)nk * 4u : (uint32_t)nk * (uint32_t)p.S * 4u);
-    const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);
+    const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);   // depends on w & 1 only
+    // tile row this lane loads in piece i of the A tile
+    auto piece_row = [&](int i) { return i < 2 ? 8 * (i * NW + w) + (lane >> 3) : 128 + 8 * (w & 3) + (lane >> 3); };
+    auto piece_row0 = [&](int i) { return i < 2 ? 8 * (i * NW + w) : 128 + 8 * (w & 3); };
 
     // GATHER: sorted slot indices of the activation rows this lane loads for an item (NA tile pieces
     // and the scale row). They are fetched two items ahead with loads the compiler does not see
@@ -152,10 +163,10 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
         const int row_start = scalar_load_x4(p.items + idx).y;
 #pragma unroll
         for (int i = 0; i < NA; ++i) {
-            const uint32_t off = (uint32_t)min(row_start + 8 * (i * NW + w) + (lane >> 3), p.S - 1) * 4u;
+            const uint32_t off = (uint32_t)min(row_start + piece_row(i), p.S - 1) * 4u;
             asm volatile("global_load_dword %0, %1, %2" : "=v"(o.a[i]) : "v"(off), "s"(p.sorted_slots) : "memory");
         }
-        const uint32_t off = (uint32_t)min(row_start + w * (kMoeBM / 8) + (lane & (kMoeBM / 8 - 1)), p.S - 1) * 4u;
+        const uint32_t off = (uint32_t)min(row_start + w * SR + min(lane, SR - 1), p.S - 1) * 4u;
         asm volatile("global_load_dword %0, %1, %2" : "=v"(o.s) : "v"(off), "s"(p.sorted_slots) : "memory");
     };
     auto landed_ids = [&](SlotIds& o) __attribute__((always_inline)) {
@@ -181,10 +192,10 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
             // rows past the item's count are not fetched at all (bit 31: out of range, LDS gets zeros)
 #pragma unroll
             for (int i = 0; i < NA; ++i)
-                a.gvoff_a[i] = 8 * (i * NW + w) + (lane >> 3) < a.rows
+                a.gvoff_a[i] = piece_row(i) < a.rows
                                    ? (ids.a[i] / (uint32_t)p.topk) * (uint32_t)p.K + chunk16 * 16u
                                    : 0x80000000u;
-            a.gvoff_sa = w * (kMoeBM / 8) + (lane & (kMoeBM / 8 - 1)) < a.rows
+            a.gvoff_sa = w * SR + min(lane, SR - 1) < a.rows
                              ? (ids.s / (uint32_t)p.topk) * (uint32_t)nk * 4u
                              : 0x80000000u;
         }
@@ -200,12 +211,17 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-    const uint32_t lds_sa_wave = to_sgpr(lds0 + kF8ScaleBase + (uint32_t)w * (kMoeBM / 8) * 4u);
+    const uint32_t lds_sa_wave = to_sgpr(lds0 + kF8ScaleBase + (uint32_t)w * SR * 4u);
+    // LDS offset of this wave's part of A piece i within a stage
+    const uint32_t lds_a2 = to_sgpr(lds0 + (uint32_t)(2 * NW + (w & 3)) * 1024u);
+    auto a_piece_dst = [&](int stage, int i) {
+        return (i < 2 ? lds_wave + (uint32_t)i * NW * 1024 : lds_a2) + (uint32_t)stage * kF8Stage;
+    };
     uint32_t voff_a[NA];
 #pragma unroll
-    for (int i = 0; i < NA; ++i) voff_a[i] = (uint32_t)(8 * (i * NW + w) + (lane >> 3)) * 128u + chunk16 * 16u;
-    const uint32_t voff_sa = (uint32_t)((w * (kMoeBM / 8) + lane) * 4);
-    constexpr uint64_t kSaMask = (1ull << (kMoeBM / 8)) - 1ull;
+    for (int i = 0; i < NA; ++i) voff_a[i] = (uint32_t)piece_row(i) * 128u + chunk16 * 16u;
+    const uint32_t voff_sa = (uint32_t)((w * SR + lane) * 4);
+    constexpr uint64_t kSaMask = (1ull << SR) - 1ull;
 
     auto issue_tile = [&](const MoeFp8Addr& a, int stage, int kt) {
         v4i sa = srd_a, sb = a.srd_b, ssa = srd_sa;
@@ -215,17 +231,17 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
 #pragma unroll
         for (int i = 0; i < NA; ++i) {
             if (GATHER) {
-                dma16(sa, dst + i * NW * 1024, a.gvoff_a[i], (uint32_t)kt * 128u);
+                dma16(sa, a_piece_dst(stage, i), a.gvoff_a[i], (uint32_t)kt * 128u);
             } else {
                 v4i sai = sa;   // the piece's 8 rows lie past the item's count: nothing is fetched
-                if (8 * (i * NW + w) >= a.rows) sai.z = 0;
-                dma16(sai, dst + i * NW * 1024, voff_a[i], row_base * 128u);
+                if (piece_row0(i) >= a.rows) sai.z = 0;
+                dma16(sai, a_piece_dst(stage, i), voff_a[i], row_base * 128u);
             }
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) dma16(sb, dst + kF8ATile + i * NW * 1024, a.voff_b[i], (uint32_t)kt * 128u);
-        if (GATHER) dma4_lanes(ssa, lds_sa_wave + (uint32_t)stage * (kMoeBM * 4), a.gvoff_sa, (uint32_t)kt * 4u, kSaMask);
-        else dma4_lanes(ssa, lds_sa_wave + (uint32_t)stage * (kMoeBM * 4), voff_sa, row_base * 4u, kSaMask);
+        if (GATHER) dma4_lanes(ssa, lds_sa_wave + (uint32_t)stage * (kF8BM * 4), a.gvoff_sa, (uint32_t)kt * 4u, kSaMask);
+        else dma4_lanes(ssa, lds_sa_wave + (uint32_t)stage * (kF8BM * 4), voff_sa, row_base * 4u, kSaMask);
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
@@ -243,7 +259,7 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
     auto compute = [&](int st, int rows, int kt) {
         uint32_t a_lo = a_lo0 + (uint32_t)st * kF8Stage, a_hi = a_hi0 + (uint32_t)st * kF8Stage;
         uint32_t b_lo = b_lo0 + (uint32_t)st * kF8Stage, b_hi = b_hi0 + (uint32_t)st * kF8Stage;
-        uint32_t sa_rd = sa_rd0 + (uint32_t)st * (kMoeBM * 4);
+        uint32_t sa_rd = sa_rd0 + (uint32_t)st * (kF8BM * 4);
         asm volatile("" : "+v"(a_lo), "+v"(a_hi), "+v"(b_lo), "+v"(b_hi), "+v"(sa_rd));
         const float ws0 = __int_as_float(scalar_load_x1(cur.sb0 + kt));
         const float ws1 = MODE == 0 ? __int_as_float(scalar_load_x1(cur.sb1 + kt)) : ws0;
@@ -266,7 +282,7 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
         }
     };
 
-    auto epilogue = [&](const MoeFp8Addr& a) {
+    auto epilogue = [&](const MoeFp8Addr& a, int free_stage) {
         const int rows = a.rows, row_start = a.row_start, n0 = a.n0;
         if (MODE == 1) {
             uint16_t* out = (uint16_t*)p.out0;
@@ -292,7 +308,9 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
             // waves are combined through LDS.
             uint8_t* hq = (uint8_t*)p.out0;
             float h[MT][8];
-            const uint32_t xch = lds0 + kF8XchBase;
+            // every wave is done with the K loop's last stage: its A tile becomes the exchange buffer
+            const uint32_t xch = lds0 + (uint32_t)free_stage * kF8Stage;
+            __syncthreads();
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
 #pragma unroll
@@ -358,7 +376,7 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
             compute(st, cur.rows, kt);
             st = st == 2 ? 0 : st + 1;
         }
-        epilogue(cur);
+        epilogue(cur, st == 0 ? 2 : st - 1);
         it += it_stride;
         if (it >= it_end) break;
         cur = nxt;
@@ -396,7 +414,7 @@ static Fp8Ws fp8_ws_layout(int T, int H, int I, int E, int k) {
     const size_t S = (size_t)T * k;
     L.ids = take(S * 4); L.w = take(S * 4); L.sorted = take(S * 4); L.offsets = take((size_t)(E + 1) * 4);
     L.inv = take(S * 4); L.sort_ws = take(hk_moe_sort_workspace_bytes(T, k, E));
-    const int max_tiles = (int)(S / kMoeBM) + E;
+    const int max_tiles = (int)(S / kF8BM) + E;
     L.max_items1 = max_tiles * (I / 128);
     L.max_items2 = max_tiles * ((H + 255) / 256);
     L.items1 = take((size_t)L.max_items1 * sizeof(MoeItem));
@@ -457,7 +475,7 @@ extern "C" int hk_moe_fp8blk_experts_ex(const void* x_e4m3, const float* x_scale
     uint8_t* ws = (uint8_t*)workspace;
     const int S = T * k;
     int32_t* nitems = (int32_t*)(ws + L.nitems);
-    moe_launch_build_items(expert_offsets, E, kMoeBM, I / 128, (MoeItem*)(ws + L.items1), (H + 255) / 256,
+    moe_launch_build_items(expert_offsets, E, kF8BM, I / 128, (MoeItem*)(ws + L.items1), (H + 255) / 256,
                            (MoeItem*)(ws + L.items2), nitems, s);
 
     MoeFp8Params p{};

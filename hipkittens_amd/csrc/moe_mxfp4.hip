@@ -127,10 +127,15 @@ __device__ __forceinline__ void moe_build_items_block(const int32_t* __restrict_
     int base = scan[t] - mine;
 #pragma unroll
     for (int j = 0; j < EPT; ++j) {
+        // an expert's rows are spread evenly over its items (in whole 16-row fragments): items of one
+        // expert then take the same time, run side by side and share the expert's weights in L2
+        const int R = hi[j] - lo[j];
+        int per = cnt[j] > 0 ? ((R + cnt[j] - 1) / cnt[j] + 15) & ~15 : bm;
+        if (per > bm || (cnt[j] - 1) * per >= R) per = bm;
         for (int n = part; n < n_tiles_n; n += nparts)
             for (int m = 0; m < cnt[j]; ++m) {
                 MoeItem it;
-                it.expert = t * EPT + j; it.row_start = lo[j] + m * bm; it.rows = min(bm, hi[j] - it.row_start);
+                it.expert = t * EPT + j; it.row_start = lo[j] + m * per; it.rows = min(per, hi[j] - it.row_start);
                 it.n_tile = n;
                 items[base + n * cnt[j] + m] = it;
             }
