@@ -65,8 +65,10 @@ CASES = [
     (300, 8, 4, 4, 2, 512, 384),      # several m-tiles per expert
     (200, 32, 8, 8, 4, 1024, 256),    # DeepSeek-like routing parameters, small dims
     (96, 64, 4, 8, 4, 384, 128),      # many experts with few rows, some empty
-    (600, 8, 4, 4, 2, 256, 128),      # about 300 rows per expert: the 256-row item kernel, two items per expert
+    (600, 8, 4, 4, 2, 256, 128),      # about 300 rows per expert: two items of up to 160 rows per expert
     (520, 4, 2, 2, 1, 128, 256),      # 260 rows per expert, a single K-step in the gate+up GEMM
+    (1000, 4, 2, 2, 1, 256, 128),     # about 500 rows per expert: four items, the rows spread evenly over them
+    (330, 2, 2, 1, 1, 128, 128),      # 330 rows per expert (every token takes both experts): 112 + 112 + 106
 ]
 
 
