@@ -162,54 +162,64 @@ __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __r
 // The same launch pads the second tiled matrix of the layer (h, contraction length K2): the part
 // of its last K-step past K2 that the producing GEMM epilogue never writes is set to zero data
 // and neutral scales (nothing to do when K2 is a multiple of 256).
-// Launch: 128 threads = 4 K-steps x 32 threads (8 elements each); grid (S + 2, ceil(nk / 4)).
-// The two workgroups past S (blockIdx.y == 0) build the layer's two work-item lists instead, which
+// Launch: 128 threads = 4 K-steps x 32 threads (8 elements each) for kQpRows rows; grid
+// (ceil(S / kQpRows) + 2, ceil(nk / 4)).
+// The two workgroups past the rows (blockIdx.y == 0) build the layer's two work-item lists instead, which
 // need only expert_offsets and so ride along in the shadow of the quantization.
+constexpr int kQpRows = 4;   // rows per workgroup
 __global__ __launch_bounds__(128) void mxfp4_quantize_permute_kernel(
     const uint16_t* __restrict__ x, const int32_t* __restrict__ sorted_slots, int topk, int S, int cols,
     uint8_t* __restrict__ tiled, uint8_t* __restrict__ tiled_scales, uint8_t* __restrict__ tiled2,
     uint8_t* __restrict__ tiled2_scales, int K2, const int32_t* __restrict__ expert_offsets, int E,
     MoeBuildItems items, int32_t* __restrict__ num_items) {
     __shared__ int scan[128];
-    if ((int)blockIdx.x >= S) {
+    const int row_blocks = (S + kQpRows - 1) / kQpRows;
+    if ((int)blockIdx.x >= row_blocks) {
         if (blockIdx.y == 0)
-            moe_build_items_block<128>(expert_offsets, E, items, (int)blockIdx.x - S, num_items, scan);
+            moe_build_items_block<128>(expert_offsets, E, items, (int)blockIdx.x - row_blocks, num_items, scan);
         return;
     }
     const int nk = (cols / 2 + 127) >> 7;
-    const int pos = blockIdx.x;
     const int kt = blockIdx.y * 4 + (threadIdx.x >> 5), c = threadIdx.x & 31;  // K-step, 4-byte column
+    const int pos0 = blockIdx.x * kQpRows;
     if (blockIdx.y == 0 && threadIdx.x < 32 && (K2 & 255)) {
         const int Kb2 = K2 >> 1, nk2 = (Kb2 + 127) >> 7;
         const int valid = Kb2 - (nk2 - 1) * 128;  // valid bytes of the last K-step, a multiple of 16
-        const size_t tile_row2 = (size_t)(nk2 - 1) * S + pos;
-        if (c * 4 >= valid) *(uint32_t*)(tiled2 + tile_row2 * 128 + c * 4) = 0u;
-        if (c < 8 && c * 16 >= valid) tiled2_scales[tile_row2 * 8 + c] = 127;
+        for (int j = 0; j < kQpRows && pos0 + j < S; ++j) {
+            const size_t tile_row2 = (size_t)(nk2 - 1) * S + pos0 + j;
+            if (c * 4 >= valid) *(uint32_t*)(tiled2 + tile_row2 * 128 + c * 4) = 0u;
+            if (c < 8 && c * 16 >= valid) tiled2_scales[tile_row2 * 8 + c] = 127;
+        }
     }
     if (kt >= nk) return;
-    const int row = sorted_slots[pos] / topk;
     const int col = kt * 256 + c * 8;
-    float v[8];
-    if (col < cols) {
-        const v4i raw = *(const v4i*)(x + (size_t)row * cols + col);
+    // the loads of the workgroup's rows are issued together: a thread's 16 bytes per row are all it has in flight
+    int row[kQpRows];
+#pragma unroll
+    for (int j = 0; j < kQpRows; ++j) row[j] = sorted_slots[min(pos0 + j, S - 1)] / topk;
+    v4i raw[kQpRows];
+#pragma unroll
+    for (int j = 0; j < kQpRows; ++j)
+        raw[j] = col < cols ? *(const v4i*)(x + (size_t)row[j] * cols + col) : v4i{0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < kQpRows; ++j) {
+        if (pos0 + j >= S) break;
+        float v[8];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            v[2 * i] = __uint_as_float((uint32_t)raw[i] << 16);
-            v[2 * i + 1] = __uint_as_float((uint32_t)raw[i] & 0xffff0000u);
+            v[2 * i] = __uint_as_float((uint32_t)raw[j][i] << 16);
+            v[2 * i + 1] = __uint_as_float((uint32_t)raw[j][i] & 0xffff0000u);
         }
-    } else {
+        float amax = 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = 0.f;
+        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+        const int e = mx_block_exponent(amax);
+        const size_t tile_row = (size_t)kt * S + pos0 + j;
+        *(uint32_t*)(tiled + tile_row * 128 + c * 4) = pack8_e2m1(v, e);
+        if ((c & 3) == 0) tiled_scales[tile_row * 8 + (c >> 2)] = (uint8_t)(e + 127);
     }
-    float amax = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
-    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-    const int e = mx_block_exponent(amax);
-    const size_t tile_row = (size_t)kt * S + pos;
-    *(uint32_t*)(tiled + tile_row * 128 + c * 4) = pack8_e2m1(v, e);
-    if ((c & 3) == 0) tiled_scales[tile_row * 8 + (c >> 2)] = (uint8_t)(e + 127);
 }
 
 // ---------------------------------------------------------------------- weight pre-shuffle
@@ -1185,7 +1195,7 @@ extern "C" int hk_moe_mxfp4_experts_ex(const void* x_bf16, const void* w13, cons
         b.bm = weight_layout ? kStBM : kMoeBM;
         b.items[0] = (MoeItem*)(ws + L.items1); b.items[1] = (MoeItem*)(ws + L.items2);
         b.n_tiles[0] = (I + 127) / 128; b.n_tiles[1] = (H + 255) / 256;
-        hipLaunchKernelGGL(mxfp4_quantize_permute_kernel, dim3(S + 2, (nk1 + 3) / 4), dim3(128), 0, s,
+        hipLaunchKernelGGL(mxfp4_quantize_permute_kernel, dim3((S + kQpRows - 1) / kQpRows + 2, (nk1 + 3) / 4), dim3(128), 0, s,
                            (const uint16_t*)x_bf16, sorted_slots, k, S, H, ws + L.xq, ws + L.xs, ws + L.hq,
                            ws + L.hs, I, expert_offsets, E, b, nitems);
     }
