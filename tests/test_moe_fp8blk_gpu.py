@@ -183,3 +183,41 @@ def test_moe_fp8blk_full_width_properties(hk):
         w13q[ut].view(torch.uint8).cpu().numpy(), w13s[ut].cpu().numpy(),
         w2q[ut].view(torch.uint8).cpu().numpy(), w2s[ut].cpu().numpy()))
     assert GM.rel_fro_error(y[sel].float().cpu().numpy(), want) <= TOL
+
+
+def _drawn_layer_shapes(seed, count):
+    """Seeded random layer shapes and routing parameters; H and I down to one 128-wide block."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        G = int(rng.choice([1, 2, 4, 8]))
+        per = int(rng.choice([1, 2, 4, 8, 16]))
+        KG = int(rng.integers(1, G + 1))
+        k = int(rng.integers(1, min(KG * per, 8) + 1))
+        T, H, I = int(rng.integers(1, 900)), int(rng.integers(1, 7)) * 128, int(rng.integers(1, 5)) * 128
+        while G * per * I * H > 6e6 and (H > 128 or I > 128):
+            H, I = max(128, H // 256 * 128), max(128, I // 256 * 128)
+        out.append((T, G * per, k, G, KG, H, I))
+    return out
+
+
+@pytest.mark.parametrize("T,E,k,G,KG,H,I", _drawn_layer_shapes(78, 10))
+def test_moe_fp8blk_forward_drawn_shapes(hk, T, E, k, G, KG, H, I):
+    print(f"moe_fp8blk drawn T={T} E={E} k={k} G={G} KG={KG} H={H} I={I}", flush=True)
+    rng = np.random.default_rng(T * 3 + E + H + I)
+    xq, xs, w13q, w13s, w2q, w2s = _case(rng, T, E, H, I)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    if (T + E) % 2:
+        logits[:, rng.choice(E, size=max(1, E // 8), replace=False)] += 3.0
+    bias = (rng.standard_normal(E) * 0.05).astype(np.float32)
+    ws = torch.empty(hk.tk_kernel.moe_fp8blk_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=DEV)
+    y = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_fp8blk(
+        _fp8(xq), torch.from_numpy(xs).to(DEV), torch.from_numpy(logits).to(DEV), torch.from_numpy(bias).to(DEV),
+        _fp8(w13q), torch.from_numpy(w13s).to(DEV), _fp8(w2q), torch.from_numpy(w2s).to(DEV), y, k, G, KG, 2.5, ws)
+    torch.cuda.synchronize()
+    got = y.float().cpu().numpy()
+    ids, w = O.topk_grouped_sigmoid(logits, bias, k, G, KG, 2.5)
+    want = F.bf16_to_f32(O.moe_fp8blk_forward(xq, xs, ids, w, w13q, w13s, w2q, w2s))
+    assert np.isfinite(got).all()
+    assert GM.rel_fro_error(got, want) <= TOL

@@ -267,3 +267,33 @@ def test_moe_mxfp4_full_shape_properties(hk):
         w2p[ut].cpu().numpy(), w2s[ut][:, :, :I // 32].cpu().numpy())[0])
     got = y[sel].float().cpu().numpy()
     assert G.rel_fro_error(got, want) <= TOL
+
+
+def _drawn_layer_shapes(seed, count):
+    """Seeded random layer shapes: few and many experts, H and I down to one MX block."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        E = int(rng.choice([1, 2, 3, 8, 33, 128]))
+        k = int(rng.integers(1, min(E, 8) + 1))
+        T, H, I = int(rng.integers(1, 700)), int(rng.integers(1, 25)) * 32, int(rng.integers(1, 17)) * 32
+        while E * I * H > 6e6:
+            H, I = max(32, H // 64 * 32), max(32, I // 64 * 32)
+        out.append((T, E, k, H, I))
+    return out
+
+
+@pytest.mark.parametrize("T,E,k,H,I", _drawn_layer_shapes(77, 10))
+def test_moe_mxfp4_forward_drawn_shapes(hk, T, E, k, H, I):
+    print(f"moe_mxfp4 drawn T={T} E={E} k={k} H={H} I={I}", flush=True)
+    rng = np.random.default_rng(T * 3 + E + H + I)
+    x = _bf16(rng.standard_normal((T, H)))
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    if (T + E) % 2:  # a few hot experts: many rows on some experts, none on others
+        logits[:, rng.choice(E, size=max(1, E // 8), replace=False)] += 3.0
+    w13p, w13s, w2p, w2s = _weights(rng, E, I, H)
+    got = _run_forward(hk, x, logits, w13p, w13s, w2p, w2s, k)
+    ids, w = O.topk_softmax(logits, k)
+    want = F.bf16_to_f32(O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s)[0])
+    assert np.isfinite(got).all()
+    assert G.rel_fro_error(got, want) <= TOL
