@@ -8,16 +8,26 @@ Protocol follows the reference's harness (kernels/gemm/bf16fp32/mi350x/test_pyth
 
   python bench.py [--gpus 1] [--steps 100] [--warmup 500] [--only-headline] [--no-cpu-baseline]
   python bench.py --traffic-calibration     (a 1 GiB copy + the headline GEMM, for counter runs)
+  python bench.py --only LEG[,LEG]          (selected legs of `extra`, for profiler runs)
 
-`roofline` is measured with HIP events on the launch stream around the timed region.
-`cpu_baseline` times the CPU counterpart (PyTorch-CPU dequantize + fp32 matmul) on the host cores.
-`extra` holds the other configurations of the path (FP8 size sweep, MXFP4 GEMM 8192^3, MXFP4 MoE at
-the GPT-OSS-like shape, FP8 block-scaled MoE at the DeepSeek-V3-like shape, routing kernels) and the
-measured power-limited MFMA ceiling for the benchmark's operand bit distribution.
+Clock settling: an MI355X that has been idle runs its first tens of milliseconds of work below the
+clock it sustains, so a short warm-up (the driver's `--warmup 5` is 2 ms of work) times the ramp, not
+the kernel. Before `--warmup` the headline launch is therefore repeated, untimed, for `--settle-ms`
+milliseconds (default 600, about what the reference's 500 warm-up launches of its own protocol take
+together with its timed ones); the count is printed as `settle_launches`. The timed region is
+unchanged: exactly `--steps` launches between two events on the launch stream.
+
+`roofline` objects: `achieved` = algorithmic flop (or bytes) per call / measured time per call (HIP
+events on the launch stream around the timed region); `peak` = the published MI355X figure; `traffic`
+= HBM-side bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs scaled by the same
+counters' reading for a plain copy (summaries under profiles/), or null where no such run exists.
+`cpu_baseline` times the CPU counterpart (PyTorch-CPU dequantize + fp32 matmul; the oracle's MoE
+forward on a stated subset) on the host cores.
 """
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -30,10 +40,22 @@ PEAK_FP8 = 5033.0     # MI355X dense FP8 MFMA peak, TFLOP/s (256 CU x 2.4 GHz x 
 PEAK_FP4 = 10066.0    # dense MXFP4
 PEAK_BF16 = 2516.5    # dense bf16
 PEAK_HBM = 8000.0     # GB/s
-# HBM-side bytes per 8192^3 launch of the headline kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter
-# runs of `bench.py --traffic-calibration`, each scaled by the same counter's reading for a 1 GiB copy
-# (factors 2.0 and 1.0): 805.8 MB read + 137.3 MB written (profiles/fp8_gemm_4wave_ring_kernel_8192.md).
+# HBM-side bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs, each scaled by the same
+# counter's reading for a 1 GiB copy (`bench.py --traffic-calibration`; factors 2.0 and 1.0). Sources:
+# profiles/fp8_gemm_4wave_ring_kernel_8192.md (805.8 MB read + 137.3 MB written).
 TRAFFIC_FP8_8192 = 943.1e6
+TRAFFIC = {}   # other legs: filled from profiles/ where a counter run exists (see _traffic)
+
+
+def _traffic(key):
+    return TRAFFIC.get(key)
+
+
+def _roofline(bound, achieved, peak, unit, kernel, traffic=None, **more):
+    out = {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+           "frac": round(achieved / peak, 4), "kernel": kernel, "traffic": traffic}
+    out.update(more)
+    return out
 
 
 def _timeit(torch, fn, warmup, iters):
@@ -49,6 +71,18 @@ def _timeit(torch, fn, warmup, iters):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / iters
     return wall, e0.elapsed_time(e1) / iters
+
+
+def _settle(torch, fn, ms):
+    """Repeat `fn` untimed until `ms` milliseconds of GPU work have been queued and finished."""
+    n = 0
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(50):
+            fn()
+        n += 50
+        torch.cuda.synchronize()
+    return n
 
 
 def _timeit_graph(torch, fn, out, iters, replays=10):
@@ -78,15 +112,24 @@ def _timeit_graph(torch, fn, out, iters, replays=10):
     return e0.elapsed_time(e1) / (iters * replays)
 
 
-def bench_fp8(torch, hk, n, warmup, iters, dev, keep=False, graph=False):
+def _np_bits(t):
+    import numpy as np
+    import torch
+    return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+# ------------------------------------------------------------------------------------- FP8 GEMM
+def bench_fp8(torch, hk, n, warmup, iters, dev, keep=False, graph=False, settle_ms=0.0):
     g = torch.Generator(device=dev).manual_seed(0)
     Aq, sa = hk.quant.quantize_fp8_per_tensor(torch.randn(n, n, device=dev, generator=g))
     Bq, sb = hk.quant.quantize_fp8_per_tensor(torch.randn(n, n, device=dev, generator=g))
     C = torch.empty(n, n, dtype=torch.bfloat16, device=dev)
-    wall, kern = _timeit(torch, lambda: hk.tk_kernel.dispatch_fp8_gemm(Aq, Bq, C, sa, sb), warmup, iters)
-    res = {"wall_ms": wall, "kernel_ms": kern, "tflops": 2.0 * n ** 3 / (kern * 1e-3) / 1e12}
+    call = lambda: hk.tk_kernel.dispatch_fp8_gemm(Aq, Bq, C, sa, sb)
+    settled = _settle(torch, call, settle_ms) if settle_ms > 0 else 0
+    wall, kern = _timeit(torch, call, warmup, iters)
+    res = {"wall_ms": wall, "kernel_ms": kern, "tflops": 2.0 * n ** 3 / (kern * 1e-3) / 1e12, "settle_launches": settled}
     if graph:
-        gms = _timeit_graph(torch, lambda: hk.tk_kernel.dispatch_fp8_gemm(Aq, Bq, C, sa, sb), C, iters)
+        gms = _timeit_graph(torch, call, C, iters)
         res["tflops_graph"] = 2.0 * n ** 3 / (gms * 1e-3) / 1e12
     if keep:
         res.update(A=Aq, B=Bq, C=C, sa=sa, sb=sb)
@@ -104,7 +147,8 @@ def bench_fp8_reference_inputs(torch, hk, n, warmup, iters, dev):
     _, kern = _timeit(torch, lambda: hk.tk_kernel.dispatch_fp8_gemm(A, B, C, 1.0, 1.0), warmup, iters)
     tf = 2.0 * n ** 3 / (kern * 1e-3) / 1e12
     return {"workload": f"fp8_gemm M=N=K={n}, uniform(-1,1) -> e4m3, unit scales", "kernel_ms": round(kern, 5),
-            "tflops": round(tf, 1), "vs_reference_3327.46": round(tf / 3327.46, 4) if n == 8192 else None}
+            "tflops": round(tf, 1), "vs_reference_3327.46": round(tf / 3327.46, 4) if n == 8192 else None,
+            "roofline": _roofline("mfma", tf, PEAK_FP8, "TFLOP/s", "fp8_gemm_4wave_ring_kernel")}
 
 
 def bench_library_baselines(torch, n, warmup, iters, dev):
@@ -133,15 +177,20 @@ def bench_library_baselines(torch, n, warmup, iters, dev):
 
 
 def bench_bf16(torch, hk, n, warmup, iters, dev):
+    from oracle import gemm as OG
+
     g = torch.Generator(device=dev).manual_seed(0)
     A = torch.randn(n, n, device=dev, generator=g).to(torch.bfloat16)
     B = torch.randn(n, n, device=dev, generator=g).to(torch.bfloat16)
     C = torch.empty(n, n, dtype=torch.bfloat16, device=dev)
     _, kern = _timeit(torch, lambda: hk.tk_kernel.dispatch_bf16_gemm(A, B, C), warmup, iters)
     tf = 2.0 * n ** 3 / (kern * 1e-3) / 1e12
+    rows = torch.arange(0, n, max(1, n // 16), device=dev)
+    rel = OG.rel_fro_error(C[rows].float().cpu().numpy(), OG.bf16_gemm(_np_bits(A[rows]), _np_bits(B)))
     # reference: 1610.5 TFLOP/s at 8192^3 on MI355X (analysis/bf16_gemm/mi350x/mi355x_bf16_gemm.json)
     return {"workload": f"bf16_gemm M=N=K={n}", "kernel_ms": round(kern, 5), "tflops": round(tf, 1),
-            "frac_of_bf16_peak": round(tf / PEAK_BF16, 4), "vs_reference_1610.5": round(tf / 1610.5, 4)}
+            "vs_reference_1610.5": round(tf / 1610.5, 4), "rel_fro_err_vs_oracle": rel,
+            "roofline": _roofline("mfma", tf, PEAK_BF16, "TFLOP/s", "bf16 256x256x64 tile kernel", _traffic("bf16_gemm"))}
 
 
 def bench_fp8_decode(torch, hk, warmup, iters, dev):
@@ -158,8 +207,9 @@ def bench_fp8_decode(torch, hk, warmup, iters, dev):
         _, split = _timeit(torch, lambda: hk.tk_kernel.dispatch_fp8_gemm(A, B, C, 1.0, 1.0, workspace=ws), warmup, iters)
         byts = M * K + N * K + 2 * M * N
         out.append({"shape": f"M={M} N=K=8192", "us_without_workspace": round(plain * 1e3, 1),
-                    "us_split_k": round(split * 1e3, 1), "GB/s": round(byts / (split * 1e-3) / 1e9, 1),
-                    "frac_of_hbm": round(byts / (split * 1e-3) / 1e9 / PEAK_HBM, 4)})
+                    "us_split_k": round(split * 1e3, 1),
+                    "roofline": _roofline("hbm", byts / (split * 1e-3) / 1e9, PEAK_HBM, "GB/s",
+                                          "fp8_gemm_small_tile_kernel<64,4,SPLIT> + splitk_reduce_kernel")})
     return out
 
 
@@ -176,23 +226,38 @@ def bench_mxfp4_decode(torch, hk, warmup, iters, dev):
         _, split = _timeit(torch, lambda: hk.tk_kernel.dispatch_mxfp4_gemm(A, SA, B, SB, C, workspace=ws), warmup, iters)
         byts = (M + N) * (K // 2 + K // 32) + 2 * M * N
         out.append({"shape": f"M={M} N={N} K={K}", "us_without_workspace": round(plain * 1e3, 1),
-                    "us_split_k": round(split * 1e3, 1), "GB/s": round(byts / (split * 1e-3) / 1e9, 1),
-                    "frac_of_hbm": round(byts / (split * 1e-3) / 1e9 / PEAK_HBM, 4)})
+                    "us_split_k": round(split * 1e3, 1),
+                    "roofline": _roofline("hbm", byts / (split * 1e-3) / 1e9, PEAK_HBM, "GB/s",
+                                          "mxfp4_gemm_small_tile_kernel<64,4,SPLIT> + splitk_reduce_kernel")})
     return out
 
 
 def bench_mxfp4(torch, hk, n, warmup, iters, dev):
+    from oracle import gemm as OG
+
     g = torch.Generator(device=dev).manual_seed(0)
     A, SA = hk.quant.quantize_mxfp4(torch.randn(n, n, device=dev, generator=g))
     B, SB = hk.quant.quantize_mxfp4(torch.randn(n, n, device=dev, generator=g))
     C = torch.empty(n, n, dtype=torch.bfloat16, device=dev)
     _, kern = _timeit(torch, lambda: hk.tk_kernel.dispatch_mxfp4_gemm(A, SA, B, SB, C), warmup, iters)
     tf = 2.0 * n ** 3 / (kern * 1e-3) / 1e12
+    # parity spot check against the oracle on a row sample (outside the timed region)
+    rows = torch.arange(0, n, max(1, n // 16), device=dev)
+    ref = OG.mxfp4_gemm(A[rows].cpu().numpy(), SA[rows].cpu().numpy(), B.cpu().numpy(), SB.cpu().numpy())
+    rel = OG.rel_fro_error(C[rows].float().cpu().numpy(), ref)
     return {"workload": f"mxfp4_gemm M=N=K={n}", "kernel_ms": round(kern, 5), "tflops": round(tf, 1),
-            "frac_of_mxfp4_peak": round(tf / PEAK_FP4, 4)}
+            "rel_fro_err_vs_oracle": rel,
+            "roofline": _roofline("mfma", tf, PEAK_FP4, "TFLOP/s", "mxfp4 256x256x256 tile kernel", _traffic("mxfp4_gemm"))}
 
 
+# ------------------------------------------------------------------------------------- MoE layers
 def bench_moe_mxfp4(torch, hk, warmup, iters, dev, graph=True):
+    import numpy as np
+
+    from oracle import formats as F
+    from oracle import gemm as OG
+    from oracle import moe as OM
+
     T, E, k, H, I = 4096, 128, 4, 2880, 2880
     g = torch.Generator(device=dev).manual_seed(0)
     x = torch.randn(T, H, device=dev, generator=g).to(torch.bfloat16)
@@ -208,18 +273,34 @@ def bench_moe_mxfp4(torch, hk, warmup, iters, dev, graph=True):
         a, s = hk.quant.quantize_mxfp4(torch.randn(H, I, device=dev, generator=g) * 0.02)
         w2p[e], w2s[e] = a, hk.quant.pad_scales(s)
     W = hk.tk_kernel.MoeMxfp4ShuffledWeights.from_plain(w13p, w13s, w2p, w2s)
-    wbytes = W.w13.numel() + W.w2.numel() + W.w13_scales.numel() + W.w2_scales.numel()
+    # the oracle's inputs for a sample of tokens: their routing and the plain weights of the experts they use
+    sel = np.arange(5, T, T // 8)[:8]
+    ids_s, w_s = OM.topk_softmax(logits[torch.from_numpy(sel).to(dev)].cpu().numpy(), k)
+    used = np.unique(ids_s)
+    ut = torch.from_numpy(used.astype(np.int64)).to(dev)
+    plain = [t[ut].cpu().numpy() for t in (w13p, w13s[:, :, :H // 32], w2p, w2s[:, :, :I // 32])]
     del w13p, w13s, w2p, w2s
     ws = torch.empty(hk.tk_kernel.moe_mxfp4_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=dev)
     y = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
-    _, kern = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_mxfp4(x, logits, W, None, None, None, y, k, ws),
-                      warmup, iters)
-    # the layer's nine launches replayed from a HIP graph (no host work or launch gaps between them)
-    kern_graph = _timeit_graph(torch, lambda: hk.tk_kernel.dispatch_moe_mxfp4(x, logits, W, None, None, None, y, k, ws),
-                               y, iters) if graph else None
+    call = lambda: hk.tk_kernel.dispatch_moe_mxfp4(x, logits, W, None, None, None, y, k, ws)
+    _, kern = _timeit(torch, call, warmup, iters)
+    # parity spot check (outside the timed region)
+    remap = {int(e): i for i, e in enumerate(used)}
+    ids_l = np.vectorize(remap.get)(ids_s).astype(np.int32)
+    st = torch.from_numpy(sel).to(dev)
+    want, _ = OM.moe_mxfp4_forward(F.bf16_to_f32(_np_bits(x[st])), ids_l, w_s, *plain)
+    got = y[st].float().cpu().numpy()
+    rel = OG.rel_fro_error(got, F.bf16_to_f32(want))
+    assert float(np.abs(got).max()) > 0.0 and np.isfinite(got).all(), "MoE output sample is empty or not finite"
+    # (the FP4 x FP4 products and their fp32 sums are exact for these magnitudes whatever the order of summation,
+    # so a relative error of exactly 0 against the oracle is the expected reading here, not an empty comparison)
+    # the layer's launches replayed from a HIP graph (no host work or launch gaps between them)
+    kern_graph = _timeit_graph(torch, call, y, iters) if graph else None
     flop = 2.0 * T * k * (H * 2 * I + I * H)
     tf = flop / (kern * 1e-3) / 1e12
-    compulsory = wbytes + 2 * T * H * 2  # weights once + x in + y out
+    # algorithmic bytes: every expert's weights and scales once (unpadded: 4-bit elements + one e8m0 byte
+    # per 32), x in, y out (the pre-shuffled tensors pad K 2880 -> 3072 with zeros that are never fetched)
+    compulsory = E * 3 * I * H * (0.5 + 1.0 / 32) + 2 * T * H * 2
     # the same layer with the GPT-OSS expert epilogues: biases and clamped SwiGLU (the row order of
     # the source weights was resolved by the pre-shuffle, so the same shuffled weights serve)
     b13 = torch.randn(E, 2 * I, device=dev, generator=g)
@@ -229,8 +310,10 @@ def bench_moe_mxfp4(torch, hk, warmup, iters, dev, graph=True):
     return {"workload": "moe_mxfp4 T=4096 H=2880 I=2880 E=128 top-4 softmax, MXFP4 activations and weights "
                         "(routing + sort + quantize/permute + 2 grouped GEMMs + un-permute)",
             "ms": round(kern, 5), "tflops": round(tf, 1), "frac_of_mxfp4_peak": round(tf / PEAK_FP4, 4),
-            "compulsory_GB": round(compulsory / 1e9, 3),
-            "frac_of_hbm_roofline": round(compulsory / (kern * 1e-3) / 1e9 / PEAK_HBM, 4),
+            "compulsory_GB": round(compulsory / 1e9, 3), "rel_fro_err_vs_oracle_8_tokens": rel,
+            "roofline": _roofline("hbm", compulsory / (kern * 1e-3) / 1e9, PEAK_HBM, "GB/s",
+                                  "whole layer (5 launches); dominant: moe_mxfp4 gate+up grouped GEMM",
+                                  _traffic("moe_mxfp4")),
             "ms_graph_replay": round(kern_graph, 5) if graph else None, "ms_with_biases_and_clamped_swiglu": round(kern_oai, 5)}
 
 
@@ -239,8 +322,6 @@ def cpu_baseline_moe_mxfp4(torch, hk, dev):
     sample of the workload: 8 of the 128 experts and 256 of the 4096 tokens at the full H = I = 2880,
     top-4 routing, i.e. the same 128 rows per expert. Weights are quantized on the GPU beforehand;
     only the oracle's forward pass is timed."""
-    import os
-
     import numpy as np
 
     from oracle import formats as F
@@ -254,7 +335,7 @@ def cpu_baseline_moe_mxfp4(torch, hk, dev):
     q2 = [hk.quant.quantize_mxfp4(torch.randn(H, I, device=dev, generator=g) * 0.02) for _ in range(E)]
     w13p = np.stack([a.cpu().numpy() for a, _ in q13]); w13s = np.stack([b.cpu().numpy() for _, b in q13])
     w2p = np.stack([a.cpu().numpy() for a, _ in q2]); w2s = np.stack([b.cpu().numpy() for _, b in q2])
-    xf = F.bf16_to_f32(x.view(torch.int16).cpu().numpy().view(np.uint16))
+    xf = F.bf16_to_f32(_np_bits(x))
     ids, w = OM.topk_softmax(logits, k)
     best = float("inf")
     for _ in range(2):
@@ -267,6 +348,12 @@ def cpu_baseline_moe_mxfp4(torch, hk, dev):
 
 
 def bench_moe_fp8blk(torch, hk, warmup, iters, dev):
+    import numpy as np
+
+    from oracle import formats as F
+    from oracle import gemm as OG
+    from oracle import moe as OM
+
     T, E, k, H, I, G, KG = 8192, 256, 8, 7168, 2048, 8, 4
     g = torch.Generator(device=dev).manual_seed(0)
     xq, xs = hk.quant.quantize_fp8_blocks(torch.randn(T, H, device=dev, generator=g), 1, 128)
@@ -282,16 +369,62 @@ def bench_moe_fp8blk(torch, hk, warmup, iters, dev):
     y = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
     _, kern = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_fp8blk(xq, xs, logits, None, w13q, w13s, w2q, w2s, y,
                                                                       k, G, KG, 1.0, ws), warmup, iters)
+    # parity spot check on four tokens (outside the timed region)
+    sel = np.array([3, 2731, 5461, T - 1])
+    st = torch.from_numpy(sel).to(dev)
+    ids_s, w_s = OM.topk_grouped_sigmoid(logits[st].cpu().numpy(), None, k, G, KG, 1.0)
+    used = np.unique(ids_s)
+    remap = {int(e): i for i, e in enumerate(used)}
+    ids_l = np.vectorize(remap.get)(ids_s).astype(np.int32)
+    ut = torch.from_numpy(used.astype(np.int64)).to(dev)
+    want = F.bf16_to_f32(OM.moe_fp8blk_forward(
+        xq[st].view(torch.uint8).cpu().numpy(), xs[st].cpu().numpy(), ids_l, w_s,
+        w13q[ut].view(torch.uint8).cpu().numpy(), w13s[ut].cpu().numpy(),
+        w2q[ut].view(torch.uint8).cpu().numpy(), w2s[ut].cpu().numpy()))
+    rel = OG.rel_fro_error(y[st].float().cpu().numpy(), want)
     flop = 2.0 * T * k * (H * 2 * I + I * H)
     tf = flop / (kern * 1e-3) / 1e12
-    compulsory = w13q.numel() + w2q.numel() + T * H + T * H * 2
+    # algorithmic bytes: weights and their scales once, x (e4m3 + scales) in, y out
+    compulsory = w13q.numel() + w2q.numel() + 4 * (w13s.numel() + w2s.numel()) + T * H + 4 * xs.numel() + T * H * 2
     return {"workload": "moe_fp8blk T=8192 H=7168 I=2048 E=256 top-8 sigmoid (8 groups / top-4), e4m3 with "
                         "1x128 / 128x128 fp32 scales",
             "ms": round(kern, 5), "tflops": round(tf, 1), "frac_of_fp8_peak": round(tf / PEAK_FP8, 4),
-            "compulsory_GB": round(compulsory / 1e9, 3),
-            "frac_of_hbm_roofline": round(compulsory / (kern * 1e-3) / 1e9 / PEAK_HBM, 4)}
+            "compulsory_GB": round(compulsory / 1e9, 3), "rel_fro_err_vs_oracle_4_tokens": rel,
+            "roofline": _roofline("hbm", compulsory / (kern * 1e-3) / 1e9, PEAK_HBM, "GB/s",
+                                  "whole layer (7 launches); dominant: moe_fp8blk gate+up grouped GEMM",
+                                  _traffic("moe_fp8blk"),
+                                  note="MFMA time at peak 1.15 ms vs 1.43 ms for the bytes: HBM is the binding roofline")}
 
 
+def cpu_baseline_moe_fp8blk(torch, hk, dev):
+    """The CPU oracle's FP8 block-scaled MoE forward on a 1/32 sample of the DeepSeek-V3-like workload:
+    8 of the 256 experts and 256 of the 8192 tokens at the full H = 7168, I = 2048, every token routed
+    to all 8 experts (top-8), i.e. the workload's 256 rows per expert. Only the forward pass is timed."""
+    import numpy as np
+
+    from oracle import moe as OM
+
+    T, E, k, H, I = 256, 8, 8, 7168, 2048
+    g = torch.Generator(device=dev).manual_seed(2)
+    xq, xs = hk.quant.quantize_fp8_blocks(torch.randn(T, H, device=dev, generator=g), 1, 128)
+    q13 = [hk.quant.quantize_fp8_blocks(torch.randn(2 * I, H, device=dev, generator=g) * 0.02, 128, 128) for _ in range(E)]
+    q2 = [hk.quant.quantize_fp8_blocks(torch.randn(H, I, device=dev, generator=g) * 0.02, 128, 128) for _ in range(E)]
+    w13q = np.stack([a.view(torch.uint8).cpu().numpy() for a, _ in q13]); w13s = np.stack([b.cpu().numpy() for _, b in q13])
+    w2q = np.stack([a.view(torch.uint8).cpu().numpy() for a, _ in q2]); w2s = np.stack([b.cpu().numpy() for _, b in q2])
+    logits = torch.randn(T, E, device=dev, generator=g).cpu().numpy()
+    ids, w = OM.topk_grouped_sigmoid(logits, None, k, 1, 1, 1.0)
+    xqn, xsn = xq.view(torch.uint8).cpu().numpy(), xs.cpu().numpy()
+    best = float("inf")
+    for _ in range(2):
+        t0 = time.perf_counter()
+        OM.moe_fp8blk_forward(xqn, xsn, ids, w, w13q, w13s, w2q, w2s)
+        best = min(best, time.perf_counter() - t0)
+    flop = 2.0 * T * k * (H * 2 * I + I * H)
+    return {"value": round(flop / best / 1e12, 4), "unit": "TFLOP/s", "cores": os.cpu_count() or 1, "kind": "port",
+            "sample": f"oracle MoE forward on 8 of 256 experts x 256 of 8192 tokens (256 rows per expert), best of 2: {best:.2f} s"}
+
+
+# ------------------------------------------------------------------------------------- routing
 def bench_routing(torch, hk, warmup, iters, dev):
     out = []
     g = torch.Generator(device=dev).manual_seed(0)
@@ -301,10 +434,9 @@ def bench_routing(torch, hk, warmup, iters, dev):
     w = torch.empty((T, k), dtype=torch.float32, device=dev)
     _, ms = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_topk_softmax(logits, ids, w), warmup, iters)
     by = T * E * 4 + T * k * 8
-    out.append({"kernel": "topk_softmax T=262144 E=128 k=4", "ms": round(ms, 5), "GB/s": round(by / ms / 1e6, 1),
-                "frac_of_hbm": round(by / ms / 1e6 / PEAK_HBM, 4)})
-    # the DeepSeek-V3 router: sigmoid scores + selection bias, 8 groups / top-4 groups, top-8. The fixed,
-    # bit-reproducible fp32 sigmoid (an exact division per expert) makes this kernel VALU bound
+    out.append({"kernel": "topk_softmax T=262144 E=128 k=4", "ms": round(ms, 5),
+                "roofline": _roofline("hbm", by / ms / 1e6, PEAK_HBM, "GB/s", "moe_topk_softmax_kernel<16>")})
+    # the DeepSeek-V3 router: sigmoid scores + selection bias, 8 groups / top-4 groups, top-8
     Tg, Eg, kg = 65536, 256, 8
     lg = torch.randn(Tg, Eg, device=dev, generator=g)
     bg = torch.randn(Eg, device=dev, generator=g) * 0.05
@@ -314,16 +446,16 @@ def bench_routing(torch, hk, warmup, iters, dev):
                     warmup, iters)
     by = Tg * Eg * 4 + Tg * kg * 8
     out.append({"kernel": "topk_grouped_sigmoid T=65536 E=256 k=8 (8 groups / top-4)", "ms": round(ms, 5),
-                "GB/s": round(by / ms / 1e6, 1), "frac_of_hbm": round(by / ms / 1e6 / PEAK_HBM, 4)})
+                "roofline": _roofline("hbm", by / ms / 1e6, PEAK_HBM, "GB/s", "moe_topk_grouped_sigmoid16_kernel<16>")})
     del lg, idg, wg
     ss = torch.empty(T * k, dtype=torch.int32, device=dev)
     off = torch.empty(E + 1, dtype=torch.int32, device=dev)
     inv = torch.empty(T * k, dtype=torch.int32, device=dev)
     wsb = torch.empty(hk.tk_kernel.moe_sort_workspace_bytes(T, k, E), dtype=torch.uint8, device=dev)
     _, ms = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_sort(ids, ss, off, inv, wsb), warmup, iters)
-    by = T * k * 4 * 2 + (2 * T * k + E + 1) * 4  # ids read by count and scatter; two outputs
-    out.append({"kernel": "moe_sort T*k=1048576 E=128", "ms": round(ms, 5), "GB/s": round(by / ms / 1e6, 1),
-                "frac_of_hbm": round(by / ms / 1e6 / PEAK_HBM, 4)})
+    by = T * k * 4 + (2 * T * k + E + 1) * 4  # ids in; sorted_slots, slot_to_pos and offsets out
+    out.append({"kernel": "moe_sort T*k=1048576 E=128", "ms": round(ms, 5),
+                "roofline": _roofline("hbm", by / ms / 1e6, PEAK_HBM, "GB/s", "moe_sort (count, scan, scatter)")})
     T2, k2, H = 8192, 8, 7168
     o = torch.randn(T2 * k2, H, device=dev, generator=g).to(torch.bfloat16)
     w2 = torch.rand(T2, k2, device=dev, generator=g)
@@ -331,27 +463,36 @@ def bench_routing(torch, hk, warmup, iters, dev):
     y = torch.empty(T2, H, dtype=torch.bfloat16, device=dev)
     _, ms = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_unpermute(o, w2, inv2, y), warmup, iters)
     by = T2 * k2 * H * 2 + T2 * H * 2
-    out.append({"kernel": "moe_unpermute T=8192 k=8 H=7168", "ms": round(ms, 5), "GB/s": round(by / ms / 1e6, 1),
-                "frac_of_hbm": round(by / ms / 1e6 / PEAK_HBM, 4)})
+    out.append({"kernel": "moe_unpermute T=8192 k=8 H=7168", "ms": round(ms, 5),
+                "roofline": _roofline("hbm", by / ms / 1e6, PEAK_HBM, "GB/s", "moe_unpermute_kernel")})
     return out
 
 
-def mfma_ceiling(torch, hk, Aq, dev):
-    """Register-only FP8 MFMA loop on operand bits drawn from the benchmark's own A matrix."""
-    import ctypes
-
-    lib = hk.load_library()
+def mfma_ceiling(torch, Aq, dev):
+    """Register-only FP8 MFMA loop on operand bits drawn from the benchmark's own A matrix (bench-only
+    library libhk355_bench.so, built with the product library but not part of it)."""
+    path = os.path.join(ROOT, "hipkittens_amd", "libhk355_bench.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    lib.hkbench_mfma_rate.restype = ctypes.c_int
+    lib.hkbench_mfma_rate.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                      ctypes.c_void_p]
     pattern = Aq.view(torch.uint8).flatten()[:65536].contiguous().view(torch.int32)
     blocks, iters = 1024, 2000
     sink = torch.empty(blocks * 512, dtype=torch.float32, device=dev)
     st = torch.cuda.current_stream().cuda_stream
 
     def run():
-        rc = lib.hk_probe_mfma_rate(pattern.data_ptr(), sink.data_ptr(), blocks, iters, 0, ctypes.c_void_p(st))
+        rc = lib.hkbench_mfma_rate(pattern.data_ptr(), sink.data_ptr(), blocks, iters, 0, ctypes.c_void_p(st))
         assert rc == 0
 
     _, ms = _timeit(torch, run, 2, 5)
     return blocks * 8 * iters * 32 * 65536.0 / (ms * 1e-3) / 1e12
+
+
+LEGS = ("ceiling", "sweep", "reference_inputs", "decode", "bf16", "library", "mxfp4", "mxfp4_decode", "moe_mxfp4",
+        "moe_fp8blk", "routing")
 
 
 def main() -> int:
@@ -360,7 +501,10 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--size", type=int, default=8192)
+    ap.add_argument("--settle-ms", type=float, default=600.0,
+                    help="untimed repetitions of the headline launch before --warmup, until this many ms have passed")
     ap.add_argument("--only-headline", action="store_true")
+    ap.add_argument("--only", type=str, default="", help="comma-separated legs of `extra` to run: " + ",".join(LEGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--traffic-calibration", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph timings (for runs under a profiler)")
@@ -380,6 +524,13 @@ def main() -> int:
     hk.load_library()  # raises if libhk355.so has not been built
     dev = torch.device("cuda:0")
     n = args.size
+    legs = set(LEGS) if not args.only else set(args.only.split(","))
+    if args.only_headline:
+        legs = set()
+    unknown = legs - set(LEGS)
+    if unknown:
+        print(f"bench.py: unknown legs {sorted(unknown)}", file=sys.stderr)
+        return 2
 
     if args.traffic_calibration:
         # For the HBM-traffic counters: a plain copy of known size (1 GiB read + 1 GiB written per
@@ -395,7 +546,7 @@ def main() -> int:
                                                   "copy_launches": 5, "gemm_launches": 10, "n": n}}))
         return 0
 
-    head = bench_fp8(torch, hk, n, args.warmup, args.steps, dev, keep=True)
+    head = bench_fp8(torch, hk, n, args.warmup, args.steps, dev, keep=True, settle_ms=args.settle_ms)
     tflops = 2.0 * n ** 3 / (head["wall_ms"] * 1e-3) / 1e12
 
     # parity spot check against the oracle on a row sample (outside the timed region)
@@ -407,9 +558,14 @@ def main() -> int:
     rel = OG.rel_fro_error(head["C"][rows].float().cpu().numpy(), ref)
 
     extra = {}
-    if not args.only_headline:
-        quick_w, quick_i = 20, 20
-        extra["mfma_fp8_ceiling_tflops_for_this_data"] = round(mfma_ceiling(torch, hk, head["A"], dev), 1)
+    ceiling = None
+    quick_w, quick_i = 50, 100
+    if "ceiling" in legs:
+        ceiling = mfma_ceiling(torch, head["A"], dev)
+        extra["mfma_fp8_ceiling_tflops_for_this_data"] = round(ceiling, 1) if ceiling else None
+    del head["A"], head["B"], head["C"]
+    torch.cuda.empty_cache()
+    if "sweep" in legs:
         sweep = {m: bench_fp8(torch, hk, m, 500, 100, dev, graph=m <= 4096 and not args.no_graph)  # the reference's protocol
                  for m in (1024, 2048, 4096, 16384)}
         # per call through the Python boundary (about 9 us of host time per call bounds the small sizes) ...
@@ -418,23 +574,33 @@ def main() -> int:
         extra["fp8_gemm_sweep_tflops_graph_replay"] = {
             str(m): round(r["tflops_graph"], 1) for m, r in sweep.items() if "tflops_graph" in r}
         del sweep
-        del head["A"], head["B"], head["C"]
         torch.cuda.empty_cache()
-        extra["fp8_gemm_reference_inputs"] = bench_fp8_reference_inputs(torch, hk, n, 100, 100, dev)
+    if "reference_inputs" in legs:
+        extra["fp8_gemm_reference_inputs"] = bench_fp8_reference_inputs(torch, hk, n, 500, 100, dev)
+    if "decode" in legs:
         extra["fp8_gemm_decode"] = bench_fp8_decode(torch, hk, 50, 50, dev)
+    if "bf16" in legs:
         extra["bf16_gemm"] = bench_bf16(torch, hk, 8192, 500, 100, dev)
+    if "library" in legs:
         extra["library_on_this_box_8192"] = bench_library_baselines(torch, 8192, 500, 100, dev)
         torch.cuda.empty_cache()
+    if "mxfp4" in legs:
         extra["mxfp4_gemm"] = bench_mxfp4(torch, hk, 8192, 500, 100, dev)
+    if "mxfp4_decode" in legs:
         extra["mxfp4_gemm_decode"] = bench_mxfp4_decode(torch, hk, 50, 50, dev)
+    if "moe_mxfp4" in legs:
         extra["moe_mxfp4"] = bench_moe_mxfp4(torch, hk, quick_w, quick_i, dev, graph=not args.no_graph)
         torch.cuda.empty_cache()
-        extra["moe_fp8blk"] = bench_moe_fp8blk(torch, hk, 5, 10, dev)
+        if not args.no_cpu_baseline:
+            extra["moe_mxfp4"]["cpu_baseline"] = cpu_baseline_moe_mxfp4(torch, hk, dev)
+    if "moe_fp8blk" in legs:
+        extra["moe_fp8blk"] = bench_moe_fp8blk(torch, hk, 10, 20, dev)
         torch.cuda.empty_cache()
+        if not args.no_cpu_baseline:
+            extra["moe_fp8blk"]["cpu_baseline"] = cpu_baseline_moe_fp8blk(torch, hk, dev)
+    if "routing" in legs:
         extra["routing"] = bench_routing(torch, hk, quick_w, quick_i, dev)
 
-    if not args.no_cpu_baseline and not args.only_headline:
-        extra["moe_mxfp4"]["cpu_baseline"] = cpu_baseline_moe_mxfp4(torch, hk, dev)
     cpu = None
     if not args.no_cpu_baseline:
         r = OG.cpu_baseline_fp8_gemm(n, n, n, seed=0, repeats=12)
@@ -448,6 +614,7 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_launches": head["settle_launches"],
         "ms_per_step": round(head["wall_ms"], 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -457,10 +624,12 @@ def main() -> int:
         "config": {"workload": f"fp8_gemm M=N=K={n}, A row-major, B [N,K], per-tensor fp32 scales, randn inputs"},
         "pct_of_fp8_peak": round(100.0 * tflops / PEAK_FP8, 2),
         "rel_fro_err_vs_oracle": rel,
-        "roofline": {"bound": "mfma", "achieved": round(head["tflops"], 2), "peak": PEAK_FP8, "unit": "TFLOP/s",
-                     "frac": round(head["tflops"] / PEAK_FP8, 4),
-                     "traffic": TRAFFIC_FP8_8192 if n == 8192 else None,
-                     "kernel_ms": round(head["kernel_ms"], 5)},
+        "roofline": _roofline("mfma", head["tflops"], PEAK_FP8, "TFLOP/s", "fp8_gemm_4wave_ring_kernel",
+                              TRAFFIC_FP8_8192 if n == 8192 else None, kernel_ms=round(head["kernel_ms"], 5),
+                              # the register-only MFMA loop on the same operand bits: what the power limit
+                              # leaves of the nominal peak on this data
+                              measured_mfma_ceiling=round(ceiling, 1) if ceiling else None,
+                              frac_of_measured_ceiling=round(head["tflops"] / ceiling, 4) if ceiling else None),
         "cpu_baseline": cpu,
         "extra": extra,
     }

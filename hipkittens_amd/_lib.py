@@ -63,7 +63,6 @@ SIGNATURES = {
     "hk_moe_fp8blk_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p,
                                       c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                       c_void_p, c_size_t, c_void_p]),
-    "hk_probe_mfma_rate": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
 }
 
 

@@ -17,6 +17,9 @@ PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 BUILD_DIR = PKG_DIR / "csrc" / "build"
 LIB_PATH = PKG_DIR / "libhk355.so"
+# bench-only tooling (csrc/bench/*.hip: a register-only MFMA rate probe). A library of its own so that
+# nothing of it is exported by, or linked into, the product library; only bench.py loads it.
+BENCH_LIB_PATH = PKG_DIR / "libhk355_bench.so"
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -45,7 +48,7 @@ def _hipcc() -> str:
 
 
 def _compile_one(src: Path, extra: list[str]) -> Path:
-    obj = BUILD_DIR / (src.stem + ".o")
+    obj = BUILD_DIR / (("bench_" if src.parent.name == "bench" else "") + src.stem + ".o")
     cmd = [_hipcc(), *HIPCC_FLAGS, *PER_FILE_FLAGS.get(src.name, []), *extra, "-c", str(src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
@@ -60,17 +63,25 @@ def build(verbose: bool = True, extra_flags: list[str] | None = None, jobs: int 
     sources = sorted(CSRC.glob("*.hip"))
     if not sources:
         raise RuntimeError(f"no .hip sources under {CSRC}")
+    bench_sources = sorted((CSRC / "bench").glob("*.hip"))
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(lambda s: _compile_one(s, extra), sources))
-    tmp = LIB_PATH.with_suffix(".so.tmp")
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
-    os.replace(tmp, LIB_PATH)
+        all_objs = list(pool.map(lambda s: _compile_one(s, extra), sources + bench_sources))
+    objs, bench_objs = all_objs[:len(sources)], all_objs[len(sources):]
+    _link(objs, LIB_PATH)
+    if bench_objs:
+        _link(bench_objs, BENCH_LIB_PATH)
     if verbose:
         print(f"built {LIB_PATH} from {len(sources)} sources", file=sys.stderr)
     return LIB_PATH
+
+
+def _link(objs: list[Path], out: Path) -> None:
+    tmp = out.with_suffix(".so.tmp")
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link of {out.name} failed:\n{res.stdout}\n{res.stderr}")
+    os.replace(tmp, out)
 
 
 if __name__ == "__main__":

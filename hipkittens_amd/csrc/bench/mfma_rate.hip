@@ -1,9 +1,9 @@
-// Calibration probe: sustained MFMA rate of this GPU from a register-only loop (no memory
-// traffic), for a chosen operand bit pattern. On MI355X the matrix pipes are power limited, so the
+// Bench-only calibration probe, built into libhk355_bench.so (not part of libhk355.so or of its
+// C ABI; only bench.py loads it): sustained MFMA rate of this GPU from a register-only loop (no
+// memory traffic), for a chosen operand bit pattern. On MI355X the matrix pipes are power limited, so the
 // rate a GEMM can reach depends on how many operand bits toggle; this probe measures that ceiling
 // for the data a benchmark actually uses. No counterpart in the reference.
-#include "hk_device.h"
-#include "../../include/hk355.h"
+#include "../hk_device.h"
 
 namespace hk {
 
@@ -45,15 +45,15 @@ __global__ __launch_bounds__(512) void mfma_rate_kernel(const int* __restrict__ 
 // distribution); sink: >= blocks*512 device floats. Launches `blocks` workgroups of 8 waves running
 // `iters` x 32 MFMAs (16x16x128, fp8 if fp4 == 0 else fp4) per wave. The caller times it;
 // flops = blocks * 8 * iters * 32 * 65536.
-extern "C" int hk_probe_mfma_rate(const void* pattern, void* sink, int blocks, int iters, int fp4, void* stream) {
+extern "C" int hkbench_mfma_rate(const void* pattern, void* sink, int blocks, int iters, int fp4, void* stream) {
     using namespace hk;
-    if (!pattern || !sink) return HK_ERR_NULL_POINTER;
-    if (blocks <= 0 || iters <= 0) return HK_ERR_BAD_SHAPE;
+    if (!pattern || !sink) return -1;
+    if (blocks <= 0 || iters <= 0) return -2;
     if (fp4)
         hipLaunchKernelGGL(mfma_rate_kernel<1>, dim3(blocks), dim3(512), 0, (hipStream_t)stream, (const int*)pattern,
                            (float*)sink, iters);
     else
         hipLaunchKernelGGL(mfma_rate_kernel<0>, dim3(blocks), dim3(512), 0, (hipStream_t)stream, (const int*)pattern,
                            (float*)sink, iters);
-    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+    return hipGetLastError() == hipSuccess ? 0 : -5;
 }

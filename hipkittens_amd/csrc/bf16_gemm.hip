@@ -278,13 +278,8 @@ template <int TILE, int STAGES, bool EDGE>
 static int launch_bf16_small_tile(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream) {
     auto kern = bf16_gemm_small_tile_kernel<TILE, STAGES, EDGE, false>;
     constexpr int lds_bytes = STAGES * 2 * TILE * BK;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) !=
-            hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, lds_bytes, configured)) return HK_ERR_LAUNCH;
     const int tiles_m = (M + TILE - 1) / TILE, tiles_n = (N + TILE - 1) / TILE;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream, (const uint8_t*)A,
                        (const uint8_t*)B, (uint16_t*)C, M, N, 2 * K, 1.0f, tiles_m, tiles_n, 0, (float*)nullptr);
@@ -294,7 +289,7 @@ static int launch_bf16_small_tile(const void* A, const void* B, void* C, int M, 
 template <bool EDGE>
 static int launch_bf16_splitk(const void* A, const void* B, void* C, int M, int N, int K, int splits, float* partial,
                               hipStream_t stream) {
-    static bool configured = false;
+    static DeviceOnce configured;
     return launch_small_tile_splitk(bf16_gemm_small_tile_kernel<kTinyTile, kTinyStages, EDGE, true>, configured, A,
                                     B, C, M, N, 2 * K, 1.0f, splits, partial, stream);
 }
@@ -303,13 +298,8 @@ template <bool EDGE>
 static int launch_bf16_ring(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream) {
     auto kern = bf16_gemm_4wave_ring_kernel<EDGE>;
     constexpr int lds_bytes = 5 * kTileBytes;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) !=
-            hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, lds_bytes, configured)) return HK_ERR_LAUNCH;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream, (const uint8_t*)A,
                        (const uint8_t*)B, (uint16_t*)C, M, N, K, 1.0f, tiles_m, tiles_n,

@@ -543,13 +543,8 @@ template <int WM, int WN, bool EDGE>
 static int launch_tile(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                        hipStream_t stream) {
     auto kern = fp8_gemm_tile_kernel<WM, WN, EDGE>;
-    static bool configured = false;  // attribute is per function; set once per process
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kLdsBytes) != hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, kLdsBytes, configured)) return HK_ERR_LAUNCH;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(WM * WN * 64), kLdsBytes, stream,
                        (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
@@ -562,13 +557,8 @@ static int launch_small_tile(const void* A, const void* B, void* C, int M, int N
                              hipStream_t stream) {
     auto kern = fp8_gemm_small_tile_kernel<TILE, STAGES, EDGE, false>;
     constexpr int lds_bytes = STAGES * 2 * TILE * BK;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                lds_bytes) != hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, lds_bytes, configured)) return HK_ERR_LAUNCH;
     const int tiles_m = (M + TILE - 1) / TILE, tiles_n = (N + TILE - 1) / TILE;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream,
                        (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
@@ -579,7 +569,7 @@ static int launch_small_tile(const void* A, const void* B, void* C, int M, int N
 template <bool EDGE>
 static int launch_tile128_splitk(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                                  int splits, float* partial, hipStream_t stream) {
-    static bool configured = false;
+    static DeviceOnce configured;
     return launch_small_tile_splitk(fp8_gemm_small_tile_kernel<kTinyTile, kTinyStages, EDGE, true>, configured, A,
                                     B, C, M, N, K, alpha, splits, partial, stream);
 }
@@ -589,13 +579,8 @@ static int launch_4wave(const void* A, const void* B, void* C, int M, int N, int
                         hipStream_t stream) {
     auto kern = RING ? fp8_gemm_4wave_ring_kernel<EDGE> : fp8_gemm_4wave_kernel<EDGE>;
     constexpr int lds_bytes = RING ? 5 * kTileBytes : kLdsBytes;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                lds_bytes) != hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, lds_bytes, configured)) return HK_ERR_LAUNCH;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream,
                        (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,

@@ -2,6 +2,7 @@
 // row in both; only the MFMA differs).
 #pragma once
 #include "gemm_tile.h"
+#include "hk_host.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -253,15 +254,10 @@ static inline int splitk_ranges(int M, int N, int K, int min_nk = 48) {
 // Launches `kern` (a small-tile kernel instantiated with SPLIT over 64x64 tiles) on `splits` K ranges
 // and the reduction behind it. K in bytes.
 template <typename Kern>
-static inline int launch_small_tile_splitk(Kern kern, bool& configured, const void* A, const void* B, void* C, int M,
+static inline int launch_small_tile_splitk(Kern kern, DeviceOnce& configured, const void* A, const void* B, void* C, int M,
                                            int N, int K, float alpha, int splits, float* partial,
                                            hipStream_t stream) {
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kTinyLdsBytes) != hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
+    if (!set_lds_limit_once((const void*)kern, kTinyLdsBytes, configured)) return HK_ERR_LAUNCH;
     const int tiles_m = (M + kTinyTile - 1) / kTinyTile, tiles_n = (N + kTinyTile - 1) / kTinyTile;
     const int nk = (K + BK - 1) / BK;
     const int kps = (nk + splits - 1) / splits;

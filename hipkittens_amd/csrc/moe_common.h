@@ -2,6 +2,7 @@
 // weight rows to LDS rows of the B tile, and host helpers implemented in moe_mxfp4.hip.
 #pragma once
 #include "gemm_tile.h"
+#include "hk_host.h"
 
 namespace hk {
 
@@ -26,7 +27,7 @@ constexpr int kMoeBM = 128;
 struct MoeItem { int expert, row_start, rows, n_tile; };
 
 inline int moe_round_up(int x, int m) { return (x + m - 1) / m * m; }
-// Number of CUs of the current device (cached).
+// Number of CUs of the current device (cached per device ordinal).
 int moe_num_compute_units();
 // Item lists of the two grouped GEMMs of a layer from expert_offsets [E+1], m-tiles of up to `bm`
 // rows: items1 / num_items[0] for n_tiles_n1 tiles of weight rows, items2 / num_items[1] for

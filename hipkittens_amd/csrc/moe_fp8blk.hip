@@ -392,12 +392,8 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
 template <int MODE, bool GATHER>
 static int launch_fp8blk_gemm(const MoeFp8Params& p, int max_items, hipStream_t s) {
     auto kern = moe_fp8blk_gemm_kernel<MODE, GATHER>;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kF8Lds) != hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, kF8Lds, configured)) return HK_ERR_LAUNCH;
     const int grid = min(max_items, moe_num_compute_units());
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kF8Lds, s, p);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;

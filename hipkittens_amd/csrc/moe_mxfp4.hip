@@ -1006,13 +1006,12 @@ __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __re
 }
 
 int moe_num_compute_units() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256;
-        cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-    }
+    static std::atomic<int> cached[64];   // per device ordinal; 0 = not queried yet
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (dev >= 0 && dev < 64 && (cus = cached[dev].load(std::memory_order_relaxed)) > 0) return cus;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 256;
+    if (dev >= 0 && dev < 64) cached[dev].store(cus, std::memory_order_relaxed);
     return cus;
 }
 
@@ -1029,13 +1028,8 @@ void moe_launch_build_items(const int32_t* expert_offsets, int E, int bm, int n_
 template <int MODE, bool EXT>
 static int launch_moe_stream(MoeGemmParams p, int max_items, hipStream_t s) {
     auto kern = moe_mxfp4_stream_kernel<MODE, EXT>;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kStLds) !=
-            hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, kStLds, configured)) return HK_ERR_LAUNCH;
     // persistent: one workgroup per CU, each walking its share of the item list
     const int grid = min(max_items, moe_num_compute_units());
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kStLds, s, p);
@@ -1045,13 +1039,8 @@ static int launch_moe_stream(MoeGemmParams p, int max_items, hipStream_t s) {
 template <int MODE, bool EXT>
 static int launch_moe_gemm(MoeGemmParams p, int max_items, hipStream_t s) {
     auto kern = moe_mxfp4_gemm_kernel<MODE, EXT>;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kMoeLds) !=
-            hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, kMoeLds, configured)) return HK_ERR_LAUNCH;
     // persistent: one workgroup per CU, each walking its share of the item list
     const int grid = min(max_items, moe_num_compute_units());
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kMoeLds, s, p);

@@ -310,7 +310,10 @@ __global__ __launch_bounds__(256) void moe_sort_count_kernel(const int32_t* __re
 #pragma unroll
     for (int i = 0; i < kSortChunk / 256; ++i) {
         const int sidx = base + i * 256 + threadIdx.x;
-        if (sidx < S) atomicAdd(&cnt[ids[sidx]], 1);
+        if (sidx < S) {
+            const int e = ids[sidx];
+            if ((unsigned)e < (unsigned)E) atomicAdd(&cnt[e], 1);   // ids outside [0, E) take no part
+        }
     }
     __syncthreads();
     for (int e = threadIdx.x; e < E; e += 256) ws[(size_t)blockIdx.x * E + e] = cnt[e];

@@ -339,13 +339,8 @@ static int launch_mxfp4_small_tile(const void* A, const void* SA, const void* B,
                                    int M, int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
     auto kern = mxfp4_gemm_small_tile_kernel<TILE, STAGES, EDGE>;
     constexpr int lds_bytes = small_tile_lds_bytes<TILE, STAGES>(true);
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) !=
-            hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, lds_bytes, configured)) return HK_ERR_LAUNCH;
     const int tiles_m = (M + TILE - 1) / TILE, tiles_n = (N + TILE - 1) / TILE;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream, (const uint8_t*)A,
                        (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB, (uint16_t*)C, M, N, K / 2,
@@ -375,13 +370,8 @@ static int launch_mxfp4_splitk(const void* A, const void* SA, const void* B, con
                                int K, int sa_pitch, int sb_pitch, int splits, float* partial, hipStream_t stream) {
     auto kern = mxfp4_gemm_small_tile_kernel<kTinyTile, kTinyStages, EDGE, true>;
     constexpr int lds_bytes = small_tile_lds_bytes<kTinyTile, kTinyStages>(true);
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) !=
-            hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, lds_bytes, configured)) return HK_ERR_LAUNCH;
     const int tiles_m = (M + kTinyTile - 1) / kTinyTile, tiles_n = (N + kTinyTile - 1) / kTinyTile;
     const int nk = (K / 2 + BK - 1) / BK;
     const int kps = ((nk + splits - 1) / splits + 1) & ~1;
@@ -399,13 +389,8 @@ template <bool EDGE>
 static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, const void* SB, void* C,
                               int M, int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
     auto kern = mxfp4_gemm_4wave_kernel<EDGE>;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kLdsBytesFp4) != hipSuccess)
-            return HK_ERR_LAUNCH;
-        configured = true;
-    }
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, kLdsBytesFp4, configured)) return HK_ERR_LAUNCH;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), kLdsBytesFp4, stream,
                        (const uint8_t*)A, (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB,

@@ -164,6 +164,9 @@ int hk_moe_topk_grouped_sigmoid(const float* logits, const float* bias_or_null, 
  * sorted_slots [T*k]: slot indices t*k+j ordered by expert, ascending slot index inside an
  * expert; expert_offsets [E+1]: exclusive prefix sum of per-expert counts; slot_to_pos [T*k]
  * (optional): position of each slot in sorted_slots. workspace: hk_moe_sort_workspace_bytes().
+ * Slots whose id lies outside [0, E) (e.g. -1 for a masked or padded token) take no part: they are
+ * not counted, the valid slots fill sorted_slots[0 .. expert_offsets[E]) and the entries of
+ * sorted_slots behind that, like slot_to_pos of the dropped slots, are left untouched.
  * Requirements: E <= 512. */
 size_t hk_moe_sort_workspace_bytes(int T, int k, int E);
 int hk_moe_sort(const int32_t* ids, int T, int k, int E, int32_t* sorted_slots,
@@ -302,13 +305,6 @@ int hk_moe_fp8blk_forward_ex(const void* x_e4m3, const float* x_scales, const fl
                              const void* w2, const float* w2_scales, void* y_bf16, int T, int H, int I,
                              int E, int k, const void* y_add_bf16_or_null, void* workspace,
                              size_t workspace_bytes, void* stream);
-
-/* Calibration probe (no counterpart in the reference): runs `blocks` workgroups of 8 waves, each
- * wave `iters` x 32 register-only 16x16x128 MFMAs (fp8 if fp4 == 0, else fp4) on operand bits
- * taken from `pattern` (16384 device ints); `sink` receives blocks*512 floats. The caller times
- * the launch; flops = blocks * 8 * iters * 32 * 65536. Gives the power-limited MFMA ceiling for a
- * given operand bit distribution. */
-int hk_probe_mfma_rate(const void* pattern, void* sink, int blocks, int iters, int fp4, void* stream);
 
 #ifdef __cplusplus
 }

@@ -106,6 +106,10 @@ def quantize_e4m3_blocks(x: np.ndarray, block_rows: int, block_cols: int):
 def dequantize_e4m3_blocks(q: np.ndarray, s: np.ndarray, block_rows: int, block_cols: int):
     v = e4m3_decode(q)
     R, C = v.shape
+    if R % block_rows == 0 and C % block_cols == 0:   # whole blocks: broadcast instead of repeating the scales
+        blk = v.reshape(R // block_rows, block_rows, C // block_cols, block_cols)
+        blk *= np.asarray(s, dtype=np.float32)[:, None, :, None]   # v is a fresh array (table lookup)
+        return v
     sr = np.repeat(np.repeat(s, block_rows, axis=0)[:R], block_cols, axis=1)[:, :C]
     return (v * sr).astype(np.float32)
 

@@ -32,6 +32,17 @@ def test_library_exports_every_declared_symbol():
     assert lib.hk_status_string(0) == b"ok" and lib.hk_status_string(-2) == b"bad shape"
 
 
+def test_product_library_exports_nothing_but_the_declared_abi():
+    """Every exported hk* function is declared in include/hk355.h: bench-only tooling (the MFMA rate
+    probe) lives in a library of its own and is not part of the product's ABI."""
+    import subprocess
+
+    out = subprocess.run(["nm", "-D", "--defined-only", str(_lib.lib_path())], capture_output=True, text=True,
+                         check=True).stdout
+    exported = sorted({ln.split()[-1] for ln in out.splitlines() if " T " in ln and ln.split()[-1].startswith("hk")})
+    assert exported == _declared_symbols()
+
+
 def test_c_entry_points_reject_bad_arguments_without_a_gpu():
     lib = hk.load_library()
     buf = ctypes.create_string_buffer(4096 + 64)

@@ -1,0 +1,144 @@
+"""The benchmark configurations at their full sizes, checked for correctness on the GPU.
+
+The CPU oracle cannot multiply 8192^3 in a test's time, so each full-size case combines (i) the oracle
+on a sample of output rows / tokens, (ii) a second kernel of this library that walks the same
+arithmetic through a different launch geometry and must agree everywhere (bit for bit where both
+accumulate in the same order), and (iii) a size-independent property (token-permutation equivariance
+for the MoE layers). Tolerance for floating point: relative Frobenius error <= 1e-2 (the stated bound;
+observed about 2e-3), integers bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import formats as F
+from oracle import gemm as G
+from oracle import moe as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 1e-2
+
+
+@pytest.mark.parametrize("n", [2048, 4096, 16384])
+def test_fp8_gemm_sweep_sizes_against_sampled_oracle(hk, n):
+    """The sweep sizes of the FP8 GEMM next to 8192^3 (which has a test of its own): the kernel the
+    library picks by itself against the CPU oracle on every 509th row, and against the 128x128-tile
+    kernel (same K order, same MFMA: identical bits) over the whole output."""
+    print(f"fp8_gemm full size n={n}", flush=True)
+    g = torch.Generator(device=DEV).manual_seed(n)
+    Aq, sa = hk.quant.quantize_fp8_per_tensor(torch.randn(n, n, device=DEV, generator=g))
+    Bq, sb = hk.quant.quantize_fp8_per_tensor(torch.randn(n, n, device=DEV, generator=g))
+    C = torch.full((n, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    C5 = torch.full((n, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_fp8_gemm(Aq, Bq, C, sa, sb)
+    hk.tk_kernel.dispatch_fp8_gemm(Aq, Bq, C5, sa, sb, variant=5)
+    torch.cuda.synchronize()
+    assert torch.equal(C.view(torch.int16), C5.view(torch.int16))
+    rows = torch.arange(3, n, 509, device=DEV)
+    ref = G.fp8_gemm(Aq.view(torch.uint8)[rows].cpu().numpy(), Bq.view(torch.uint8).cpu().numpy(), sa, sb)
+    out = C[rows].float().cpu().numpy()
+    assert np.isfinite(out).all()
+    assert G.rel_fro_error(out, ref) <= 5e-3
+
+
+def test_mxfp4_gemm_8192_against_other_tiles_and_sampled_oracle(hk):
+    """MXFP4 GEMM at M = N = K = 8192: the kernel hk_mxfp4_gemm picks (1024 workgroups of 256x256
+    tiles, XCD-chunked order, 32 K-steps), the same kernel forced, and the 128x128-tile kernel must
+    give identical bits; every 257th row is compared with the CPU oracle."""
+    n = 8192
+    print("mxfp4_gemm full size 8192", flush=True)
+    g = torch.Generator(device=DEV).manual_seed(0)
+    A, SA = hk.quant.quantize_mxfp4(torch.randn(n, n, device=DEV, generator=g))
+    B, SB = hk.quant.quantize_mxfp4(torch.randn(n, n, device=DEV, generator=g))
+    outs = []
+    for variant in (-1, 1, 2):
+        C = torch.full((n, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+        hk.tk_kernel.dispatch_mxfp4_gemm(A, SA, B, SB, C, variant=variant)
+        torch.cuda.synchronize()
+        outs.append(C)
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
+    rows = torch.arange(0, n, 257, device=DEV)
+    ref = G.mxfp4_gemm(A[rows].cpu().numpy(), SA[rows].cpu().numpy(), B.cpu().numpy(), SB.cpu().numpy())
+    out = outs[0][rows].float().cpu().numpy()
+    assert np.isfinite(out).all()
+    assert G.rel_fro_error(out, ref) <= 5e-3
+
+
+def test_bf16_gemm_8192_against_other_tiles_and_sampled_oracle(hk):
+    n = 8192
+    print("bf16_gemm full size 8192", flush=True)
+    g = torch.Generator(device=DEV).manual_seed(1)
+    A = torch.randn(n, n, device=DEV, generator=g).to(torch.bfloat16)
+    B = torch.randn(n, n, device=DEV, generator=g).to(torch.bfloat16)
+    C = torch.full((n, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    C2 = torch.full((n, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_bf16_gemm(A, B, C)
+    hk.tk_kernel.dispatch_bf16_gemm(A, B, C2, variant=2)
+    torch.cuda.synchronize()
+    assert torch.equal(C.view(torch.int16), C2.view(torch.int16))
+    rows = torch.arange(5, n, 509, device=DEV)
+    bits = lambda t: t.view(torch.int16).cpu().numpy().view(np.uint16)
+    ref = G.bf16_gemm(bits(A[rows]), bits(B))
+    assert G.rel_fro_error(C[rows].float().cpu().numpy(), ref) <= 5e-3
+
+
+def test_moe_fp8blk_full_deepseek_v3_like_shape(hk):
+    """The FP8 block-scaled MoE at its benchmark shape: 8192 tokens, hidden 7168, intermediate 2048,
+    256 DISTINCT experts (11.3 GB of weights, quantized expert by expert on the device), top-8
+    sigmoid routing over 8 groups / top-4 groups: the 65536-slot sort path, the long work-item list
+    and the > 4 GiB weight addressing. Checks: ids and routing weights of all tokens bit-exact against
+    the oracle; the layer is equivariant under a permutation of the tokens (bit for bit); y of eight
+    sampled tokens against the oracle's forward pass over the experts those tokens use."""
+    T, E, k, G_, KG, H, I = 8192, 256, 8, 8, 4, 7168, 2048
+    print("moe_fp8blk full DeepSeek-V3-like shape", flush=True)
+    g = torch.Generator(device=DEV).manual_seed(0)
+    xq, xs = hk.quant.quantize_fp8_blocks(torch.randn(T, H, device=DEV, generator=g), 1, 128)
+    logits = torch.randn(T, E, device=DEV, generator=g)
+    w13q = torch.empty((E, 2 * I, H), dtype=torch.float8_e4m3fn, device=DEV)
+    w13s = torch.empty((E, 2 * I // 128, H // 128), dtype=torch.float32, device=DEV)
+    w2q = torch.empty((E, H, I), dtype=torch.float8_e4m3fn, device=DEV)
+    w2s = torch.empty((E, H // 128, I // 128), dtype=torch.float32, device=DEV)
+    for e in range(E):
+        w13q[e], w13s[e] = hk.quant.quantize_fp8_blocks(torch.randn(2 * I, H, device=DEV, generator=g) * 0.02, 128, 128)
+        w2q[e], w2s[e] = hk.quant.quantize_fp8_blocks(torch.randn(H, I, device=DEV, generator=g) * 0.02, 128, 128)
+    ws = torch.empty(hk.tk_kernel.moe_fp8blk_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=DEV)
+    y = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_fp8blk(xq, xs, logits, None, w13q, w13s, w2q, w2s, y, k, G_, KG, 1.0, ws)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all()
+
+    # routing of every token, bit-exact
+    ids_d = torch.empty((T, k), dtype=torch.int32, device=DEV)
+    w_d = torch.empty((T, k), dtype=torch.float32, device=DEV)
+    hk.tk_kernel.dispatch_moe_topk_grouped_sigmoid(logits, None, ids_d, w_d, G_, KG, 1.0)
+    torch.cuda.synchronize()
+    ids, w = O.topk_grouped_sigmoid(logits.cpu().numpy(), None, k, G_, KG, 1.0)
+    assert np.array_equal(ids_d.cpu().numpy(), ids) and np.array_equal(w_d.cpu().numpy(), w)
+    assert len(np.unique(ids)) == E
+
+    # permutation equivariance over tokens
+    perm = torch.randperm(T, device=DEV, generator=g)
+    y2 = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_fp8blk(xq[perm].contiguous(), xs[perm].contiguous(), logits[perm].contiguous(), None,
+                                     w13q, w13s, w2q, w2s, y2, k, G_, KG, 1.0, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(y2.view(torch.int16), y[perm].view(torch.int16))
+
+    # oracle on eight tokens spread over the batch (first and last included)
+    sel = np.array([0, 1171, 2342, 3513, 4684, 5855, 7026, T - 1])
+    ids_s, w_s = ids[sel], w[sel]
+    used = np.unique(ids_s)
+    remap = {int(e): i for i, e in enumerate(used)}
+    ids_l = np.vectorize(remap.get)(ids_s).astype(np.int32)
+    ut = torch.from_numpy(used.astype(np.int64)).to(DEV)
+    st = torch.from_numpy(sel).to(DEV)
+    want = F.bf16_to_f32(O.moe_fp8blk_forward(
+        xq[st].view(torch.uint8).cpu().numpy(), xs[st].cpu().numpy(), ids_l, w_s,
+        w13q[ut].view(torch.uint8).cpu().numpy(), w13s[ut].cpu().numpy(),
+        w2q[ut].view(torch.uint8).cpu().numpy(), w2s[ut].cpu().numpy()))
+    got = y[st].float().cpu().numpy()
+    assert G.rel_fro_error(got, want) <= TOL
+    row_err = np.linalg.norm(got - want, axis=1) / np.linalg.norm(want, axis=1)
+    assert row_err.max() <= 2e-2, row_err

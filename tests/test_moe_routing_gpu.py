@@ -96,6 +96,33 @@ def test_moe_sort_skewed_and_empty_experts(hk):
     assert np.array_equal(off, roff) and np.array_equal(ss, ro) and np.array_equal(inv, rinv)
 
 
+@pytest.mark.parametrize("T,k,E", [(3000, 4, 128), (20000, 4, 512), (70000, 2, 100), (300, 2, 5)])
+def test_moe_sort_drops_ids_outside_the_expert_range(hk, T, k, E):
+    """Ids outside [0, E) (masked or padded tokens: -1, E, a large value) take no part on either
+    launch path (one launch up to 16384 slots; count / scan / scatter above): the valid slots are
+    sorted as if the others were absent, the tail of sorted_slots and the dropped slots' slot_to_pos
+    keep the caller's contents, and nothing outside the outputs is written."""
+    print(f"moe_sort invalid ids T={T} k={k} E={E}", flush=True)
+    rng = np.random.default_rng(T + k + E)
+    ids = rng.integers(0, E, size=(T, k)).astype(np.int32)
+    bad = rng.random((T, k)) < 0.1
+    ids[bad] = rng.choice(np.array([-1, E, E + 7, 511, 512, 2 ** 31 - 1, -2 ** 31], dtype=np.int64),
+                          size=int(bad.sum())).astype(np.int32)
+    bad = (ids < 0) | (ids >= E)
+    ss, off, inv = _sort(hk, ids, E)
+    flat = ids.reshape(-1)
+    valid = np.nonzero(~bad.reshape(-1))[0].astype(np.int32)
+    order = valid[np.argsort(flat[valid], kind="stable")]
+    counts = np.bincount(flat[valid], minlength=E)
+    assert np.array_equal(off, np.concatenate([[0], np.cumsum(counts)]).astype(np.int32))
+    n = valid.size
+    assert np.array_equal(ss[:n], order)
+    assert np.all(ss[n:] == -1)                       # untouched (the test pre-fills -1)
+    want_inv = np.full(T * k, -1, dtype=np.int32)
+    want_inv[order] = np.arange(n, dtype=np.int32)
+    assert np.array_equal(inv, want_inv)
+
+
 def test_routing_rejects_bad_arguments(hk):
     lg = torch.zeros((4, 1024), dtype=torch.float32, device=DEV)
     ids = torch.zeros((4, 2), dtype=torch.int32, device=DEV)

@@ -136,6 +136,21 @@ def test_block_quant_1x128_and_128x128():
         assert np.abs(d - x).max() <= np.abs(x).max() * 2.0 ** -4
 
 
+def test_block_dequantize_element_by_element():
+    """dequantize_e4m3_blocks against a scalar loop (value of the code times the scale of the block
+    the element lies in), for whole blocks and for ragged last blocks, with distinct scales per block
+    so that a transposed or shifted scale index shows."""
+    rng = np.random.default_rng(3)
+    tbl = F.e4m3_decode_table()
+    for (R, C, br, bc) in ((256, 384, 128, 128), (3, 256, 1, 128), (130, 300, 128, 128), (5, 130, 1, 128)):
+        q = rng.integers(0, 0x7E, size=(R, C), dtype=np.uint8)
+        s = (1.0 + np.arange(-(-R // br) * -(-C // bc), dtype=np.float32)).reshape(-(-R // br), -(-C // bc))
+        d = F.dequantize_e4m3_blocks(q, s, br, bc)
+        assert d.shape == (R, C) and d.dtype == np.float32
+        for r, c in [(0, 0), (R - 1, C - 1), (R - 1, 0), (0, C - 1)] + [(int(rng.integers(R)), int(rng.integers(C))) for _ in range(200)]:
+            assert d[r, c] == np.float32(tbl[q[r, c]] * s[r // br, c // bc])
+
+
 def test_reference_random_init_matches_std_mt19937():
     # first outputs of std::mt19937(42) are 1608637542, 3421126067, 4083286876 (known values)
     rs = np.random.RandomState(42)

@@ -244,3 +244,48 @@ def test_moe_fp8blk_shared_expert_and_residual():
     assert np.array_equal(O.moe_fp8blk_forward(xq, xs, ids, w, w13q, w13s, w2q, w2s, y_add=np.zeros((T, H), np.float32)), base)
     both = F.bf16_to_f32(O.moe_fp8blk_forward(xq, xs, ids, w, w13q, w13s, w2q, w2s, y_add=F.bf16_to_f32(shared)))
     assert np.array_equal(both, 2 * F.bf16_to_f32(shared))  # doubling is exact in bf16
+
+
+def test_moe_fp8blk_forward_brute_force_multi_expert():
+    """T=9, E=4, k=3: token by token and choice by choice instead of expert by expert, with explicit
+    per-block scale products in float64 over the raw codes (no dequantized matrices, no sort, no
+    inverse map), so that the oracle's gather by sorted slot, its per-expert weight selection and its
+    un-permute are checked against plain indexing by ids[t, j]."""
+    rng = np.random.default_rng(8)
+    T, E, k, H, I = 9, 4, 3, 256, 128
+    xq, xs = F.quantize_e4m3_blocks(rng.standard_normal((T, H)).astype(np.float32), 1, 128)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    ids, w = O.topk_grouped_sigmoid(logits, None, k, 2, 2)
+    assert len(set(ids.reshape(-1).tolist())) == E          # every expert is used
+    w13 = [F.quantize_e4m3_blocks((rng.standard_normal((2 * I, H)) * 0.2).astype(np.float32), 128, 128) for _ in range(E)]
+    w2 = [F.quantize_e4m3_blocks((rng.standard_normal((H, I)) * 0.2).astype(np.float32), 128, 128) for _ in range(E)]
+    w13q, w13s = np.stack([a for a, _ in w13]), np.stack([s for _, s in w13])
+    w2q, w2s = np.stack([a for a, _ in w2]), np.stack([s for _, s in w2])
+    y = O.moe_fp8blk_forward(xq, xs, ids, w, w13q, w13s, w2q, w2s)
+
+    xv = F.e4m3_decode(xq).astype(np.float64)
+    want = np.zeros((T, H), dtype=np.float32)
+    for t in range(T):
+        for j in range(k):
+            e = int(ids[t, j])
+            wv = F.e4m3_decode(w13q[e]).astype(np.float64)
+            gu = np.zeros(2 * I)
+            for kb in range(H // 128):
+                part = wv[:, kb * 128:(kb + 1) * 128] @ xv[t, kb * 128:(kb + 1) * 128]
+                gu += part * float(xs[t, kb]) * np.repeat(w13s[e][:, kb], 128).astype(np.float64)
+            g, u = gu[:I], gu[I:]
+            h = (g / (1 + np.exp(-g)) * u).astype(np.float32)
+            hq, hs = F.quantize_e4m3_blocks(h[None, :], 1, 128)
+            hv = F.e4m3_decode(hq[0]).astype(np.float64)
+            o = np.zeros(H)
+            for kb in range(I // 128):
+                part = F.e4m3_decode(w2q[e][:, kb * 128:(kb + 1) * 128]).astype(np.float64) @ hv[kb * 128:(kb + 1) * 128]
+                o += part * float(hs[0, kb]) * np.repeat(w2s[e][:, kb], 128).astype(np.float64)
+            o_bf = F.bf16_to_f32(F.bf16_round(o.astype(np.float32)))
+            want[t] += w[t, j] * o_bf
+    got, want = F.bf16_to_f32(y), F.bf16_to_f32(F.bf16_round(want))
+    # h may land on a neighbouring e4m3 code where fp32 and fp64 accumulation differ by an ulp
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) < 5e-3
+    # a wrong expert for one (token, choice) or a mis-placed row would be an O(1) error in that row
+    row_err = np.linalg.norm(got - want, axis=1) / np.linalg.norm(want, axis=1)
+    assert row_err.max() < 2e-2
