@@ -24,6 +24,8 @@ SIGNATURES = {
     "hk_bf16_gemm_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "hk_bf16_gemm_ws": (c_int, [c_void_p] * 3 + [c_int] * 3 + [c_void_p, c_size_t, c_void_p]),
     "hk_fp8_gemm_ws": (c_int, [c_void_p] * 3 + [c_int] * 3 + [c_float] * 2 + [c_void_p, c_size_t, c_void_p]),
+    "hk_fp8_gemm_static_ws_max_bytes": (c_size_t, []),
+    "hk_fp8_gemm_static_ws": (c_int, [c_void_p] * 3 + [c_int] * 3 + [c_float] * 2 + [c_void_p]),
     "hk_bf16_gemm_variant": (c_int, [c_void_p] * 3 + [c_int] * 4 + [c_void_p]),
     "hk_moe_topk_softmax": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "hk_moe_topk_grouped_sigmoid": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,

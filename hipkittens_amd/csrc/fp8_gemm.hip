@@ -655,6 +655,50 @@ extern "C" int hk_fp8_gemm_ws(const void* A, const void* B, void* C, int M, int 
                 : launch_tile128_splitk<false>(A, B, C, M, N, K, alpha, splits, (float*)workspace, (hipStream_t)stream);
 }
 
+// ---------------------------------------------------------------------------------------
+// Split-K partial sums in device memory that belongs to the library: a file-scope array that every
+// GPU the library is loaded on holds from then until the process ends. 8 MiB covers every shape the
+// split-K path takes on a 256-CU device (ranges x 64x64 tiles <= 512 workgroups, 16 KiB of fp32
+// partial sums each).
+namespace hk {
+constexpr size_t kStaticScratchBytes = 8u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+// The array's address on each device (every GPU has its own copy at its own address), looked up
+// once per device with that device current. Host code uses these pointers, never the array's name.
+static std::atomic<void*> scratch_ptr[64];
+
+static int static_scratch(void** out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return HK_ERR_LAUNCH;
+    if (dev < 0 || dev >= 64) return HK_ERR_UNSUPPORTED;
+    void* p = scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return HK_ERR_LAUNCH;
+        scratch_ptr[dev].store(p, std::memory_order_release);   // a racing thread stores the same address
+    }
+    *out = p;
+    return HK_OK;
+}
+}  // namespace hk
+
+extern "C" size_t hk_fp8_gemm_static_ws_max_bytes(void) { return hk::kStaticScratchBytes; }
+
+extern "C" int hk_fp8_gemm_static_ws(const void* A, const void* B, void* C, int M, int N, int K, float scale_a,
+                                     float scale_b, void* stream) {
+    using namespace hk;
+    if (M <= 0 || N <= 0 || K <= 0) return HK_ERR_BAD_SHAPE;
+    const int splits = splitk_ranges(M, N, K);
+    if (splits < 2) return hk_fp8_gemm(A, B, C, M, N, K, scale_a, scale_b, stream);   // no scratch needed
+    const size_t need = (size_t)splits * M * N * sizeof(float);
+    if (need > kStaticScratchBytes) return HK_ERR_WORKSPACE;   // more partial sums than the array holds
+    void* ws = nullptr;
+    const int st = static_scratch(&ws);
+    if (st != HK_OK) return st;
+    // every partial sum that the reduction reads is written by this call's first kernel: nothing in
+    // the array needs clearing between calls
+    return hk_fp8_gemm_ws(A, B, C, M, N, K, scale_a, scale_b, ws, kStaticScratchBytes, stream);
+}
+
 extern "C" int hk_fp8_gemm(const void* A, const void* B, void* C, int M, int N, int K,
                            float scale_a, float scale_b, void* stream) {
     using namespace hk;

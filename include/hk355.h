@@ -61,6 +61,20 @@ size_t hk_fp8_gemm_workspace_bytes(int M, int N, int K);
 int hk_fp8_gemm_ws(const void* A_e4m3, const void* B_e4m3, void* C_bf16, int M, int N, int K,
                    float scale_a, float scale_b, void* workspace, size_t workspace_bytes, void* stream);
 
+/* hk_fp8_gemm_ws without a workspace argument, for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart
+ * in the reference. The split-K partial sums go to a file-scope device array of
+ * hk_fp8_gemm_static_ws_max_bytes() = 8 MiB inside the library, which every GPU the library runs on
+ * holds until the process ends; the call allocates and frees nothing. The first call on a device looks
+ * the array's address up (make it before a capture starts). Shapes that the split-K path does not take
+ * run as hk_fp8_gemm; a shape whose partial sums exceed the array returns HK_ERR_WORKSPACE (cannot
+ * happen on a 256-CU device: at most 512 workgroups x 16 KiB). Results are bit-identical to
+ * hk_fp8_gemm_ws. All calls on one GPU share the one array: calls that overlap in time on the same GPU
+ * (different streams or threads) race and must be serialized by the caller. */
+size_t hk_fp8_gemm_static_ws_max_bytes(void);
+int hk_fp8_gemm_static_ws(const void* A_e4m3, const void* B_e4m3, void* C_bf16, int M, int N, int K,
+                          float scale_a, float scale_b, void* stream);
+
 /* Same contract, forced onto one kernel variant (for tests and tuning):
  * 0 = portable kernel (any shape), 1 = 256x256x128 tile, 8 waves, 2 = 256x256x128 tile,
  * 4 waves, hand-interleaved schedule over two LDS stages, 3 = 256x256x128 tile, 4 waves, plain
