@@ -62,6 +62,15 @@ SIGNATURES = {
     "hk_moe_fp8blk_forward_ex": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                          c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hk_moe_fp8blk_preshuffle_bytes": (c_int, [c_int, c_int, c_int, c_int, ctypes.POINTER(c_size_t)]),
+    "hk_moe_fp8blk_preshuffle": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "hk_moe_fp8blk_experts_ex2": (c_int, [c_void_p] * 11 + [c_int] * 6 + [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hk_moe_fp8blk_forward_ex2": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p,
+                                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                          c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hk_moe_fp8blk_forward_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p,
+                                           c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                           c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hk_moe_fp8blk_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p,
                                       c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                       c_void_p, c_size_t, c_void_p]),

@@ -165,8 +165,11 @@ __device__ __forceinline__ int scalar_load_x1(const void* p) {
 // complete out of order with respect to each other, so a compiler that sees both kinds pending
 // waits for all of them (vmcnt(0)) before the first use of any loaded register; kernels that
 // keep register loads in flight across an epilogue issue the epilogue's stores through these.
+// (A store of more than 8 bytes reads its data registers for two more cycles after issue: a VALU
+// instruction that overwrites them must keep that distance. The compiler spaces its own stores; for
+// this one, which it cannot see, the two wait states are part of the statement.)
 __device__ __forceinline__ void store_global_b128(void* p, v4i v) {
-    asm volatile("global_store_dwordx4 %0, %1, off" ::"v"(p), "v"(v) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
 }
 __device__ __forceinline__ void store_global_b32(void* p, uint32_t v) {
     asm volatile("global_store_dword %0, %1, off" ::"v"(p), "v"(v) : "memory");

@@ -389,6 +389,489 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
     wait_vmcnt<0>();
 }
 
+// ------------------------------------------------------- grouped GEMM, pre-shuffled weights
+// The kernel above moves both operands through LDS with two K-steps in flight; it is bound by how
+// fast tiles are delivered to the CU (latency x bytes in flight) and by LDS traffic. This one is
+// built around more bytes in flight and fewer LDS bytes per MFMA:
+//   * 4 waves, one per SIMD (512 registers each). Wave w owns weight rows [64 w, +64) of the 256-row
+//     tile (four MFMA fragments) x all rows of the item (up to 160 = ten fragments): 160 accumulator
+//     registers, 4 MFMAs per activation fragment read;
+//   * weights never touch LDS: the pre-shuffled layout (moe_fp8blk_preshuffle_kernel) stores, for
+//     every (expert, n-tile, K-step), each wave's four fragments as contiguous 1 KiB pieces in lane
+//     order, and the wave loads them straight into accumulation registers (AGPRs, which the MFMA
+//     reads as its weight operand) four K-steps ahead: a ring of five sets of 32 registers;
+//   * the activation tile (20 KiB + row scales) goes through a ring of five LDS stages, filled four
+//     K-steps ahead by direct global->LDS loads (gate+up: gathered from the caller's x by token);
+//   * the fp32 block scales are applied as before: every K-step's MFMAs write fresh partial sums,
+//     acc += partial * (x_scale[row] * w_scale), here with hand-placed instructions: the FMAs of an
+//     MFMA follow two MFMAs later, the next fragment's LDS reads and the loads of position + 4 are
+//     spread over the MFMA slots. One wave per SIMD issues one instruction per four cycles, which
+//     with 16 FMAs per fragment is as much as the MFMA pipe takes: no instruction is spent on
+//     branches in the main path: every K-step runs all ten fragments (rows past an item's count are
+//     zeros in LDS and are never stored), because accumulators behind branches cost register copies.
+// The stream of (item, K-step) positions runs across item boundaries. All vector-memory loads are
+// inline asm and counted by hand: per position a wave issues 14 loads (5 activation pieces, the row
+// scales, 8 weight pieces; GATHER: 6 more per item for the slot ids), loads return in order, and the
+// wait for position p + 1 sits in step p behind the loads of position p + 4: vmcnt(3 x 14).
+// Results are bit-identical to the kernel above (same MFMA, K order and scaling FMAs).
+constexpr int kF8sMT = kF8BM / 16;                       // 10 row fragments per item
+constexpr int kF8sStages = 5;
+constexpr int kF8sStage = 21504;                         // 160 x 128 B, then 16 x 12 row scales, padded to a multiple of 256 B
+constexpr int kF8sXch = kF8sStages * kF8sStage;          // epilogue exchange buffer: 160 x 4 floats
+constexpr int kF8sLds = kF8sXch + kF8BM * 16;            // 107.5 KiB
+constexpr int kF8sBTile = 256 * 128;                     // one (n-tile, K-step) block of the pre-shuffled weights
+constexpr int kF8sLoads = 14;                            // loads per wave and position
+static_assert(kF8sStage >= kF8ATile + 16 * 12 * 4 && kF8sStage % 256 == 0 && kF8sLds <= 160 * 1024, "LDS plan");
+static_assert(3 * kF8sLoads < 64 && kF8sMT == 10, "vmcnt range; the slot plan below is written for ten fragments");
+
+// The weight ring lives in fixed accumulation registers: fragment F = 4 * set + n of the ring in
+// a[8 F .. 8 F + 7] (low / high K half in the first / last four). Naming them in the constraints keeps the two
+// 16-byte loads of a fragment and the MFMA that reads all 32 bytes on the same registers without copies.
+#define HK_F8S_BREGS(X) \
+    X(0, "{a[0:3]}", "{a[4:7]}", "{a[0:7]}") \
+    X(1, "{a[8:11]}", "{a[12:15]}", "{a[8:15]}") \
+    X(2, "{a[16:19]}", "{a[20:23]}", "{a[16:23]}") \
+    X(3, "{a[24:27]}", "{a[28:31]}", "{a[24:31]}") \
+    X(4, "{a[32:35]}", "{a[36:39]}", "{a[32:39]}") \
+    X(5, "{a[40:43]}", "{a[44:47]}", "{a[40:47]}") \
+    X(6, "{a[48:51]}", "{a[52:55]}", "{a[48:55]}") \
+    X(7, "{a[56:59]}", "{a[60:63]}", "{a[56:63]}") \
+    X(8, "{a[64:67]}", "{a[68:71]}", "{a[64:71]}") \
+    X(9, "{a[72:75]}", "{a[76:79]}", "{a[72:79]}") \
+    X(10, "{a[80:83]}", "{a[84:87]}", "{a[80:87]}") \
+    X(11, "{a[88:91]}", "{a[92:95]}", "{a[88:95]}") \
+    X(12, "{a[96:99]}", "{a[100:103]}", "{a[96:103]}") \
+    X(13, "{a[104:107]}", "{a[108:111]}", "{a[104:111]}") \
+    X(14, "{a[112:115]}", "{a[116:119]}", "{a[112:119]}") \
+    X(15, "{a[120:123]}", "{a[124:127]}", "{a[120:127]}") \
+    X(16, "{a[128:131]}", "{a[132:135]}", "{a[128:135]}") \
+    X(17, "{a[136:139]}", "{a[140:143]}", "{a[136:143]}") \
+    X(18, "{a[144:147]}", "{a[148:151]}", "{a[144:151]}") \
+    X(19, "{a[152:155]}", "{a[156:159]}", "{a[152:159]}")
+
+struct F8Cursor { int it, kt, expert, row_start, rows, n_tile; bool valid; };
+
+template <int MODE, bool GATHER>
+__global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Params p) {
+    static_assert(!GATHER || MODE == 0, "only the gate+up GEMM reads the caller's activations");
+    constexpr int MT = kF8sMT, NT = 4, NA = 5;
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    const int lane = lane_id(), w = wave_id();
+
+    const int n_items = scalar_load_x1(p.num_items);
+    const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+    const int it_stride = ((int)gridDim.x - xcd + kNumXcd - 1) / kNumXcd;
+    const int per_xcd = (n_items + kNumXcd - 1) / kNumXcd;
+    const int it0 = xcd * per_xcd + slot;
+    const int it_end = min(n_items, (xcd + 1) * per_xcd);
+    if (it0 >= it_end) return;
+
+    const int nk = p.K >> 7;
+    const v4i srd_a = make_srd(p.A, GATHER ? (uint32_t)p.T * (uint32_t)p.K : (uint32_t)nk * (uint32_t)p.S * 128u);
+    const v4i srd_sa = make_srd(p.SA, GATHER ? (uint32_t)p.T * (uint32_t)nk * 4u : (uint32_t)nk * (uint32_t)p.S * 4u);
+    // Activation tile: wave w fetches rows [40 w, +40) in five 1 KiB pieces of 8 rows; lane l lands in
+    // row + l / 8, physical chunk l % 8 and so fetches logical chunk swz(row, l % 8).
+    auto piece_row = [&](int i) { return 40 * w + 8 * i + (lane >> 3); };
+    // Row scales of a stage: [row % 16][row / 16, padded to 12] floats, so that a lane's scale of fragment
+    // m sits at a fixed offset from its base. Wave w fetches slots [48 w, +48) with lanes 0..47.
+    const int sf = 48 * w + min(lane, 47);
+    const int scale_row = (sf % 12) < MT ? 16 * (sf % 12) + sf / 12 : -1;   // -1: padding slot, nothing fetched
+    constexpr uint64_t kSaMask = (1ull << 48) - 1ull;
+
+    // ---- cursors over this workgroup's stream of (item, K-step) positions -----------------------
+    auto load_item = [&](F8Cursor& c) __attribute__((always_inline)) {
+        c.valid = c.it < it_end;
+        const v4i item = scalar_load_x4(p.items + (c.valid ? c.it : it_end - 1));
+        c.expert = item.x; c.row_start = item.y; c.rows = item.z; c.n_tile = item.w;
+    };
+    auto advance = [&](F8Cursor& c) __attribute__((always_inline)) {
+        if (++c.kt == nk) { c.kt = 0; c.it += it_stride; load_item(c); }
+    };
+    F8Cursor cc{it0, 0}, cn, cf;   // compute position, the one after it, fetch position (+4)
+    load_item(cc);
+    cn = cc; advance(cn);
+    cf = cc;
+
+    // ---- GATHER: slot ids of the rows this lane fetches, one item ahead of the fetch cursor --------
+    struct SlotIds { uint32_t a[NA]; uint32_t s; };
+    auto issue_ids = [&](int idx, SlotIds& o) __attribute__((always_inline)) {
+        if (idx >= it_end) idx = it_end - 1;
+        const int row_start = scalar_load_x4(p.items + idx).y;
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            const uint32_t off = (uint32_t)min(row_start + piece_row(i), p.S - 1) * 4u;
+            asm volatile("global_load_dword %0, %1, %2" : "=v"(o.a[i]) : "v"(off), "s"(p.sorted_slots) : "memory");
+        }
+        const uint32_t off = (uint32_t)min(row_start + max(scale_row, 0), p.S - 1) * 4u;
+        asm volatile("global_load_dword %0, %1, %2" : "=v"(o.s) : "v"(off), "s"(p.sorted_slots) : "memory");
+    };
+    auto landed_ids = [&](SlotIds& o) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NA; ++i) asm volatile("" : "+v"(o.a[i]));
+        asm volatile("" : "+v"(o.s));
+    };
+    SlotIds ids_next{};
+    // per-lane source offsets of the fetch cursor's item (GATHER: by token; else fixed tile offsets)
+    uint32_t a_voff[NA], sa_voff;
+    auto make_offsets = [&](const F8Cursor& c, const SlotIds& ids) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            const uint32_t ch = swz_chunk(piece_row(i), lane & 7) * 16u;
+            // GATHER: rows past the item's count are not fetched at all (bit 31: out of range, LDS gets zeros)
+            if (GATHER) a_voff[i] = piece_row(i) < c.rows ? (ids.a[i] / (uint32_t)p.topk) * (uint32_t)p.K + ch : 0x80000000u;
+            else a_voff[i] = (uint32_t)piece_row(i) * 128u + ch;
+        }
+        if (GATHER) sa_voff = scale_row >= 0 && scale_row < c.rows ? (ids.s / (uint32_t)p.topk) * (uint32_t)nk * 4u : 0x80000000u;
+        else sa_voff = scale_row >= 0 ? (uint32_t)scale_row * 4u : 0x80000000u;
+    };
+    // uniform state of the fetch position, refreshed by fetch_begin() once per step
+    v4i f_srd_a, f_srd_sa, f_srd_b;
+    uint32_t f_soff_a, f_soff_sa, f_soff_b;
+    int f_pieces;   // (not GATHER) pieces of this wave that hold rows of the item; the others fetch nothing
+    auto fetch_begin = [&]() __attribute__((always_inline)) {
+        f_srd_a = srd_a; f_srd_sa = srd_sa;
+                if (!cf.valid) { f_srd_a.z = 0; f_srd_sa.z = 0; }
+        f_srd_b = make_srd(p.B + (size_t)cf.expert * p.b_expert_stride + (size_t)cf.n_tile * nk * kF8sBTile,
+                           cf.valid ? (uint32_t)nk * kF8sBTile : 0u);
+        const uint32_t row_base = (uint32_t)cf.kt * (uint32_t)p.S + (uint32_t)cf.row_start;
+        f_soff_a = GATHER ? (uint32_t)cf.kt * 128u : row_base * 128u;
+        f_soff_sa = GATHER ? (uint32_t)cf.kt * 4u : row_base * 4u;
+        f_soff_b = (uint32_t)cf.kt * kF8sBTile + (uint32_t)w * 8192u;
+        f_pieces = GATHER ? NA : (cf.rows - 40 * w + 7) >> 3;
+    };
+    auto fetch_advance = [&]() __attribute__((always_inline)) {
+        if (++cf.kt == nk) {
+            cf.kt = 0; cf.it += it_stride; load_item(cf);
+            if (GATHER) {
+                // the ids were requested when the cursor entered the previous item, ahead of that
+                // position's loads, which an earlier step has waited for unless the item was shorter
+                // than the wait's reach
+                if (nk < 5) wait_vmcnt<0>();
+                landed_ids(ids_next);
+                make_offsets(cf, ids_next);
+                issue_ids(cf.it + it_stride, ids_next);
+            }
+        }
+    };
+
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+    const uint32_t lds_wave_a = to_sgpr(lds0 + (uint32_t)w * 5120u);
+    const uint32_t lds_wave_sa = to_sgpr(lds0 + kF8ATile + (uint32_t)w * 192u);
+    const uint32_t voff_b = lane * 16;
+    struct BFrag { v4i lo, hi; };
+    BFrag bw[5][NT];   // weight fragments of five positions, in AGPRs
+    // Load L (0..13) of the fetch position into LDS stage / register set PF. Order: an activation
+    // piece or the scales, then a weight piece, alternating.
+    auto fetch_load = [&]<int PF, int L>() __attribute__((always_inline)) {
+        constexpr int kind = L < 12 ? (L & 1) : 1;            // 0: activation side, 1: weight piece
+        constexpr int ai = L >> 1;                            // activation piece 0..4, 5 = row scales
+        constexpr int bi = L < 12 ? (L >> 1) : L - 6;         // weight piece 0..7 = (fragment, K half)
+        if constexpr (kind == 0 && ai < NA) {
+            v4i s = f_srd_a;
+            if (!GATHER && ai >= f_pieces) s.z = 0;
+            dma16(s, lds_wave_a + PF * kF8sStage + ai * 1024, a_voff[ai], f_soff_a);
+        } else if constexpr (kind == 0) {
+            dma4_lanes(f_srd_sa, lds_wave_sa + PF * kF8sStage, sa_voff, f_soff_sa, kSaMask);
+        } else {
+            constexpr int n = bi >> 1, half = bi & 1, F = PF * NT + n;
+            constexpr int imm = (n & 1) * 2048 + half * 1024;
+            const uint32_t soff = f_soff_b + (n >= 2 ? 4096u : 0u);
+            v4i& dst = half ? bw[PF][n].hi : bw[PF][n].lo;
+#define HK_X(F_, LO, HI, ALL)                                                                                        \
+    if constexpr (F == F_ && half == 0)                                                                              \
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4" : "=" LO(dst) : "v"(voff_b), "s"(f_srd_b), "s"(soff), "n"(imm) : "memory"); \
+    if constexpr (F == F_ && half == 1)                                                                              \
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4" : "=" HI(dst) : "v"(voff_b), "s"(f_srd_b), "s"(soff), "n"(imm) : "memory");
+            HK_F8S_BREGS(HK_X)
+#undef HK_X
+        }
+    };
+    auto fetch_all = [&]<int PF>() __attribute__((always_inline)) {
+        fetch_load.template operator()<PF, 0>(); fetch_load.template operator()<PF, 1>();
+        fetch_load.template operator()<PF, 2>(); fetch_load.template operator()<PF, 3>();
+        fetch_load.template operator()<PF, 4>(); fetch_load.template operator()<PF, 5>();
+        fetch_load.template operator()<PF, 6>(); fetch_load.template operator()<PF, 7>();
+        fetch_load.template operator()<PF, 8>(); fetch_load.template operator()<PF, 9>();
+        fetch_load.template operator()<PF, 10>(); fetch_load.template operator()<PF, 11>();
+        fetch_load.template operator()<PF, 12>(); fetch_load.template operator()<PF, 13>();
+    };
+    auto landed = [&]<int PS>() __attribute__((always_inline)) {
+#define HK_X(F_, LO, HI, ALL) \
+    if constexpr (F_ / NT == PS) asm volatile("" : "+" LO(bw[PS][F_ % NT].lo), "+" HI(bw[PS][F_ % NT].hi));
+        HK_F8S_BREGS(HK_X)
+#undef HK_X
+    };
+
+    // ---- LDS -> registers -------------------------------------------------------------------------
+    const uint32_t r = lane & 15, g = lane >> 4;
+    const uint32_t rd_lo = lds0 + r * 128u + swz_chunk(r, g) * 16u;
+    const uint32_t rd_hi = lds0 + r * 128u + swz_chunk(r, g + 4) * 16u;
+    const uint32_t rd_sa = lds0 + kF8ATile + r * 48u;
+
+    float acc[MT][NT][4];
+    auto zero_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[m][n][e] = 0.f;
+    };
+    v4f part[4] = {};        // partial sums of the last four MFMAs (slot n of a fragment writes part[n])
+    v8i af[2];               // activation fragments, by fragment parity
+    float xs_r[2];           // their rows' scales
+    float sc[2][2] = {};     // by fragment parity: x_scale * w_scale of the gate (even) / up (odd) weight fragments
+    float ws0 = 0.f, ws1 = 0.f;           // weight scales of the compute position
+    float ws0_next = 0.f, ws1_next = 0.f; // ... of the position after it, requested one step earlier
+    // D(16 weight rows x 16 rows) = W . A^T into fresh registers; weights from AGPRs
+    auto mfma = [&]<int F>(v4f& d, const v8i& a) __attribute__((always_inline)) {
+        const BFrag& b = bw[F / NT][F % NT];
+        const v8i b8 = __builtin_shufflevector(b.lo, b.hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#define HK_X(F_, LO, HI, ALL) \
+    if constexpr (F == F_) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=v"(d) : ALL(b8), "v"(a));
+        HK_F8S_BREGS(HK_X)
+#undef HK_X
+    };
+    // acc += part * s; placed by hand two MFMAs behind the one that produced `part` (the compiler does not
+    // know the MFMA's latency), hence asm
+    auto fma4 = [&](float (&a)[4], const v4f& pt, float s) __attribute__((always_inline)) {
+        asm volatile("v_fma_f32 %0, %4, %8, %0\n\tv_fma_f32 %1, %5, %8, %1\n\tv_fma_f32 %2, %6, %8, %2\n\tv_fma_f32 %3, %7, %8, %3"
+                     : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3])
+                     : "v"(pt.x), "v"(pt.y), "v"(pt.z), "v"(pt.w), "v"(s));
+    };
+    // weight scales of a position, through the scalar cache, not waited for here
+    auto request_ws = [&](const F8Cursor& c) __attribute__((always_inline)) {
+        const float* sb = p.SB + (size_t)c.expert * p.sb_expert_stride;
+        const float* s0;
+        const float* s1;
+        if (MODE == 0) {
+            s0 = sb + (size_t)c.n_tile * nk + c.kt;                    // gate rows of the tile
+            s1 = sb + (size_t)(p.N / 128 + c.n_tile) * nk + c.kt;      // up rows
+        } else {
+            s0 = sb + (size_t)min(2 * c.n_tile + (w >> 1), p.N / 128 - 1) * nk + c.kt;
+            s1 = s0;
+        }
+        asm volatile("s_load_dword %0, %1, 0x0" : "=s"(ws0_next) : "s"(s0) : "memory");
+        asm volatile("s_load_dword %0, %1, 0x0" : "=s"(ws1_next) : "s"(s1) : "memory");
+    };
+
+    auto epilogue = [&](const F8Cursor& a) __attribute__((always_inline)) {
+        const int rows = a.rows, row_start = a.row_start;
+        const int n0 = a.n_tile * (MODE == 0 ? 128 : 256);
+        if (MODE == 1) {
+            uint16_t* out = (uint16_t*)p.out0;
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const int row = 16 * m + (int)r;
+                if (row >= rows) continue;
+                const size_t pos = (size_t)(row_start + row);
+#pragma unroll
+                for (int q = 0; q < NT / 2; ++q) {
+                    const int col = n0 + w * 64 + 32 * q + 8 * (int)g;
+                    if (col + 8 > p.N) continue;
+                    const float (&x)[4] = acc[m][2 * q];
+                    const float (&y)[4] = acc[m][2 * q + 1];
+                    v4i o4;
+                    o4.x = pack_bf16(x[0], x[1]); o4.y = pack_bf16(x[2], x[3]);
+                    o4.z = pack_bf16(y[0], y[1]); o4.w = pack_bf16(y[2], y[3]);
+                    store_global_b128(out + pos * p.N + col, o4);
+                }
+            }
+        } else {
+            // h = silu(gate) * up for this wave's 32 of the tile's 128 h columns; the tile's 128
+            // columns are one 1 x 128 quantization block, so the row maxima of the four waves are
+            // combined through LDS.
+            uint8_t* hq = (uint8_t*)p.out0;
+            float h[MT][8];
+            const uint32_t xch = lds0 + kF8sXch;
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+#pragma unroll
+                for (int q = 0; q < 2; ++q)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float gv = acc[m][2 * q][j];
+                        h[m][4 * q + j] = gv / (1.0f + __expf(-gv)) * acc[m][2 * q + 1][j];
+                    }
+                float amax = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(h[m][i]));
+                amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+                const int row = 16 * m + (int)r;
+                if (g == 0) *(lds_f32_mut_t*)(uintptr_t)(xch + (row * 4 + w) * 4) = amax;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const int row = 16 * m + (int)r;
+                const v4f am = *(lds_v4f_t*)(uintptr_t)(xch + row * 16);
+                const float s = e4m3_block_scale(fmaxf(fmaxf(am.x, am.y), fmaxf(am.z, am.w)));
+                if (row < rows) {
+                    const size_t tile_row = (size_t)a.n_tile * p.S + (size_t)(row_start + row);
+                    const v2i q8 = quant8_e4m3(h[m], s);
+                    asm volatile("global_store_dwordx2 %0, %1, off" ::"v"(hq + tile_row * 128 + 32 * w + 8 * g), "v"(q8) : "memory");
+                    if (w == 0 && g == 0) store_global_b32(p.out_scales + tile_row, __float_as_uint(s));
+                }
+            }
+            __syncthreads();   // the exchange buffer is rewritten by the next item's epilogue
+        }
+    };
+
+    // ---- prologue: positions 0..3 in flight, the first position's first fragment in registers -------
+    SlotIds ids0{};
+    if (GATHER) {
+        issue_ids(it0, ids0);
+        issue_ids(it0 + it_stride, ids_next);
+        wait_vmcnt<0>();
+        landed_ids(ids0);
+    }
+    make_offsets(cf, ids0);
+    fetch_begin(); fetch_all.template operator()<0>(); fetch_advance();
+    fetch_begin(); fetch_all.template operator()<1>(); fetch_advance();
+    fetch_begin(); fetch_all.template operator()<2>(); fetch_advance();
+    fetch_begin(); fetch_all.template operator()<3>(); fetch_advance();
+    request_ws(cc);
+    zero_acc();
+    wait_vmcnt<3 * kF8sLoads>();
+    block_barrier();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    asm volatile("" : "+s"(ws0_next), "+s"(ws1_next));   // the requested scales are in their registers from here on
+    ws0 = ws0_next; ws1 = ws1_next;
+    request_ws(cn);
+    af[0] = lds_frag(rd_lo, rd_hi, 0);
+    xs_r[0] = *(lds_f32_t*)(uintptr_t)rd_sa;
+
+    // One stream position on LDS stage / weight register set P (both = position % 5). Every position
+    // runs all ten fragments (rows past the item's count are zeros in LDS and are never stored): a
+    // fragment count that varies would put the accumulators behind branches.
+    auto step = [&]<int P>() __attribute__((always_inline)) {
+        constexpr int PF = (P + 4) % 5, PN = (P + 1) % 5;
+        fetch_begin();
+        landed.template operator()<P>();
+        const uint32_t a_lo = rd_lo + P * kF8sStage, a_hi = rd_hi + P * kF8sStage, a_sa = rd_sa + P * kF8sStage;
+        // Behind fragment 8's third MFMA, when every LDS read of this position has been issued: the next
+        // position's tile is waited for, its first fragment and scale are read, its weight scales arrive.
+        auto transition = [&]() __attribute__((always_inline)) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this position's last LDS reads and the scale request
+            asm volatile("" : "+s"(ws0_next), "+s"(ws1_next));
+            wait_vmcnt<3 * kF8sLoads>();
+            block_barrier();   // everyone's part of the next position's tile has landed; everyone has read this position's
+            af[0] = lds_frag(rd_lo + PN * kF8sStage, rd_hi + PN * kF8sStage, 0);
+            xs_r[0] = *(lds_f32_t*)(uintptr_t)(rd_sa + PN * kF8sStage);
+        };
+        // Fragment M: four MFMA slots; the FMAs of an MFMA follow two slots later (fragment 0 starts with
+        // those of fragment 9 of the previous K-step).
+        auto block = [&]<int M>() __attribute__((always_inline)) {
+            constexpr int MP = M == 0 ? MT - 1 : M - 1;   // the fragment whose last two FMA groups are still owed
+            const v8i& a_cur = af[M & 1];
+            // slot 0
+            mfma.template operator()<P * NT + 0>(part[0], a_cur);
+            if constexpr (M < MT - 2) {
+                af[(M + 1) & 1] = lds_frag(a_lo, a_hi, (M + 1) * 2048);
+                xs_r[(M + 1) & 1] = *(lds_f32_t*)(uintptr_t)(a_sa + (M + 1) * 4);
+            }
+            fma4(acc[MP][2], part[2], sc[MP & 1][0]);
+            if constexpr (M <= 6) fetch_load.template operator()<PF, 2 * M>();
+            __builtin_amdgcn_sched_barrier(0);
+            // slot 1
+            mfma.template operator()<P * NT + 1>(part[1], a_cur);
+            fma4(acc[MP][3], part[3], sc[MP & 1][1]);
+            sc[M & 1][0] = xs_r[M & 1] * ws0;
+            sc[M & 1][1] = xs_r[M & 1] * ws1;
+            if constexpr (M <= 6) fetch_load.template operator()<PF, 2 * M + 1>();
+            __builtin_amdgcn_sched_barrier(0);
+            // slot 2
+            mfma.template operator()<P * NT + 2>(part[2], a_cur);
+            fma4(acc[M][0], part[0], sc[M & 1][0]);
+            if constexpr (M == MT - 2) {
+                // fragment 9 is read here, ahead of the barrier that frees this stage
+                af[(M + 1) & 1] = lds_frag(a_lo, a_hi, (M + 1) * 2048);
+                xs_r[(M + 1) & 1] = *(lds_f32_t*)(uintptr_t)(a_sa + (M + 1) * 4);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // slot 3
+            mfma.template operator()<P * NT + 3>(part[3], a_cur);
+            fma4(acc[M][1], part[1], sc[M & 1][1]);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        block.template operator()<0>();
+        block.template operator()<1>();
+        block.template operator()<2>();
+        block.template operator()<3>();
+        block.template operator()<4>();
+        block.template operator()<5>();
+        block.template operator()<6>();
+        block.template operator()<7>();
+        block.template operator()<8>();
+        // fragment 9, with the transition to the next position behind its first MFMA: ws0 / ws1 keep this
+        // position's values until the end of the step
+        {
+            constexpr int M = MT - 1, MP = M - 1;
+            const v8i& a_cur = af[M & 1];
+            mfma.template operator()<P * NT + 0>(part[0], a_cur);
+            fma4(acc[MP][2], part[2], sc[MP & 1][0]);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma.template operator()<P * NT + 1>(part[1], a_cur);
+            fma4(acc[MP][3], part[3], sc[MP & 1][1]);
+            sc[M & 1][0] = xs_r[M & 1] * ws0;
+            sc[M & 1][1] = xs_r[M & 1] * ws1;
+            transition();
+            __builtin_amdgcn_sched_barrier(0);
+            mfma.template operator()<P * NT + 2>(part[2], a_cur);
+            fma4(acc[M][0], part[0], sc[M & 1][0]);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma.template operator()<P * NT + 3>(part[3], a_cur);
+            fma4(acc[M][1], part[1], sc[M & 1][1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        fetch_advance();
+        if (cc.valid && cc.kt == nk - 1) {
+            // the item is complete: the two FMA groups still owed, then the epilogue
+            mfma_drain();
+            fma4(acc[MT - 1][2], part[2], sc[(MT - 1) & 1][0]);
+            fma4(acc[MT - 1][3], part[3], sc[(MT - 1) & 1][1]);
+            epilogue(cc);
+            zero_acc();
+            sc[(MT - 1) & 1][0] = 0.f; sc[(MT - 1) & 1][1] = 0.f;   // what the next K-step adds for "fragment 9 of the previous K-step"
+        }
+        cc = cn;
+        advance(cn);
+        ws0 = ws0_next; ws1 = ws1_next;
+        request_ws(cn);
+    };
+    while (cc.valid) {
+        step.template operator()<0>();
+        step.template operator()<1>();
+        step.template operator()<2>();
+        step.template operator()<3>();
+        step.template operator()<4>();
+    }
+    wait_vmcnt<0>();   // nothing may still be writing LDS when the workgroup retires
+}
+
+// Pre-shuffle of FP8 expert weights for moe_fp8blk_stream_kernel (offline, once per checkpoint).
+// One thread per 16 bytes of the output. mode 0: gate+up matrix [E, 2N, K] (N = I); mode 1: down
+// matrix [E, N, K] (N = H). Output: [E][n-tile][K-step][column wave 4][fragment 4][K half 2][lane 64][16],
+// lane l = (r, g) holding row 64 wn + 16 f + r of the tile (moe_b_row) and bytes 16 (g + 4 half) .. +16
+// of the K-step.
+__global__ __launch_bounds__(256) void moe_fp8blk_preshuffle_kernel(const uint8_t* __restrict__ w, int N, int K,
+                                                                    int mode, int n_tiles, long long expert_stride,
+                                                                    uint8_t* __restrict__ out) {
+    const int nk = K >> 7;
+    const long long chunk = (long long)blockIdx.x * 256 + threadIdx.x;   // 16-byte chunk within the expert
+    const long long per_expert = (long long)n_tiles * nk * (kF8sBTile / 16);
+    if (chunk >= per_expert) return;
+    const int e = blockIdx.y;
+    const int lane = (int)(chunk & 63), half = (int)((chunk >> 6) & 1), f = (int)((chunk >> 7) & 3), wn = (int)((chunk >> 9) & 3);
+    const long long blk = chunk >> 11;
+    const int kt = (int)(blk % nk), nt = (int)(blk / nk);
+    const int R = 64 * wn + 16 * f + (lane & 15);
+    const int row = moe_b_row(mode, R, nt, N);
+    const v4i v = *(const v4i*)(w + (size_t)e * expert_stride + (size_t)row * K + (size_t)kt * 128 + 16 * ((lane >> 4) + 4 * half));
+    *(v4i*)(out + ((size_t)e * per_expert + chunk) * 16) = v;
+}
+
 template <int MODE, bool GATHER>
 static int launch_fp8blk_gemm(const MoeFp8Params& p, int max_items, hipStream_t s) {
     auto kern = moe_fp8blk_gemm_kernel<MODE, GATHER>;
@@ -398,6 +881,20 @@ static int launch_fp8blk_gemm(const MoeFp8Params& p, int max_items, hipStream_t 
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kF8Lds, s, p);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
+
+template <int MODE, bool GATHER>
+static int launch_fp8blk_stream(const MoeFp8Params& p, int max_items, hipStream_t s) {
+    auto kern = moe_fp8blk_stream_kernel<MODE, GATHER>;
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, kF8sLds, configured)) return HK_ERR_LAUNCH;
+    const int grid = min(max_items, moe_num_compute_units());
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), kF8sLds, s, p);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
+// n-tiles of 256 weight rows of the two GEMMs: gate+up (mode 0: 128 h columns = 128 gate + 128 up rows
+// per tile) and down (mode 1).
+static inline int fp8blk_n_tiles(int mode, int N) { return mode == 0 ? N / 128 : (N + 255) / 256; }
 
 struct Fp8Ws {
     size_t ids, w, sorted, offsets, inv, sort_ws, items1, items2, nitems, xq, xs, hq, hs, o, total;
@@ -416,7 +913,9 @@ static Fp8Ws fp8_ws_layout(int T, int H, int I, int E, int k) {
     L.items1 = take((size_t)L.max_items1 * sizeof(MoeItem));
     L.items2 = take((size_t)L.max_items2 * sizeof(MoeItem));
     L.nitems = take(8);
-    L.xq = L.xs = off;   // (the gate+up GEMM gathers the caller's activations in place: no permuted copy)
+    // e4m3 copy of x and its 1 x 128 scales, used only by the bf16-input entry point (the gate+up GEMM
+    // gathers activation rows by token index: there is no permuted copy)
+    L.xq = take((size_t)T * H); L.xs = take((size_t)T * (H / 128) * 4);
     L.hq = take(S * (size_t)I); L.hs = take(S * (size_t)(I / 128) * 4);
     L.o = take(S * (size_t)H * 2);
     L.total = off;
@@ -452,12 +951,34 @@ extern "C" size_t hk_moe_fp8blk_workspace_bytes(int T, int H, int I, int E, int 
     return fp8_ws_layout(T, H, I, E, k).total;
 }
 
-extern "C" int hk_moe_fp8blk_experts_ex(const void* x_e4m3, const float* x_scales, const void* w13,
-                                        const float* w13_scales, const void* w2, const float* w2_scales,
-                                        const float* topk_w, const int32_t* sorted_slots,
-                                        const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
-                                        int T, int H, int I, int E, int k, const void* y_add_bf16_or_null,
-                                        void* workspace, size_t workspace_bytes, void* stream) {
+extern "C" int hk_moe_fp8blk_preshuffle_bytes(int E, int N, int K, int mode, size_t* w_bytes) {
+    if (!w_bytes) return HK_ERR_NULL_POINTER;
+    if (E <= 0 || N <= 0 || K <= 0 || (K % 128) != 0 || (N % 128) != 0 || mode < 0 || mode > 1) return HK_ERR_BAD_SHAPE;
+    *w_bytes = (size_t)E * fp8blk_n_tiles(mode, N) * (K / 128) * kF8sBTile;
+    return HK_OK;
+}
+
+extern "C" int hk_moe_fp8blk_preshuffle(const void* w, int E, int N, int K, int mode, void* out_w, void* stream) {
+    if (!w || !out_w) return HK_ERR_NULL_POINTER;
+    if (E <= 0 || N <= 0 || K <= 0 || (K % 128) != 0 || (N % 128) != 0 || mode < 0 || mode > 1) return HK_ERR_BAD_SHAPE;
+    if (E > 65535 || (long long)2 * N * K >= (1ll << 32)) return HK_ERR_BAD_SHAPE;
+    if (((uintptr_t)w | (uintptr_t)out_w) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    const int n_tiles = fp8blk_n_tiles(mode, N);
+    const long long chunks = (long long)n_tiles * (K / 128) * (kF8sBTile / 16);
+    const long long rows = mode == 0 ? 2ll * N : N;
+    hipLaunchKernelGGL(moe_fp8blk_preshuffle_kernel, dim3((unsigned)((chunks + 255) / 256), E), dim3(256), 0,
+                       (hipStream_t)stream, (const uint8_t*)w, N, K, mode, n_tiles, rows * K, (uint8_t*)out_w);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
+extern "C" int hk_moe_fp8blk_experts_ex2(const void* x_e4m3, const float* x_scales, const void* w13,
+                                         const float* w13_scales, const void* w2, const float* w2_scales,
+                                         const float* topk_w, const int32_t* sorted_slots,
+                                         const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
+                                         int T, int H, int I, int E, int k, int weight_layout,
+                                         const void* y_add_bf16_or_null, void* workspace, size_t workspace_bytes,
+                                         void* stream) {
+    if (weight_layout < 0 || weight_layout > 1) return HK_ERR_UNSUPPORTED;
     if (!x_e4m3 || !x_scales || !w13 || !w13_scales || !w2 || !w2_scales || !topk_w || !sorted_slots ||
         !expert_offsets || !slot_to_pos || !y_bf16)
         return HK_ERR_NULL_POINTER;
@@ -482,7 +1003,12 @@ extern "C" int hk_moe_fp8blk_experts_ex(const void* x_e4m3, const float* x_scale
     p.items = (const MoeItem*)(ws + L.items1); p.num_items = nitems;
     p.out0 = ws + L.hq; p.out_scales = (float*)(ws + L.hs);
     p.K = H; p.N = I; p.n_tiles_n = I / 128;
-    st = launch_fp8blk_gemm<0, true>(p, L.max_items1, s);
+    if (weight_layout == 1) {
+        p.b_expert_stride = (long long)fp8blk_n_tiles(0, I) * (H / 128) * kF8sBTile;
+        st = launch_fp8blk_stream<0, true>(p, L.max_items1, s);
+    } else {
+        st = launch_fp8blk_gemm<0, true>(p, L.max_items1, s);
+    }
     if (st != HK_OK) return st;
 
     MoeFp8Params q{};
@@ -492,9 +1018,25 @@ extern "C" int hk_moe_fp8blk_experts_ex(const void* x_e4m3, const float* x_scale
     q.items = (const MoeItem*)(ws + L.items2); q.num_items = nitems + 1;
     q.out0 = ws + L.o; q.out_scales = nullptr;
     q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
-    st = launch_fp8blk_gemm<1, false>(q, L.max_items2, s);
+    if (weight_layout == 1) {
+        q.b_expert_stride = (long long)fp8blk_n_tiles(1, H) * (I / 128) * kF8sBTile;
+        st = launch_fp8blk_stream<1, false>(q, L.max_items2, s);
+    } else {
+        st = launch_fp8blk_gemm<1, false>(q, L.max_items2, s);
+    }
     if (st != HK_OK) return st;
     return hk_moe_unpermute_add(ws + L.o, topk_w, slot_to_pos, T, k, H, y_add_bf16_or_null, y_bf16, stream);
+}
+
+extern "C" int hk_moe_fp8blk_experts_ex(const void* x_e4m3, const float* x_scales, const void* w13,
+                                        const float* w13_scales, const void* w2, const float* w2_scales,
+                                        const float* topk_w, const int32_t* sorted_slots,
+                                        const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
+                                        int T, int H, int I, int E, int k, const void* y_add_bf16_or_null,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
+    return hk_moe_fp8blk_experts_ex2(x_e4m3, x_scales, w13, w13_scales, w2, w2_scales, topk_w, sorted_slots,
+                                     expert_offsets, slot_to_pos, y_bf16, T, H, I, E, k, 0, y_add_bf16_or_null,
+                                     workspace, workspace_bytes, stream);
 }
 
 extern "C" int hk_moe_fp8blk_experts(const void* x_e4m3, const float* x_scales, const void* w13,
@@ -507,12 +1049,12 @@ extern "C" int hk_moe_fp8blk_experts(const void* x_e4m3, const float* x_scales, 
                                     workspace_bytes, stream);
 }
 
-extern "C" int hk_moe_fp8blk_forward_ex(const void* x_e4m3, const float* x_scales, const float* router_logits,
-                                        const float* router_bias_or_null, int n_group, int topk_group,
-                                        float routed_scale, const void* w13, const float* w13_scales,
-                                        const void* w2, const float* w2_scales, void* y_bf16, int T, int H, int I,
-                                        int E, int k, const void* y_add_bf16_or_null, void* workspace,
-                                        size_t workspace_bytes, void* stream) {
+extern "C" int hk_moe_fp8blk_forward_ex2(const void* x_e4m3, const float* x_scales, const float* router_logits,
+                                         const float* router_bias_or_null, int n_group, int topk_group,
+                                         float routed_scale, const void* w13, const float* w13_scales,
+                                         const void* w2, const float* w2_scales, void* y_bf16, int T, int H, int I,
+                                         int E, int k, int weight_layout, const void* y_add_bf16_or_null,
+                                         void* workspace, size_t workspace_bytes, void* stream) {
     if (!router_logits) return HK_ERR_NULL_POINTER;
     int st = fp8blk_check(T, H, I, E, k);
     if (st != HK_OK) return st;
@@ -525,10 +1067,43 @@ extern "C" int hk_moe_fp8blk_forward_ex(const void* x_e4m3, const float* x_scale
     st = hk_moe_sort((const int32_t*)(ws + L.ids), T, k, E, (int32_t*)(ws + L.sorted), (int32_t*)(ws + L.offsets),
                      (int32_t*)(ws + L.inv), ws + L.sort_ws, hk_moe_sort_workspace_bytes(T, k, E), stream);
     if (st != HK_OK) return st;
-    return hk_moe_fp8blk_experts_ex(x_e4m3, x_scales, w13, w13_scales, w2, w2_scales, (const float*)(ws + L.w),
-                                    (const int32_t*)(ws + L.sorted), (const int32_t*)(ws + L.offsets),
-                                    (const int32_t*)(ws + L.inv), y_bf16, T, H, I, E, k, y_add_bf16_or_null,
-                                    workspace, workspace_bytes, stream);
+    return hk_moe_fp8blk_experts_ex2(x_e4m3, x_scales, w13, w13_scales, w2, w2_scales, (const float*)(ws + L.w),
+                                     (const int32_t*)(ws + L.sorted), (const int32_t*)(ws + L.offsets),
+                                     (const int32_t*)(ws + L.inv), y_bf16, T, H, I, E, k, weight_layout,
+                                     y_add_bf16_or_null, workspace, workspace_bytes, stream);
+}
+
+extern "C" int hk_moe_fp8blk_forward_ex(const void* x_e4m3, const float* x_scales, const float* router_logits,
+                                        const float* router_bias_or_null, int n_group, int topk_group,
+                                        float routed_scale, const void* w13, const float* w13_scales,
+                                        const void* w2, const float* w2_scales, void* y_bf16, int T, int H, int I,
+                                        int E, int k, const void* y_add_bf16_or_null, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
+    return hk_moe_fp8blk_forward_ex2(x_e4m3, x_scales, router_logits, router_bias_or_null, n_group, topk_group,
+                                     routed_scale, w13, w13_scales, w2, w2_scales, y_bf16, T, H, I, E, k, 0,
+                                     y_add_bf16_or_null, workspace, workspace_bytes, stream);
+}
+
+extern "C" int hk_moe_fp8blk_forward_bf16(const void* x_bf16, const float* router_logits,
+                                          const float* router_bias_or_null, int n_group, int topk_group,
+                                          float routed_scale, const void* w13, const float* w13_scales,
+                                          const void* w2, const float* w2_scales, void* y_bf16, int T, int H, int I,
+                                          int E, int k, int weight_layout, const void* y_add_bf16_or_null,
+                                          void* workspace, size_t workspace_bytes, void* stream) {
+    if (!x_bf16) return HK_ERR_NULL_POINTER;
+    int st = fp8blk_check(T, H, I, E, k);
+    if (st != HK_OK) return st;
+    const Fp8Ws L = fp8_ws_layout(T, H, I, E, k);
+    if (!workspace || workspace_bytes < L.total) return HK_ERR_WORKSPACE;
+    if ((uintptr_t)workspace & 15u) return HK_ERR_BAD_ALIGNMENT;
+    uint8_t* ws = (uint8_t*)workspace;
+    // every token is quantized once (T rows), ahead of the gather that repeats it for its k experts
+    st = hk_fp8_quantize_rows_1x128(x_bf16, T, H, ws + L.xq, (float*)(ws + L.xs), stream);
+    if (st != HK_OK) return st;
+    return hk_moe_fp8blk_forward_ex2(ws + L.xq, (const float*)(ws + L.xs), router_logits, router_bias_or_null,
+                                     n_group, topk_group, routed_scale, w13, w13_scales, w2, w2_scales, y_bf16, T,
+                                     H, I, E, k, weight_layout, y_add_bf16_or_null, workspace, workspace_bytes,
+                                     stream);
 }
 
 extern "C" int hk_moe_fp8blk_forward(const void* x_e4m3, const float* x_scales, const float* router_logits,

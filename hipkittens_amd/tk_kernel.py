@@ -439,22 +439,71 @@ def moe_fp8blk_workspace_bytes(T: int, H: int, I: int, E: int, k: int) -> int:
     return int(_lib.load_library().hk_moe_fp8blk_workspace_bytes(T, H, I, E, k))
 
 
-def _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y):
-    _check_tensor(x, "x", _FP8, 2)
-    _check_tensor(x_scales, "x_scales", _F32, 2)
-    _check_tensor(w13, "w13", _FP8, 3)
-    _check_tensor(w13_scales, "w13_scales", _F32, 3)
-    _check_tensor(w2, "w2", _FP8, 3)
-    _check_tensor(w2_scales, "w2_scales", _F32, 3)
+class MoeFp8BlkShuffledWeights:
+    """FP8 block-scaled expert weights in the pre-shuffled tile layout (hk_moe_fp8blk_preshuffle): built
+    once, offline, from the plain [E, 2I, H] / [E, H, I] e4m3 tensors; the fp32 block scales are kept
+    as they are. Pass it as `w13` to the dispatch_moe_fp8blk* functions (w13_scales, w2, w2_scales None)."""
+
+    def __init__(self, w13, w13_scales, w2, w2_scales, E: int, H: int, I: int):
+        self.w13, self.w13_scales, self.w2, self.w2_scales = w13, w13_scales, w2, w2_scales
+        self.E, self.H, self.I = E, H, I
+
+    @staticmethod
+    def _shuffle(w, N: int, K: int, mode: int):
+        import ctypes
+        lib = _lib.load_library()
+        E = w.shape[0]
+        nbytes = ctypes.c_size_t(0)
+        _lib.check(lib.hk_moe_fp8blk_preshuffle_bytes(E, N, K, mode, ctypes.byref(nbytes)), "moe_fp8blk_preshuffle_bytes")
+        out = torch.empty(nbytes.value, dtype=torch.uint8, device=w.device)
+        _lib.check(lib.hk_moe_fp8blk_preshuffle(w.data_ptr(), E, N, K, mode, out.data_ptr(), _stream(w)),
+                   "moe_fp8blk_preshuffle")
+        return out
+
+    @classmethod
+    def from_plain(cls, w13, w13_scales, w2, w2_scales):
+        _check_tensor(w13, "w13", _FP8, 3)
+        _check_tensor(w13_scales, "w13_scales", _F32, 3)
+        _check_tensor(w2, "w2", _FP8, 3)
+        _check_tensor(w2_scales, "w2_scales", _F32, 3)
+        E, twoI, H = w13.shape
+        I = twoI // 2
+        if H % 128 or I % 128 or tuple(w2.shape) != (E, H, I) or \
+                tuple(w13_scales.shape) != (E, twoI // 128, H // 128) or tuple(w2_scales.shape) != (E, H // 128, I // 128):
+            raise RuntimeError("shape mismatch between w13, w13_scales, w2 and w2_scales")
+        return cls(cls._shuffle(w13, I, H, 0), w13_scales, cls._shuffle(w2, H, I, 1), w2_scales, E, H, I)
+
+
+def _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y, x_dtypes=None):
+    """-> (T, H, I, E, weight_layout, w13, w13_scales, w2, w2_scales)"""
+    _check_tensor(x, "x", x_dtypes or _FP8, 2)
+    if x_scales is not None:
+        _check_tensor(x_scales, "x_scales", _F32, 2)
     _check_tensor(y, "y", _BF16, 2)
     T, H = x.shape
-    E, twoI, H2 = w13.shape
-    I = twoI // 2
-    if H2 != H or H % 128 or I % 128 or tuple(w2.shape) != (E, H, I) or tuple(y.shape) != (T, H) or \
-            tuple(x_scales.shape) != (T, H // 128) or tuple(w13_scales.shape) != (E, twoI // 128, H // 128) or \
-            tuple(w2_scales.shape) != (E, H // 128, I // 128):
+    layout = 0
+    if isinstance(w13, MoeFp8BlkShuffledWeights):
+        W = w13
+        w13, w13_scales, w2, w2_scales, layout = W.w13, W.w13_scales, W.w2, W.w2_scales, 1
+        E, I = W.E, W.I
+        if W.H != H:
+            raise RuntimeError("shape mismatch between x and the shuffled weights")
+    else:
+        _check_tensor(w13, "w13", _FP8, 3)
+        _check_tensor(w2, "w2", _FP8, 3)
+        E, twoI, H2 = w13.shape
+        I = twoI // 2
+        if H2 != H or tuple(w2.shape) != (E, H, I):
+            raise RuntimeError("shape mismatch between x, w13 and w2")
+    _check_tensor(w13_scales, "w13_scales", _F32, 3)
+    _check_tensor(w2_scales, "w2_scales", _F32, 3)
+    if H % 128 or I % 128 or tuple(y.shape) != (T, H) or \
+            (x_scales is not None and tuple(x_scales.shape) != (T, H // 128)) or \
+            tuple(w13_scales.shape) != (E, 2 * I // 128, H // 128) or tuple(w2_scales.shape) != (E, H // 128, I // 128):
         raise RuntimeError("shape mismatch between x, x_scales, w13, w13_scales, w2, w2_scales and y")
-    return T, H, I, E
+    if len({t.device for t in (x, w13, w13_scales, w2, w2_scales, y)}) != 1:
+        raise RuntimeError("all tensors must be on the same device")
+    return T, H, I, E, layout, w13, w13_scales, w2, w2_scales
 
 
 def _check_y_add(y_add, y):
@@ -470,7 +519,7 @@ def dispatch_moe_fp8blk_experts(x, x_scales, w13, w13_scales, w2, w2_scales, wei
                                 expert_offsets, slot_to_pos, y, workspace, y_add=None) -> None:
     """FP8 block-scaled expert MLP on routed + sorted tokens (include/hk355.h: hk_moe_fp8blk_experts_ex).
     y_add [T,H] bf16: residual added before the output rounding (a shared expert's output)."""
-    T, H, I, E = _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y)
+    T, H, I, E, layout, w13, w13_scales, w2, w2_scales = _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y)
     p_add = _check_y_add(y_add, y)
     _check_tensor(weights, "weights", _F32, 2)
     _check_tensor(sorted_slots, "sorted_slots", _I32, 1)
@@ -481,10 +530,10 @@ def dispatch_moe_fp8blk_experts(x, x_scales, w13, w13_scales, w2, w2_scales, wei
     if weights.shape[0] != T or sorted_slots.shape[0] != T * k or expert_offsets.shape[0] != E + 1 or \
             slot_to_pos.shape[0] != T * k:
         raise RuntimeError("shape mismatch between routing tensors")
-    st = _lib.load_library().hk_moe_fp8blk_experts_ex(
+    st = _lib.load_library().hk_moe_fp8blk_experts_ex2(
         x.data_ptr(), x_scales.data_ptr(), w13.data_ptr(), w13_scales.data_ptr(), w2.data_ptr(),
         w2_scales.data_ptr(), weights.data_ptr(), sorted_slots.data_ptr(), expert_offsets.data_ptr(),
-        slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, p_add, workspace.data_ptr(), workspace.numel(),
+        slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, layout, p_add, workspace.data_ptr(), workspace.numel(),
         _stream(x))
     _lib.check(st, "dispatch_moe_fp8blk_experts")
 
@@ -506,18 +555,33 @@ def dispatch_moe_fp8blk(x, x_scales, router_logits, router_bias, w13, w13_scales
                         n_group: int, topk_group: int, routed_scale: float, workspace, y_add=None) -> None:
     """Whole FP8 block-scaled MoE layer with group-limited sigmoid routing (router_bias: the
     selection-only score correction). y_add [T,H] bf16: residual added before the output rounding
-    (dispatch_moe_fp8blk_shared_expert's output)."""
-    T, H, I, E = _check_fp8blk(x, x_scales, w13, w13_scales, w2, w2_scales, y)
+    (dispatch_moe_fp8blk_shared_expert's output). `w13` may be a MoeFp8BlkShuffledWeights (then pass None
+    for w13_scales, w2, w2_scales). `x` may be bf16 with x_scales None: the layer then quantizes every
+    token to e4m3 with 1 x 128 scales itself (hk_moe_fp8blk_forward_bf16)."""
+    bf16_in = isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16
+    if bf16_in != (x_scales is None):
+        raise RuntimeError("x_scales must be given for e4m3 activations and None for bf16 activations")
+    T, H, I, E, layout, w13, w13_scales, w2, w2_scales = _check_fp8blk(
+        x, x_scales, w13, w13_scales, w2, w2_scales, y, x_dtypes=_BF16 if bf16_in else None)
     p_add = _check_y_add(y_add, y)
     _check_tensor(router_logits, "router_logits", _F32, 2)
     if router_bias is not None:
         _check_tensor(router_bias, "router_bias", _F32, 1)
+        if router_bias.shape[0] != E:
+            raise RuntimeError("router_bias must be [E]")
     _check_tensor(workspace, "workspace", (torch.uint8,), 1)
     if tuple(router_logits.shape) != (T, E):
         raise RuntimeError("router_logits must be [T, E]")
-    st = _lib.load_library().hk_moe_fp8blk_forward_ex(
-        x.data_ptr(), x_scales.data_ptr(), router_logits.data_ptr(),
-        router_bias.data_ptr() if router_bias is not None else None, int(n_group), int(topk_group),
-        float(routed_scale), w13.data_ptr(), w13_scales.data_ptr(), w2.data_ptr(), w2_scales.data_ptr(),
-        y.data_ptr(), T, H, I, E, int(topk), p_add, workspace.data_ptr(), workspace.numel(), _stream(x))
+    lib = _lib.load_library()
+    p_bias = router_bias.data_ptr() if router_bias is not None else None
+    if bf16_in:
+        st = lib.hk_moe_fp8blk_forward_bf16(
+            x.data_ptr(), router_logits.data_ptr(), p_bias, int(n_group), int(topk_group), float(routed_scale),
+            w13.data_ptr(), w13_scales.data_ptr(), w2.data_ptr(), w2_scales.data_ptr(), y.data_ptr(), T, H, I, E,
+            int(topk), layout, p_add, workspace.data_ptr(), workspace.numel(), _stream(x))
+    else:
+        st = lib.hk_moe_fp8blk_forward_ex2(
+            x.data_ptr(), x_scales.data_ptr(), router_logits.data_ptr(), p_bias, int(n_group), int(topk_group),
+            float(routed_scale), w13.data_ptr(), w13_scales.data_ptr(), w2.data_ptr(), w2_scales.data_ptr(),
+            y.data_ptr(), T, H, I, E, int(topk), layout, p_add, workspace.data_ptr(), workspace.numel(), _stream(x))
     _lib.check(st, "dispatch_moe_fp8blk")

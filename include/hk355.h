@@ -320,6 +320,44 @@ int hk_moe_fp8blk_forward_ex(const void* x_e4m3, const float* x_scales, const fl
                              int E, int k, const void* y_add_bf16_or_null, void* workspace,
                              size_t workspace_bytes, void* stream);
 
+/* Offline pre-shuffle of FP8 block-scaled expert weights (weight_layout = 1 below; no counterpart in
+ * the reference). For every expert, tile of 256 weight rows and K-step of 128 columns the 32 KiB
+ * weight tile is stored contiguously as the MFMA operand fragments of the kernel's four column waves
+ * (1 KiB pieces in lane order), so that the grouped GEMMs load weights from HBM straight into MFMA
+ * operand registers instead of staging them in LDS. mode 0: gate+up matrix [E, 2N, K] with N = I,
+ * K = H; mode 1: down matrix [E, N, K] with N = H, K = I. The fp32 block scales keep their layout.
+ * Requirements: N % 128 == 0, K % 128 == 0, w and out_w 16-byte aligned. */
+int hk_moe_fp8blk_preshuffle_bytes(int E, int N, int K, int mode, size_t* w_bytes);
+int hk_moe_fp8blk_preshuffle(const void* w, int E, int N, int K, int mode, void* out_w, void* stream);
+
+/* hk_moe_fp8blk_experts_ex / hk_moe_fp8blk_forward_ex with a choice of weight layout: 0 = w13 / w2 in
+ * the plain row-major layout, 1 = outputs of hk_moe_fp8blk_preshuffle (the scale tensors are the
+ * plain ones in both cases). Both layouts give bit-identical results; layout 1 is the fast path. */
+int hk_moe_fp8blk_experts_ex2(const void* x_e4m3, const float* x_scales, const void* w13,
+                              const float* w13_scales, const void* w2, const float* w2_scales,
+                              const float* topk_w, const int32_t* sorted_slots,
+                              const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
+                              int T, int H, int I, int E, int k, int weight_layout,
+                              const void* y_add_bf16_or_null, void* workspace, size_t workspace_bytes,
+                              void* stream);
+int hk_moe_fp8blk_forward_ex2(const void* x_e4m3, const float* x_scales, const float* router_logits,
+                              const float* router_bias_or_null, int n_group, int topk_group,
+                              float routed_scale, const void* w13, const float* w13_scales,
+                              const void* w2, const float* w2_scales, void* y_bf16, int T, int H, int I,
+                              int E, int k, int weight_layout, const void* y_add_bf16_or_null,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
+/* The whole layer from bf16 activations x [T, H]: every token is quantized once to e4m3 with 1 x 128
+ * fp32 scales (hk_fp8_quantize_rows_1x128, into the workspace) ahead of the gather that repeats it
+ * for its k experts, then hk_moe_fp8blk_forward_ex2. Same result as quantizing with
+ * hk_fp8_quantize_rows_1x128 and calling hk_moe_fp8blk_forward_ex2. */
+int hk_moe_fp8blk_forward_bf16(const void* x_bf16, const float* router_logits,
+                               const float* router_bias_or_null, int n_group, int topk_group,
+                               float routed_scale, const void* w13, const float* w13_scales,
+                               const void* w2, const float* w2_scales, void* y_bf16, int T, int H, int I,
+                               int E, int k, int weight_layout, const void* y_add_bf16_or_null,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

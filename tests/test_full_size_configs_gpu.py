@@ -88,7 +88,8 @@ def test_moe_fp8blk_full_deepseek_v3_like_shape(hk):
     """The FP8 block-scaled MoE at its benchmark shape: 8192 tokens, hidden 7168, intermediate 2048,
     256 DISTINCT experts (11.3 GB of weights, quantized expert by expert on the device), top-8
     sigmoid routing over 8 groups / top-4 groups: the 65536-slot sort path, the long work-item list
-    and the > 4 GiB weight addressing. Checks: ids and routing weights of all tokens bit-exact against
+    and the > 4 GiB weight addressing, with the weights in the plain and in the pre-shuffled layout
+    (identical bits). Checks: ids and routing weights of all tokens bit-exact against
     the oracle; the layer is equivariant under a permutation of the tokens (bit for bit); y of eight
     sampled tokens against the oracle's forward pass over the experts those tokens use."""
     T, E, k, G_, KG, H, I = 8192, 256, 8, 8, 4, 7168, 2048
@@ -118,13 +119,21 @@ def test_moe_fp8blk_full_deepseek_v3_like_shape(hk):
     assert np.array_equal(ids_d.cpu().numpy(), ids) and np.array_equal(w_d.cpu().numpy(), w)
     assert len(np.unique(ids)) == E
 
+    # weights in the pre-shuffled layout (the fast path; another 11.3 GB): identical bits
+    W = hk.tk_kernel.MoeFp8BlkShuffledWeights.from_plain(w13q, w13s, w2q, w2s)
+    y1 = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_fp8blk(xq, xs, logits, None, W, None, None, None, y1, k, G_, KG, 1.0, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(y1.view(torch.int16), y.view(torch.int16))
+
     # permutation equivariance over tokens
     perm = torch.randperm(T, device=DEV, generator=g)
     y2 = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
     hk.tk_kernel.dispatch_moe_fp8blk(xq[perm].contiguous(), xs[perm].contiguous(), logits[perm].contiguous(), None,
-                                     w13q, w13s, w2q, w2s, y2, k, G_, KG, 1.0, ws)
+                                     W, None, None, None, y2, k, G_, KG, 1.0, ws)
     torch.cuda.synchronize()
     assert torch.equal(y2.view(torch.int16), y[perm].view(torch.int16))
+    del W
 
     # oracle on eight tokens spread over the batch (first and last included)
     sel = np.array([0, 1171, 2342, 3513, 4684, 5855, 7026, T - 1])

@@ -93,6 +93,64 @@ def test_moe_fp8blk_forward_matches_oracle(hk, T, E, k, G, KG, H, I):
     assert err <= TOL, err
 
 
+@pytest.mark.parametrize("T,E,k,G,KG,H,I", CASES + [(40, 4, 2, 2, 1, 2048, 1024), (1, 8, 8, 1, 1, 256, 384),
+                                                     (700, 16, 8, 4, 2, 896, 640)])
+def test_moe_fp8blk_preshuffled_weights_give_identical_bits(hk, T, E, k, G, KG, H, I):
+    """Weights in the pre-shuffled layout (loaded straight into MFMA operand registers, the fast path)
+    against the plain layout (both operands through LDS): same MFMA, same K order, same scaling FMAs,
+    so y must agree bit for bit; the plain path is the one the oracle tests above cover. Includes
+    a single K-step per GEMM, experts without rows, one token, and several items per expert."""
+    print(f"moe_fp8blk preshuffled T={T} E={E} k={k} H={H} I={I}", flush=True)
+    rng = np.random.default_rng(T + E + H + I + 7)
+    xq, xs, w13q, w13s, w2q, w2s = _case(rng, T, E, H, I)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    dev = lambda a: torch.from_numpy(a).to(DEV)
+    X, XS, LG = _fp8(xq), dev(xs), dev(logits)
+    W13, S13, W2, S2 = _fp8(w13q), dev(w13s), _fp8(w2q), dev(w2s)
+    ws = torch.empty(hk.tk_kernel.moe_fp8blk_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=DEV)
+    y0 = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_fp8blk(X, XS, LG, None, W13, S13, W2, S2, y0, k, G, KG, 1.0, ws)
+    torch.cuda.synchronize()
+    W = hk.tk_kernel.MoeFp8BlkShuffledWeights.from_plain(W13, S13, W2, S2)
+    y1 = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ws.fill_(0xFF)
+    hk.tk_kernel.dispatch_moe_fp8blk(X, XS, LG, None, W, None, None, None, y1, k, G, KG, 1.0, ws)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y1.float()).all()
+    assert torch.equal(y0.view(torch.int16), y1.view(torch.int16))
+    # and directly against the oracle
+    ids, w = O.topk_grouped_sigmoid(logits, None, k, G, KG, 1.0)
+    want = F.bf16_to_f32(O.moe_fp8blk_forward(xq, xs, ids, w, w13q, w13s, w2q, w2s))
+    assert GM.rel_fro_error(y1.float().cpu().numpy(), want) <= TOL
+
+
+def test_moe_fp8blk_bf16_activations_are_quantized_once_per_token(hk):
+    """The bf16-input layer = hk_fp8_quantize_rows_1x128 (bit-exact against the oracle, tested above)
+    followed by the e4m3 layer: identical bits, plain and pre-shuffled weights."""
+    T, E, k, G, KG, H, I = 150, 16, 4, 4, 2, 512, 256
+    rng = np.random.default_rng(5)
+    _, _, w13q, w13s, w2q, w2s = _case(rng, 1, E, H, I)
+    x = torch.from_numpy(rng.standard_normal((T, H)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    logits = torch.from_numpy(rng.standard_normal((T, E)).astype(np.float32)).to(DEV)
+    dev = lambda a: torch.from_numpy(a).to(DEV)
+    W13, S13, W2, S2 = _fp8(w13q), dev(w13s), _fp8(w2q), dev(w2s)
+    xq = torch.zeros((T, H), dtype=torch.uint8, device=DEV)
+    xs = torch.zeros((T, H // 128), dtype=torch.float32, device=DEV)
+    hk.tk_kernel.dispatch_fp8_quantize_rows_1x128(x, xq, xs)
+    ws = torch.empty(hk.tk_kernel.moe_fp8blk_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=DEV)
+    y0 = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_fp8blk(xq.view(torch.float8_e4m3fn), xs, logits, None, W13, S13, W2, S2, y0, k, G, KG, 1.0, ws)
+    torch.cuda.synchronize()
+    for weights in ((W13, S13, W2, S2), (hk.tk_kernel.MoeFp8BlkShuffledWeights.from_plain(W13, S13, W2, S2), None, None, None)):
+        y1 = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ws.fill_(0xFF)
+        hk.tk_kernel.dispatch_moe_fp8blk(x, None, logits, None, *weights, y1, k, G, KG, 1.0, ws)
+        torch.cuda.synchronize()
+        assert torch.equal(y0.view(torch.int16), y1.view(torch.int16))
+    with pytest.raises(RuntimeError):   # bf16 activations come without scales, e4m3 ones with
+        hk.tk_kernel.dispatch_moe_fp8blk(x, xs, logits, None, W13, S13, W2, S2, y1, k, G, KG, 1.0, ws)
+
+
 @pytest.mark.parametrize("T,E,k,G,KG,H,I,IS", [(64, 8, 2, 4, 2, 256, 128, 256), (200, 32, 8, 8, 4, 1024, 256, 128)])
 def test_moe_fp8blk_with_shared_expert_matches_oracle(hk, T, E, k, G, KG, H, I, IS):
     """DeepSeek-V3 layer: routed experts (selection-only score bias) + a shared expert of
