@@ -250,6 +250,31 @@ def bench_mxfp4(torch, hk, n, warmup, iters, dev):
             "roofline": _roofline("mfma", tf, PEAK_FP4, "TFLOP/s", "mxfp4 256x256x256 tile kernel", _traffic("mxfp4_gemm"))}
 
 
+def bench_schedules(torch, hk, n, warmup, iters, dev):
+    """The two schedules of the 256x256-tile GEMMs side by side (kernels/gemm/fp8fp32/README.md:3-5 names both
+    for the reference): 4 waves with hand-interleaved slots (one wave per SIMD; what the library picks) and
+    8 waves in two ping-pong groups (two waves per SIMD). Same tile format, identical bits."""
+    out = {}
+    g = torch.Generator(device=dev).manual_seed(0)
+    a = torch.randn(n, n, device=dev, generator=g)
+    b = torch.randn(n, n, device=dev, generator=g)
+    C = torch.empty(n, n, dtype=torch.bfloat16, device=dev)
+    tf = lambda ms: round(2.0 * n ** 3 / (ms * 1e-3) / 1e12, 1)
+    A8, sa = hk.quant.quantize_fp8_per_tensor(a)
+    B8, sb = hk.quant.quantize_fp8_per_tensor(b)
+    out["fp8"] = {name: tf(_timeit(torch, lambda: hk.tk_kernel.dispatch_fp8_gemm(A8, B8, C, sa, sb, variant=v), warmup, iters)[1])
+                  for name, v in (("4wave_interleave", 4), ("8wave_pingpong", 1))}
+    Ab, Bb = a.to(torch.bfloat16), b.to(torch.bfloat16)
+    out["bf16"] = {name: tf(_timeit(torch, lambda: hk.tk_kernel.dispatch_bf16_gemm(Ab, Bb, C, variant=v), warmup, iters)[1])
+                   for name, v in (("4wave_interleave", 1), ("8wave_pingpong", 4))}
+    Ap, As = hk.quant.quantize_mxfp4(a)
+    Bp, Bs = hk.quant.quantize_mxfp4(b)
+    out["mxfp4"] = {name: tf(_timeit(torch, lambda: hk.tk_kernel.dispatch_mxfp4_gemm(Ap, As, Bp, Bs, C, variant=v), warmup, iters)[1])
+                    for name, v in (("4wave_interleave", 1), ("8wave_pingpong", 4))}
+    out["workload"] = f"M=N=K={n}, TFLOP/s"
+    return out
+
+
 # ------------------------------------------------------------------------------------- MoE layers
 def bench_moe_mxfp4(torch, hk, warmup, iters, dev, graph=True):
     import numpy as np
@@ -497,8 +522,8 @@ def mfma_ceiling(torch, Aq, dev):
     return blocks * 8 * iters * 32 * 65536.0 / (ms * 1e-3) / 1e12
 
 
-LEGS = ("ceiling", "sweep", "reference_inputs", "decode", "bf16", "library", "mxfp4", "mxfp4_decode", "moe_mxfp4",
-        "moe_fp8blk", "routing")
+LEGS = ("ceiling", "sweep", "reference_inputs", "decode", "bf16", "library", "mxfp4", "mxfp4_decode", "schedules",
+        "moe_mxfp4", "moe_fp8blk", "routing")
 
 
 def main() -> int:
@@ -594,6 +619,9 @@ def main() -> int:
         extra["mxfp4_gemm"] = bench_mxfp4(torch, hk, 8192, 500, 100, dev)
     if "mxfp4_decode" in legs:
         extra["mxfp4_gemm_decode"] = bench_mxfp4_decode(torch, hk, 50, 50, dev)
+    if "schedules" in legs:
+        extra["gemm_schedules_8192"] = bench_schedules(torch, hk, 8192, 200, 100, dev)
+        torch.cuda.empty_cache()
     if "moe_mxfp4" in legs:
         extra["moe_mxfp4"] = bench_moe_mxfp4(torch, hk, quick_w, quick_i, dev, graph=not args.no_graph)
         torch.cuda.empty_cache()

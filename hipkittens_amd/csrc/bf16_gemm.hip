@@ -10,6 +10,7 @@
 // two v_mfma_f32_16x16x32_bf16 (16 cycles each, together as long as one FP8 MFMA).
 #include "gemm_tile.h"
 #include "gemm_small_tile.h"
+#include "gemm_pingpong.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -138,8 +139,9 @@ __global__ __launch_bounds__(256) void bf16_gemm_4wave_ring_kernel(
     // B ring positions (byte offsets): tile kt+1 is read from off1, tile kt+2 is loaded to off2.
     uint32_t off1 = kTileBytes, off2 = 2 * kTileBytes;
 
-    // One K-step with A slot / fragment parity P. Every step runs the same code (see the
-    // kernel above for how the tail is kept uniform).
+    // One K-step with A slot / fragment parity P. Every step runs the same code (refills past the end
+    // of K go against a zero-sized buffer, the last step's prefetch reads are never used: see
+    // fp8_gemm_4wave_ring_kernel).
     auto step = [&]<int P>(int kt) {
         const uint32_t k2 = (uint32_t)(kt + 2) * BK;
         v4i sa = srd_a, sb = srd_b;
@@ -274,6 +276,28 @@ __global__ __launch_bounds__(256) void bf16_gemm_small_tile_kernel(
                                                              partial);
 }
 
+// 8-wave ping-pong kernel (gemm_pingpong.h) with the bf16 MFMA: the schedule of the reference's flagship
+// kernel (kernels/gemm/bf16fp32/mi325x/256_256_64_16.cpp:73-155). K: the operands' row length in bytes.
+template <bool EDGE>
+__global__ __launch_bounds__(512) void bf16_gemm_pingpong_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n, int band_n) {
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    gemm_pingpong_body<Bf16Mma, EDGE>(smem, A, B, C, M, N, K, alpha, tiles_m, tiles_n, band_n);
+}
+
+template <bool EDGE>
+static int launch_bf16_pingpong(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream) {
+    auto kern = bf16_gemm_pingpong_kernel<EDGE>;
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, kPpLdsBytes, configured)) return HK_ERR_LAUNCH;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(512), kPpLdsBytes, stream, (const uint8_t*)A,
+                       (const uint8_t*)B, (uint16_t*)C, M, N, 2 * K, 1.0f, tiles_m, tiles_n,
+                       raster_band(((long long)M + N) * K * 2, tiles_n));
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
 template <int TILE, int STAGES, bool EDGE>
 static int launch_bf16_small_tile(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream) {
     auto kern = bf16_gemm_small_tile_kernel<TILE, STAGES, EDGE, false>;
@@ -315,7 +339,7 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 8) != 0) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < 0 || variant > 3) return HK_ERR_UNSUPPORTED;
+    if (variant < 0 || variant > 4) return HK_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {
         if ((long long)((M + 63) / 64) > 65535) return HK_ERR_BAD_SHAPE;
@@ -336,6 +360,8 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
                       : launch_bf16_small_tile<kTinyTile, kTinyStages, false>(A, B, C, M, N, K, s);
     }
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
+    if (variant == 4)
+        return edge ? launch_bf16_pingpong<true>(A, B, C, M, N, K, s) : launch_bf16_pingpong<false>(A, B, C, M, N, K, s);
     return edge ? launch_bf16_ring<true>(A, B, C, M, N, K, s) : launch_bf16_ring<false>(A, B, C, M, N, K, s);
 }
 

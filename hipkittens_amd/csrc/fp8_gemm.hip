@@ -4,293 +4,30 @@
 // schedules, kernels/gemm/fp8fp32/README.md:3-21); helper layer studied:
 // kernels/gemm/fp8fp32/FP8_4wave/utils.cpp:23-174.
 //
-// Tile kernel: one workgroup owns a 256x256 tile of C and walks K in steps of 128.
-// A and B tiles (256 rows x 128 bytes each) are fetched with direct global->LDS
-// loads into a two-stage ring of swizzled LDS tiles; each wave reads its operand
-// fragments with ds_read_b128 and issues v_mfma_f32_16x16x128_f8f6f4.
-// The MFMA is issued with the operand roles swapped (B rows as the "A" operand) so
-// that a lane's 4 accumulator values are 4 consecutive columns of one C row, and
-// the B tile's rows are permuted on their way into LDS so that two neighbouring
-// MFMA tiles give a lane 8 consecutive columns = one 16-byte bf16 store.
+// Tile kernels: one workgroup owns a 256x256 tile of C and walks K in steps of 128. A and B tiles
+// (256 rows x 128 bytes each) are fetched with direct global->LDS loads into swizzled LDS tiles; each
+// wave reads its operand fragments with ds_read_b128 and issues v_mfma_f32_16x16x128_f8f6f4. The MFMA
+// is issued with the operand roles swapped (B rows as the "A" operand) so that a lane's 4 accumulator
+// values are 4 consecutive columns of one C row, and the B tile's rows are permuted on their way into
+// LDS so that two neighbouring MFMA tiles give a lane 8 consecutive columns = one 16-byte bf16 store.
+// Two schedules, as in the reference: 4 waves with hand-interleaved slots (fp8_gemm_4wave_ring_kernel,
+// the default) and 8 waves in two ping-pong groups (gemm_pingpong.h).
 #include "gemm_tile.h"
 #include "gemm_small_tile.h"
+#include "gemm_pingpong.h"
 #include "../../include/hk355.h"
 
 namespace hk {
-}
-
-namespace hk {
-
-template <int WM, int WN, bool EDGE>
-__global__ __launch_bounds__(WM * WN * 64) void fp8_gemm_tile_kernel(
-    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, float alpha, int tiles_m, int tiles_n, int band_n) {
-    constexpr int NW = WM * WN;
-    constexpr int TM = BM / WM, TN = BN / WN;  // per-wave tile of C
-    constexpr int MT = TM / 16, NT = TN / 16;  // MFMA tiles per wave
-    constexpr int NDMA = kTileBytes / (NW * 1024);  // loads per wave per operand per K-step
-    static_assert(NT % 2 == 0, "column pairs");
-    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
-
-    const int lane = lane_id();
-    const int w = wave_id();
-    const int wm = w / WN, wn = w % WN;
-
-    int pm, pn;
-    {
-        const int num_wg = tiles_m * tiles_n;
-        const int id = xcd_chunk_order(blockIdx.x, num_wg, kCuPerXcd);
-        banded_raster(id, tiles_m, tiles_n, 4, band_n, pm, pn);
-    }
-    const int row0 = pm * BM, col0 = pn * BN;
-
-    // ---- global -> LDS addressing -------------------------------------------------
-    const uint8_t* a_base = A + (size_t)row0 * K;
-    const uint8_t* b_base = B + (size_t)col0 * K;
-    const int a_rows = min(M - row0, BM), b_rows = min(N - col0, BN);
-    const v4i srd_a = make_srd(a_base, (uint32_t)a_rows * (uint32_t)K);
-    const v4i srd_b = make_srd(b_base, (uint32_t)b_rows * (uint32_t)K);
-
-    // Load i of this wave fills LDS rows 8*(i*NW + w) .. +8 of the tile; lane l lands
-    // in row +l/8, physical chunk l%8, and therefore fetches logical chunk
-    // swz(row, l%8) (the swizzle is an involution).
-    uint32_t voff_a[EDGE ? NDMA : 1], voff_b[EDGE ? NDMA : 1];
-    {
-#pragma unroll
-        for (int i = 0; i < (EDGE ? NDMA : 1); ++i) {
-            const int R = 8 * (i * NW + w) + (lane >> 3);
-            const uint32_t c = swz_chunk(R, lane & 7);
-            int ra = R, rb = b_row_to_col(R);
-            if (EDGE) {
-                ra = min(ra, a_rows - 1);
-                rb = min(rb, b_rows - 1);
-            }
-            voff_a[i] = (uint32_t)ra * (uint32_t)K + c * 16u;
-            voff_b[i] = (uint32_t)rb * (uint32_t)K + c * 16u;
-        }
-    }
-    const uint32_t dma_row_stride = to_sgpr((uint32_t)(8 * NW) * (uint32_t)K);
-    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
-    const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-
-    auto issue_tile = [&](int stage, int kt) {
-        const uint32_t k0 = (uint32_t)kt * BK;
-        const uint32_t dst = lds_wave + (uint32_t)stage * kStageBytes;
-#pragma unroll
-        for (int i = 0; i < NDMA; ++i) {
-            if (EDGE)
-                dma16(srd_a, dst + i * NW * 1024, voff_a[i], k0);
-            else
-                dma16(srd_a, dst + i * NW * 1024, voff_a[0], k0 + i * dma_row_stride);
-        }
-#pragma unroll
-        for (int i = 0; i < NDMA; ++i) {
-            if (EDGE)
-                dma16(srd_b, dst + kTileBytes + i * NW * 1024, voff_b[i], k0);
-            else
-                dma16(srd_b, dst + kTileBytes + i * NW * 1024, voff_b[0], k0 + i * dma_row_stride);
-        }
-    };
-
-    // ---- LDS -> register addressing -----------------------------------------------
-    const uint32_t r = lane & 15, g = lane >> 4;
-    const uint32_t rd_lo = r * 128u + swz_chunk(r, g) * 16u;
-    const uint32_t rd_hi = r * 128u + swz_chunk(r, g + 4) * 16u;
-    uint32_t a_lo = lds0 + wm * (TM * BK) + rd_lo, a_hi = lds0 + wm * (TM * BK) + rd_hi;
-    uint32_t b_lo = lds0 + kTileBytes + wn * (TN * BK) + rd_lo;
-    uint32_t b_hi = lds0 + kTileBytes + wn * (TN * BK) + rd_hi;
-
-    v4f acc[MT][NT];
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
-
-    const int nk = K / BK;
-    issue_tile(0, 0);
-    for (int kt = 0; kt < nk; ++kt) {
-        wait_vmcnt<0>();
-        block_barrier();
-        if (kt + 1 < nk) issue_tile((kt + 1) & 1, kt + 1);
-
-        v8i bf[NT];
-#pragma unroll
-        for (int n = 0; n < NT; ++n) bf[n] = lds_frag(b_lo, b_hi, n * 16 * BK);
-#pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            const v8i af = lds_frag(a_lo, a_hi, m * 16 * BK);
-#pragma unroll
-            for (int n = 0; n < NT; ++n) acc[m][n] = mfma_fp8_16x16x128(bf[n], af, acc[m][n]);
-        }
-        a_lo ^= kStageBytes; a_hi ^= kStageBytes;
-        b_lo ^= kStageBytes; b_hi ^= kStageBytes;
-    }
-
-    store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
-}
-
-// ---------------------------------------------------------------------------------------
-// 4-wave interleaved kernel: one wave per SIMD, each owning a 128x128 patch of the 256x256
-// tile (8x8 MFMA tiles, 256 accumulator registers). Every LDS read, global->LDS load and
-// MFMA has a fixed place in the instruction stream (one MFMA per "slot", memory operations
-// attached to slots) so that operand fragments for the next MFMA group and the next K-step
-// are in flight while the matrix pipe works:
-//   groups 0..PG   : MFMAs with A fragment m; LDS read of A fragment m+3 (4 rotating buffers)
-//   after group PG : all reads of this stage are issued -> wait for the next tile's loads,
-//                    one barrier, then refill this stage with tile kt+2
-//   groups PG+1..7 : MFMAs; LDS reads of the next K-step's B fragments and first A fragments.
-// Schedule idea after the reference's 4-wave kernel (kernels/gemm/fp8fp32/README.md:3-5,
-// per-instruction helpers in FP8_4wave/utils.cpp:44-52, 131-137, 150-161).
-template <bool EDGE>
-__global__ __launch_bounds__(256) void fp8_gemm_4wave_kernel(
-    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, float alpha, int tiles_m, int tiles_n, int band_n) {
-    constexpr int NW = 4, TM = 128, TN = 128, MT = 8, NT = 8;
-    constexpr int NDMA = kTileBytes / (NW * 1024);  // 8 loads per wave per operand per K-step
-    constexpr int PG = 4;                            // barrier sits after MFMA group PG
-    constexpr int AD = 3;                            // A fragments are read AD groups ahead
-    static_assert(PG == 4 && AD == 3 && MT == 8, "slot plan below is written for these");
-    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
-
-    const int lane = lane_id();
-    const int w = wave_id();
-    const int wm = w >> 1, wn = w & 1;
-
-    int pm, pn;
-    {
-        const int id = xcd_chunk_order(blockIdx.x, tiles_m * tiles_n, kCuPerXcd);
-        banded_raster(id, tiles_m, tiles_n, 4, band_n, pm, pn);
-    }
-    const int row0 = pm * BM, col0 = pn * BN;
-
-    const int a_rows = min(M - row0, BM), b_rows = min(N - col0, BN);
-    const v4i srd_a = make_srd(A + (size_t)row0 * K, (uint32_t)a_rows * (uint32_t)K);
-    const v4i srd_b = make_srd(B + (size_t)col0 * K, (uint32_t)b_rows * (uint32_t)K);
-
-    uint32_t voff_a[EDGE ? NDMA : 1], voff_b[EDGE ? NDMA : 1];
-#pragma unroll
-    for (int i = 0; i < (EDGE ? NDMA : 1); ++i) {
-        const int R = 8 * (i * NW + w) + (lane >> 3);
-        const uint32_t c = swz_chunk(R, lane & 7);
-        int ra = R, rb = b_row_to_col(R);
-        if (EDGE) {
-            ra = min(ra, a_rows - 1);
-            rb = min(rb, b_rows - 1);
-        }
-        voff_a[i] = (uint32_t)ra * (uint32_t)K + c * 16u;
-        voff_b[i] = (uint32_t)rb * (uint32_t)K + c * 16u;
-    }
-    const uint32_t dma_row_stride = to_sgpr((uint32_t)(8 * NW) * (uint32_t)K);
-    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
-    const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-
-    // One global->LDS load: operand op (0 = A, 1 = B), load index i, into `stage`.
-    auto dma_one = [&](int op, int i, int stage, uint32_t k0, v4i srd) {
-        const uint32_t dst = lds_wave + (uint32_t)stage * kStageBytes + op * kTileBytes + i * NW * 1024;
-        if (EDGE)
-            dma16(srd, dst, op ? voff_b[i] : voff_a[i], k0);
-        else
-            dma16(srd, dst, op ? voff_b[0] : voff_a[0], k0 + i * dma_row_stride);
-    };
-
-    const uint32_t r = lane & 15, g = lane >> 4;
-    const uint32_t rd_lo = r * 128u + swz_chunk(r, g) * 16u;
-    const uint32_t rd_hi = r * 128u + swz_chunk(r, g + 4) * 16u;
-    uint32_t a_lo[2], a_hi[2], b_lo[2], b_hi[2];
-#pragma unroll
-    for (int st = 0; st < 2; ++st) {
-        a_lo[st] = lds0 + st * kStageBytes + wm * (TM * BK) + rd_lo;
-        a_hi[st] = lds0 + st * kStageBytes + wm * (TM * BK) + rd_hi;
-        b_lo[st] = lds0 + st * kStageBytes + kTileBytes + wn * (TN * BK) + rd_lo;
-        b_hi[st] = lds0 + st * kStageBytes + kTileBytes + wn * (TN * BK) + rd_hi;
-    }
-
-    v4f acc[MT][NT];
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
-    v8i bf[2][NT];  // B fragments of the current / next K-step
-    v8i af[4];      // rotating A fragments
-
-    const int nk = K / BK;
-
-    // ---- prologue: tile 0 (and 1) in flight, first fragments in registers -----------------
-#pragma unroll
-    for (int i = 0; i < NDMA; ++i) dma_one(0, i, 0, 0, srd_a);
-#pragma unroll
-    for (int i = 0; i < NDMA; ++i) dma_one(1, i, 0, 0, srd_b);
-    wait_vmcnt<0>();
-    block_barrier();
-    if (nk > 1) {
-#pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma_one(0, i, 1, BK, srd_a);
-#pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma_one(1, i, 1, BK, srd_b);
-    }
-#pragma unroll
-    for (int n = 0; n < NT; ++n) bf[0][n] = lds_frag(b_lo[0], b_hi[0], n * 16 * BK);
-#pragma unroll
-    for (int m = 0; m < AD; ++m) af[m] = lds_frag(a_lo[0], a_hi[0], m * 16 * BK);
-
-    // One K-step with stage/parity P. Every step runs the same code: the last step's
-    // prefetch reads return stale LDS contents that are never used, and refills past the
-    // end of K are issued against a zero-sized buffer (out of range for every lane, no
-    // memory traffic), so that no step needs a differently scheduled body.
-    auto step = [&]<int P>(int kt) {
-        const uint32_t k2 = (uint32_t)(kt + 2) * BK;
-        v4i sa = srd_a, sb = srd_b;
-        if (kt + 2 >= nk) { sa.z = 0; sb.z = 0; }
-#pragma unroll
-        for (int m = 0; m < MT; ++m) {
-#pragma unroll
-            for (int n = 0; n < NT; ++n) {
-                mfma_fp8_16x16x128_acc(acc[m][n], bf[P][n], af[m & 3]);
-                if (m <= PG) {
-                    // A fragment m+AD, early in the group
-                    if (n == 0) af[(m + AD) & 3] = lds_frag(a_lo[P], a_hi[P], (m + AD) * 16 * BK);
-                } else {
-                    const int j = (m - PG - 1) * NT + n;  // slot index after the barrier
-                    if (j < NT) {
-                        bf[P ^ 1][j] = lds_frag(b_lo[P ^ 1], b_hi[P ^ 1], j * 16 * BK);
-                    } else if (j == NT || j == NT + 1) {
-                        // buffers 0 and 1 were last used by groups PG and PG+1
-                        af[j - NT] = lds_frag(a_lo[P ^ 1], a_hi[P ^ 1], (j - NT) * 16 * BK);
-                    } else if (j == 2 * NT) {
-                        // buffer 2 is in use until group PG+2 has been issued
-                        af[2] = lds_frag(a_lo[P ^ 1], a_hi[P ^ 1], 2 * 16 * BK);
-                    }
-                    if (j < 2 * NDMA) dma_one(j / NDMA, j % NDMA, P, k2, j / NDMA ? sb : sa);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if (m == PG) {
-                // every read of stage P by this wave has been issued; once they have returned
-                // and the next tile has landed for all waves, stage P may be refilled
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                wait_vmcnt<0>();
-                block_barrier();
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-    };
-
-    int kt = 0;
-    for (; kt + 1 < nk; kt += 2) {
-        step.template operator()<0>(kt);
-        step.template operator()<1>(kt + 1);
-    }
-    if (kt < nk) step.template operator()<0>(kt);
-    wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
-    mfma_drain();
-
-    store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
-}
 
 // ---------------------------------------------------------------------------------------
 // 4-wave kernel with a five-slot LDS ring (all 160 KiB): two slots for A tiles, three for B
-// tiles. Same fragment plan as the kernel above, but the global->LDS loads are spread over
-// the whole K-step instead of being bunched behind the barrier: the address unit of a CU
+// tiles. One wave per SIMD, each owning a 128x128 patch of the 256x256 tile (8x8 MFMA tiles, 256
+// accumulator registers); every LDS read, global->LDS load and MFMA has a fixed place in the
+// instruction stream (one MFMA per "slot", memory operations attached to slots): A fragment m + 3 is
+// read while the MFMAs of fragment m issue, the next K-step's B fragments after the single barrier per
+// K-step (schedule idea after the reference's 4-wave kernel, kernels/gemm/fp8fp32/README.md:3-5,
+// per-instruction helpers in FP8_4wave/utils.cpp:44-52, 131-137, 150-161). The global->LDS loads are
+// spread over the whole K-step instead of being bunched behind the barrier: the address unit of a CU
 // needs 16 cycles per 1 KiB load, 16 loads per wave and step, and a wave that cannot hand
 // its load over also cannot issue its next MFMA. B fragments of tile kt are read one step
 // early (after barrier kt-1), so with a third B slot tile kt+2 of B may be fetched during
@@ -412,8 +149,10 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
     // B ring positions (byte offsets): tile kt+1 is read from off1, tile kt+2 is loaded to off2.
     uint32_t off1 = kTileBytes, off2 = 2 * kTileBytes;
 
-    // One K-step with A slot / fragment parity P. Every step runs the same code (see the
-    // kernel above for how the tail is kept uniform).
+    // One K-step with A slot / fragment parity P. Every step runs the same code: the last step's
+    // prefetch reads return stale LDS contents that are never used, and refills past the end of K
+    // are issued against a zero-sized buffer (out of range for every lane, no memory traffic), so
+    // that no step needs a differently scheduled body.
     auto step = [&]<int P>(int kt) {
         const uint32_t k2 = (uint32_t)(kt + 2) * BK;
         v4i sa = srd_a, sb = srd_b;
@@ -475,6 +214,16 @@ struct Fp8Mma {
         acc = mfma_fp8_16x16x128(b, a, acc);
     }
 };
+// 8-wave ping-pong kernel (gemm_pingpong.h) with the FP8 MFMA: the reference's second FP8 schedule
+// (kernels/gemm/fp8fp32/README.md:3-5).
+template <bool EDGE>
+__global__ __launch_bounds__(512) void fp8_gemm_pingpong_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n, int band_n) {
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    gemm_pingpong_body<Fp8Mma, EDGE>(smem, A, B, C, M, N, K, alpha, tiles_m, tiles_n, band_n);
+}
+
 template <int TILE, int STAGES, bool EDGE, bool SPLIT>
 __global__ __launch_bounds__(256) void fp8_gemm_small_tile_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
@@ -539,16 +288,15 @@ __global__ __launch_bounds__(256) void fp8_gemm_portable_kernel(
     }
 }
 
-template <int WM, int WN, bool EDGE>
-static int launch_tile(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
-                       hipStream_t stream) {
-    auto kern = fp8_gemm_tile_kernel<WM, WN, EDGE>;
+template <bool EDGE>
+static int launch_pingpong(const void* A, const void* B, void* C, int M, int N, int K, float alpha, hipStream_t stream) {
+    auto kern = fp8_gemm_pingpong_kernel<EDGE>;
     static DeviceOnce configured;
-    if (!set_lds_limit_once((const void*)kern, kLdsBytes, configured)) return HK_ERR_LAUNCH;
+    if (!set_lds_limit_once((const void*)kern, kPpLdsBytes, configured)) return HK_ERR_LAUNCH;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(WM * WN * 64), kLdsBytes, stream,
-                       (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m,
-                       tiles_n, raster_band(((long long)M + N) * K, tiles_n));
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(512), kPpLdsBytes, stream, (const uint8_t*)A,
+                       (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m, tiles_n,
+                       raster_band(((long long)M + N) * K, tiles_n));
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
@@ -574,11 +322,11 @@ static int launch_tile128_splitk(const void* A, const void* B, void* C, int M, i
                                     B, C, M, N, K, alpha, splits, partial, stream);
 }
 
-template <bool EDGE, bool RING>
+template <bool EDGE>
 static int launch_4wave(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                         hipStream_t stream) {
-    auto kern = RING ? fp8_gemm_4wave_ring_kernel<EDGE> : fp8_gemm_4wave_kernel<EDGE>;
-    constexpr int lds_bytes = RING ? 5 * kTileBytes : kLdsBytes;
+    auto kern = fp8_gemm_4wave_ring_kernel<EDGE>;
+    constexpr int lds_bytes = 5 * kTileBytes;
     static DeviceOnce configured;
     if (!set_lds_limit_once((const void*)kern, lds_bytes, configured)) return HK_ERR_LAUNCH;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
@@ -596,10 +344,9 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 16) != 0) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < 0 || variant > 6) return HK_ERR_UNSUPPORTED;
-    // K tails: the ring kernel (4) and the small-tile kernels (5, 6) take any K % 16 == 0
+    if (variant < 0 || variant > 6 || variant == 2 || variant == 3) return HK_ERR_UNSUPPORTED;
+    // K tails: the tile kernels zero-fill the last K-step of any K % 16 == 0
     if (variant != 0 && (long long)K * BM >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
-    if (variant >= 1 && variant <= 3 && (K % BK) != 0) return HK_ERR_BAD_SHAPE;
     const float alpha = scale_a * scale_b;
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {
@@ -621,16 +368,8 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
     }
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
     if (variant == 1)
-        return edge ? launch_tile<2, 4, true>(A, B, C, M, N, K, alpha, s)
-                    : launch_tile<2, 4, false>(A, B, C, M, N, K, alpha, s);
-    if (variant == 3)
-        return edge ? launch_tile<2, 2, true>(A, B, C, M, N, K, alpha, s)
-                    : launch_tile<2, 2, false>(A, B, C, M, N, K, alpha, s);
-    if (variant == 4)
-        return edge ? launch_4wave<true, true>(A, B, C, M, N, K, alpha, s)
-                    : launch_4wave<false, true>(A, B, C, M, N, K, alpha, s);
-    return edge ? launch_4wave<true, false>(A, B, C, M, N, K, alpha, s)
-                : launch_4wave<false, false>(A, B, C, M, N, K, alpha, s);
+        return edge ? launch_pingpong<true>(A, B, C, M, N, K, alpha, s) : launch_pingpong<false>(A, B, C, M, N, K, alpha, s);
+    return edge ? launch_4wave<true>(A, B, C, M, N, K, alpha, s) : launch_4wave<false>(A, B, C, M, N, K, alpha, s);
 }
 
 extern "C" size_t hk_fp8_gemm_workspace_bytes(int M, int N, int K) {

@@ -19,6 +19,7 @@
 // MFMA reads.
 #include "gemm_tile.h"
 #include "gemm_small_tile.h"
+#include "gemm_pingpong.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -181,7 +182,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     for (int n = 0; n < NT; ++n) shift_scale(bs[0][n]);
     shift_scale(as[0]);  // as[1], as[2] are shifted inside the first step (groups 0 and 1)
 
-    // One K-step (see the FP8 4-wave kernel for the slot plan). Scale handling: the raw
+    // One K-step (slot plan of fp8_gemm_4wave_ring_kernel, fp8_gemm.hip, over two LDS stages). Scale handling: the raw
     // 8 bytes of a fragment are read together with the fragment; the shift that exposes
     // this lane's byte is placed well after the read (B: group 7; A fragment f: group f-1).
     auto step = [&]<int P>(int kt) {
@@ -385,6 +386,31 @@ static int launch_mxfp4_splitk(const void* A, const void* SA, const void* B, con
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
+// 8-wave ping-pong kernel (gemm_pingpong.h) with the scaled FP4 MFMA. K: the operands' row length in bytes.
+template <bool EDGE>
+__global__ __launch_bounds__(512) void mxfp4_gemm_pingpong_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
+    const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int sa_pitch,
+    int sb_pitch, int tiles_m, int tiles_n, int band_n) {
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    gemm_pingpong_body<Mxfp4Mma, EDGE>(smem, A, B, C, M, N, K, 1.0f, tiles_m, tiles_n, band_n,
+                                       SmallTileScales{SA, SB, sa_pitch, sb_pitch});
+}
+
+template <bool EDGE>
+static int launch_mxfp4_pingpong(const void* A, const void* SA, const void* B, const void* SB, void* C,
+                                 int M, int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
+    auto kern = mxfp4_gemm_pingpong_kernel<EDGE>;
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, kPpLdsBytesScaled, configured)) return HK_ERR_LAUNCH;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(512), kPpLdsBytesScaled, stream,
+                       (const uint8_t*)A, (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB,
+                       (uint16_t*)C, M, N, K / 2, sa_pitch, sb_pitch, tiles_m, tiles_n,
+                       raster_band(((long long)M + N) * (K / 2), tiles_n));
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
 template <bool EDGE>
 static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, const void* SB, void* C,
                               int M, int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
@@ -401,7 +427,8 @@ static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, cons
 
 }  // namespace hk
 
-// variant: -1 = choose, 0 = portable kernel, 1 = 256x256 tile kernel, 2 / 3 = 128x128 / 64x64 tiles.
+// variant: -1 = choose, 0 = portable kernel, 1 = 256x256 tile kernel (4 waves), 2 / 3 = 128x128 / 64x64 tiles,
+// 4 = 256x256 tile kernel with the 8-wave ping-pong schedule.
 // Scale rows are sa_pitch / sb_pitch bytes apart (>= K / 32).
 static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, const void* B, const void* B_scales,
                            int sb_pitch, void* C, int M, int N, int K, int variant, void* stream) {
@@ -410,7 +437,7 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
     if (M <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || sa_pitch < K / 32 || sb_pitch < K / 32)
         return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < -1 || variant > 3) return HK_ERR_UNSUPPORTED;
+    if (variant < -1 || variant > 4) return HK_ERR_UNSUPPORTED;
     // the tile kernel fetches a row's scales 16 bytes per lane, two K-steps of 8 bytes at a time:
     // rows must start 4-byte aligned and hold whole groups of 8 bytes
     const int groups = (K / 32 + 7) / 8 * 8;
@@ -447,6 +474,9 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
                  : launch_mxfp4_small_tile<kTinyTile, kTinyStages, false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
     }
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
+    if (variant == 4)
+        return edge ? launch_mxfp4_pingpong<true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s)
+                    : launch_mxfp4_pingpong<false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
     return edge ? launch_mxfp4_4wave<true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s)
                 : launch_mxfp4_4wave<false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
 }

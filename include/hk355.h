@@ -76,14 +76,15 @@ int hk_fp8_gemm_static_ws(const void* A_e4m3, const void* B_e4m3, void* C_bf16, 
                           float scale_a, float scale_b, void* stream);
 
 /* Same contract, forced onto one kernel variant (for tests and tuning):
- * 0 = portable kernel (any shape), 1 = 256x256x128 tile, 8 waves, 2 = 256x256x128 tile,
- * 4 waves, hand-interleaved schedule over two LDS stages, 3 = 256x256x128 tile, 4 waves, plain
- * loop, 4 = 256x256x128 tile, 4 waves, hand-interleaved schedule over a five-slot LDS ring with
- * the loads spread over the whole K-step (what hk_fp8_gemm picks when the problem has at least 128
- * such tiles), 5 = 128x128x128 tile, 4 waves, plain loop over three LDS stages (picked for smaller
- * problems), 6 = the same loop with 64x64 tiles and four stages, two workgroups per CU (picked
- * when the problem has at most 128 tiles of 128x128).
- * Variants 1-3 need K % 128 == 0; 4, 5 and 6 zero-fill the last K-step of any K % 16 == 0. */
+ * 0 = portable kernel (any shape), 1 = 256x256x128 tile, 8 waves in two ping-pong groups (the
+ * reference's second FP8 schedule, kernels/gemm/fp8fp32/README.md:3-5, schedule of
+ * kernels/gemm/bf16fp32/mi325x/256_256_64_16.cpp:73-155), 4 = 256x256x128 tile, 4 waves,
+ * hand-interleaved schedule over a five-slot LDS ring with the loads spread over the whole K-step
+ * (what hk_fp8_gemm picks when the problem has at least 128 such tiles), 5 = 128x128x128 tile, 4
+ * waves, plain loop over three LDS stages (picked for smaller problems), 6 = the same loop with
+ * 64x64 tiles and four stages, two workgroups per CU (picked when the problem has at most 128
+ * tiles of 128x128). 2 and 3 are not in use (HK_ERR_UNSUPPORTED). All tile kernels zero-fill the last
+ * K-step of any K % 16 == 0 and give identical bits. */
 int hk_fp8_gemm_variant(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
                         int M, int N, int K, float scale_a, float scale_b,
                         int variant, void* stream);
@@ -100,9 +101,10 @@ int hk_mxfp4_gemm(const void* A_e2m1, const void* A_scales_e8m0, const void* B_e
                   const void* B_scales_e8m0, void* C_bf16, int M, int N, int K, void* stream);
 
 /* Same contract on a chosen kernel: 0 = portable kernel (any shape), 1 = 256x256x256 tile
- * kernel, 2 = 128x128 tiles / three LDS stages, 3 = 64x64 tiles / four stages (the small-tile
- * kernels of the FP8 GEMM with the scaled FP4 MFMA; hk_mxfp4_gemm picks by tile count as
- * hk_fp8_gemm does). 1-3 need K % 256 == 0 (dense scale rows) and 4-byte aligned scale pointers. */
+ * kernel (4 waves, hand-interleaved), 2 = 128x128 tiles / three LDS stages, 3 = 64x64 tiles / four
+ * stages (the small-tile kernels of the FP8 GEMM with the scaled FP4 MFMA; hk_mxfp4_gemm picks by tile
+ * count as hk_fp8_gemm does), 4 = 256x256x256 tile kernel with the 8-wave ping-pong schedule. 1-4 need
+ * K % 256 == 0 (dense scale rows) and 4-byte aligned scale pointers. */
 int hk_mxfp4_gemm_variant(const void* A_e2m1, const void* A_scales_e8m0, const void* B_e2m1,
                           const void* B_scales_e8m0, void* C_bf16, int M, int N, int K,
                           int variant, void* stream);
@@ -150,7 +152,9 @@ int hk_bf16_gemm_ws(const void* A_bf16, const void* B_bf16, void* C_bf16, int M,
 /* Same contract on a chosen kernel: 0 = portable kernel (any shape), 1 = 256x256x64 tile kernel
  * (the FP8 ring schedule; the last K-step of a K that is not a multiple of 64 is zero-filled),
  * 2 = 128x128 tiles / three LDS stages, 3 = 64x64 tiles / four stages (the FP8 GEMM's small-tile
- * kernels with the bf16 MFMA; hk_bf16_gemm picks them by tile count as hk_fp8_gemm does). */
+ * kernels with the bf16 MFMA; hk_bf16_gemm picks them by tile count as hk_fp8_gemm does), 4 = 256x256x64
+ * tile kernel with the reference's 8-wave ping-pong schedule
+ * (kernels/gemm/bf16fp32/mi325x/256_256_64_16.cpp:73-155). */
 int hk_bf16_gemm_variant(const void* A_bf16, const void* B_bf16, void* C_bf16, int M, int N, int K,
                          int variant, void* stream);
 

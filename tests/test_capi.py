@@ -51,7 +51,7 @@ def test_c_entry_points_reject_bad_arguments_without_a_gpu():
     assert lib.hk_fp8_gemm(p, p, p, 0, 256, 256, 1.0, 1.0, None) == -2
     assert lib.hk_fp8_gemm(p, p, p, 256, 256, 250, 1.0, 1.0, None) == -2      # K % 16
     assert lib.hk_fp8_gemm(p + 1, p, p, 256, 256, 256, 1.0, 1.0, None) == -3
-    assert lib.hk_fp8_gemm_variant(p, p, p, 256, 256, 272, 1.0, 1.0, 2, None) == -2  # K % 128 for tile kernels
+    assert lib.hk_fp8_gemm_variant(p, p, p, 256, 256, 256, 1.0, 1.0, 2, None) == -6  # a variant that no longer exists
     assert lib.hk_fp8_gemm_variant(p, p, p, 256, 256, 256, 1.0, 1.0, 9, None) == -6
     assert lib.hk_mxfp4_gemm(p, None, p, p, p, 64, 64, 64, None) == -1
     assert lib.hk_mxfp4_gemm(p, p, p, p, p, 64, 64, 48, None) == -2           # K % 32
