@@ -615,7 +615,9 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
 // boundaries. All vector-memory operations are inline asm and counted by hand (the compiler
 // never waits for them): every use of loaded registers is preceded by a vmcnt wait and
 // `landed`, which makes the compiler see a new value there. Results are bit-identical to
-// moe_mxfp4_gemm_kernel (same accumulation order per output element).
+// moe_mxfp4_gemm_kernel (same accumulation order per output element). Launched for the extended
+// epilogues (biases, clamped SwiGLU, interleaved source rows); the plain ones take the 4-wave
+// kernel below.
 constexpr int kStBM = 192;                              // rows per work item
 constexpr int kStStages = 5;
 constexpr int kStATile = kStBM * 128;                   // 24 KiB
@@ -650,8 +652,12 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
         const v4i item = scalar_load_x4(p.items + (c.valid ? c.it : it_end - 1));
         c.expert = item.x; c.row_start = item.y; c.rows = item.z; c.n_tile = item.w;
     };
+    // An item takes nk4 positions, nk rounded up to a multiple of four (the length of the ring of
+    // register sets): its last position is then always one of set 3, and the epilogue code exists
+    // once instead of once per set. The padding positions fetch and compute nothing.
+    const int nk4 = (nk + 3) & ~3;
     auto advance = [&](Cursor& c) __attribute__((always_inline)) {
-        if (++c.kt == nk) { c.kt = 0; c.it += it_stride; load_item(c); }
+        if (++c.kt == nk4) { c.kt = 0; c.it += it_stride; load_item(c); }
     };
     Cursor cc{it0, 0}, ca{it0, 0}, cb{it0, 0};  // compute, activation fetch, weight fetch
     load_item(cc);
@@ -666,7 +672,7 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
     };
     cb_descriptors();
     auto advance_cb = [&]() __attribute__((always_inline)) {
-        if (++cb.kt == nk) { cb.kt = 0; cb.it += it_stride; load_item(cb); cb_descriptors(); }
+        if (++cb.kt == nk4) { cb.kt = 0; cb.it += it_stride; load_item(cb); cb_descriptors(); }
     };
 
     // ---- activation tile: global -> LDS -------------------------------------------------------
@@ -682,8 +688,8 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
     // empty buffer, past the item's last fragment) and the row scales of rows [24 w, +24)
     auto issue_a = [&](const Cursor& c, int stage) __attribute__((always_inline)) {
         v4i ssa = srd_sa;
-        if (!c.valid) ssa.z = 0;
-        const int rows_up = c.valid ? (c.rows + 15) & ~15 : 0;
+        if (!c.valid || c.kt >= nk) ssa.z = 0;
+        const int rows_up = c.valid && c.kt < nk ? (c.rows + 15) & ~15 : 0;
         const uint32_t row_base = (uint32_t)c.kt * (uint32_t)p.S + (uint32_t)c.row_start;
         const uint32_t dst = lds_wave + (uint32_t)stage * kStStage;
 #pragma unroll
@@ -706,7 +712,8 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
     // zeros without fetching them (K = 2880: 6 % of the weight bytes).
     const int last_valid = Kb - (nk - 1) * 128;
     auto load_b_half = [&](const Cursor& c, v4i (&dst)[NT], int half) __attribute__((always_inline)) {
-        const v4i rs = cb_srd_b;
+        v4i rs = cb_srd_b;
+        if (c.kt >= nk) rs.z = 0;
         const uint32_t soff = (uint32_t)c.kt * kMoeBTile + (uint32_t)w * 4096u + (uint32_t)half * 1024u;
         // first padded lane * 16 - 1 (uniform); voff_b = 16 l exceeds it exactly in the padded lanes
         const int thr = c.kt == nk - 1 ? 16 * min(max(last_valid - 64 * half, 0), 64) - 1 : 0x7fffffff;
@@ -719,7 +726,8 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
                          : "memory");
     };
     auto load_b_scales = [&](const Cursor& c, int& dst) __attribute__((always_inline)) {
-        const v4i rss = cb_srd_sb;
+        v4i rss = cb_srd_sb;
+        if (c.kt >= nk) rss.z = 0;
         asm volatile("buffer_load_dword %0, %1, %2, %3 offen"
                      : "=v"(dst)
                      : "v"(voff_sb), "s"(rss), "s"((uint32_t)c.kt * kMoeScaleB + (uint32_t)w * 256u)
@@ -936,7 +944,7 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
         landed(bw[P][0]);
         asm volatile("" : "+v"(bsc[P]));
         const int sc = bsc[P];
-        const int rows = cc.valid ? cc.rows : 0;  // past the end of the stream: no MFMAs, empty loads
+        const int rows = cc.valid && cc.kt < nk ? cc.rows : 0;  // padding / past the end of the stream: no MFMAs, empty loads
         compute_half(st, 0, rows, bw[P][0], sc);
         load_b_half(cb, bw[P][0], 0);
         wait_vmcnt<33>();
@@ -945,10 +953,12 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
         load_b_scales(cb, bsc[P]);
         load_b_half(cb, bw[P][1], 1);
         advance_cb();
-        if (cc.valid && cc.kt == nk - 1) {
-            mfma_drain();
-            epilogue(cc);
-            zero_acc();
+        if constexpr (P == 3) {
+            if (cc.valid && cc.kt == nk4 - 1) {
+                mfma_drain();
+                epilogue(cc);
+                zero_acc();
+            }
         }
         advance(cc);
     };
@@ -962,6 +972,322 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
         step.template operator()<1>(st); next_stage();
         step.template operator()<2>(st); next_stage();
         step.template operator()<3>(st); next_stage();
+    }
+    wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
+}
+
+// ------------------------------------------------------- 4-wave weight-streaming grouped GEMM
+// The same stream with one wave per SIMD, for the plain epilogues (SiLU-mul with MX re-quantization,
+// bf16 store); the 8-wave kernel above serves the extended ones. Wave W takes what waves 2W and
+// 2W + 1 of that kernel take: weight rows [64 W, +64) of the 256-row tile (four fragments) x all
+// rows of the item, 192 accumulator registers per lane, updated in place in AGPRs. What that buys:
+//   * the 32 h columns of a wave are exactly one MX block, so the gate+up epilogue needs no
+//     exchange between waves, no LDS and no workgroup barrier: block maxima and a row's 16 packed
+//     bytes are gathered inside the wave by swapping rows of 16 lanes in registers
+//     (v_permlane16_swap / v_permlane32_swap), one 16-byte store per 16 rows;
+//   * the epilogue of row fragment M - 1 runs right behind the MFMAs of fragment M in the item's
+//     last K-step, and the loads of the position three ahead are spread over the fragments of every
+//     K-step, the last one included: the wave keeps requesting weights while it finishes an item.
+// Per position a wave issues 17 loads: six 1 KiB pieces of the activation tile and its 384 bytes of
+// row scales (global -> LDS, four stages), eight 1 KiB weight fragments and two scale dwords
+// (global -> VGPRs, four register sets). Position q's loads are issued during position q - 3; they
+// return in order, so at the start of position q everything of it has landed when at most the 34
+// loads of positions q + 1 and q + 2 are outstanding. Bit-identical to the kernels above.
+// Measured at the GPT-OSS-like shape (kernel trace, us, gate+up / down): 275 / 148 (8-wave kernel:
+// 293 / 152); without epilogues 227 / 115; loads, waits and barriers only 206 / 103; the K loop's
+// MFMAs and LDS reads on empty loads 148 / 78. The K loop hides behind the weight stream, the
+// epilogue does not: while a wave spends about 8 k clocks finishing an item, the three positions it
+// has in flight (about 6.6 k clocks of the stream) run dry. An epilogue copy per register set (four
+// times the code) cost another 7 %: the loop then no longer fits the instruction cache.
+constexpr int kS4Stages = 4;
+constexpr int kS4Lds = kS4Stages * kStStage;   // 102 KiB
+constexpr int kS4Loads = 17;
+constexpr int kS4Ahead = 3;  // positions between fetch and compute (two measure the same)
+
+template <int MODE>
+__global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmParams p) {
+    constexpr int MT = kStBM / 16;
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    const int lane = lane_id(), w = wave_id();
+    const int n_items = scalar_load_x1(p.num_items);
+    const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+    const int it_stride = ((int)gridDim.x - xcd + kNumXcd - 1) / kNumXcd;  // workgroups on this XCD
+    const int per_xcd = (n_items + kNumXcd - 1) / kNumXcd;
+    const int it0 = xcd * per_xcd + slot;
+    const int it_end = min(n_items, (xcd + 1) * per_xcd);
+    if (it0 >= it_end) return;
+
+    const int Kb = p.K >> 1;
+    const int nk = (Kb + 127) >> 7;
+    const v4i srd_a = make_srd(p.A, (uint32_t)nk * (uint32_t)p.S * 128u);
+    const v4i srd_sa = make_srd(p.SA, (uint32_t)nk * (uint32_t)p.S * 8u);
+
+    // ---- cursors over the stream of (item, K-step) positions of this workgroup ---------------
+    struct Cursor { int it, kt, expert, row_start, rows, n_tile; bool valid; };
+    auto load_item = [&](Cursor& c) __attribute__((always_inline)) {
+        c.valid = c.it < it_end;
+        const v4i item = scalar_load_x4(p.items + (c.valid ? c.it : it_end - 1));
+        c.expert = item.x; c.row_start = item.y; c.rows = item.z; c.n_tile = item.w;
+    };
+    // An item takes nk4 positions, nk rounded up to a multiple of four (the length of the ring of
+    // register sets): its last position is then always one of set 3, and the epilogue code exists
+    // once instead of once per set. The padding positions fetch and compute nothing.
+    const int nk4 = (nk + 3) & ~3;
+    Cursor cc{it0, 0}, cf{it0, 0};  // compute, fetch (three positions ahead)
+    load_item(cc);
+    cf = cc;
+    // per fetch item: weight and weight-scale descriptors, rows rounded up to fragments
+    v4i cf_srd_b, cf_srd_sb;
+    auto cf_descriptors = [&]() __attribute__((always_inline)) {
+        cf_srd_b = make_srd(p.B + (size_t)cf.expert * p.b_expert_stride + (size_t)cf.n_tile * nk * kMoeBTile,
+                            cf.valid ? (uint32_t)nk * kMoeBTile : 0u);
+        cf_srd_sb = make_srd(p.SB + (size_t)cf.expert * p.sb_expert_stride + (size_t)cf.n_tile * nk * kMoeScaleB,
+                             cf.valid ? (uint32_t)nk * kMoeScaleB : 0u);
+    };
+    cf_descriptors();
+    auto advance_cf = [&]() __attribute__((always_inline)) {
+        if (++cf.kt == nk4) { cf.kt = 0; cf.it += it_stride; load_item(cf); cf_descriptors(); }
+    };
+
+    // ---- loads of one position ------------------------------------------------------------------
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+    const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
+    const uint32_t lds_sa_wave = to_sgpr(lds0 + kStATile + (uint32_t)w * 384u);
+    // piece i of the activation tile = rows 8 (4 i + w) .. +8; the swizzle of a row depends on its
+    // bits 1..3, i.e. on w and the lane only
+    const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);
+    const uint32_t voff_a0 = (uint32_t)(8 * w + (lane >> 3)) * 128u + chunk16 * 16u;  // + i * 4096
+    const uint32_t voff_sa = (uint32_t)(w * 384 + lane * 16);
+    const uint32_t voff_b = lane * 16, voff_sb = lane * 4;
+    v4i bw[4][8];   // [position mod 4][4 * (weight fragment pair) + 2 * fragment + K half]
+    int bsc[4][2];  // [position mod 4][pair]: the lane's scale bytes, byte 2 * half + fragment
+    // Bytes of the last K-step that lie inside K (the layout pads every row to whole K-steps with
+    // zeros): lane l's 16 bytes of half h start at byte 64 h + 16 (l / 16) of the K-step. Lanes
+    // past the end get bit 31 in their offset: outside the buffer, so the load returns the same
+    // zeros without fetching them.
+    const int last_valid = Kb - (nk - 1) * 128;
+    // load L (0..16) of the fetch position, into LDS stage / register set P
+    auto fetch_load = [&]<int P, int L>() __attribute__((always_inline)) {
+        if constexpr (L < 6) {
+            const int rows_up = cf.valid && cf.kt < nk ? (cf.rows + 15) & ~15 : 0;
+            v4i sa = srd_a;
+            if (8 * (4 * L + w) >= rows_up) sa.z = 0;  // past the item's last fragment: nothing is fetched
+            const uint32_t row_base = (uint32_t)cf.kt * (uint32_t)p.S + (uint32_t)cf.row_start;
+            dma16(sa, lds_wave + (uint32_t)(P * kStStage + L * 4096), voff_a0 + L * 4096u, row_base * 128u);
+        } else if constexpr (L == 6) {
+            v4i ssa = srd_sa;
+            if (!cf.valid || cf.kt >= nk) ssa.z = 0;
+            const uint32_t row_base = (uint32_t)cf.kt * (uint32_t)p.S + (uint32_t)cf.row_start;
+            dma16_lanes(ssa, lds_sa_wave + (uint32_t)(P * kStStage), voff_sa, row_base * 8u, 0xffffffull);
+        } else if constexpr (L < 15) {
+            constexpr int f = L - 7, pair = f >> 2, half = f & 1;
+            const int thr = cf.kt == nk - 1 ? 16 * min(max(last_valid - 64 * half, 0), 64) - 1 : 0x7fffffff;
+            const uint32_t voff = voff_b | ((uint32_t)(thr - (int)voff_b) & 0x80000000u);
+            const uint32_t soff = (uint32_t)cf.kt * kMoeBTile + (uint32_t)(2 * w + pair) * 4096u;
+            v4i rs = cf_srd_b;
+            if (cf.kt >= nk) rs.z = 0;
+            asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4"
+                         : "=v"(bw[P][f])
+                         : "v"(voff), "s"(rs), "s"(soff), "n"(((f >> 1) & 1) * 2048 + half * 1024)
+                         : "memory");
+        } else if constexpr (L < kS4Loads) {
+            constexpr int pair = L - 15;
+            int& dst = bsc[P][pair];
+            v4i rss = cf_srd_sb;
+            if (cf.kt >= nk) rss.z = 0;
+            const uint32_t voff = voff_sb;
+            asm volatile("buffer_load_dword %0, %1, %2, %3 offen"
+                         : "=v"(dst)
+                         : "v"(voff), "s"(rss), "s"((uint32_t)cf.kt * kMoeScaleB + (uint32_t)(2 * w + pair) * 256u)
+                         : "memory");
+        }
+    };
+    auto fetch_all = [&]<int P>() __attribute__((always_inline)) {
+        [&]<int... L>(std::integer_sequence<int, L...>) __attribute__((always_inline)) {
+            (fetch_load.template operator()<P, L>(), ...);
+        }(std::make_integer_sequence<int, kS4Loads>{});
+        advance_cf();
+    };
+
+    // ---- LDS -> registers (activation fragments) ------------------------------------------------
+    const uint32_t r = lane & 15, g = lane >> 4;
+    const uint32_t rd_half[2] = {lds0 + r * 128u + swz_chunk(r, g) * 16u, lds0 + r * 128u + swz_chunk(r, g + 4) * 16u};
+    const uint32_t sa_rd0 = lds0 + kStATile + r * 8u;
+    const uint32_t sh = 8u * g;  // byte g of each scale dword belongs to this lane
+
+    v4f acc[MT][4];  // [row fragment][2 * pair + fragment]
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int n = 0; n < 4; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
+    auto mfma = [&](v4f& c, const v4i& x, const v4i& y, int sx, int sy) __attribute__((always_inline)) {
+        asm volatile(
+            "v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+            : "+a"(c)
+            : "v"(x), "v"(y), "v"(sx), "v"(sy));
+    };
+
+    // ---- epilogue of row fragment m of the compute item (its accumulators are final) -------------
+    // Stores go through buffer descriptors that end at the item's last row: rows of the last
+    // fragment beyond it (they belong to the next expert) are dropped by the range check, so the
+    // epilogue needs no per-lane row test and no 64-bit address arithmetic. Lanes that do not
+    // store at all carry bit 31 in their offset. Set up once per item by begin_epilogue().
+    v4i st_srd0, st_srd1;     // MODE 0: packed h / its scales; MODE 1: the bf16 output
+    uint32_t st_voff0 = 0, st_voff1 = 0;
+    bool st_ok[2] = {false, false};  // MODE 0: [0] the wave's MX block lies inside N; MODE 1: its two 32-column groups
+    auto begin_epilogue = [&]() __attribute__((always_inline)) {
+        if (MODE == 1) {
+            const uint32_t pitch = (uint32_t)p.N * 2u;
+            st_srd0 = make_srd((uint8_t*)p.out0 + (size_t)cc.row_start * pitch, (uint32_t)cc.rows * pitch);
+            const int wcol0 = cc.n_tile * 256 + 64 * w;  // N % 32 == 0: a group of 32 columns is valid as a whole
+            st_ok[0] = wcol0 < p.N; st_ok[1] = wcol0 + 32 < p.N;
+            st_voff0 = r * pitch + (uint32_t)(wcol0 + 8 * (int)g) * 2u;
+        } else {
+            const size_t row0 = (size_t)(cc.n_tile >> 1) * p.S + (size_t)cc.row_start;
+            st_srd0 = make_srd((uint8_t*)p.out0 + row0 * 128, (uint32_t)cc.rows * 128u);
+            st_srd1 = make_srd(p.out_scales + row0 * 8, (uint32_t)cc.rows * 8u);
+            const uint32_t seg = (uint32_t)(cc.n_tile & 1) * 64u;  // the n-tile's 128 columns are half of a K-step row
+            st_ok[0] = cc.n_tile * 128 + 32 * w < p.N;
+            st_voff0 = g == 0 ? r * 128u + seg + 16u * (uint32_t)w : 0x80000000u;
+            st_voff1 = g == 0 ? r * 8u + (seg >> 4) + (uint32_t)w : 0x80000000u;
+        }
+    };
+    auto epilogue = [&]<int M>(bool drain) __attribute__((always_inline)) {
+        // The accumulators are operands of this statement: the compiler sees no hazard behind the
+        // MFMA statements and would otherwise move the reads of the accumulators up to them.
+        asm volatile("" : "+a"(acc[M][0]), "+a"(acc[M][1]), "+a"(acc[M][2]), "+a"(acc[M][3]));
+        // fragment M's MFMAs are followed by those of fragment M + 1 unless it was the item's last
+        if (drain) asm volatile("s_nop 15\n\ts_nop 7" : "+a"(acc[M][0]), "+a"(acc[M][1]), "+a"(acc[M][2]), "+a"(acc[M][3]));
+        if (MODE == 1) {
+            // lane (r, g) holds, for row 16 M + r, the columns 64 w + 32 o + 8 g .. +8 (o = 0, 1)
+#pragma unroll
+            for (int o = 0; o < 2; ++o) {
+                const v4f x = acc[M][2 * o], y = acc[M][2 * o + 1];
+                v4i o4;
+                o4.x = pack_bf16(x.x, x.y); o4.y = pack_bf16(x.z, x.w);
+                o4.z = pack_bf16(y.x, y.y); o4.w = pack_bf16(y.z, y.w);
+                if (st_ok[o])
+                    asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen offset:%3\n\ts_nop 1"
+                                 :: "v"(o4), "v"(st_voff0), "s"(st_srd0), "n"(o * 64) : "memory");
+            }
+            st_voff0 += 32u * (uint32_t)p.N;  // 16 rows
+        } else {
+            // h = act(gate, up): lane (r, g) holds, for row 16 M + r, the h columns
+            // 128 n_tile + 32 w + 16 o + 4 g .. +4 (o = 0, 1): the wave's 32 columns are one MX block
+            float h[2][4];
+            float amax = 0.f;
+#pragma unroll
+            for (int o = 0; o < 2; ++o) {
+                const v4f gt = acc[M][2 * o], up = acc[M][2 * o + 1];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    h[o][j] = silu_mul(gt[j], up[j]);
+                    amax = fmaxf(amax, fabsf(h[o][j]));
+                }
+            }
+            // maximum over the four lanes (r, 0..3) of a row: rows of 16 lanes swapped in registers
+            {
+                const uint32_t a = __float_as_uint(amax);
+                const auto s16 = __builtin_amdgcn_permlane16_swap(a, a, false, false);
+                const uint32_t m1 = __float_as_uint(fmaxf(__uint_as_float(s16[0]), __uint_as_float(s16[1])));
+                const auto s32 = __builtin_amdgcn_permlane32_swap(m1, m1, false, false);
+                amax = fmaxf(__uint_as_float(s32[0]), __uint_as_float(s32[1]));
+            }
+            int e = mx_block_exponent(amax);
+            const float scale = __uint_as_float(e > -127 ? (uint32_t)(e + 127) << 23 : 0x00400000u);
+            uint32_t pk = 0;  // low half: columns 4 g .. +4 of the block's first 16, high half: of its second 16
+            pk = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(pk, h[0][0], h[0][1], scale, 0);
+            pk = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(pk, h[0][2], h[0][3], scale, 1);
+            pk = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(pk, h[1][0], h[1][1], scale, 2);
+            pk = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(pk, h[1][2], h[1][3], scale, 3);
+            if (!st_ok[0]) { pk = 0; e = 0; }  // columns past N (uniform): zeros with a scale of one
+            // every lane of a row gets the packed values of all four: p[g'] = pk of lane (r, g')
+            const auto q16 = __builtin_amdgcn_permlane16_swap(pk, pk, false, false);       // [p0 p0 p2 p2], [p1 p1 p3 p3]
+            const auto q02 = __builtin_amdgcn_permlane32_swap(q16[0], q16[0], false, false);  // p0, p2
+            const auto q13 = __builtin_amdgcn_permlane32_swap(q16[1], q16[1], false, false);  // p1, p3
+            v4i o4;  // the row's 16 bytes: the first 16 columns' codes (low halves), then the second 16's
+            o4.x = (int)__builtin_amdgcn_perm(q13[0], q02[0], 0x05040100u);
+            o4.y = (int)__builtin_amdgcn_perm(q13[1], q02[1], 0x05040100u);
+            o4.z = (int)__builtin_amdgcn_perm(q13[0], q02[0], 0x07060302u);
+            o4.w = (int)__builtin_amdgcn_perm(q13[1], q02[1], 0x07060302u);
+            asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1"
+                         :: "v"(o4), "v"(st_voff0), "s"(st_srd0) : "memory");
+            asm volatile("buffer_store_byte %0, %1, %2, 0 offen"
+                         :: "v"(e + 127), "v"(st_voff1), "s"(st_srd1) : "memory");
+            st_voff0 += 16u * 128u;
+            st_voff1 += 16u * 8u;
+        }
+#pragma unroll
+        for (int n = 0; n < 4; ++n) acc[M][n] = v4f{0.f, 0.f, 0.f, 0.f};
+    };
+
+    // ---- prologue: positions 0..2 -----------------------------------------------------------------
+    fetch_all.template operator()<0>();
+    fetch_all.template operator()<1>();
+    fetch_all.template operator()<2>();
+
+    // One stream position on LDS stage / register set P; the loads of the position three ahead go
+    // to stage / set (P + 3) % 4, which the previous position has just finished with.
+    auto step = [&]<int P>() __attribute__((always_inline)) {
+        constexpr int PF = (P + kS4Ahead) % 4;
+        wait_vmcnt<(kS4Ahead - 1) * kS4Loads>();
+        block_barrier();  // everyone's part of this position's tile has landed; stage PF is free
+#pragma unroll
+        for (int f = 0; f < 8; ++f) asm volatile("" : "+v"(bw[P][f]));
+        asm volatile("" : "+v"(bsc[P][0]), "+v"(bsc[P][1]));
+        const int rows = cc.valid && cc.kt < nk ? cc.rows : 0;  // padding, or past the end of the stream: no MFMAs
+        const int mt = (rows + 15) >> 4;
+        const int mt_item = cc.valid ? (cc.rows + 15) >> 4 : 0;
+        const bool last = P == 3 && cc.valid && cc.kt == nk4 - 1;
+        if (last) begin_epilogue();
+        int bs[8];  // scale of weight fragment f = 4 pair + 2 n + half: byte 2 half + n of the pair's dword
+#pragma unroll
+        for (int f = 0; f < 8; ++f) bs[f] = (int)((uint32_t)bsc[P][f >> 2] >> (8 * (2 * (f & 1) + ((f >> 1) & 1))));
+        uint32_t a_rd0 = rd_half[0] + (uint32_t)(P * kStStage), a_rd1 = rd_half[1] + (uint32_t)(P * kStStage);
+        uint32_t sa_rd = sa_rd0 + (uint32_t)(P * kStStage);
+        asm volatile("" : "+v"(a_rd0), "+v"(a_rd1), "+v"(sa_rd));  // bases in registers, offsets as immediates
+        v4i af[3][2];
+        v2i as[3];
+        auto rd = [&](int m) __attribute__((always_inline)) {
+            af[m % 3][0] = *(lds_v4i_t*)(uintptr_t)(a_rd0 + m * 2048);
+            af[m % 3][1] = *(lds_v4i_t*)(uintptr_t)(a_rd1 + m * 2048);
+            as[m % 3] = *(lds_v2i_t*)(uintptr_t)(sa_rd + m * 128);
+        };
+        if (mt > 0) { rd(0); rd(1); }
+        auto frag = [&]<int M>() __attribute__((always_inline)) {
+            if (M < mt) {
+                if (M + 2 < MT) rd(M + 2);  // rows past the tile's count are readable, never used
+                const int sa[2] = {(int)((uint32_t)as[M % 3].x >> sh), (int)((uint32_t)as[M % 3].y >> sh)};
+#pragma unroll
+                for (int half = 0; half < 2; ++half)
+#pragma unroll
+                    for (int n = 0; n < 4; ++n) {
+                        const int f = 4 * (n >> 1) + 2 * (n & 1) + half;
+                        mfma(acc[M][n], bw[P][f], af[M % 3][half], bs[f], sa[half]);
+                    }
+            }
+            fetch_load.template operator()<PF, M>();
+            if constexpr (M + 12 < kS4Loads) fetch_load.template operator()<PF, M + 12>();
+            if constexpr (M >= 1) {
+                if constexpr (P == 3)
+                    if (last && M - 1 < mt_item) epilogue.template operator()<M - 1>(M >= mt);
+            }
+        };
+        [&]<int... M>(std::integer_sequence<int, M...>) __attribute__((always_inline)) {
+            (frag.template operator()<M>(), ...);
+        }(std::make_integer_sequence<int, MT>{});
+        advance_cf();
+        if constexpr (P == 3)
+            if (last && MT - 1 < mt_item) epilogue.template operator()<MT - 1>(true);
+        if (++cc.kt == nk4) { cc.kt = 0; cc.it += it_stride; load_item(cc); }
+    };
+    // Four positions per trip (stages and register sets rotate); positions past the end of the
+    // stream degenerate to their barrier and empty loads.
+    while (cc.valid) {
+        step.template operator()<0>();
+        step.template operator()<1>();
+        step.template operator()<2>();
+        step.template operator()<3>();
     }
     wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
 }
@@ -1027,12 +1353,19 @@ void moe_launch_build_items(const int32_t* expert_offsets, int E, int bm, int n_
 
 template <int MODE, bool EXT>
 static int launch_moe_stream(MoeGemmParams p, int max_items, hipStream_t s) {
-    auto kern = moe_mxfp4_stream_kernel<MODE, EXT>;
+    // Plain epilogues (SiLU-mul / bf16 store): the 4-wave kernel. With biases, the clamped SwiGLU or
+    // interleaved source rows the per-element work of the epilogue is larger and two waves per SIMD
+    // hide it better: the 8-wave kernel (measured: 0.51 against 0.57 ms for the layer).
+    constexpr int lds = EXT ? kStLds : kS4Lds, threads = EXT ? 512 : 256;
+    const void* kern;
+    if constexpr (EXT) kern = (const void*)moe_mxfp4_stream_kernel<MODE, true>;
+    else kern = (const void*)moe_mxfp4_stream4_kernel<MODE>;
     static DeviceOnce configured;
-    if (!set_lds_limit_once((const void*)kern, kStLds, configured)) return HK_ERR_LAUNCH;
+    if (!set_lds_limit_once(kern, lds, configured)) return HK_ERR_LAUNCH;
     // persistent: one workgroup per CU, each walking its share of the item list
     const int grid = min(max_items, moe_num_compute_units());
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kStLds, s, p);
+    void* args[] = {&p};
+    if (hipLaunchKernel(kern, dim3(grid), dim3(threads), args, lds, s) != hipSuccess) return HK_ERR_LAUNCH;
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
