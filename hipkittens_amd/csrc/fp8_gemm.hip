@@ -201,7 +201,7 @@ __global__ __launch_bounds__(256) void fp8_gemm_4wave_ring_kernel(
     }
     if (kt < nk) step.template operator()<0>(kt);
     wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
-    mfma_drain();
+    mfma_drain_agpr(acc);
 
     store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
 }

@@ -189,6 +189,26 @@ __device__ __forceinline__ void mfma_fp8_16x16x128_acc(v4f& acc, const v8i& a, c
 // Wait states between the last MFMA and the first read of its result by a
 // non-MFMA instruction (the longest case on this ISA is 18 cycles for a 16-pass MFMA).
 __device__ __forceinline__ void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 7" ::: "memory"); }
+// mfma_drain() for accumulators written by the asm MFMA statements: every later read of `acc`
+// depends on the drain. Reads of registers are not memory operations, and the compiler, which sees
+// no hazard behind those statements, may otherwise move them above it, next to the MFMAs.
+// (Volatile asm statements keep their order; each accumulator passes through one.)
+template <int M, int N>
+__device__ __forceinline__ void mfma_drain_agpr(v4f (&acc)[M][N]) {
+    mfma_drain();
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int n = 0; n < N; ++n) asm volatile("" : "+a"(acc[m][n]));
+}
+template <int M, int N>
+__device__ __forceinline__ void mfma_drain_vgpr(v4f (&acc)[M][N]) {
+    mfma_drain();
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int n = 0; n < N; ++n) asm volatile("" : "+v"(acc[m][n]));
+}
 
 // Two fp32 -> packed bf16 (round to nearest even); `lo` goes to bits [15:0].
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {

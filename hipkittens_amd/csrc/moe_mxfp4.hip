@@ -588,7 +588,7 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
             }
             st = st == 2 ? 0 : st + 1;
         }
-        mfma_drain();
+        mfma_drain_vgpr(acc);
         epilogue(cur);
         it += it_stride;
         if (it >= it_end) break;
@@ -955,7 +955,7 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
         advance_cb();
         if constexpr (P == 3) {
             if (cc.valid && cc.kt == nk4 - 1) {
-                mfma_drain();
+                mfma_drain_vgpr(acc);
                 epilogue(cc);
                 zero_acc();
             }

@@ -252,7 +252,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     }
     if (kt < nk) step.template operator()<0>(kt);
     wait_vmcnt<0>();
-    mfma_drain();
+    mfma_drain_agpr(acc);
 
     store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, 1.0f);
 }
