@@ -332,6 +332,13 @@ def bench_moe_mxfp4(torch, hk, warmup, iters, dev, graph=True):
     b2 = torch.randn(E, H, device=dev, generator=g)
     _, kern_oai = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_mxfp4(
         x, logits, W, None, None, None, y, k, ws, bias13=b13, bias2=b2, activation="swiglu_oai"), warmup, iters)
+    # the same layer with MXFP8 activations (W4A8: mixed fp4 x fp8 MFMA), checked against the oracle on the sample
+    ws8 = torch.empty(hk.tk_kernel.moe_mxfp4_workspace_bytes(T, H, I, E, k, act_format="mxfp8"), dtype=torch.uint8,
+                      device=dev)
+    call8 = lambda: hk.tk_kernel.dispatch_moe_mxfp4(x, logits, W, None, None, None, y, k, ws8, act_format="mxfp8")
+    _, kern_a8 = _timeit(torch, call8, warmup, iters)
+    want8, _ = OM.moe_mxfp4_forward(F.bf16_to_f32(_np_bits(x[st])), ids_l, w_s, *plain, act_format="mxfp8")
+    rel8 = OG.rel_fro_error(y[st].float().cpu().numpy(), F.bf16_to_f32(want8))
     return {"workload": "moe_mxfp4 T=4096 H=2880 I=2880 E=128 top-4 softmax, MXFP4 activations and weights "
                         "(routing + sort + quantize/permute + 2 grouped GEMMs + un-permute)",
             "ms": round(kern, 5), "tflops": round(tf, 1), "frac_of_mxfp4_peak": round(tf / PEAK_FP4, 4),
@@ -339,7 +346,8 @@ def bench_moe_mxfp4(torch, hk, warmup, iters, dev, graph=True):
             "roofline": _roofline("hbm", compulsory / (kern * 1e-3) / 1e9, PEAK_HBM, "GB/s",
                                   "whole layer (5 launches); dominant: moe_mxfp4 gate+up grouped GEMM",
                                   _traffic("moe_mxfp4")),
-            "ms_graph_replay": round(kern_graph, 5) if graph else None, "ms_with_biases_and_clamped_swiglu": round(kern_oai, 5)}
+            "ms_graph_replay": round(kern_graph, 5) if graph else None, "ms_with_biases_and_clamped_swiglu": round(kern_oai, 5),
+            "ms_with_mxfp8_activations": round(kern_a8, 5), "rel_fro_err_mxfp8_activations_vs_oracle_8_tokens": rel8}
 
 
 def cpu_baseline_moe_mxfp4(torch, hk, dev):

@@ -51,6 +51,14 @@ SIGNATURES = {
     "hk_moe_mxfp4_forward_ex": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int,
                                         c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                                         c_int, c_float, c_float, c_int, c_void_p, c_size_t, c_void_p]),
+    "hk_mxfp8_quantize_rows": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
+    "hk_moe_mxfp4_a8_workspace_bytes": (c_size_t, [c_int] * 5),
+    "hk_moe_mxfp4_a8_experts": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p,
+                                        c_void_p, c_int, c_float, c_float, c_int, c_void_p, c_size_t, c_void_p]),
+    "hk_moe_mxfp4_a8_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float,
+                                        c_float, c_int, c_void_p, c_size_t, c_void_p]),
     "hk_moe_mxfp4_preshuffle_bytes": (c_int, [c_int, c_int, c_int, c_int, ctypes.POINTER(c_size_t),
                                               ctypes.POINTER(c_size_t)]),
     "hk_moe_mxfp4_preshuffle": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,

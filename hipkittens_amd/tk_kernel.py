@@ -255,6 +255,20 @@ def dispatch_mxfp4_quantize_rows(x, packed, scales) -> None:
     _lib.check(st, "dispatch_mxfp4_quantize_rows")
 
 
+def dispatch_mxfp8_quantize_rows(x, codes, scales) -> None:
+    """x [R,C] bf16 -> codes [R,C] e4m3 (MX blocks of 32, shared exponent floor(log2 amax) - 8,
+    saturating), scales [R,pitch] uint8 e8m0 (pitch >= C/32, multiple of 8)."""
+    _check_tensor(x, "x", _BF16, 2)
+    _check_tensor(codes, "codes", _FP8, 2)
+    _check_tensor(scales, "scales", _E8M0, 2)
+    R, C = x.shape
+    if tuple(codes.shape) != (R, C) or scales.shape[0] != R:
+        raise RuntimeError("shape mismatch between x, codes and scales")
+    st = _lib.load_library().hk_mxfp8_quantize_rows(x.data_ptr(), R, C, codes.data_ptr(), scales.data_ptr(),
+                                                    scales.shape[1], _stream(x))
+    _lib.check(st, "dispatch_mxfp8_quantize_rows")
+
+
 def dispatch_moe_unpermute(o, weights, slot_to_pos, y, add=None) -> None:
     """y [T,H] bf16 = (add [T,H] bf16 if given) + sum_j weights[t,j] * o[slot_to_pos[t*k+j]] with
     o [T*k,H] bf16."""
@@ -276,8 +290,14 @@ def dispatch_moe_unpermute(o, weights, slot_to_pos, y, add=None) -> None:
     _lib.check(st, "dispatch_moe_unpermute")
 
 
-def moe_mxfp4_workspace_bytes(T: int, H: int, I: int, E: int, k: int) -> int:
-    return int(_lib.load_library().hk_moe_mxfp4_workspace_bytes(T, H, I, E, k))
+def moe_mxfp4_workspace_bytes(T: int, H: int, I: int, E: int, k: int, act_format: str = "mxfp4") -> int:
+    """Workspace of the MXFP4-weight MoE; act_format "mxfp8": with MXFP8 activations (W4A8)."""
+    lib = _lib.load_library()
+    if act_format == "mxfp8":
+        return int(lib.hk_moe_mxfp4_a8_workspace_bytes(T, H, I, E, k))
+    if act_format != "mxfp4":
+        raise RuntimeError("act_format must be 'mxfp4' or 'mxfp8'")
+    return int(lib.hk_moe_mxfp4_workspace_bytes(T, H, I, E, k))
 
 
 class MoeMxfp4ShuffledWeights:
@@ -379,11 +399,14 @@ def _moe_ext_args(w13, E, H, I, bias13, bias2, activation, interleaved):
 
 def dispatch_moe_mxfp4_experts(x, w13, w13_scales, w2, w2_scales, weights, sorted_slots, expert_offsets,
                                slot_to_pos, y, workspace, bias13=None, bias2=None, activation: str = "silu",
-                               alpha: float = 1.702, limit: float = 7.0, interleaved=None) -> None:
+                               alpha: float = 1.702, limit: float = 7.0, interleaved=None,
+                               act_format: str = "mxfp4") -> None:
     """Expert MLP on routed + sorted tokens (see include/hk355.h: hk_moe_mxfp4_experts_ex). `w13` may be
     a MoeMxfp4ShuffledWeights, in which case w13_scales, w2 and w2_scales are ignored (pass None).
     Model-faithful options: bias13 [E, 2I] / bias2 [E, H] fp32, activation "swiglu_oai" (clamped
-    SwiGLU with alpha and limit), interleaved gate / up rows of w13 and bias13."""
+    SwiGLU with alpha and limit), interleaved gate / up rows of w13 and bias13. act_format "mxfp8":
+    activations re-quantized to MXFP8 instead of MXFP4 (hk_moe_mxfp4_a8_experts; pre-shuffled weights
+    only)."""
     T, H, I, E, layout, pw13, ps13, pitch13, pw2, ps2, pitch2 = _moe_weight_args(x, w13, w13_scales, w2, w2_scales, y)
     pb13, pb2, act, inter = _moe_ext_args(w13, E, H, I, bias13, bias2, activation, interleaved)
     _check_tensor(weights, "weights", _F32, 2)
@@ -395,16 +418,32 @@ def dispatch_moe_mxfp4_experts(x, w13, w13_scales, w2, w2_scales, weights, sorte
     if weights.shape[0] != T or sorted_slots.shape[0] != T * k or expert_offsets.shape[0] != E + 1 or \
             slot_to_pos.shape[0] != T * k:
         raise RuntimeError("shape mismatch between routing tensors")
-    st = _lib.load_library().hk_moe_mxfp4_experts_ex(
-        x.data_ptr(), pw13, ps13, pitch13, pw2, ps2, pitch2, weights.data_ptr(), sorted_slots.data_ptr(),
-        expert_offsets.data_ptr(), slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, layout,
-        pb13, pb2, act, float(alpha), float(limit), inter, workspace.data_ptr(), workspace.numel(), _stream(x))
+    if _a8(act_format, layout):
+        st = _lib.load_library().hk_moe_mxfp4_a8_experts(
+            x.data_ptr(), pw13, ps13, pw2, ps2, weights.data_ptr(), sorted_slots.data_ptr(),
+            expert_offsets.data_ptr(), slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k,
+            pb13, pb2, act, float(alpha), float(limit), inter, workspace.data_ptr(), workspace.numel(), _stream(x))
+    else:
+        st = _lib.load_library().hk_moe_mxfp4_experts_ex(
+            x.data_ptr(), pw13, ps13, pitch13, pw2, ps2, pitch2, weights.data_ptr(), sorted_slots.data_ptr(),
+            expert_offsets.data_ptr(), slot_to_pos.data_ptr(), y.data_ptr(), T, H, I, E, k, layout,
+            pb13, pb2, act, float(alpha), float(limit), inter, workspace.data_ptr(), workspace.numel(), _stream(x))
     _lib.check(st, "dispatch_moe_mxfp4_experts")
+
+
+def _a8(act_format: str, layout: int) -> bool:
+    if act_format == "mxfp4":
+        return False
+    if act_format != "mxfp8":
+        raise RuntimeError("act_format must be 'mxfp4' or 'mxfp8'")
+    if layout != 1:
+        raise RuntimeError("MXFP8 activations need pre-shuffled weights (MoeMxfp4ShuffledWeights)")
+    return True
 
 
 def dispatch_moe_mxfp4(x, router_logits, w13, w13_scales, w2, w2_scales, y, topk: int, workspace,
                        bias13=None, bias2=None, activation: str = "silu", alpha: float = 1.702,
-                       limit: float = 7.0, interleaved=None) -> None:
+                       limit: float = 7.0, interleaved=None, act_format: str = "mxfp4") -> None:
     """Whole MXFP4 MoE layer: top-k softmax routing, sort, expert MLP, un-permute into y. `w13` may be
     a MoeMxfp4ShuffledWeights (then pass None for w13_scales, w2, w2_scales). Options as in
     dispatch_moe_mxfp4_experts."""
@@ -414,10 +453,16 @@ def dispatch_moe_mxfp4(x, router_logits, w13, w13_scales, w2, w2_scales, y, topk
     _check_tensor(workspace, "workspace", (torch.uint8,), 1)
     if tuple(router_logits.shape) != (T, E):
         raise RuntimeError("router_logits must be [T, E]")
-    st = _lib.load_library().hk_moe_mxfp4_forward_ex(
-        x.data_ptr(), router_logits.data_ptr(), pw13, ps13, pitch13, pw2, ps2, pitch2, y.data_ptr(), T, H, I, E,
-        int(topk), layout, pb13, pb2, act, float(alpha), float(limit), inter, workspace.data_ptr(),
-        workspace.numel(), _stream(x))
+    if _a8(act_format, layout):
+        st = _lib.load_library().hk_moe_mxfp4_a8_forward(
+            x.data_ptr(), router_logits.data_ptr(), pw13, ps13, pw2, ps2, y.data_ptr(), T, H, I, E,
+            int(topk), pb13, pb2, act, float(alpha), float(limit), inter, workspace.data_ptr(),
+            workspace.numel(), _stream(x))
+    else:
+        st = _lib.load_library().hk_moe_mxfp4_forward_ex(
+            x.data_ptr(), router_logits.data_ptr(), pw13, ps13, pitch13, pw2, ps2, pitch2, y.data_ptr(), T, H, I, E,
+            int(topk), layout, pb13, pb2, act, float(alpha), float(limit), inter, workspace.data_ptr(),
+            workspace.numel(), _stream(x))
     _lib.check(st, "dispatch_moe_mxfp4")
 
 

@@ -274,6 +274,28 @@ int hk_moe_mxfp4_forward_ex(const void* x_bf16, const float* router_logits, cons
                             int activation, float alpha, float limit, int w13_interleaved,
                             void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same layer with MXFP8 activations (W4A8; no counterpart in the reference): x and h are
+ * re-quantized to e4m3 elements with one e8m0 scale per 32 (OCP MX rule: shared exponent
+ * floor(log2(amax)) - 8, elements rounded to nearest even and saturated at +-448) instead of e2m1,
+ * and the grouped GEMMs run the mixed MFMA (fp4 weights x fp8 activations). Weights must be in
+ * the pre-shuffled layout (outputs of hk_moe_mxfp4_preshuffle); the other arguments are those of
+ * hk_moe_mxfp4_experts_ex / hk_moe_mxfp4_forward_ex. The workspace is larger than for MXFP4
+ * activations (256 bytes per row and K-step): hk_moe_mxfp4_a8_workspace_bytes. */
+int hk_mxfp8_quantize_rows(const void* x_bf16, int rows, int cols, void* codes_e4m3, void* scales,
+                           int scale_pitch, void* stream);
+size_t hk_moe_mxfp4_a8_workspace_bytes(int T, int H, int I, int E, int k);
+int hk_moe_mxfp4_a8_experts(const void* x_bf16, const void* w13_shuffled, const void* w13_scales_shuffled,
+                            const void* w2_shuffled, const void* w2_scales_shuffled, const float* topk_w,
+                            const int32_t* sorted_slots, const int32_t* expert_offsets,
+                            const int32_t* slot_to_pos, void* y_bf16, int T, int H, int I, int E, int k,
+                            const float* bias13, const float* bias2, int activation, float alpha, float limit,
+                            int w13_interleaved, void* workspace, size_t workspace_bytes, void* stream);
+int hk_moe_mxfp4_a8_forward(const void* x_bf16, const float* router_logits, const void* w13_shuffled,
+                            const void* w13_scales_shuffled, const void* w2_shuffled,
+                            const void* w2_scales_shuffled, void* y_bf16, int T, int H, int I, int E, int k,
+                            const float* bias13, const float* bias2, int activation, float alpha, float limit,
+                            int w13_interleaved, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------- FP8 block-scaled fused MoE
  * No counterpart in the reference. DeepSeek-V3 style quantization:
  *   x          [T, H] e4m3, x_scales [T, H/128] fp32 (one scale per 1 x 128 block: x ~ q * s)

@@ -176,6 +176,33 @@ def quantize_mxfp4(x: np.ndarray):
     return packed, (e + 127).astype(np.uint8)
 
 
+def quantize_mxfp8(x: np.ndarray):
+    """OCP MX quantization along the last axis in blocks of 32 with e4m3 elements (MXFP8).
+
+    Shared exponent e = floor(log2(amax)) - 8 (8 = emax of e4m3: 448 = 1.75 * 2^8), clamped to
+    [-127, 127] and stored as e + 127; elements = e4m3(x / 2^e), round to nearest even,
+    saturating at +-448 (a block maximum in [1.75, 2) * 2^(e+8) saturates). amax == 0 -> byte 127.
+    Returns (codes uint8 [..., K], scales uint8 [..., K/32]). No counterpart in the reference
+    repository; the rule is the one of the OCP Microscaling Formats specification v1.0."""
+    x = np.asarray(x, dtype=np.float32)
+    K = x.shape[-1]
+    assert K % 32 == 0
+    blk = x.reshape(*x.shape[:-1], K // 32, 32)
+    amax = np.abs(blk).max(axis=-1)
+    _, ex = np.frexp(amax.astype(np.float64))
+    e = np.clip(ex - 1 - 8, -127, 127)
+    e = np.where(amax > 0, e, 0).astype(np.int32)
+    scaled = blk.astype(np.float64) * np.ldexp(1.0, -e)[..., None]
+    codes = e4m3_encode(scaled.astype(np.float32)).reshape(*x.shape[:-1], K)
+    return codes, (e + 127).astype(np.uint8)
+
+
+def dequantize_mxfp8(codes: np.ndarray, scales: np.ndarray) -> np.ndarray:
+    v = e4m3_decode(codes)
+    s = np.repeat(e8m0_decode(scales), 32, axis=-1)
+    return (v * s).astype(np.float32)
+
+
 def dequantize_mxfp4(packed: np.ndarray, scales: np.ndarray) -> np.ndarray:
     packed = np.asarray(packed, dtype=np.uint8)
     tbl = e2m1_decode_table()

@@ -118,6 +118,18 @@ def quantize_act_mxfp4(x: np.ndarray):
     return F.quantize_mxfp4(x)
 
 
+def quantize_act(x: np.ndarray, act_format: str):
+    """Activation quantizer of the MXFP4-weight MoE: MX blocks of 32 along the last axis with
+    e2m1 ("mxfp4") or e4m3 ("mxfp8") elements. Returns (data, scales, dequantized fp32)."""
+    if act_format == "mxfp4":
+        q, s = F.quantize_mxfp4(x)
+        return q, s, F.dequantize_mxfp4(q, s)
+    if act_format == "mxfp8":
+        q, s = F.quantize_mxfp8(x)
+        return q, s, F.dequantize_mxfp8(q, s)
+    raise ValueError(act_format)
+
+
 def swiglu_clamped(gate, up, alpha: float, limit: float):
     """The gated activation of the GPT-OSS experts (published model code: gate clamped from above,
     up clamped to [-limit, limit], glu = gate * sigmoid(alpha * gate), result (up + 1) * glu).
@@ -130,7 +142,7 @@ def swiglu_clamped(gate, up, alpha: float, limit: float):
 
 def moe_mxfp4_forward(x_bf16_as_f32, ids, w, w13_packed, w13_scales, w2_packed, w2_scales,
                       bias13=None, bias2=None, activation: str = "silu", alpha: float = 1.702,
-                      limit: float = 7.0, interleaved: bool = False):
+                      limit: float = 7.0, interleaved: bool = False, act_format: str = "mxfp4"):
     """Reference forward of the MXFP4 MoE. x [T,H] (bf16 values as fp32); ids/w [T,k];
     w13_packed [E, 2I, H/2], w13_scales [E, 2I, H/32]; w2_packed [E, H, I/2], w2_scales
     [E, H, I/32]. Returns (y as bf16 bits [T,H], dict of intermediates).
@@ -138,16 +150,16 @@ def moe_mxfp4_forward(x_bf16_as_f32, ids, w, w13_packed, w13_scales, w2_packed, 
     Model-faithful options (GPT-OSS): bias13 [E, 2I] / bias2 [E, H] fp32 added to the GEMM
     results before the activation / before the weighted sum; activation "swiglu_oai" =
     swiglu_clamped; interleaved: rows 2i / 2i+1 of w13 (and of bias13) are gate / up of column i
-    instead of rows i / I+i."""
+    instead of rows i / I+i. act_format "mxfp8": x and h are quantized to MXFP8 (e4m3 elements,
+    [S, I] codes in "hq") instead of MXFP4."""
     T, H = x_bf16_as_f32.shape
     E, twoI, _ = w13_packed.shape
     I = twoI // 2
     k = ids.shape[1]
     order, offs, inv = moe_sort(ids, E)
-    xq, xs = quantize_act_mxfp4(x_bf16_as_f32)
-    xd = F.dequantize_mxfp4(xq, xs)
+    xq, xs, xd = quantize_act(x_bf16_as_f32, act_format)
     S = T * k
-    hq = np.zeros((S, I // 2), dtype=np.uint8)
+    hq = np.zeros((S, I // 2 if act_format == "mxfp4" else I), dtype=np.uint8)
     hs = np.zeros((S, I // 32), dtype=np.uint8)
     o = np.zeros((S, H), dtype=np.float32)
     for e in range(E):
@@ -166,10 +178,10 @@ def moe_mxfp4_forward(x_bf16_as_f32, ids, w, w13_packed, w13_scales, w2_packed, 
             h = swiglu_clamped(gate, up, alpha, limit)
         else:
             raise ValueError(activation)
-        q, s = quantize_act_mxfp4(h)
+        q, s, hd = quantize_act(h, act_format)
         hq[lo:hi], hs[lo:hi] = q, s
         w2 = F.dequantize_mxfp4(w2_packed[e], w2_scales[e])
-        o[lo:hi] = F.dequantize_mxfp4(q, s) @ w2.T
+        o[lo:hi] = hd @ w2.T
         if bias2 is not None:
             o[lo:hi] += np.asarray(bias2[e], dtype=np.float32)[None, :]
     o_bf = F.bf16_to_f32(F.bf16_round(o))

@@ -123,6 +123,42 @@ def test_mx_quantize_error_bound_random():
     assert np.all(np.abs(d - x)[unsat] <= 1.0 * scale[unsat] + 1e-12)
 
 
+def test_mxfp8_quantize_rules_and_brute_force():
+    """MXFP8 (e4m3 elements, e8m0 per 32): the shared exponent is floor(log2(amax)) - 8, elements
+    round to the nearest e4m3 value (ties to the even code) and saturate at 448. Pinned by known
+    answers and by a brute-force nearest-value search over the 254 finite e4m3 codes."""
+    x = np.zeros((1, 96), dtype=np.float32)
+    x[0, 0] = 448.0; x[0, 1] = -1.0; x[0, 2] = 2.0 ** -9            # amax 448 -> e = 0
+    x[0, 32] = 500.0; x[0, 33] = 17.0                               # amax 500 -> e = 0: 500 saturates to 448
+    x[0, 64] = 512.0; x[0, 65] = 1.0                                # amax 512 -> e = 1: 256 exactly
+    c, s = F.quantize_mxfp8(x)
+    assert list(s[0]) == [127, 127, 128]
+    d = F.dequantize_mxfp8(c, s)
+    assert d[0, 0] == 448.0 and d[0, 1] == -1.0 and d[0, 2] == 2.0 ** -9
+    assert c[0, 0] == 0x7E and c[0, 1] == 0xB8
+    assert d[0, 32] == 448.0 and d[0, 33] == 16.0                   # 17 lies between 16 and 18: tie -> even mantissa
+    assert d[0, 64] == 512.0 and d[0, 65] == 1.0
+    z, sz = F.quantize_mxfp8(np.zeros((2, 32), dtype=np.float32))
+    assert not z.any() and np.all(sz == 127)
+    # brute force: nearest finite e4m3 value of x / 2^e, ties to the even code
+    rng = np.random.default_rng(8)
+    y = (rng.standard_normal((16, 64)) * np.exp2(rng.integers(-20, 20, size=(16, 1)))).astype(np.float32)
+    c, s = F.quantize_mxfp8(y)
+    tbl = F.e4m3_decode_table().astype(np.float64)
+    pos = np.array([i for i in range(0x7F)], dtype=np.int64)           # finite non-negative codes, ascending values
+    vals = tbl[pos]
+    amax = np.abs(y.reshape(16, 2, 32)).max(-1)
+    e = np.floor(np.log2(amax)).astype(np.int64) - 8
+    assert np.array_equal(s.astype(np.int64) - 127, e)
+    scaled = np.abs(y.astype(np.float64)) / np.repeat(np.exp2(e.astype(np.float64)), 32, axis=1)
+    for a, code in zip(scaled.ravel(), (c & 0x7F).ravel()):
+        dist = np.abs(vals - min(a, 448.0))
+        best = np.flatnonzero(dist == dist.min())
+        want = best[0] if len(best) == 1 else [b for b in best if b % 2 == 0][0]
+        assert code == want, (a, code, want)
+    assert np.array_equal((c >> 7).astype(bool), np.signbit(y))
+
+
 def test_block_quant_1x128_and_128x128():
     rng = np.random.default_rng(2)
     x = rng.standard_normal((130, 300)).astype(np.float32)

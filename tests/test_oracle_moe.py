@@ -130,6 +130,39 @@ def test_moe_mxfp4_forward_brute_force_tiny():
     assert np.allclose(got, F.bf16_to_f32(F.bf16_round(want)), rtol=2e-2, atol=1e-6)
 
 
+def test_moe_mxfp4_forward_mxfp8_activations_brute_force_tiny():
+    """act_format "mxfp8": the same token-by-token loop with the MXFP8 activation quantizer; and the
+    result lies closer to the forward pass on unquantized activations than the MXFP4 one does."""
+    rng = np.random.default_rng(14)
+    T, E, k, H, I = 8, 4, 2, 64, 32
+    x = F.bf16_to_f32(F.bf16_round(rng.standard_normal((T, H)).astype(np.float32)))
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    ids, w = O.topk_softmax(logits, k)
+    w13p, w13s = F.quantize_mxfp4((rng.standard_normal((E, 2 * I, H)) * 0.2).astype(np.float32))
+    w2p, w2s = F.quantize_mxfp4((rng.standard_normal((E, H, I)) * 0.2).astype(np.float32))
+    y8, mid = O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s, act_format="mxfp8")
+    y4, _ = O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s)
+    assert mid["hq"].shape == (T * k, I) and mid["xq"].shape == (T, H)
+    xd = F.dequantize_mxfp8(*F.quantize_mxfp8(x))
+    want = np.zeros((T, H), dtype=np.float32)
+    exact = np.zeros((T, H), dtype=np.float64)
+    for j in range(k):
+        for t in range(T):
+            e = ids[t, j]
+            W13, W2 = F.dequantize_mxfp4(w13p[e], w13s[e]), F.dequantize_mxfp4(w2p[e], w2s[e])
+            gu = xd[t:t + 1] @ W13.T
+            h = (O.silu(gu[:, :I]) * gu[:, I:]).astype(np.float32)
+            hd = F.dequantize_mxfp8(*F.quantize_mxfp8(h))
+            want[t] += w[t, j] * F.bf16_to_f32(F.bf16_round(hd @ W2.T))[0]
+            gx = x[t:t + 1].astype(np.float64) @ W13.T.astype(np.float64)
+            hx = gx[:, :I] / (1 + np.exp(-gx[:, :I])) * gx[:, I:]
+            exact[t] += w[t, j] * (hx @ W2.T.astype(np.float64))[0]
+    assert np.allclose(F.bf16_to_f32(y8), F.bf16_to_f32(F.bf16_round(want)), rtol=2e-2, atol=1e-6)
+    err8 = np.linalg.norm(F.bf16_to_f32(y8) - exact) / np.linalg.norm(exact)
+    err4 = np.linalg.norm(F.bf16_to_f32(y4) - exact) / np.linalg.norm(exact)
+    assert err8 < 0.5 * err4 and err8 < 0.1, (err8, err4)
+
+
 def test_moe_fp8blk_forward_single_expert_reduces_to_two_gemms():
     """E = 1, k = 1, w = 1: dequantize -> GEMM -> SiLU-mul -> 1x128 re-quantize -> GEMM, written out
     here with explicit per-block scale products instead of dequantized matrices."""
