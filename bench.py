@@ -44,7 +44,8 @@ PEAK_HBM = 8000.0     # GB/s
 # counter's reading for a 1 GiB copy (`bench.py --traffic-calibration`; factors 2.0 and 1.0). Sources:
 # profiles/fp8_gemm_4wave_ring_kernel_8192.md (805.8 MB read + 137.3 MB written).
 TRAFFIC_FP8_8192 = 943.1e6
-TRAFFIC = {}   # other legs: filled from profiles/ where a counter run exists (see _traffic)
+# Other legs: profiles/traffic_counters_moe_and_gemm_legs.md (MoE legs: sum over the layer's launches).
+TRAFFIC = {"moe_mxfp4": 2.195e9, "moe_fp8blk": 14.30e9, "mxfp4_gemm": 562.7e6, "bf16_gemm": 1.748e9}
 
 
 def _traffic(key):
