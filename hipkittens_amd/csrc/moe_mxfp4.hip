@@ -187,57 +187,68 @@ __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __r
 // 128-byte aligned runs for the global->LDS loads.
 //
 // Quantize-and-permute: row `pos` of the output is token sorted_slots[pos] / topk of x, so that
-// each expert's rows are contiguous for the grouped GEMM (the "permute" step of the MoE).
+// each expert's rows are contiguous for the grouped GEMM (the "permute" step of the MoE). The
+// kernel walks tokens, not output rows: a row of x is read and quantized once and stored to the
+// positions of the token's topk slots (slot_to_pos), instead of being fetched once per slot.
+// A slot's position is used only if sorted_slots maps it back to the slot (slots that took no
+// part in the sort have no position).
 // The same launch pads the second tiled matrix of the layer (h, contraction length K2): the part
 // of its last K-step past K2 that the producing GEMM epilogue never writes is set to zero data
 // and neutral scales (nothing to do when K2 is a multiple of 256).
-// Launch: 128 threads = 4 K-steps x 32 threads (8 elements each) for kQpRows rows; grid
-// (ceil(S / kQpRows) + 2, ceil(nk / 4)).
-// The two workgroups past the rows (blockIdx.y == 0) build the layer's two work-item lists instead, which
+// Launch: 128 threads = 4 K-steps x 32 threads (8 elements each) for kQpRows tokens; grid
+// (ceil(T / kQpRows) + 2, ceil(nk / 4)).
+// The two workgroups past the tokens (blockIdx.y == 0) build the layer's two work-item lists instead, which
 // need only expert_offsets and so ride along in the shadow of the quantization.
 // A8: MXFP8 activations (e4m3 elements): 256 bytes per row and K-step in both tiled matrices.
-constexpr int kQpRows = 4;   // rows per workgroup
+constexpr int kQpRows = 4;   // tokens per workgroup
 template <bool A8>
 __global__ __launch_bounds__(128) void mx_quantize_permute_kernel(
-    const uint16_t* __restrict__ x, const int32_t* __restrict__ sorted_slots, int topk, int S, int cols,
+    const uint16_t* __restrict__ x, const int32_t* __restrict__ sorted_slots,
+    const int32_t* __restrict__ slot_to_pos, int topk, int T, int cols,
     uint8_t* __restrict__ tiled, uint8_t* __restrict__ tiled_scales, uint8_t* __restrict__ tiled2,
     uint8_t* __restrict__ tiled2_scales, int K2, const int32_t* __restrict__ expert_offsets, int E,
     MoeBuildItems items, int32_t* __restrict__ num_items) {
     __shared__ int scan[128];
-    const int row_blocks = (S + kQpRows - 1) / kQpRows;
-    if ((int)blockIdx.x >= row_blocks) {
+    const int tok_blocks = (T + kQpRows - 1) / kQpRows;
+    if ((int)blockIdx.x >= tok_blocks) {
         if (blockIdx.y == 0)
-            moe_build_items_block<128>(expert_offsets, E, items, (int)blockIdx.x - row_blocks, num_items, scan);
+            moe_build_items_block<128>(expert_offsets, E, items, (int)blockIdx.x - tok_blocks, num_items, scan);
         return;
     }
+    const int S = T * topk;
     const int nk = (cols / 2 + 127) >> 7;
     const int kt = blockIdx.y * 4 + (threadIdx.x >> 5), c = threadIdx.x & 31;  // K-step, column of 8 elements
-    const int pos0 = blockIdx.x * kQpRows;
+    const int t0 = blockIdx.x * kQpRows;
+    // position of slot `slot`, or -1
+    auto position = [&](int slot) -> int {
+        const int pos = slot_to_pos[slot];
+        return (unsigned)pos < (unsigned)S && sorted_slots[pos] == slot ? pos : -1;
+    };
     if (blockIdx.y == 0 && threadIdx.x < 32 && (K2 & 255)) {
         const int nk2 = (K2 + 255) >> 8;
         const int valid = K2 - (nk2 - 1) * 256;  // valid elements of the last K-step, a multiple of 32
-        for (int j = 0; j < kQpRows && pos0 + j < S; ++j) {
-            const size_t tile_row2 = (size_t)(nk2 - 1) * S + pos0 + j;
-            if (c * 8 >= valid) {
-                if (A8) *(v2i*)(tiled2 + tile_row2 * 256 + c * 8) = v2i{0, 0};
-                else *(uint32_t*)(tiled2 + tile_row2 * 128 + c * 4) = 0u;
+        for (int j = 0; j < kQpRows && t0 + j < T; ++j)
+            for (int q = 0; q < topk; ++q) {
+                const int pos = position((t0 + j) * topk + q);
+                if (pos < 0) continue;
+                const size_t tile_row2 = (size_t)(nk2 - 1) * S + pos;
+                if (c * 8 >= valid) {
+                    if (A8) *(v2i*)(tiled2 + tile_row2 * 256 + c * 8) = v2i{0, 0};
+                    else *(uint32_t*)(tiled2 + tile_row2 * 128 + c * 4) = 0u;
+                }
+                if (c < 8 && c * 32 >= valid) tiled2_scales[tile_row2 * 8 + c] = 127;
             }
-            if (c < 8 && c * 32 >= valid) tiled2_scales[tile_row2 * 8 + c] = 127;
-        }
     }
     if (kt >= nk) return;
     const int col = kt * 256 + c * 8;
     // the loads of the workgroup's rows are issued together: a thread's 16 bytes per row are all it has in flight
-    int row[kQpRows];
-#pragma unroll
-    for (int j = 0; j < kQpRows; ++j) row[j] = sorted_slots[min(pos0 + j, S - 1)] / topk;
     v4i raw[kQpRows];
 #pragma unroll
     for (int j = 0; j < kQpRows; ++j)
-        raw[j] = col < cols ? *(const v4i*)(x + (size_t)row[j] * cols + col) : v4i{0, 0, 0, 0};
+        raw[j] = col < cols ? *(const v4i*)(x + (size_t)min(t0 + j, T - 1) * cols + col) : v4i{0, 0, 0, 0};
 #pragma unroll
     for (int j = 0; j < kQpRows; ++j) {
-        if (pos0 + j >= S) break;
+        if (t0 + j >= T) break;
         float v[8];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -250,10 +261,18 @@ __global__ __launch_bounds__(128) void mx_quantize_permute_kernel(
         amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
         amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
         const int e = A8 ? mx8_block_exponent(amax) : mx_block_exponent(amax);
-        const size_t tile_row = (size_t)kt * S + pos0 + j;
-        if (A8) *(v2i*)(tiled + tile_row * 256 + c * 8) = pack8_e4m3(v, e);
-        else *(uint32_t*)(tiled + tile_row * 128 + c * 4) = pack8_e2m1(v, e);
-        if ((c & 3) == 0) tiled_scales[tile_row * 8 + (c >> 2)] = (uint8_t)(e + 127);
+        v2i q8 = {0, 0};
+        uint32_t q4 = 0;
+        if (A8) q8 = pack8_e4m3(v, e);
+        else q4 = pack8_e2m1(v, e);
+        for (int q = 0; q < topk; ++q) {
+            const int pos = position((t0 + j) * topk + q);
+            if (pos < 0) continue;
+            const size_t tile_row = (size_t)kt * S + pos;
+            if (A8) *(v2i*)(tiled + tile_row * 256 + c * 8) = q8;
+            else *(uint32_t*)(tiled + tile_row * 128 + c * 4) = q4;
+            if ((c & 3) == 0) tiled_scales[tile_row * 8 + (c >> 2)] = (uint8_t)(e + 127);
+        }
     }
 }
 
@@ -1033,7 +1052,9 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
 // MFMAs and LDS reads on empty loads 148 / 78. The K loop hides behind the weight stream, the
 // epilogue does not: while a wave spends about 8 k clocks finishing an item, the three positions it
 // has in flight (about 6.6 k clocks of the stream) run dry. An epilogue copy per register set (four
-// times the code) cost another 7 %: the loop then no longer fits the instruction cache.
+// times the code) cost another 7 %: the loop then no longer fits the instruction cache. Requesting
+// the weights of one or two further positions into L2 at the start of an item's last position
+// (one dword per 64 bytes into a dump area of LDS) changed nothing / cost 2 %: not kept.
 //
 // A8: the activations are MXFP8 (e4m3 elements, 256 bytes per row and K-step, same e8m0 scale
 // layout) and the MFMA is the mixed form (fp4 weights x fp8 activations, 32 cycles). The
@@ -1694,9 +1715,9 @@ static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const voi
         b.items[0] = (MoeItem*)(ws + L.items1); b.items[1] = (MoeItem*)(ws + L.items2);
         b.n_tiles[0] = (I + 127) / 128; b.n_tiles[1] = (H + 255) / 256;
         auto qp = a8 ? mx_quantize_permute_kernel<true> : mx_quantize_permute_kernel<false>;
-        hipLaunchKernelGGL(qp, dim3((S + kQpRows - 1) / kQpRows + 2, (nk1 + 3) / 4), dim3(128), 0, s,
-                           (const uint16_t*)x_bf16, sorted_slots, k, S, H, ws + L.xq, ws + L.xs, ws + L.hq,
-                           ws + L.hs, I, expert_offsets, E, b, nitems);
+        hipLaunchKernelGGL(qp, dim3((T + kQpRows - 1) / kQpRows + 2, (nk1 + 3) / 4), dim3(128), 0, s,
+                           (const uint16_t*)x_bf16, sorted_slots, slot_to_pos, k, T, H, ws + L.xq, ws + L.xs,
+                           ws + L.hq, ws + L.hs, I, expert_offsets, E, b, nitems);
     }
 
     MoeGemmParams p{};
