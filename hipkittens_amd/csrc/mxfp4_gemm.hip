@@ -182,7 +182,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     for (int n = 0; n < NT; ++n) shift_scale(bs[0][n]);
     shift_scale(as[0]);  // as[1], as[2] are shifted inside the first step (groups 0 and 1)
 
-    // One K-step (slot plan of fp8_gemm_4wave_ring_kernel, fp8_gemm.hip, over two LDS stages). Scale handling: the raw
+    // One K-step (slot plan of gemm_ring.h over two LDS stages). Scale handling: the raw
     // 8 bytes of a fragment are read together with the fragment; the shift that exposes
     // this lane's byte is placed well after the read (B: group 7; A fragment f: group f-1).
     auto step = [&]<int P>(int kt) {
