@@ -91,6 +91,18 @@ def test_c_entry_points_reject_bad_arguments_without_a_gpu():
     assert lib.hk_moe_mxfp4_experts_ex(*args, None, None, 1, 1.702, 0.0, 0, p, 1 << 30, None) == -2   # limit <= 0
     assert lib.hk_moe_mxfp4_experts_ex(*args, p + 4, None, 0, 0.0, 0.0, 0, p, 1 << 30, None) == -3    # bias alignment
     assert lib.hk_moe_mxfp4_experts_ex(*args, None, None, 0, 0.0, 0.0, 0, None, 0, None) == -4        # workspace
+    # MXFP8-activation entry points (pre-shuffled weights only): same option and workspace checks
+    a8 = (p, p, p, p, p, p, p, p, p, p, 16, 64, 32, 4, 2)
+    assert lib.hk_moe_mxfp4_a8_experts(*a8, None, None, 7, 1.702, 7.0, 0, p, 1 << 30, None) == -6
+    assert lib.hk_moe_mxfp4_a8_experts(*a8, None, None, 0, 0.0, 0.0, 0, None, 0, None) == -4
+    assert lib.hk_moe_mxfp4_a8_experts(None, *a8[1:], None, None, 0, 0.0, 0.0, 0, p, 1 << 30, None) == -1
+    assert lib.hk_moe_mxfp4_a8_experts(*a8[:10], 16, 60, 32, 4, 2, None, None, 0, 0.0, 0.0, 0, p, 1 << 30, None) == -2  # H % 32
+    assert lib.hk_moe_mxfp4_a8_forward(p, None, p, p, p, p, p, 16, 64, 32, 4, 2, None, None, 0, 0.0, 0.0, 0, p, 1 << 30, None) == -1
+    assert lib.hk_moe_mxfp4_a8_workspace_bytes(16, 64, 32, 4, 2) > lib.hk_moe_mxfp4_workspace_bytes(16, 64, 32, 4, 2)
+    assert lib.hk_moe_mxfp4_a8_workspace_bytes(0, 64, 32, 4, 2) == 0
+    assert lib.hk_mxfp8_quantize_rows(p, 4, 48, p, p, 8, None) == -2          # cols % 32
+    assert lib.hk_mxfp8_quantize_rows(p, 4, 64, None, p, 8, None) == -1
+    assert lib.hk_mxfp8_quantize_rows(p, 4, 64, p, p, 4, None) == -2          # scale pitch % 8
     assert lib.hk_moe_unpermute_add(p, p, p, 4, 2, 60, None, p, None) == -2                            # H % 8
     assert lib.hk_moe_unpermute_add(p, p, p, 4, 2, 64, p + 2, p, None) == -3
 
