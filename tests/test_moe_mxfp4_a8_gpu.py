@@ -175,3 +175,51 @@ def test_moe_mxfp4_a8_needs_preshuffled_weights(hk):
     shuf = hk.tk_kernel.MoeMxfp4ShuffledWeights.from_plain(*tw)
     with pytest.raises(RuntimeError):
         hk.tk_kernel.dispatch_moe_mxfp4(x, lt, shuf, None, None, None, y, k, small, act_format="mxfp8")
+
+
+def test_moe_mxfp4_a8_full_shape_properties(hk):
+    """GPT-OSS-like shape (T=4096, H=I=2880, E=128, k=4) with MXFP8 activations: token-permutation
+    equivariance (bit for bit), the extended epilogue with zero biases and SiLU equals the plain
+    one (bit for bit: two instantiations of the kernel), and the oracle on 16 sampled tokens."""
+    T, E, k, H, I = 4096, 128, 4, 2880, 2880
+    print("moe_mxfp4 a8 full shape", flush=True)
+    g = torch.Generator(device=DEV).manual_seed(0)
+    x = torch.randn(T, H, device=DEV, generator=g).to(torch.bfloat16)
+    logits = torch.randn(T, E, device=DEV, generator=g)
+    w13p = torch.empty((E, 2 * I, H // 2), dtype=torch.uint8, device=DEV)
+    w13s = torch.empty((E, 2 * I, 96), dtype=torch.uint8, device=DEV)
+    w2p = torch.empty((E, H, I // 2), dtype=torch.uint8, device=DEV)
+    w2s = torch.empty((E, H, 96), dtype=torch.uint8, device=DEV)
+    for e in range(E):  # per expert, to bound temporaries
+        a, s = hk.quant.quantize_mxfp4(torch.randn(2 * I, H, device=DEV, generator=g) * 0.02)
+        w13p[e], w13s[e] = a, hk.quant.pad_scales(s)
+        a, s = hk.quant.quantize_mxfp4(torch.randn(H, I, device=DEV, generator=g) * 0.02)
+        w2p[e], w2s[e] = a, hk.quant.pad_scales(s)
+    shuf = hk.tk_kernel.MoeMxfp4ShuffledWeights.from_plain(w13p, w13s, w2p, w2s)
+    ws = torch.empty(hk.tk_kernel.moe_mxfp4_workspace_bytes(T, H, I, E, k, act_format="mxfp8"), dtype=torch.uint8,
+                     device=DEV)
+    run = lambda xx, ll, out, **kw: hk.tk_kernel.dispatch_moe_mxfp4(xx, ll, shuf, None, None, None, out, k, ws,
+                                                                   act_format="mxfp8", **kw)
+    y = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    run(x, logits, y)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all()
+    perm = torch.randperm(T, device=DEV, generator=g)
+    y2 = torch.empty_like(y)
+    run(x[perm].contiguous(), logits[perm].contiguous(), y2)
+    torch.cuda.synchronize()
+    assert torch.equal(y2, y[perm])
+    y3 = torch.empty_like(y)
+    run(x, logits, y3, bias13=torch.zeros((E, 2 * I), device=DEV), bias2=torch.zeros((E, H), device=DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(y3, y)
+    sel = torch.arange(0, T, T // 16, device=DEV)[:16]
+    ids, w = O.topk_softmax(logits[sel].cpu().numpy(), k)
+    used = np.unique(ids)
+    remap = {int(e): i for i, e in enumerate(used)}
+    ids_l = np.vectorize(remap.get)(ids).astype(np.int32)
+    ut = torch.from_numpy(used.astype(np.int64)).to(DEV)
+    want = F.bf16_to_f32(O.moe_mxfp4_forward(
+        x[sel].float().cpu().numpy(), ids_l, w, w13p[ut].cpu().numpy(), w13s[ut][:, :, :H // 32].cpu().numpy(),
+        w2p[ut].cpu().numpy(), w2s[ut][:, :, :I // 32].cpu().numpy(), act_format="mxfp8")[0])
+    assert G.rel_fro_error(y[sel].float().cpu().numpy(), want) <= TOL
