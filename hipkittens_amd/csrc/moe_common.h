@@ -26,6 +26,13 @@ __device__ __forceinline__ int moe_b_row(int mode, int R, int n_tile, int N, boo
 constexpr int kMoeBM = 128;
 struct MoeItem { int expert, row_start, rows, n_tile; };
 
+// SiLU(g) * u of the gate+up epilogues: g / (1 + exp(-g)) with the hardware exp2 and reciprocal
+// (about 1 ulp each; every grouped GEMM kernel of the two MoE layers uses this same sequence, which
+// is what keeps their results bit-identical to one another).
+__device__ __forceinline__ float silu_mul(float g, float u) {
+    return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
+}
+
 inline int moe_round_up(int x, int m) { return (x + m - 1) / m * m; }
 // Number of CUs of the current device (cached per device ordinal).
 int moe_num_compute_units();

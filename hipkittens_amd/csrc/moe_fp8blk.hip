@@ -319,7 +319,7 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const float gv = gt[j];
-                        h[m][4 * q + j] = gv / (1.0f + __expf(-gv)) * up[j];
+                        h[m][4 * q + j] = silu_mul(gv, up[j]);
                     }
                 }
                 float amax = 0.f;
@@ -404,7 +404,7 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
 //     K-steps ahead by direct global->LDS loads (gate+up: gathered from the caller's x by token);
 //   * the fp32 block scales are applied as before: every K-step's MFMAs write fresh partial sums,
 //     acc += partial * (x_scale[row] * w_scale), here with hand-placed instructions: the FMAs of an
-//     MFMA follow two MFMAs later, the next fragment's LDS reads and the loads of position + 4 are
+//     MFMA follow two MFMAs later, the next fragment's LDS reads and the loads of position + 3 are
 //     spread over the MFMA slots. One wave per SIMD issues one instruction per four cycles, which
 //     with 16 FMAs per fragment is as much as the MFMA pipe takes: no instruction is spent on
 //     branches in the main path: every K-step runs all ten fragments (rows past an item's count are
@@ -412,17 +412,22 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
 // The stream of (item, K-step) positions runs across item boundaries. All vector-memory loads are
 // inline asm and counted by hand: per position a wave issues 14 loads (5 activation pieces, the row
 // scales, 8 weight pieces; GATHER: 6 more per item for the slot ids), loads return in order, and the
-// wait for position p + 1 sits in step p behind the loads of position p + 4: vmcnt(3 x 14).
+// wait for position p + 1 sits in step p behind the loads of position p + 3: vmcnt(2 x 14). (Four
+// positions ahead on five stages measured the same.) An item takes nk4 positions, nk rounded up to
+// a multiple of the four register sets: its last position then always falls on set 3 and the
+// epilogue code exists once (with a copy per set the kernel is 139 KB of code and every epilogue
+// runs from a cold instruction cache). Padding positions fetch nothing: their LDS tile, row scales
+// and weight registers read as zeros and add nothing.
 // Results are bit-identical to the kernel above (same MFMA, K order and scaling FMAs).
 constexpr int kF8sMT = kF8BM / 16;                       // 10 row fragments per item
-constexpr int kF8sStages = 5;
+constexpr int kF8sStages = 4;                           // LDS stages = weight register sets = positions per trip of the K loop
 constexpr int kF8sStage = 21504;                         // 160 x 128 B, then 16 x 12 row scales, padded to a multiple of 256 B
 constexpr int kF8sXch = kF8sStages * kF8sStage;          // epilogue exchange buffer: 160 x 4 floats
-constexpr int kF8sLds = kF8sXch + kF8BM * 16;            // 107.5 KiB
+constexpr int kF8sLds = kF8sXch + kF8BM * 16;            // 86.5 KiB
 constexpr int kF8sBTile = 256 * 128;                     // one (n-tile, K-step) block of the pre-shuffled weights
 constexpr int kF8sLoads = 14;                            // loads per wave and position
 static_assert(kF8sStage >= kF8ATile + 16 * 12 * 4 && kF8sStage % 256 == 0 && kF8sLds <= 160 * 1024, "LDS plan");
-static_assert(3 * kF8sLoads < 64 && kF8sMT == 10, "vmcnt range; the slot plan below is written for ten fragments");
+static_assert((kF8sStages - 2) * kF8sLoads < 64 && kF8sStages == 4 && kF8sMT == 10, "vmcnt range; the slot plan below is written for ten fragments");
 
 // The weight ring lives in fixed accumulation registers: fragment F = 4 * set + n of the ring in
 // a[8 F .. 8 F + 7] (low / high K half in the first / last four). Naming them in the constraints keeps the two
@@ -467,6 +472,7 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
     if (it0 >= it_end) return;
 
     const int nk = p.K >> 7;
+    const int nk4 = (nk + kF8sStages - 1) / kF8sStages * kF8sStages;
     const v4i srd_a = make_srd(p.A, GATHER ? (uint32_t)p.T * (uint32_t)p.K : (uint32_t)nk * (uint32_t)p.S * 128u);
     const v4i srd_sa = make_srd(p.SA, GATHER ? (uint32_t)p.T * (uint32_t)nk * 4u : (uint32_t)nk * (uint32_t)p.S * 4u);
     // Activation tile: wave w fetches rows [40 w, +40) in five 1 KiB pieces of 8 rows; lane l lands in
@@ -485,9 +491,9 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
         c.expert = item.x; c.row_start = item.y; c.rows = item.z; c.n_tile = item.w;
     };
     auto advance = [&](F8Cursor& c) __attribute__((always_inline)) {
-        if (++c.kt == nk) { c.kt = 0; c.it += it_stride; load_item(c); }
+        if (++c.kt == nk4) { c.kt = 0; c.it += it_stride; load_item(c); }
     };
-    F8Cursor cc{it0, 0}, cn, cf;   // compute position, the one after it, fetch position (+4)
+    F8Cursor cc{it0, 0}, cn, cf;   // compute position, the one after it, fetch position (+3)
     load_item(cc);
     cn = cc; advance(cn);
     cf = cc;
@@ -530,9 +536,10 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
     int f_pieces;   // (not GATHER) pieces of this wave that hold rows of the item; the others fetch nothing
     auto fetch_begin = [&]() __attribute__((always_inline)) {
         f_srd_a = srd_a; f_srd_sa = srd_sa;
-                if (!cf.valid) { f_srd_a.z = 0; f_srd_sa.z = 0; }
+        const bool live = cf.valid && cf.kt < nk;   // not past the stream's end, not a padding position
+        if (!live) { f_srd_a.z = 0; f_srd_sa.z = 0; }
         f_srd_b = make_srd(p.B + (size_t)cf.expert * p.b_expert_stride + (size_t)cf.n_tile * nk * kF8sBTile,
-                           cf.valid ? (uint32_t)nk * kF8sBTile : 0u);
+                           live ? (uint32_t)nk * kF8sBTile : 0u);
         const uint32_t row_base = (uint32_t)cf.kt * (uint32_t)p.S + (uint32_t)cf.row_start;
         f_soff_a = GATHER ? (uint32_t)cf.kt * 128u : row_base * 128u;
         f_soff_sa = GATHER ? (uint32_t)cf.kt * 4u : row_base * 4u;
@@ -540,13 +547,13 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
         f_pieces = GATHER ? NA : (cf.rows - 40 * w + 7) >> 3;
     };
     auto fetch_advance = [&]() __attribute__((always_inline)) {
-        if (++cf.kt == nk) {
+        if (++cf.kt == nk4) {
             cf.kt = 0; cf.it += it_stride; load_item(cf);
             if (GATHER) {
                 // the ids were requested when the cursor entered the previous item, ahead of that
                 // position's loads, which an earlier step has waited for unless the item was shorter
                 // than the wait's reach
-                if (nk < 5) wait_vmcnt<0>();
+                if (nk4 < kF8sStages) wait_vmcnt<0>();
                 landed_ids(ids_next);
                 make_offsets(cf, ids_next);
                 issue_ids(cf.it + it_stride, ids_next);
@@ -559,7 +566,7 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
     const uint32_t lds_wave_sa = to_sgpr(lds0 + kF8ATile + (uint32_t)w * 192u);
     const uint32_t voff_b = lane * 16;
     struct BFrag { v4i lo, hi; };
-    BFrag bw[5][NT];   // weight fragments of five positions, in AGPRs
+    BFrag bw[kF8sStages][NT];   // weight fragments of four positions, in AGPRs
     // Load L (0..13) of the fetch position into LDS stage / register set PF. Order: an activation
     // piece or the scales, then a weight piece, alternating.
     auto fetch_load = [&]<int PF, int L>() __attribute__((always_inline)) {
@@ -642,46 +649,55 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
     // weight scales of a position, through the scalar cache, not waited for here
     auto request_ws = [&](const F8Cursor& c) __attribute__((always_inline)) {
         const float* sb = p.SB + (size_t)c.expert * p.sb_expert_stride;
+        const int kt = min(c.kt, nk - 1);   // a padding position multiplies zeros by the last K-step's scale
         const float* s0;
         const float* s1;
         if (MODE == 0) {
-            s0 = sb + (size_t)c.n_tile * nk + c.kt;                    // gate rows of the tile
-            s1 = sb + (size_t)(p.N / 128 + c.n_tile) * nk + c.kt;      // up rows
+            s0 = sb + (size_t)c.n_tile * nk + kt;                      // gate rows of the tile
+            s1 = sb + (size_t)(p.N / 128 + c.n_tile) * nk + kt;        // up rows
         } else {
-            s0 = sb + (size_t)min(2 * c.n_tile + (w >> 1), p.N / 128 - 1) * nk + c.kt;
+            s0 = sb + (size_t)min(2 * c.n_tile + (w >> 1), p.N / 128 - 1) * nk + kt;
             s1 = s0;
         }
         asm volatile("s_load_dword %0, %1, 0x0" : "=s"(ws0_next) : "s"(s0) : "memory");
         asm volatile("s_load_dword %0, %1, 0x0" : "=s"(ws1_next) : "s"(s1) : "memory");
     };
 
+    // Stores go through buffer descriptors that end at the item's last row: rows of the last
+    // fragments beyond it are dropped by the range check (no per-lane row test, no 64-bit address
+    // arithmetic); lanes that do not store carry bit 31 in their offset.
     auto epilogue = [&](const F8Cursor& a) __attribute__((always_inline)) {
-        const int rows = a.rows, row_start = a.row_start;
-        const int n0 = a.n_tile * (MODE == 0 ? 128 : 256);
         if (MODE == 1) {
-            uint16_t* out = (uint16_t*)p.out0;
+            // lane (r, g) holds, for row 16 m + r, the columns n0 + 64 w + 32 q + 8 g .. +8 (q = 0, 1)
+            const uint32_t pitch = (uint32_t)p.N * 2u;
+            const v4i srd = make_srd((uint8_t*)p.out0 + (size_t)a.row_start * pitch, (uint32_t)a.rows * pitch);
+            const int wcol0 = a.n_tile * 256 + w * 64;   // N % 128 == 0: a group of 32 columns is valid as a whole
+            const bool ok0 = wcol0 < p.N, ok1 = wcol0 + 32 < p.N;
+            uint32_t voff = r * pitch + (uint32_t)(wcol0 + 8 * (int)g) * 2u;
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
-                const int row = 16 * m + (int)r;
-                if (row >= rows) continue;
-                const size_t pos = (size_t)(row_start + row);
 #pragma unroll
                 for (int q = 0; q < NT / 2; ++q) {
-                    const int col = n0 + w * 64 + 32 * q + 8 * (int)g;
-                    if (col + 8 > p.N) continue;
                     const float (&x)[4] = acc[m][2 * q];
                     const float (&y)[4] = acc[m][2 * q + 1];
                     v4i o4;
                     o4.x = pack_bf16(x[0], x[1]); o4.y = pack_bf16(x[2], x[3]);
                     o4.z = pack_bf16(y[0], y[1]); o4.w = pack_bf16(y[2], y[3]);
-                    store_global_b128(out + pos * p.N + col, o4);
+                    if (q == 0 ? ok0 : ok1)
+                        asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen offset:%3\n\ts_nop 1"
+                                     :: "v"(o4), "v"(voff), "s"(srd), "n"(q * 64) : "memory");
                 }
+                voff += 16u * pitch;
             }
         } else {
             // h = silu(gate) * up for this wave's 32 of the tile's 128 h columns; the tile's 128
             // columns are one 1 x 128 quantization block, so the row maxima of the four waves are
             // combined through LDS.
-            uint8_t* hq = (uint8_t*)p.out0;
+            const size_t row0 = (size_t)a.n_tile * p.S + (size_t)a.row_start;
+            const v4i srd_h = make_srd((uint8_t*)p.out0 + row0 * 128, (uint32_t)a.rows * 128u);
+            const v4i srd_s = make_srd(p.out_scales + row0, (uint32_t)a.rows * 4u);
+            uint32_t voff_h = r * 128u + 32u * (uint32_t)w + 8u * g;
+            uint32_t voff_s = w == 0 && g == 0 ? r * 4u : 0x80000000u;
             float h[MT][8];
             const uint32_t xch = lds0 + kF8sXch;
 #pragma unroll
@@ -689,15 +705,16 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
 #pragma unroll
                 for (int q = 0; q < 2; ++q)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const float gv = acc[m][2 * q][j];
-                        h[m][4 * q + j] = gv / (1.0f + __expf(-gv)) * acc[m][2 * q + 1][j];
-                    }
+                    for (int j = 0; j < 4; ++j) h[m][4 * q + j] = silu_mul(acc[m][2 * q][j], acc[m][2 * q + 1][j]);
                 float amax = 0.f;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(h[m][i]));
-                amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+                // maximum over the four lanes (r, 0..3) of a row: rows of 16 lanes swapped in registers
+                const uint32_t am = __float_as_uint(amax);
+                const auto s16 = __builtin_amdgcn_permlane16_swap(am, am, false, false);
+                const uint32_t m1 = __float_as_uint(fmaxf(__uint_as_float(s16[0]), __uint_as_float(s16[1])));
+                const auto s32 = __builtin_amdgcn_permlane32_swap(m1, m1, false, false);
+                amax = fmaxf(__uint_as_float(s32[0]), __uint_as_float(s32[1]));
                 const int row = 16 * m + (int)r;
                 if (g == 0) *(lds_f32_mut_t*)(uintptr_t)(xch + (row * 4 + w) * 4) = amax;
             }
@@ -707,12 +724,11 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
                 const int row = 16 * m + (int)r;
                 const v4f am = *(lds_v4f_t*)(uintptr_t)(xch + row * 16);
                 const float s = e4m3_block_scale(fmaxf(fmaxf(am.x, am.y), fmaxf(am.z, am.w)));
-                if (row < rows) {
-                    const size_t tile_row = (size_t)a.n_tile * p.S + (size_t)(row_start + row);
-                    const v2i q8 = quant8_e4m3(h[m], s);
-                    asm volatile("global_store_dwordx2 %0, %1, off" ::"v"(hq + tile_row * 128 + 32 * w + 8 * g), "v"(q8) : "memory");
-                    if (w == 0 && g == 0) store_global_b32(p.out_scales + tile_row, __float_as_uint(s));
-                }
+                const v2i q8 = quant8_e4m3(h[m], s);
+                asm volatile("buffer_store_dwordx2 %0, %1, %2, 0 offen" :: "v"(q8), "v"(voff_h), "s"(srd_h) : "memory");
+                asm volatile("buffer_store_dword %0, %1, %2, 0 offen" :: "v"(s), "v"(voff_s), "s"(srd_s) : "memory");
+                voff_h += 16u * 128u;
+                voff_s += 16u * 4u;
             }
             __syncthreads();   // the exchange buffer is rewritten by the next item's epilogue
         }
@@ -730,10 +746,9 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
     fetch_begin(); fetch_all.template operator()<0>(); fetch_advance();
     fetch_begin(); fetch_all.template operator()<1>(); fetch_advance();
     fetch_begin(); fetch_all.template operator()<2>(); fetch_advance();
-    fetch_begin(); fetch_all.template operator()<3>(); fetch_advance();
     request_ws(cc);
     zero_acc();
-    wait_vmcnt<3 * kF8sLoads>();
+    wait_vmcnt<(kF8sStages - 2) * kF8sLoads>();
     block_barrier();
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     asm volatile("" : "+s"(ws0_next), "+s"(ws1_next));   // the requested scales are in their registers from here on
@@ -742,11 +757,11 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
     af[0] = lds_frag(rd_lo, rd_hi, 0);
     xs_r[0] = *(lds_f32_t*)(uintptr_t)rd_sa;
 
-    // One stream position on LDS stage / weight register set P (both = position % 5). Every position
+    // One stream position on LDS stage / weight register set P (both = position % 4). Every position
     // runs all ten fragments (rows past the item's count are zeros in LDS and are never stored): a
     // fragment count that varies would put the accumulators behind branches.
     auto step = [&]<int P>() __attribute__((always_inline)) {
-        constexpr int PF = (P + 4) % 5, PN = (P + 1) % 5;
+        constexpr int PF = (P + kF8sStages - 1) % kF8sStages, PN = (P + 1) % kF8sStages;
         fetch_begin();
         landed.template operator()<P>();
         const uint32_t a_lo = rd_lo + P * kF8sStage, a_hi = rd_hi + P * kF8sStage, a_sa = rd_sa + P * kF8sStage;
@@ -755,7 +770,7 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
         auto transition = [&]() __attribute__((always_inline)) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this position's last LDS reads and the scale request
             asm volatile("" : "+s"(ws0_next), "+s"(ws1_next));
-            wait_vmcnt<3 * kF8sLoads>();
+            wait_vmcnt<(kF8sStages - 2) * kF8sLoads>();
             block_barrier();   // everyone's part of the next position's tile has landed; everyone has read this position's
             af[0] = lds_frag(rd_lo + PN * kF8sStage, rd_hi + PN * kF8sStage, 0);
             xs_r[0] = *(lds_f32_t*)(uintptr_t)(rd_sa + PN * kF8sStage);
@@ -826,14 +841,16 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
             __builtin_amdgcn_sched_barrier(0);
         }
         fetch_advance();
-        if (cc.valid && cc.kt == nk - 1) {
-            // the item is complete: the two FMA groups still owed, then the epilogue
-            mfma_drain();
-            fma4(acc[MT - 1][2], part[2], sc[(MT - 1) & 1][0]);
-            fma4(acc[MT - 1][3], part[3], sc[(MT - 1) & 1][1]);
-            epilogue(cc);
-            zero_acc();
-            sc[(MT - 1) & 1][0] = 0.f; sc[(MT - 1) & 1][1] = 0.f;   // what the next K-step adds for "fragment 9 of the previous K-step"
+        if constexpr (P == kF8sStages - 1) {
+            if (cc.valid && cc.kt == nk4 - 1) {
+                // the item is complete: the two FMA groups still owed, then the epilogue
+                mfma_drain();
+                fma4(acc[MT - 1][2], part[2], sc[(MT - 1) & 1][0]);
+                fma4(acc[MT - 1][3], part[3], sc[(MT - 1) & 1][1]);
+                epilogue(cc);
+                zero_acc();
+                sc[(MT - 1) & 1][0] = 0.f; sc[(MT - 1) & 1][1] = 0.f;   // what the next K-step adds for "fragment 9 of the previous K-step"
+            }
         }
         cc = cn;
         advance(cn);
@@ -845,7 +862,6 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
         step.template operator()<1>();
         step.template operator()<2>();
         step.template operator()<3>();
-        step.template operator()<4>();
     }
     wait_vmcnt<0>();   // nothing may still be writing LDS when the workgroup retires
 }

@@ -67,11 +67,6 @@ __device__ __forceinline__ v2i pack8_e4m3(const float (&v)[8], int e) {
     hi = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(hi, c[6], c[7], scale, true);
     return v2i{__builtin_bit_cast(int, lo), __builtin_bit_cast(int, hi)};
 }
-// SiLU(g) * u of the gate+up epilogue: g / (1 + exp(-g)) with the hardware exp2 and reciprocal
-// (about 1 ulp each; both grouped GEMM kernels use this same sequence).
-__device__ __forceinline__ float silu_mul(float g, float u) {
-    return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
-}
 // Gated activation of the extended epilogues. act 0: SiLU(g) * u; act 1: the clamped SwiGLU of
 // the GPT-OSS experts, (clamp(u, -limit, limit) + 1) * g' * sigmoid(alpha * g') with
 // g' = min(g, limit).
