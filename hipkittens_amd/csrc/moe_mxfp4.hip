@@ -1693,6 +1693,10 @@ static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const voi
     int st = moe_mxfp4_check(T, H, I, E, k, weight_layout ? moe_round_up(H / 32, 8) : w13_scale_pitch,
                              weight_layout ? moe_round_up(I / 32, 8) : w2_scale_pitch);
     if (st != HK_OK) return st;
+    // MXFP8 activation tiles are twice as large: their 32-bit buffer offsets must still fit
+    if (a8 && ((long long)T * k * ((H + 255) / 256 * 256) >= (1ll << 31) ||
+               (long long)T * k * ((I + 255) / 256 * 256) >= (1ll << 31)))
+        return HK_ERR_BAD_SHAPE;
     const MoeWs L = moe_ws_layout(T, H, I, E, k, a8);
     if (!workspace || workspace_bytes < L.total) return HK_ERR_WORKSPACE;
     if (((uintptr_t)x_bf16 | (uintptr_t)w13 | (uintptr_t)w2 | (uintptr_t)y_bf16 | (uintptr_t)workspace) & 15u)

@@ -98,6 +98,9 @@ def test_c_entry_points_reject_bad_arguments_without_a_gpu():
     assert lib.hk_moe_mxfp4_a8_experts(None, *a8[1:], None, None, 0, 0.0, 0.0, 0, p, 1 << 30, None) == -1
     assert lib.hk_moe_mxfp4_a8_experts(*a8[:10], 16, 60, 32, 4, 2, None, None, 0, 0.0, 0.0, 0, p, 1 << 30, None) == -2  # H % 32
     assert lib.hk_moe_mxfp4_a8_forward(p, None, p, p, p, p, p, 16, 64, 32, 4, 2, None, None, 0, 0.0, 0.0, 0, p, 1 << 30, None) == -1
+    # 1 M rows x 2880: the MXFP4 tiles fit 32-bit offsets, the MXFP8 ones do not
+    big = (p, p, p, p, p, p, p, p, p, p, 250000, 2880, 2880, 128, 4)
+    assert lib.hk_moe_mxfp4_a8_experts(*big, None, None, 0, 0.0, 0.0, 0, p, 1 << 50, None) == -2
     assert lib.hk_moe_mxfp4_a8_workspace_bytes(16, 64, 32, 4, 2) > lib.hk_moe_mxfp4_workspace_bytes(16, 64, 32, 4, 2)
     assert lib.hk_moe_mxfp4_a8_workspace_bytes(0, 64, 32, 4, 2) == 0
     assert lib.hk_mxfp8_quantize_rows(p, 4, 48, p, p, 8, None) == -2          # cols % 32
