@@ -213,11 +213,9 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
 extern "C" int hk_bf16_gemm(const void* A, const void* B, void* C, int M, int N, int K, void* stream) {
     using namespace hk;
     const bool tile_ok = K > 0 && (long long)2 * K * BM < (1ll << 31);
-    // the same choice of tile as hk_fp8_gemm: the largest that still gives every CU work
-    const long long tiles256 = (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-    const long long tiles128 =
-        (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
-    const int variant = !tile_ok ? 0 : tiles128 <= 128 ? 3 : tiles256 < 128 ? 2 : 1;
+    // the same choice of tile as hk_fp8_gemm (pick_tile), with this format's measured corrections
+    const int tile = pick_tile(M, N, (int)((2ll * K + BK - 1) / BK), TileRule{32, 64, 96});
+    const int variant = !tile_ok ? 0 : tile == kTinyTile ? 3 : tile == kSmallTile ? 2 : 1;
     return hk_bf16_gemm_variant(A, B, C, M, N, K, variant, stream);
 }
 

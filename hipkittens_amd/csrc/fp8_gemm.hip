@@ -276,12 +276,8 @@ extern "C" int hk_fp8_gemm(const void* A, const void* B, void* C, int M, int N, 
                            float scale_a, float scale_b, void* stream) {
     using namespace hk;
     const bool tile_ok = K > 0 && (long long)K * BM < (1ll << 31);
-    // The tile is the largest that still gives every CU of an MI355X work: 256x256 (five-slot ring
-    // kernel) from 128 such tiles on; below that 128x128 tiles, and 64x64 tiles (two workgroups
-    // per CU) when even those number at most 128.
-    const long long tiles256 = (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-    const long long tiles128 =
-        (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
-    const int variant = !tile_ok ? 0 : tiles128 <= 128 ? 6 : tiles256 < 128 ? 5 : 4;
+    // 256x256 tiles (five-slot ring kernel), 128x128 or 64x64: see pick_tile
+    const int tile = pick_tile(M, N, (K + BK - 1) / BK, TileRule{16, 32, 80});
+    const int variant = !tile_ok ? 0 : tile == kTinyTile ? 6 : tile == kSmallTile ? 5 : 4;
     return hk_fp8_gemm_variant(A, B, C, M, N, K, scale_a, scale_b, variant, stream);
 }

@@ -233,6 +233,29 @@ static __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* 
     }
 }
 
+// Which tile a GEMM gets when the caller does not pin a kernel: 256 (the large-tile kernels), 128 or
+// 64. The rule is the largest tile that still gives every CU of an MI355X work: 64x64 tiles (two
+// workgroups per CU) when 128x128 tiles number at most 128, else 128x128 tiles below 128 tiles of
+// 256x256. Two corrections measured on a grid of 110 shapes per format (M 16..8192, N and K
+// 1024..14336), in K-steps of the format's kernels (nk):
+//  - with exactly 128 large tiles and a K of at most `short_nk` steps the 128x128 tile is 2-10 % faster
+//    (prologue and epilogue are a large share of so short a loop, and 512 small tiles overlap them);
+//  - from `long_tiles` large tiles on, a K of at least `long_nk` steps runs 3-15 % faster on the
+//    large-tile kernel although some CUs idle: its K loop moves half the LDS bytes per flop
+//    (long_tiles 0: never, the format's two kernels tie there).
+struct TileRule {
+    int short_nk, long_nk, long_tiles;
+};
+static inline int pick_tile(int M, int N, int nk, TileRule r) {
+    const long long tiles256 = (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    const long long tiles128 =
+        (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
+    if (tiles128 <= 128) return kTinyTile;
+    if (tiles256 > 128) return BM;
+    if (tiles256 == 128) return nk <= r.short_nk ? kSmallTile : BM;
+    return r.long_tiles > 0 && tiles256 >= r.long_tiles && nk >= r.long_nk ? BM : kSmallTile;
+}
+
 int moe_num_compute_units();  // number of CUs of the current device, cached (moe_mxfp4.hip)
 
 // Number of K ranges the split-K path would use: as many as fill the CUs, each at least 4

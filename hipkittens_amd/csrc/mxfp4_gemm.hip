@@ -445,11 +445,9 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
                           ((((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) == 0);
     const bool size_ok = (long long)(K / 2) * BM < (1ll << 31) && (long long)BM * max(sa_pitch, sb_pitch) < (1ll << 31);
     if (variant < 0) {
-        // the largest tile that still gives every CU work, as in hk_fp8_gemm
-        const long long tiles256 = (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-        const long long tiles128 =
-            (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
-        variant = !(pitch_ok && size_ok) ? 0 : tiles128 <= 128 ? 3 : tiles256 < 128 ? 2 : 1;
+        // the choice of tile of hk_fp8_gemm (pick_tile); a K-step is 256 elements here
+        const int tile = pick_tile(M, N, (K / 2 + BK - 1) / BK, TileRule{8, 0, 0});
+        variant = !(pitch_ok && size_ok) ? 0 : tile == kTinyTile ? 3 : tile == kSmallTile ? 2 : 1;
     }
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {

@@ -80,7 +80,8 @@ int hk_fp8_gemm_static_ws(const void* A_e4m3, const void* B_e4m3, void* C_bf16, 
  * reference's second FP8 schedule, kernels/gemm/fp8fp32/README.md:3-5, schedule of
  * kernels/gemm/bf16fp32/mi325x/256_256_64_16.cpp:73-155), 4 = 256x256x128 tile, 4 waves,
  * hand-interleaved schedule over a five-slot LDS ring with the loads spread over the whole K-step
- * (what hk_fp8_gemm picks when the problem has at least 128 such tiles), 5 = 128x128x128 tile, 4
+ * (what hk_fp8_gemm picks when the problem has more than 128 such tiles, or 80 to 128 of them and
+ * K >= 4096, or exactly 128 and K > 2048), 5 = 128x128x128 tile, 4
  * waves, plain loop over three LDS stages (picked for smaller problems), 6 = the same loop with
  * 64x64 tiles and four stages, two workgroups per CU (picked when the problem has at most 128
  * tiles of 128x128). 2 and 3 are not in use (HK_ERR_UNSUPPORTED). All tile kernels zero-fill the last
