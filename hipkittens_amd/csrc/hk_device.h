@@ -81,6 +81,22 @@ __device__ __forceinline__ void dma16_lanes(v4i srd, uint32_t lds_base, uint32_t
         : "memory", "m0");
 }
 
+// dma4 restricted to the lanes set in `mask` (lane l still lands at lds_base + 4*l).
+__device__ __forceinline__ void dma4_lanes(v4i srd, uint32_t lds_base, uint32_t voff, uint32_t soff,
+                                           uint64_t mask) {
+    uint64_t saved;
+    asm volatile(
+        "s_mov_b64 %0, exec\n\t"
+        "s_mov_b64 exec, %5\n\t"
+        "s_mov_b32 m0, %1\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dword %2, %3, %4 offen lds\n\t"
+        "s_mov_b64 exec, %0"
+        : "=&s"(saved)
+        : "s"(lds_base), "v"(voff), "s"(srd), "s"(soff), "s"(mask)
+        : "memory", "m0");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");

@@ -94,22 +94,6 @@ constexpr int kF8Lds = kF8ScaleBase + 3 * kF8BM * 4;   // 157.9 KiB
 // (the gate+up epilogue's exchange buffer, kF8BM x 4 floats, lies in the stage the K loop used last)
 static_assert(kF8Lds <= 160 * 1024 && kF8BM % 32 == 0 && kF8BM > 128 && kF8BM <= 192, "see the A-tile loads");
 
-// dword global->LDS load restricted to the lanes in `mask` (lane l lands at lds_base + 4*l)
-__device__ __forceinline__ void dma4_lanes(v4i srd, uint32_t lds_base, uint32_t voff, uint32_t soff,
-                                           uint64_t mask) {
-    uint64_t saved;
-    asm volatile(
-        "s_mov_b64 %0, exec\n\t"
-        "s_mov_b64 exec, %5\n\t"
-        "s_mov_b32 m0, %1\n\t"
-        "s_nop 0\n\t"
-        "buffer_load_dword %2, %3, %4 offen lds\n\t"
-        "s_mov_b64 exec, %0"
-        : "=&s"(saved)
-        : "s"(lds_base), "v"(voff), "s"(srd), "s"(soff), "s"(mask)
-        : "memory", "m0");
-}
-
 struct MoeFp8Addr {
     v4i srd_b;
     uint32_t voff_b[4];

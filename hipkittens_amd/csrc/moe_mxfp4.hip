@@ -14,6 +14,7 @@
 // path: weights go straight from HBM into MFMA operand registers, 192-row m-tiles) and
 // moe_mxfp4_gemm_kernel for the plain layout (both operands through an LDS ring, 128-row m-tiles).
 #include "moe_common.h"
+#include "moe_sort.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -120,24 +121,21 @@ __global__ __launch_bounds__(256) void mx_quantize_rows_kernel(const uint16_t* _
 // threads per list; thread t owns experts [t * 512 / NT, (t + 1) * 512 / NT). `scan`: NT ints of LDS.
 // With nparts > 1 workgroups per list, workgroup `part` writes the n-tiles part, part + nparts, ...
 struct MoeBuildItems { MoeItem* items[2]; int n_tiles[2]; int bm; };
+// moe_build_items_ranges: the same from the experts' row ranges [lo[j], hi[j]) held by the threads
+// (thread t: experts t * 512 / NT + j).
 template <int NT>
-__device__ __forceinline__ void moe_build_items_block(const int32_t* __restrict__ expert_offsets, int E,
-                                                      const MoeBuildItems& b, int which,
-                                                      int32_t* __restrict__ num_items, int* scan,
-                                                      int part = 0, int nparts = 1) {
+__device__ __forceinline__ void moe_build_items_ranges(const int (&lo)[512 / NT], const int (&hi)[512 / NT], int E,
+                                                       const MoeBuildItems& b, int which,
+                                                       int32_t* __restrict__ num_items, int* scan,
+                                                       int part = 0, int nparts = 1) {
     constexpr int EPT = 512 / NT;
     const int n_tiles_n = b.n_tiles[which], bm = b.bm;
     MoeItem* __restrict__ items = b.items[which];
     const int t = threadIdx.x;
-    int lo[EPT], hi[EPT], cnt[EPT], mine = 0;
+    int cnt[EPT], mine = 0;
 #pragma unroll
     for (int j = 0; j < EPT; ++j) {
-        const int e = t * EPT + j;
-        lo[j] = hi[j] = cnt[j] = 0;
-        if (e < E) {
-            lo[j] = expert_offsets[e]; hi[j] = expert_offsets[e + 1];
-            cnt[j] = (hi[j] - lo[j] + bm - 1) / bm;
-        }
+        cnt[j] = t * EPT + j < E ? (hi[j] - lo[j] + bm - 1) / bm : 0;
         mine += cnt[j] * n_tiles_n;
     }
     scan[t] = mine;
@@ -167,6 +165,21 @@ __device__ __forceinline__ void moe_build_items_block(const int32_t* __restrict_
     }
     if (t == NT - 1 && part == 0) num_items[which] = scan[NT - 1];
 }
+template <int NT>
+__device__ __forceinline__ void moe_build_items_block(const int32_t* __restrict__ expert_offsets, int E,
+                                                      const MoeBuildItems& b, int which,
+                                                      int32_t* __restrict__ num_items, int* scan,
+                                                      int part = 0, int nparts = 1) {
+    constexpr int EPT = 512 / NT;
+    int lo[EPT], hi[EPT];
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+        const int e = threadIdx.x * EPT + j;
+        lo[j] = e < E ? expert_offsets[e] : 0;
+        hi[j] = e < E ? expert_offsets[e + 1] : 0;
+    }
+    moe_build_items_ranges<NT>(lo, hi, E, b, which, num_items, scan, part, nparts);
+}
 
 __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __restrict__ expert_offsets,
                                                               int E, MoeBuildItems b,
@@ -192,34 +205,42 @@ __global__ __launch_bounds__(512) void moe_build_items_kernel(const int32_t* __r
 // and neutral scales (nothing to do when K2 is a multiple of 256).
 // Launch: 128 threads = 4 K-steps x 32 threads (8 elements each) for kQpRows tokens; grid
 // (ceil(T / kQpRows) + 2, ceil(nk / 4)).
-// The two workgroups past the tokens (blockIdx.y == 0) build the layer's two work-item lists instead, which
-// need only expert_offsets and so ride along in the shadow of the quantization.
+// The two columns of workgroups past the tokens build the layer's two work-item lists instead (the
+// gridDim.y workgroups of a column share a list's n-tiles), which need only expert_offsets and so
+// ride along in the shadow of the quantization.
 // A8: MXFP8 activations (e4m3 elements): 256 bytes per row and K-step in both tiled matrices.
+// PERMUTE false: no permutation, one output row per token (data [nk][T][..]; the 4-wave streaming
+// kernel gathers its rows by token and needs neither the topk copies of a row nor the sort's result
+// here: sorted_slots / slot_to_pos are not read), and the scales of 16 K-steps share a 128-byte row:
+// scales [ceil(nk / 16)][T][128], K-step kt at byte 8 (kt % 16) of the row of super-step kt / 16.
 constexpr int kQpRows = 4;   // tokens per workgroup
-template <bool A8>
-__global__ __launch_bounds__(128) void mx_quantize_permute_kernel(
-    const uint16_t* __restrict__ x, const int32_t* __restrict__ sorted_slots,
-    const int32_t* __restrict__ slot_to_pos, int topk, int T, int cols,
-    uint8_t* __restrict__ tiled, uint8_t* __restrict__ tiled_scales, uint8_t* __restrict__ tiled2,
-    uint8_t* __restrict__ tiled2_scales, int K2, const int32_t* __restrict__ expert_offsets, int E,
-    MoeBuildItems items, int32_t* __restrict__ num_items) {
-    __shared__ int scan[128];
-    const int tok_blocks = (T + kQpRows - 1) / kQpRows;
-    if ((int)blockIdx.x >= tok_blocks) {
-        if (blockIdx.y == 0)
-            moe_build_items_block<128>(expert_offsets, E, items, (int)blockIdx.x - tok_blocks, num_items, scan);
-        return;
-    }
+struct MxQuantizeArgs {
+    const uint16_t* x; const int32_t* sorted_slots; const int32_t* slot_to_pos;
+    int topk, T, cols;
+    uint8_t* tiled; uint8_t* tiled_scales; uint8_t* tiled2; uint8_t* tiled2_scales;
+    int K2;
+};
+// The work of 32 threads (c = 0..31: 8 elements each) on K-step kt of tokens t0 .. t0 + kQpRows - 1;
+// `pad` set for one group of 32 threads per token block: it also pads the second matrix.
+template <bool A8, bool PERMUTE>
+__device__ __forceinline__ void mx_quantize_tokens(const MxQuantizeArgs& a, int t0, int kt, int c, bool pad) {
+    const int T = a.T, topk = a.topk, cols = a.cols, K2 = a.K2;
+    const uint16_t* __restrict__ x = a.x;
+    const int32_t* __restrict__ sorted_slots = a.sorted_slots;
+    const int32_t* __restrict__ slot_to_pos = a.slot_to_pos;
+    uint8_t* __restrict__ tiled = a.tiled;
+    uint8_t* __restrict__ tiled_scales = a.tiled_scales;
+    uint8_t* __restrict__ tiled2 = a.tiled2;
+    uint8_t* __restrict__ tiled2_scales = a.tiled2_scales;
     const int S = T * topk;
     const int nk = (cols / 2 + 127) >> 7;
-    const int kt = blockIdx.y * 4 + (threadIdx.x >> 5), c = threadIdx.x & 31;  // K-step, column of 8 elements
-    const int t0 = blockIdx.x * kQpRows;
     // position of slot `slot`, or -1
     auto position = [&](int slot) -> int {
+        if (!PERMUTE) return slot;
         const int pos = slot_to_pos[slot];
         return (unsigned)pos < (unsigned)S && sorted_slots[pos] == slot ? pos : -1;
     };
-    if (blockIdx.y == 0 && threadIdx.x < 32 && (K2 & 255)) {
+    if (pad && (K2 & 255)) {
         const int nk2 = (K2 + 255) >> 8;
         const int valid = K2 - (nk2 - 1) * 256;  // valid elements of the last K-step, a multiple of 32
         for (int j = 0; j < kQpRows && t0 + j < T; ++j)
@@ -260,15 +281,71 @@ __global__ __launch_bounds__(128) void mx_quantize_permute_kernel(
         uint32_t q4 = 0;
         if (A8) q8 = pack8_e4m3(v, e);
         else q4 = pack8_e2m1(v, e);
-        for (int q = 0; q < topk; ++q) {
-            const int pos = position((t0 + j) * topk + q);
+        for (int q = 0; q < (PERMUTE ? topk : 1); ++q) {
+            const int pos = PERMUTE ? position((t0 + j) * topk + q) : t0 + j;
             if (pos < 0) continue;
-            const size_t tile_row = (size_t)kt * S + pos;
+            const size_t tile_row = (size_t)kt * (PERMUTE ? S : T) + pos;
             if (A8) *(v2i*)(tiled + tile_row * 256 + c * 8) = q8;
             else *(uint32_t*)(tiled + tile_row * 128 + c * 4) = q4;
-            if ((c & 3) == 0) tiled_scales[tile_row * 8 + (c >> 2)] = (uint8_t)(e + 127);
+            if ((c & 3) == 0) {
+                if (PERMUTE) tiled_scales[tile_row * 8 + (c >> 2)] = (uint8_t)(e + 127);
+                else tiled_scales[((size_t)(kt >> 4) * T + pos) * 128 + (kt & 15) * 8 + (c >> 2)] = (uint8_t)(e + 127);
+            }
         }
     }
+}
+
+template <bool A8, bool PERMUTE>
+__global__ __launch_bounds__(128) void mx_quantize_permute_kernel(MxQuantizeArgs a,
+                                                                  const int32_t* __restrict__ expert_offsets, int E,
+                                                                  MoeBuildItems items, int32_t* __restrict__ num_items) {
+    __shared__ int scan[128];
+    const int tok_blocks = (a.T + kQpRows - 1) / kQpRows;
+    if ((int)blockIdx.x >= tok_blocks) {
+        // list blockIdx.x - tok_blocks, its n-tiles shared by the gridDim.y workgroups of this column
+        moe_build_items_block<128>(expert_offsets, E, items, (int)blockIdx.x - tok_blocks, num_items, scan,
+                                   blockIdx.y, gridDim.y);
+        return;
+    }
+    mx_quantize_tokens<A8, PERMUTE>(a, blockIdx.x * kQpRows, blockIdx.y * 4 + (threadIdx.x >> 5), threadIdx.x & 31,
+                                    blockIdx.y == 0 && threadIdx.x < 32);
+}
+
+// One launch for a layer of at most kSortSmallMax slots whose gate+up kernel gathers its rows by
+// token: the sort of the slots (moe_sort_small_block, workgroups [0, nchunks)), the layer's two
+// work-item lists (2 * kFusedItemParts workgroups: each repeats the sort's histogram and scan, which
+// gives it the experts' row ranges without waiting for anyone, and writes a share of one list) and
+// the quantization of x (the remaining workgroups: 8 K-steps x 32 threads for kQpRows tokens), which
+// needs nothing from the sort. The quantization then costs the layer no time of its own.
+constexpr int kFusedItemParts = 4;
+template <bool A8>
+__global__ __launch_bounds__(256) void moe_sort_quantize_kernel(const int32_t* __restrict__ ids, int E,
+                                                                int32_t* __restrict__ expert_offsets,
+                                                                int32_t* __restrict__ sorted_slots,
+                                                                int32_t* __restrict__ slot_to_pos, MxQuantizeArgs a,
+                                                                MoeBuildItems items, int32_t* __restrict__ num_items) {
+    __shared__ MoeSortSmallLds lds;
+    const int S = a.T * a.topk;
+    const int nchunks = (S + kSortChunk - 1) / kSortChunk;
+    int b = blockIdx.x;
+    int lo[2], hi[2];
+    if (b < nchunks) {
+        moe_sort_small_block(ids, S, E, b, true, expert_offsets, sorted_slots, slot_to_pos, lds, lo, hi);
+        return;
+    }
+    b -= nchunks;
+    if (b < 2 * kFusedItemParts) {
+        moe_sort_small_block(ids, S, E, nchunks, false, expert_offsets, sorted_slots, slot_to_pos, lds, lo, hi);
+        __syncthreads();   // the scan array below reuses the sort's LDS
+        moe_build_items_ranges<256>(lo, hi, E, items, b / kFusedItemParts, num_items, &lds.round_cnt[0][0],
+                                    b % kFusedItemParts, kFusedItemParts);
+        return;
+    }
+    b -= 2 * kFusedItemParts;
+    const int nk = (a.cols / 2 + 127) >> 7, kgroups = (nk + 7) / 8;
+    const int kg = b % kgroups;
+    mx_quantize_tokens<A8, false>(a, (b / kgroups) * kQpRows, kg * 8 + (threadIdx.x >> 5), threadIdx.x & 31,
+                                  kg == 0 && threadIdx.x < 32);
 }
 
 // ---------------------------------------------------------------------- weight pre-shuffle
@@ -339,6 +416,11 @@ struct MoeGemmParams {
     long long b_expert_stride, sb_expert_stride;
     int b_pitch, sb_pitch;   // plain weight layout only
     int S;                   // rows of the activation matrices (T * topk)
+    // Gathered activations (the 4-wave streaming kernel, MODE 0): A / SA hold one row per TOKEN
+    // ([nk][a_rows][..], a_rows = T) and sorted row `pos` of the GEMM is token row_slots[pos] / topk.
+    const int32_t* row_slots;
+    int a_rows;
+    uint32_t topk_magic;     // ceil(2^32 / topk), or 0 for topk == 1: slot / topk = umulhi(slot, magic) for slot < 2^24
     int K;                   // contraction length in elements
     int N;                   // MODE 0: I (h columns; weight rows i and I+i); MODE 1: output columns
     int n_tiles_n;
@@ -1059,23 +1141,39 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
 // (four 33 KiB stages), and the gate+up epilogue re-quantizes h to MXFP8.
 // EXT: biases / clamped SwiGLU / interleaved source rows in the epilogue (instantiated with A8
 // only; for MXFP4 activations the 8-wave kernel is the faster one there).
+// GATHER (gate+up, plain epilogue): the item's rows are fetched by token from x quantized once per
+// token, and their scales once per 16 K-steps; see the kernel body. 16 loads per position then.
 template <bool A8>
 struct S4Cfg {
     static constexpr int kBM = A8 ? 128 : kStBM;       // rows per work item
     static constexpr int kRow = A8 ? 256 : 128;        // activation bytes per row and K-step
     static constexpr int kATile = kBM * kRow;
-    static constexpr int kStage = kATile + kBM * 8;    // + row scales
-    static constexpr int kLds = 4 * kStage;            // 102 KiB / 132 KiB
+    static constexpr int kStage = kATile + kBM * 8;    // + row scales (MODE 1; MODE 0 leaves that part unused)
+    static constexpr int kScaleTile = kBM * 128;       // MODE 0: row scales of 16 K-steps, two buffers behind the stages
+    static constexpr int kLds = 4 * kStage;            // MODE 1: 102 KiB / 132 KiB
+    static constexpr int kLdsGather = 4 * kATile + 2 * kScaleTile;   // MODE 0: 144 KiB / 160 KiB
     static constexpr int kPieces = kATile / 4096;      // 1 KiB activation loads per wave and position
-    static constexpr int kLoads = kPieces + 1 + 10;    // + row scales, 8 weight fragments, 2 weight scale dwords
 };
+static_assert(S4Cfg<true>::kLdsGather <= 160 * 1024 && S4Cfg<false>::kLdsGather <= 160 * 1024, "LDS of a CU");
 constexpr int kS4Ahead = 3;  // positions between fetch and compute (two measure the same)
 
-template <int MODE, bool EXT, bool A8>
+template <int MODE, bool EXT, bool A8, bool GATHER = false>
 __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmParams p) {
+    static_assert(!GATHER || (MODE == 0 && !EXT), "rows are gathered by the gate+up kernel with the plain epilogue only");
     using Cfg = S4Cfg<A8>;
-    constexpr int kBM = Cfg::kBM, kRow = Cfg::kRow, kATile = Cfg::kATile, kStage = Cfg::kStage;
-    constexpr int kPieces = Cfg::kPieces, kLoads = Cfg::kLoads;
+    // GATHER (gate+up kernel, plain epilogue): the activation rows are fetched by token; the quantized x
+    // is then stored once per token instead of once per routed slot (see tok_cur below), and its row
+    // scales are stored 16 K-steps ("super-step") to a 128-byte row and fetched once per super-step
+    // instead of once per position. (With the extended epilogue's registers on top, the slot
+    // registers no longer fit.) Measured at the GPT-OSS-like shape, layer time with / without: 64 to
+    // 4096 tokens 5-7 us less (the quantization rides in the sort's launch and writes a quarter of
+    // the bytes), 16384 tokens 30 us more, 65536 tokens 70 us more: every XCD then reads all of x
+    // instead of its experts' rows, and x no longer stays in its L2. The host picks by the size of x.
+    constexpr int kBM = Cfg::kBM, kRow = Cfg::kRow, kATile = Cfg::kATile;
+    constexpr int kStage = GATHER ? Cfg::kATile : Cfg::kStage, kScaleTile = Cfg::kScaleTile;
+    constexpr int kPieces = Cfg::kPieces;
+    constexpr int kScaleLoads = GATHER ? 0 : 1;
+    constexpr int kLoads = kPieces + kScaleLoads + 10;   // + 8 weight fragments, 2 weight scale dwords
     constexpr int MT = kBM / 16;
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
     const int lane = lane_id(), w = wave_id();
@@ -1089,8 +1187,10 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
 
     const int Kb = p.K >> 1;
     const int nk = (Kb + 127) >> 7;
-    const v4i srd_a = make_srd(p.A, (uint32_t)nk * (uint32_t)p.S * (uint32_t)kRow);
-    const v4i srd_sa = make_srd(p.SA, (uint32_t)nk * (uint32_t)p.S * 8u);
+    const int a_rows = GATHER ? p.a_rows : p.S;   // rows of the activation matrices
+    const v4i srd_a = make_srd(p.A, (uint32_t)nk * (uint32_t)a_rows * (uint32_t)kRow);
+    const v4i srd_sa = make_srd(p.SA, GATHER ? (uint32_t)((nk + 15) >> 4) * (uint32_t)a_rows * 128u
+                                             : (uint32_t)nk * (uint32_t)a_rows * 8u);
 
     // ---- cursors over the stream of (item, K-step) positions of this workgroup ---------------
     struct Cursor { int it, kt, expert, row_start, rows, n_tile; bool valid; };
@@ -1115,17 +1215,93 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
                              cf.valid ? (uint32_t)nk * kMoeScaleB : 0u);
     };
     cf_descriptors();
+    // GATHER: byte offset of the lane's row inside a K-step plane of A for each activation piece i
+    // (the row is 8 (4 i + w) + lane / 8), plus the lane's 16-byte chunk: for the fetch item
+    // (tok_cur) and, as raw slot numbers still in flight, for the item after it (tok_nxt). The slots
+    // of an item are requested one item ahead: by the time the fetch cursor reaches it, at least four
+    // positions of counted loads have been waited for behind them. They are extra loads in the
+    // counted stream; the waits only become stricter by them. Rows past the item (the rest of its
+    // last fragment, or past the end of the list, which reads as slot 0) map to some valid token;
+    // their results are dropped.
+    // piece i of the activation (half-)tile = rows 8 (4 i + w) .. +8; the swizzle of a row depends
+    // on its bits 1..3, i.e. on w and the lane only
+    const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);
+    constexpr int kNp = A8 ? 4 : kPieces;
+    constexpr int kTok = GATHER ? kNp : 1;
+    uint32_t tok_cur[kTok], tok_nxt[kTok];
+    const v4i srd_slots = make_srd(p.row_slots, GATHER ? (uint32_t)p.S * 4u : 0u);
+    auto request_tokens = [&](int row_start) __attribute__((always_inline)) {
+#pragma unroll
+        for (int q = 0; q < kTok; ++q) {
+            const uint32_t voff = (uint32_t)(row_start + 8 * (4 * q + w) + (lane >> 3)) * 4u;
+            uint32_t& dst = tok_nxt[q];
+            const v4i rs = srd_slots;
+            asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=v"(dst) : "v"(voff), "s"(rs) : "memory");
+        }
+    };
+    auto adopt_tokens = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int q = 0; q < kTok; ++q) {
+            const uint32_t slot = tok_nxt[q];
+            const uint32_t tok = p.topk_magic ? __umulhi(slot, p.topk_magic) : slot;
+            tok_cur[q] = tok * (uint32_t)kRow + chunk16 * 16u;
+        }
+    };
+    // requests the slots of the item after the fetch item
+    auto request_next_item = [&]() __attribute__((always_inline)) {
+        const int it = min(cf.it + it_stride, it_end - 1);
+        const v4i item = scalar_load_x4(p.items + it);
+        request_tokens(item.y);
+    };
+    // GATHER: row scales. SA is [ceil(nk / 16)][a_rows][128]: a row's 8 scale bytes of K-step kt sit at
+    // byte 8 (kt % 16) of its 128-byte row of super-step kt / 16. When the fetch cursor enters a
+    // super-step, the wave fetches the scale rows of the rows it fetches activation pieces for into one
+    // of two LDS buffers (the compute cursor is at most three positions behind, in this super-step or
+    // the one before). A row's eight 16-byte chunks are stored rotated by bits 1..3 of the row number
+    // (chunk c at position c ^ key), which spreads the 16 rows a fragment read touches over all banks.
+    // Chunks past the super-step's last K-step are not fetched (their lanes write zeros).
+    const uint32_t lds_ss = (uint32_t)(uintptr_t)smem + 4u * kStage;
+    const uint32_t ss_key = (uint32_t)(4 * w + (lane >> 4)) & 7u;       // key of the rows this lane fetches
+    const uint32_t ss_chunk = ((uint32_t)lane & 7u) ^ ss_key;           // the chunk it fetches
+    uint32_t cf_ss = kScaleTile, cc_ss = kScaleTile;   // byte offset of the cursor's buffer (toggled on entering a super-step)
+    auto fetch_scale_rows = [&]() __attribute__((always_inline)) {
+        cf_ss ^= (uint32_t)kScaleTile;
+        const int rows_up = cf.valid ? (cf.rows + 15) & ~15 : 0;
+        const int chunks = (min(16, nk - cf.kt) + 1) >> 1;
+        const uint32_t kill = (int)ss_chunk >= chunks ? 0x80000000u : 0u;
+#pragma unroll
+        for (int i = 0; i < kNp; ++i) {
+            v4i ssa = srd_sa;
+            if (8 * (4 * i + w) >= rows_up) ssa.z = 0;
+            uint32_t base = tok_cur[i] - chunk16 * 16u;   // token * kRow
+            if (A8) base >>= 1;
+            dma16(ssa, to_sgpr(lds_ss + cf_ss + (uint32_t)(w * 1024 + i * 4096)), (base + ss_chunk * 16u) | kill,
+                  (uint32_t)(cf.kt >> 4) * (uint32_t)a_rows * 128u);
+        }
+    };
+    if constexpr (GATHER) {
+        request_tokens(cf.row_start);
+        wait_vmcnt<0>();
+        adopt_tokens();
+        request_next_item();
+        fetch_scale_rows();
+    }
+    // The 2 kNp loads a change of the fetch item adds (slots, scale rows) sit between the counted loads
+    // of two positions: the waits of the next three positions allow for them.
+    int cf_extra = 0;
     auto advance_cf = [&]() __attribute__((always_inline)) {
-        if (++cf.kt == nk4) { cf.kt = 0; cf.it += it_stride; load_item(cf); cf_descriptors(); }
+        if (++cf.kt == nk4) {
+            cf.kt = 0; cf.it += it_stride; load_item(cf); cf_descriptors();
+            if constexpr (GATHER) { adopt_tokens(); request_next_item(); cf_extra = 3; }
+        }
+        if constexpr (GATHER)
+            if ((cf.kt & 15) == 0) fetch_scale_rows();
     };
 
     // ---- loads of one position ------------------------------------------------------------------
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
     const uint32_t lds_sa_wave = to_sgpr(lds0 + kATile + (uint32_t)w * (2u * kBM));
-    // piece i of the activation (half-)tile = rows 8 (4 i + w) .. +8; the swizzle of a row depends
-    // on its bits 1..3, i.e. on w and the lane only
-    const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);
     const uint32_t voff_a0 = (uint32_t)(8 * w + (lane >> 3)) * (uint32_t)kRow + chunk16 * 16u;  // + 32 i rows (+ 128 for the second K half)
     const uint32_t voff_sa = (uint32_t)(w * 2 * kBM + lane * 16);   // the row scales of rows [kBM / 4 * w, + kBM / 4)
     const uint32_t voff_b = lane * 16, voff_sb = lane * 4;
@@ -1143,16 +1319,21 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
             const int rows_up = cf.valid && cf.kt < nk ? (cf.rows + 15) & ~15 : 0;
             v4i sa = srd_a;
             if (8 * (4 * i + w) >= rows_up) sa.z = 0;  // past the item's last fragment: nothing is fetched
-            const uint32_t row_base = (uint32_t)cf.kt * (uint32_t)p.S + (uint32_t)cf.row_start;
-            dma16(sa, lds_wave + (uint32_t)(P * kStage + khalf * (kBM * 128) + i * 4096),
-                  voff_a0 + (uint32_t)(i * 32 * kRow + khalf * 128), row_base * (uint32_t)kRow);
-        } else if constexpr (L == kPieces) {
+            const uint32_t dst = lds_wave + (uint32_t)(P * kStage + khalf * (kBM * 128) + i * 4096);
+            if constexpr (GATHER) {
+                dma16(sa, dst, tok_cur[i],
+                      (uint32_t)cf.kt * (uint32_t)a_rows * (uint32_t)kRow + (uint32_t)(khalf * 128));
+            } else {
+                const uint32_t row_base = (uint32_t)cf.kt * (uint32_t)p.S + (uint32_t)cf.row_start;
+                dma16(sa, dst, voff_a0 + (uint32_t)(i * 32 * kRow + khalf * 128), row_base * (uint32_t)kRow);
+            }
+        } else if constexpr (L < kPieces + kScaleLoads) {
             v4i ssa = srd_sa;
             if (!cf.valid || cf.kt >= nk) ssa.z = 0;
             const uint32_t row_base = (uint32_t)cf.kt * (uint32_t)p.S + (uint32_t)cf.row_start;
             dma16_lanes(ssa, lds_sa_wave + (uint32_t)(P * kStage), voff_sa, row_base * 8u, (1ull << (kBM / 8)) - 1ull);
-        } else if constexpr (L < kPieces + 9) {
-            constexpr int f = L - kPieces - 1, pair = f >> 2, half = f & 1;
+        } else if constexpr (L < kPieces + kScaleLoads + 8) {
+            constexpr int f = L - kPieces - kScaleLoads, pair = f >> 2, half = f & 1;
             const int thr = cf.kt == nk - 1 ? 16 * min(max(last_valid - 64 * half, 0), 64) - 1 : 0x7fffffff;
             const uint32_t voff = voff_b | ((uint32_t)(thr - (int)voff_b) & 0x80000000u);
             const uint32_t soff = (uint32_t)cf.kt * kMoeBTile + (uint32_t)(2 * w + pair) * 4096u;
@@ -1163,7 +1344,7 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
                          : "v"(voff), "s"(rs), "s"(soff), "n"(((f >> 1) & 1) * 2048 + half * 1024)
                          : "memory");
         } else if constexpr (L < kLoads) {
-            constexpr int pair = L - kPieces - 9;
+            constexpr int pair = L - kPieces - kScaleLoads - 8;
             int& dst = bsc[P][pair];
             v4i rss = cf_srd_sb;
             if (cf.kt >= nk) rss.z = 0;
@@ -1382,7 +1563,12 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
     // to stage / set (P + 3) % 4, which the previous position has just finished with.
     auto step = [&]<int P>() __attribute__((always_inline)) {
         constexpr int PF = (P + kS4Ahead) % 4;
-        wait_vmcnt<(kS4Ahead - 1) * kLoads>();
+        if (GATHER && cf_extra > 0) {
+            --cf_extra;
+            wait_vmcnt<(kS4Ahead - 1) * kLoads + 2 * kNp>();
+        } else {
+            wait_vmcnt<(kS4Ahead - 1) * kLoads>();
+        }
         block_barrier();  // everyone's part of this position's tile has landed; stage PF is free
 #pragma unroll
         for (int f = 0; f < 8; ++f) asm volatile("" : "+v"(bw[P][f]));
@@ -1404,6 +1590,12 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
 #pragma unroll
             for (int j = 0; j < 2; ++j) a_rd[hh][j] = rd_half[hh][j] + (uint32_t)(P * kStage);
         uint32_t sa_rd = sa_rd0 + (uint32_t)(P * kStage);
+        if constexpr (GATHER) {
+            // the row's 8 bytes of this K-step in the scale buffer of the compute cursor's super-step
+            if ((cc.kt & 15) == 0) cc_ss ^= (uint32_t)kScaleTile;
+            sa_rd = lds_ss + cc_ss + r * 128u + (((((uint32_t)cc.kt & 15u) >> 1) ^ ((r >> 1) & 7u)) << 4) +
+                    ((uint32_t)cc.kt & 1u) * 8u;
+        }
         // bases in registers, offsets as immediates
         asm volatile("" : "+v"(a_rd[0][0]), "+v"(a_rd[1][0]), "+v"(sa_rd));
         if (A8) asm volatile("" : "+v"(a_rd[0][1]), "+v"(a_rd[1][1]));
@@ -1418,7 +1610,7 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
                 af[m % 3][0] = *(lds_v4i_t*)(uintptr_t)(a_rd[0][0] + m * 2048);
                 af[m % 3][1] = *(lds_v4i_t*)(uintptr_t)(a_rd[1][0] + m * 2048);
             }
-            as[m % 3] = *(lds_v2i_t*)(uintptr_t)(sa_rd + m * 128);
+            as[m % 3] = *(lds_v2i_t*)(uintptr_t)(sa_rd + m * (GATHER ? 2048 : 128));
         };
         if (mt > 0) { rd(0); rd(1); }
         auto frag = [&]<int M>() __attribute__((always_inline)) {
@@ -1521,17 +1713,17 @@ void moe_launch_build_items(const int32_t* expert_offsets, int E, int bm, int n_
     hipLaunchKernelGGL(moe_build_items_kernel, dim3(2, 8), dim3(512), 0, s, expert_offsets, E, b, num_items);
 }
 
-template <int MODE, bool EXT, bool A8>
+template <int MODE, bool EXT, bool A8, bool GATHER = false>
 static int launch_moe_stream(MoeGemmParams p, int max_items, hipStream_t s) {
     // Plain epilogues (SiLU-mul / bf16 store): the 4-wave kernel. With biases, the clamped SwiGLU or
     // interleaved source rows the per-element work of the epilogue is larger and two waves per SIMD
     // hide it better: the 8-wave kernel (measured: 0.51 against 0.57 ms for the layer). MXFP8
     // activations: the 4-wave kernel in both cases.
     constexpr bool k8wave = EXT && !A8;
-    constexpr int lds = k8wave ? kStLds : S4Cfg<A8>::kLds, threads = k8wave ? 512 : 256;
+    constexpr int lds = k8wave ? kStLds : GATHER ? S4Cfg<A8>::kLdsGather : S4Cfg<A8>::kLds, threads = k8wave ? 512 : 256;
     const void* kern;
     if constexpr (k8wave) kern = (const void*)moe_mxfp4_stream_kernel<MODE, true>;
-    else kern = (const void*)moe_mxfp4_stream4_kernel<MODE, EXT && A8, A8>;
+    else kern = (const void*)moe_mxfp4_stream4_kernel<MODE, EXT && A8, A8, GATHER>;
     static DeviceOnce configured;
     if (!set_lds_limit_once(kern, lds, configured)) return HK_ERR_LAUNCH;
     // persistent: one workgroup per CU, each walking its share of the item list
@@ -1642,7 +1834,7 @@ static MoeWs moe_ws_layout(int T, int H, int I, int E, int k, bool a8 = false) {
     L.nitems = take(8);
     const size_t nk1 = (H / 2 + 127) / 128, nk2 = (I / 2 + 127) / 128;  // K-step-major activation tiles
     const size_t row = a8 ? 256 : 128;  // activation bytes per row and K-step
-    L.xq = take(nk1 * S * row); L.xs = take(nk1 * S * 8);
+    L.xq = take(nk1 * S * row); L.xs = take(std::max(nk1 * S * 8, (nk1 + 15) / 16 * (size_t)T * 128));
     L.hq = take(nk2 * S * row); L.hs = take(nk2 * S * 8);
     L.o = take(S * (size_t)H * 2);
     L.total = off;
@@ -1671,6 +1863,31 @@ static int moe_mxfp4_check(int T, int H, int I, int E, int k, int w13_scale_pitc
     return HK_OK;
 }
 
+static MoeBuildItems moe_items_args(uint8_t* ws, const MoeWs& L, int I, int H, bool a8, int weight_layout) {
+    MoeBuildItems b;
+    b.bm = a8 ? S4Cfg<true>::kBM : weight_layout ? kStBM : kMoeBM;
+    b.items[0] = (MoeItem*)(ws + L.items1); b.items[1] = (MoeItem*)(ws + L.items2);
+    b.n_tiles[0] = (I + 127) / 128; b.n_tiles[1] = (H + 255) / 256;
+    return b;
+}
+static MxQuantizeArgs moe_quantize_args(const void* x_bf16, const int32_t* sorted_slots, const int32_t* slot_to_pos,
+                                        int k, int T, int H, int I, uint8_t* ws, const MoeWs& L) {
+    MxQuantizeArgs a;
+    a.x = (const uint16_t*)x_bf16; a.sorted_slots = sorted_slots; a.slot_to_pos = slot_to_pos;
+    a.topk = k; a.T = T; a.cols = H;
+    a.tiled = ws + L.xq; a.tiled_scales = ws + L.xs; a.tiled2 = ws + L.hq; a.tiled2_scales = ws + L.hs;
+    a.K2 = I;
+    return a;
+}
+// Whether the layer's gate+up kernel gathers its activation rows by token (the 4-wave streaming
+// kernel with the plain epilogue): x is then quantized once per token; the other kernels take it
+// permuted into sorted order, one row per slot.
+// It pays while the quantized x stays in an XCD's L2 next to the weight stream (measured: up to
+// 4096 tokens of 2880 MXFP4 columns, 1024 of MXFP8).
+static bool moe_gathers(int weight_layout, bool ext, bool a8, int T, int H) {
+    return weight_layout == 1 && !ext && (long long)T * H * (a8 ? 2 : 1) <= 12ll << 20;
+}
+
 // Expert MLP on already routed and sorted tokens (steps 3-6 of the forward pass). a8: MXFP8
 // activations (pre-shuffled weights only).
 static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const void* w13_scales,
@@ -1680,7 +1897,7 @@ static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const voi
                                   int T, int H, int I, int E, int k, int weight_layout,
                                   const float* bias13, const float* bias2, int activation, float alpha,
                                   float limit, int w13_interleaved, void* workspace,
-                                  size_t workspace_bytes, void* stream, bool a8) {
+                                  size_t workspace_bytes, void* stream, bool a8, bool x_quantized = false) {
     if (activation != 0 && activation != 1) return HK_ERR_UNSUPPORTED;
     if (a8 && weight_layout != 1) return HK_ERR_UNSUPPORTED;
     if (activation == 1 && !(limit > 0.f)) return HK_ERR_BAD_SHAPE;
@@ -1707,20 +1924,21 @@ static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const voi
     const int S = T * k;
 
     int32_t* nitems = (int32_t*)(ws + L.nitems);
-    {
+    const bool gather = moe_gathers(weight_layout, ext, a8, T, H);
+    if (!x_quantized) {   // (the forward pass of a small layer has done this in its sort launch)
         const int nk1 = (H / 2 + 127) / 128;
-        MoeBuildItems b;
-        b.bm = a8 ? S4Cfg<true>::kBM : weight_layout ? kStBM : kMoeBM;
-        b.items[0] = (MoeItem*)(ws + L.items1); b.items[1] = (MoeItem*)(ws + L.items2);
-        b.n_tiles[0] = (I + 127) / 128; b.n_tiles[1] = (H + 255) / 256;
-        auto qp = a8 ? mx_quantize_permute_kernel<true> : mx_quantize_permute_kernel<false>;
-        hipLaunchKernelGGL(qp, dim3((T + kQpRows - 1) / kQpRows + 2, (nk1 + 3) / 4), dim3(128), 0, s,
-                           (const uint16_t*)x_bf16, sorted_slots, slot_to_pos, k, T, H, ws + L.xq, ws + L.xs,
-                           ws + L.hq, ws + L.hs, I, expert_offsets, E, b, nitems);
+        const MoeBuildItems b = moe_items_args(ws, L, I, H, a8, weight_layout);
+        const MxQuantizeArgs qa = moe_quantize_args(x_bf16, sorted_slots, slot_to_pos, k, T, H, I, ws, L);
+        auto qp = a8 ? (gather ? mx_quantize_permute_kernel<true, false> : mx_quantize_permute_kernel<true, true>)
+                     : (gather ? mx_quantize_permute_kernel<false, false> : mx_quantize_permute_kernel<false, true>);
+        hipLaunchKernelGGL(qp, dim3((T + kQpRows - 1) / kQpRows + 2, (nk1 + 3) / 4), dim3(128), 0, s, qa,
+                           expert_offsets, E, b, nitems);
     }
 
     MoeGemmParams p{};
     p.A = ws + L.xq; p.SA = ws + L.xs; p.S = S;
+    p.row_slots = gather ? sorted_slots : nullptr; p.a_rows = gather ? T : S;
+    p.topk_magic = k == 1 ? 0u : (uint32_t)(((1ull << 32) + (uint64_t)k - 1) / (uint64_t)k);
     p.B = (const uint8_t*)w13; p.SB = (const uint8_t*)w13_scales;
     p.b_pitch = H / 2; p.sb_pitch = w13_scale_pitch;
     p.b_expert_stride = (long long)2 * I * (H / 2); p.sb_expert_stride = (long long)2 * I * w13_scale_pitch;
@@ -1733,11 +1951,14 @@ static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const voi
     p.K = H; p.N = I; p.n_tiles_n = (I + 127) / 128;
     p.bias = bias13; p.act = activation; p.alpha = alpha; p.limit = limit; p.interleaved = w13_interleaved != 0;
     if (a8)
-        st = ext ? launch_moe_stream<0, true, true>(p, L.max_items1, s) : launch_moe_stream<0, false, true>(p, L.max_items1, s);
+        st = ext ? launch_moe_stream<0, true, true>(p, L.max_items1, s)
+                 : gather ? launch_moe_stream<0, false, true, true>(p, L.max_items1, s)
+                          : launch_moe_stream<0, false, true>(p, L.max_items1, s);
     else if (ext)
         st = weight_layout ? launch_moe_stream<0, true, false>(p, L.max_items1, s) : launch_moe_gemm<0, true>(p, L.max_items1, s);
     else
-        st = weight_layout ? launch_moe_stream<0, false, false>(p, L.max_items1, s) : launch_moe_gemm<0, false>(p, L.max_items1, s);
+        st = gather ? launch_moe_stream<0, false, false, true>(p, L.max_items1, s)
+             : weight_layout ? launch_moe_stream<0, false, false>(p, L.max_items1, s) : launch_moe_gemm<0, false>(p, L.max_items1, s);
     if (st != HK_OK) return st;
 
     MoeGemmParams q{};
@@ -1819,14 +2040,32 @@ static int moe_mxfp4_forward_impl(const void* x_bf16, const float* router_logits
     uint8_t* ws = (uint8_t*)workspace;
     st = hk_moe_topk_softmax(router_logits, T, E, k, (int32_t*)(ws + L.ids), (float*)(ws + L.w), stream);
     if (st != HK_OK) return st;
-    st = hk_moe_sort((const int32_t*)(ws + L.ids), T, k, E, (int32_t*)(ws + L.sorted), (int32_t*)(ws + L.offsets),
-                     (int32_t*)(ws + L.inv), ws + L.sort_ws, hk_moe_sort_workspace_bytes(T, k, E), stream);
-    if (st != HK_OK) return st;
+    const bool ext = bias13 || bias2 || activation != 0 || w13_interleaved;
+    bool fused = false;
+    if (moe_gathers(weight_layout, ext, a8, T, H) && (long long)T * k <= kSortSmallMax && x_bf16 &&
+        (((uintptr_t)x_bf16 | (uintptr_t)workspace) & 15u) == 0) {
+        // sort, item lists and the quantization of x in one launch (moe_sort_quantize_kernel)
+        const int S = T * k, nchunks = (S + kSortChunk - 1) / kSortChunk;
+        const int nk1 = (H / 2 + 127) / 128;
+        const MoeBuildItems b = moe_items_args(ws, L, I, H, a8, weight_layout);
+        const MxQuantizeArgs qa = moe_quantize_args(x_bf16, nullptr, nullptr, k, T, H, I, ws, L);
+        const int grid = nchunks + 2 * kFusedItemParts + (T + kQpRows - 1) / kQpRows * ((nk1 + 7) / 8);
+        auto kern = a8 ? moe_sort_quantize_kernel<true> : moe_sort_quantize_kernel<false>;
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const int32_t*)(ws + L.ids), E,
+                           (int32_t*)(ws + L.offsets), (int32_t*)(ws + L.sorted), (int32_t*)(ws + L.inv), qa, b,
+                           (int32_t*)(ws + L.nitems));
+        if (hipGetLastError() != hipSuccess) return HK_ERR_LAUNCH;
+        fused = true;
+    } else {
+        st = hk_moe_sort((const int32_t*)(ws + L.ids), T, k, E, (int32_t*)(ws + L.sorted), (int32_t*)(ws + L.offsets),
+                         (int32_t*)(ws + L.inv), ws + L.sort_ws, hk_moe_sort_workspace_bytes(T, k, E), stream);
+        if (st != HK_OK) return st;
+    }
     return moe_mxfp4_experts_impl(x_bf16, w13, w13_scales, w13_scale_pitch, w2, w2_scales, w2_scale_pitch,
                                   (const float*)(ws + L.w), (const int32_t*)(ws + L.sorted),
                                   (const int32_t*)(ws + L.offsets), (const int32_t*)(ws + L.inv), y_bf16, T, H, I,
                                   E, k, weight_layout, bias13, bias2, activation, alpha, limit, w13_interleaved,
-                                  workspace, workspace_bytes, stream, a8);
+                                  workspace, workspace_bytes, stream, a8, fused);
 }
 
 extern "C" int hk_moe_mxfp4_forward_ex(const void* x_bf16, const float* router_logits, const void* w13,

@@ -297,3 +297,92 @@ def test_moe_mxfp4_forward_drawn_shapes(hk, T, E, k, H, I):
     want = F.bf16_to_f32(O.moe_mxfp4_forward(x, ids, w, w13p, w13s, w2p, w2s)[0])
     assert np.isfinite(got).all()
     assert G.rel_fro_error(got, want) <= TOL
+
+
+def _device_layer(hk, T, E, k, H, I, seed):
+    """Seeded layer on the device: x, logits, plain weights (scale rows padded to a multiple of 8)."""
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    x = torch.randn(T, H, device=DEV, generator=g).to(torch.bfloat16)
+    logits = torch.randn(T, E, device=DEV, generator=g)
+    pitch = (max(H, I) // 32 + 7) // 8 * 8
+    w13p = torch.empty((E, 2 * I, H // 2), dtype=torch.uint8, device=DEV)
+    w13s = torch.full((E, 2 * I, (H // 32 + 7) // 8 * 8), 127, dtype=torch.uint8, device=DEV)
+    w2p = torch.empty((E, H, I // 2), dtype=torch.uint8, device=DEV)
+    w2s = torch.full((E, H, (I // 32 + 7) // 8 * 8), 127, dtype=torch.uint8, device=DEV)
+    for e in range(E):
+        a, s = hk.quant.quantize_mxfp4(torch.randn(2 * I, H, device=DEV, generator=g) * 0.1)
+        w13p[e], w13s[e] = a, hk.quant.pad_scales(s)
+        a, s = hk.quant.quantize_mxfp4(torch.randn(H, I, device=DEV, generator=g) * 0.1)
+        w2p[e], w2s[e] = a, hk.quant.pad_scales(s)
+    del pitch
+    return x, logits, w13p, w13s, w2p, w2s
+
+
+def _oracle_on_sample(x, logits, w13p, w13s, w2p, w2s, k, y, count, act_format="mxfp4"):
+    """Oracle on `count` evenly spaced tokens, evaluating only the experts they use."""
+    T, H = x.shape
+    I = w2p.shape[2] * 2
+    sel = torch.arange(0, T, max(1, T // count), device=DEV)[:count]
+    ids, w = O.topk_softmax(logits[sel].cpu().numpy(), k)
+    used = np.unique(ids)
+    remap = {int(e): i for i, e in enumerate(used)}
+    ids_l = np.vectorize(remap.get)(ids).astype(np.int32)
+    ut = torch.from_numpy(used.astype(np.int64)).to(DEV)
+    want = F.bf16_to_f32(O.moe_mxfp4_forward(
+        x[sel].float().cpu().numpy(), ids_l, w, w13p[ut].cpu().numpy(), w13s[ut][:, :, :H // 32].cpu().numpy(),
+        w2p[ut].cpu().numpy(), w2s[ut][:, :, :I // 32].cpu().numpy(), act_format=act_format)[0])
+    return G.rel_fro_error(y[sel].float().cpu().numpy(), want)
+
+
+# The gate+up kernel fetches its activation rows either by token from x quantized once per token
+# (small x; up to 16384 slots the quantization rides in the sort's launch) or from x permuted into
+# sorted order; the cases below reach every combination through both entry points.
+PATH_CASES = [
+    # T, E, k, H, I, act_format
+    (300, 8, 2, 512, 384, "mxfp4"),      # gathered rows, one fused sort + quantize launch
+    (300, 8, 2, 512, 384, "mxfp8"),
+    (8192, 16, 4, 1024, 128, "mxfp4"),   # gathered rows, 32768 slots: three-launch sort, separate quantizer
+    (8192, 8, 2, 1664, 256, "mxfp4"),    # x too large to gather: permuted rows
+    (4096, 8, 2, 1664, 256, "mxfp8"),    # the same with MXFP8 activations
+    (2048, 8, 2, 4352, 128, "mxfp4"),    # gathered rows, K of 17 K-steps: two scale super-steps per item
+]
+
+
+@pytest.mark.parametrize("T,E,k,H,I,act_format", PATH_CASES)
+def test_moe_mxfp4_activation_paths_and_experts_entry(hk, T, E, k, H, I, act_format):
+    print(f"moe_mxfp4 paths T={T} E={E} k={k} H={H} I={I} {act_format}", flush=True)
+    x, logits, w13p, w13s, w2p, w2s = _device_layer(hk, T, E, k, H, I, seed=T + H)
+    shuf = hk.tk_kernel.MoeMxfp4ShuffledWeights.from_plain(w13p, w13s, w2p, w2s)
+    ws = torch.empty(hk.tk_kernel.moe_mxfp4_workspace_bytes(T, H, I, E, k, act_format=act_format), dtype=torch.uint8,
+                     device=DEV)
+    y = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_mxfp4(x, logits, shuf, None, None, None, y, k, ws, act_format=act_format)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all()
+    assert _oracle_on_sample(x, logits, w13p, w13s, w2p, w2s, k, y, 32, act_format) <= TOL
+    # the extended epilogue with zero biases: the kernel that takes permuted rows; identical arithmetic
+    yb = torch.full_like(y, float("nan"))
+    hk.tk_kernel.dispatch_moe_mxfp4(x, logits, shuf, None, None, None, yb, k, ws, act_format=act_format,
+                                    bias13=torch.zeros((E, 2 * I), device=DEV), bias2=torch.zeros((E, H), device=DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(yb, y)
+    if act_format == "mxfp4":  # plain weight layout (MXFP4 activations only): permuted rows as well
+        yp = torch.full_like(y, float("nan"))
+        hk.tk_kernel.dispatch_moe_mxfp4(x, logits, w13p, w13s, w2p, w2s, yp, k, ws)
+        torch.cuda.synchronize()
+        assert torch.equal(yp, y)
+    # the experts entry point on the caller's routing
+    ids = torch.empty((T, k), dtype=torch.int32, device=DEV)
+    wts = torch.empty((T, k), dtype=torch.float32, device=DEV)
+    hk.tk_kernel.dispatch_moe_topk_softmax(logits, ids, wts)
+    sorted_slots = torch.empty(T * k, dtype=torch.int32, device=DEV)
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=DEV)
+    inv = torch.empty(T * k, dtype=torch.int32, device=DEV)
+    sws = torch.empty(hk.tk_kernel.moe_sort_workspace_bytes(T, k, E), dtype=torch.uint8, device=DEV)
+    hk.tk_kernel.dispatch_moe_sort(ids, sorted_slots, offsets, inv, sws)
+    ye = torch.full_like(y, float("nan"))
+    ws.fill_(0x5A)
+    hk.tk_kernel.dispatch_moe_mxfp4_experts(x, shuf, None, None, None, wts, sorted_slots, offsets, inv, ye, ws,
+                                            act_format=act_format)
+    torch.cuda.synchronize()
+    assert torch.equal(ye, y)
