@@ -62,7 +62,7 @@ __device__ __forceinline__ float exp_neg_f32(float x) {
 __device__ __forceinline__ float sigmoid_f32(float x) {
     const float e = exp_neg_f32(-fabsf(x));
     const float d = __fadd_rn(1.0f, e);
-    return x >= 0.f ? __fdiv_rn(1.0f, d) : __fdiv_rn(e, d);
+    return __fdiv_rn(x >= 0.f ? 1.0f : e, d);   // 1 / d or e / d: one division
 }
 
 constexpr int kMaxPerLane = 8;  // experts per lane: E <= 512
@@ -80,32 +80,42 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const float* __re
     const int t = (blockIdx.x * 4 + (threadIdx.x >> 6)) * TPW + lane / LPT;
     const bool live = t < T;
     const float* row = logits + (size_t)(live ? t : 0) * E;
-    uint64_t cand[kMaxPerLane];
+    // Selection in 32-bit operations: per round the largest key over the token's lanes, then the
+    // lowest id among its holders (the order of pack_choice). Key 0 = taken or absent (the key of a
+    // number is never 0).
+    uint32_t ck[kMaxPerLane];
     const int per = (E + LPT - 1) / LPT;
 #pragma unroll
     for (int i = 0; i < kMaxPerLane; ++i) {
         const int e = i * LPT + sub;  // coalesced within the token's row
-        cand[i] = (live && i < per && e < E) ? pack_choice(row[e], e) : 0ull;
+        ck[i] = (live && i < per && e < E) ? float_key(row[e]) : 0u;
     }
     float my_logit = 0.f, top_logit = 0.f;
     int my_id = 0;
     for (int j = 0; j < k; ++j) {
-        uint64_t best = 0;
+        uint32_t bk = 0;
 #pragma unroll
-        for (int i = 0; i < kMaxPerLane; ++i) best = cand[i] > best ? cand[i] : best;
+        for (int i = 0; i < kMaxPerLane; ++i) bk = ck[i] > bk ? ck[i] : bk;
 #pragma unroll
         for (int off = LPT / 2; off >= 1; off >>= 1) {
-            const uint64_t o = __shfl_xor(best, off, 64);
-            best = o > best ? o : best;
+            const uint32_t o = __shfl_xor(bk, off, 64);
+            bk = o > bk ? o : bk;
         }
-        const int id = live ? choice_id(best) : 0;
+        int id = 0x7fffffff;
+#pragma unroll
+        for (int i = kMaxPerLane - 1; i >= 0; --i) id = ck[i] == bk ? i * LPT + sub : id;
+#pragma unroll
+        for (int off = LPT / 2; off >= 1; off >>= 1) {
+            const int o = __shfl_xor(id, off, 64);
+            id = o < id ? o : id;
+        }
+        if (!live) id = 0;
 #pragma unroll
         for (int i = 0; i < kMaxPerLane; ++i)
-            if (cand[i] == best) cand[i] = 0ull;  // ids are unique, only the owner matches
+            if (i * LPT + sub == id) ck[i] = 0u;
         // the logit back from its key (exact; -0 comes back as +0, which the softmax cannot tell apart):
         // no dependent reload of row[id]
-        const uint32_t key = (uint32_t)(best >> 32);
-        const float v = __uint_as_float((key & 0x80000000u) ? key ^ 0x80000000u : ~key);
+        const float v = __uint_as_float((bk & 0x80000000u) ? bk ^ 0x80000000u : ~bk);
         if (j == 0) top_logit = v;
         if (sub == j) { my_logit = v; my_id = id; }
     }
@@ -259,26 +269,36 @@ __global__ __launch_bounds__(256) void moe_topk_grouped_sigmoid16_kernel(
         }
         if (gc == b) { gc = 0ull; kept = true; }
     }
-    if (!kept) {
+    // The k best of the kept groups, in the order of the (key, id) pairs: per round the largest 32-bit
+    // key over the token's 16 lanes, then the lowest id among its holders (ids grow with i and with
+    // the lane), all in 32-bit operations. A key of 0 marks a choice that is taken or not kept (the
+    // key of a real score is never 0).
+    uint32_t ck[PER];
 #pragma unroll
-        for (int i = 0; i < PER; ++i) cand[i] = 0ull;
-    }
+    for (int i = 0; i < PER; ++i) ck[i] = kept ? (uint32_t)(cand[i] >> 32) : 0u;
     float my_s = 0.f;
     int my_id = 0;
     for (int j = 0; j < k; ++j) {
-        uint64_t best = 0;
+        uint32_t bk = 0;
 #pragma unroll
-        for (int i = 0; i < PER; ++i) best = cand[i] > best ? cand[i] : best;
+        for (int i = 0; i < PER; ++i) bk = ck[i] > bk ? ck[i] : bk;
 #pragma unroll
         for (int off = 8; off >= 1; off >>= 1) {
-            const uint64_t o = __shfl_xor(best, off, 64);
-            best = o > best ? o : best;
+            const uint32_t o = __shfl_xor(bk, off, 64);
+            bk = o > bk ? o : bk;
         }
-        const int id = choice_id(best);
+        int id = 0x7fffffff;
+#pragma unroll
+        for (int i = PER - 1; i >= 0; --i) id = ck[i] == bk ? sub * PER + i : id;
+#pragma unroll
+        for (int off = 8; off >= 1; off >>= 1) {
+            const int o = __shfl_xor(id, off, 64);
+            id = o < id ? o : id;
+        }
         float sv = 0.f;
 #pragma unroll
         for (int i = 0; i < PER; ++i)
-            if (cand[i] == best) { cand[i] = 0ull; sv = s[i]; }
+            if (sub * PER + i == id) { ck[i] = 0u; sv = s[i]; }
         sv = __shfl(sv, seg + id / PER, 64);
         if (sub == j) { my_s = sv; my_id = id; }
     }
