@@ -1658,16 +1658,30 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
 // y[t, :] = bf16( add[t, :] + sum_j w[t, j] * o[slot_to_pos[t*k + j], :] ), fp32 accumulation in
 // choice order starting from add (bf16 [T, H], e.g. a shared expert's output) or from 0 when add
 // is null.
+// KU > 0: k <= KU, the token's positions and weights are read once and the k rows' loads of a column
+// chunk are issued together; KU == 0: any k, one row at a time. Same operations in the same order.
+template <int KU>
 __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __restrict__ o,
                                                             const float* __restrict__ w,
                                                             const int32_t* __restrict__ slot_to_pos, int T,
                                                             int k, int H, const uint16_t* __restrict__ add,
                                                             uint16_t* __restrict__ y) {
     const int t = blockIdx.x;
+    int pos[KU > 0 ? KU : 1];
+    float wt[KU > 0 ? KU : 1];
+#pragma unroll
+    for (int j = 0; j < KU; ++j) {
+        pos[j] = j < k ? slot_to_pos[(size_t)t * k + j] : 0;
+        wt[j] = j < k ? w[(size_t)t * k + j] : 0.f;
+    }
     for (int c = threadIdx.x; c < H / 8; c += 256) {
         float acc[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+        v4i rows[KU > 0 ? KU : 1];
+#pragma unroll
+        for (int j = 0; j < KU; ++j)
+            if (j < k) rows[j] = *(const v4i*)(o + (size_t)pos[j] * H + c * 8);
         if (add) {
             const v4i raw = *(const v4i*)(add + (size_t)t * H + c * 8);
 #pragma unroll
@@ -1676,14 +1690,26 @@ __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __re
                 acc[2 * i + 1] = __uint_as_float((uint32_t)raw[i] & 0xffff0000u);
             }
         }
-        for (int j = 0; j < k; ++j) {
-            const int pos = slot_to_pos[(size_t)t * k + j];
-            const float wj = w[(size_t)t * k + j];
-            const v4i raw = *(const v4i*)(o + (size_t)pos * H + c * 8);
+        if constexpr (KU > 0) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                acc[2 * i] += wj * __uint_as_float((uint32_t)raw[i] << 16);
-                acc[2 * i + 1] += wj * __uint_as_float((uint32_t)raw[i] & 0xffff0000u);
+            for (int j = 0; j < KU; ++j)
+                if (j < k) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        acc[2 * i] += wt[j] * __uint_as_float((uint32_t)rows[j][i] << 16);
+                        acc[2 * i + 1] += wt[j] * __uint_as_float((uint32_t)rows[j][i] & 0xffff0000u);
+                    }
+                }
+        } else {
+            for (int j = 0; j < k; ++j) {
+                const int pj = slot_to_pos[(size_t)t * k + j];
+                const float wj = w[(size_t)t * k + j];
+                const v4i raw = *(const v4i*)(o + (size_t)pj * H + c * 8);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[2 * i] += wj * __uint_as_float((uint32_t)raw[i] << 16);
+                    acc[2 * i + 1] += wj * __uint_as_float((uint32_t)raw[i] & 0xffff0000u);
+                }
             }
         }
         v4i out;
@@ -1779,7 +1805,8 @@ extern "C" int hk_moe_unpermute_add(const void* o_bf16, const float* w, const in
     if (!o_bf16 || !w || !slot_to_pos || !y_bf16) return HK_ERR_NULL_POINTER;
     if (T <= 0 || k <= 0 || H <= 0 || (H % 8) != 0) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)o_bf16 | (uintptr_t)y_bf16 | (uintptr_t)add_bf16_or_null) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    hipLaunchKernelGGL(moe_unpermute_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)o_bf16,
+    auto kern = k <= 4 ? moe_unpermute_kernel<4> : k <= 8 ? moe_unpermute_kernel<8> : moe_unpermute_kernel<0>;
+    hipLaunchKernelGGL(kern, dim3(T), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)o_bf16,
                        w, slot_to_pos, T, k, H, (const uint16_t*)add_bf16_or_null, (uint16_t*)y_bf16);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
