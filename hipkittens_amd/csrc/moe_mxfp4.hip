@@ -10,7 +10,7 @@
 // Weights dominate HBM traffic, so workgroups are persistent (one per CU) and keep their operand
 // pipelines running across item boundaries. Items that share an expert run at the same time on
 // the CUs of one XCD, so activation tiles come out of that XCD's L2 and every weight byte leaves
-// HBM once. Two kernels: moe_mxfp4_stream_kernel for weights in the pre-shuffled layout (the fast
+// HBM once. Two kernels: moe_mxfp4_stream4_kernel for weights in the pre-shuffled layout (the fast
 // path: weights go straight from HBM into MFMA operand registers, 192-row m-tiles) and
 // moe_mxfp4_gemm_kernel for the plain layout (both operands through an LDS ring, 128-row m-tiles).
 #include "moe_common.h"
@@ -350,7 +350,8 @@ __global__ __launch_bounds__(256) void moe_sort_quantize_kernel(const int32_t* _
 
 // ---------------------------------------------------------------------- weight pre-shuffle
 // Tile row R (0..255) of n-tile `n_tile` in the pre-shuffled layout -> row of the expert's weight
-// matrix. Wave w of moe_mxfp4_stream_kernel owns tile rows [32 w, +32) = two MFMA fragments.
+// matrix. The layout is written in units of 32 tile rows (`w` below, two MFMA fragments); wave W of
+// moe_mxfp4_stream4_kernel owns units 2 W and 2 W + 1, i.e. tile rows [64 W, +64).
 // mode 0 (gate+up, N = I): fragment 0 holds the gate rows and fragment 1 the up rows of h columns
 // 128 n_tile + 16 w .. +16, in order; mode 1 (down, N = H): the b_row_to_col permutation, which
 // gives a lane 8 consecutive output columns from its two fragments. Rows past N repeat row N - 1.
@@ -362,10 +363,10 @@ __device__ __forceinline__ int moe_stream_b_row(int mode, int R, int n_tile, int
     return mode == 2 ? 2 * hcol + f : f * N + hcol;
 }
 
-// Pre-shuffled weight layout, made for moe_mxfp4_stream_kernel: weights go from HBM straight
+// Pre-shuffled weight layout, made for moe_mxfp4_stream4_kernel: weights go from HBM straight
 // into MFMA operand registers, so for every (expert, n-tile of 256 tile rows, K-step of 256
-// elements) one contiguous 32 KiB block holds, wave by wave (wave w = tile rows [32 w, +32)),
-// the wave's four B fragments f = 2 * nfrag + half as 1 KiB pieces in lane order: lane l's 16
+// elements) one contiguous 32 KiB block holds, unit by unit (unit w = tile rows [32 w, +32)),
+// the unit's four B fragments f = 2 * nfrag + half as 1 KiB pieces in lane order: lane l's 16
 // bytes are tile row 32 w + 16 nfrag + l % 16 (moe_stream_b_row gives the weight row), K bytes
 // 128 kt + 64 half + 16 (l / 16) .. +16, zero past the end of K. A second array holds the
 // scales the same way, 4 bytes per lane: byte 2 half + nfrag is the e8m0 scale of that row's
@@ -732,386 +733,19 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
 // Weight-streaming grouped GEMM for the pre-shuffled layout. At MoE shapes the grouped GEMMs are
 // bound by reading every expert's weights once from HBM, so the kernel is built around keeping
 // as many weight bytes in flight per CU as possible and around reading them once:
-//   * weights never touch LDS: the pre-shuffled layout stores, for every (expert, n-tile, K-step,
-//     wave), the wave's four MFMA B fragments as four contiguous 1 KiB pieces (lane l's 16 bytes
-//     at 16*l), and each wave loads them straight into registers 3.5 K-steps ahead of their use
-//     (a ring of eight half-K-step register sets); their e8m0 scales come the same way;
+//   * weights never touch LDS: the pre-shuffled layout stores, for every (expert, n-tile, K-step)
+//     the MFMA B fragments as contiguous 1 KiB pieces (lane l's 16 bytes at 16*l), and each wave
+//     loads its eight straight into registers three positions ahead of their use (a ring of four
+//     register sets); their e8m0 scales come the same way;
 //   * a work item covers up to 192 rows of an expert (12 activation fragments), so that an expert
 //     with a few rows more than 128 still needs one pass over its weights;
-//   * only the activation tile (shared by the waves, re-read from L2) goes through LDS, in a ring
-//     of five 25.5 KiB stages filled by direct global->LDS loads four K-steps ahead. Loads return
-//     in order, so the activation tile has to be requested before the weights of the same K-step.
-// One workgroup of 8 waves per CU; wave w owns weight rows [32 w, +32) of the 256-row tile (two
-// fragments) x all rows of the item: 96 accumulator registers. The K-step stream runs across item
-// boundaries. All vector-memory operations are inline asm and counted by hand (the compiler
-// never waits for them): every use of loaded registers is preceded by a vmcnt wait and
-// `landed`, which makes the compiler see a new value there. Results are bit-identical to
-// moe_mxfp4_gemm_kernel (same accumulation order per output element). Launched for the extended
-// epilogues (biases, clamped SwiGLU, interleaved source rows); the plain ones take the 4-wave
-// kernel below.
-constexpr int kStBM = 192;                              // rows per work item
-constexpr int kStStages = 5;
-constexpr int kStATile = kStBM * 128;                   // 24 KiB
-constexpr int kStStage = kStATile + kStBM * 8;          // + 1.5 KiB of row scales
-constexpr int kStXch = kStStages * kStStage;            // epilogue: row maxima [kStBM][8 waves] floats
-constexpr int kStHTile = kStXch + kStBM * 8 * 4;        // epilogue: packed h tile [kStBM][64 bytes]
-constexpr int kStHScale = kStHTile + kStBM * 64;        // epilogue: h scales [kStBM][4 bytes]
-constexpr int kStLds = kStHScale + kStBM * 4;           // 146.25 KiB
-
-template <int MODE, bool EXT>
-__global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmParams p) {
-    constexpr int MT = kStBM / 16, NT = 2;
-    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
-    const int lane = lane_id(), w = wave_id();
-    const int n_items = scalar_load_x1(p.num_items);
-    const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
-    const int it_stride = ((int)gridDim.x - xcd + kNumXcd - 1) / kNumXcd;  // workgroups on this XCD
-    const int per_xcd = (n_items + kNumXcd - 1) / kNumXcd;
-    const int it0 = xcd * per_xcd + slot;
-    const int it_end = min(n_items, (xcd + 1) * per_xcd);
-    if (it0 >= it_end) return;
-
-    const int Kb = p.K >> 1;
-    const int nk = (Kb + 127) >> 7;
-    const v4i srd_a = make_srd(p.A, (uint32_t)nk * (uint32_t)p.S * 128u);
-    const v4i srd_sa = make_srd(p.SA, (uint32_t)nk * (uint32_t)p.S * 8u);
-
-    // ---- cursors over the stream of (item, K-step) positions of this workgroup ---------------
-    struct Cursor { int it, kt, expert, row_start, rows, n_tile; bool valid; };
-    auto load_item = [&](Cursor& c) __attribute__((always_inline)) {
-        c.valid = c.it < it_end;
-        const v4i item = scalar_load_x4(p.items + (c.valid ? c.it : it_end - 1));
-        c.expert = item.x; c.row_start = item.y; c.rows = item.z; c.n_tile = item.w;
-    };
-    // An item takes nk4 positions, nk rounded up to a multiple of four (the length of the ring of
-    // register sets): its last position is then always one of set 3, and the epilogue code exists
-    // once instead of once per set. The padding positions fetch and compute nothing.
-    const int nk4 = (nk + 3) & ~3;
-    auto advance = [&](Cursor& c) __attribute__((always_inline)) {
-        if (++c.kt == nk4) { c.kt = 0; c.it += it_stride; load_item(c); }
-    };
-    Cursor cc{it0, 0}, ca{it0, 0}, cb{it0, 0};  // compute, activation fetch, weight fetch
-    load_item(cc);
-    ca = cc; cb = cc;
-    // buffer descriptors of the weight fetch position's item, rebuilt only when the item changes
-    v4i cb_srd_b, cb_srd_sb;
-    auto cb_descriptors = [&]() __attribute__((always_inline)) {
-        cb_srd_b = make_srd(p.B + (size_t)cb.expert * p.b_expert_stride + (size_t)cb.n_tile * nk * kMoeBTile,
-                            cb.valid ? (uint32_t)nk * kMoeBTile : 0u);
-        cb_srd_sb = make_srd(p.SB + (size_t)cb.expert * p.sb_expert_stride + (size_t)cb.n_tile * nk * kMoeScaleB,
-                             cb.valid ? (uint32_t)nk * kMoeScaleB : 0u);
-    };
-    cb_descriptors();
-    auto advance_cb = [&]() __attribute__((always_inline)) {
-        if (++cb.kt == nk4) { cb.kt = 0; cb.it += it_stride; load_item(cb); cb_descriptors(); }
-    };
-
-    // ---- activation tile: global -> LDS -------------------------------------------------------
-    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
-    const uint32_t lds_wave = to_sgpr(lds0 + (uint32_t)w * 1024u);
-    const uint32_t lds_sa_wave = to_sgpr(lds0 + kStATile + (uint32_t)w * 192u);
-    const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);
-    uint32_t voff_a[3];
-#pragma unroll
-    for (int i = 0; i < 3; ++i) voff_a[i] = (uint32_t)(8 * (i * 8 + w) + (lane >> 3)) * 128u + chunk16 * 16u;
-    const uint32_t voff_sa = (uint32_t)(w * 192 + lane * 16);
-    // 4 loads: rows 8(8i + w) .. +8 of the tile for i = 0..2 (skipped, i.e. issued against an
-    // empty buffer, past the item's last fragment) and the row scales of rows [24 w, +24)
-    auto issue_a = [&](const Cursor& c, int stage) __attribute__((always_inline)) {
-        v4i ssa = srd_sa;
-        if (!c.valid || c.kt >= nk) ssa.z = 0;
-        const int rows_up = c.valid && c.kt < nk ? (c.rows + 15) & ~15 : 0;
-        const uint32_t row_base = (uint32_t)c.kt * (uint32_t)p.S + (uint32_t)c.row_start;
-        const uint32_t dst = lds_wave + (uint32_t)stage * kStStage;
-#pragma unroll
-        for (int i = 0; i < 3; ++i) {
-            v4i sa = srd_a;
-            if (8 * (i * 8 + w) >= rows_up) sa.z = 0;
-            dma16(sa, dst + i * 8192, voff_a[i], row_base * 128u);
-        }
-        dma16_lanes(ssa, lds_sa_wave + (uint32_t)stage * kStStage, voff_sa, row_base * 8u, 0xfffull);
-    };
-
-    // ---- weights: global -> registers -----------------------------------------------------------
-    // pre-shuffled layout (moe_preshuffle_kernel): [expert][n-tile][K-step][wave][fragment][lane][16]
-    const uint32_t voff_b = lane * 16, voff_sb = lane * 4;
-    v4i bw[4][2][NT];  // [K-step mod 4][K half][fragment]
-    int bsc[4];        // [K-step mod 4]: the lane's scale bytes, byte 2 * half + fragment
-    // Bytes of the last K-step that lie inside K (the layout pads every row to whole K-steps with
-    // zeros): lane l's 16 bytes of half h start at byte 64 h + 16 (l / 16) of the K-step. Lanes
-    // past the end get bit 31 in their offset: outside the buffer, so the load returns the same
-    // zeros without fetching them (K = 2880: 6 % of the weight bytes).
-    const int last_valid = Kb - (nk - 1) * 128;
-    auto load_b_half = [&](const Cursor& c, v4i (&dst)[NT], int half) __attribute__((always_inline)) {
-        v4i rs = cb_srd_b;
-        if (c.kt >= nk) rs.z = 0;
-        const uint32_t soff = (uint32_t)c.kt * kMoeBTile + (uint32_t)w * 4096u + (uint32_t)half * 1024u;
-        // first padded lane * 16 - 1 (uniform); voff_b = 16 l exceeds it exactly in the padded lanes
-        const int thr = c.kt == nk - 1 ? 16 * min(max(last_valid - 64 * half, 0), 64) - 1 : 0x7fffffff;
-        const uint32_t voff = voff_b | ((uint32_t)(thr - (int)voff_b) & 0x80000000u);
-#pragma unroll
-        for (int n = 0; n < NT; ++n)
-            asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"
-                         : "=v"(dst[n])
-                         : "v"(voff), "s"(rs), "s"(soff + n * 2048u)
-                         : "memory");
-    };
-    auto load_b_scales = [&](const Cursor& c, int& dst) __attribute__((always_inline)) {
-        v4i rss = cb_srd_sb;
-        if (c.kt >= nk) rss.z = 0;
-        asm volatile("buffer_load_dword %0, %1, %2, %3 offen"
-                     : "=v"(dst)
-                     : "v"(voff_sb), "s"(rss), "s"((uint32_t)c.kt * kMoeScaleB + (uint32_t)w * 256u)
-                     : "memory");
-    };
-    auto landed = [&](v4i (&x)[NT]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int n = 0; n < NT; ++n) asm volatile("" : "+v"(x[n]));
-    };
-
-    // ---- LDS -> registers (activation fragments) ------------------------------------------------
-    const uint32_t r = lane & 15, g = lane >> 4;
-    const uint32_t rd_half[2] = {lds0 + r * 128u + swz_chunk(r, g) * 16u, lds0 + r * 128u + swz_chunk(r, g + 4) * 16u};
-    const uint32_t sa_rd0 = lds0 + kStATile + r * 8u;
-    const uint32_t sh = 8u * g;  // byte g of each scale dword belongs to this lane
-
-    v4f acc[MT][NT];
-    auto zero_acc = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int m = 0; m < MT; ++m)
-#pragma unroll
-            for (int n = 0; n < NT; ++n) acc[m][n] = v4f{0.f, 0.f, 0.f, 0.f};
-    };
-    auto mfma = [&](v4f& c, const v4i& x, const v4i& y, int sx, int sy) __attribute__((always_inline)) {
-        asm volatile(
-            "v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"
-            : "+v"(c)
-            : "v"(x), "v"(y), "v"(sx), "v"(sy));
-    };
-    // MFMAs of one K half (128 of the K-step's 256 elements) on LDS stage st. Activation fragment
-    // m + 2 is read from LDS before the MFMAs of fragment m are issued; fragments past the tile's
-    // row count are skipped (the conditions are uniform and nested).
-    auto compute_half = [&](int st, int half, int rows, const v4i (&bfr)[NT], int bscale)
-                            __attribute__((always_inline)) {
-        uint32_t a_rd = rd_half[half] + (uint32_t)st * kStStage;
-        uint32_t sa_rd = sa_rd0 + (uint32_t)st * kStStage + 4u * half;
-        asm volatile("" : "+v"(a_rd), "+v"(sa_rd));  // keep the bases in registers, offsets as immediates
-        int bs[NT];
-#pragma unroll
-        for (int n = 0; n < NT; ++n) bs[n] = (int)((uint32_t)bscale >> (8 * (2 * half + n)));
-        const int mt = (rows + 15) >> 4;
-        v4i af[3];
-        uint32_t as[3];
-        auto rd = [&](int m) __attribute__((always_inline)) {
-            af[m % 3] = *(lds_v4i_t*)(uintptr_t)(a_rd + m * 2048);
-            as[m % 3] = *(__attribute__((address_space(3))) const uint32_t*)(uintptr_t)(sa_rd + m * 128);
-        };
-        // nested conditions (fragment m is reached only through fragment m - 1), so that every
-        // block has one way in and the compiler's LDS wait counts stay exact
-        auto frag = [&]<int M>(auto&& self) __attribute__((always_inline)) {
-            if constexpr (M < MT) {
-                if (M < mt) {
-                    if (M + 2 < MT) rd(M + 2);  // rows past the tile's count are readable, never used
-                    const int sa = (int)(as[M % 3] >> sh);
-#pragma unroll
-                    for (int n = 0; n < NT; ++n) mfma(acc[M][n], bfr[n], af[M % 3], bs[n], sa);
-                    self.template operator()<M + 1>(self);
-                }
-            }
-        };
-        if (mt > 0) {
-            rd(0);
-            rd(1);
-            frag.template operator()<0>(frag);
-        }
-    };
-
-    auto epilogue = [&](const Cursor& c) __attribute__((always_inline)) {
-        const int rows = c.rows, row_start = c.row_start;
-        if (MODE == 1) {
-            // lane (r, g) holds, for row 16 m + r, the 8 consecutive columns 32 w + 8 g .. +8
-            uint16_t* out = (uint16_t*)p.out0;
-            const int col = c.n_tile * 256 + w * 32 + 8 * (int)g;
-            // extended epilogue: the wave's 32 bias values come through the scalar cache (vector
-            // loads here would make the compiler drain the weight prefetch), each lane group picks
-            // its 8. N % 32 == 0: the wave's columns are valid or not as a whole.
-            v4f b0 = {0.f, 0.f, 0.f, 0.f}, b1 = {0.f, 0.f, 0.f, 0.f};
-            const int wcol0 = c.n_tile * 256 + w * 32;
-            if (EXT && p.bias && wcol0 < p.N) {
-                float lo[16], hi[16];
-                const float* bb = p.bias + (size_t)c.expert * p.N + wcol0;
-                scalar_load_f16(bb, lo);
-                scalar_load_f16(bb + 16, hi);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    b0[i] = g == 0 ? lo[i] : g == 1 ? lo[8 + i] : g == 2 ? hi[i] : hi[8 + i];
-                    b1[i] = g == 0 ? lo[4 + i] : g == 1 ? lo[12 + i] : g == 2 ? hi[4 + i] : hi[12 + i];
-                }
-            }
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                const int row = 16 * m + (int)r;
-                if (row >= rows || col + 8 > p.N) continue;  // N % 8 == 0
-                v4f x = acc[m][0], y = acc[m][1];
-                if (EXT) { x += b0; y += b1; }
-                v4i o4;
-                o4.x = pack_bf16(x.x, x.y); o4.y = pack_bf16(x.z, x.w);
-                o4.z = pack_bf16(y.x, y.y); o4.w = pack_bf16(y.z, y.w);
-                store_global_b128(out + (size_t)(row_start + row) * p.N + col, o4);
-            }
-        } else {
-            // h = silu(gate) * up: lane (r, g) holds, for row 16 m + r, the h columns
-            // 128 n_tile + 16 w + 4 g .. +4. An MX block of 32 columns spans waves 2u and 2u + 1:
-            // row maxima are exchanged through LDS, the packed tile (64 bytes per row) and its
-            // scales are assembled in LDS and leave with 16-byte stores.
-            typedef __attribute__((address_space(3))) float lds_f32_mut_t;
-            typedef __attribute__((address_space(3))) uint16_t lds_u16_mut_t;
-            typedef __attribute__((address_space(3))) uint8_t lds_u8_mut_t;
-            const int hcol0 = c.n_tile * 128 + 16 * w;  // first of the wave's 16 h columns
-            const bool col_ok = hcol0 < p.N;            // N % 32 == 0: a block is valid as a whole
-            // extended epilogue: biases of this lane's 4 h columns hcol0 + 4 g .. +4
-            // (through the scalar cache, as above: 16 gate + 16 up values per wave)
-            float bg[4] = {0.f, 0.f, 0.f, 0.f}, bu[4] = {0.f, 0.f, 0.f, 0.f};
-            if (EXT && p.bias && col_ok) {
-                const float* bb = p.bias + (size_t)c.expert * 2 * p.N;
-                float x0[16], x1[16];   // plain rows: gate / up; interleaved: columns 0-7 / 8-15, gate and up alternating
-                scalar_load_f16(p.interleaved ? bb + 2 * hcol0 : bb + hcol0, x0);
-                scalar_load_f16(p.interleaved ? bb + 2 * hcol0 + 16 : bb + p.N + hcol0, x1);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float pg = g == 0 ? x0[j] : g == 1 ? x0[4 + j] : g == 2 ? x0[8 + j] : x0[12 + j];
-                    const float pu = g == 0 ? x1[j] : g == 1 ? x1[4 + j] : g == 2 ? x1[8 + j] : x1[12 + j];
-                    // interleaved: lane group g's columns 4 g + j sit at floats 8 g + 2 j (+ 1) of the 32
-                    const float ig = g == 0 ? x0[2 * j] : g == 1 ? x0[8 + 2 * j] : g == 2 ? x1[2 * j] : x1[8 + 2 * j];
-                    const float iu = g == 0 ? x0[2 * j + 1] : g == 1 ? x0[9 + 2 * j] : g == 2 ? x1[2 * j + 1] : x1[9 + 2 * j];
-                    bg[j] = p.interleaved ? ig : pg;
-                    bu[j] = p.interleaved ? iu : pu;
-                }
-            }
-            // two groups of six fragments, to keep the number of live h values small
-#pragma unroll
-            for (int m0 = 0; m0 < MT; m0 += MT / 2) {
-                float h[MT / 2][4];
-#pragma unroll
-                for (int mm = 0; mm < MT / 2; ++mm) {
-                    const int m = m0 + mm;
-                    if (16 * m >= rows) continue;  // uniform: the whole fragment is padding
-                    const v4f gt = acc[m][0], up = acc[m][1];
-                    float amax = 0.f;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        if (EXT) h[mm][j] = col_ok ? glu_act(p.act, gt[j] + bg[j], up[j] + bu[j], p.alpha, p.limit) : 0.f;
-                        else h[mm][j] = col_ok ? silu_mul(gt[j], up[j]) : 0.f;
-                        amax = fmaxf(amax, fabsf(h[mm][j]));
-                    }
-                    amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-                    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-                    if (g == 0) *(lds_f32_mut_t*)(uintptr_t)(lds0 + kStXch + ((16 * m + r) * 8 + w) * 4) = amax;
-                }
-                __syncthreads();
-#pragma unroll
-                for (int mm = 0; mm < MT / 2; ++mm) {
-                    const int m = m0 + mm;
-                    if (16 * m >= rows) continue;
-                    const uint32_t row = 16 * m + r;
-                    const v2f am = *(__attribute__((address_space(3))) const v2f*)(uintptr_t)(lds0 + kStXch + (row * 8 + (w & ~1)) * 4);
-                    const int e = mx_block_exponent(fmaxf(am.x, am.y));
-                    const float scale = __uint_as_float(e > -127 ? (uint32_t)(e + 127) << 23 : 0x00400000u);
-                    uint32_t pk = 0;
-                    pk = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(pk, h[mm][0], h[mm][1], scale, 0);
-                    pk = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(pk, h[mm][2], h[mm][3], scale, 1);
-                    *(lds_u16_mut_t*)(uintptr_t)(lds0 + kStHTile + row * 64 + 8 * w + 2 * g) = (uint16_t)pk;
-                    if (g == 0 && (w & 1) == 0)
-                        *(lds_u8_mut_t*)(uintptr_t)(lds0 + kStHScale + row * 4 + (w >> 1)) = col_ok ? (uint8_t)(e + 127) : (uint8_t)127;
-                }
-            }
-            __syncthreads();
-            uint8_t* hq = (uint8_t*)p.out0;
-            const size_t kt2 = (size_t)(c.n_tile >> 1);
-            const int seg = (c.n_tile & 1) * 64;  // the n-tile's 128 columns are half of a K-step row
-#pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                const int chunk = (int)threadIdx.x + 512 * q;  // 16-byte chunk of the [kStBM][64] tile
-                const int row = chunk >> 2, part = chunk & 3;
-                if (row < rows) {
-                    const v4i v = *(lds_v4i_t*)(uintptr_t)(lds0 + kStHTile + chunk * 16);
-                    store_global_b128(hq + (kt2 * p.S + (size_t)(row_start + row)) * 128 + seg + part * 16, v);
-                }
-            }
-            if ((int)threadIdx.x < rows) {
-                const uint32_t v = *(__attribute__((address_space(3))) const uint32_t*)(uintptr_t)(lds0 + kStHScale + threadIdx.x * 4);
-                store_global_b32(p.out_scales + (kt2 * p.S + (size_t)(row_start + threadIdx.x)) * 8 + (seg >> 4), v);
-            }
-        }
-    };
-
-    // ---- prologue: activation positions 0..3 and weight positions 0..3, in the order the K loop
-    // issues them (4 activation loads, then 2 + 3 weight loads per position)
-    auto load_b_set = [&]<int P>() __attribute__((always_inline)) {
-        load_b_half(cb, bw[P][0], 0);
-        load_b_scales(cb, bsc[P]);
-        load_b_half(cb, bw[P][1], 1);
-        advance_cb();
-    };
-    issue_a(ca, 0); advance(ca); load_b_set.template operator()<0>();
-    issue_a(ca, 1); advance(ca); load_b_set.template operator()<1>();
-    issue_a(ca, 2); advance(ca); load_b_set.template operator()<2>();
-    issue_a(ca, 3); advance(ca); load_b_set.template operator()<3>();
-    zero_acc();
-
-    // One stream position on LDS stage st with register set P. In program order a wave issues per
-    // position 9 loads: 4 activation loads (position +4), after the first K half 2 weight loads,
-    // after the second one 1 scale load + 2 weight loads (position +4, into the registers the
-    // MFMAs before them have just finished with). Loads return in order, so counting the loads
-    // issued after the ones needed gives the waits:
-    //   first K half:  scales and weights are followed by 2 + 27 (three positions)   -> vmcnt(29)
-    //   second K half: by 27 + 4 + 2 (this position so far)                          -> vmcnt(33)
-    // and the position's activation tile is older than both. Stores share the counter and
-    // complete out of order, which only makes these waits stricter.
-    auto step = [&]<int P>(int st) __attribute__((always_inline)) {
-        wait_vmcnt<29>();
-        block_barrier();  // everyone's part of this position's tile has landed; stage st-1 is free
-        issue_a(ca, st == 0 ? kStStages - 1 : st - 1); advance(ca);
-        landed(bw[P][0]);
-        asm volatile("" : "+v"(bsc[P]));
-        const int sc = bsc[P];
-        const int rows = cc.valid && cc.kt < nk ? cc.rows : 0;  // padding / past the end of the stream: no MFMAs, empty loads
-        compute_half(st, 0, rows, bw[P][0], sc);
-        load_b_half(cb, bw[P][0], 0);
-        wait_vmcnt<33>();
-        landed(bw[P][1]);
-        compute_half(st, 1, rows, bw[P][1], sc);
-        load_b_scales(cb, bsc[P]);
-        load_b_half(cb, bw[P][1], 1);
-        advance_cb();
-        if constexpr (P == 3) {
-            if (cc.valid && cc.kt == nk4 - 1) {
-                mfma_drain_vgpr(acc);
-                epilogue(cc);
-                zero_acc();
-            }
-        }
-        advance(cc);
-    };
-    // Four positions per trip (the register sets rotate); positions past the end of the stream
-    // degenerate to their barrier and empty loads. No exit inside a trip: a second way into the
-    // loop head would hand the compiler two load histories to merge.
-    int st = 0;
-    auto next_stage = [&]() __attribute__((always_inline)) { st = st == kStStages - 1 ? 0 : st + 1; };
-    while (cc.valid) {
-        step.template operator()<0>(st); next_stage();
-        step.template operator()<1>(st); next_stage();
-        step.template operator()<2>(st); next_stage();
-        step.template operator()<3>(st); next_stage();
-    }
-    wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
-}
-
-// ------------------------------------------------------- 4-wave weight-streaming grouped GEMM
-// The same stream with one wave per SIMD, for the plain epilogues (SiLU-mul with MX re-quantization,
-// bf16 store); the 8-wave kernel above serves the extended ones. Wave W takes what waves 2W and
-// 2W + 1 of that kernel take: weight rows [64 W, +64) of the 256-row tile (four fragments) x all
-// rows of the item, 192 accumulator registers per lane, updated in place in AGPRs. What that buys:
+//   * only the activation tile (shared by the waves, re-read from L2) goes through LDS, in four
+//     stages filled by direct global->LDS loads. Loads return in order.
+// One workgroup of 4 waves per CU, one wave per SIMD. Wave W owns weight rows [64 W, +64) of the
+// 256-row tile (four fragments) x all rows of the item: 192 accumulator registers per lane,
+// updated in place in AGPRs. The K-step stream runs across item boundaries. All vector-memory
+// operations are inline asm and counted by hand (the compiler never waits for them). Results are
+// bit-identical to moe_mxfp4_gemm_kernel (same accumulation order per output element).
 //   * the 32 h columns of a wave are exactly one MX block, so the gate+up epilogue needs no
 //     exchange between waves, no LDS and no workgroup barrier: block maxima and a row's 16 packed
 //     bytes are gathered inside the wave by swapping rows of 16 lanes in registers
@@ -1123,15 +757,17 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
 // row scales (global -> LDS, four stages), eight 1 KiB weight fragments and two scale dwords
 // (global -> VGPRs, four register sets). Position q's loads are issued during position q - 3; they
 // return in order, so at the start of position q everything of it has landed when at most the 34
-// loads of positions q + 1 and q + 2 are outstanding. Bit-identical to the kernels above.
-// Measured at the GPT-OSS-like shape (kernel trace, us, gate+up / down): 275 / 148 (8-wave kernel:
-// 293 / 152); without epilogues 227 / 115; loads, waits and barriers only 206 / 103; the K loop's
-// MFMAs and LDS reads on empty loads 148 / 78. The K loop hides behind the weight stream, the
-// epilogue does not: while a wave spends about 8 k clocks finishing an item, the three positions it
-// has in flight (about 6.6 k clocks of the stream) run dry. An epilogue copy per register set (four
-// times the code) cost another 7 %: the loop then no longer fits the instruction cache. Requesting
-// the weights of one or two further positions into L2 at the start of an item's last position
-// (one dword per 64 bytes into a dump area of LDS) changed nothing / cost 2 %: not kept.
+// loads of positions q + 1 and q + 2 are outstanding.
+// Measured at the GPT-OSS-like shape (kernel trace, us, gate+up / down): 275 / 148; without
+// epilogues 227 / 115; loads, waits and barriers only 206 / 103; the K loop's MFMAs and LDS reads
+// on empty loads 148 / 78. The K loop hides behind the weight stream, the epilogue does not. An
+// epilogue copy per register set (four times the code) cost another 7 %: the loop then no longer
+// fits the instruction cache. Requesting the weights of one or two further positions into L2 at
+// the start of an item's last position changed nothing / cost 2 %; parking four fragments'
+// accumulators in the spare AGPRs and finishing them in the next item's first position cost
+// 6 us per layer: not kept. A predecessor with 8 waves (two per SIMD, 32 weight rows per wave,
+// an LDS exchange in the gate+up epilogue) took 293 / 152 us with the plain epilogues and, for the
+// extended ones, 9 us more per layer than this kernel; it is no longer in the tree.
 //
 // A8: the activations are MXFP8 (e4m3 elements, 256 bytes per row and K-step, same e8m0 scale
 // layout) and the MFMA is the mixed form (fp4 weights x fp8 activations, 32 cycles). The
@@ -1139,10 +775,10 @@ __global__ __launch_bounds__(512, 2) void moe_mxfp4_stream_kernel(const MoeGemmP
 // swizzle, the load pieces and the fragment addressing stay those of the FP4 tile; a lane's
 // 32 bytes of a K half are the 16-byte chunks g and g + 4. Items have up to 128 rows then
 // (four 33 KiB stages), and the gate+up epilogue re-quantizes h to MXFP8.
-// EXT: biases / clamped SwiGLU / interleaved source rows in the epilogue (instantiated with A8
-// only; for MXFP4 activations the 8-wave kernel is the faster one there).
+// EXT: biases / clamped SwiGLU / interleaved source rows in the epilogue.
 // GATHER (gate+up, plain epilogue): the item's rows are fetched by token from x quantized once per
 // token, and their scales once per 16 K-steps; see the kernel body. 16 loads per position then.
+constexpr int kStBM = 192;                              // rows per work item
 template <bool A8>
 struct S4Cfg {
     static constexpr int kBM = A8 ? 128 : kStBM;       // rows per work item
@@ -1215,6 +851,54 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
                              cf.valid ? (uint32_t)nk * kMoeScaleB : 0u);
     };
     cf_descriptors();
+    // EXT: the lane's bias values. They are fetched when the FETCH cursor enters an item (four
+    // 16-byte loads into bias_nxt: extra loads in the counted stream, which only makes the waits
+    // stricter) and taken over when the compute cursor enters it, three positions later. (Fetching
+    // them in the item's last K-step through the scalar cache stalled the wave for the latency of
+    // two dependent loads per item: 62 us per layer at the GPT-OSS-like shape.)
+    // MODE 0: lane (r, g) needs gate / up biases of h columns 128 n_tile + 32 w + 16 o + 4 g .. +4:
+    // loads 2 o / 2 o + 1 = gate / up (plain row order) or the 8 interleaved floats (gate and up
+    // alternating). MODE 1: output columns 256 n_tile + 64 w + 32 o + 8 g .. +8: loads 2 o, 2 o + 1.
+    // Columns past N read other experts' values or zeros; their results are dropped.
+    float bias_a[2][4], bias_b[2][4];  // MODE 0: [pair][j] gate / up; MODE 1: [pair][j] columns 8 g + j / 8 g + 4 + j
+    v4f bias_nxt[4];
+    const v4i srd_bias = make_srd(p.bias, EXT && p.bias ? 0xffffffffu : 0u);
+    auto request_bias = [&]() __attribute__((always_inline)) {
+        if constexpr (EXT) {
+            const uint32_t gq = (uint32_t)(lane >> 4);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int o = q >> 1, part = q & 1;
+                uint32_t idx;  // float index into the bias array
+                if (MODE == 1) {
+                    idx = (uint32_t)cf.expert * (uint32_t)p.N + (uint32_t)(cf.n_tile * 256 + 64 * w + 32 * o) + 8u * gq + 4u * part;
+                } else {
+                    const uint32_t hcol = (uint32_t)(cf.n_tile * 128 + 32 * w + 16 * o) + 4u * gq;
+                    idx = (uint32_t)cf.expert * 2u * (uint32_t)p.N +
+                          (p.interleaved ? 2u * hcol + 4u * part : (uint32_t)(part * p.N) + hcol);
+                }
+                v4f& dst = bias_nxt[q];
+                const v4i rs = srd_bias;
+                const uint32_t voff = idx * 4u;
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(dst) : "v"(voff), "s"(rs) : "memory");
+            }
+        }
+    };
+    auto adopt_bias = [&]() __attribute__((always_inline)) {
+        if constexpr (EXT) {
+#pragma unroll
+            for (int o = 0; o < 2; ++o) {
+                const v4f x0 = bias_nxt[2 * o], x1 = bias_nxt[2 * o + 1];
+                if (MODE == 0 && p.interleaved) {
+                    bias_a[o][0] = x0.x; bias_b[o][0] = x0.y; bias_a[o][1] = x0.z; bias_b[o][1] = x0.w;
+                    bias_a[o][2] = x1.x; bias_b[o][2] = x1.y; bias_a[o][3] = x1.z; bias_b[o][3] = x1.w;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) { bias_a[o][j] = x0[j]; bias_b[o][j] = x1[j]; }
+                }
+            }
+        }
+    };
     // GATHER: byte offset of the lane's row inside a K-step plane of A for each activation piece i
     // (the row is 8 (4 i + w) + lane / 8), plus the lane's 16-byte chunk: for the fetch item
     // (tok_cur) and, as raw slot numbers still in flight, for the item after it (tok_nxt). The slots
@@ -1286,12 +970,18 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
         request_next_item();
         fetch_scale_rows();
     }
+    if constexpr (EXT) {
+        request_bias();
+        wait_vmcnt<0>();
+        adopt_bias();
+    }
     // The 2 kNp loads a change of the fetch item adds (slots, scale rows) sit between the counted loads
     // of two positions: the waits of the next three positions allow for them.
     int cf_extra = 0;
     auto advance_cf = [&]() __attribute__((always_inline)) {
         if (++cf.kt == nk4) {
             cf.kt = 0; cf.it += it_stride; load_item(cf); cf_descriptors();
+            request_bias();
             if constexpr (GATHER) { adopt_tokens(); request_next_item(); cf_extra = 3; }
         }
         if constexpr (GATHER)
@@ -1396,52 +1086,6 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
     };
 
     // ---- epilogue of row fragment m of the compute item (its accumulators are final) -------------
-    // EXT: the lane's bias values, fetched at the start of the item's last K-step
-    float bias_a[2][4], bias_b[2][4];  // MODE 0: [pair][j] gate / up; MODE 1: [pair][j] columns 8 g + j / 8 g + 4 + j
-    auto load_bias = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int o = 0; o < 2; ++o)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) bias_a[o][j] = bias_b[o][j] = 0.f;
-        if (!EXT || !p.bias) return;
-        // through the scalar cache: vector loads here would join the counted weight stream
-        if (MODE == 1) {
-#pragma unroll
-            for (int o = 0; o < 2; ++o) {
-                const int wcol0 = cc.n_tile * 256 + (2 * w + o) * 32;  // N % 32 == 0: valid or not as a whole
-                if (wcol0 >= p.N) continue;
-                float lo[16], hi[16];
-                const float* bb = p.bias + (size_t)cc.expert * p.N + wcol0;
-                scalar_load_f16(bb, lo);
-                scalar_load_f16(bb + 16, hi);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    bias_a[o][i] = g == 0 ? lo[i] : g == 1 ? lo[8 + i] : g == 2 ? hi[i] : hi[8 + i];
-                    bias_b[o][i] = g == 0 ? lo[4 + i] : g == 1 ? lo[12 + i] : g == 2 ? hi[4 + i] : hi[12 + i];
-                }
-            }
-        } else {
-#pragma unroll
-            for (int o = 0; o < 2; ++o) {
-                const int hcol0 = cc.n_tile * 128 + 32 * w + 16 * o;
-                if (hcol0 >= p.N) continue;
-                const float* bb = p.bias + (size_t)cc.expert * 2 * p.N;
-                float x0[16], x1[16];   // plain rows: gate / up; interleaved: columns 0-7 / 8-15, gate and up alternating
-                scalar_load_f16(p.interleaved ? bb + 2 * hcol0 : bb + hcol0, x0);
-                scalar_load_f16(p.interleaved ? bb + 2 * hcol0 + 16 : bb + p.N + hcol0, x1);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float pg = g == 0 ? x0[j] : g == 1 ? x0[4 + j] : g == 2 ? x0[8 + j] : x0[12 + j];
-                    const float pu = g == 0 ? x1[j] : g == 1 ? x1[4 + j] : g == 2 ? x1[8 + j] : x1[12 + j];
-                    // interleaved: lane group g's columns 4 g + j sit at floats 8 g + 2 j (+ 1) of the 32
-                    const float ig = g == 0 ? x0[2 * j] : g == 1 ? x0[8 + 2 * j] : g == 2 ? x1[2 * j] : x1[8 + 2 * j];
-                    const float iu = g == 0 ? x0[2 * j + 1] : g == 1 ? x0[9 + 2 * j] : g == 2 ? x1[2 * j + 1] : x1[9 + 2 * j];
-                    bias_a[o][j] = p.interleaved ? ig : pg;
-                    bias_b[o][j] = p.interleaved ? iu : pu;
-                }
-            }
-        }
-    };
     // Stores go through buffer descriptors that end at the item's last row: rows of the last
     // fragment beyond it (they belong to the next expert) are dropped by the range check, so the
     // epilogue needs no per-lane row test and no 64-bit address arithmetic. Lanes that do not
@@ -1578,7 +1222,6 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
         const int mt_item = cc.valid ? (cc.rows + 15) >> 4 : 0;
         const bool last = P == 3 && cc.valid && cc.kt == nk4 - 1;
         if (last) {
-            if (EXT) load_bias();
             begin_epilogue();
         }
         int bs[8];  // scale of weight fragment f = 4 pair + 2 n + half: byte 2 half + n of the pair's dword
@@ -1641,7 +1284,7 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
         advance_cf();
         if constexpr (P == 3)
             if (last && MT - 1 < mt_item) epilogue.template operator()<MT - 1>(true);
-        if (++cc.kt == nk4) { cc.kt = 0; cc.it += it_stride; load_item(cc); }
+        if (++cc.kt == nk4) { cc.kt = 0; cc.it += it_stride; load_item(cc); adopt_bias(); }
     };
     // Four positions per trip (stages and register sets rotate); positions past the end of the
     // stream degenerate to their barrier and empty loads.
@@ -1741,15 +1384,8 @@ void moe_launch_build_items(const int32_t* expert_offsets, int E, int bm, int n_
 
 template <int MODE, bool EXT, bool A8, bool GATHER = false>
 static int launch_moe_stream(MoeGemmParams p, int max_items, hipStream_t s) {
-    // Plain epilogues (SiLU-mul / bf16 store): the 4-wave kernel. With biases, the clamped SwiGLU or
-    // interleaved source rows the per-element work of the epilogue is larger and two waves per SIMD
-    // hide it better: the 8-wave kernel (measured: 0.51 against 0.57 ms for the layer). MXFP8
-    // activations: the 4-wave kernel in both cases.
-    constexpr bool k8wave = EXT && !A8;
-    constexpr int lds = k8wave ? kStLds : GATHER ? S4Cfg<A8>::kLdsGather : S4Cfg<A8>::kLds, threads = k8wave ? 512 : 256;
-    const void* kern;
-    if constexpr (k8wave) kern = (const void*)moe_mxfp4_stream_kernel<MODE, true>;
-    else kern = (const void*)moe_mxfp4_stream4_kernel<MODE, EXT && A8, A8, GATHER>;
+    constexpr int lds = GATHER ? S4Cfg<A8>::kLdsGather : S4Cfg<A8>::kLds, threads = 256;
+    const void* kern = (const void*)moe_mxfp4_stream4_kernel<MODE, EXT, A8, GATHER>;
     static DeviceOnce configured;
     if (!set_lds_limit_once(kern, lds, configured)) return HK_ERR_LAUNCH;
     // persistent: one workgroup per CU, each walking its share of the item list
