@@ -1284,7 +1284,11 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
         advance_cf();
         if constexpr (P == 3)
             if (last && MT - 1 < mt_item) epilogue.template operator()<MT - 1>(true);
-        if (++cc.kt == nk4) { cc.kt = 0; cc.it += it_stride; load_item(cc); adopt_bias(); }
+        if (++cc.kt == nk4) {
+            // the fetch cursor entered this item three positions ago and is still in it (nk4 >= 4)
+            cc = cf; cc.kt = 0;
+            adopt_bias();
+        }
     };
     // Four positions per trip (stages and register sets rotate); positions past the end of the
     // stream degenerate to their barrier and empty loads.
