@@ -1320,6 +1320,8 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
 // is null.
 // KU > 0: k <= KU, the token's positions and weights are read once and the k rows' loads of a column
 // chunk are issued together; KU == 0: any k, one row at a time. Same operations in the same order.
+// The rows of o are read exactly once: non-temporal loads (213 -> 187 us at T = 8192, k = 8,
+// H = 7168, i.e. 5.7 TB/s; the GPT-OSS-like layer 10 us less).
 template <int KU>
 __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __restrict__ o,
                                                             const float* __restrict__ w,
@@ -1341,7 +1343,7 @@ __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __re
         v4i rows[KU > 0 ? KU : 1];
 #pragma unroll
         for (int j = 0; j < KU; ++j)
-            if (j < k) rows[j] = *(const v4i*)(o + (size_t)pos[j] * H + c * 8);
+            if (j < k) rows[j] = __builtin_nontemporal_load((const v4i*)(o + (size_t)pos[j] * H + c * 8));
         if (add) {
             const v4i raw = *(const v4i*)(add + (size_t)t * H + c * 8);
 #pragma unroll
