@@ -45,7 +45,7 @@ PEAK_HBM = 8000.0     # GB/s
 # profiles/fp8_gemm_4wave_ring_kernel_8192.md (805.8 MB read + 137.3 MB written).
 TRAFFIC_FP8_8192 = 943.1e6
 # Other legs: profiles/traffic_counters_moe_and_gemm_legs.md (MoE legs: sum over the layer's launches).
-TRAFFIC = {"moe_mxfp4": 2.195e9, "moe_fp8blk": 14.30e9, "mxfp4_gemm": 562.7e6, "bf16_gemm": 1.748e9}
+TRAFFIC = {"moe_mxfp4": 2.094e9, "moe_fp8blk": 14.30e9, "mxfp4_gemm": 562.7e6, "bf16_gemm": 1.748e9}
 
 
 def _traffic(key):
