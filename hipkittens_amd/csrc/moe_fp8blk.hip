@@ -521,12 +521,17 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
     v4i f_srd_a, f_srd_sa, f_srd_b;
     uint32_t f_soff_a, f_soff_sa, f_soff_b;
     int f_pieces;   // (not GATHER) pieces of this wave that hold rows of the item; the others fetch nothing
+    // the fetch item's weight tile: found when the cursor enters the item, inside the branch that loads
+    // the item (written as a conditional assignment elsewhere the compiler computes it at every position)
+    auto b_tile_of = [&](const F8Cursor& c) __attribute__((always_inline)) {
+        return p.B + (size_t)c.expert * p.b_expert_stride + (size_t)c.n_tile * nk * kF8sBTile;
+    };
+    const uint8_t* f_b_base = b_tile_of(cf);
     auto fetch_begin = [&]() __attribute__((always_inline)) {
         f_srd_a = srd_a; f_srd_sa = srd_sa;
         const bool live = cf.valid && cf.kt < nk;   // not past the stream's end, not a padding position
         if (!live) { f_srd_a.z = 0; f_srd_sa.z = 0; }
-        f_srd_b = make_srd(p.B + (size_t)cf.expert * p.b_expert_stride + (size_t)cf.n_tile * nk * kF8sBTile,
-                           live ? (uint32_t)nk * kF8sBTile : 0u);
+        f_srd_b = make_srd(f_b_base, live ? (uint32_t)nk * kF8sBTile : 0u);
         const uint32_t row_base = (uint32_t)cf.kt * (uint32_t)p.S + (uint32_t)cf.row_start;
         f_soff_a = GATHER ? (uint32_t)cf.kt * 128u : row_base * 128u;
         f_soff_sa = GATHER ? (uint32_t)cf.kt * 4u : row_base * 4u;
@@ -536,6 +541,7 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
     auto fetch_advance = [&]() __attribute__((always_inline)) {
         if (++cf.kt == nk4) {
             cf.kt = 0; cf.it += it_stride; load_item(cf);
+            f_b_base = b_tile_of(cf);
             if (GATHER) {
                 // the ids were requested when the cursor entered the previous item, ahead of that
                 // position's loads, which an earlier step has waited for unless the item was shorter
@@ -638,20 +644,24 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
                      : "v"(pt.x), "v"(pt.y), "v"(pt.z), "v"(pt.w), "v"(s));
     };
     // weight scales of a position, through the scalar cache, not waited for here
-    auto request_ws = [&](const F8Cursor& c) __attribute__((always_inline)) {
+    // The scale rows of an item's two row blocks are found when a cursor enters the item (ws_rows_of, called
+    // inside the branch that loads the item); a position then adds 4 kt.
+    const float* ws_row0 = nullptr;
+    const float* ws_row1 = nullptr;
+    auto ws_rows_of = [&](const F8Cursor& c) __attribute__((always_inline)) {
         const float* sb = p.SB + (size_t)c.expert * p.sb_expert_stride;
-        const int kt = min(c.kt, nk - 1);   // a padding position multiplies zeros by the last K-step's scale
-        const float* s0;
-        const float* s1;
         if (MODE == 0) {
-            s0 = sb + (size_t)c.n_tile * nk + kt;                      // gate rows of the tile
-            s1 = sb + (size_t)(p.N / 128 + c.n_tile) * nk + kt;        // up rows
+            ws_row0 = sb + (size_t)c.n_tile * nk;                      // gate rows of the tile
+            ws_row1 = sb + (size_t)(p.N / 128 + c.n_tile) * nk;        // up rows
         } else {
-            s0 = sb + (size_t)min(2 * c.n_tile + (w >> 1), p.N / 128 - 1) * nk + kt;
-            s1 = s0;
+            ws_row0 = sb + (size_t)min(2 * c.n_tile + (w >> 1), p.N / 128 - 1) * nk;
+            ws_row1 = ws_row0;
         }
-        asm volatile("s_load_dword %0, %1, 0x0" : "=s"(ws0_next) : "s"(s0) : "memory");
-        asm volatile("s_load_dword %0, %1, 0x0" : "=s"(ws1_next) : "s"(s1) : "memory");
+    };
+    auto request_ws = [&](const F8Cursor& c) __attribute__((always_inline)) {
+        const uint32_t off = (uint32_t)min(c.kt, nk - 1) * 4u;   // a padding position multiplies zeros by the last K-step's scale
+        asm volatile("s_load_dword %0, %1, %2" : "=s"(ws0_next) : "s"(ws_row0), "s"(off) : "memory");
+        asm volatile("s_load_dword %0, %1, %2" : "=s"(ws1_next) : "s"(ws_row1), "s"(off) : "memory");
     };
 
     // Stores go through buffer descriptors that end at the item's last row: rows of the last
@@ -737,6 +747,7 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
     fetch_begin(); fetch_all.template operator()<0>(); fetch_advance();
     fetch_begin(); fetch_all.template operator()<1>(); fetch_advance();
     fetch_begin(); fetch_all.template operator()<2>(); fetch_advance();
+    ws_rows_of(cc);   // cn is still in this item (an item has at least four positions)
     request_ws(cc);
     zero_acc();
     wait_vmcnt<(kF8sStages - 2) * kF8sLoads>();
@@ -844,7 +855,7 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
             }
         }
         cc = cn;
-        advance(cn);
+        if (++cn.kt == nk4) { cn.kt = 0; cn.it += it_stride; load_item(cn); ws_rows_of(cn); }
         ws0 = ws0_next; ws1 = ws1_next;
         request_ws(cn);
     };
