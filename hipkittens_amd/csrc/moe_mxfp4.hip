@@ -427,6 +427,7 @@ struct MoeGemmParams {
     int n_tiles_n;
     // extended epilogues (kernels instantiated with EXT) only:
     const float* bias;       // null or fp32 [E][rows of B] in the caller's row order, added to the GEMM result
+    uint32_t bias_bytes;     // size of that array (the streaming kernel reads it through a range-checked descriptor)
     int act;                 // MODE 0: 0 = SiLU(gate) * up, 1 = clamped SwiGLU (glu_act)
     float alpha, limit;
     int interleaved;         // MODE 0: the caller's gate / up rows (and biases) of h column c are 2c / 2c + 1
@@ -869,7 +870,9 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
     // Columns past N read other experts' values or zeros; their results are dropped.
     float bias_a[2][4], bias_b[2][4];  // MODE 0: [pair][j] gate / up; MODE 1: [pair][j] columns 8 g + j / 8 g + 4 + j
     v4f bias_nxt[4];
-    const v4i srd_bias = make_srd(p.bias, EXT && p.bias ? 0xffffffffu : 0u);
+    // (range-checked: the lanes of an n-tile's columns past N index past their expert's values, for the
+    // last expert past the array: they read zeros)
+    const v4i srd_bias = make_srd(p.bias, EXT && p.bias ? p.bias_bytes : 0u);
     auto request_bias = [&]() __attribute__((always_inline)) {
         if constexpr (EXT) {
             const uint32_t gq = (uint32_t)(lane >> 4);
@@ -1591,6 +1594,9 @@ static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const voi
     if (activation == 1 && !(limit > 0.f)) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)bias13 | (uintptr_t)bias2) & 15u) return HK_ERR_BAD_ALIGNMENT;
     const bool ext = bias13 || bias2 || activation != 0 || w13_interleaved;
+    // the bias arrays are addressed with 32-bit byte offsets
+    if ((bias13 && (unsigned long long)E * 2 * I * 4 >= (1ull << 32)) || (bias2 && (unsigned long long)E * H * 4 >= (1ull << 32)))
+        return HK_ERR_BAD_SHAPE;
     if (!x_bf16 || !w13 || !w13_scales || !w2 || !w2_scales || !topk_w || !sorted_slots || !expert_offsets ||
         !slot_to_pos || !y_bf16)
         return HK_ERR_NULL_POINTER;
@@ -1639,7 +1645,7 @@ static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const voi
     p.items = (const MoeItem*)(ws + L.items1); p.num_items = nitems;
     p.out0 = ws + L.hq; p.out_scales = ws + L.hs;
     p.K = H; p.N = I; p.n_tiles_n = (I + 127) / 128;
-    p.bias = bias13; p.act = activation; p.alpha = alpha; p.limit = limit; p.interleaved = w13_interleaved != 0;
+    p.bias = bias13; p.bias_bytes = (uint32_t)((size_t)E * 2 * I * 4); p.act = activation; p.alpha = alpha; p.limit = limit; p.interleaved = w13_interleaved != 0;
     if (a8)
         st = ext ? launch_moe_stream<0, true, true>(p, L.max_items1, s, nt)
                  : gather ? launch_moe_stream<0, false, true, true>(p, L.max_items1, s, nt)
@@ -1663,7 +1669,7 @@ static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const voi
     q.items = (const MoeItem*)(ws + L.items2); q.num_items = nitems + 1;
     q.out0 = ws + L.o; q.out_scales = nullptr;
     q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
-    q.bias = bias2;
+    q.bias = bias2; q.bias_bytes = (uint32_t)((size_t)E * H * 4);
     if (a8)
         st = bias2 ? launch_moe_stream<1, true, true>(q, L.max_items2, s, nt) : launch_moe_stream<1, false, true>(q, L.max_items2, s, nt);
     else if (bias2)
