@@ -236,7 +236,11 @@ int hk_moe_mxfp4_preshuffle(const void* w, const void* scales, int scale_pitch, 
  * hk_moe_sort): activation quantization, grouped gate+up GEMM with SiLU-mul and MX
  * re-quantization, grouped down GEMM, weighted un-permute. weight_layout 0: w13 / w2 and their
  * scales in the plain row-major layout above; 1: outputs of hk_moe_mxfp4_preshuffle (the scale
- * pitch arguments are then ignored). Both layouts give bit-identical results. */
+ * pitch arguments are then ignored). Both layouts give bit-identical results. sorted_slots,
+ * expert_offsets and slot_to_pos must be one consistent result of hk_moe_sort: the kernels index
+ * activations and outputs with them (through range-checked descriptors where they fetch rows by
+ * token, so slots outside [0, T*k) read zeros or neighbouring workspace, never outside it; the
+ * un-permute reads o at slot_to_pos unchecked). */
 int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const void* w13_scales,
                          int w13_scale_pitch, const void* w2, const void* w2_scales,
                          int w2_scale_pitch, const float* topk_w, const int32_t* sorted_slots,
