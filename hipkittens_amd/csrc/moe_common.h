@@ -35,10 +35,11 @@ __device__ __forceinline__ float silu_mul(float g, float u) {
 
 inline int moe_round_up(int x, int m) { return (x + m - 1) / m * m; }
 // Bytes a layer's workspace carries behind its last region. The grouped GEMMs fetch the activation
-// rows and row scales of a work item in whole pieces (8 or 16 rows, up to 192 rows of scales): the
-// last item's fetches run up to 3840 bytes past the end of their region into the regions behind it
-// (the values are never used), and for a layer of a few tokens those regions are shorter than that.
-constexpr size_t kMoeWsTail = 4096;
+// rows and row scales of a work item in whole pieces (the streaming kernels 8 or 16 rows at a time,
+// the LDS-staged MXFP4 kernel its whole tile of 128 rows of 128 bytes): the last item's fetches run
+// past the end of their region into the regions behind it (the values are never used), and for a
+// layer of a few tokens those regions are shorter than that.
+constexpr size_t kMoeWsTail = 32768;
 // Number of CUs of the current device (cached per device ordinal).
 int moe_num_compute_units();
 // Item lists of the two grouped GEMMs of a layer from expert_offsets [E+1], m-tiles of up to `bm`
