@@ -141,6 +141,9 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
     // (a visible load would make it drain the whole load pipeline with vmcnt(0) before the
     // first use); the K loop's own waits cover them: they are queued behind the loads of the
     // item's first two K-steps and complete before the second wait returns.
+    // (s_nop 4: when the kernel spills scalar registers, the compiler restores the base address with
+    // v_readlane_b32 directly in front of the statement, and a vector-memory instruction that reads a
+    // scalar register within five wait states of a vector-ALU write may see its old value.)
     struct SlotIds { uint32_t a[NA]; uint32_t s; };
     auto issue_ids = [&](int idx, SlotIds& o) __attribute__((always_inline)) {
         if (idx >= it_end) idx = it_end - 1;
@@ -148,10 +151,10 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
 #pragma unroll
         for (int i = 0; i < NA; ++i) {
             const uint32_t off = (uint32_t)min(row_start + piece_row(i), p.S - 1) * 4u;
-            asm volatile("global_load_dword %0, %1, %2" : "=v"(o.a[i]) : "v"(off), "s"(p.sorted_slots) : "memory");
+            asm volatile("s_nop 4\n\tglobal_load_dword %0, %1, %2" : "=v"(o.a[i]) : "v"(off), "s"(p.sorted_slots) : "memory");
         }
         const uint32_t off = (uint32_t)min(row_start + w * SR + min(lane, SR - 1), p.S - 1) * 4u;
-        asm volatile("global_load_dword %0, %1, %2" : "=v"(o.s) : "v"(off), "s"(p.sorted_slots) : "memory");
+        asm volatile("s_nop 4\n\tglobal_load_dword %0, %1, %2" : "=v"(o.s) : "v"(off), "s"(p.sorted_slots) : "memory");
     };
     auto landed_ids = [&](SlotIds& o) __attribute__((always_inline)) {
 #pragma unroll
@@ -486,6 +489,9 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
     cf = cc;
 
     // ---- GATHER: slot ids of the rows this lane fetches, one item ahead of the fetch cursor --------
+    // (s_nop 4: when the kernel spills scalar registers, the compiler restores the base address with
+    // v_readlane_b32 directly in front of the statement, and a vector-memory instruction that reads a
+    // scalar register within five wait states of a vector-ALU write may see its old value.)
     struct SlotIds { uint32_t a[NA]; uint32_t s; };
     auto issue_ids = [&](int idx, SlotIds& o) __attribute__((always_inline)) {
         if (idx >= it_end) idx = it_end - 1;
@@ -493,10 +499,10 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
 #pragma unroll
         for (int i = 0; i < NA; ++i) {
             const uint32_t off = (uint32_t)min(row_start + piece_row(i), p.S - 1) * 4u;
-            asm volatile("global_load_dword %0, %1, %2" : "=v"(o.a[i]) : "v"(off), "s"(p.sorted_slots) : "memory");
+            asm volatile("s_nop 4\n\tglobal_load_dword %0, %1, %2" : "=v"(o.a[i]) : "v"(off), "s"(p.sorted_slots) : "memory");
         }
         const uint32_t off = (uint32_t)min(row_start + max(scale_row, 0), p.S - 1) * 4u;
-        asm volatile("global_load_dword %0, %1, %2" : "=v"(o.s) : "v"(off), "s"(p.sorted_slots) : "memory");
+        asm volatile("s_nop 4\n\tglobal_load_dword %0, %1, %2" : "=v"(o.s) : "v"(off), "s"(p.sorted_slots) : "memory");
     };
     auto landed_ids = [&](SlotIds& o) __attribute__((always_inline)) {
 #pragma unroll

@@ -1,0 +1,61 @@
+"""The kernels' device code holds no place where an instruction inside (or next to) an inline-assembly
+statement reads a register sooner than the hardware allows after the instruction that wrote it.
+
+The compiler does not apply its hazard rules to inline assembly; hipkittens_amd/isa_check.py states the
+two rules checked (vector-ALU write of a scalar register -> vector-memory read: five wait states;
+scalar write of M0 -> global->LDS load: one). Compiles every csrc/*.hip to assembly: about two minutes
+on eight cores, no GPU needed.
+"""
+import shutil
+
+import pytest
+
+from hipkittens_amd import isa_check
+
+
+def test_scanner_reports_the_two_hazards_and_accepts_enough_wait_states():
+    bad = """
+_Z3fooPi:
+	v_readlane_b32 s4, v254, 3
+	s_mov_b32 s5, s9
+	;;#ASMSTART
+	buffer_load_dwordx4 v[0:3], v9, s[4:7], s12 offen offset:16
+	;;#ASMEND
+	s_mov_b32 m0, s20
+	buffer_load_dwordx4 v9, s[4:7], s12 offen lds
+	v_readfirstlane_b32 s12, v1
+	s_nop 3
+	buffer_store_dword v0, v9, s[4:7], s12 offen
+"""
+    found = isa_check.scan(bad)
+    assert [(f.register, f.wait_states, f.needed) for f in found] == [
+        ("s4", 1, 5), ("s4", 3, 5), ("m0", 0, 1), ("s12", 4, 5)]
+    good = """
+_Z3fooPi:
+	v_readlane_b32 s4, v254, 3
+	s_nop 4
+	buffer_load_dwordx4 v[0:3], v9, s[4:7], s12 offen
+	v_readlane_b32 s12, v254, 4
+	s_mov_b32 s12, s13
+	s_mov_b32 m0, s20
+	s_nop 0
+	buffer_load_dwordx4 v9, s[4:7], s12 offen lds
+"""
+    assert isa_check.scan(good) == []
+    # along a taken branch only: the fall-through path has the nops, the branch skips them
+    branch = """
+_Z3barPi:
+	v_readfirstlane_b32 s8, v3
+	s_cbranch_scc1 .LBB0_2
+	s_nop 4
+.LBB0_2:
+	global_load_dword v1, v2, s[8:9]
+	s_endpgm
+"""
+    assert [(f.register, f.wait_states) for f in isa_check.scan(branch)] == [("s8", 1)]
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_no_unseen_wait_state_violation_in_any_kernel():
+    findings = isa_check.check_sources()
+    assert not findings, "\n".join(str(f) for f in findings)
