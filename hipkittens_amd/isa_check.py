@@ -1,21 +1,28 @@
 """Wait states between instructions that the compiler does not provide around inline assembly.
 
-The kernels issue their vector-memory instructions from inline assembly. The compiler treats such a
-statement as opaque: it places what the statement needs in front of it (a scalar register restored
-from a spill slot with v_readlane_b32, a uniform value made scalar with v_readfirstlane_b32) and does
-not apply its own hazard rules to what is inside. gfx950 has no interlock for two cases that matter
-here:
+The kernels issue their vector-memory and matrix instructions from inline assembly. The compiler
+treats such a statement as opaque: it places what the statement needs in front of it (a scalar
+register restored from a spill slot with v_readlane_b32, a uniform value made scalar with
+v_readfirstlane_b32), schedules its own instructions around it, and does not apply its hazard rules to
+what is inside. gfx950 has no interlock for three cases that matter here:
 
 * a scalar register written by a vector-ALU instruction and read by a vector-memory instruction
   (descriptor, scalar offset or base address) needs five wait states in between; with fewer the
   memory instruction may see the register's previous value: a load from a wild address;
-* M0 written by a scalar instruction and read by a global->LDS load needs one wait state.
+* M0 written by a scalar instruction and read by a global->LDS load needs one wait state;
+* the result registers of a matrix instruction of N passes (one pass = four clocks = one wait state)
+  must not be read or written by any other kind of instruction, nor read as the A / B / scale operand
+  of a matrix instruction, for N + 4 wait states after it issues (the distance the compiler keeps
+  behind a matrix instruction it knows: 12 for the 8-pass FP8 one). A matrix instruction that
+  follows another waits until the pipe has taken the one before it (N wait states after that one
+  issued); that wait counts.
 
 `python -m hipkittens_amd.isa_check` compiles every csrc/*.hip to device assembly with the build's
 flags and reports each place that some path through a kernel's code reaches with fewer wait states
 than that (a taken branch counts as one wait state, like any instruction). A kernel that spills
-scalar registers is the usual source: the restore lands directly in front of the statement that uses
-the register. The fix is an `s_nop` at the head of that statement, or fewer live scalar values.
+scalar registers is the usual source of the first: the restore lands directly in front of the
+statement that uses the register. The fix is an `s_nop` at the head of that statement, or fewer live
+scalar values.
 """
 from __future__ import annotations
 
@@ -24,13 +31,14 @@ import subprocess
 import sys
 import tempfile
 from concurrent.futures import ThreadPoolExecutor
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from pathlib import Path
 
 from . import build as _build
 
 VALU_SGPR_TO_VMEM = 5
 M0_TO_LDS_DMA = 1
+MFMA_RESULT_EXTRA = 4   # wait states beyond the instruction's passes (what the compiler leaves behind its own)
 
 _VMEM = ("buffer_", "global_", "flat_", "scratch_")
 # scalar-ALU / scalar-load instructions whose first operand is a destination
@@ -42,6 +50,7 @@ _SALU_WRITERS = (
 )
 # vector-ALU instructions whose second operand is a scalar carry / flag destination in the 64-bit encoding
 _VALU_SECOND_DST = re.compile(r"v_(add|sub|subrev|addc|subb|subbrev)_co_|v_mad_[ui]64_[ui]32|v_div_scale")
+_HORIZON = 32   # wait states after which a scalar write is forgotten (longer than any rule)
 
 
 @dataclass
@@ -54,7 +63,7 @@ class Finding:
     needed: int
 
     def __str__(self) -> str:
-        return (f"{self.function}: line {self.line}: {self.instruction} reads {self.register} "
+        return (f"{self.function}: line {self.line}: {self.instruction} touches {self.register} "
                 f"{self.wait_states} wait states after it was written (needs {self.needed})")
 
 
@@ -67,7 +76,23 @@ def _sgprs(token: str) -> list[int]:
     return [int(m.group(1))] if m else []
 
 
-_HORIZON = 32   # wait states after which a write is forgotten (longer than any rule)
+def _vector_registers(token: str) -> list[str]:
+    """Vector and accumulation registers named by an operand: 'v[4:5]' -> ['v4', 'v5']."""
+    token = token.strip()
+    m = re.fullmatch(r"([va])\[(\d+):(\d+)\]", token)
+    if m:
+        return [f"{m.group(1)}{i}" for i in range(int(m.group(2)), int(m.group(3)) + 1)]
+    return [token] if re.fullmatch(r"[va]\d+", token) else []
+
+
+def mfma_passes(op: str, args: str) -> int:
+    """Passes of a matrix instruction (16 for one this table does not know: the longest there is)."""
+    if "16x16x128_f8f6f4" in op:   # 8 passes with an fp8 operand, 4 when both are fp6 / fp4
+        fmt = [int(m.group(1)) if m else 0 for m in (re.search(r"cbsz:(\d)", args), re.search(r"blgp:(\d)", args))]
+        return 4 if min(fmt) >= 2 else 8
+    if "16x16x32_bf16" in op or "16x16x32_f16" in op:
+        return 4
+    return 16
 
 
 def _instruction(line: str):
@@ -77,39 +102,89 @@ def _instruction(line: str):
     return op, args, operands
 
 
-def _step(state: dict, instr, function: str, findings: list | None) -> None:
-    """Advances `state` (scalar register -> wait states since a vector-ALU instruction wrote it; "m0" ->
-    wait states since a scalar instruction wrote M0) over one instruction; reports into `findings`."""
+@dataclass
+class _State:
+    since: dict = field(default_factory=dict)    # scalar register (or "m0") -> wait states since the write in question
+    pending: dict = field(default_factory=dict)  # vector register -> (wait states still needed, out of)
+    pipe: int = 0                                # wait states until the matrix pipe takes another instruction
+
+    def copy(self) -> "_State":
+        return _State(dict(self.since), dict(self.pending), self.pipe)
+
+    def advance(self, states: int) -> None:
+        for key in list(self.since):
+            self.since[key] += states
+            if self.since[key] >= _HORIZON:
+                del self.since[key]
+        for key in list(self.pending):
+            left, total = self.pending[key]
+            if left <= states:
+                del self.pending[key]
+            else:
+                self.pending[key] = (left - states, total)
+        self.pipe = max(0, self.pipe - states)
+
+    def merge(self, other: "_State") -> "_State":
+        """The least favourable of two states (two ways to reach the same place)."""
+        out = self.copy()
+        for key, value in other.since.items():
+            out.since[key] = min(out.since.get(key, _HORIZON), value)
+        for key, value in other.pending.items():
+            out.pending[key] = max(out.pending.get(key, (0, 0)), value)
+        out.pipe = min(out.pipe, other.pipe)
+        return out
+
+    def __eq__(self, other) -> bool:
+        return (self.since, self.pending, self.pipe) == (other.since, other.pending, other.pipe)
+
+
+def _step(state: _State, instr, function: str, findings: list | None) -> None:
+    """Advances `state` over one instruction; reports into `findings`."""
     number, op, args, operands = instr
+
+    def touches(operand_list):
+        for operand in operand_list:
+            for word in operand.split():
+                for reg in _vector_registers(word):
+                    if reg in state.pending and findings is not None:
+                        left, total = state.pending[reg]
+                        findings.append(Finding(function, number, op, reg, total - left, total))
+
+    if op.startswith("v_mfma"):
+        touches(operands[1:3] + operands[4:6])   # A, B and scale operands (C chains on its own result)
+        state.advance(state.pipe)                # waits for the pipe
+        state.advance(1)
+        passes = mfma_passes(op, args)
+        state.pipe = passes - 1
+        for reg in _vector_registers(operands[0]):
+            state.pending[reg] = (passes + MFMA_RESULT_EXTRA, passes + MFMA_RESULT_EXTRA)
+        return
+    touches(operands)
     if op.startswith(_VMEM):
         for operand in operands:
             for word in operand.split():
                 for reg in _sgprs(word):
-                    if state.get(reg, _HORIZON) < VALU_SGPR_TO_VMEM and findings is not None:
-                        findings.append(Finding(function, number, op, f"s{reg}", state[reg], VALU_SGPR_TO_VMEM))
-        if re.search(r"\blds\b", args) and state.get("m0", _HORIZON) < M0_TO_LDS_DMA and findings is not None:
-            findings.append(Finding(function, number, op, "m0", state["m0"], M0_TO_LDS_DMA))
-    states = int(args.strip(), 0) + 1 if op == "s_nop" else 1
-    for key in list(state):
-        state[key] += states
-        if state[key] >= _HORIZON:
-            del state[key]
+                    if state.since.get(reg, _HORIZON) < VALU_SGPR_TO_VMEM and findings is not None:
+                        findings.append(Finding(function, number, op, f"s{reg}", state.since[reg], VALU_SGPR_TO_VMEM))
+        if re.search(r"\blds\b", args) and state.since.get("m0", _HORIZON) < M0_TO_LDS_DMA and findings is not None:
+            findings.append(Finding(function, number, op, "m0", state.since["m0"], M0_TO_LDS_DMA))
+    state.advance(int(args.strip(), 0) + 1 if op == "s_nop" else 1)
     if op.startswith("v_") and operands:
         written = _sgprs(operands[0])
         if len(operands) > 1 and _VALU_SECOND_DST.match(op):
             written += _sgprs(operands[1])
         for reg in written:
-            state[reg] = 0
+            state.since[reg] = 0
     elif op.startswith(_SALU_WRITERS) and operands:
         if operands[0] == "m0":
-            state["m0"] = 0
+            state.since["m0"] = 0
         for reg in _sgprs(operands[0]):
-            state.pop(reg, None)   # now a scalar-ALU result: no hazard towards vector memory
+            state.since.pop(reg, None)   # now a scalar-ALU result: no hazard towards vector memory
 
 
 def _scan_function(function: str, blocks: list) -> list[Finding]:
     """blocks: [label or None, [instructions]] in layout order. The state at the head of a block is the
-    minimum over the ends of its predecessors (fall-through and branches that name its label)."""
+    least favourable over the ends of its predecessors (fall-through and branches that name its label)."""
     index = {b[0]: i for i, b in enumerate(blocks) if b[0] is not None}
     successors = []
     for i, (_, instrs) in enumerate(blocks):
@@ -126,29 +201,24 @@ def _scan_function(function: str, blocks: list) -> list[Finding]:
         if falls and i + 1 < len(blocks):
             succ.append(i + 1)
         successors.append(succ)
-    heads: list[dict | None] = [None] * len(blocks)
-    heads[0] = {}
+    heads: list[_State | None] = [None] * len(blocks)
+    heads[0] = _State()
     work = [0]
     while work:
         i = work.pop()
-        state = dict(heads[i])
+        state = heads[i].copy()
         for instr in blocks[i][1]:
             _step(state, instr, function, None)
         for j in successors[i]:
-            merged = dict(heads[j]) if heads[j] is not None else None
-            if merged is None:
-                merged = dict(state)
-            else:
-                for key, value in state.items():
-                    merged[key] = min(merged.get(key, _HORIZON), value)
-            if merged != heads[j]:
+            merged = state.copy() if heads[j] is None else heads[j].merge(state)
+            if heads[j] is None or merged != heads[j]:
                 heads[j] = merged
                 work.append(j)
     findings: list[Finding] = []
     for i, (_, instrs) in enumerate(blocks):
         if heads[i] is None:
             continue   # not reachable
-        state = dict(heads[i])
+        state = heads[i].copy()
         for instr in instrs:
             _step(state, instr, function, findings)
     return findings
@@ -158,9 +228,11 @@ def scan(asm_text: str) -> list[Finding]:
     """Findings in the text of one `hipcc -S` device assembly file."""
     findings: list[Finding] = []
     function, blocks = None, []
+
     def flush():
         if function is not None and blocks:
             findings.extend(_scan_function(function, blocks))
+
     for number, raw in enumerate(asm_text.split("\n"), 1):
         line = raw.split(";")[0].strip()
         if not line:

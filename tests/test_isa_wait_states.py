@@ -2,8 +2,8 @@
 statement reads a register sooner than the hardware allows after the instruction that wrote it.
 
 The compiler does not apply its hazard rules to inline assembly; hipkittens_amd/isa_check.py states the
-two rules checked (vector-ALU write of a scalar register -> vector-memory read: five wait states;
-scalar write of M0 -> global->LDS load: one). Compiles every csrc/*.hip to assembly: about two minutes
+rules checked (vector-ALU write of a scalar register -> vector-memory read: five wait states; scalar
+write of M0 -> global->LDS load: one; result of a matrix instruction -> any other use: its passes + 4). Compiles every csrc/*.hip to assembly: about two minutes
 on eight cores, no GPU needed.
 """
 import shutil
@@ -53,6 +53,34 @@ _Z3barPi:
 	s_endpgm
 """
     assert [(f.register, f.wait_states) for f in isa_check.scan(branch)] == [("s8", 1)]
+
+
+def test_scanner_matrix_results():
+    # 8-pass FP8 instruction: its result may be touched 12 wait states after it issues; a second matrix
+    # instruction waits 8 for the pipe, which counts towards the first one's 12
+    text = """
+_Z3bazPi:
+	v_mfma_f32_16x16x128_f8f6f4 a[0:3], v[0:7], v[8:15], a[0:3]
+	v_mfma_f32_16x16x128_f8f6f4 a[4:7], v[0:7], v[8:15], a[4:7]
+	v_accvgpr_read_b32 v20, a0
+	s_nop 2
+	v_accvgpr_read_b32 v20, a1
+	s_nop 5
+	v_accvgpr_read_b32 v21, a4
+	s_nop 1
+	v_mov_b32_e32 v22, 0
+	v_accvgpr_write_b32 a5, v22
+	v_mfma_scale_f32_16x16x128_f8f6f4 a[8:11], v[0:3], v[8:11], a[8:11], v30, v31 op_sel_hi:[0,0,0] cbsz:4 blgp:4
+	s_nop 6
+	v_accvgpr_read_b32 v23, a8
+	v_accvgpr_read_b32 v23, a9
+	s_endpgm
+"""
+    found = [(f.line, f.register, f.wait_states, f.needed) for f in isa_check.scan(text)]
+    assert found == [(5, "a0", 8, 12), (9, "a4", 11, 12), (15, "a8", 7, 8)]
+    assert isa_check.mfma_passes("v_mfma_f32_16x16x32_bf16", "") == 4
+    assert isa_check.mfma_passes("v_mfma_scale_f32_16x16x128_f8f6f4", "cbsz:4") == 8   # fp4 x fp8
+    assert isa_check.mfma_passes("v_mfma_f32_32x32x64_f8f6f4", "") == 16
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
