@@ -19,6 +19,47 @@ def test_sigmoid_f32_close_to_libm_and_monotone():
     assert O.sigmoid_f32(np.array([0.0], np.float32))[0] == 0.5
 
 
+def test_exp_neg_f32_against_libm_and_its_fixed_points():
+    x = np.linspace(-87, 0, 30001).astype(np.float32)
+    e = O.exp_neg_f32(x)
+    ref = np.exp(x.astype(np.float64))
+    assert e.dtype == np.float32
+    assert np.max(np.abs(e - ref) / ref) < 3e-7          # a few fp32 ulps over the whole range
+    assert np.all(np.diff(e) >= 0)
+    assert O.exp_neg_f32(np.array([0.0], np.float32))[0] == 1.0
+    # powers of two come out exactly when x is the fp32 nearest to n ln 2 only up to the polynomial's error
+    n = np.arange(-60, 0)
+    xe = (n * np.log(2.0)).astype(np.float32)
+    assert np.max(np.abs(O.exp_neg_f32(xe) - np.exp(xe.astype(np.float64))) / np.exp(xe.astype(np.float64))) < 3e-7
+    # below the clamp the value of the clamp is returned (no underflow to a denormal, no zero)
+    lo = O.exp_neg_f32(np.array([-87.0, -100.0, -1e30], np.float32))
+    assert lo[0] == lo[1] == lo[2] and 0 < lo[0] < 2e-38 * 10
+
+
+def test_quantize_act_is_the_format_quantizer_plus_its_dequantization():
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((7, 96)) * 3).astype(np.float32)
+    q4, s4, d4 = O.quantize_act(x, "mxfp4")
+    rq, rs = F.quantize_mxfp4(x)
+    assert np.array_equal(q4, rq) and np.array_equal(s4, rs) and np.array_equal(d4, F.dequantize_mxfp4(rq, rs))
+    aq, as_ = O.quantize_act_mxfp4(x)
+    assert np.array_equal(aq, rq) and np.array_equal(as_, rs)
+    q8, s8, d8 = O.quantize_act(x, "mxfp8")
+    rq, rs = F.quantize_mxfp8(x)
+    assert np.array_equal(q8, rq) and np.array_equal(s8, rs) and np.array_equal(d8, F.dequantize_mxfp8(rq, rs))
+    # an e4m3 element is within 2^-4 of its input unless it is the block's largest: the block scale maps
+    # that one into [256, 512) and 448 is the largest code, so it may lose up to 1 - 448/512
+    assert np.max(np.abs(d8 - x) / np.maximum(np.abs(x), 1e-3)) <= 0.125
+    assert np.mean(np.abs(d8 - x) / np.maximum(np.abs(x), 1e-3) <= 0.0625) > 0.9
+    # e2m1: the largest maps into [4, 8) with 6 the largest code (up to a quarter lost)
+    assert np.max(np.abs(d4 - x) / np.max(np.abs(x))) <= 0.25
+    try:
+        O.quantize_act(x, "int8")
+        raise AssertionError("unknown format accepted")
+    except ValueError:
+        pass
+
+
 def test_topk_softmax_brute_force():
     rng = np.random.default_rng(0)
     logits = rng.standard_normal((37, 16)).astype(np.float32)
