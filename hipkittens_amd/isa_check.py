@@ -4,7 +4,7 @@ The kernels issue their vector-memory and matrix instructions from inline assemb
 treats such a statement as opaque: it places what the statement needs in front of it (a scalar
 register restored from a spill slot with v_readlane_b32, a uniform value made scalar with
 v_readfirstlane_b32), schedules its own instructions around it, and does not apply its hazard rules to
-what is inside. gfx950 has no interlock for three cases that matter here:
+what is inside. gfx950 has no interlock for four cases that matter here:
 
 * a scalar register written by a vector-ALU instruction and read by a vector-memory instruction
   (descriptor, scalar offset or base address) needs five wait states in between; with fewer the
@@ -15,7 +15,9 @@ what is inside. gfx950 has no interlock for three cases that matter here:
   of a matrix instruction, for N + 4 wait states after it issues (the distance the compiler keeps
   behind a matrix instruction it knows: 12 for the 8-pass FP8 one). A matrix instruction that
   follows another waits until the pipe has taken the one before it (N wait states after that one
-  issued); that wait counts.
+  issued); that wait counts;
+* the data registers of a vector-memory store of more than 64 bits must not be written by a vector-ALU
+  instruction for two wait states after the store.
 
 `python -m hipkittens_amd.isa_check` compiles every csrc/*.hip to device assembly with the build's
 flags and reports each place that some path through a kernel's code reaches with fewer wait states
@@ -38,6 +40,7 @@ from . import build as _build
 
 VALU_SGPR_TO_VMEM = 5
 M0_TO_LDS_DMA = 1
+WIDE_STORE_TO_VALU_WRITE = 2
 MFMA_RESULT_EXTRA = 4   # wait states beyond the instruction's passes (what the compiler leaves behind its own)
 
 _VMEM = ("buffer_", "global_", "flat_", "scratch_")
@@ -50,6 +53,7 @@ _SALU_WRITERS = (
 )
 # vector-ALU instructions whose second operand is a scalar carry / flag destination in the 64-bit encoding
 _VALU_SECOND_DST = re.compile(r"v_(add|sub|subrev|addc|subb|subbrev)_co_|v_mad_[ui]64_[ui]32|v_div_scale")
+_WIDE_STORE = re.compile(r"(buffer|global|flat|scratch)_store_(dwordx[34]|format_xyzw?|format_d16_xyzw)")
 _HORIZON = 32   # wait states after which a scalar write is forgotten (longer than any rule)
 
 
@@ -107,9 +111,10 @@ class _State:
     since: dict = field(default_factory=dict)    # scalar register (or "m0") -> wait states since the write in question
     pending: dict = field(default_factory=dict)  # vector register -> (wait states still needed, out of)
     pipe: int = 0                                # wait states until the matrix pipe takes another instruction
+    stored: dict = field(default_factory=dict)   # data register of a wide store -> wait states since the store
 
     def copy(self) -> "_State":
-        return _State(dict(self.since), dict(self.pending), self.pipe)
+        return _State(dict(self.since), dict(self.pending), self.pipe, dict(self.stored))
 
     def advance(self, states: int) -> None:
         for key in list(self.since):
@@ -123,6 +128,10 @@ class _State:
             else:
                 self.pending[key] = (left - states, total)
         self.pipe = max(0, self.pipe - states)
+        for key in list(self.stored):
+            self.stored[key] += states
+            if self.stored[key] >= WIDE_STORE_TO_VALU_WRITE:
+                del self.stored[key]
 
     def merge(self, other: "_State") -> "_State":
         """The least favourable of two states (two ways to reach the same place)."""
@@ -132,10 +141,12 @@ class _State:
         for key, value in other.pending.items():
             out.pending[key] = max(out.pending.get(key, (0, 0)), value)
         out.pipe = min(out.pipe, other.pipe)
+        for key, value in other.stored.items():
+            out.stored[key] = min(out.stored.get(key, _HORIZON), value)
         return out
 
     def __eq__(self, other) -> bool:
-        return (self.since, self.pending, self.pipe) == (other.since, other.pending, other.pipe)
+        return (self.since, self.pending, self.pipe, self.stored) == (other.since, other.pending, other.pipe, other.stored)
 
 
 def _step(state: _State, instr, function: str, findings: list | None) -> None:
@@ -168,7 +179,15 @@ def _step(state: _State, instr, function: str, findings: list | None) -> None:
                         findings.append(Finding(function, number, op, f"s{reg}", state.since[reg], VALU_SGPR_TO_VMEM))
         if re.search(r"\blds\b", args) and state.since.get("m0", _HORIZON) < M0_TO_LDS_DMA and findings is not None:
             findings.append(Finding(function, number, op, "m0", state.since["m0"], M0_TO_LDS_DMA))
+    if op.startswith("v_") and operands and findings is not None:
+        for reg in _vector_registers(operands[0]):
+            if reg in state.stored:
+                findings.append(Finding(function, number, op, reg, state.stored[reg], WIDE_STORE_TO_VALU_WRITE))
     state.advance(int(args.strip(), 0) + 1 if op == "s_nop" else 1)
+    if _WIDE_STORE.match(op):
+        data = operands[1] if op.startswith(("global_", "flat_", "scratch_")) else operands[0]
+        for reg in _vector_registers(data):
+            state.stored[reg] = 0
     if op.startswith("v_") and operands:
         written = _sgprs(operands[0])
         if len(operands) > 1 and _VALU_SECOND_DST.match(op):

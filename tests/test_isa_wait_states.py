@@ -3,7 +3,8 @@ statement reads a register sooner than the hardware allows after the instruction
 
 The compiler does not apply its hazard rules to inline assembly; hipkittens_amd/isa_check.py states the
 rules checked (vector-ALU write of a scalar register -> vector-memory read: five wait states; scalar
-write of M0 -> global->LDS load: one; result of a matrix instruction -> any other use: its passes + 4). Compiles every csrc/*.hip to assembly: about two minutes
+write of M0 -> global->LDS load: one; result of a matrix instruction -> any other use: its passes + 4;
+data registers of a store of more than 64 bits -> vector-ALU write: two). Compiles every csrc/*.hip to assembly: about two minutes
 on eight cores, no GPU needed.
 """
 import shutil
@@ -81,6 +82,25 @@ _Z3bazPi:
     assert isa_check.mfma_passes("v_mfma_f32_16x16x32_bf16", "") == 4
     assert isa_check.mfma_passes("v_mfma_scale_f32_16x16x128_f8f6f4", "cbsz:4") == 8   # fp4 x fp8
     assert isa_check.mfma_passes("v_mfma_f32_32x32x64_f8f6f4", "") == 16
+
+
+def test_scanner_wide_store_data():
+    text = """
+_Z3quxPi:
+	buffer_store_dwordx4 v[4:7], v9, s[4:7], 0 offen
+	v_mov_b32_e32 v5, 0
+	global_store_dwordx4 v[10:11], v[12:15], off
+	s_nop 0
+	v_add_f32_e32 v15, v1, v2
+	buffer_store_dwordx4 v[4:7], v9, s[4:7], 0 offen
+	s_nop 1
+	v_mov_b32_e32 v5, 0
+	buffer_store_dwordx2 v[4:5], v9, s[4:7], 0 offen
+	v_mov_b32_e32 v5, 0
+	s_endpgm
+"""
+    found = [(f.line, f.register, f.wait_states, f.needed) for f in isa_check.scan(text)]
+    assert found == [(4, "v5", 0, 2), (7, "v15", 1, 2)]
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
