@@ -91,6 +91,9 @@ def test_c_entry_points_reject_bad_arguments_without_a_gpu():
     assert lib.hk_moe_mxfp4_experts_ex(*args, None, None, 1, 1.702, 0.0, 0, p, 1 << 30, None) == -2   # limit <= 0
     assert lib.hk_moe_mxfp4_experts_ex(*args, p + 4, None, 0, 0.0, 0.0, 0, p, 1 << 30, None) == -3    # bias alignment
     assert lib.hk_moe_mxfp4_experts_ex(*args, None, None, 0, 0.0, 0.0, 0, None, 0, None) == -4        # workspace
+    # a bias array of 4 GiB or more cannot be addressed by the kernels' 32-bit offsets (512 x 2 x 2^20 floats)
+    huge = (p, p, p, 8, p, p, 32768, p, p, p, p, p, 1, 32, 1 << 20, 512, 1, 0)
+    assert lib.hk_moe_mxfp4_experts_ex(*huge, p, None, 0, 0.0, 0.0, 0, p, 1 << 40, None) == -2
     # MXFP8-activation entry points (pre-shuffled weights only): same option and workspace checks
     a8 = (p, p, p, p, p, p, p, p, p, p, 16, 64, 32, 4, 2)
     assert lib.hk_moe_mxfp4_a8_experts(*a8, None, None, 7, 1.702, 7.0, 0, p, 1 << 30, None) == -6
