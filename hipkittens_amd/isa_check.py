@@ -286,8 +286,8 @@ def device_assembly(src: Path, out: Path) -> None:
 
 
 def check_sources(sources: list[Path] | None = None, jobs: int = 8) -> list[Finding]:
-    """Compiles the sources (default: every csrc/*.hip) to device assembly and scans them."""
-    sources = sources or sorted((_build.PKG_DIR / "csrc").glob("*.hip"))
+    """Compiles the sources (default: every .hip file under csrc/) to device assembly and scans them."""
+    sources = sources or sorted((_build.PKG_DIR / "csrc").rglob("*.hip"))
     with tempfile.TemporaryDirectory() as tmp:
         outs = [Path(tmp) / (s.stem + ".s") for s in sources]
         with ThreadPoolExecutor(max_workers=jobs) as pool:
