@@ -24,7 +24,9 @@ flags and reports each place that some path through a kernel's code reaches with
 than that (a taken branch counts as one wait state, like any instruction). A kernel that spills
 scalar registers is the usual source of the first: the restore lands directly in front of the
 statement that uses the register. The fix is an `s_nop` at the head of that statement, or fewer live
-scalar values.
+scalar values. It also reports any kernel that keeps registers in scratch memory (the compiler's
+spill traffic would sit uncounted among the loads that the kernels wait for by count), and
+`--resources` prints every kernel's register, spill, scratch and LDS figures.
 """
 from __future__ import annotations
 
@@ -277,6 +279,48 @@ def scan(asm_text: str) -> list[Finding]:
     return findings
 
 
+def kernel_resources(asm_text: str) -> dict[str, dict[str, int]]:
+    """Per kernel, from the metadata at the end of a `hipcc -S` file: register counts, spill counts,
+    bytes of scratch (private segment) and of static LDS."""
+    out: dict[str, dict[str, int]] = {}
+    entry: dict[str, int] = {}
+    name = None
+    keys = {".agpr_count": "agprs", ".vgpr_count": "vgprs", ".sgpr_count": "sgprs",
+            ".sgpr_spill_count": "sgpr_spills", ".vgpr_spill_count": "vgpr_spills",
+            ".private_segment_fixed_size": "scratch_bytes", ".group_segment_fixed_size": "lds_bytes"}
+
+    def flush():
+        if name is not None:
+            out[name] = entry
+
+    for raw in asm_text.split("\n"):
+        line = raw.strip()
+        if raw.startswith("  - ."):         # first key of the next kernel's record (argument records sit deeper)
+            flush()
+            entry, name = {}, None
+            line = line[2:]
+        m = re.match(r"(\.\w+):\s+(\S+)$", line)
+        if not m:
+            continue
+        if m.group(1) == ".name":
+            name = m.group(2)
+        elif m.group(1) in keys:
+            entry[keys[m.group(1)]] = int(m.group(2))
+    flush()
+    return out
+
+
+def memory_spills(asm_text: str) -> list[Finding]:
+    """Kernels that keep registers in scratch memory. The compiler's spill stores and reloads are
+    vector-memory operations of their own: they would sit, uncounted, between the loads whose
+    completion the kernels track with hand-counted `s_waitcnt vmcnt(N)`."""
+    findings = []
+    for name, res in kernel_resources(asm_text).items():
+        if res.get("scratch_bytes", 0) or res.get("vgpr_spills", 0):
+            findings.append(Finding(name, 0, "kernel", "scratch memory", res.get("scratch_bytes", 0), 0))
+    return findings
+
+
 def device_assembly(src: Path, out: Path) -> None:
     cmd = [_build._hipcc(), *_build.HIPCC_FLAGS, *_build.PER_FILE_FLAGS.get(src.name, []),
            "--cuda-device-only", "-S", str(src), "-o", str(out)]
@@ -294,11 +338,20 @@ def check_sources(sources: list[Path] | None = None, jobs: int = 8) -> list[Find
             list(pool.map(device_assembly, sources, outs))
         findings: list[Finding] = []
         for out in outs:
-            findings += scan(out.read_text())
+            text = out.read_text()
+            findings += scan(text) + memory_spills(text)
     return findings
 
 
 def main() -> int:
+    if "--resources" in sys.argv[1:]:   # a table of every kernel's registers, spills, scratch and LDS
+        with tempfile.TemporaryDirectory() as tmp:
+            for src in sorted((_build.PKG_DIR / "csrc").rglob("*.hip")):
+                out = Path(tmp) / (src.stem + ".s")
+                device_assembly(src, out)
+                for name, res in kernel_resources(out.read_text()).items():
+                    print(src.name, name, " ".join(f"{k}={v}" for k, v in res.items()))
+        return 0
     findings = check_sources()
     for f in findings:
         print(f)

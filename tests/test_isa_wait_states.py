@@ -103,6 +103,37 @@ _Z3quxPi:
     assert found == [(4, "v5", 0, 2), (7, "v15", 1, 2)]
 
 
+def test_kernel_resources_and_scratch_rule():
+    meta = """
+amdhsa.kernels:
+  - .agpr_count:     16
+    .args:
+      - .address_space:  global
+        .offset:         0
+        .size:           8
+    .group_segment_fixed_size: 1024
+    .name:           _Z1kPi
+    .private_segment_fixed_size: 0
+    .sgpr_count:     40
+    .sgpr_spill_count: 3
+    .vgpr_count:     48
+    .vgpr_spill_count: 0
+  - .agpr_count:     0
+    .args:           []
+    .group_segment_fixed_size: 0
+    .name:           _Z1sPi
+    .private_segment_fixed_size: 72
+    .sgpr_count:     20
+    .sgpr_spill_count: 0
+    .vgpr_count:     256
+    .vgpr_spill_count: 18
+"""
+    res = isa_check.kernel_resources(meta)
+    assert res["_Z1kPi"] == {"agprs": 16, "lds_bytes": 1024, "scratch_bytes": 0, "sgprs": 40, "sgpr_spills": 3,
+                             "vgprs": 48, "vgpr_spills": 0}
+    assert [f.function for f in isa_check.memory_spills(meta)] == ["_Z1sPi"]
+
+
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
 def test_no_unseen_wait_state_violation_in_any_kernel():
     findings = isa_check.check_sources()
