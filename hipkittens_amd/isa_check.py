@@ -4,7 +4,8 @@ The kernels issue their vector-memory and matrix instructions from inline assemb
 treats such a statement as opaque: it places what the statement needs in front of it (a scalar
 register restored from a spill slot with v_readlane_b32, a uniform value made scalar with
 v_readfirstlane_b32), schedules its own instructions around it, and does not apply its hazard rules to
-what is inside. gfx950 has no interlock for four cases that matter here:
+what is inside. gfx950 has no interlock for four cases that matter here, and a fifth check covers the
+scalar loads that the kernels issue from inline assembly and wait for later:
 
 * a scalar register written by a vector-ALU instruction and read by a vector-memory instruction
   (descriptor, scalar offset or base address) needs five wait states in between; with fewer the
@@ -17,7 +18,10 @@ what is inside. gfx950 has no interlock for four cases that matter here:
   follows another waits until the pipe has taken the one before it (N wait states after that one
   issued); that wait counts;
 * the data registers of a vector-memory store of more than 64 bits must not be written by a vector-ALU
-  instruction for two wait states after the store.
+  instruction for two wait states after the store;
+* the destination of a scalar load must not be touched before an `s_waitcnt lgkmcnt(0)` (scalar loads
+  return out of order): the compiler takes the destination of an inline-assembly statement for
+  written when the statement ends and is free to copy it to a spill slot at once.
 
 `python -m hipkittens_amd.isa_check` compiles every csrc/*.hip to device assembly with the build's
 flags and reports each place that some path through a kernel's code reaches with fewer wait states
@@ -114,9 +118,10 @@ class _State:
     pending: dict = field(default_factory=dict)  # vector register -> (wait states still needed, out of)
     pipe: int = 0                                # wait states until the matrix pipe takes another instruction
     stored: dict = field(default_factory=dict)   # data register of a wide store -> wait states since the store
+    loading: set = field(default_factory=set)    # scalar registers a scalar load may not have written yet
 
     def copy(self) -> "_State":
-        return _State(dict(self.since), dict(self.pending), self.pipe, dict(self.stored))
+        return _State(dict(self.since), dict(self.pending), self.pipe, dict(self.stored), set(self.loading))
 
     def advance(self, states: int) -> None:
         for key in list(self.since):
@@ -145,10 +150,12 @@ class _State:
         out.pipe = min(out.pipe, other.pipe)
         for key, value in other.stored.items():
             out.stored[key] = min(out.stored.get(key, _HORIZON), value)
+        out.loading |= other.loading
         return out
 
     def __eq__(self, other) -> bool:
-        return (self.since, self.pending, self.pipe, self.stored) == (other.since, other.pending, other.pipe, other.stored)
+        return ((self.since, self.pending, self.pipe, self.stored, self.loading) ==
+                (other.since, other.pending, other.pipe, other.stored, other.loading))
 
 
 def _step(state: _State, instr, function: str, findings: list | None) -> None:
@@ -163,6 +170,19 @@ def _step(state: _State, instr, function: str, findings: list | None) -> None:
                         left, total = state.pending[reg]
                         findings.append(Finding(function, number, op, reg, total - left, total))
 
+    if op == "s_waitcnt":
+        if re.search(r"lgkmcnt\(0\)", args):
+            state.loading.clear()
+    else:
+        scalar_load = op.startswith(("s_load_", "s_buffer_load_"))
+        if state.loading and findings is not None:
+            for operand in (operands[1:] if scalar_load else operands):
+                for word in operand.split():
+                    for reg in _sgprs(word):
+                        if reg in state.loading:
+                            findings.append(Finding(function, number, op, f"s{reg} (scalar load in flight)", 0, 0))
+        if scalar_load and operands:
+            state.loading.update(_sgprs(operands[0]))
     if op.startswith("v_mfma"):
         touches(operands[1:3] + operands[4:6])   # A, B and scale operands (C chains on its own result)
         state.advance(state.pipe)                # waits for the pipe

@@ -103,6 +103,22 @@ _Z3quxPi:
     assert found == [(4, "v5", 0, 2), (7, "v15", 1, 2)]
 
 
+def test_scanner_scalar_load_destinations():
+    text = """
+_Z3quuPi:
+	s_load_dword s20, s[4:5], s9
+	s_load_dwordx4 s[24:27], s[4:5], 0x10
+	s_waitcnt vmcnt(0) lgkmcnt(1)
+	v_writelane_b32 v254, s20, 3
+	s_add_u32 s4, s4, 8
+	s_waitcnt lgkmcnt(0)
+	v_writelane_b32 v254, s25, 4
+	s_endpgm
+"""
+    found = [(f.line, f.register) for f in isa_check.scan(text)]
+    assert found == [(6, "s20 (scalar load in flight)")]
+
+
 def test_kernel_resources_and_scratch_rule():
     meta = """
 amdhsa.kernels:
