@@ -182,7 +182,7 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
                                     void* stream) {
     using namespace hk;
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
-    if (M <= 0 || N <= 0 || K <= 0 || (K % 8) != 0) return HK_ERR_BAD_SHAPE;
+    if (M <= 0 || N <= 0 || K <= 0 || (K % 8) != 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
     if (variant < 0 || variant > 4) return HK_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
@@ -212,6 +212,7 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
 
 extern "C" int hk_bf16_gemm(const void* A, const void* B, void* C, int M, int N, int K, void* stream) {
     using namespace hk;
+    if (gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     const bool tile_ok = K > 0 && (long long)2 * K * BM < (1ll << 31);
     // the same choice of tile as hk_fp8_gemm (pick_tile), with this format's measured corrections
     const int tile = pick_tile(M, N, (int)((2ll * K + BK - 1) / BK), TileRule{32, 64, 96});
@@ -220,7 +221,7 @@ extern "C" int hk_bf16_gemm(const void* A, const void* B, void* C, int M, int N,
 }
 
 extern "C" size_t hk_bf16_gemm_workspace_bytes(int M, int N, int K) {
-    if (M <= 0 || N <= 0 || K <= 0 || K >= (1 << 30)) return 0;
+    if (M <= 0 || N <= 0 || K <= 0 || K >= (1 << 29) || hk::gemm_dims_too_large(M, N, K)) return 0;
     const int s = hk::splitk_ranges(M, N, 2 * K);
     return s < 2 ? 0 : (size_t)s * M * N * sizeof(float);
 }
@@ -228,8 +229,8 @@ extern "C" size_t hk_bf16_gemm_workspace_bytes(int M, int N, int K) {
 extern "C" int hk_bf16_gemm_ws(const void* A, const void* B, void* C, int M, int N, int K, void* workspace,
                                size_t workspace_bytes, void* stream) {
     using namespace hk;
-    if (M <= 0 || N <= 0 || K <= 0) return HK_ERR_BAD_SHAPE;
-    const int splits = K < (1 << 30) ? splitk_ranges(M, N, 2 * K) : 1;
+    if (M <= 0 || N <= 0 || K <= 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
+    const int splits = K < (1 << 29) ? splitk_ranges(M, N, 2 * K) : 1;
     const bool can_split = splits >= 2 && workspace && workspace_bytes >= (size_t)splits * M * N * sizeof(float) &&
                            (K % 8) == 0 && (long long)2 * K * BM < (1ll << 31) && (long long)M * N < (1ll << 40);
     if (!can_split) return hk_bf16_gemm(A, B, C, M, N, K, stream);

@@ -176,7 +176,7 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
                                    float scale_a, float scale_b, int variant, void* stream) {
     using namespace hk;
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
-    if (M <= 0 || N <= 0 || K <= 0 || (K % 16) != 0) return HK_ERR_BAD_SHAPE;
+    if (M <= 0 || N <= 0 || K <= 0 || (K % 16) != 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
     if (variant < 0 || variant > 6 || variant == 2 || variant == 3) return HK_ERR_UNSUPPORTED;
     // K tails: the tile kernels zero-fill the last K-step of any K % 16 == 0
@@ -207,7 +207,7 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
 }
 
 extern "C" size_t hk_fp8_gemm_workspace_bytes(int M, int N, int K) {
-    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (M <= 0 || N <= 0 || K <= 0 || hk::gemm_dims_too_large(M, N, K)) return 0;
     const int s = hk::splitk_ranges(M, N, K);
     return s < 2 ? 0 : (size_t)s * M * N * sizeof(float);
 }
@@ -215,7 +215,7 @@ extern "C" size_t hk_fp8_gemm_workspace_bytes(int M, int N, int K) {
 extern "C" int hk_fp8_gemm_ws(const void* A, const void* B, void* C, int M, int N, int K, float scale_a,
                               float scale_b, void* workspace, size_t workspace_bytes, void* stream) {
     using namespace hk;
-    if (M <= 0 || N <= 0 || K <= 0) return HK_ERR_BAD_SHAPE;
+    if (M <= 0 || N <= 0 || K <= 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     const int splits = splitk_ranges(M, N, K);
     const bool can_split = splits >= 2 && workspace && workspace_bytes >= (size_t)splits * M * N * sizeof(float) &&
                            (K % 16) == 0 && (long long)K * BM < (1ll << 31) && (long long)M * N < (1ll << 40);
@@ -259,7 +259,7 @@ extern "C" size_t hk_fp8_gemm_static_ws_max_bytes(void) { return hk::kStaticScra
 extern "C" int hk_fp8_gemm_static_ws(const void* A, const void* B, void* C, int M, int N, int K, float scale_a,
                                      float scale_b, void* stream) {
     using namespace hk;
-    if (M <= 0 || N <= 0 || K <= 0) return HK_ERR_BAD_SHAPE;
+    if (M <= 0 || N <= 0 || K <= 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     const int splits = splitk_ranges(M, N, K);
     if (splits < 2) return hk_fp8_gemm(A, B, C, M, N, K, scale_a, scale_b, stream);   // no scratch needed
     const size_t need = (size_t)splits * M * N * sizeof(float);
@@ -275,6 +275,7 @@ extern "C" int hk_fp8_gemm_static_ws(const void* A, const void* B, void* C, int 
 extern "C" int hk_fp8_gemm(const void* A, const void* B, void* C, int M, int N, int K,
                            float scale_a, float scale_b, void* stream) {
     using namespace hk;
+    if (gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     const bool tile_ok = K > 0 && (long long)K * BM < (1ll << 31);
     // 256x256 tiles (five-slot ring kernel), 128x128 or 64x64: see pick_tile
     const int tile = pick_tile(M, N, (K + BK - 1) / BK, TileRule{16, 32, 80});

@@ -263,8 +263,9 @@ int moe_num_compute_units();  // number of CUs of the current device, cached (mo
 // K: the operands' row length in bytes; min_nk: the shortest K (in K-steps) that is split.
 static inline int splitk_ranges(int M, int N, int K, int min_nk = 48) {
     // 64x64 tiles, two workgroups per CU
-    const long long tiles = (long long)((M + kTinyTile - 1) / kTinyTile) * ((N + kTinyTile - 1) / kTinyTile);
-    const int nk = (K + BK - 1) / BK;
+    // (64-bit: the size queries pass whatever the caller asks about)
+    const long long tiles = (((long long)M + kTinyTile - 1) / kTinyTile) * (((long long)N + kTinyTile - 1) / kTinyTile);
+    const long long nk = ((long long)K + BK - 1) / BK;
     const int cus = moe_num_compute_units();   // 256 when no device can be queried
     // shorter K: the 64x64-tile kernel without a second launch is as fast or faster
     if (tiles > cus || nk < min_nk) return 1;

@@ -26,4 +26,13 @@ inline bool set_lds_limit_once(const void* kern, int bytes, DeviceOnce& once) {
     return true;
 }
 
+// Whether a GEMM's dimensions are beyond what the launchers' 32-bit arithmetic covers: a dimension of 2^30
+// or more, or 2^31 and more tiles of 64 x 64 (tile counts and grid sizes are ints). Every public GEMM entry
+// point refuses such a shape before it computes anything from it.
+inline bool gemm_dims_too_large(int M, int N, int K) {
+    if (M >= (1 << 30) || N >= (1 << 30) || K >= (1 << 30)) return true;
+    if (M <= 0 || N <= 0) return false;
+    return (((long long)M + 63) / 64) * (((long long)N + 63) / 64) >= (1ll << 31);
+}
+
 }  // namespace hk

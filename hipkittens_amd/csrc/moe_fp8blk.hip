@@ -924,7 +924,7 @@ static int launch_fp8blk_stream(const MoeFp8Params& p, int max_items, hipStream_
 
 // n-tiles of 256 weight rows of the two GEMMs: gate+up (mode 0: 128 h columns = 128 gate + 128 up rows
 // per tile) and down (mode 1).
-static inline int fp8blk_n_tiles(int mode, int N) { return mode == 0 ? N / 128 : (N + 255) / 256; }
+static inline int fp8blk_n_tiles(int mode, int N) { return mode == 0 ? N / 128 : (int)(((long long)N + 255) / 256); }
 
 struct Fp8Ws {
     size_t ids, w, sorted, offsets, inv, sort_ws, items1, items2, nitems, xq, xs, hq, hs, o, total;
@@ -976,8 +976,9 @@ extern "C" int hk_fp8_quantize_rows_1x128(const void* x_bf16, int rows, int cols
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
+// (0 for a shape the entry points refuse)
 extern "C" size_t hk_moe_fp8blk_workspace_bytes(int T, int H, int I, int E, int k) {
-    if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || k <= 0) return 0;
+    if (fp8blk_check(T, H, I, E, k) != HK_OK) return 0;
     return fp8_ws_layout(T, H, I, E, k).total;
 }
 

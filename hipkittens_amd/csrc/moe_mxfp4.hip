@@ -1483,8 +1483,9 @@ extern "C" int hk_moe_unpermute(const void* o_bf16, const float* w, const int32_
 extern "C" int hk_moe_mxfp4_preshuffle_bytes(int E, int N, int K, int mode, size_t* w_bytes, size_t* s_bytes) {
     if (!w_bytes || !s_bytes) return HK_ERR_NULL_POINTER;
     if (E <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || mode < 0 || mode > 2) return HK_ERR_BAD_SHAPE;
-    const size_t n_tiles = mode != 1 ? (N + 127) / 128 : (N + 255) / 256;
-    const size_t nk = (K / 2 + 127) / 128;
+    const size_t n_tiles = mode != 1 ? ((size_t)N + 127) / 128 : ((size_t)N + 255) / 256;
+    const size_t nk = ((size_t)K / 2 + 127) / 128;
+    if ((double)E * (double)n_tiles * (double)nk * kMoeBTile >= 4e18) return HK_ERR_BAD_SHAPE;   // beyond size_t
     *w_bytes = (size_t)E * n_tiles * nk * kMoeBTile;
     *s_bytes = (size_t)E * n_tiles * nk * kMoeScaleB;
     return HK_OK;
@@ -1496,9 +1497,12 @@ extern "C" int hk_moe_mxfp4_preshuffle(const void* w, const void* scales, int sc
     if (E <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || scale_pitch < K / 32 || mode < 0 || mode > 2)
         return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)w | (uintptr_t)out_w) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    if (N > (1 << 30)) return HK_ERR_BAD_SHAPE;
     const int n_tiles = mode != 1 ? (N + 127) / 128 : (N + 255) / 256;
-    const long long total = (long long)E * n_tiles * ((K / 2 + 127) / 128) * 2048;
-    if ((total + 255) / 256 >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
+    // one thread per 16 bytes of the output; the grid holds 2^31 - 1 blocks of 256
+    const long long per_tile = (long long)((K / 2 + 127) / 128) * 2048, tiles = (long long)E * n_tiles;
+    if (tiles > ((1ll << 39) - 256) / per_tile) return HK_ERR_BAD_SHAPE;
+    const long long total = tiles * per_tile;
     hipLaunchKernelGGL(moe_preshuffle_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, (const uint8_t*)w, (const uint8_t*)scales, E, N, K, scale_pitch, mode,
                        n_tiles, (uint8_t*)out_w, (uint8_t*)out_s);
@@ -1532,24 +1536,32 @@ static MoeWs moe_ws_layout(int T, int H, int I, int E, int k, bool a8 = false) {
     return L;
 }
 
+static bool moe_mxfp4_shape_ok(int T, int H, int I, int E, int k);
+// (0 for a shape the entry points refuse)
 extern "C" size_t hk_moe_mxfp4_workspace_bytes(int T, int H, int I, int E, int k) {
-    if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || k <= 0) return 0;
+    if (!moe_mxfp4_shape_ok(T, H, I, E, k)) return 0;
     return moe_ws_layout(T, H, I, E, k).total;
 }
 extern "C" size_t hk_moe_mxfp4_a8_workspace_bytes(int T, int H, int I, int E, int k) {
-    if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || k <= 0) return 0;
+    if (!moe_mxfp4_shape_ok(T, H, I, E, k)) return 0;
+    if ((long long)T * k * (((long long)H + 255) / 256 * 256) >= (1ll << 31) ||
+        (long long)T * k * (((long long)I + 255) / 256 * 256) >= (1ll << 31))
+        return 0;   // MXFP8 rows are twice as long
     return moe_ws_layout(T, H, I, E, k, true).total;
 }
 
+// The shapes the layer's kernels address with 32-bit offsets.
+static bool moe_mxfp4_shape_ok(int T, int H, int I, int E, int k) {
+    if (T <= 0 || E <= 0 || k <= 0 || k > E || k > 64 || E > 512) return false;
+    if (H <= 0 || I <= 0 || (H % 32) != 0 || (I % 32) != 0) return false;
+    return (long long)T * k < (1ll << 24) && (long long)T * k * (((I / 2 + 127) / 128) * 128) < (1ll << 31) &&
+           (long long)T * k * (((H / 2 + 127) / 128) * 128) < (1ll << 31) && (long long)2 * I * (H / 2) < (1ll << 31) &&
+           (long long)H * (I / 2) < (1ll << 31);
+}
 static int moe_mxfp4_check(int T, int H, int I, int E, int k, int w13_scale_pitch, int w2_scale_pitch) {
-    if (T <= 0 || E <= 0 || k <= 0 || k > E || k > 64 || E > 512) return HK_ERR_BAD_SHAPE;
-    if (H <= 0 || I <= 0 || (H % 32) != 0 || (I % 32) != 0) return HK_ERR_BAD_SHAPE;
+    if (!moe_mxfp4_shape_ok(T, H, I, E, k)) return HK_ERR_BAD_SHAPE;
     if (w13_scale_pitch < H / 32 || (w13_scale_pitch % 8) != 0 || w2_scale_pitch < I / 32 ||
         (w2_scale_pitch % 8) != 0)
-        return HK_ERR_BAD_SHAPE;
-    if ((long long)T * k >= (1ll << 24) || (long long)T * k * (((I / 2 + 127) / 128) * 128) >= (1ll << 31) ||
-        (long long)T * k * (((H / 2 + 127) / 128) * 128) >= (1ll << 31) || (long long)2 * I * (H / 2) >= (1ll << 31) ||
-        (long long)H * (I / 2) >= (1ll << 31))
         return HK_ERR_BAD_SHAPE;
     return HK_OK;
 }

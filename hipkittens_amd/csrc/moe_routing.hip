@@ -461,7 +461,7 @@ extern "C" int hk_moe_topk_softmax(const float* logits, int T, int E, int k, int
                                    void* stream) {
     using namespace hk;
     if (!logits || !ids || !w) return HK_ERR_NULL_POINTER;
-    if (T <= 0 || E <= 0 || k <= 0 || k > E || k > 64 || E > 64 * kMaxPerLane) return HK_ERR_BAD_SHAPE;
+    if (T <= 0 || T > (1 << 30) || E <= 0 || k <= 0 || k > E || k > 64 || E > 64 * kMaxPerLane) return HK_ERR_BAD_SHAPE;
     if (E <= 128 && k <= 16)
         hipLaunchKernelGGL(moe_topk_softmax_kernel<16>, dim3((T + 15) / 16), dim3(256), 0, (hipStream_t)stream,
                            logits, T, E, k, ids, w);
@@ -476,7 +476,7 @@ extern "C" int hk_moe_topk_grouped_sigmoid(const float* logits, const float* bia
                                            int32_t* ids, float* w, void* stream) {
     using namespace hk;
     if (!logits || !ids || !w) return HK_ERR_NULL_POINTER;
-    if (T <= 0 || E <= 0 || k <= 0 || k > 64 || E > 64 * kMaxPerLane || n_group <= 0 || n_group > 64 ||
+    if (T <= 0 || T > (1 << 30) || E <= 0 || k <= 0 || k > 64 || E > 64 * kMaxPerLane || n_group <= 0 || n_group > 64 ||
         (E % n_group) != 0 || topk_group <= 0 || topk_group > n_group ||
         k > topk_group * (E / n_group))
         return HK_ERR_BAD_SHAPE;
@@ -516,7 +516,8 @@ extern "C" int hk_moe_sort(const int32_t* ids, int T, int k, int E, int32_t* sor
                            size_t workspace_bytes, void* stream) {
     using namespace hk;
     if (!ids || !sorted_slots || !expert_offsets) return HK_ERR_NULL_POINTER;
-    if (T <= 0 || k <= 0 || E <= 0 || E > kSortMaxE || (long long)T * k >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
+    // (2^30 slots: the kernels index slots and chunk ends with ints)
+    if (T <= 0 || k <= 0 || E <= 0 || E > kSortMaxE || (long long)T * k > (1ll << 30)) return HK_ERR_BAD_SHAPE;
     if (!workspace || workspace_bytes < hk_moe_sort_workspace_bytes(T, k, E)) return HK_ERR_WORKSPACE;
     const int S = T * k;
     const int nchunks = (S + kSortChunk - 1) / kSortChunk;

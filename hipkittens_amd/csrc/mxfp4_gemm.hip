@@ -434,7 +434,8 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
                            int sb_pitch, void* C, int M, int N, int K, int variant, void* stream) {
     using namespace hk;
     if (!A || !A_scales || !B || !B_scales || !C) return HK_ERR_NULL_POINTER;
-    if (M <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || sa_pitch < K / 32 || sb_pitch < K / 32)
+    if (M <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || sa_pitch < K / 32 || sb_pitch < K / 32 ||
+        gemm_dims_too_large(M, N, K))
         return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
     if (variant < -1 || variant > 4) return HK_ERR_UNSUPPORTED;
@@ -492,7 +493,7 @@ extern "C" int hk_mxfp4_gemm(const void* A, const void* A_scales, const void* B,
 }
 
 extern "C" size_t hk_mxfp4_gemm_workspace_bytes(int M, int N, int K) {
-    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (M <= 0 || N <= 0 || K <= 0 || hk::gemm_dims_too_large(M, N, K)) return 0;
     const int s = hk::mxfp4_splitk_ranges(M, N, K);
     return s < 2 ? 0 : (size_t)s * M * N * sizeof(float);
 }
@@ -501,7 +502,7 @@ extern "C" int hk_mxfp4_gemm_ws(const void* A, const void* A_scales, int a_scale
                                 const void* B_scales, int b_scale_pitch, void* C, int M, int N, int K,
                                 void* workspace, size_t workspace_bytes, void* stream) {
     using namespace hk;
-    if (M <= 0 || N <= 0 || K <= 0 || (K % 32) != 0) return HK_ERR_BAD_SHAPE;
+    if (M <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     const int splits = mxfp4_splitk_ranges(M, N, K);
     const int groups = (K / 32 + 7) / 8 * 8;
     // what the tile kernels need of the scale rows (see mxfp4_gemm_impl); anything else takes the plain path

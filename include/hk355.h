@@ -220,6 +220,8 @@ int hk_moe_unpermute(const void* o_bf16, const float* w, const int32_t* slot_to_
 int hk_moe_unpermute_add(const void* o_bf16, const float* w, const int32_t* slot_to_pos, int T, int k,
                          int H, const void* add_bf16_or_null, void* y_bf16, void* stream);
 
+/* Bytes of workspace a layer of this shape needs; 0 for a shape the entry points refuse with
+ * HK_ERR_BAD_SHAPE (the other hk_moe_*_workspace_bytes functions likewise). */
 size_t hk_moe_mxfp4_workspace_bytes(int T, int H, int I, int E, int k);
 
 /* Offline weight pre-shuffle (weight_layout = 1 below). For every expert, n-tile and K-step the

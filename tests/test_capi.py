@@ -85,6 +85,23 @@ def test_c_entry_points_reject_bad_arguments_without_a_gpu():
     assert lib.hk_mxfp4_gemm_workspace_bytes(16, 1024, 8192) % (16 * 1024 * 4) == 0
     assert lib.hk_mxfp4_gemm_workspace_bytes(16, 1024, 8192) > 0
     assert lib.hk_mxfp4_gemm_workspace_bytes(8192, 8192, 8192) == 0
+    # dimensions beyond the launchers' 32-bit arithmetic are refused before anything is computed from them
+    imax = 2**31 - 1
+    for M, N, K in ((imax, 64, 128), (64, imax, 128), (64, 64, imax - 15), (1 << 24, 1 << 24, 128)):
+        assert lib.hk_fp8_gemm(p, p, p, M, N, K & ~15, 1.0, 1.0, None) == -2
+        assert lib.hk_fp8_gemm_ws(p, p, p, M, N, K & ~15, 1.0, 1.0, p, 1 << 40, None) == -2
+        assert lib.hk_fp8_gemm_static_ws(p, p, p, M, N, K & ~15, 1.0, 1.0, None) == -2
+        assert lib.hk_bf16_gemm(p, p, p, M, N, K & ~7, None) == -2
+        assert lib.hk_bf16_gemm_ws(p, p, p, M, N, K & ~7, p, 1 << 40, None) == -2
+        assert lib.hk_mxfp4_gemm(p, p, p, p, p, M, N, K & ~31, None) == -2
+        assert lib.hk_fp8_gemm_workspace_bytes(M, N, K) == 0
+        assert lib.hk_bf16_gemm_workspace_bytes(M, N, K) == 0
+        assert lib.hk_mxfp4_gemm_workspace_bytes(M, N, K) == 0
+    assert lib.hk_moe_mxfp4_workspace_bytes(16, 64, 32, imax, 2) == 0       # shapes the entry points refuse
+    assert lib.hk_moe_mxfp4_workspace_bytes(16, 64, 32, 4, 8) == 0          # k > E
+    assert lib.hk_moe_fp8blk_workspace_bytes(16, 128, 128, 513, 2) == 0
+    assert lib.hk_moe_topk_softmax(p, imax, 128, 4, p, p, None) == -2
+    assert lib.hk_moe_sort(p, imax, 8, 128, p, p, None, p, 1 << 40, None) == -2
     # extended MoE entry points: option checks come before anything touches memory
     args = (p, p, p, 8, p, p, 8, p, p, p, p, p, 16, 64, 32, 4, 2, 0)
     assert lib.hk_moe_mxfp4_experts_ex(*args, None, None, 7, 1.702, 7.0, 0, p, 1 << 30, None) == -6   # activation
