@@ -56,8 +56,12 @@ def _compile_one(src: Path, extra: list[str]) -> Path:
     return obj
 
 
-def build(verbose: bool = True, extra_flags: list[str] | None = None, jobs: int = 8) -> Path:
-    """Compile every csrc/*.hip and link libhk355.so. Always recompiles."""
+def build(verbose: bool = True, extra_flags: list[str] | None = None, jobs: int = 8, check: bool = True) -> Path:
+    """Compile every csrc/*.hip and link libhk355.so. Always recompiles.
+
+    check: also scan the kernels' assembly for the wait states the compiler does not provide around
+    inline assembly (isa_check) and refuse a library with findings: a kernel whose register allocation
+    puts a spill restore next to a hand-written load reads from a wild address on the GPU."""
     extra = list(extra_flags or [])
     BUILD_DIR.mkdir(parents=True, exist_ok=True)
     sources = sorted(CSRC.glob("*.hip"))
@@ -72,6 +76,16 @@ def build(verbose: bool = True, extra_flags: list[str] | None = None, jobs: int 
         _link(bench_objs, BENCH_LIB_PATH)
     if verbose:
         print(f"built {LIB_PATH} from {len(sources)} sources", file=sys.stderr)
+    if check and not extra:
+        from . import isa_check
+
+        findings = isa_check.check_sources(sources + bench_sources, jobs=jobs)
+        if findings:
+            LIB_PATH.unlink(missing_ok=True)
+            raise RuntimeError("isa_check: the built kernels break wait-state rules around inline assembly; "
+                               "library removed:\n" + "\n".join(str(f) for f in findings))
+        if verbose:
+            print("isa_check: 0 findings", file=sys.stderr)
     return LIB_PATH
 
 
@@ -85,4 +99,4 @@ def _link(objs: list[Path], out: Path) -> None:
 
 
 if __name__ == "__main__":
-    build()
+    build(check="--no-check" not in sys.argv[1:])

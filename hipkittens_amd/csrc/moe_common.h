@@ -34,6 +34,13 @@ __device__ __forceinline__ float silu_mul(float g, float u) {
 }
 
 inline int moe_round_up(int x, int m) { return (x + m - 1) / m * m; }
+// Whether most experts' rows fit one work item of `bm` rows: mean + one standard deviation of the rows
+// per expert when T * k slots spread uniformly over E experts. (The streaming kernels then read every
+// weight byte once and load the weights with the non-temporal hint.)
+inline bool moe_rows_fit_one_item(int T, int k, int E, int bm) {
+    const double mu = (double)T * k / E;
+    return mu + __builtin_sqrt(mu) <= bm;
+}
 // Bytes a layer's workspace carries behind its last region. The grouped GEMMs fetch the activation
 // rows and row scales of a work item in whole pieces (the streaming kernels 8 or 16 rows at a time,
 // the LDS-staged MXFP4 kernel its whole tile of 128 rows of 128 bytes): the last item's fetches run

@@ -1026,7 +1026,7 @@ extern "C" int hk_moe_fp8blk_experts_ex2(const void* x_e4m3, const float* x_scal
     moe_launch_build_items(expert_offsets, E, kF8BM, I / 128, (MoeItem*)(ws + L.items1), (H + 255) / 256,
                            (MoeItem*)(ws + L.items2), nitems, s);
     // non-temporal weight loads while most experts' rows fit one work item (their weights are then read once)
-    const bool nt = (long long)T * k * 4 <= (long long)E * 3 * kF8BM;
+    const bool nt = moe_rows_fit_one_item(T, k, E, kF8BM);
 
     MoeFp8Params p{};
     p.A = (const uint8_t*)x_e4m3; p.SA = x_scales; p.S = S;   // gathered by token index inside the kernel

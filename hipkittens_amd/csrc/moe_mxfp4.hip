@@ -787,24 +787,31 @@ __global__ __launch_bounds__(512) void moe_mxfp4_gemm_kernel(const MoeGemmParams
 // instead of from L2 (1.32 against 1.29 ms; 65536 tokens: 5.24 against 4.87): the host sets NT by
 // the average number of rows per expert.
 constexpr int kStBM = 192;                              // rows per work item
-template <bool A8>
+template <bool A8, bool GATHER>
 struct S4Cfg {
-    static constexpr int kBM = A8 ? 128 : kStBM;       // rows per work item
+    // rows per work item: what four LDS stages of the activation tile leave room for. MXFP8 rows are
+    // twice as long: 144 rows (random routing of 4096 tokens gives 128 +- 11 rows per expert: with 128-row
+    // items every second expert needed a second pass over its weights), 128 when the row scales' two
+    // super-step buffers have to fit as well
+    static constexpr int kBM = A8 ? (GATHER ? 128 : 144) : kStBM;
     static constexpr int kRow = A8 ? 256 : 128;        // activation bytes per row and K-step
     static constexpr int kATile = kBM * kRow;
-    static constexpr int kStage = kATile + kBM * 8;    // + row scales (MODE 1; MODE 0 leaves that part unused)
-    static constexpr int kScaleTile = kBM * 128;       // MODE 0: row scales of 16 K-steps, two buffers behind the stages
-    static constexpr int kLds = 4 * kStage;            // MODE 1: 102 KiB / 132 KiB
-    static constexpr int kLdsGather = 4 * kATile + 2 * kScaleTile;   // MODE 0: 144 KiB / 160 KiB
-    static constexpr int kPieces = kATile / 4096;      // 1 KiB activation loads per wave and position
+    static constexpr int kStage = GATHER ? kATile : kATile + kBM * 8;    // + row scales of the position (not GATHER)
+    static constexpr int kScaleTile = kBM * 128;       // GATHER: row scales of 16 K-steps, two buffers behind the stages
+    static constexpr int kGroups = (kBM + 31) / 32;    // groups of 32 rows: wave w loads rows 8 w .. +8 of each
+    static constexpr int kPieces = (A8 ? 2 : 1) * kGroups;   // 1 KiB activation loads per wave and position
+    // a last group that is not full: its pieces of the waves past the tile's end go to a dump area
+    static constexpr int kDump = kBM % 32 ? 4096 : 0;
+    static constexpr int kLds = 4 * kStage + (GATHER ? 2 * kScaleTile : 0) + kDump;   // 102 / 144 KiB (MXFP8: 149 / 160)
 };
-static_assert(S4Cfg<true>::kLdsGather <= 160 * 1024 && S4Cfg<false>::kLdsGather <= 160 * 1024, "LDS of a CU");
+static_assert(S4Cfg<true, true>::kLds <= 160 * 1024 && S4Cfg<false, true>::kLds <= 160 * 1024 &&
+              S4Cfg<true, false>::kLds <= 160 * 1024 && S4Cfg<false, false>::kLds <= 160 * 1024, "LDS of a CU");
 constexpr int kS4Ahead = 3;  // positions between fetch and compute (two measure the same)
 
 template <int MODE, bool EXT, bool A8, bool GATHER = false, bool NT = false>
 __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmParams p) {
     static_assert(!GATHER || (MODE == 0 && !EXT), "rows are gathered by the gate+up kernel with the plain epilogue only");
-    using Cfg = S4Cfg<A8>;
+    using Cfg = S4Cfg<A8, GATHER>;
     // GATHER (gate+up kernel, plain epilogue): the activation rows are fetched by token; the quantized x
     // is then stored once per token instead of once per routed slot (see tok_cur below), and its row
     // scales are stored 16 K-steps ("super-step") to a 128-byte row and fetched once per super-step
@@ -814,8 +821,8 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
     // the bytes), 16384 tokens 30 us more, 65536 tokens 70 us more: every XCD then reads all of x
     // instead of its experts' rows, and x no longer stays in its L2. The host picks by the size of x.
     constexpr int kBM = Cfg::kBM, kRow = Cfg::kRow, kATile = Cfg::kATile;
-    constexpr int kStage = GATHER ? Cfg::kATile : Cfg::kStage, kScaleTile = Cfg::kScaleTile;
-    constexpr int kPieces = Cfg::kPieces;
+    constexpr int kStage = Cfg::kStage, kScaleTile = Cfg::kScaleTile;
+    constexpr int kPieces = Cfg::kPieces, kGroups = Cfg::kGroups;
     constexpr int kScaleLoads = GATHER ? 0 : 1;
     constexpr int kLoads = kPieces + kScaleLoads + 10;   // + 8 weight fragments, 2 weight scale dwords
     constexpr int MT = kBM / 16;
@@ -890,7 +897,9 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
                 v4f& dst = bias_nxt[q];
                 const v4i rs = srd_bias;
                 const uint32_t voff = idx * 4u;
-                asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(dst) : "v"(voff), "s"(rs) : "memory");
+                // (s_nop 4: the descriptor may have been restored from a spill slot by a vector-ALU
+                // instruction directly in front of the statement)
+                asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(dst) : "v"(voff), "s"(rs) : "memory");
             }
         }
     };
@@ -920,7 +929,7 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
     // piece i of the activation (half-)tile = rows 8 (4 i + w) .. +8; the swizzle of a row depends
     // on its bits 1..3, i.e. on w and the lane only
     const uint32_t chunk16 = swz_chunk(8 * w + (lane >> 3), lane & 7);
-    constexpr int kNp = A8 ? 4 : kPieces;
+    constexpr int kNp = kGroups;
     constexpr int kTok = GATHER ? kNp : 1;
     uint32_t tok_cur[kTok], tok_nxt[kTok];
     const v4i srd_slots = make_srd(p.row_slots, GATHER ? (uint32_t)p.S * 4u : 0u);
@@ -991,6 +1000,8 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
     auto advance_cf = [&]() __attribute__((always_inline)) {
         if (++cf.kt == nk4) {
             cf.kt = 0; cf.it += it_stride; load_item(cf); cf_descriptors();
+            // the counter of outstanding vector-memory operations has six bits: room for the four bias loads
+            if constexpr (EXT && kS4Ahead * kLoads + 4 > 63) wait_vmcnt<63 - 4>();
             request_bias();
             if constexpr (GATHER) { adopt_tokens(); request_next_item(); cf_extra = 3; }
         }
@@ -1015,11 +1026,14 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
     // load L (0 .. kLoads - 1) of the fetch position, into LDS stage / register set P
     auto fetch_load = [&]<int P, int L>() __attribute__((always_inline)) {
         if constexpr (L < kPieces) {
-            constexpr int i = A8 ? (L & 3) : L, khalf = A8 ? (L >> 2) : 0;
+            constexpr int i = L % kGroups, khalf = L / kGroups;
             const int rows_up = cf.valid && cf.kt < nk ? (cf.rows + 15) & ~15 : 0;
             v4i sa = srd_a;
             if (8 * (4 * i + w) >= rows_up) sa.z = 0;  // past the item's last fragment: nothing is fetched
-            const uint32_t dst = lds_wave + (uint32_t)(P * kStage + khalf * (kBM * 128) + i * 4096);
+            uint32_t dst = lds_wave + (uint32_t)(P * kStage + khalf * (kBM * 128) + i * 4096);
+            // a piece past the tile's end (last, partial group of 32 rows): never holds rows, lands in the dump area
+            if constexpr (32 * i + 32 > kBM)
+                if (8 * (4 * i + w) >= kBM) dst = lds_wave + (uint32_t)(Cfg::kLds - Cfg::kDump);
             if constexpr (GATHER) {
                 dma16(sa, dst, tok_cur[i],
                       (uint32_t)cf.kt * (uint32_t)a_rows * (uint32_t)kRow + (uint32_t)(khalf * 128));
@@ -1039,16 +1053,19 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
             const uint32_t soff = (uint32_t)cf.kt * kMoeBTile + (uint32_t)(2 * w + pair) * 4096u;
             v4i rs = cf_srd_b;
             if (cf.kt >= nk) rs.z = 0;
-            if constexpr (NT)
-                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4 nt"
-                             : "=v"(bw[P][f])
-                             : "v"(voff), "s"(rs), "s"(soff), "n"(((f >> 1) & 1) * 2048 + half * 1024)
-                             : "memory");
-            else
-                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4"
-                             : "=v"(bw[P][f])
-                             : "v"(voff), "s"(rs), "s"(soff), "n"(((f >> 1) & 1) * 2048 + half * 1024)
-                             : "memory");
+            // (the first weight load of an MXFP8 position starts with s_nop 4: the descriptor's size word may
+            // have been restored from a spill slot by a vector-ALU instruction directly in front of the statement)
+#define HK_WLOAD(PRE, POST)                                                                      \
+    asm volatile(PRE "buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4" POST                   \
+                 : "=v"(bw[P][f])                                                                \
+                 : "v"(voff), "s"(rs), "s"(soff), "n"(((f >> 1) & 1) * 2048 + half * 1024)       \
+                 : "memory")
+            if constexpr (A8 && f == 0) {
+                if constexpr (NT) HK_WLOAD("s_nop 4\n\t", " nt"); else HK_WLOAD("s_nop 4\n\t", "");
+            } else {
+                if constexpr (NT) HK_WLOAD("", " nt"); else HK_WLOAD("", "");
+            }
+#undef HK_WLOAD
         } else if constexpr (L < kLoads) {
             constexpr int pair = L - kPieces - kScaleLoads - 8;
             int& dst = bsc[P][pair];
@@ -1325,6 +1342,8 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
 // chunk are issued together; KU == 0: any k, one row at a time. Same operations in the same order.
 // The rows of o are read exactly once: non-temporal loads (213 -> 187 us at T = 8192, k = 8,
 // H = 7168, i.e. 5.7 TB/s; the GPT-OSS-like layer 10 us less).
+// o has T * k rows; a position outside [0, T * k) (a caller's broken slot_to_pos) is not read and adds
+// nothing, like an expert id out of range in the sort.
 template <int KU>
 __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __restrict__ o,
                                                             const float* __restrict__ w,
@@ -1336,9 +1355,10 @@ __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __re
     float wt[KU > 0 ? KU : 1];
 #pragma unroll
     for (int j = 0; j < KU; ++j) {
-        pos[j] = j < k ? slot_to_pos[(size_t)t * k + j] : 0;
+        pos[j] = j < k ? slot_to_pos[(size_t)t * k + j] : -1;
         wt[j] = j < k ? w[(size_t)t * k + j] : 0.f;
     }
+    const uint32_t n_rows = (uint32_t)T * (uint32_t)k;
     for (int c = threadIdx.x; c < H / 8; c += 256) {
         float acc[8];
 #pragma unroll
@@ -1346,7 +1366,7 @@ __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __re
         v4i rows[KU > 0 ? KU : 1];
 #pragma unroll
         for (int j = 0; j < KU; ++j)
-            if (j < k) rows[j] = __builtin_nontemporal_load((const v4i*)(o + (size_t)pos[j] * H + c * 8));
+            if ((uint32_t)pos[j] < n_rows) rows[j] = __builtin_nontemporal_load((const v4i*)(o + (size_t)pos[j] * H + c * 8));
         if (add) {
             const v4i raw = *(const v4i*)(add + (size_t)t * H + c * 8);
 #pragma unroll
@@ -1358,7 +1378,7 @@ __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __re
         if constexpr (KU > 0) {
 #pragma unroll
             for (int j = 0; j < KU; ++j)
-                if (j < k) {
+                if ((uint32_t)pos[j] < n_rows) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         acc[2 * i] += wt[j] * __uint_as_float((uint32_t)rows[j][i] << 16);
@@ -1368,6 +1388,7 @@ __global__ __launch_bounds__(256) void moe_unpermute_kernel(const uint16_t* __re
         } else {
             for (int j = 0; j < k; ++j) {
                 const int pj = slot_to_pos[(size_t)t * k + j];
+                if ((uint32_t)pj >= n_rows) continue;
                 const float wj = w[(size_t)t * k + j];
                 const v4i raw = *(const v4i*)(o + (size_t)pj * H + c * 8);
 #pragma unroll
@@ -1406,7 +1427,7 @@ void moe_launch_build_items(const int32_t* expert_offsets, int E, int bm, int n_
 
 template <int MODE, bool EXT, bool A8, bool GATHER, bool NT>
 static int launch_moe_stream_nt(MoeGemmParams p, int max_items, hipStream_t s) {
-    constexpr int lds = GATHER ? S4Cfg<A8>::kLdsGather : S4Cfg<A8>::kLds, threads = 256;
+    constexpr int lds = S4Cfg<A8, GATHER>::kLds, threads = 256;
     const void* kern = (const void*)moe_mxfp4_stream4_kernel<MODE, EXT, A8, GATHER, NT>;
     static DeviceOnce configured;
     if (!set_lds_limit_once(kern, lds, configured)) return HK_ERR_LAUNCH;
@@ -1566,9 +1587,9 @@ static int moe_mxfp4_check(int T, int H, int I, int E, int k, int w13_scale_pitc
     return HK_OK;
 }
 
-static MoeBuildItems moe_items_args(uint8_t* ws, const MoeWs& L, int I, int H, bool a8, int weight_layout) {
+static MoeBuildItems moe_items_args(uint8_t* ws, const MoeWs& L, int I, int H, bool a8, int weight_layout, bool gather) {
     MoeBuildItems b;
-    b.bm = a8 ? S4Cfg<true>::kBM : weight_layout ? kStBM : kMoeBM;
+    b.bm = a8 ? (gather ? S4Cfg<true, true>::kBM : S4Cfg<true, false>::kBM) : weight_layout ? kStBM : kMoeBM;
     b.items[0] = (MoeItem*)(ws + L.items1); b.items[1] = (MoeItem*)(ws + L.items2);
     b.n_tiles[0] = (I + 127) / 128; b.n_tiles[1] = (H + 255) / 256;
     return b;
@@ -1631,11 +1652,12 @@ static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const voi
 
     int32_t* nitems = (int32_t*)(ws + L.nitems);
     const bool gather = moe_gathers(weight_layout, ext, a8, T, H);
-    // non-temporal weight loads while most experts' rows fit one work item (their weights are then read once)
-    const bool nt = (long long)T * k * 4 <= (long long)E * 3 * (a8 ? S4Cfg<true>::kBM : kStBM);
+    // non-temporal weight loads while most experts' rows fit one work item (their weights are then read
+    // once): mean + one standard deviation of the rows per expert under uniform routing
+    const bool nt = moe_rows_fit_one_item(T, k, E, a8 ? (gather ? S4Cfg<true, true>::kBM : S4Cfg<true, false>::kBM) : kStBM);
     if (!x_quantized) {   // (the forward pass of a small layer has done this in its sort launch)
         const int nk1 = (H / 2 + 127) / 128;
-        const MoeBuildItems b = moe_items_args(ws, L, I, H, a8, weight_layout);
+        const MoeBuildItems b = moe_items_args(ws, L, I, H, a8, weight_layout, gather);
         const MxQuantizeArgs qa = moe_quantize_args(x_bf16, sorted_slots, slot_to_pos, k, T, H, I, ws, L);
         auto qp = a8 ? (gather ? mx_quantize_permute_kernel<true, false> : mx_quantize_permute_kernel<true, true>)
                      : (gather ? mx_quantize_permute_kernel<false, false> : mx_quantize_permute_kernel<false, true>);
@@ -1755,7 +1777,7 @@ static int moe_mxfp4_forward_impl(const void* x_bf16, const float* router_logits
         // sort, item lists and the quantization of x in one launch (moe_sort_quantize_kernel)
         const int S = T * k, nchunks = (S + kSortChunk - 1) / kSortChunk;
         const int nk1 = (H / 2 + 127) / 128;
-        const MoeBuildItems b = moe_items_args(ws, L, I, H, a8, weight_layout);
+        const MoeBuildItems b = moe_items_args(ws, L, I, H, a8, weight_layout, true);
         const MxQuantizeArgs qa = moe_quantize_args(x_bf16, nullptr, nullptr, k, T, H, I, ws, L);
         const int grid = nchunks + 2 * kFusedItemParts + (T + kQpRows - 1) / kQpRows * ((nk1 + 7) / 8);
         auto kern = a8 ? moe_sort_quantize_kernel<true> : moe_sort_quantize_kernel<false>;

@@ -212,7 +212,8 @@ int hk_moe_sort(const int32_t* ids, int T, int k, int E, int32_t* sorted_slots,
 int hk_mxfp4_quantize_rows(const void* x_bf16, int rows, int cols, void* packed, void* scales,
                            int scale_pitch, void* stream);
 
-/* y[t,:] = bf16(sum_j w[t,j] * o[slot_to_pos[t*k+j], :]), o [T*k, H] bf16. H % 8 == 0. */
+/* y[t,:] = bf16(sum_j w[t,j] * o[slot_to_pos[t*k+j], :]), o [T*k, H] bf16. H % 8 == 0.
+ * A position outside [0, T*k) is not read and adds nothing to its token. */
 int hk_moe_unpermute(const void* o_bf16, const float* w, const int32_t* slot_to_pos, int T, int k,
                      int H, void* y_bf16, void* stream);
 /* As hk_moe_unpermute with a residual: y[t,:] = bf16(add[t,:] + sum_j ...), add [T, H] bf16 or NULL
@@ -242,7 +243,7 @@ int hk_moe_mxfp4_preshuffle(const void* w, const void* scales, int scale_pitch, 
  * expert_offsets and slot_to_pos must be one consistent result of hk_moe_sort: the kernels index
  * activations and outputs with them (through range-checked descriptors where they fetch rows by
  * token, so slots outside [0, T*k) read zeros or neighbouring workspace, never outside it; the
- * un-permute reads o at slot_to_pos unchecked). */
+ * un-permute skips positions outside [0, T*k)). */
 int hk_moe_mxfp4_experts(const void* x_bf16, const void* w13, const void* w13_scales,
                          int w13_scale_pitch, const void* w2, const void* w2_scales,
                          int w2_scale_pitch, const float* topk_w, const int32_t* sorted_slots,

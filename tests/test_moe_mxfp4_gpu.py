@@ -386,3 +386,58 @@ def test_moe_mxfp4_activation_paths_and_experts_entry(hk, T, E, k, H, I, act_for
                                             act_format=act_format)
     torch.cuda.synchronize()
     assert torch.equal(ye, y)
+
+
+def test_unpermute_skips_positions_outside_the_rows_of_o(hk):
+    """A position outside [0, T*k) in slot_to_pos is not read and adds nothing: o sits at the end of a
+    NaN-filled pool, so a read past it (or in front of it) would show in y."""
+    rng = np.random.default_rng(5)
+    for T, k, H in ((50, 4, 512), (9, 8, 1024), (6, 11, 256)):
+        S = T * k
+        pool = torch.full(((S + 64) * H,), float("nan"), dtype=torch.bfloat16, device=DEV)
+        o = pool[32 * H:(32 + S) * H].view(S, H)
+        o.copy_(_to_bf16_tensor(_bf16(rng.standard_normal((S, H)))))
+        w = rng.random((T, k)).astype(np.float32)
+        inv = rng.permutation(S).astype(np.int32)
+        bad = rng.random(S) < 0.3
+        inv_bad = inv.copy()
+        inv_bad[bad] = rng.choice(np.array([-1, -7, S, S + 3, 2 ** 31 - 1, -2 ** 31], dtype=np.int64),
+                                  size=int(bad.sum())).astype(np.int32)
+        y = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+        hk.tk_kernel.dispatch_moe_unpermute(o, torch.from_numpy(w).to(DEV), torch.from_numpy(inv_bad).to(DEV), y)
+        # the same call with the bad slots' weights zeroed and their positions valid
+        w0 = np.where(bad.reshape(T, k), 0.0, w).astype(np.float32)
+        y0 = torch.full_like(y, float("nan"))
+        hk.tk_kernel.dispatch_moe_unpermute(o, torch.from_numpy(w0).to(DEV), torch.from_numpy(inv).to(DEV), y0)
+        torch.cuda.synchronize()
+        assert torch.isfinite(y.float()).all()
+        assert torch.equal(y, y0)
+
+
+def test_moe_mxfp4_experts_with_positions_out_of_range(hk):
+    """hk_moe_mxfp4_experts on a slot_to_pos with entries outside [0, T*k): normal exit, finite output,
+    and the tokens whose positions are intact get what the intact call gives them."""
+    T, E, k, H, I = 200, 8, 2, 512, 256
+    x, logits, w13p, w13s, w2p, w2s = _device_layer(hk, T, E, k, H, I, seed=11)
+    shuf = hk.tk_kernel.MoeMxfp4ShuffledWeights.from_plain(w13p, w13s, w2p, w2s)
+    ws = torch.empty(hk.tk_kernel.moe_mxfp4_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device=DEV)
+    ids = torch.empty((T, k), dtype=torch.int32, device=DEV)
+    wts = torch.empty((T, k), dtype=torch.float32, device=DEV)
+    hk.tk_kernel.dispatch_moe_topk_softmax(logits, ids, wts)
+    sorted_slots = torch.empty(T * k, dtype=torch.int32, device=DEV)
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=DEV)
+    inv = torch.empty(T * k, dtype=torch.int32, device=DEV)
+    sws = torch.empty(hk.tk_kernel.moe_sort_workspace_bytes(T, k, E), dtype=torch.uint8, device=DEV)
+    hk.tk_kernel.dispatch_moe_sort(ids, sorted_slots, offsets, inv, sws)
+    y = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hk.tk_kernel.dispatch_moe_mxfp4_experts(x, shuf, None, None, None, wts, sorted_slots, offsets, inv, y, ws)
+    inv_bad = inv.clone()
+    broken_tokens = torch.tensor([0, 17, 63, T - 1], device=DEV)
+    inv_bad.view(T, k)[broken_tokens, 0] = torch.tensor([-1, T * k, 2 ** 31 - 1, -2 ** 31], dtype=torch.int32, device=DEV)
+    yb = torch.full_like(y, float("nan"))
+    hk.tk_kernel.dispatch_moe_mxfp4_experts(x, shuf, None, None, None, wts, sorted_slots, offsets, inv_bad, yb, ws)
+    torch.cuda.synchronize()
+    assert torch.isfinite(yb.float()).all()
+    intact = torch.ones(T, dtype=torch.bool, device=DEV)
+    intact[broken_tokens] = False
+    assert torch.equal(yb[intact], y[intact])
