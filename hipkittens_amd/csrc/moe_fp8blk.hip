@@ -406,7 +406,11 @@ __global__ __launch_bounds__(512) void moe_fp8blk_gemm_kernel(const MoeFp8Params
 // runs from a cold instruction cache). Padding positions fetch nothing: their LDS tile, row scales
 // and weight registers read as zeros and add nothing.
 // Results are bit-identical to the kernel above (same MFMA, K order and scaling FMAs).
-constexpr int kF8sMT = kF8BM / 16;                       // 10 row fragments per item
+constexpr int kF8sMT = kF8BM / 16;                       // at most 10 row fragments per item
+// Items of nine fragments (144 rows): every K-step then runs nine fragments instead of ten. The host picks them
+// when they do not add a pass over the weights (moe_fp8blk_item_rows): at 256 +- 16 rows per expert (the
+// DeepSeek-V3-like layer at 8192 tokens) two items of up to 144 rows cover all but one expert in fifty.
+constexpr int kF8BMShort = 144;
 constexpr int kF8sStages = 4;                           // LDS stages = weight register sets = positions per trip of the K loop
 constexpr int kF8sStage = 21504;                         // 160 x 128 B, then 16 x 12 row scales, padded to a multiple of 256 B
 constexpr int kF8sXch = kF8sStages * kF8sStage;          // epilogue exchange buffer: 160 x 4 floats
@@ -414,7 +418,7 @@ constexpr int kF8sLds = kF8sXch + kF8BM * 16;            // 86.5 KiB
 constexpr int kF8sBTile = 256 * 128;                     // one (n-tile, K-step) block of the pre-shuffled weights
 constexpr int kF8sLoads = 14;                            // loads per wave and position
 static_assert(kF8sStage >= kF8ATile + 16 * 12 * 4 && kF8sStage % 256 == 0 && kF8sLds <= 160 * 1024, "LDS plan");
-static_assert((kF8sStages - 2) * kF8sLoads < 64 && kF8sStages == 4 && kF8sMT == 10, "vmcnt range; the slot plan below is written for ten fragments");
+static_assert((kF8sStages - 2) * kF8sLoads < 64 && kF8sStages == 4 && kF8sMT == 10 && kF8BMShort == 144, "vmcnt range; the slot plan below is written for nine or ten fragments");
 
 // The weight ring lives in fixed accumulation registers: fragment F = 4 * set + n of the ring in
 // a[8 F .. 8 F + 7] (low / high K half in the first / last four). Naming them in the constraints keeps the two
@@ -446,10 +450,11 @@ struct F8Cursor { int it, kt, expert, row_start, rows, n_tile; bool valid; };
 // NONTEMP: weight loads with the non-temporal hint, for layers whose experts' rows fit one work item
 // (the weights are then read once; see moe_mxfp4_stream4_kernel). At the DeepSeek-V3-like shape
 // (256 rows per expert = two items) the second item would fetch them from HBM again: 4.24 against 4.12 ms.
-template <int MODE, bool GATHER, bool NONTEMP = false>
+template <int MODE, bool GATHER, bool NONTEMP = false, int MT = kF8sMT>
 __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Params p) {
     static_assert(!GATHER || MODE == 0, "only the gate+up GEMM reads the caller's activations");
-    constexpr int MT = kF8sMT, NT = 4, NA = 5;
+    static_assert(MT == kF8sMT || MT == kF8BMShort / 16, "row fragments of an item");
+    constexpr int NT = 4, NA = 5;
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
     const int lane = lane_id(), w = wave_id();
 
@@ -770,6 +775,10 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
     // fragment count that varies would put the accumulators behind branches.
     auto step = [&]<int P>() __attribute__((always_inline)) {
         constexpr int PF = (P + kF8sStages - 1) % kF8sStages, PN = (P + 1) % kF8sStages;
+        // af / xs_r / sc are double buffers indexed by fragment parity. With an odd number of fragments the
+        // first fragment of consecutive positions would meet the last one of the position before in the same
+        // buffer, so odd positions start on buffer 1 (an item has a multiple of four positions).
+        constexpr int PAR = (MT & 1) ? (P & 1) : 0, PAR_PREV = (MT & 1) ? (PAR ^ 1) : 0, PAR_NEXT = PAR_PREV;
         fetch_begin();
         landed.template operator()<P>();
         const uint32_t a_lo = rd_lo + P * kF8sStage, a_hi = rd_hi + P * kF8sStage, a_sa = rd_sa + P * kF8sStage;
@@ -780,42 +789,44 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
             asm volatile("" : "+s"(ws0_next), "+s"(ws1_next));
             wait_vmcnt<(kF8sStages - 2) * kF8sLoads>();
             block_barrier();   // everyone's part of the next position's tile has landed; everyone has read this position's
-            af[0] = lds_frag(rd_lo + PN * kF8sStage, rd_hi + PN * kF8sStage, 0);
-            xs_r[0] = *(lds_f32_t*)(uintptr_t)(rd_sa + PN * kF8sStage);
+            af[PAR_NEXT] = lds_frag(rd_lo + PN * kF8sStage, rd_hi + PN * kF8sStage, 0);
+            xs_r[PAR_NEXT] = *(lds_f32_t*)(uintptr_t)(rd_sa + PN * kF8sStage);
         };
         // Fragment M: four MFMA slots; the FMAs of an MFMA follow two slots later (fragment 0 starts with
         // those of fragment 9 of the previous K-step).
         auto block = [&]<int M>() __attribute__((always_inline)) {
             constexpr int MP = M == 0 ? MT - 1 : M - 1;   // the fragment whose last two FMA groups are still owed
-            const v8i& a_cur = af[M & 1];
+            constexpr int B = (M + PAR) & 1, BN = B ^ 1;  // this fragment's buffer, the next one's
+            constexpr int BP = M == 0 ? (MT - 1 + PAR_PREV) & 1 : BN;   // the buffer of fragment MP
+            const v8i& a_cur = af[B];
             // slot 0
             mfma.template operator()<P * NT + 0>(part[0], a_cur);
             if constexpr (M < MT - 2) {
-                af[(M + 1) & 1] = lds_frag(a_lo, a_hi, (M + 1) * 2048);
-                xs_r[(M + 1) & 1] = *(lds_f32_t*)(uintptr_t)(a_sa + (M + 1) * 4);
+                af[BN] = lds_frag(a_lo, a_hi, (M + 1) * 2048);
+                xs_r[BN] = *(lds_f32_t*)(uintptr_t)(a_sa + (M + 1) * 4);
             }
-            fma4(acc[MP][2], part[2], sc[MP & 1][0]);
+            fma4(acc[MP][2], part[2], sc[BP][0]);
             if constexpr (M <= 6) fetch_load.template operator()<PF, 2 * M>();
             __builtin_amdgcn_sched_barrier(0);
             // slot 1
             mfma.template operator()<P * NT + 1>(part[1], a_cur);
-            fma4(acc[MP][3], part[3], sc[MP & 1][1]);
-            sc[M & 1][0] = xs_r[M & 1] * ws0;
-            sc[M & 1][1] = xs_r[M & 1] * ws1;
+            fma4(acc[MP][3], part[3], sc[BP][1]);
+            sc[B][0] = xs_r[B] * ws0;
+            sc[B][1] = xs_r[B] * ws1;
             if constexpr (M <= 6) fetch_load.template operator()<PF, 2 * M + 1>();
             __builtin_amdgcn_sched_barrier(0);
             // slot 2
             mfma.template operator()<P * NT + 2>(part[2], a_cur);
-            fma4(acc[M][0], part[0], sc[M & 1][0]);
+            fma4(acc[M][0], part[0], sc[B][0]);
             if constexpr (M == MT - 2) {
                 // fragment 9 is read here, ahead of the barrier that frees this stage
-                af[(M + 1) & 1] = lds_frag(a_lo, a_hi, (M + 1) * 2048);
-                xs_r[(M + 1) & 1] = *(lds_f32_t*)(uintptr_t)(a_sa + (M + 1) * 4);
+                af[BN] = lds_frag(a_lo, a_hi, (M + 1) * 2048);
+                xs_r[BN] = *(lds_f32_t*)(uintptr_t)(a_sa + (M + 1) * 4);
             }
             __builtin_amdgcn_sched_barrier(0);
             // slot 3
             mfma.template operator()<P * NT + 3>(part[3], a_cur);
-            fma4(acc[M][1], part[1], sc[M & 1][1]);
+            fma4(acc[M][1], part[1], sc[B][1]);
             __builtin_amdgcn_sched_barrier(0);
         };
         block.template operator()<0>();
@@ -826,26 +837,27 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
         block.template operator()<5>();
         block.template operator()<6>();
         block.template operator()<7>();
-        block.template operator()<8>();
-        // fragment 9, with the transition to the next position behind its first MFMA: ws0 / ws1 keep this
-        // position's values until the end of the step
+        if constexpr (MT > 9) block.template operator()<8>();
+        // the last fragment, with the transition to the next position behind its first MFMA: ws0 / ws1 keep
+        // this position's values until the end of the step
         {
             constexpr int M = MT - 1, MP = M - 1;
-            const v8i& a_cur = af[M & 1];
+            constexpr int B = (M + PAR) & 1, BP = B ^ 1;
+            const v8i& a_cur = af[B];
             mfma.template operator()<P * NT + 0>(part[0], a_cur);
-            fma4(acc[MP][2], part[2], sc[MP & 1][0]);
+            fma4(acc[MP][2], part[2], sc[BP][0]);
             __builtin_amdgcn_sched_barrier(0);
             mfma.template operator()<P * NT + 1>(part[1], a_cur);
-            fma4(acc[MP][3], part[3], sc[MP & 1][1]);
-            sc[M & 1][0] = xs_r[M & 1] * ws0;
-            sc[M & 1][1] = xs_r[M & 1] * ws1;
+            fma4(acc[MP][3], part[3], sc[BP][1]);
+            sc[B][0] = xs_r[B] * ws0;
+            sc[B][1] = xs_r[B] * ws1;
             transition();
             __builtin_amdgcn_sched_barrier(0);
             mfma.template operator()<P * NT + 2>(part[2], a_cur);
-            fma4(acc[M][0], part[0], sc[M & 1][0]);
+            fma4(acc[M][0], part[0], sc[B][0]);
             __builtin_amdgcn_sched_barrier(0);
             mfma.template operator()<P * NT + 3>(part[3], a_cur);
-            fma4(acc[M][1], part[1], sc[M & 1][1]);
+            fma4(acc[M][1], part[1], sc[B][1]);
             __builtin_amdgcn_sched_barrier(0);
         }
         fetch_advance();
@@ -853,11 +865,12 @@ __global__ __launch_bounds__(256) void moe_fp8blk_stream_kernel(const MoeFp8Para
             if (cc.valid && cc.kt == nk4 - 1) {
                 // the item is complete: the two FMA groups still owed, then the epilogue
                 mfma_drain();
-                fma4(acc[MT - 1][2], part[2], sc[(MT - 1) & 1][0]);
-                fma4(acc[MT - 1][3], part[3], sc[(MT - 1) & 1][1]);
+                fma4(acc[MT - 1][2], part[2], sc[(MT - 1 + PAR) & 1][0]);
+                fma4(acc[MT - 1][3], part[3], sc[(MT - 1 + PAR) & 1][1]);
                 epilogue(cc);
                 zero_acc();
-                sc[(MT - 1) & 1][0] = 0.f; sc[(MT - 1) & 1][1] = 0.f;   // what the next K-step adds for "fragment 9 of the previous K-step"
+                // what the next K-step adds for "the last fragment of the previous K-step"
+                sc[(MT - 1 + PAR) & 1][0] = 0.f; sc[(MT - 1 + PAR) & 1][1] = 0.f;
             }
         }
         cc = cn;
@@ -906,9 +919,9 @@ static int launch_fp8blk_gemm(const MoeFp8Params& p, int max_items, hipStream_t 
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
-template <int MODE, bool GATHER, bool NT>
+template <int MODE, bool GATHER, bool NT, int MT>
 static int launch_fp8blk_stream_nt(const MoeFp8Params& p, int max_items, hipStream_t s) {
-    auto kern = moe_fp8blk_stream_kernel<MODE, GATHER, NT>;
+    auto kern = moe_fp8blk_stream_kernel<MODE, GATHER, NT, MT>;
     static DeviceOnce configured;
     if (!set_lds_limit_once((const void*)kern, kF8sLds, configured)) return HK_ERR_LAUNCH;
     const int grid = min(max_items, moe_num_compute_units());
@@ -916,10 +929,25 @@ static int launch_fp8blk_stream_nt(const MoeFp8Params& p, int max_items, hipStre
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
+// bm: rows per work item the item lists were built for (kF8BM or kF8BMShort)
 template <int MODE, bool GATHER>
-static int launch_fp8blk_stream(const MoeFp8Params& p, int max_items, hipStream_t s, bool nt) {
-    return nt ? launch_fp8blk_stream_nt<MODE, GATHER, true>(p, max_items, s)
-              : launch_fp8blk_stream_nt<MODE, GATHER, false>(p, max_items, s);
+static int launch_fp8blk_stream(const MoeFp8Params& p, int max_items, hipStream_t s, bool nt, int bm) {
+    constexpr int kShort = kF8BMShort / 16;
+    if (bm == kF8BMShort)
+        return nt ? launch_fp8blk_stream_nt<MODE, GATHER, true, kShort>(p, max_items, s)
+                  : launch_fp8blk_stream_nt<MODE, GATHER, false, kShort>(p, max_items, s);
+    return nt ? launch_fp8blk_stream_nt<MODE, GATHER, true, kF8sMT>(p, max_items, s)
+              : launch_fp8blk_stream_nt<MODE, GATHER, false, kF8sMT>(p, max_items, s);
+}
+
+// Rows per work item of the streaming kernels for a layer of T * k slots over E experts: 144 unless
+// that costs a pass over the weights that 160 would not (judged at mean + two standard deviations of
+// an expert's rows under uniform routing).
+static int moe_fp8blk_item_rows(int T, int k, int E) {
+    const double mu = (double)T * k / E, hi = mu + 2.0 * __builtin_sqrt(mu);
+    const long long n_short = (long long)((hi + kF8BMShort - 1) / kF8BMShort);
+    const long long n_long = (long long)((hi + kF8BM - 1) / kF8BM);
+    return n_short <= n_long ? kF8BMShort : kF8BM;
 }
 
 // n-tiles of 256 weight rows of the two GEMMs: gate+up (mode 0: 128 h columns = 128 gate + 128 up rows
@@ -937,7 +965,7 @@ static Fp8Ws fp8_ws_layout(int T, int H, int I, int E, int k) {
     const size_t S = (size_t)T * k;
     L.ids = take(S * 4); L.w = take(S * 4); L.sorted = take(S * 4); L.offsets = take((size_t)(E + 1) * 4);
     L.inv = take(S * 4); L.sort_ws = take(hk_moe_sort_workspace_bytes(T, k, E));
-    const int max_tiles = (int)(S / kF8BM) + E;
+    const int max_tiles = (int)(S / kF8BMShort) + E;   // whichever item size the layer runs with
     L.max_items1 = max_tiles * (I / 128);
     L.max_items2 = max_tiles * ((H + 255) / 256);
     L.items1 = take((size_t)L.max_items1 * sizeof(MoeItem));
@@ -1023,10 +1051,11 @@ extern "C" int hk_moe_fp8blk_experts_ex2(const void* x_e4m3, const float* x_scal
     uint8_t* ws = (uint8_t*)workspace;
     const int S = T * k;
     int32_t* nitems = (int32_t*)(ws + L.nitems);
-    moe_launch_build_items(expert_offsets, E, kF8BM, I / 128, (MoeItem*)(ws + L.items1), (H + 255) / 256,
+    const int bm = weight_layout == 1 ? moe_fp8blk_item_rows(T, k, E) : kF8BM;
+    moe_launch_build_items(expert_offsets, E, bm, I / 128, (MoeItem*)(ws + L.items1), (H + 255) / 256,
                            (MoeItem*)(ws + L.items2), nitems, s);
     // non-temporal weight loads while most experts' rows fit one work item (their weights are then read once)
-    const bool nt = moe_rows_fit_one_item(T, k, E, kF8BM);
+    const bool nt = moe_rows_fit_one_item(T, k, E, bm);
 
     MoeFp8Params p{};
     p.A = (const uint8_t*)x_e4m3; p.SA = x_scales; p.S = S;   // gathered by token index inside the kernel
@@ -1038,7 +1067,7 @@ extern "C" int hk_moe_fp8blk_experts_ex2(const void* x_e4m3, const float* x_scal
     p.K = H; p.N = I; p.n_tiles_n = I / 128;
     if (weight_layout == 1) {
         p.b_expert_stride = (long long)fp8blk_n_tiles(0, I) * (H / 128) * kF8sBTile;
-        st = launch_fp8blk_stream<0, true>(p, L.max_items1, s, nt);
+        st = launch_fp8blk_stream<0, true>(p, L.max_items1, s, nt, bm);
     } else {
         st = launch_fp8blk_gemm<0, true>(p, L.max_items1, s);
     }
@@ -1053,7 +1082,7 @@ extern "C" int hk_moe_fp8blk_experts_ex2(const void* x_e4m3, const float* x_scal
     q.K = I; q.N = H; q.n_tiles_n = (H + 255) / 256;
     if (weight_layout == 1) {
         q.b_expert_stride = (long long)fp8blk_n_tiles(1, H) * (I / 128) * kF8sBTile;
-        st = launch_fp8blk_stream<1, false>(q, L.max_items2, s, nt);
+        st = launch_fp8blk_stream<1, false>(q, L.max_items2, s, nt, bm);
     } else {
         st = launch_fp8blk_gemm<1, false>(q, L.max_items2, s);
     }
