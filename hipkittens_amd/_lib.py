@@ -12,6 +12,7 @@ _lib = None
 SIGNATURES = {
     "hk_status_string": (ctypes.c_char_p, [c_int]),
     "hk_version": (c_int, []),
+    "hk_gemm_tile_choice": (c_int, [c_int] * 5),
     "hk_fp8_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p]),
     "hk_fp8_gemm_variant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_int, c_void_p]),
     "hk_mxfp4_gemm": (c_int, [c_void_p] * 5 + [c_int] * 3 + [c_void_p]),

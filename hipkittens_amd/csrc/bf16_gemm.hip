@@ -215,7 +215,7 @@ extern "C" int hk_bf16_gemm(const void* A, const void* B, void* C, int M, int N,
     if (gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     const bool tile_ok = K > 0 && (long long)2 * K * BM < (1ll << 31);
     // the same choice of tile as hk_fp8_gemm (pick_tile), with this format's measured corrections
-    const int tile = pick_tile(M, N, (int)((2ll * K + BK - 1) / BK), TileRule{32, 64, 96});
+    const int tile = pick_tile(kFmtBf16, M, N, (int)((2ll * K + BK - 1) / BK), kTileRuleBf16);
     const int variant = !tile_ok ? 0 : tile == kTinyTile ? 3 : tile == kSmallTile ? 2 : 1;
     return hk_bf16_gemm_variant(A, B, C, M, N, K, variant, stream);
 }

@@ -272,13 +272,22 @@ extern "C" int hk_fp8_gemm_static_ws(const void* A, const void* B, void* C, int 
     return hk_fp8_gemm_ws(A, B, C, M, N, K, scale_a, scale_b, ws, kStaticScratchBytes, stream);
 }
 
+extern "C" int hk_gemm_tile_choice(int format, int M, int N, int K, int consult_table) {
+    using namespace hk;
+    if (format < 0 || format > 2 || M <= 0 || N <= 0 || K <= 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
+    const long long row_bytes = format == kFmtFp8 ? K : format == kFmtBf16 ? 2ll * K : K / 2;
+    const int nk = (int)((row_bytes + BK - 1) / BK);
+    const TileRule rule = format == kFmtFp8 ? kTileRuleFp8 : format == kFmtBf16 ? kTileRuleBf16 : kTileRuleMxfp4;
+    return pick_tile(format, M, N, nk, rule, consult_table != 0);
+}
+
 extern "C" int hk_fp8_gemm(const void* A, const void* B, void* C, int M, int N, int K,
                            float scale_a, float scale_b, void* stream) {
     using namespace hk;
     if (gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     const bool tile_ok = K > 0 && (long long)K * BM < (1ll << 31);
     // 256x256 tiles (five-slot ring kernel), 128x128 or 64x64: see pick_tile
-    const int tile = pick_tile(M, N, (K + BK - 1) / BK, TileRule{16, 32, 80});
+    const int tile = pick_tile(kFmtFp8, M, N, (K + BK - 1) / BK, kTileRuleFp8);
     const int variant = !tile_ok ? 0 : tile == kTinyTile ? 6 : tile == kSmallTile ? 5 : 4;
     return hk_fp8_gemm_variant(A, B, C, M, N, K, scale_a, scale_b, variant, stream);
 }

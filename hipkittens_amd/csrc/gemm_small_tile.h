@@ -32,7 +32,17 @@ constexpr int kTinyLdsBytes = kTinyStages * 2 * kTinyTile * BK;  // 64 KiB
 // MMA::kScaled (MXFP4): every operand row also has e8m0 block scales, 8 bytes per K-step, in rows of
 // sa_pitch / sb_pitch bytes (multiples of 8); `MMA::mma(acc, b, a, sb, sa)` then takes, per fragment,
 // the lane's scale bytes of the K-step's two halves in bits [7:0] of .x / .y.
-struct SmallTileScales { const uint8_t* SA; const uint8_t* SB; int sa_pitch, sb_pitch; };
+// tail_pair / tail_shift: the pair of K-steps whose scale fetch starts tail_shift bytes early (rows that do not
+// hold whole groups of 16 scale bytes; see mxfp4_gemm.hip), -1 / 0: none.
+// row_bytes: scale bytes of a row that may be fetched (0: the whole pitch); the last row of an operand is in
+// the descriptor's range up to there.
+struct SmallTileScales {
+    const uint8_t* SA; const uint8_t* SB; int sa_pitch, sb_pitch; int tail_pair = -1, tail_shift = 0, row_bytes = 0;
+};
+// bytes of the scale rows [row0, row0 + rows) that a descriptor covers
+__device__ __forceinline__ uint32_t scale_rows_bytes(int rows, int pitch, int row_bytes) {
+    return (uint32_t)(rows - 1) * (uint32_t)pitch + (uint32_t)(row_bytes ? row_bytes : pitch);
+}
 template <int TILE, int STAGES>
 constexpr int small_tile_lds_bytes(bool scaled) { return STAGES * 2 * TILE * BK + (scaled ? 4 * 2 * TILE * 16 : 0); }
 
@@ -99,8 +109,8 @@ __device__ __forceinline__ void gemm_small_tile_body(
         int rr = op ? b_row_to_col(R) : R;
         if (EDGE) rr = min(rr, (op ? b_rows : a_rows) - 1);
         const int pitch = op ? sc.sb_pitch : sc.sa_pitch;
-        srd_s = op ? make_srd(sc.SB + (size_t)col0 * pitch, (uint32_t)b_rows * (uint32_t)pitch)
-                   : make_srd(sc.SA + (size_t)row0 * pitch, (uint32_t)a_rows * (uint32_t)pitch);
+        srd_s = op ? make_srd(sc.SB + (size_t)col0 * pitch, scale_rows_bytes(b_rows, pitch, sc.row_bytes))
+                   : make_srd(sc.SA + (size_t)row0 * pitch, scale_rows_bytes(a_rows, pitch, sc.row_bytes));
         voff_s = (uint32_t)rr * (uint32_t)pitch;
         lds_s = to_sgpr(lds0 + kScaleBase + (uint32_t)op * (TILE * 16) + (uint32_t)srow0 * 16u);
     }
@@ -113,7 +123,9 @@ __device__ __forceinline__ void gemm_small_tile_body(
         for (int i = 0; i < NDMA; ++i) dma16(srd_a, dst + i * NW * 1024, voff_a[i] | vor, k0);
 #pragma unroll
         for (int i = 0; i < NDMA; ++i) dma16(srd_b, dst + kTB + i * NW * 1024, voff_b[i] | vor, k0);
-        if (kScaled) dma16(srd_s, lds_s + (uint32_t)((kt >> 1) & 3) * kScaleSlot, voff_s, (uint32_t)(kt >> 1) * 16u);
+        if (kScaled)
+            dma16(srd_s, lds_s + (uint32_t)((kt >> 1) & 3) * kScaleSlot, voff_s,
+                  (uint32_t)(kt >> 1) * 16u - ((kt >> 1) == sc.tail_pair ? (uint32_t)sc.tail_shift : 0u));
     };
     // wait until at most `tiles` of the most recently issued K-steps' loads are still in flight
     auto wait_tiles = [&](int tiles) {
@@ -158,7 +170,8 @@ __device__ __forceinline__ void gemm_small_tile_body(
         if constexpr (kScaled) {
             // the lane's scale bytes: row 16 f + r of the wave's patch, byte g of each half's dword
             const int ktg = kt0 + kt;
-            const uint32_t sbase = lds0 + kScaleBase + (uint32_t)((ktg >> 1) & 3) * kScaleSlot + (uint32_t)(ktg & 1) * 8u + r * 16u;
+            const uint32_t sbase = lds0 + kScaleBase + (uint32_t)((ktg >> 1) & 3) * kScaleSlot + (uint32_t)(ktg & 1) * 8u + r * 16u +
+                                   ((ktg >> 1) == sc.tail_pair ? (uint32_t)sc.tail_shift : 0u);
             const uint32_t sh = 8u * g;
             v2i bs[NT];
 #pragma unroll
@@ -234,29 +247,50 @@ static __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* 
 }
 
 // Which tile a GEMM gets when the caller does not pin a kernel: 256 (the large-tile kernels), 128 or
-// 64. The rule is the largest tile that still gives every CU of an MI355X work: 64x64 tiles (two
-// workgroups per CU) when 128x128 tiles number at most 128, else 128x128 tiles below 128 tiles of
-// 256x256. Two corrections measured on a grid of 110 shapes per format (M 16..8192, N and K
-// 1024..14336), in K-steps of the format's kernels (nk):
-//  - with exactly 128 large tiles and a K of at most `short_nk` steps the 128x128 tile is 2-10 % faster
-//    (prologue and epilogue are a large share of so short a loop, and 512 small tiles overlap them);
-//  - from `long_tiles` large tiles on, a K of at least `long_nk` steps runs 3-15 % faster on the
-//    large-tile kernel although some CUs idle: its K loop moves half the LDS bytes per flop
-//    (long_tiles 0: never, the format's two kernels tie there).
+// 64. Two layers:
+//  1. a rule: the largest tile that still gives every CU of the device work: 64x64 tiles (two workgroups per
+//     CU) when 128x128 tiles number at most half the CUs, else 128x128 tiles below that many tiles of
+//     256x256, with two corrections measured on an MI355X, in K-steps of the format's kernels (nk):
+//      - with exactly CUs / 2 large tiles and a K of at most `short_nk` steps the 128x128 tile is 2-10 % faster
+//        (prologue and epilogue are a large share of so short a loop, and four times as many tiles overlap them);
+//      - from `long_tiles` large tiles on (scaled with the CU count), a K of at least `long_nk` steps runs
+//        3-15 % faster on the large-tile kernel although some CUs idle: its K loop moves half the LDS bytes
+//        per flop (long_tiles 0: never, the format's two kernels tie there);
+//  2. a generated table of the shapes on which a sweep found the rule's choice more than a few percent behind
+//     another tile (tile_table.inc, written by `python -m hipkittens_amd.tile_sweep FORMAT --emit`; the
+//     counterpart of the reference's per-shape analysis/baselines/gemm/utils/tuned.yaml). An entry is keyed by
+//     the format, the numbers of 64-row / 64-column blocks of M and N and the K-step count, and applies on
+//     devices with the CU count the sweep ran on.
 struct TileRule {
     int short_nk, long_nk, long_tiles;
 };
-static inline int pick_tile(int M, int N, int nk, TileRule r) {
+enum TileFormat { kFmtFp8 = 0, kFmtBf16 = 1, kFmtMxfp4 = 2 };
+struct TileTableEntry { unsigned char fmt; unsigned short m64, n64, nk, tile; };
+#include "tile_table.inc"   // kTileTableCus, kTileTable[]
+
+int moe_num_compute_units();  // number of CUs of the current device, cached (moe_mxfp4.hip)
+
+static inline int pick_tile_rule(int M, int N, int nk, TileRule r, int cus) {
+    const long long half = cus / 2;
     const long long tiles256 = (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     const long long tiles128 =
         (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
-    if (tiles128 <= 128) return kTinyTile;
-    if (tiles256 > 128) return BM;
-    if (tiles256 == 128) return nk <= r.short_nk ? kSmallTile : BM;
-    return r.long_tiles > 0 && tiles256 >= r.long_tiles && nk >= r.long_nk ? BM : kSmallTile;
+    if (tiles128 <= half) return kTinyTile;
+    if (tiles256 > half) return BM;
+    if (tiles256 == half) return nk <= r.short_nk ? kSmallTile : BM;
+    return r.long_tiles > 0 && tiles256 * 256 >= (long long)r.long_tiles * cus && nk >= r.long_nk ? BM : kSmallTile;
 }
-
-int moe_num_compute_units();  // number of CUs of the current device, cached (moe_mxfp4.hip)
+static inline int pick_tile(int fmt, int M, int N, int nk, TileRule r, bool consult_table = true) {
+    const int cus = moe_num_compute_units();   // 256 when no device can be queried
+    if (consult_table && cus == kTileTableCus) {
+        const long long m64 = ((long long)M + 63) / 64, n64 = ((long long)N + 63) / 64;
+        for (const TileTableEntry& e : kTileTable)
+            if (e.fmt == fmt && e.m64 == m64 && e.n64 == n64 && e.nk == nk) return e.tile;
+    }
+    return pick_tile_rule(M, N, nk, r, cus);
+}
+// the formats' rules (K-steps: 128 bytes of an operand row)
+constexpr TileRule kTileRuleFp8{16, 32, 80}, kTileRuleBf16{32, 64, 96}, kTileRuleMxfp4{8, 0, 0};
 
 // Number of K ranges the split-K path would use: as many as fill the CUs, each at least 4
 // K-steps long, at most 16; 1 = the problem has enough tiles or too short a K.

@@ -17,6 +17,14 @@
 // come in as few loads as possible: 2 per wave and pair of K-steps). They are read back with
 // one ds_read_b64 per fragment and K-step; a per-lane shift moves byte g into the position the
 // MFMA reads.
+//
+// Scale rows of any pitch and alignment (dense [rows, K / 32] rows for any K): a global->LDS load takes
+// a source address of any byte alignment, so the only special case is the last pair of K-steps of a
+// row that does not hold whole groups of 16 scale bytes. Its fetch would run past the end of the row
+// and, for the last row of the array, past the array. That pair is fetched `tail_shift` (0..3) bytes
+// early, so that a dword of the fetch ends exactly at the end of the row's scales: the dwords behind
+// it are out of the descriptor's range for the last row (nothing is fetched, zeros land in LDS) and
+// belong to K blocks past K otherwise; the readers add the same shift to their LDS address.
 #include "gemm_tile.h"
 #include "gemm_small_tile.h"
 #include "gemm_pingpong.h"
@@ -43,7 +51,7 @@ template <bool EDGE>
 __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
     const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int sa_pitch,
-    int sb_pitch, int tiles_m, int tiles_n, int band_n) {
+    int sb_pitch, int tiles_m, int tiles_n, int band_n, int tail_pair, int tail_shift, int scale_row_bytes) {
     constexpr int NW = 4, TM = 128, TN = 128, MT = 8, NT = 8;
     constexpr int NDMA = kTileBytes / (NW * 1024);
     constexpr int PG = 4, AD = 3;
@@ -64,8 +72,8 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     const int a_rows = min(M - row0, BM), b_rows = min(N - col0, BN);
     const v4i srd_a = make_srd(A + (size_t)row0 * Kb, (uint32_t)a_rows * (uint32_t)Kb);
     const v4i srd_b = make_srd(B + (size_t)col0 * Kb, (uint32_t)b_rows * (uint32_t)Kb);
-    const v4i srd_sa = make_srd(SA + (size_t)row0 * sa_pitch, (uint32_t)a_rows * (uint32_t)sa_pitch);
-    const v4i srd_sb = make_srd(SB + (size_t)col0 * sb_pitch, (uint32_t)b_rows * (uint32_t)sb_pitch);
+    const v4i srd_sa = make_srd(SA + (size_t)row0 * sa_pitch, scale_rows_bytes(a_rows, sa_pitch, scale_row_bytes));
+    const v4i srd_sb = make_srd(SB + (size_t)col0 * sb_pitch, scale_rows_bytes(b_rows, sb_pitch, scale_row_bytes));
 
     // operand tiles: as in the FP8 kernel
     uint32_t voff_a[EDGE ? NDMA : 1], voff_b[EDGE ? NDMA : 1];
@@ -111,7 +119,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     // this wave's scale load of operand `op` for the pair of K-steps `pair` (stage pair % 2)
     auto dma_scale = [&](int op, uint32_t pair, v4i srd) {
         const uint32_t dst = lds_scale_wave + (pair & 1u) * kScaleStageBytes + op * kScaleTileBytes;
-        dma16(srd, dst, op ? voff_sb : voff_sa, pair * 16u);
+        dma16(srd, dst, op ? voff_sb : voff_sa, pair * 16u - ((int)pair == tail_pair ? (uint32_t)tail_shift : 0u));
     };
 
     const uint32_t r = lane & 15, g = lane >> 4;
@@ -191,8 +199,10 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
         if (kt + 2 >= nk) { sa.z = 0; sb.z = 0; ssa.z = 0; ssb.z = 0; }
         const uint32_t vor = kt + 2 == nk - 1 ? tail_or : 0u;
         // scales of the next K-step: same pair (P == 0) or the next pair, in the other stage
-        const uint32_t sa_nx = P ? sa_rd ^ kScaleStageBytes : sa_rd;
-        const uint32_t sb_nx = P ? sb_rd ^ kScaleStageBytes : sb_rd;
+        // (entering the pair that was fetched tail_shift bytes early: see the head of the file)
+        const uint32_t early = P && ((kt + 1) >> 1) == tail_pair ? (uint32_t)tail_shift : 0u;
+        const uint32_t sa_nx = P ? (sa_rd ^ kScaleStageBytes) + early : sa_rd;
+        const uint32_t sb_nx = P ? (sb_rd ^ kScaleStageBytes) + early : sb_rd;
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             // first the 8 MFMAs on the low K-half (MX block g), then the 8 on the high half
@@ -329,15 +339,37 @@ template <int TILE, int STAGES, bool EDGE, bool SPLIT = false>
 __global__ __launch_bounds__(256) void mxfp4_gemm_small_tile_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
     const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int sa_pitch,
-    int sb_pitch, int tiles_m, int tiles_n, int kps, float* __restrict__ partial) {
+    int sb_pitch, int tiles_m, int tiles_n, int kps, float* __restrict__ partial, int tail_pair, int tail_shift,
+    int scale_row_bytes) {
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
-    gemm_small_tile_body<Mxfp4Mma, TILE, STAGES, EDGE, SPLIT>(smem, A, B, C, M, N, K, 1.0f, tiles_m, tiles_n, kps,
-                                                              partial, SmallTileScales{SA, SB, sa_pitch, sb_pitch});
+    gemm_small_tile_body<Mxfp4Mma, TILE, STAGES, EDGE, SPLIT>(
+        smem, A, B, C, M, N, K, 1.0f, tiles_m, tiles_n, kps, partial,
+        SmallTileScales{SA, SB, sa_pitch, sb_pitch, tail_pair, tail_shift, scale_row_bytes});
+}
+
+// What the tile kernels need to know about the scale rows (see the head of the file).
+// ok: the tile kernels can take these rows; tail_pair / tail_shift: the pair of K-steps fetched early and by how
+// many bytes (-1 / 0: none); row_bytes: what the scale descriptors cover of an operand's last row (0: its pitch).
+struct Mxfp4ScaleRows { bool ok; int tail_pair, tail_shift, row_bytes; };
+static Mxfp4ScaleRows mxfp4_scale_rows(int K, int sa_pitch, int sb_pitch) {
+    const int nb = K / 32;                       // scale bytes of a row
+    const int groups = (nb + 7) / 8 * 8;
+    if (sa_pitch < nb || sb_pitch < nb) return {false, -1, 0, 0};
+    // rows padded to whole groups of 8 bytes: a pair's fetch stays inside the row or ends on a dword of it
+    if ((sa_pitch % 8) == 0 && (sb_pitch % 8) == 0 && sa_pitch >= groups && sb_pitch >= groups) return {true, -1, 0, 0};
+    // any other pitch: nothing past a row's nb bytes is relied on, and the last row ends there. Rows of fewer than
+    // 16 bytes (K < 512) stay with the portable kernel: the early fetch would start in front of the first row, and
+    // the fetch of a row before the last could reach across the last one to the end of the array.
+    if (nb < 16) return {false, -1, 0, 0};
+    const int shift = (4 - nb % 4) % 4;
+    if ((nb % 16) == 0 || shift == 0) return {true, -1, 0, nb};
+    return {true, (nb - 1) / 16, shift, nb};
 }
 
 template <int TILE, int STAGES, bool EDGE>
 static int launch_mxfp4_small_tile(const void* A, const void* SA, const void* B, const void* SB, void* C,
-                                   int M, int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
+                                   int M, int N, int K, int sa_pitch, int sb_pitch, Mxfp4ScaleRows sr,
+                                   hipStream_t stream) {
     auto kern = mxfp4_gemm_small_tile_kernel<TILE, STAGES, EDGE>;
     constexpr int lds_bytes = small_tile_lds_bytes<TILE, STAGES>(true);
     static DeviceOnce configured;
@@ -345,7 +377,8 @@ static int launch_mxfp4_small_tile(const void* A, const void* SA, const void* B,
     const int tiles_m = (M + TILE - 1) / TILE, tiles_n = (N + TILE - 1) / TILE;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream, (const uint8_t*)A,
                        (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB, (uint16_t*)C, M, N, K / 2,
-                       sa_pitch, sb_pitch, tiles_m, tiles_n, 0, (float*)nullptr);
+                       sa_pitch, sb_pitch, tiles_m, tiles_n, 0, (float*)nullptr, sr.tail_pair, sr.tail_shift,
+                       sr.row_bytes);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
@@ -368,7 +401,8 @@ static int mxfp4_splitk_ranges(int M, int N, int K) {
 }
 template <bool EDGE>
 static int launch_mxfp4_splitk(const void* A, const void* SA, const void* B, const void* SB, void* C, int M, int N,
-                               int K, int sa_pitch, int sb_pitch, int splits, float* partial, hipStream_t stream) {
+                               int K, int sa_pitch, int sb_pitch, Mxfp4ScaleRows sr, int splits, float* partial,
+                               hipStream_t stream) {
     auto kern = mxfp4_gemm_small_tile_kernel<kTinyTile, kTinyStages, EDGE, true>;
     constexpr int lds_bytes = small_tile_lds_bytes<kTinyTile, kTinyStages>(true);
     static DeviceOnce configured;
@@ -379,7 +413,7 @@ static int launch_mxfp4_splitk(const void* A, const void* SA, const void* B, con
     const int used = (nk + kps - 1) / kps;   // ranges that hold at least one K-step
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, used), dim3(256), lds_bytes, stream, (const uint8_t*)A,
                        (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB, (uint16_t*)C, M, N, K / 2,
-                       sa_pitch, sb_pitch, tiles_m, tiles_n, kps, partial);
+                       sa_pitch, sb_pitch, tiles_m, tiles_n, kps, partial, sr.tail_pair, sr.tail_shift, sr.row_bytes);
     const long long mn = (long long)M * N;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((mn / 4 + 256) / 256)), dim3(256), 0, stream,
                        (const float*)partial, used, mn, 1.0f, (uint16_t*)C);
@@ -413,7 +447,7 @@ static int launch_mxfp4_pingpong(const void* A, const void* SA, const void* B, c
 
 template <bool EDGE>
 static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, const void* SB, void* C,
-                              int M, int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
+                              int M, int N, int K, int sa_pitch, int sb_pitch, Mxfp4ScaleRows sr, hipStream_t stream) {
     auto kern = mxfp4_gemm_4wave_kernel<EDGE>;
     static DeviceOnce configured;
     if (!set_lds_limit_once((const void*)kern, kLdsBytesFp4, configured)) return HK_ERR_LAUNCH;
@@ -421,7 +455,7 @@ static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, cons
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), kLdsBytesFp4, stream,
                        (const uint8_t*)A, (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB,
                        (uint16_t*)C, M, N, K, sa_pitch, sb_pitch, tiles_m, tiles_n,
-                       raster_band(((long long)M + N) * (K / 2), tiles_n));
+                       raster_band(((long long)M + N) * (K / 2), tiles_n), sr.tail_pair, sr.tail_shift, sr.row_bytes);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
@@ -439,16 +473,13 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
         return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
     if (variant < -1 || variant > 4) return HK_ERR_UNSUPPORTED;
-    // the tile kernel fetches a row's scales 16 bytes per lane, two K-steps of 8 bytes at a time:
-    // rows must start 4-byte aligned and hold whole groups of 8 bytes
-    const int groups = (K / 32 + 7) / 8 * 8;
-    const bool pitch_ok = (sa_pitch % 8) == 0 && (sb_pitch % 8) == 0 && sa_pitch >= groups && sb_pitch >= groups &&
-                          ((((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) == 0);
+    // what the tile kernels need of the scale rows (any pitch and alignment; see mxfp4_scale_rows)
+    const Mxfp4ScaleRows sr = mxfp4_scale_rows(K, sa_pitch, sb_pitch);
     const bool size_ok = (long long)(K / 2) * BM < (1ll << 31) && (long long)BM * max(sa_pitch, sb_pitch) < (1ll << 31);
     if (variant < 0) {
         // the choice of tile of hk_fp8_gemm (pick_tile); a K-step is 256 elements here
-        const int tile = pick_tile(M, N, (K / 2 + BK - 1) / BK, TileRule{8, 0, 0});
-        variant = !(pitch_ok && size_ok) ? 0 : tile == kTinyTile ? 3 : tile == kSmallTile ? 2 : 1;
+        const int tile = pick_tile(kFmtMxfp4, M, N, (K / 2 + BK - 1) / BK, kTileRuleMxfp4);
+        variant = !(sr.ok && size_ok) ? 0 : tile == kTinyTile ? 3 : tile == kSmallTile ? 2 : 1;
     }
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {
@@ -459,25 +490,27 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
                            (uint16_t*)C, M, N, K, sa_pitch, sb_pitch);
         return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
     }
-    if (!size_ok || (sa_pitch % 8) != 0 || (sb_pitch % 8) != 0 || sa_pitch < groups || sb_pitch < groups)
-        return HK_ERR_BAD_SHAPE;
-    if (((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) return HK_ERR_BAD_ALIGNMENT;
+    if (!size_ok || !sr.ok) return HK_ERR_BAD_SHAPE;
     if (variant == 2) {
         const bool e = (M % kSmallTile) != 0 || (N % kSmallTile) != 0;
-        return e ? launch_mxfp4_small_tile<kSmallTile, kSmallStages, true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s)
-                 : launch_mxfp4_small_tile<kSmallTile, kSmallStages, false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
+        return e ? launch_mxfp4_small_tile<kSmallTile, kSmallStages, true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, sr, s)
+                 : launch_mxfp4_small_tile<kSmallTile, kSmallStages, false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, sr, s);
     }
     if (variant == 3) {
         const bool e = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
-        return e ? launch_mxfp4_small_tile<kTinyTile, kTinyStages, true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s)
-                 : launch_mxfp4_small_tile<kTinyTile, kTinyStages, false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
+        return e ? launch_mxfp4_small_tile<kTinyTile, kTinyStages, true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, sr, s)
+                 : launch_mxfp4_small_tile<kTinyTile, kTinyStages, false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, sr, s);
     }
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
-    if (variant == 4)
+    if (variant == 4) {
+        // the ping-pong kernel keeps the padded-row form (rows of whole groups of 8 scale bytes)
+        if (sr.row_bytes != 0) return HK_ERR_BAD_SHAPE;
+        if (((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) return HK_ERR_BAD_ALIGNMENT;
         return edge ? launch_mxfp4_pingpong<true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s)
                     : launch_mxfp4_pingpong<false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
-    return edge ? launch_mxfp4_4wave<true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s)
-                : launch_mxfp4_4wave<false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
+    }
+    return edge ? launch_mxfp4_4wave<true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, sr, s)
+                : launch_mxfp4_4wave<false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, sr, s);
 }
 
 extern "C" int hk_mxfp4_gemm_variant(const void* A, const void* A_scales, const void* B,
@@ -504,12 +537,9 @@ extern "C" int hk_mxfp4_gemm_ws(const void* A, const void* A_scales, int a_scale
     using namespace hk;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 32) != 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     const int splits = mxfp4_splitk_ranges(M, N, K);
-    const int groups = (K / 32 + 7) / 8 * 8;
     // what the tile kernels need of the scale rows (see mxfp4_gemm_impl); anything else takes the plain path
-    const bool tile_ok = (a_scale_pitch % 8) == 0 && (b_scale_pitch % 8) == 0 && a_scale_pitch >= groups &&
-                         b_scale_pitch >= groups && A_scales && B_scales &&
-                         ((((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) == 0) &&
-                         (long long)(K / 2) * BM < (1ll << 31) &&
+    const Mxfp4ScaleRows sr = mxfp4_scale_rows(K, a_scale_pitch, b_scale_pitch);
+    const bool tile_ok = sr.ok && A_scales && B_scales && (long long)(K / 2) * BM < (1ll << 31) &&
                          (long long)BM * max(a_scale_pitch, b_scale_pitch) < (1ll << 31);
     const bool can_split = splits >= 2 && workspace && workspace_bytes >= (size_t)splits * M * N * sizeof(float) &&
                            tile_ok && (long long)M * N < (1ll << 40);
@@ -518,9 +548,9 @@ extern "C" int hk_mxfp4_gemm_ws(const void* A, const void* A_scales, int a_scale
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)workspace) & 15u) return HK_ERR_BAD_ALIGNMENT;
     const bool edge = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
-    return edge ? launch_mxfp4_splitk<true>(A, A_scales, B, B_scales, C, M, N, K, a_scale_pitch, b_scale_pitch, splits,
-                                            (float*)workspace, (hipStream_t)stream)
-                : launch_mxfp4_splitk<false>(A, A_scales, B, B_scales, C, M, N, K, a_scale_pitch, b_scale_pitch,
+    return edge ? launch_mxfp4_splitk<true>(A, A_scales, B, B_scales, C, M, N, K, a_scale_pitch, b_scale_pitch, sr,
+                                            splits, (float*)workspace, (hipStream_t)stream)
+                : launch_mxfp4_splitk<false>(A, A_scales, B, B_scales, C, M, N, K, a_scale_pitch, b_scale_pitch, sr,
                                              splits, (float*)workspace, (hipStream_t)stream);
 }
 

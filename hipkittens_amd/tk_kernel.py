@@ -44,6 +44,18 @@ def _stream(t) -> int:
 _FP8 = (torch.float8_e4m3fn, torch.uint8)
 
 
+def gemm_tile_choice(fmt: str, M: int, N: int, K: int, consult_table: bool = True) -> int:
+    """Tile (256, 128 or 64) the library picks for a GEMM of format "fp8", "bf16" or "mxfp4" on the current
+    device; consult_table False: the rule alone, without the generated per-shape table (tile_sweep.py)."""
+    code = {"fp8": 0, "bf16": 1, "mxfp4": 2}.get(fmt)
+    if code is None:
+        raise RuntimeError(f"unknown GEMM format {fmt!r}")
+    tile = int(_lib.load_library().hk_gemm_tile_choice(code, int(M), int(N), int(K), 1 if consult_table else 0))
+    if tile < 0:
+        _lib.check(tile, "gemm_tile_choice")
+    return tile
+
+
 def fp8_gemm_workspace_bytes(M: int, N: int, K: int) -> int:
     """Bytes of workspace with which dispatch_fp8_gemm splits K for this shape (0: it would not)."""
     return int(_lib.load_library().hk_fp8_gemm_workspace_bytes(int(M), int(N), int(K)))

@@ -37,6 +37,13 @@ const char* hk_status_string(int status);
 /* Library version, e.g. 100 = 0.1.0 (no reference counterpart). */
 int hk_version(void);
 
+/* Tile (256, 128 or 64) that hk_fp8_gemm / hk_bf16_gemm / hk_mxfp4_gemm (format 0 / 1 / 2) pick for a shape
+ * on the current device when the tile kernels can take it; consult_table 0: the rule alone, without the
+ * generated per-shape table (what the sweep that writes the table compares against). Negative: a status.
+ * Counterpart of the reference's per-shape solution selection
+ * (analysis/baselines/gemm/utils/solution_selection.py, tuned.yaml). */
+int hk_gemm_tile_choice(int format, int M, int N, int K, int consult_table);
+
 /*
  * FP8 e4m3 (OCP e4m3fn) GEMM:  C[M,N] = bf16( (scale_a*scale_b) * sum_k A[m,k]*B[n,k] ).
  * A is [M,K] row-major, B is [N,K] row-major ("column-major B"), both 1 byte per

@@ -159,3 +159,31 @@ def test_device_independent_quantizers_match_oracle_on_cpu():
     q, sc = hk.quant.quantize_fp8_per_tensor(torch.from_numpy(x))
     qo, sco = F.quantize_e4m3_per_tensor(x)
     assert np.float32(sc) == sco and np.array_equal(q.view(torch.uint8).numpy(), qo)
+
+
+def test_tile_choice_rule_and_generated_table():
+    """The choice of GEMM tile (no GPU needed: without a device the library assumes 256 CUs, the count the
+    committed table was measured on): the rule's landmarks, and every entry of csrc/tile_table.inc is what
+    the default entry points would pick for a shape with the entry's key."""
+    tk = hk.tk_kernel
+    for fmt in ("fp8", "bf16", "mxfp4"):
+        assert tk.gemm_tile_choice(fmt, 8192, 8192, 8192, False) == 256     # 1024 large tiles
+        assert tk.gemm_tile_choice(fmt, 1024, 1024, 1024, False) == 64      # 64 tiles of 128 x 128
+        assert tk.gemm_tile_choice(fmt, 2048, 4096, 1024, False) == 128     # 128 large tiles, short K
+        assert tk.gemm_tile_choice(fmt, 16, 8192, 8192, False) == 64
+    assert tk.gemm_tile_choice("fp8", 2048, 2560, 8192, False) == 256       # 80 large tiles, long K
+    assert tk.gemm_tile_choice("mxfp4", 2048, 2560, 16384, False) == 128    # (no such correction for MXFP4)
+    with pytest.raises(RuntimeError):
+        tk.gemm_tile_choice("fp8", 0, 8, 8)
+    text = open(os.path.join(ROOT, "hipkittens_amd", "csrc", "tile_table.inc")).read()
+    assert re.search(r"kTileTableCus = 256;", text)
+    entries = [tuple(int(x) for x in m.groups()) for m in re.finditer(r"\{(\d+), (\d+), (\d+), (\d+), (\d+)\},", text)]
+    entries = [e for e in entries if e[0] != 255]
+    assert entries and len(set(e[:4] for e in entries)) == len(entries)     # one tile per key
+    k_per_step = {0: 128, 1: 64, 2: 256}
+    for code, m64, n64, nk, tile in entries:
+        assert tile in (256, 128, 64)
+        fmt = ("fp8", "bf16", "mxfp4")[code]
+        M, N, K = 64 * m64 - 5, 64 * n64, nk * k_per_step[code]
+        assert tk.gemm_tile_choice(fmt, M, N, K) == tile
+        assert tk.gemm_tile_choice(fmt, M, N, K, False) != tile             # an entry that repeats the rule is noise

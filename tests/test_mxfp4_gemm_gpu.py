@@ -60,10 +60,79 @@ def test_mxfp4_gemm_k_not_multiple_of_256(hk, variant):
 
 
 def test_mxfp4_gemm_tile_kernel_rejects_k_tail(hk):
+    """Dense scale rows of fewer than 16 bytes (K < 512) that are not whole groups of 8: portable kernel only."""
     rng = np.random.default_rng(7)
     (a, sa), (b, sb) = _rand_mx(rng, 64, 160), _rand_mx(rng, 64, 160)
     with pytest.raises(RuntimeError):
         _run(hk, a, sa, b, sb, 1)
+
+
+def _run_in_pool(hk, a, sa, b, sb, variant, misalign, workspace=False):
+    """The GEMM with every operand array surrounded by bytes 0xFF (a scale byte fetched in front of or behind an
+    array would be the e8m0 NaN) and the scale arrays starting `misalign` bytes off a 16-byte boundary."""
+    dev = torch.device("cuda:0")
+    views, pools = [], []
+    for arr, mis in ((a, 0), (sa, misalign), (b, 0), (sb, misalign)):
+        pool = torch.full((16 + mis + arr.size + 64,), 0xFF, dtype=torch.uint8, device=dev)
+        view = pool[16 + mis:16 + mis + arr.size].view(arr.shape)
+        view.copy_(torch.from_numpy(arr).to(dev))
+        assert view.data_ptr() % 16 == mis
+        pools.append(pool)
+        views.append(view)
+    A, SA, B, SB = views
+    C = torch.full((a.shape[0], b.shape[0]), float("nan"), dtype=torch.bfloat16, device=dev)
+    ws = None
+    if workspace:
+        need = hk.tk_kernel.mxfp4_gemm_workspace_bytes(a.shape[0], b.shape[0], a.shape[1] * 2)
+        assert need > 0
+        ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    hk.tk_kernel.dispatch_mxfp4_gemm(A, SA, B, SB, C, variant=variant, workspace=ws)
+    torch.cuda.synchronize()
+    return C.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+# K / 32 scale bytes per row, dense rows: 90 (the GPT-OSS hidden size, tail fetched 2 bytes early), and one case
+# for each remainder of K / 32 modulo 4 and for rows of whole and broken groups of 16
+DENSE_RAGGED = [(512, 2880, 2880), (300, 200, 2880), (130, 520, 32 * 17), (257, 255, 32 * 19), (64, 384, 32 * 20),
+                (96, 80, 32 * 47), (256, 256, 32 * 33), (200, 136, 32 * 18)]
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3, -1])
+@pytest.mark.parametrize("shape", DENSE_RAGGED)
+def test_mxfp4_gemm_dense_scale_rows_any_k_on_the_tile_kernels(hk, shape, variant):
+    """Dense [rows, K / 32] scale rows with K / 32 not a multiple of 8 (rows of any byte alignment) run on every
+    tile kernel: same bits as the call with rows padded to a multiple of 8 bytes, oracle-close, and nothing past
+    the arrays is fetched."""
+    M, N, K = shape
+    print(f"mxfp4_gemm dense ragged shape={shape} variant={variant}", flush=True)
+    rng = np.random.default_rng(3 + M + N + K)
+    (a, sa), (b, sb) = _rand_mx(rng, M, K), _rand_mx(rng, N, K)
+    ref = G.mxfp4_gemm(a, sa, b, sb)
+    for mis in (0, 1, 3):
+        bits = _run_in_pool(hk, a, sa, b, sb, variant, mis)
+        out = F.bf16_to_f32(bits)
+        assert np.isfinite(out).all(), (shape, variant, mis)
+        assert G.rel_fro_error(out, ref) <= 5e-3, (shape, variant, mis)
+        if mis == 0:
+            first = bits
+        assert np.array_equal(bits, first), (shape, variant, mis)
+    pitch = (K // 32 + 7) // 8 * 8
+    padded = _run(hk, a, _pad_rows(rng, sa, pitch), b, _pad_rows(rng, sb, pitch))   # picks the same tile
+    if variant == -1:
+        assert np.array_equal(first, padded)
+        # ... and it is the tile kernel of the library's choice of tile, not the portable kernel
+        forced = {256: 1, 128: 2, 64: 3}[hk.tk_kernel.gemm_tile_choice("mxfp4", M, N, K)]
+        assert np.array_equal(first, _run_in_pool(hk, a, sa, b, sb, forced, 0))
+
+
+def test_mxfp4_gemm_dense_scale_rows_split_k(hk):
+    """The split-K path on dense scale rows whose last pair of K-steps is fetched early (K / 32 = 263)."""
+    M, N, K = 16, 1024, 32 * 263
+    rng = np.random.default_rng(21)
+    (a, sa), (b, sb) = _rand_mx(rng, M, K), _rand_mx(rng, N, K)
+    out = F.bf16_to_f32(_run_in_pool(hk, a, sa, b, sb, -1, 1, workspace=True))
+    assert np.isfinite(out).all()
+    assert G.rel_fro_error(out, G.mxfp4_gemm(a, sa, b, sb)) <= 5e-3
 
 
 @pytest.mark.parametrize("variant", [0, 1])
@@ -130,7 +199,7 @@ def test_mxfp4_gemm_padded_scale_rows_and_k_tails(hk, case):
     """Scale rows padded to a pitch (a multiple of 8 bytes keeps any K % 32 == 0 on the tile kernel:
     the last K-step's bytes past the row end are not fetched; the operand buffers sit at the end of
     a pool filled with 0xFF so that a fetch past the row would show). The last case has a pitch that
-    is not a multiple of 8 and takes the portable kernel."""
+    is not a multiple of 8: its last pair of K-steps is fetched two bytes early."""
     M, N, K, pa, pb = case
     print(f"mxfp4_gemm pitched case={case}", flush=True)
     rng = np.random.default_rng(11 + M + N + K)
