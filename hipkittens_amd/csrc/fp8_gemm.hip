@@ -243,7 +243,7 @@ static std::atomic<void*> scratch_ptr[64];
 static int static_scratch(void** out) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return HK_ERR_LAUNCH;
-    if (dev < 0 || dev >= 64) return HK_ERR_UNSUPPORTED;
+    if (dev < 0 || dev >= 64) return HK_ERR_UNSUPPORTED;   // (the caller then runs without a split)
     void* p = scratch_ptr[dev].load(std::memory_order_acquire);
     if (!p) {
         if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return HK_ERR_LAUNCH;
@@ -262,10 +262,17 @@ extern "C" int hk_fp8_gemm_static_ws(const void* A, const void* B, void* C, int 
     if (M <= 0 || N <= 0 || K <= 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     const int splits = splitk_ranges(M, N, K);
     if (splits < 2) return hk_fp8_gemm(A, B, C, M, N, K, scale_a, scale_b, stream);   // no scratch needed
+    // splitk_ranges gives at most two workgroups per CU, 16 KiB of partial sums each: the array covers devices
+    // of up to 256 CUs; a larger device can ask for more, which is refused (the caller then uses hk_fp8_gemm_ws
+    // or hk_fp8_gemm)
+    static_assert(kStaticScratchBytes == (size_t)2 * 256 * kTinyTile * kTinyTile * sizeof(float), "512 workgroups' partial sums");
     const size_t need = (size_t)splits * M * N * sizeof(float);
     if (need > kStaticScratchBytes) return HK_ERR_WORKSPACE;   // more partial sums than the array holds
     void* ws = nullptr;
     const int st = static_scratch(&ws);
+    // a device ordinal this table does not cover: the same result without a split, as hk_fp8_gemm_ws does
+    // without a workspace
+    if (st == HK_ERR_UNSUPPORTED) return hk_fp8_gemm(A, B, C, M, N, K, scale_a, scale_b, stream);
     if (st != HK_OK) return st;
     // every partial sum that the reduction reads is written by this call's first kernel: nothing in
     // the array needs clearing between calls

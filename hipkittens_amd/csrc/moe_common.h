@@ -49,6 +49,9 @@ inline bool moe_rows_fit_one_item(int T, int k, int E, int bm) {
 constexpr size_t kMoeWsTail = 32768;
 // Number of CUs of the current device (cached per device ordinal).
 int moe_num_compute_units();
+// Shape check of hk_moe_topk_grouped_sigmoid (moe_routing.hip), for entry points that launch other work in
+// front of the routing: HK_OK or HK_ERR_BAD_SHAPE.
+int moe_topk_grouped_sigmoid_check(int T, int E, int k, int n_group, int topk_group);
 // Item lists of the two grouped GEMMs of a layer from expert_offsets [E+1], m-tiles of up to `bm`
 // rows: items1 / num_items[0] for n_tiles_n1 tiles of weight rows, items2 / num_items[1] for
 // n_tiles_n2 (one launch).

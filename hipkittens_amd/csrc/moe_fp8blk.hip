@@ -989,6 +989,24 @@ static int fp8blk_check(int T, int H, int I, int E, int k) {
     return HK_OK;
 }
 
+// Every argument check of the expert MLP, made before the first launch of a call (the forward entry points run
+// quantization, routing and sort in front of the expert GEMMs: a call that is going to be refused must not have
+// started any of them). x_e4m3 / x_scales: the caller's, or where the bf16 entry point will put them.
+static int fp8blk_validate(const void* x_e4m3, const void* x_scales, const void* w13, const void* w13_scales,
+                           const void* w2, const void* w2_scales, const void* y_bf16, int T, int H, int I, int E,
+                           int k, int weight_layout, const void* y_add, const void* workspace,
+                           size_t workspace_bytes) {
+    if (weight_layout < 0 || weight_layout > 1) return HK_ERR_UNSUPPORTED;
+    if (!x_e4m3 || !x_scales || !w13 || !w13_scales || !w2 || !w2_scales || !y_bf16) return HK_ERR_NULL_POINTER;
+    const int st = fp8blk_check(T, H, I, E, k);
+    if (st != HK_OK) return st;
+    if (!workspace || workspace_bytes < fp8_ws_layout(T, H, I, E, k).total) return HK_ERR_WORKSPACE;
+    if (((uintptr_t)x_e4m3 | (uintptr_t)w13 | (uintptr_t)w2 | (uintptr_t)y_bf16 | (uintptr_t)workspace |
+         (uintptr_t)y_add) & 15u)
+        return HK_ERR_BAD_ALIGNMENT;
+    return HK_OK;
+}
+
 }  // namespace hk
 
 using namespace hk;
@@ -1037,16 +1055,11 @@ extern "C" int hk_moe_fp8blk_experts_ex2(const void* x_e4m3, const float* x_scal
                                          int T, int H, int I, int E, int k, int weight_layout,
                                          const void* y_add_bf16_or_null, void* workspace, size_t workspace_bytes,
                                          void* stream) {
-    if (weight_layout < 0 || weight_layout > 1) return HK_ERR_UNSUPPORTED;
-    if (!x_e4m3 || !x_scales || !w13 || !w13_scales || !w2 || !w2_scales || !topk_w || !sorted_slots ||
-        !expert_offsets || !slot_to_pos || !y_bf16)
-        return HK_ERR_NULL_POINTER;
-    int st = fp8blk_check(T, H, I, E, k);
+    if (!topk_w || !sorted_slots || !expert_offsets || !slot_to_pos) return HK_ERR_NULL_POINTER;
+    int st = fp8blk_validate(x_e4m3, x_scales, w13, w13_scales, w2, w2_scales, y_bf16, T, H, I, E, k, weight_layout,
+                             y_add_bf16_or_null, workspace, workspace_bytes);
     if (st != HK_OK) return st;
     const Fp8Ws L = fp8_ws_layout(T, H, I, E, k);
-    if (!workspace || workspace_bytes < L.total) return HK_ERR_WORKSPACE;
-    if (((uintptr_t)x_e4m3 | (uintptr_t)w13 | (uintptr_t)w2 | (uintptr_t)y_bf16 | (uintptr_t)workspace) & 15u)
-        return HK_ERR_BAD_ALIGNMENT;
     hipStream_t s = (hipStream_t)stream;
     uint8_t* ws = (uint8_t*)workspace;
     const int S = T * k;
@@ -1118,10 +1131,12 @@ extern "C" int hk_moe_fp8blk_forward_ex2(const void* x_e4m3, const float* x_scal
                                          int E, int k, int weight_layout, const void* y_add_bf16_or_null,
                                          void* workspace, size_t workspace_bytes, void* stream) {
     if (!router_logits) return HK_ERR_NULL_POINTER;
-    int st = fp8blk_check(T, H, I, E, k);
+    int st = fp8blk_validate(x_e4m3, x_scales, w13, w13_scales, w2, w2_scales, y_bf16, T, H, I, E, k, weight_layout,
+                             y_add_bf16_or_null, workspace, workspace_bytes);
+    if (st != HK_OK) return st;
+    st = moe_topk_grouped_sigmoid_check(T, E, k, n_group, topk_group);
     if (st != HK_OK) return st;
     const Fp8Ws L = fp8_ws_layout(T, H, I, E, k);
-    if (!workspace || workspace_bytes < L.total) return HK_ERR_WORKSPACE;
     uint8_t* ws = (uint8_t*)workspace;
     st = hk_moe_topk_grouped_sigmoid(router_logits, router_bias_or_null, T, E, k, n_group, topk_group, routed_scale,
                                      (int32_t*)(ws + L.ids), (float*)(ws + L.w), stream);
@@ -1152,12 +1167,15 @@ extern "C" int hk_moe_fp8blk_forward_bf16(const void* x_bf16, const float* route
                                           const void* w2, const float* w2_scales, void* y_bf16, int T, int H, int I,
                                           int E, int k, int weight_layout, const void* y_add_bf16_or_null,
                                           void* workspace, size_t workspace_bytes, void* stream) {
-    if (!x_bf16) return HK_ERR_NULL_POINTER;
-    int st = fp8blk_check(T, H, I, E, k);
+    if (!x_bf16 || !router_logits) return HK_ERR_NULL_POINTER;
+    if ((uintptr_t)x_bf16 & 15u) return HK_ERR_BAD_ALIGNMENT;
+    // (the quantized copy of x and its scales will lie in the workspace: any non-null pointer stands in for them)
+    int st = fp8blk_validate(workspace, workspace, w13, w13_scales, w2, w2_scales, y_bf16, T, H, I, E, k, weight_layout,
+                             y_add_bf16_or_null, workspace, workspace_bytes);
+    if (st != HK_OK) return st;
+    st = moe_topk_grouped_sigmoid_check(T, E, k, n_group, topk_group);
     if (st != HK_OK) return st;
     const Fp8Ws L = fp8_ws_layout(T, H, I, E, k);
-    if (!workspace || workspace_bytes < L.total) return HK_ERR_WORKSPACE;
-    if ((uintptr_t)workspace & 15u) return HK_ERR_BAD_ALIGNMENT;
     uint8_t* ws = (uint8_t*)workspace;
     // every token is quantized once (T rows), ahead of the gather that repeats it for its k experts
     st = hk_fp8_quantize_rows_1x128(x_bf16, T, H, ws + L.xq, (float*)(ws + L.xs), stream);

@@ -939,7 +939,9 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
             const uint32_t voff = (uint32_t)(row_start + 8 * (4 * q + w) + (lane >> 3)) * 4u;
             uint32_t& dst = tok_nxt[q];
             const v4i rs = srd_slots;
-            asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=v"(dst) : "v"(voff), "s"(rs) : "memory");
+            // (once per item; s_nop 4: the descriptor may have been restored from a spill slot by a vector-ALU
+            // instruction directly in front of the statement)
+            asm volatile("s_nop 4\n\tbuffer_load_dword %0, %1, %2, 0 offen" : "=v"(dst) : "v"(voff), "s"(rs) : "memory");
         }
     };
     auto adopt_tokens = [&]() __attribute__((always_inline)) {
@@ -1053,14 +1055,14 @@ __global__ __launch_bounds__(256) void moe_mxfp4_stream4_kernel(const MoeGemmPar
             const uint32_t soff = (uint32_t)cf.kt * kMoeBTile + (uint32_t)(2 * w + pair) * 4096u;
             v4i rs = cf_srd_b;
             if (cf.kt >= nk) rs.z = 0;
-            // (the first weight load of an MXFP8 position starts with s_nop 4: the descriptor's size word may
-            // have been restored from a spill slot by a vector-ALU instruction directly in front of the statement)
+            // (the first weight load of a position starts with s_nop 4: the descriptor's size word may have
+            // been restored from a spill slot by a vector-ALU instruction directly in front of the statement)
 #define HK_WLOAD(PRE, POST)                                                                      \
     asm volatile(PRE "buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4" POST                   \
                  : "=v"(bw[P][f])                                                                \
                  : "v"(voff), "s"(rs), "s"(soff), "n"(((f >> 1) & 1) * 2048 + half * 1024)       \
                  : "memory")
-            if constexpr (A8 && f == 0) {
+            if constexpr (f == 0) {
                 if constexpr (NT) HK_WLOAD("s_nop 4\n\t", " nt"); else HK_WLOAD("s_nop 4\n\t", "");
             } else {
                 if constexpr (NT) HK_WLOAD("", " nt"); else HK_WLOAD("", "");
@@ -1612,30 +1614,24 @@ static bool moe_gathers(int weight_layout, bool ext, bool a8, int T, int H) {
     return weight_layout == 1 && !ext && (long long)T * H * (a8 ? 2 : 1) <= 12ll << 20;
 }
 
-// Expert MLP on already routed and sorted tokens (steps 3-6 of the forward pass). a8: MXFP8
-// activations (pre-shuffled weights only).
-static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const void* w13_scales,
-                                  int w13_scale_pitch, const void* w2, const void* w2_scales,
-                                  int w2_scale_pitch, const float* topk_w, const int32_t* sorted_slots,
-                                  const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
-                                  int T, int H, int I, int E, int k, int weight_layout,
-                                  const float* bias13, const float* bias2, int activation, float alpha,
-                                  float limit, int w13_interleaved, void* workspace,
-                                  size_t workspace_bytes, void* stream, bool a8, bool x_quantized = false) {
+// Every argument check of the expert MLP, made before the first launch of a call (the forward entry points run
+// top-k, sort and quantization in front of the expert GEMMs: a call that is going to be refused must not have
+// started any of them).
+static int moe_mxfp4_validate(const void* x_bf16, const void* w13, const void* w13_scales, int w13_scale_pitch,
+                              const void* w2, const void* w2_scales, int w2_scale_pitch, const void* y_bf16, int T,
+                              int H, int I, int E, int k, int weight_layout, const float* bias13, const float* bias2,
+                              int activation, float limit, const void* workspace, size_t workspace_bytes, bool a8) {
     if (activation != 0 && activation != 1) return HK_ERR_UNSUPPORTED;
     if (a8 && weight_layout != 1) return HK_ERR_UNSUPPORTED;
     if (activation == 1 && !(limit > 0.f)) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)bias13 | (uintptr_t)bias2) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    const bool ext = bias13 || bias2 || activation != 0 || w13_interleaved;
     // the bias arrays are addressed with 32-bit byte offsets
     if ((bias13 && (unsigned long long)E * 2 * I * 4 >= (1ull << 32)) || (bias2 && (unsigned long long)E * H * 4 >= (1ull << 32)))
         return HK_ERR_BAD_SHAPE;
-    if (!x_bf16 || !w13 || !w13_scales || !w2 || !w2_scales || !topk_w || !sorted_slots || !expert_offsets ||
-        !slot_to_pos || !y_bf16)
-        return HK_ERR_NULL_POINTER;
+    if (!x_bf16 || !w13 || !w13_scales || !w2 || !w2_scales || !y_bf16) return HK_ERR_NULL_POINTER;
     if (weight_layout != 0 && weight_layout != 1) return HK_ERR_UNSUPPORTED;
-    int st = moe_mxfp4_check(T, H, I, E, k, weight_layout ? moe_round_up(H / 32, 8) : w13_scale_pitch,
-                             weight_layout ? moe_round_up(I / 32, 8) : w2_scale_pitch);
+    const int st = moe_mxfp4_check(T, H, I, E, k, weight_layout ? moe_round_up(H / 32, 8) : w13_scale_pitch,
+                                   weight_layout ? moe_round_up(I / 32, 8) : w2_scale_pitch);
     if (st != HK_OK) return st;
     // MXFP8 activation tiles are twice as large: their 32-bit buffer offsets must still fit
     if (a8 && ((long long)T * k * ((H + 255) / 256 * 256) >= (1ll << 31) ||
@@ -1646,6 +1642,26 @@ static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const voi
     if (((uintptr_t)x_bf16 | (uintptr_t)w13 | (uintptr_t)w2 | (uintptr_t)y_bf16 | (uintptr_t)workspace) & 15u)
         return HK_ERR_BAD_ALIGNMENT;
     if (((uintptr_t)w13_scales | (uintptr_t)w2_scales) & 3u) return HK_ERR_BAD_ALIGNMENT;
+    return HK_OK;
+}
+
+// Expert MLP on already routed and sorted tokens (steps 3-6 of the forward pass). a8: MXFP8
+// activations (pre-shuffled weights only).
+static int moe_mxfp4_experts_impl(const void* x_bf16, const void* w13, const void* w13_scales,
+                                  int w13_scale_pitch, const void* w2, const void* w2_scales,
+                                  int w2_scale_pitch, const float* topk_w, const int32_t* sorted_slots,
+                                  const int32_t* expert_offsets, const int32_t* slot_to_pos, void* y_bf16,
+                                  int T, int H, int I, int E, int k, int weight_layout,
+                                  const float* bias13, const float* bias2, int activation, float alpha,
+                                  float limit, int w13_interleaved, void* workspace,
+                                  size_t workspace_bytes, void* stream, bool a8, bool x_quantized = false) {
+    if (!topk_w || !sorted_slots || !expert_offsets || !slot_to_pos) return HK_ERR_NULL_POINTER;
+    int st = moe_mxfp4_validate(x_bf16, w13, w13_scales, w13_scale_pitch, w2, w2_scales, w2_scale_pitch, y_bf16, T, H,
+                                I, E, k, weight_layout, bias13, bias2, activation, limit, workspace, workspace_bytes,
+                                a8);
+    if (st != HK_OK) return st;
+    const bool ext = bias13 || bias2 || activation != 0 || w13_interleaved;
+    const MoeWs L = moe_ws_layout(T, H, I, E, k, a8);
     hipStream_t s = (hipStream_t)stream;
     uint8_t* ws = (uint8_t*)workspace;
     const int S = T * k;
@@ -1761,12 +1777,11 @@ static int moe_mxfp4_forward_impl(const void* x_bf16, const float* router_logits
                                   int w13_interleaved, void* workspace, size_t workspace_bytes,
                                   void* stream, bool a8) {
     if (!router_logits) return HK_ERR_NULL_POINTER;
-    if (weight_layout != 0 && weight_layout != 1) return HK_ERR_UNSUPPORTED;
-    int st = moe_mxfp4_check(T, H, I, E, k, weight_layout ? moe_round_up(H / 32, 8) : w13_scale_pitch,
-                             weight_layout ? moe_round_up(I / 32, 8) : w2_scale_pitch);
+    int st = moe_mxfp4_validate(x_bf16, w13, w13_scales, w13_scale_pitch, w2, w2_scales, w2_scale_pitch, y_bf16, T, H,
+                                I, E, k, weight_layout, bias13, bias2, activation, limit, workspace, workspace_bytes,
+                                a8);
     if (st != HK_OK) return st;
     const MoeWs L = moe_ws_layout(T, H, I, E, k, a8);
-    if (!workspace || workspace_bytes < L.total) return HK_ERR_WORKSPACE;
     uint8_t* ws = (uint8_t*)workspace;
     st = hk_moe_topk_softmax(router_logits, T, E, k, (int32_t*)(ws + L.ids), (float*)(ws + L.w), stream);
     if (st != HK_OK) return st;

@@ -455,6 +455,15 @@ __global__ __launch_bounds__(256) void moe_sort_small_kernel(const int32_t* __re
     moe_sort_small_block(ids, S, E, blockIdx.x, true, expert_offsets, sorted_slots, slot_to_pos, lds, lo, hi);
 }
 
+// (declared in moe_common.h for the layers that launch other work in front of the routing)
+int moe_topk_grouped_sigmoid_check(int T, int E, int k, int n_group, int topk_group) {
+    if (T <= 0 || T > (1 << 30) || E <= 0 || k <= 0 || k > 64 || E > 64 * kMaxPerLane || n_group <= 0 || n_group > 64 ||
+        (E % n_group) != 0 || topk_group <= 0 || topk_group > n_group ||
+        k > topk_group * (E / n_group))
+        return HK_ERR_BAD_SHAPE;
+    return HK_OK;
+}
+
 }  // namespace hk
 
 extern "C" int hk_moe_topk_softmax(const float* logits, int T, int E, int k, int32_t* ids, float* w,
@@ -476,10 +485,7 @@ extern "C" int hk_moe_topk_grouped_sigmoid(const float* logits, const float* bia
                                            int32_t* ids, float* w, void* stream) {
     using namespace hk;
     if (!logits || !ids || !w) return HK_ERR_NULL_POINTER;
-    if (T <= 0 || T > (1 << 30) || E <= 0 || k <= 0 || k > 64 || E > 64 * kMaxPerLane || n_group <= 0 || n_group > 64 ||
-        (E % n_group) != 0 || topk_group <= 0 || topk_group > n_group ||
-        k > topk_group * (E / n_group))
-        return HK_ERR_BAD_SHAPE;
+    if (moe_topk_grouped_sigmoid_check(T, E, k, n_group, topk_group) != HK_OK) return HK_ERR_BAD_SHAPE;
     // 16 lanes per token when the experts split into 16 equal runs and every group is a
     // power-of-two number of whole runs
     const int per = E / 16, gs = E / n_group;

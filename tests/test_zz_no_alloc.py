@@ -1,7 +1,9 @@
 """The split-K FP8 GEMM entry point that allocates nothing (hk_fp8_gemm_static_ws: partial sums in a
 device array inside the library) against hk_fp8_gemm_ws with a caller workspace, through the C ABI
 (ctypes on libhk355.so): identical bits, on calls in a row that share the array, the later ones
-smaller than the first, with device memory unchanged across the calls."""
+smaller than the first, with device memory unchanged across the calls; and the same calls recorded
+under HIP graph capture (where an allocation inside the library would fail the capture), replayed
+against the oracle-tested sibling's bits."""
 import ctypes
 
 import numpy as np
@@ -64,3 +66,46 @@ def test_fp8_gemm_static_ws_matches_caller_workspace_entry_point():
     assert lib.hk_fp8_gemm_static_ws(None, b.data_ptr(), c.data_ptr(), 16, 1024, 8192, 1.0, 1.0, stream) == -1
     assert lib.hk_fp8_gemm_static_ws(a.data_ptr(), b.data_ptr(), c.data_ptr(), 0, 1024, 8192, 1.0, 1.0, stream) == -2
     assert lib.hk_fp8_gemm_static_ws(a.data_ptr(), b.data_ptr(), c.data_ptr(), 16, 1024, 8190, 1.0, 1.0, stream) == -2
+
+
+def test_fp8_gemm_static_ws_records_into_a_graph():
+    """Stream capture refuses hipMalloc / hipFree: a capture of the entry point that succeeds shows that the
+    call path allocates nothing. Replays (with eager work of the program that dirties the shared array in
+    between) must reproduce hk_fp8_gemm_ws's bits, the second call of the graph on a smaller shape."""
+    lib = _lib.load_library()
+    shapes = [(64, 2048, 8192), (16, 1024, 8192)]
+    cases = []
+    for i, (M, N, K) in enumerate(shapes):
+        A, B = _operands(M, N, K, 30 + i)
+        need = lib.hk_fp8_gemm_workspace_bytes(M, N, K)
+        assert 0 < need <= lib.hk_fp8_gemm_static_ws_max_bytes()
+        ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+        want = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        got = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        rc = lib.hk_fp8_gemm_ws(A.data_ptr(), B.data_ptr(), want.data_ptr(), M, N, K, 0.5, 2.0, ws.data_ptr(), ws.numel(),
+                                ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0
+        cases.append((M, N, K, A, B, want, got))
+    # set-up call outside the capture (the per-device address look-up happens on a device's first call)
+    M, N, K, A, B, want, got = cases[1]
+    assert lib.hk_fp8_gemm_static_ws(A.data_ptr(), B.data_ptr(), got.data_ptr(), M, N, K, 0.5, 2.0,
+                                     ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for (M, N, K, A, B, want, got) in cases:
+            assert lib.hk_fp8_gemm_static_ws(A.data_ptr(), B.data_ptr(), got.data_ptr(), M, N, K, 0.5, 2.0, stream) == 0
+    big = _operands(128, 8192, 8192, 99)
+    sink = torch.empty((128, 8192), dtype=torch.bfloat16, device=DEV)
+    for rep in range(3):
+        for c in cases:
+            c[6].fill_(float("nan"))
+        # an eager call on the largest shape overwrites the whole shared array between the replays
+        assert lib.hk_fp8_gemm_static_ws(big[0].data_ptr(), big[1].data_ptr(), sink.data_ptr(), 128, 8192, 8192, 1.0, 1.0,
+                                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for (M, N, K, A, B, want, got) in cases:
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (rep, M, N, K)
