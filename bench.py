@@ -40,16 +40,96 @@ PEAK_FP8 = 5033.0     # MI355X dense FP8 MFMA peak, TFLOP/s (256 CU x 2.4 GHz x 
 PEAK_FP4 = 10066.0    # dense MXFP4
 PEAK_BF16 = 2516.5    # dense bf16
 PEAK_HBM = 8000.0     # GB/s
-# HBM-side bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs, each scaled by the same
-# counter's reading for a 1 GiB copy (`bench.py --traffic-calibration`; factors 2.0 and 1.0). Sources:
-# profiles/fp8_gemm_4wave_ring_kernel_8192.md (805.8 MB read + 137.3 MB written).
-TRAFFIC_FP8_8192 = 943.1e6
-# Other legs: profiles/traffic_counters_moe_and_gemm_legs.md (MoE legs: sum over the layer's launches).
-TRAFFIC = {"moe_mxfp4": 2.094e9, "moe_fp8blk": 14.30e9, "mxfp4_gemm": 562.7e6, "bf16_gemm": 1.748e9}
+# HBM-side bytes per launch (`traffic` of the roofline objects): profiles/traffic.json, written by
+# `python bench.py --collect-traffic DIR` from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs (one directory
+# per run under DIR, see collect_traffic), each counter scaled by its reading for a 1 GiB copy
+# (`bench.py --traffic-calibration`). The file is the only source of these figures: a profile refresh
+# rewrites it and the next bench line carries the new values.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+# The launches that make up one call of each leg's default workload, as rocprofv3 names the kernels.
+TRAFFIC_LEGS = {
+    "fp8_gemm_8192": ("calibration", ["fp8_gemm_4wave_ring_kernel<false>"]),
+    "mxfp4_gemm": ("mxfp4", ["mxfp4_gemm_4wave_kernel<false>"]),
+    "bf16_gemm": ("bf16", ["bf16_gemm_4wave_ring_kernel<false>"]),
+    "moe_mxfp4": ("moe_mxfp4", ["moe_topk_softmax_kernel<16>", "moe_sort_quantize_kernel<false>",
+                                "moe_mxfp4_stream4_kernel<0, false, false, true, true>",
+                                "moe_mxfp4_stream4_kernel<1, false, false, false, true>", "moe_unpermute_kernel<4>"]),
+    "moe_fp8blk": ("moe_fp8blk", ["moe_topk_grouped_sigmoid16_kernel<16>", "moe_sort_count_kernel",
+                                  "moe_sort_scan_offsets_kernel", "moe_sort_scatter_kernel", "moe_build_items_kernel",
+                                  "moe_fp8blk_stream_kernel<0, true, false, 9>",
+                                  "moe_fp8blk_stream_kernel<1, false, false, 9>", "moe_unpermute_kernel<8>"]),
+}
+_traffic_cache = None
 
 
 def _traffic(key):
-    return TRAFFIC.get(key)
+    """HBM-side bytes per call of leg `key` from profiles/traffic.json, or None."""
+    global _traffic_cache
+    if _traffic_cache is None:
+        try:
+            with open(TRAFFIC_FILE) as f:
+                _traffic_cache = json.load(f).get("legs", {})
+        except (OSError, ValueError):
+            _traffic_cache = {}
+    leg = _traffic_cache.get(key)
+    return float(leg["total_bytes"]) if leg else None
+
+
+def collect_traffic(root):
+    """Reads the counter runs under `root` and rewrites profiles/traffic.json.
+
+    Expected below `root`, each the -d directory of one run of
+        rocprofv3 --pmc COUNTER --output-format csv -d root/RUN_COUNTER -o x -- python3 bench.py ARGS
+    with COUNTER = FETCH_SIZE and WRITE_SIZE: RUN = calibration (ARGS: --traffic-calibration) and one RUN per
+    leg of TRAFFIC_LEGS (ARGS: --only RUN --no-cpu-baseline --no-graph --steps 5 --warmup 2 --settle-ms 50).
+    A counter's KiB per dispatch are scaled by 1 GiB / its reading for the calibration run's copy kernel."""
+    import collections
+    import csv
+    import glob
+
+    def per_kernel(run, counter, reduce="mean"):
+        acc = collections.defaultdict(list)
+        files = glob.glob(os.path.join(root, f"{run}_{counter}", "**", "*counter_collection.csv"), recursive=True)
+        if not files:
+            raise RuntimeError(f"no counter_collection.csv under {root}/{run}_{counter}")
+        for path in files:
+            with open(path) as f:
+                for row in csv.DictReader(f):
+                    if row["Counter_Name"] == counter:
+                        acc[row["Kernel_Name"]].append(float(row["Counter_Value"]))
+        return {k: (max(v) if reduce == "max" else sum(v) / len(v)) for k, v in acc.items()}
+
+    def one(avgs, needle, what):
+        hits = [v for k, v in avgs.items() if needle in k]
+        if len(hits) != 1:
+            raise RuntimeError(f"{what}: {len(hits)} kernels match {needle!r} (the leg's launches changed: update TRAFFIC_LEGS)")
+        return hits[0]
+
+    factor = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        # the largest dispatch of the runtime's buffer-copy kernel is the 1 GiB copy (smaller copies ride along)
+        cal = per_kernel("calibration", counter, reduce="max")
+        copies = [v for k, v in cal.items() if "copyBuffer" in k]
+        if not copies or max(copies) < 1000.0:
+            raise RuntimeError(f"calibration run of {counter}: no 1 GiB copy found among {sorted(cal)}")
+        factor[counter] = (1 << 20) / max(copies)           # 1 GiB = 2^20 KiB moved per copy launch
+    legs = {}
+    for key, (run, kernels) in TRAFFIC_LEGS.items():
+        rd = per_kernel(run, "FETCH_SIZE")
+        wr = per_kernel(run, "WRITE_SIZE")
+        detail = {}
+        for name in kernels:
+            detail[name] = {"read_bytes": round(one(rd, name, key) * factor["FETCH_SIZE"] * 1024),
+                            "written_bytes": round(one(wr, name, key) * factor["WRITE_SIZE"] * 1024)}
+        legs[key] = {"read_bytes": sum(d["read_bytes"] for d in detail.values()),
+                     "written_bytes": sum(d["written_bytes"] for d in detail.values()), "kernels": detail}
+        legs[key]["total_bytes"] = legs[key]["read_bytes"] + legs[key]["written_bytes"]
+    out = {"source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, KiB per dispatch x calibration factor (bench.py --collect-traffic)",
+           "calibration_factor": {k: round(v, 4) for k, v in factor.items()}, "legs": legs}
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(out, f, indent=1)
+        f.write("\n")
+    return out
 
 
 def _roofline(bound, achieved, peak, unit, kernel, traffic=None, **more):
@@ -252,9 +332,11 @@ def bench_mxfp4(torch, hk, n, warmup, iters, dev):
 
 
 def bench_schedules(torch, hk, n, warmup, iters, dev):
-    """The two schedules of the 256x256-tile GEMMs side by side (kernels/gemm/fp8fp32/README.md:3-5 names both
-    for the reference): 4 waves with hand-interleaved slots (one wave per SIMD; what the library picks) and
-    8 waves in two ping-pong groups (two waves per SIMD). Same tile format, identical bits."""
+    """The schedules of the large-tile GEMMs side by side (kernels/gemm/fp8fp32/README.md:3-5 names the first two
+    for the reference): 4 waves with hand-interleaved slots (one wave per SIMD; what the library picks), 8 waves
+    in two ping-pong groups (two waves per SIMD), and the wave-specialised 4 producer + 12 consumer waves on a
+    192x256 tile (kernels/gemm/bf16fp32/mi350x/micros/producer_consumer in the reference). Same tile format,
+    identical bits."""
     out = {}
     g = torch.Generator(device=dev).manual_seed(0)
     a = torch.randn(n, n, device=dev, generator=g)
@@ -264,14 +346,14 @@ def bench_schedules(torch, hk, n, warmup, iters, dev):
     A8, sa = hk.quant.quantize_fp8_per_tensor(a)
     B8, sb = hk.quant.quantize_fp8_per_tensor(b)
     out["fp8"] = {name: tf(_timeit(torch, lambda: hk.tk_kernel.dispatch_fp8_gemm(A8, B8, C, sa, sb, variant=v), warmup, iters)[1])
-                  for name, v in (("4wave_interleave", 4), ("8wave_pingpong", 1))}
+                  for name, v in (("4wave_interleave", 4), ("8wave_pingpong", 1), ("producer_consumer_12c4p", 7))}
     Ab, Bb = a.to(torch.bfloat16), b.to(torch.bfloat16)
     out["bf16"] = {name: tf(_timeit(torch, lambda: hk.tk_kernel.dispatch_bf16_gemm(Ab, Bb, C, variant=v), warmup, iters)[1])
-                   for name, v in (("4wave_interleave", 1), ("8wave_pingpong", 4))}
+                   for name, v in (("4wave_interleave", 1), ("8wave_pingpong", 4), ("producer_consumer_12c4p", 5))}
     Ap, As = hk.quant.quantize_mxfp4(a)
     Bp, Bs = hk.quant.quantize_mxfp4(b)
     out["mxfp4"] = {name: tf(_timeit(torch, lambda: hk.tk_kernel.dispatch_mxfp4_gemm(Ap, As, Bp, Bs, C, variant=v), warmup, iters)[1])
-                    for name, v in (("4wave_interleave", 1), ("8wave_pingpong", 4))}
+                    for name, v in (("4wave_interleave", 1), ("8wave_pingpong", 4), ("producer_consumer_12c4p", 5))}
     out["workload"] = f"M=N=K={n}, TFLOP/s"
     return out
 
@@ -300,7 +382,7 @@ def bench_moe_mxfp4(torch, hk, warmup, iters, dev, graph=True):
         w2p[e], w2s[e] = a, hk.quant.pad_scales(s)
     W = hk.tk_kernel.MoeMxfp4ShuffledWeights.from_plain(w13p, w13s, w2p, w2s)
     # the oracle's inputs for a sample of tokens: their routing and the plain weights of the experts they use
-    sel = np.arange(5, T, T // 8)[:8]
+    sel = np.arange(5, T, T // 32)[:32]
     ids_s, w_s = OM.topk_softmax(logits[torch.from_numpy(sel).to(dev)].cpu().numpy(), k)
     used = np.unique(ids_s)
     ut = torch.from_numpy(used.astype(np.int64)).to(dev)
@@ -343,12 +425,12 @@ def bench_moe_mxfp4(torch, hk, warmup, iters, dev, graph=True):
     return {"workload": "moe_mxfp4 T=4096 H=2880 I=2880 E=128 top-4 softmax, MXFP4 activations and weights "
                         "(top-k, sort + activation quantization in one launch, 2 grouped GEMMs, un-permute)",
             "ms": round(kern, 5), "tflops": round(tf, 1), "frac_of_mxfp4_peak": round(tf / PEAK_FP4, 4),
-            "compulsory_GB": round(compulsory / 1e9, 3), "rel_fro_err_vs_oracle_8_tokens": rel,
+            "compulsory_GB": round(compulsory / 1e9, 3), "rel_fro_err_vs_oracle_32_tokens": rel,
             "roofline": _roofline("hbm", compulsory / (kern * 1e-3) / 1e9, PEAK_HBM, "GB/s",
                                   "whole layer (5 launches); dominant: moe_mxfp4 gate+up grouped GEMM",
                                   _traffic("moe_mxfp4")),
             "ms_graph_replay": round(kern_graph, 5) if graph else None, "ms_with_biases_and_clamped_swiglu": round(kern_oai, 5),
-            "ms_with_mxfp8_activations": round(kern_a8, 5), "rel_fro_err_mxfp8_activations_vs_oracle_8_tokens": rel8}
+            "ms_with_mxfp8_activations": round(kern_a8, 5), "rel_fro_err_mxfp8_activations_vs_oracle_32_tokens": rel8}
 
 
 def cpu_baseline_moe_mxfp4(torch, hk, dev):
@@ -547,8 +629,14 @@ def main() -> int:
     ap.add_argument("--only", type=str, default="", help="comma-separated legs of `extra` to run: " + ",".join(LEGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--traffic-calibration", action="store_true")
+    ap.add_argument("--collect-traffic", type=str, default="", metavar="DIR",
+                    help="rewrite profiles/traffic.json from the rocprofv3 counter runs under DIR (no GPU needed)")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph timings (for runs under a profiler)")
     args = ap.parse_args()
+    if args.collect_traffic:
+        out = collect_traffic(args.collect_traffic)
+        print(json.dumps({k: v["total_bytes"] for k, v in out["legs"].items()}))
+        return 0
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (--gpus 1); "
               "no multi-GPU path exists for this kernel library.", file=sys.stderr)
@@ -668,7 +756,7 @@ def main() -> int:
         "pct_of_fp8_peak": round(100.0 * tflops / PEAK_FP8, 2),
         "rel_fro_err_vs_oracle": rel,
         "roofline": _roofline("mfma", head["tflops"], PEAK_FP8, "TFLOP/s", "fp8_gemm_4wave_ring_kernel",
-                              TRAFFIC_FP8_8192 if n == 8192 else None, kernel_ms=round(head["kernel_ms"], 5),
+                              _traffic("fp8_gemm_8192") if n == 8192 else None, kernel_ms=round(head["kernel_ms"], 5),
                               # the register-only MFMA loop on the same operand bits: what the power limit
                               # leaves of the nominal peak on this data
                               measured_mfma_ceiling=round(ceiling, 1) if ceiling else None,

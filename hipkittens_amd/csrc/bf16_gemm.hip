@@ -12,6 +12,7 @@
 #include "gemm_ring.h"
 #include "gemm_small_tile.h"
 #include "gemm_pingpong.h"
+#include "gemm_prodcons.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -143,6 +144,28 @@ static int launch_bf16_pingpong(const void* A, const void* B, void* C, int M, in
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
+// Producer / consumer kernel (gemm_prodcons.h) with the bf16 MFMA: the reference's wave-specialised micro kernel
+// (kernels/gemm/bf16fp32/mi350x/micros/producer_consumer/32x16/micro_04_2stage_12c4p.cpp) on this library's tile
+// format. K: the operands' row length in bytes.
+template <bool EDGE>
+__global__ __launch_bounds__(kPcThreads) void bf16_gemm_prodcons_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n) {
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    gemm_prodcons_body<Bf16Mma, EDGE>(smem, A, B, C, M, N, K, alpha, tiles_m, tiles_n);
+}
+
+template <bool EDGE>
+static int launch_bf16_prodcons(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream) {
+    auto kern = bf16_gemm_prodcons_kernel<EDGE>;
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, kPcLdsBytes, configured)) return HK_ERR_LAUNCH;
+    const int tiles_m = (M + kPcBM - 1) / kPcBM, tiles_n = (N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kPcThreads), kPcLdsBytes, stream, (const uint8_t*)A,
+                       (const uint8_t*)B, (uint16_t*)C, M, N, 2 * K, 1.0f, tiles_m, tiles_n);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
 template <int TILE, int STAGES, bool EDGE>
 static int launch_bf16_small_tile(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream) {
     auto kern = bf16_gemm_small_tile_kernel<TILE, STAGES, EDGE, false>;
@@ -184,7 +207,7 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 8) != 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < 0 || variant > 4) return HK_ERR_UNSUPPORTED;
+    if (variant < 0 || variant > 5) return HK_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {
         if ((long long)((M + 63) / 64) > 65535) return HK_ERR_BAD_SHAPE;
@@ -203,6 +226,10 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
         const bool edge64 = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
         return edge64 ? launch_bf16_small_tile<kTinyTile, kTinyStages, true>(A, B, C, M, N, K, s)
                       : launch_bf16_small_tile<kTinyTile, kTinyStages, false>(A, B, C, M, N, K, s);
+    }
+    if (variant == 5) {
+        const bool e = (M % kPcBM) != 0 || (N % BN) != 0;
+        return e ? launch_bf16_prodcons<true>(A, B, C, M, N, K, s) : launch_bf16_prodcons<false>(A, B, C, M, N, K, s);
     }
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
     if (variant == 4)

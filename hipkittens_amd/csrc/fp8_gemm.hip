@@ -16,6 +16,7 @@
 #include "gemm_ring.h"
 #include "gemm_small_tile.h"
 #include "gemm_pingpong.h"
+#include "gemm_prodcons.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -56,6 +57,16 @@ __global__ __launch_bounds__(512) void fp8_gemm_pingpong_kernel(
     int M, int N, int K, float alpha, int tiles_m, int tiles_n, int band_n) {
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
     gemm_pingpong_body<Fp8Mma, EDGE>(smem, A, B, C, M, N, K, alpha, tiles_m, tiles_n, band_n);
+}
+
+// Producer / consumer kernel (gemm_prodcons.h) with the FP8 MFMA: four waves that only load, twelve that only
+// multiply (after the reference's micros/producer_consumer/32x16/micro_04_2stage_12c4p.cpp).
+template <bool EDGE>
+__global__ __launch_bounds__(kPcThreads) void fp8_gemm_prodcons_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, float alpha, int tiles_m, int tiles_n) {
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    gemm_prodcons_body<Fp8Mma, EDGE>(smem, A, B, C, M, N, K, alpha, tiles_m, tiles_n);
 }
 
 template <int TILE, int STAGES, bool EDGE, bool SPLIT>
@@ -123,6 +134,17 @@ __global__ __launch_bounds__(256) void fp8_gemm_portable_kernel(
 }
 
 template <bool EDGE>
+static int launch_prodcons(const void* A, const void* B, void* C, int M, int N, int K, float alpha, hipStream_t stream) {
+    auto kern = fp8_gemm_prodcons_kernel<EDGE>;
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, kPcLdsBytes, configured)) return HK_ERR_LAUNCH;
+    const int tiles_m = (M + kPcBM - 1) / kPcBM, tiles_n = (N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kPcThreads), kPcLdsBytes, stream, (const uint8_t*)A,
+                       (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha, tiles_m, tiles_n);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
+template <bool EDGE>
 static int launch_pingpong(const void* A, const void* B, void* C, int M, int N, int K, float alpha, hipStream_t stream) {
     auto kern = fp8_gemm_pingpong_kernel<EDGE>;
     static DeviceOnce configured;
@@ -178,7 +200,7 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 16) != 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < 0 || variant > 6 || variant == 2 || variant == 3) return HK_ERR_UNSUPPORTED;
+    if (variant < 0 || variant > 7 || variant == 2 || variant == 3) return HK_ERR_UNSUPPORTED;
     // K tails: the tile kernels zero-fill the last K-step of any K % 16 == 0
     if (variant != 0 && (long long)K * BM >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
     const float alpha = scale_a * scale_b;
@@ -199,6 +221,10 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
         const bool edge64 = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
         return edge64 ? launch_small_tile<kTinyTile, kTinyStages, true>(A, B, C, M, N, K, alpha, s)
                       : launch_small_tile<kTinyTile, kTinyStages, false>(A, B, C, M, N, K, alpha, s);
+    }
+    if (variant == 7) {
+        const bool e = (M % kPcBM) != 0 || (N % BN) != 0;
+        return e ? launch_prodcons<true>(A, B, C, M, N, K, alpha, s) : launch_prodcons<false>(A, B, C, M, N, K, alpha, s);
     }
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
     if (variant == 1)

@@ -41,12 +41,10 @@ inline bool moe_rows_fit_one_item(int T, int k, int E, int bm) {
     const double mu = (double)T * k / E;
     return mu + __builtin_sqrt(mu) <= bm;
 }
-// Bytes a layer's workspace carries behind its last region. The grouped GEMMs fetch the activation
-// rows and row scales of a work item in whole pieces (the streaming kernels 8 or 16 rows at a time,
-// the LDS-staged MXFP4 kernel its whole tile of 128 rows of 128 bytes): the last item's fetches run
-// past the end of their region into the regions behind it (the values are never used), and for a
-// layer of a few tokens those regions are shorter than that.
-constexpr size_t kMoeWsTail = 32768;
+// (A layer's workspace needs no room behind its last region: every fetch of activation rows, row scales and
+// slot ids in the grouped GEMMs goes through a buffer descriptor that ends where its region ends, or through
+// an index clamped to the region, so the piecewise fetches of a layer's last work item read zeros, not memory
+// behind the region.)
 // Number of CUs of the current device (cached per device ordinal).
 int moe_num_compute_units();
 // Shape check of hk_moe_topk_grouped_sigmoid (moe_routing.hip), for entry points that launch other work in

@@ -976,7 +976,7 @@ static Fp8Ws fp8_ws_layout(int T, int H, int I, int E, int k) {
     L.xq = take((size_t)T * H); L.xs = take((size_t)T * (H / 128) * 4);
     L.hq = take(S * (size_t)I); L.hs = take(S * (size_t)(I / 128) * 4);
     L.o = take(S * (size_t)H * 2);
-    L.total = off + kMoeWsTail;
+    L.total = off;
     return L;
 }
 

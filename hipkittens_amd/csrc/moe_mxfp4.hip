@@ -1555,7 +1555,7 @@ static MoeWs moe_ws_layout(int T, int H, int I, int E, int k, bool a8 = false) {
     L.xq = take(nk1 * S * row); L.xs = take(std::max(nk1 * S * 8, (nk1 + 15) / 16 * (size_t)T * 128));
     L.hq = take(nk2 * S * row); L.hs = take(nk2 * S * 8);
     L.o = take(S * (size_t)H * 2);
-    L.total = off + kMoeWsTail;
+    L.total = off;
     return L;
 }
 

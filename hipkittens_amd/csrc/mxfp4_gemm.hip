@@ -28,6 +28,7 @@
 #include "gemm_tile.h"
 #include "gemm_small_tile.h"
 #include "gemm_pingpong.h"
+#include "gemm_prodcons.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -431,6 +432,30 @@ __global__ __launch_bounds__(512) void mxfp4_gemm_pingpong_kernel(
                                        SmallTileScales{SA, SB, sa_pitch, sb_pitch});
 }
 
+// Producer / consumer kernel (gemm_prodcons.h) with the scaled FP4 MFMA. K: the operands' row length in bytes.
+template <bool EDGE>
+__global__ __launch_bounds__(kPcThreads) void mxfp4_gemm_prodcons_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
+    const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int sa_pitch,
+    int sb_pitch, int tiles_m, int tiles_n) {
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    gemm_prodcons_body<Mxfp4Mma, EDGE>(smem, A, B, C, M, N, K, 1.0f, tiles_m, tiles_n,
+                                       SmallTileScales{SA, SB, sa_pitch, sb_pitch});
+}
+
+template <bool EDGE>
+static int launch_mxfp4_prodcons(const void* A, const void* SA, const void* B, const void* SB, void* C,
+                                 int M, int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
+    auto kern = mxfp4_gemm_prodcons_kernel<EDGE>;
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, kPcLdsBytesScaled, configured)) return HK_ERR_LAUNCH;
+    const int tiles_m = (M + kPcBM - 1) / kPcBM, tiles_n = (N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kPcThreads), kPcLdsBytesScaled, stream,
+                       (const uint8_t*)A, (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB,
+                       (uint16_t*)C, M, N, K / 2, sa_pitch, sb_pitch, tiles_m, tiles_n);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+
 template <bool EDGE>
 static int launch_mxfp4_pingpong(const void* A, const void* SA, const void* B, const void* SB, void* C,
                                  int M, int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
@@ -462,7 +487,7 @@ static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, cons
 }  // namespace hk
 
 // variant: -1 = choose, 0 = portable kernel, 1 = 256x256 tile kernel (4 waves), 2 / 3 = 128x128 / 64x64 tiles,
-// 4 = 256x256 tile kernel with the 8-wave ping-pong schedule.
+// 4 = 256x256 tile kernel with the 8-wave ping-pong schedule, 5 = 192x256 tile producer / consumer kernel.
 // Scale rows are sa_pitch / sb_pitch bytes apart (>= K / 32).
 static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, const void* B, const void* B_scales,
                            int sb_pitch, void* C, int M, int N, int K, int variant, void* stream) {
@@ -472,7 +497,7 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
         gemm_dims_too_large(M, N, K))
         return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < -1 || variant > 4) return HK_ERR_UNSUPPORTED;
+    if (variant < -1 || variant > 5) return HK_ERR_UNSUPPORTED;
     // what the tile kernels need of the scale rows (any pitch and alignment; see mxfp4_scale_rows)
     const Mxfp4ScaleRows sr = mxfp4_scale_rows(K, sa_pitch, sb_pitch);
     const bool size_ok = (long long)(K / 2) * BM < (1ll << 31) && (long long)BM * max(sa_pitch, sb_pitch) < (1ll << 31);
@@ -502,10 +527,15 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
                  : launch_mxfp4_small_tile<kTinyTile, kTinyStages, false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, sr, s);
     }
     const bool edge = (M % BM) != 0 || (N % BN) != 0;
-    if (variant == 4) {
-        // the ping-pong kernel keeps the padded-row form (rows of whole groups of 8 scale bytes)
+    if (variant == 4 || variant == 5) {
+        // the ping-pong and producer / consumer kernels keep the padded-row form (rows of whole groups of 8 scale bytes)
         if (sr.row_bytes != 0) return HK_ERR_BAD_SHAPE;
         if (((uintptr_t)A_scales | (uintptr_t)B_scales) & 3u) return HK_ERR_BAD_ALIGNMENT;
+        if (variant == 5) {
+            const bool e = (M % kPcBM) != 0 || (N % BN) != 0;
+            return e ? launch_mxfp4_prodcons<true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s)
+                     : launch_mxfp4_prodcons<false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
+        }
         return edge ? launch_mxfp4_pingpong<true>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s)
                     : launch_mxfp4_pingpong<false>(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
     }

@@ -65,7 +65,7 @@ def dispatch_fp8_gemm(A, B, C, scale_a: float = 1.0, scale_b: float = 1.0, varia
                       workspace=None) -> None:
     """C[M,N] (bf16) = (scale_a*A[M,K]) @ (scale_b*B[N,K]).T, A and B e4m3, fp32 accumulation.
 
-    `variant` -1 lets the library choose; 0..6 force a kernel (see include/hk355.h). `workspace`
+    `variant` -1 lets the library choose; 0..7 force a kernel (see include/hk355.h). `workspace`
     (uint8, fp8_gemm_workspace_bytes(M, N, K) bytes): lets the library split K for decode-like
     shapes (hk_fp8_gemm_ws)."""
     _check_tensor(A, "A", _FP8, 2)
@@ -100,7 +100,7 @@ def bf16_gemm_workspace_bytes(M: int, N: int, K: int) -> int:
 
 def dispatch_bf16_gemm(A, B, C, variant: int = -1, workspace=None) -> None:
     """C[M,N] (bf16) = A[M,K] @ B[N,K].T for bf16 operands, fp32 accumulation
-    (include/hk355.h: hk_bf16_gemm). `variant` -1 lets the library choose; 0..3 force a kernel.
+    (include/hk355.h: hk_bf16_gemm). `variant` -1 lets the library choose; 0..5 force a kernel.
     `workspace` (uint8, bf16_gemm_workspace_bytes(M, N, K) bytes): lets the library split K for
     decode-like shapes (hk_bf16_gemm_ws)."""
     _check_tensor(A, "A", _BF16, 2)
@@ -149,7 +149,7 @@ def dispatch_mxfp4_gemm(A, A_scales, B, B_scales, C, variant: int = -1, workspac
     (low nibble = even k), A_scales [M,K/32] e8m0, B [N,K/2], B_scales [N,K/32]. The scale tensors
     may be wider than K/32 (padded rows, e.g. quant.pad_scales: any byte but 0xFF in the padding);
     rows that are a multiple of 8 bytes keep a K that is not a multiple of 256 on the tile kernels.
-    `variant` -1 lets the library choose; 0..3 force a kernel (see include/hk355.h).
+    `variant` -1 lets the library choose; 0..5 force a kernel (see include/hk355.h).
     `workspace` (uint8, mxfp4_gemm_workspace_bytes(M, N, K) bytes): lets the library split K for
     decode-like shapes (hk_mxfp4_gemm_ws)."""
     _check_tensor(A, "A", _FP4, 2)

@@ -91,8 +91,11 @@ int hk_fp8_gemm_static_ws(const void* A_e4m3, const void* B_e4m3, void* C_bf16, 
  * K >= 4096, or exactly 128 and K > 2048), 5 = 128x128x128 tile, 4
  * waves, plain loop over three LDS stages (picked for smaller problems), 6 = the same loop with
  * 64x64 tiles and four stages, two workgroups per CU (picked when the problem has at most 128
- * tiles of 128x128). 2 and 3 are not in use (HK_ERR_UNSUPPORTED). All tile kernels zero-fill the last
- * K-step of any K % 16 == 0 and give identical bits. */
+ * tiles of 128x128), 7 = 192x256x128 tile, sixteen waves: four producers that only issue the
+ * global->LDS loads and twelve consumers that only multiply (the wave-specialised structure of the
+ * reference's kernels/gemm/bf16fp32/mi350x/micros/producer_consumer/32x16/micro_04_2stage_12c4p.cpp;
+ * measured, not picked by default). 2 and 3 are not in use (HK_ERR_UNSUPPORTED). All tile kernels
+ * zero-fill the last K-step of any K % 16 == 0 and give identical bits. */
 int hk_fp8_gemm_variant(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
                         int M, int N, int K, float scale_a, float scale_b,
                         int variant, void* stream);
@@ -111,8 +114,9 @@ int hk_mxfp4_gemm(const void* A_e2m1, const void* A_scales_e8m0, const void* B_e
 /* Same contract on a chosen kernel: 0 = portable kernel (any shape), 1 = 256x256x256 tile
  * kernel (4 waves, hand-interleaved), 2 = 128x128 tiles / three LDS stages, 3 = 64x64 tiles / four
  * stages (the small-tile kernels of the FP8 GEMM with the scaled FP4 MFMA; hk_mxfp4_gemm picks by tile
- * count as hk_fp8_gemm does), 4 = 256x256x256 tile kernel with the 8-wave ping-pong schedule. 1-4 need
- * K % 256 == 0 (dense scale rows) and 4-byte aligned scale pointers. */
+ * count as hk_fp8_gemm does), 4 = 256x256x256 tile kernel with the 8-wave ping-pong schedule, 5 =
+ * 192x256x256 tile producer / consumer kernel (see hk_fp8_gemm_variant, 7). 1-3 take dense scale rows of
+ * any K >= 512 (K % 32 == 0) and any alignment; 4 and 5 need K % 256 == 0 and 4-byte aligned scale pointers. */
 int hk_mxfp4_gemm_variant(const void* A_e2m1, const void* A_scales_e8m0, const void* B_e2m1,
                           const void* B_scales_e8m0, void* C_bf16, int M, int N, int K,
                           int variant, void* stream);
@@ -162,7 +166,9 @@ int hk_bf16_gemm_ws(const void* A_bf16, const void* B_bf16, void* C_bf16, int M,
  * 2 = 128x128 tiles / three LDS stages, 3 = 64x64 tiles / four stages (the FP8 GEMM's small-tile
  * kernels with the bf16 MFMA; hk_bf16_gemm picks them by tile count as hk_fp8_gemm does), 4 = 256x256x64
  * tile kernel with the reference's 8-wave ping-pong schedule
- * (kernels/gemm/bf16fp32/mi325x/256_256_64_16.cpp:73-155). */
+ * (kernels/gemm/bf16fp32/mi325x/256_256_64_16.cpp:73-155), 5 = 192x256x64 tile producer / consumer kernel
+ * (kernels/gemm/bf16fp32/mi350x/micros/producer_consumer/32x16/micro_04_2stage_12c4p.cpp: four waves load,
+ * twelve multiply). */
 int hk_bf16_gemm_variant(const void* A_bf16, const void* B_bf16, void* C_bf16, int M, int N, int K,
                          int variant, void* stream);
 

@@ -34,7 +34,7 @@ SHAPES = [(256, 256, 64), (256, 256, 128), (256, 256, 192), (512, 768, 1024), (1
 RAGGED = [(300, 200, 256), (257, 255, 512), (64, 72, 768), (1000, 520, 320), (1, 200, 512), (5, 7, 128)]
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, -1])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, -1])
 @pytest.mark.parametrize("shape", SHAPES + RAGGED)
 def test_bf16_gemm_matches_oracle(hk, shape, variant):
     M, N, K = shape
@@ -49,7 +49,7 @@ def test_bf16_gemm_matches_oracle(hk, shape, variant):
     assert err <= 5e-3  # expected level; a layout bug gives O(1)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, -1])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, -1])
 @pytest.mark.parametrize("shape", [(96, 80, 104), (256, 256, 8), (300, 264, 200), (256, 384, 2880)])
 def test_bf16_gemm_k_not_multiple_of_64(hk, shape, variant):
     """K % 8 == 0 only: the tile kernel zero-fills the last K-step."""
@@ -62,7 +62,7 @@ def test_bf16_gemm_k_not_multiple_of_64(hk, shape, variant):
     assert G.rel_fro_error(out, G.bf16_gemm(a, b)) <= 5e-3
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
 def test_bf16_gemm_identity_is_bit_exact(hk, variant):
     # A = I (K = M): C = bf16(B)^T exactly, whatever the accumulation order
     n = 256
@@ -73,7 +73,7 @@ def test_bf16_gemm_identity_is_bit_exact(hk, variant):
     assert np.array_equal(out, b.T)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
 def test_bf16_gemm_small_integers_exact(hk, variant):
     # integer operands in [-4, 4], K = 512: all partial sums are integers < 2^14, exact in fp32;
     # the result is rounded to bf16 once, like the oracle's

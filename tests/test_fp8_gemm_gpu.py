@@ -35,7 +35,7 @@ SHAPES = [(256, 256, 256), (256, 256, 128), (512, 768, 384), (1024, 1024, 1024),
 RAGGED = [(300, 200, 256), (257, 255, 128), (64, 72, 640), (1000, 1000, 512), (1, 200, 512), (5, 7, 256)]
 
 
-@pytest.mark.parametrize("variant", [0, 1, 4, 5, 6, -1])
+@pytest.mark.parametrize("variant", [0, 1, 4, 5, 6, 7, -1])
 @pytest.mark.parametrize("shape", SHAPES + RAGGED)
 def test_fp8_gemm_matches_oracle(hk, shape, variant):
     M, N, K = shape
@@ -53,7 +53,7 @@ def test_fp8_gemm_matches_oracle(hk, shape, variant):
 K_TAIL = [(96, 80, 208), (256, 256, 16), (256, 256, 144), (300, 520, 272), (512, 384, 2880), (128, 128, 112)]
 
 
-@pytest.mark.parametrize("variant", [0, 1, 4, 5, 6, -1])
+@pytest.mark.parametrize("variant", [0, 1, 4, 5, 6, 7, -1])
 @pytest.mark.parametrize("shape", K_TAIL)
 def test_fp8_gemm_k_tail(hk, shape, variant):
     """K % 16 == 0 but K % 128 != 0 (2880 is the hidden size of the MoE models): the ring and
@@ -75,7 +75,7 @@ def test_fp8_gemm_k_tail_last_row_does_not_read_past_the_buffer(hk):
     rng = np.random.default_rng(99)
     (a, sa), (b, sb) = _random_codes(rng, M, K), _random_codes(rng, N, K)
     dev = torch.device("cuda:0")
-    for variant in (1, 4, 5, 6):
+    for variant in (1, 4, 5, 6, 7):
         pool = torch.full((4 * M * K,), 0x7F, dtype=torch.uint8, device=dev)  # e4m3fn NaN code
         A = pool[M * K:2 * M * K].view(M, K)
         B = pool[2 * M * K:3 * M * K].view(N, K)
@@ -136,7 +136,7 @@ def test_fp8_gemm_workspace_is_optional(hk):
     assert np.array_equal(C.view(torch.int16).cpu().numpy().view(np.uint16), base)
 
 
-@pytest.mark.parametrize("variant", [2, 3, 7])
+@pytest.mark.parametrize("variant", [2, 3, 8])
 def test_fp8_gemm_rejects_unknown_variants(hk, variant):
     rng = np.random.default_rng(7)
     (a, _), (b, _) = _random_codes(rng, 256, 256), _random_codes(rng, 256, 256)
@@ -144,7 +144,7 @@ def test_fp8_gemm_rejects_unknown_variants(hk, variant):
         _run(hk, a, b, 1.0, 1.0, variant)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 4, 5, 6])
+@pytest.mark.parametrize("variant", [0, 1, 4, 5, 6, 7])
 def test_fp8_gemm_identity_is_bit_exact(hk, variant):
     """A = I (K = M): C = bf16(B^T) exactly; every e4m3 value is a bf16 value."""
     n = 256
@@ -159,7 +159,7 @@ def test_fp8_gemm_identity_is_bit_exact(hk, variant):
     assert np.array_equal(F.bf16_to_f32(out), F.bf16_to_f32(expect))
 
 
-@pytest.mark.parametrize("variant", [1, 4, 5, 6])
+@pytest.mark.parametrize("variant", [1, 4, 5, 6, 7])
 def test_fp8_gemm_small_integers_exact(hk, variant):
     """Operands in {-2..2}: all products and partial sums are exact in fp32, so the result is
     order independent and must equal the integer matmul, rounded once to bf16."""

@@ -28,13 +28,13 @@ def test_tile_sizes_give_identical_bits(hk):
             assert torch.equal(outs[0], o)
 
     A8, B8 = A.to(torch.float8_e4m3fn), B.to(torch.float8_e4m3fn)
-    run(lambda C, v: hk.tk_kernel.dispatch_fp8_gemm(A8, B8, C, 0.5, 2.0, variant=v), [4, 5, 6, 1])
+    run(lambda C, v: hk.tk_kernel.dispatch_fp8_gemm(A8, B8, C, 0.5, 2.0, variant=v), [4, 5, 6, 1, 7])
     Ab, Bb = A.to(torch.bfloat16), B.to(torch.bfloat16)
-    run(lambda C, v: hk.tk_kernel.dispatch_bf16_gemm(Ab, Bb, C, variant=v), [1, 2, 3, 4])
+    run(lambda C, v: hk.tk_kernel.dispatch_bf16_gemm(Ab, Bb, C, variant=v), [1, 2, 3, 4, 5])
     K4 = 1280  # dense scale rows: K % 256 == 0
     Ap, As = hk.quant.quantize_mxfp4(A[:, :K4].contiguous())
     Bp, Bs = hk.quant.quantize_mxfp4(B[:, :K4].contiguous())
-    run(lambda C, v: hk.tk_kernel.dispatch_mxfp4_gemm(Ap, As, Bp, Bs, C, variant=v), [1, 2, 3, 4])
+    run(lambda C, v: hk.tk_kernel.dispatch_mxfp4_gemm(Ap, As, Bp, Bs, C, variant=v), [1, 2, 3, 4, 5])
 
 
 @pytest.mark.parametrize("kind", ["fp8", "bf16"])

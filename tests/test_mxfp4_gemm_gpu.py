@@ -35,7 +35,7 @@ SHAPES = [(256, 256, 256), (256, 256, 512), (512, 768, 1024), (1024, 1024, 2048)
 RAGGED = [(300, 200, 256), (257, 255, 512), (64, 72, 768), (1000, 520, 512), (1, 200, 512), (5, 7, 256), (130, 70, 1280)]
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, -1])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, -1])
 @pytest.mark.parametrize("shape", SHAPES + RAGGED)
 def test_mxfp4_gemm_matches_oracle(hk, shape, variant):
     M, N, K = shape
