@@ -194,6 +194,15 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
     // One K-step (slot plan of gemm_ring.h over two LDS stages). Scale handling: the raw
     // 8 bytes of a fragment are read together with the fragment; the shift that exposes
     // this lane's byte is placed well after the read (B: group 7; A fragment f: group f-1).
+    // A scaled FP4 MFMA of this shape runs 16 cycles and keeps the wave's issue busy for about 12 of
+    // them: one other instruction per MFMA is free, a second one already delays the next MFMA (register-only
+    // loop, one wave per SIMD, cycles per MFMA with 0 / 1 / 2 / 3 independent v_add behind each: 16.8 / 17.1 /
+    // 21.2 / 27.4; the unscaled FP8 form, 32 cycles, takes five before it slows down). Hence at most two
+    // instructions per slot below, spread over both passes. (The same kernel on the 32x32x64 form of the
+    // instruction, 64 MFMAs of 32 cycles per K-step with room for four instructions each and no per-lane
+    // shifts, was built and measured: 8192^3 on all-zero operands 5840 against 5700 TFLOP/s, on random
+    // operands 4550 against 4730: the accumulators' traffic per flop doubles, and with operands that toggle
+    // the part is power limited.)
     auto step = [&]<int P>(int kt) {
         const uint32_t k2 = (uint32_t)(kt + 2) * BK;
         v4i sa = srd_a, sb = srd_b, ssa = srd_sa, ssb = srd_sb;
@@ -204,6 +213,30 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
         const uint32_t early = P && ((kt + 1) >> 1) == tail_pair ? (uint32_t)tail_shift : 0u;
         const uint32_t sa_nx = P ? (sa_rd ^ kScaleStageBytes) + early : sa_rd;
         const uint32_t sb_nx = P ? (sb_rd ^ kScaleStageBytes) + early : sb_rd;
+        // operations behind the barrier, spread over the 48 MFMAs of both passes of groups 5..7: slot q
+        // (0..47) = 16 (m - 5) + 8 pass + n. Global->LDS loads at q = 0, 3, .., 45 (the pair's scale loads at
+        // 46, 47); LDS reads in the two slots between: unit u (fragment in the first, its scales in the
+        // second) = B0..B4, A0, B5, B6, B7, A1, -, A2 (A fragment j's registers are free once group 4 + j is done)
+        auto post_ops = [&](int q) __attribute__((always_inline)) {
+            if (q % 3 == 0) {
+                const int i = q / 3;
+                dma_one(i / NDMA, i % NDMA, P, k2, i / NDMA ? sb : sa, vor);
+            } else if (P == 0 && q >= 46) {
+                dma_scale(q - 46, (uint32_t)(kt >> 1) + 1u, q - 46 ? ssb : ssa);
+            }
+            if (q % 3 != 0) {
+                const int u = q / 3, part = q % 3 - 1;
+                constexpr int kUnit[16] = {0, 1, 2, 3, 4, 8, 5, 6, 7, 9, -1, 10, -1, -1, -1, -1};   // 0..7: B, 8..10: A
+                const int x = kUnit[u];
+                if (x >= 0 && x < 8) {
+                    if (part == 0) bf[P ^ 1][x] = lds_frag4(b_lo[P ^ 1], b_hi[P ^ 1], x * 16 * BK);
+                    else bs[P ^ 1][x] = rd_scale(sb_nx, P ^ 1, x);
+                } else if (x >= 8) {
+                    if (part == 0) af[x - 8] = lds_frag4(a_lo[P ^ 1], a_hi[P ^ 1], (x - 8) * 16 * BK);
+                    else as[x - 8] = rd_scale(sa_nx, P ^ 1, x - 8);
+                }
+            }
+        };
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             // first the 8 MFMAs on the low K-half (MX block g), then the 8 on the high half
@@ -217,27 +250,14 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_4wave_kernel(
                         as[(m + AD) & 3] = rd_scale(sa_rd, P, m + AD);
                     }
                 } else {
-                    const int j = (m - PG - 1) * NT + n;
-                    if (j < NT) {
-                        bf[P ^ 1][j] = lds_frag4(b_lo[P ^ 1], b_hi[P ^ 1], j * 16 * BK);
-                        bs[P ^ 1][j] = rd_scale(sb_nx, P ^ 1, j);
-                    } else if (j == NT || j == NT + 1) {
-                        af[j - NT] = lds_frag4(a_lo[P ^ 1], a_hi[P ^ 1], (j - NT) * 16 * BK);
-                        as[j - NT] = rd_scale(sa_nx, P ^ 1, j - NT);
-                    } else if (j == 2 * NT) {
-                        af[2] = lds_frag4(a_lo[P ^ 1], a_hi[P ^ 1], 2 * 16 * BK);
-                        as[2] = rd_scale(sa_nx, P ^ 1, 2);
-                    }
-                    if (j < 2 * NDMA) dma_one(j / NDMA, j % NDMA, P, k2, j / NDMA ? sb : sa, vor);
-                    // the next pair's scales: its stage was last read before this step's barrier
-                    // of the previous odd K-step, and is first read after the next step's barrier
-                    else if (P == 0 && j < 2 * NDMA + 2) dma_scale(j - 2 * NDMA, (uint32_t)(kt >> 1) + 1u, j - 2 * NDMA ? ssb : ssa);
+                    post_ops((m - PG - 1) * 16 + n);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
             for (int n = 0; n < NT; ++n) {
                 mfma_fp4_acc(acc[m][n], bf[P][n].hi, af[m & 3].hi, bs[P][n].y, as[m & 3].y);
+                if (m > PG) post_ops((m - PG - 1) * 16 + 8 + n);
                 if (m == MT - 1) shift_scale(bs[P ^ 1][n]);
                 // scale of A fragment m+1 (next step's fragment 0 when m == 7)
                 if (n == 4) shift_scale(as[(m + 1) & 3]);
