@@ -463,7 +463,7 @@ def cpu_baseline_moe_mxfp4(torch, hk, dev):
             "sample": f"oracle MoE forward on 8 of 128 experts x 256 of 4096 tokens (same rows per expert), best of 2: {best:.2f} s"}
 
 
-def bench_moe_fp8blk(torch, hk, warmup, iters, dev):
+def bench_moe_fp8blk(torch, hk, warmup, iters, dev, plain_weights=False):
     import numpy as np
 
     from oracle import formats as F
@@ -496,12 +496,17 @@ def bench_moe_fp8blk(torch, hk, warmup, iters, dev):
     # algorithmic bytes: weights and their scales once, x (e4m3 + scales) in, y out
     compulsory = w13q.numel() + w2q.numel() + 4 * (w13s.numel() + w2s.numel()) + T * H + 4 * xs.numel() + T * H * 2
     # weights in the pre-shuffled layout (offline step, once per checkpoint): the fast path
-    W = hk.tk_kernel.MoeFp8BlkShuffledWeights.from_plain(w13q, w13s, w2q, w2s)
-    torch.cuda.synchronize()
-    del w13q, w2q
-    torch.cuda.empty_cache()
-    _, kern = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_fp8blk(xq, xs, logits, None, W, None, None, None, y,
-                                                                      k, G, KG, 1.0, ws), warmup, iters)
+    # (--fp8blk-plain-weights: the caller's [E, rows, K] layout instead, served by the LDS-staged kernel)
+    if plain_weights:
+        _, kern = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_fp8blk(xq, xs, logits, None, w13q, w13s, w2q, w2s, y,
+                                                                          k, G, KG, 1.0, ws), warmup, iters)
+    else:
+        W = hk.tk_kernel.MoeFp8BlkShuffledWeights.from_plain(w13q, w13s, w2q, w2s)
+        torch.cuda.synchronize()
+        del w13q, w2q
+        torch.cuda.empty_cache()
+        _, kern = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_fp8blk(xq, xs, logits, None, W, None, None, None, y,
+                                                                          k, G, KG, 1.0, ws), warmup, iters)
     # parity spot check (outside the timed region)
     want = F.bf16_to_f32(OM.moe_fp8blk_forward(xq[st].view(torch.uint8).cpu().numpy(), xs[st].cpu().numpy(), ids_l, w_s,
                                                *plain))
@@ -509,12 +514,12 @@ def bench_moe_fp8blk(torch, hk, warmup, iters, dev):
     flop = 2.0 * T * k * (H * 2 * I + I * H)
     tf = flop / (kern * 1e-3) / 1e12
     return {"workload": "moe_fp8blk T=8192 H=7168 I=2048 E=256 top-8 sigmoid (8 groups / top-4), e4m3 with "
-                        "1x128 / 128x128 fp32 scales, pre-shuffled weights",
+                        "1x128 / 128x128 fp32 scales, " + ("plain weight layout" if plain_weights else "pre-shuffled weights"),
             "ms": round(kern, 5), "tflops": round(tf, 1), "frac_of_fp8_peak": round(tf / PEAK_FP8, 4),
             "compulsory_GB": round(compulsory / 1e9, 3), "rel_fro_err_vs_oracle_4_tokens": rel,
             "roofline": _roofline("hbm", compulsory / (kern * 1e-3) / 1e9, PEAK_HBM, "GB/s",
                                   "whole layer (7 launches); dominant: moe_fp8blk gate+up grouped GEMM",
-                                  _traffic("moe_fp8blk"),
+                                  None if plain_weights else _traffic("moe_fp8blk"),
                                   note="MFMA time at peak 1.15 ms vs 1.43 ms for the bytes: HBM is the binding roofline")}
 
 
@@ -613,8 +618,40 @@ def mfma_ceiling(torch, Aq, dev):
     return blocks * 8 * iters * 32 * 65536.0 / (ms * 1e-3) / 1e12
 
 
+def mfma_issue_probe(torch, dev):
+    """Shader clocks per MFMA of a register-only loop, one wave per SIMD, with 0..6 other instructions behind
+    each MFMA (bench-only library; the slot plans of the tile kernels are sized by this table)."""
+    path = os.path.join(ROOT, "hipkittens_amd", "libhk355_bench.so")
+    lib = ctypes.CDLL(path)
+    lib.hkbench_mfma_issue.restype = ctypes.c_int
+    lib.hkbench_mfma_issue.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 4 + [ctypes.c_void_p]
+    pattern = torch.zeros(1024, dtype=torch.int32, device=dev)
+    out = torch.zeros(2, dtype=torch.int64, device=dev)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    iters = 2000
+    modes = {0: ("v_mfma_f32_16x16x128_f8f6f4 fp8", 32), 1: ("v_mfma_scale_f32_16x16x128_f8f6f4 fp4", 32),
+             2: ("v_mfma_scale_f32_32x32x64_f8f6f4 fp4", 12)}
+    kinds = {0: ("v_add_u32", range(0, 7)), 1: ("s_add_u32", (2, 4, 6)), 2: ("ds_read_b128", (1, 2, 3))}
+    table = {}
+    for mode, (name, per_trip) in modes.items():
+        row = {}
+        for kind, (kname, counts) in kinds.items():
+            clocks = {}
+            for kops in counts:
+                for _ in range(2):   # the second launch is the measurement
+                    assert lib.hkbench_mfma_issue(pattern.data_ptr(), out.data_ptr(), mode, kind, kops, iters, st) == 0
+                    torch.cuda.synchronize()
+                clocks[str(kops)] = round(out[0].item() / (iters * per_trip), 1)
+            row[kname] = clocks
+        table[name] = row
+    return {"unit": "shader clocks per MFMA, one wave per SIMD, all-zero operands; key = other instructions per MFMA",
+            "clocks": table}
+
+
 LEGS = ("ceiling", "sweep", "reference_inputs", "decode", "bf16", "library", "mxfp4", "mxfp4_decode", "schedules",
-        "moe_mxfp4", "moe_fp8blk", "routing")
+        "moe_mxfp4", "moe_fp8blk", "routing", "issue_probe")
+# legs that only run when named with --only
+OPT_IN_LEGS = ("issue_probe",)
 
 
 def main() -> int:
@@ -632,6 +669,8 @@ def main() -> int:
     ap.add_argument("--collect-traffic", type=str, default="", metavar="DIR",
                     help="rewrite profiles/traffic.json from the rocprofv3 counter runs under DIR (no GPU needed)")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph timings (for runs under a profiler)")
+    ap.add_argument("--fp8blk-plain-weights", action="store_true",
+                    help="run the FP8-block MoE leg on the plain weight layout (the LDS-staged kernel)")
     args = ap.parse_args()
     if args.collect_traffic:
         out = collect_traffic(args.collect_traffic)
@@ -652,7 +691,7 @@ def main() -> int:
     hk.load_library()  # raises if libhk355.so has not been built
     dev = torch.device("cuda:0")
     n = args.size
-    legs = set(LEGS) if not args.only else set(args.only.split(","))
+    legs = set(LEGS) - set(OPT_IN_LEGS) if not args.only else set(args.only.split(","))
     if args.only_headline:
         legs = set()
     unknown = legs - set(LEGS)
@@ -725,12 +764,14 @@ def main() -> int:
         if not args.no_cpu_baseline:
             extra["moe_mxfp4"]["cpu_baseline"] = cpu_baseline_moe_mxfp4(torch, hk, dev)
     if "moe_fp8blk" in legs:
-        extra["moe_fp8blk"] = bench_moe_fp8blk(torch, hk, 10, 20, dev)
+        extra["moe_fp8blk"] = bench_moe_fp8blk(torch, hk, 10, 20, dev, args.fp8blk_plain_weights)
         torch.cuda.empty_cache()
         if not args.no_cpu_baseline:
             extra["moe_fp8blk"]["cpu_baseline"] = cpu_baseline_moe_fp8blk(torch, hk, dev)
     if "routing" in legs:
         extra["routing"] = bench_routing(torch, hk, quick_w, quick_i, dev)
+    if "issue_probe" in legs:
+        extra["mfma_issue_probe"] = mfma_issue_probe(torch, dev)
 
     cpu = None
     if not args.no_cpu_baseline:
