@@ -415,6 +415,9 @@ def bench_moe_mxfp4(torch, hk, warmup, iters, dev, graph=True):
     b2 = torch.randn(E, H, device=dev, generator=g)
     _, kern_oai = _timeit(torch, lambda: hk.tk_kernel.dispatch_moe_mxfp4(
         x, logits, W, None, None, None, y, k, ws, bias13=b13, bias2=b2, activation="swiglu_oai"), warmup, iters)
+    want_oai, _ = OM.moe_mxfp4_forward(F.bf16_to_f32(_np_bits(x[st])), ids_l, w_s, *plain, bias13=b13[ut].cpu().numpy(),
+                                       bias2=b2[ut].cpu().numpy(), activation="swiglu_oai")
+    rel_oai = OG.rel_fro_error(y[st].float().cpu().numpy(), F.bf16_to_f32(want_oai))
     # the same layer with MXFP8 activations (W4A8: mixed fp4 x fp8 MFMA), checked against the oracle on the sample
     ws8 = torch.empty(hk.tk_kernel.moe_mxfp4_workspace_bytes(T, H, I, E, k, act_format="mxfp8"), dtype=torch.uint8,
                       device=dev)
@@ -430,6 +433,7 @@ def bench_moe_mxfp4(torch, hk, warmup, iters, dev, graph=True):
                                   "whole layer (5 launches); dominant: moe_mxfp4 gate+up grouped GEMM",
                                   _traffic("moe_mxfp4")),
             "ms_graph_replay": round(kern_graph, 5) if graph else None, "ms_with_biases_and_clamped_swiglu": round(kern_oai, 5),
+            "rel_fro_err_biases_and_clamped_swiglu_vs_oracle_32_tokens": rel_oai,
             "ms_with_mxfp8_activations": round(kern_a8, 5), "rel_fro_err_mxfp8_activations_vs_oracle_32_tokens": rel8}
 
 

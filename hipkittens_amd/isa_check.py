@@ -349,18 +349,26 @@ def device_assembly(src: Path, out: Path) -> None:
         raise RuntimeError(f"hipcc -S failed for {src.name}:\n{res.stderr}")
 
 
-def check_sources(sources: list[Path] | None = None, jobs: int = 8) -> list[Finding]:
-    """Compiles the sources (default: every .hip file under csrc/) to device assembly and scans them."""
+def assembly_of_sources(sources: list[Path] | None = None, jobs: int = 8) -> dict[str, str]:
+    """Device assembly of the sources (default: every .hip file under csrc/), by source file name."""
     sources = sources or sorted((_build.PKG_DIR / "csrc").rglob("*.hip"))
     with tempfile.TemporaryDirectory() as tmp:
         outs = [Path(tmp) / (s.stem + ".s") for s in sources]
         with ThreadPoolExecutor(max_workers=jobs) as pool:
             list(pool.map(device_assembly, sources, outs))
-        findings: list[Finding] = []
-        for out in outs:
-            text = out.read_text()
-            findings += scan(text) + memory_spills(text)
+        return {s.name: out.read_text() for s, out in zip(sources, outs)}
+
+
+def check_texts(texts: dict[str, str]) -> list[Finding]:
+    findings: list[Finding] = []
+    for text in texts.values():
+        findings += scan(text) + memory_spills(text)
     return findings
+
+
+def check_sources(sources: list[Path] | None = None, jobs: int = 8) -> list[Finding]:
+    """Compiles the sources (default: every .hip file under csrc/) to device assembly and scans them."""
+    return check_texts(assembly_of_sources(sources, jobs))
 
 
 def main() -> int:
