@@ -156,6 +156,23 @@ __device__ __forceinline__ void gemm_ring_body(uint8_t* smem, const uint8_t* __r
         if (kt + 2 >= nk) { sa.z = 0; sb.z = 0; }
         const uint32_t vor = kt + 2 == nk - 1 ? tail_or : 0u;
         const uint32_t bl = b_lo0 + off1, bh = b_hi0 + off1;
+        // Two MFMAs per fragment pair (16-cycle MFMAs, each with room for about two other instructions, where
+        // the 32-cycle FP8 MFMA has room for five): the operations behind the barrier are spread over the 48
+        // MFMAs of both passes of groups 5..7 instead of the 24 of the first pass (+1.5 % for BF16 at 8192^3).
+        // Slot q (0..47) = 16 (m - 5) + 8 pass + n: LDS reads in the even slots, unit q / 2 = B0..B7, A0, A1,
+        // then A2 at q = 32 (A fragment j's registers are free once group 4 + j is done, i.e. from q = 16 j
+        // on); the eight A loads at q = 1, 5, .., 29. (Splitting a load into its M0 write and the load itself,
+        // one slot apart, which also saves the wait state between them, measured the same.)
+        auto post_ops = [&](int q) __attribute__((always_inline)) {
+            if ((q & 1) == 0) {
+                const int u = q / 2;
+                if (u < NT) bf[P ^ 1][u] = MMA::load(bl, bh, u * 16 * BK);
+                else if (u == NT || u == NT + 1) af[u - NT] = MMA::load(a_lo[P ^ 1], a_hi[P ^ 1], (u - NT) * 16 * BK);
+                else if (u == 16) af[2] = MMA::load(a_lo[P ^ 1], a_hi[P ^ 1], 2 * 16 * BK);
+            } else if (q % 4 == 1 && q / 4 < NDMA) {
+                dma_a(q / 4, P, k2, sa, vor);
+            }
+        };
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
 #pragma unroll
@@ -165,6 +182,8 @@ __device__ __forceinline__ void gemm_ring_body(uint8_t* smem, const uint8_t* __r
                     const int s = m * NT + n;  // 40 slots before the barrier: B loads at 2, 7, .., 37
                     if (n == 0) af[(m + AD) & 3] = MMA::load(a_lo[P], a_hi[P], (m + AD) * 16 * BK);
                     if (s % 5 == 2) dma_b(s / 5, off2, k2, sb, vor);
+                } else if (MMA::kPasses == 2) {
+                    post_ops((m - PG - 1) * 16 + n);
                 } else {
                     const int j = (m - PG - 1) * NT + n;  // 24 slots after the barrier
                     if (j < NT) {
@@ -183,6 +202,7 @@ __device__ __forceinline__ void gemm_ring_body(uint8_t* smem, const uint8_t* __r
 #pragma unroll
                 for (int n = 0; n < NT; ++n) {
                     MMA::template mma<1>(acc[m][n], bf[P][n], af[m & 3]);
+                    if (m > PG) post_ops((m - PG - 1) * 16 + 8 + n);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             if (m == PG) {
