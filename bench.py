@@ -50,7 +50,7 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 TRAFFIC_LEGS = {
     "fp8_gemm_8192": ("calibration", ["fp8_gemm_4wave_ring_kernel<false>"]),
     "mxfp4_gemm": ("mxfp4", ["mxfp4_gemm_4wave_kernel<false>"]),
-    "bf16_gemm": ("bf16", ["bf16_gemm_4wave_ring_kernel<false>"]),
+    "bf16_gemm": ("bf16", ["bf16_gemm_4wave_ring_kernel<false, true>"]),
     "moe_mxfp4": ("moe_mxfp4", ["moe_topk_softmax_kernel<16>", "moe_sort_quantize_kernel<false>",
                                 "moe_mxfp4_stream4_kernel<0, false, false, true, true>",
                                 "moe_mxfp4_stream4_kernel<1, false, false, false, true>", "moe_unpermute_kernel<4>"]),

@@ -40,12 +40,15 @@ struct Bf16RingMma {
     }
     static __device__ __forceinline__ int raster_group(int band_n, int tiles_n) { return band_n < tiles_n ? 4 : 8; }
 };
-template <bool EDGE>
+// STREAM_C: C is stored with the non-temporal hint; the host asks for it for large outputs of whole tiles while the
+// operands fit the memory-side cache (launch_bf16_ring has the rule and the measurements; 8192^3: 1577 -> 1593
+// TFLOP/s on one box, 1541 -> 1558 on another). (FP8 and MXFP4 at 8192^3: -1.0 / -1.5 %.)
+template <bool EDGE, bool STREAM_C = false>
 __global__ __launch_bounds__(256) void bf16_gemm_4wave_ring_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
     int M, int N, int K, float alpha, int tiles_m, int tiles_n, int band_n) {
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
-    gemm_ring_body<Bf16RingMma, EDGE>(smem, A, B, C, M, N, 2 * K, alpha, tiles_m, tiles_n, band_n);
+    gemm_ring_body<Bf16RingMma, EDGE, STREAM_C>(smem, A, B, C, M, N, 2 * K, alpha, tiles_m, tiles_n, band_n);
 }
 
 
@@ -186,17 +189,28 @@ static int launch_bf16_splitk(const void* A, const void* B, void* C, int M, int 
                                     B, C, M, N, 2 * K, 1.0f, splits, partial, stream);
 }
 
-template <bool EDGE>
-static int launch_bf16_ring(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream) {
-    auto kern = bf16_gemm_4wave_ring_kernel<EDGE>;
+template <bool EDGE, bool STREAM_C>
+static int launch_bf16_ring_kernel(const void* A, const void* B, void* C, int M, int N, int K, int band_n,
+                                  hipStream_t stream) {
+    auto kern = bf16_gemm_4wave_ring_kernel<EDGE, STREAM_C>;
     constexpr int lds_bytes = 5 * kTileBytes;
     static DeviceOnce configured;
     if (!set_lds_limit_once((const void*)kern, lds_bytes, configured)) return HK_ERR_LAUNCH;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds_bytes, stream, (const uint8_t*)A,
-                       (const uint8_t*)B, (uint16_t*)C, M, N, K, 1.0f, tiles_m, tiles_n,
-                       raster_band(((long long)M + N) * K * 2, tiles_n));
+                       (const uint8_t*)B, (uint16_t*)C, M, N, K, 1.0f, tiles_m, tiles_n, band_n);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+template <bool EDGE>
+static int launch_bf16_ring(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream) {
+    const int tiles_n = (N + BN - 1) / BN;
+    const int band_n = raster_band(((long long)M + N) * K * 2, tiles_n);
+    // whole tiles, operands that fit the memory-side cache (no bands) and a C of 96 MB or more: C goes out with the
+    // non-temporal hint (8192^3: +0.7 to 1.2 %; 4096^3, a C of 32 MB: -1.2 %; 16384^3, banded: -0.75 %)
+    if constexpr (!EDGE)
+        if (band_n >= tiles_n && (long long)M * N * 2 >= (96ll << 20))
+            return launch_bf16_ring_kernel<false, true>(A, B, C, M, N, K, band_n, stream);
+    return launch_bf16_ring_kernel<EDGE, false>(A, B, C, M, N, K, band_n, stream);
 }
 
 }  // namespace hk

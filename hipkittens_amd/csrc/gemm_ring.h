@@ -27,8 +27,9 @@ namespace hk {
 //                                 eight PASS 0 MFMAs of the same A fragment, so that two MFMAs
 //                                 into one accumulator are eight issue slots apart)
 //   raster_group(band_n, tiles_n) tile rows per raster group
-// K: operand row pitch in bytes. `smem`: the workgroup's 160 KiB of LDS.
-template <typename MMA, bool EDGE>
+// K: operand row pitch in bytes. `smem`: the workgroup's 160 KiB of LDS. STREAM_C: the epilogue's stores carry the
+// non-temporal hint (store_c_tile).
+template <typename MMA, bool EDGE, bool STREAM_C = false>
 __device__ __forceinline__ void gemm_ring_body(uint8_t* smem, const uint8_t* __restrict__ A,
                                                const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
                                                int M, int N, int K, float alpha, int tiles_m, int tiles_n,
@@ -227,7 +228,7 @@ __device__ __forceinline__ void gemm_ring_body(uint8_t* smem, const uint8_t* __r
     wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup retires
     mfma_drain_agpr(acc);
 
-    store_c_tile<MT, NT, EDGE>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
+    store_c_tile<MT, NT, EDGE, STREAM_C>(acc, C, M, N, row0 + wm * TM, col0 + wn * TN, alpha);
 }
 
 }  // namespace hk

@@ -43,7 +43,10 @@ __device__ __forceinline__ Frag4 lds_frag4(uint32_t addr_lo, uint32_t addr_hi, i
 // Epilogue of the tile kernels: alpha, bf16 (RNE), 16-byte stores.
 // acc[m][2p], acc[m][2p+1] hold, for C row `row_base + 16m + lane%16`, the 8 columns
 // `col_base + 32p + 8*(lane/16) .. +8` (see b_row_to_col).
-template <int MT, int NT, bool EDGE>
+// STREAM: the full-tile stores carry the non-temporal hint (C is written once and not read by the kernel;
+// keeping it out of the L2 leaves that cache to the operand panels). Only the BF16 ring kernel has an
+// instantiation with it (bf16_gemm.hip has the measurements).
+template <int MT, int NT, bool EDGE, bool STREAM = false>
 __device__ __forceinline__ void store_c_tile(const v4f (&acc)[MT][NT], uint16_t* __restrict__ C,
                                              int M, int N, int row_base, int col_base, float alpha) {
     const int r = lane_id() & 15, g = lane_id() >> 4;
@@ -58,7 +61,8 @@ __device__ __forceinline__ void store_c_tile(const v4f (&acc)[MT][NT], uint16_t*
                 v4i out;
                 out.x = pack_bf16(x.x, x.y); out.y = pack_bf16(x.z, x.w);
                 out.z = pack_bf16(y.x, y.y); out.w = pack_bf16(y.z, y.w);
-                *(v4i*)(C + (size_t)row * N + col) = out;
+                if (STREAM) __builtin_nontemporal_store(out, (v4i*)(C + (size_t)row * N + col));
+                else *(v4i*)(C + (size_t)row * N + col) = out;
             } else if (row < M) {
                 const float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
                 if (col + 8 <= N && (N & 7) == 0) {
