@@ -248,21 +248,24 @@ static __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* 
 
 // Which tile a GEMM gets when the caller does not pin a kernel: 256 (the large-tile kernels), 128 or
 // 64. Two layers:
-//  1. a rule: the largest tile that still gives every CU of the device work: 64x64 tiles (two workgroups per
-//     CU) when 128x128 tiles number at most half the CUs, else 128x128 tiles below that many tiles of
-//     256x256, with two corrections measured on an MI355X, in K-steps of the format's kernels (nk):
-//      - with exactly CUs / 2 large tiles and a K of at most `short_nk` steps the 128x128 tile is 2-10 % faster
-//        (prologue and epilogue are a large share of so short a loop, and four times as many tiles overlap them);
-//      - from `long_tiles` large tiles on (scaled with the CU count), a K of at least `long_nk` steps runs
-//        3-15 % faster on the large-tile kernel although some CUs idle: its K loop moves half the LDS bytes
-//        per flop (long_tiles 0: never, the format's two kernels tie there);
+//  1. a rule: the tile with the smallest estimated time. A tile kernel's workgroups run in rounds over the
+//     device's CUs (one workgroup per CU for the 256- and 128-tiles, two for the 64-tile), every round costs
+//     the same whether it is full or not, and a workgroup's time is a fixed part (prologue, epilogue, launch)
+//     plus a part per K-step:  time = ceil(tiles / (CUs x workgroups per CU)) x (fixed + per_step x K-steps).
+//     The two constants per tile and format were fitted to the sweep below on an MI355X (microseconds; they
+//     enter only through their ratios, the CU count through the rounds). This captures what a threshold on the
+//     tile count cannot: 72 tiles of 256 are one round where their 288 tiles of 128 are two (the large tile
+//     wins by 4-12 % from a K of about 4096 elements on), 64 tiles of 256 are one round of four times the work
+//     of the single round of 256 small tiles (the small tile wins by 60 %). Measured against the best of the
+//     three kernels on 360 shapes per format, the rule alone is more than 5 % behind on 8 / 6 / 10 shapes
+//     (FP8 / BF16 / MXFP4; the thresholds it replaced: 13 / 18 / 19);
 //  2. a generated table of the shapes on which a sweep found the rule's choice more than a few percent behind
 //     another tile (tile_table.inc, written by `python -m hipkittens_amd.tile_sweep FORMAT --emit`; the
 //     counterpart of the reference's per-shape analysis/baselines/gemm/utils/tuned.yaml). An entry is keyed by
 //     the format, the numbers of 64-row / 64-column blocks of M and N and the K-step count, and applies on
 //     devices with the CU count the sweep ran on.
 struct TileRule {
-    int short_nk, long_nk, long_tiles;
+    float fixed[3], per_step[3];   // 256-, 128-, 64-tile
 };
 enum TileFormat { kFmtFp8 = 0, kFmtBf16 = 1, kFmtMxfp4 = 2 };
 struct TileTableEntry { unsigned char fmt; unsigned short m64, n64, nk, tile; };
@@ -271,14 +274,17 @@ struct TileTableEntry { unsigned char fmt; unsigned short m64, n64, nk, tile; };
 int moe_num_compute_units();  // number of CUs of the current device, cached (moe_mxfp4.hip)
 
 static inline int pick_tile_rule(int M, int N, int nk, TileRule r, int cus) {
-    const long long half = cus / 2;
-    const long long tiles256 = (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-    const long long tiles128 =
-        (long long)((M + kSmallTile - 1) / kSmallTile) * ((N + kSmallTile - 1) / kSmallTile);
-    if (tiles128 <= half) return kTinyTile;
-    if (tiles256 > half) return BM;
-    if (tiles256 == half) return nk <= r.short_nk ? kSmallTile : BM;
-    return r.long_tiles > 0 && tiles256 * 256 >= (long long)r.long_tiles * cus && nk >= r.long_nk ? BM : kSmallTile;
+    const int tile[3] = {BM, kSmallTile, kTinyTile};
+    const int per_cu[3] = {1, 1, 2};
+    int best = 0;
+    double best_time = 0.0;
+    for (int i = 0; i < 3; ++i) {
+        const long long tiles = (((long long)M + tile[i] - 1) / tile[i]) * (((long long)N + tile[i] - 1) / tile[i]);
+        const long long capacity = (long long)cus * per_cu[i];
+        const double time = (double)((tiles + capacity - 1) / capacity) * ((double)r.fixed[i] + (double)r.per_step[i] * nk);
+        if (i == 0 || time < best_time) { best = i; best_time = time; }   // ties go to the larger tile
+    }
+    return tile[best];
 }
 static inline int pick_tile(int fmt, int M, int N, int nk, TileRule r, bool consult_table = true) {
     const int cus = moe_num_compute_units();   // 256 when no device can be queried
@@ -289,8 +295,10 @@ static inline int pick_tile(int fmt, int M, int N, int nk, TileRule r, bool cons
     }
     return pick_tile_rule(M, N, nk, r, cus);
 }
-// the formats' rules (K-steps: 128 bytes of an operand row)
-constexpr TileRule kTileRuleFp8{16, 32, 80}, kTileRuleBf16{32, 64, 96}, kTileRuleMxfp4{8, 0, 0};
+// the formats' constants (K-steps: 128 bytes of an operand row)
+constexpr TileRule kTileRuleFp8{{7.59f, 3.08f, 2.08f}, {0.984f, 0.571f, 0.333f}};
+constexpr TileRule kTileRuleBf16{{7.75f, 3.15f, 2.17f}, {1.051f, 0.562f, 0.336f}};
+constexpr TileRule kTileRuleMxfp4{{7.71f, 3.13f, 1.94f}, {1.316f, 0.767f, 0.549f}};
 
 // Number of K ranges the split-K path would use: as many as fill the CUs, each at least 4
 // K-steps long, at most 16; 1 = the problem has enough tiles or too short a K.

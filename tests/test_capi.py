@@ -163,16 +163,23 @@ def test_device_independent_quantizers_match_oracle_on_cpu():
 
 def test_tile_choice_rule_and_generated_table():
     """The choice of GEMM tile (no GPU needed: without a device the library assumes 256 CUs, the count the
-    committed table was measured on): the rule's landmarks, and every entry of csrc/tile_table.inc is what
-    the default entry points would pick for a shape with the entry's key."""
+    committed table was measured on): the rule's landmarks (rounds of workgroups over the CUs times a cost per
+    round), and every entry of csrc/tile_table.inc is what the default entry points would pick for a shape with
+    the entry's key."""
     tk = hk.tk_kernel
     for fmt in ("fp8", "bf16", "mxfp4"):
-        assert tk.gemm_tile_choice(fmt, 8192, 8192, 8192, False) == 256     # 1024 large tiles
-        assert tk.gemm_tile_choice(fmt, 1024, 1024, 1024, False) == 64      # 64 tiles of 128 x 128
+        assert tk.gemm_tile_choice(fmt, 8192, 8192, 8192, False) == 256     # 1024 large tiles: four full rounds
+        assert tk.gemm_tile_choice(fmt, 1024, 1024, 1024, False) == 64      # one round with any tile: the cheapest
         assert tk.gemm_tile_choice(fmt, 2048, 4096, 1024, False) == 128     # 128 large tiles, short K
         assert tk.gemm_tile_choice(fmt, 16, 8192, 8192, False) == 64
-    assert tk.gemm_tile_choice("fp8", 2048, 2560, 8192, False) == 256       # 80 large tiles, long K
-    assert tk.gemm_tile_choice("mxfp4", 2048, 2560, 16384, False) == 128    # (no such correction for MXFP4)
+        # 64 large tiles = one round of 256 small ones doing a quarter of the work each
+        assert tk.gemm_tile_choice(fmt, 1024, 4096, 4096, False) == 128
+    # 72 / 80 large tiles are one round where their 288 / 320 tiles of 128 x 128 are two: the large tile from a
+    # long K on (MXFP4, whose 64 x 64 kernel costs more per K-step, already here)
+    assert tk.gemm_tile_choice("mxfp4", 768, 6144, 6144, False) == 256
+    assert tk.gemm_tile_choice("mxfp4", 2048, 2560, 16384, False) == 256
+    assert tk.gemm_tile_choice("fp8", 2048, 2560, 16384, False) in (256, 64)
+    assert tk.gemm_tile_choice("fp8", 2048, 2560, 16384, False) != 128
     with pytest.raises(RuntimeError):
         tk.gemm_tile_choice("fp8", 0, 8, 8)
     text = open(os.path.join(ROOT, "hipkittens_amd", "csrc", "tile_table.inc")).read()
