@@ -372,12 +372,19 @@ __global__ __launch_bounds__(512) void moe_sort_scan_offsets_kernel(int32_t* __r
     const int e = threadIdx.x;
     int total = 0;
     if (e < E) {
+        // all 64 loads in flight at once through a descriptor of the counts' size: chunks beyond nchunks read as
+        // zero and their stores are dropped by the range check, so no load or store carries a condition of its own
+        // (64 wave-uniform conditions kept live cost 40 spilled scalar registers)
+        const __amdgpu_buffer_rsrc_t counts =
+            __builtin_amdgcn_make_buffer_rsrc(ws, 0, nchunks * E * (int)sizeof(int32_t), 0x00020000);
+        const int pitch = E * (int)sizeof(int32_t);
         int v[kSortFusedChunks];
 #pragma unroll
-        for (int c = 0; c < kSortFusedChunks; ++c) v[c] = c < nchunks ? ws[(size_t)c * E + e] : 0;
+        for (int c = 0; c < kSortFusedChunks; ++c)
+            v[c] = __builtin_amdgcn_raw_buffer_load_b32(counts, c * pitch + e * (int)sizeof(int32_t), 0, 0);
 #pragma unroll
         for (int c = 0; c < kSortFusedChunks; ++c) {
-            if (c < nchunks) ws[(size_t)c * E + e] = total;
+            __builtin_amdgcn_raw_buffer_store_b32(total, counts, c * pitch + e * (int)sizeof(int32_t), 0, 0);
             total += v[c];
         }
     }

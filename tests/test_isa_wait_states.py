@@ -170,7 +170,6 @@ SCALAR_SPILL_CEILINGS = {
     r"moe_mxfp4_gemm_kernel": 56,
     r"moe_fp8blk_stream_kernel": 19,
     r"moe_fp8blk_gemm_kernel": 44,
-    r"moe_sort_scan_offsets_kernel": 40,
 }
 
 
