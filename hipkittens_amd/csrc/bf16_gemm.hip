@@ -13,6 +13,7 @@
 #include "gemm_small_tile.h"
 #include "gemm_pingpong.h"
 #include "gemm_prodcons.h"
+#include "gemm_skinny.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -169,6 +170,20 @@ static int launch_bf16_prodcons(const void* A, const void* B, void* C, int M, in
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
 
+// The skinny kernel (gemm_skinny.h) with the BF16 MFMA. K: the operands' row length in bytes.
+template <int R, int NW, int D>
+__global__ __launch_bounds__(64 * NW) void bf16_gemm_skinny_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, float alpha) {
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    gemm_skinny_body<Bf16Mma, R, NW, D>(smem, A, B, C, M, N, K, alpha);
+}
+static int launch_bf16_skinny(const void* A, const void* B, void* C, int M, int N, int K_elems, hipStream_t stream) {
+    const int K = 2 * K_elems;
+    const float alpha = 1.0f;
+    HK_SKINNY_DISPATCH(bf16_gemm_skinny_kernel);
+}
+
 template <int TILE, int STAGES, bool EDGE>
 static int launch_bf16_small_tile(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream) {
     auto kern = bf16_gemm_small_tile_kernel<TILE, STAGES, EDGE, false>;
@@ -221,7 +236,8 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 8) != 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < 0 || variant > 5) return HK_ERR_UNSUPPORTED;
+    if (variant < 0 || variant > 6) return HK_ERR_UNSUPPORTED;
+    if (variant == 6 && M > kSkinnyMaxM) return HK_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {
         if ((long long)((M + 63) / 64) > 65535) return HK_ERR_BAD_SHAPE;
@@ -231,6 +247,7 @@ extern "C" int hk_bf16_gemm_variant(const void* A, const void* B, void* C, int M
         return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
     }
     if ((long long)2 * K * BM >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
+    if (variant == 6) return launch_bf16_skinny(A, B, C, M, N, K, s);
     if (variant == 2) {
         const bool edge128 = (M % kSmallTile) != 0 || (N % kSmallTile) != 0;
         return edge128 ? launch_bf16_small_tile<kSmallTile, kSmallStages, true>(A, B, C, M, N, K, s)
@@ -257,7 +274,8 @@ extern "C" int hk_bf16_gemm(const void* A, const void* B, void* C, int M, int N,
     const bool tile_ok = K > 0 && (long long)2 * K * BM < (1ll << 31);
     // the same choice of tile as hk_fp8_gemm (pick_tile), with this format's measured corrections
     const int tile = pick_tile(kFmtBf16, M, N, (int)((2ll * K + BK - 1) / BK), kTileRuleBf16);
-    const int variant = !tile_ok ? 0 : tile == kTinyTile ? 3 : tile == kSmallTile ? 2 : 1;
+    const bool skinny = tile_ok && use_skinny(M, N, (int)((2ll * K + BK - 1) / BK), false, moe_num_compute_units());
+    const int variant = !tile_ok ? 0 : skinny ? 6 : tile == kTinyTile ? 3 : tile == kSmallTile ? 2 : 1;
     return hk_bf16_gemm_variant(A, B, C, M, N, K, variant, stream);
 }
 
@@ -275,6 +293,8 @@ extern "C" int hk_bf16_gemm_ws(const void* A, const void* B, void* C, int M, int
     const bool can_split = splits >= 2 && workspace && workspace_bytes >= (size_t)splits * M * N * sizeof(float) &&
                            (K % 8) == 0 && (long long)2 * K * BM < (1ll << 31) && (long long)M * N < (1ll << 40);
     if (!can_split) return hk_bf16_gemm(A, B, C, M, N, K, stream);
+    if (use_skinny(M, N, (int)((2ll * K + BK - 1) / BK), true, moe_num_compute_units()))
+        return hk_bf16_gemm_variant(A, B, C, M, N, K, 6, stream);
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)workspace) & 15u) return HK_ERR_BAD_ALIGNMENT;
     const bool edge = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;

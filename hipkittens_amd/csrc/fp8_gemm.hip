@@ -17,6 +17,7 @@
 #include "gemm_small_tile.h"
 #include "gemm_pingpong.h"
 #include "gemm_prodcons.h"
+#include "gemm_skinny.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -133,6 +134,18 @@ __global__ __launch_bounds__(256) void fp8_gemm_portable_kernel(
     }
 }
 
+// The skinny kernel (gemm_skinny.h) with the FP8 MFMA.
+template <int R, int NW, int D>
+__global__ __launch_bounds__(64 * NW) void fp8_gemm_skinny_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, float alpha) {
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    gemm_skinny_body<Fp8Mma, R, NW, D>(smem, A, B, C, M, N, K, alpha);
+}
+static int launch_skinny(const void* A, const void* B, void* C, int M, int N, int K, float alpha, hipStream_t stream) {
+    HK_SKINNY_DISPATCH(fp8_gemm_skinny_kernel);
+}
+
 template <bool EDGE>
 static int launch_prodcons(const void* A, const void* B, void* C, int M, int N, int K, float alpha, hipStream_t stream) {
     auto kern = fp8_gemm_prodcons_kernel<EDGE>;
@@ -200,7 +213,8 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 16) != 0 || gemm_dims_too_large(M, N, K)) return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < 0 || variant > 7 || variant == 2 || variant == 3) return HK_ERR_UNSUPPORTED;
+    if (variant < 0 || variant > 8 || variant == 2 || variant == 3) return HK_ERR_UNSUPPORTED;
+    if (variant == 8 && M > kSkinnyMaxM) return HK_ERR_UNSUPPORTED;
     // K tails: the tile kernels zero-fill the last K-step of any K % 16 == 0
     if (variant != 0 && (long long)K * BM >= (1ll << 31)) return HK_ERR_BAD_SHAPE;
     const float alpha = scale_a * scale_b;
@@ -222,6 +236,7 @@ extern "C" int hk_fp8_gemm_variant(const void* A, const void* B, void* C, int M,
         return edge64 ? launch_small_tile<kTinyTile, kTinyStages, true>(A, B, C, M, N, K, alpha, s)
                       : launch_small_tile<kTinyTile, kTinyStages, false>(A, B, C, M, N, K, alpha, s);
     }
+    if (variant == 8) return launch_skinny(A, B, C, M, N, K, alpha, s);
     if (variant == 7) {
         const bool e = (M % kPcBM) != 0 || (N % BN) != 0;
         return e ? launch_prodcons<true>(A, B, C, M, N, K, alpha, s) : launch_prodcons<false>(A, B, C, M, N, K, alpha, s);
@@ -246,6 +261,9 @@ extern "C" int hk_fp8_gemm_ws(const void* A, const void* B, void* C, int M, int 
     const bool can_split = splits >= 2 && workspace && workspace_bytes >= (size_t)splits * M * N * sizeof(float) &&
                            (K % 16) == 0 && (long long)K * BM < (1ll << 31) && (long long)M * N < (1ll << 40);
     if (!can_split) return hk_fp8_gemm(A, B, C, M, N, K, scale_a, scale_b, stream);
+    // the skinny kernel adds its partial sums inside the workgroup and needs no workspace
+    if (use_skinny(M, N, (K + BK - 1) / BK, true, moe_num_compute_units()))
+        return hk_fp8_gemm_variant(A, B, C, M, N, K, scale_a, scale_b, 8, stream);
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)workspace) & 15u) return HK_ERR_BAD_ALIGNMENT;
     const bool edge = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
@@ -321,6 +339,8 @@ extern "C" int hk_fp8_gemm(const void* A, const void* B, void* C, int M, int N, 
     const bool tile_ok = K > 0 && (long long)K * BM < (1ll << 31);
     // 256x256 tiles (five-slot ring kernel), 128x128 or 64x64: see pick_tile
     const int tile = pick_tile(kFmtFp8, M, N, (K + BK - 1) / BK, kTileRuleFp8);
-    const int variant = !tile_ok ? 0 : tile == kTinyTile ? 6 : tile == kSmallTile ? 5 : 4;
+    // few rows: one pass over B by the skinny kernel where that is faster (use_skinny)
+    const bool skinny = tile_ok && use_skinny(M, N, (K + BK - 1) / BK, false, moe_num_compute_units());
+    const int variant = !tile_ok ? 0 : skinny ? 8 : tile == kTinyTile ? 6 : tile == kSmallTile ? 5 : 4;
     return hk_fp8_gemm_variant(A, B, C, M, N, K, scale_a, scale_b, variant, stream);
 }

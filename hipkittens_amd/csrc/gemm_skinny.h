@@ -1,0 +1,167 @@
+// GEMM kernel body for few rows of A against a long weight matrix (decode shapes), shared by the FP8 and BF16
+// GEMMs (a K-step is 128 bytes per operand row in both; only the MFMA differs).
+#pragma once
+#include "gemm_tile.h"
+#include "hk_host.h"
+#include "../../include/hk355.h"
+
+namespace hk {
+
+// Few rows of A against a long weight matrix (M <= 16 R): the GEMM is then one pass over
+// B at HBM speed. A workgroup of NW waves owns 32 rows of B (32 columns of C, all rows of A); wave w walks
+// its share of the K-steps on its own, without workgroup barriers: it fetches the 32 x 128-byte piece of B
+// and the 16 R x 128-byte piece of A of a K-step with direct global->LDS loads (a row's 128 bytes by eight
+// neighbouring lanes: whole cache lines, which a fetch straight into MFMA operand registers, a row per lane,
+// does not give) into a ring of D stages of LDS that belongs to the wave alone, D - 1 K-steps in flight,
+// and multiplies the stage that has landed. Rows past M or N and the 16-byte pieces past K lie outside the
+// descriptors and arrive as zeros. The NW partial sums then meet in LDS and are added in wave order, so the
+// result does not depend on timing and no second launch or workspace is needed (what the split-K path of the
+// tile kernels spends on them).
+constexpr int kSkinnyMaxM = 64;
+// MMA: the operand type's MFMA on one 16-row x 128-byte fragment pair, `MMA::mma(acc, b, a)`. K is the operands'
+// row length in BYTES (a multiple of 16); smem: the workgroup's dynamic LDS, NW * D * (32 + 16 R) * 128 bytes.
+template <typename MMA, int R, int NW, int D>
+__device__ __forceinline__ void gemm_skinny_body(
+    uint8_t* smem, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
+    int M, int N, int K, float alpha) {
+    constexpr int kWBytes = 32 * BK, kStage = kWBytes + 16 * R * BK, kRegion = D * kStage;
+    constexpr int LPT = 4 + 2 * R;   // loads per K-step
+    static_assert(D >= 2 && (D - 1) * LPT < 64, "vmcnt range");
+    static_assert(NW * R * 2 * 1024 <= NW * kRegion, "the partial sums reuse the stages");
+    const int lane = lane_id(), w = wave_id();
+    const uint32_t r = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * 32;
+    const int rows_b = N - n0 < 32 ? N - n0 : 32;
+    const v4i srd_b = make_srd(B + (size_t)n0 * K, (uint32_t)rows_b * (uint32_t)K);
+    const v4i srd_a = make_srd(A, (uint32_t)M * (uint32_t)K);
+    const int nk = (K + BK - 1) / BK;
+    const int s0 = (int)((long long)nk * w / NW), n = (int)((long long)nk * (w + 1) / NW) - s0;
+
+    // load i of a tile covers its rows 8 i .. 8 i + 7: lane l fetches, for LDS position l & 7 of row
+    // 8 i + l / 8, the 16-byte chunk that the swizzle puts there
+    uint32_t voff[2], tail_or[2];   // even / odd i (the swizzle of row 8 i + y depends on i's parity only)
+#pragma unroll
+    for (int par = 0; par < 2; ++par) {
+        const uint32_t row = 8u * par + (lane >> 3);
+        const uint32_t c = swz_chunk(row, lane & 7);
+        voff[par] = row * (uint32_t)K + c * 16u;
+        tail_or[par] = (int)(c * 16u) >= K - (nk - 1) * BK ? 0x80000000u : 0u;
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+    const uint32_t region = to_sgpr(lds0 + (uint32_t)w * kRegion);
+    auto issue = [&](int stage, int kt_local) {
+        const int kt = s0 + kt_local;
+        const uint32_t k0 = (uint32_t)kt * BK, dst = region + (uint32_t)stage * kStage;
+        const bool last = kt == nk - 1;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            dma16(srd_b, dst + i * 1024, (voff[i & 1] + (uint32_t)(i >> 1) * 16u * (uint32_t)K) | (last ? tail_or[i & 1] : 0u), k0);
+#pragma unroll
+        for (int i = 0; i < 2 * R; ++i)
+            dma16(srd_a, dst + kWBytes + i * 1024, (voff[i & 1] + (uint32_t)(i >> 1) * 16u * (uint32_t)K) | (last ? tail_or[i & 1] : 0u), k0);
+    };
+    auto wait_stages = [&](int in_flight) {   // at most `in_flight` of the most recently issued K-steps still fly
+        switch (in_flight) {
+            case 0: wait_vmcnt<0>(); break;
+            case 1: wait_vmcnt<LPT>(); break;
+            case 2: wait_vmcnt<(D > 3 ? 2 : 1) * LPT>(); break;
+            case 3: wait_vmcnt<(D > 4 ? 3 : 1) * LPT>(); break;
+            case 4: wait_vmcnt<(D > 5 ? 4 : 1) * LPT>(); break;
+            default: wait_vmcnt<(D > 6 ? 5 : 1) * LPT>(); break;
+        }
+    };
+    static_assert(D <= 7, "wait_stages covers up to five K-steps in flight");
+
+    const uint32_t rd_lo = region + r * 128u + swz_chunk(r, g) * 16u;
+    const uint32_t rd_hi = region + r * 128u + swz_chunk(r, g + 4) * 16u;
+    v4f acc[R][2];
+#pragma unroll
+    for (int i = 0; i < R; ++i) acc[i][0] = acc[i][1] = v4f{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+    for (int p = 0; p < D - 1; ++p)
+        if (p < n) issue(p, p);
+    int st = 0;
+    for (int kt = 0; kt < n; ++kt) {
+        wait_stages(min(n - 1 - kt, D - 2));   // K-step kt has landed
+        // the stage of K-step kt - 1 is free: its reads were waited for before its MFMAs
+        if (kt + D - 1 < n) issue(st == 0 ? D - 1 : st - 1, kt + D - 1);
+        const uint32_t so = (uint32_t)st * kStage;
+        v8i wf[2];
+#pragma unroll
+        for (int f = 0; f < 2; ++f) wf[f] = lds_frag(rd_lo + so, rd_hi + so, f * 16 * BK);
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const v8i af = lds_frag(rd_lo + so, rd_hi + so, kWBytes + i * 16 * BK);
+#pragma unroll
+            for (int f = 0; f < 2; ++f) MMA::mma(acc[i][f], wf[f], af);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this stage's reads are done before a later load may overwrite it
+        st = st == D - 1 ? 0 : st + 1;
+    }
+    // every wave is done with its stages (its loads have landed, its reads are complete): the partial sums take
+    // their place
+    __syncthreads();
+    v4f* red = (v4f*)smem;   // [NW][R][2][64]
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+#pragma unroll
+        for (int f = 0; f < 2; ++f) red[((w * R + i) * 2 + f) * 64 + lane] = acc[i][f];
+    __syncthreads();
+    for (int t = threadIdx.x; t < R * 128; t += 64 * NW) {
+        const int l = t & 63;
+        v4f sum = red[t];
+#pragma unroll
+        for (int ww = 1; ww < NW; ++ww) sum += red[ww * R * 128 + t];
+        sum *= alpha;
+        const int i = t >> 7, f = (t >> 6) & 1;
+        const int row = 16 * i + (l & 15), col = n0 + 16 * f + 4 * (l >> 4);
+        if (row < M) {
+            uint16_t* out = C + (size_t)row * N + col;
+            if ((N & 3) == 0 && col + 3 < N) {
+                *(uint2*)out = uint2{pack_bf16(sum.x, sum.y), pack_bf16(sum.z, sum.w)};
+            } else {
+                const float v[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (col + e < N) out[e] = (uint16_t)(pack_bf16(v[e], 0.f) & 0xffffu);
+            }
+        }
+    }
+}
+
+constexpr int skinny_lds_bytes(int R, int NW, int D) { return NW * D * (32 + 16 * R) * BK; }
+
+// Whether a GEMM entry point takes this kernel when the caller does not pin one. nk: K-steps; with_ws: the caller
+// gave a split-K workspace. From a sweep on an MI355X (M = 16 / 32 / 64, N = 512 ... 32768, K = 512 ... 16384
+// bytes per row, against the tile kernels with and without split-K): up to 32 rows it wins by 2 to 64 % while it
+// has at most 1.75 workgroups per CU (N <= 14336 on 256 CUs) and loses by 2 to 60 % from 3.5 on; with 33 to 64
+// rows it wins up to one workgroup per CU, except against split-K on few workgroups with a very long K.
+static inline bool use_skinny(int M, int N, int nk, bool with_ws, int cus) {
+    if (M > kSkinnyMaxM) return false;
+    const long long wgs = (N + 31) / 32;
+    if (M <= 32) return wgs * 4 <= 7ll * cus;
+    if (wgs > cus) return false;
+    return !(with_ws && wgs * 2 <= cus && nk >= 96);
+}
+
+// KERNEL<R, NW, D>: the format's __global__ instantiation of the body
+#define HK_SKINNY_LAUNCH(KERNEL, R, NW, D)                                                                     \
+    do {                                                                                                       \
+        auto kern = KERNEL<R, NW, D>;                                                                          \
+        constexpr int lds_bytes = skinny_lds_bytes(R, NW, D);                                                  \
+        static_assert(lds_bytes <= 160 * 1024, "LDS of one CU");                                               \
+        static DeviceOnce configured;                                                                          \
+        if (!set_lds_limit_once((const void*)kern, lds_bytes, configured)) return HK_ERR_LAUNCH;               \
+        hipLaunchKernelGGL(kern, dim3((N + 31) / 32), dim3(64 * NW), lds_bytes, stream, (const uint8_t*)A,     \
+                           (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha);                                   \
+        return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;                                        \
+    } while (0)
+// waves x stages per row count: the fastest of the combinations measured on an MI355X (N, K from 1024 to 28672;
+// eight waves with three stages, two with seven and others are within 15 % of these). K in bytes per row.
+#define HK_SKINNY_DISPATCH(KERNEL)                                \
+    if (M <= 16) HK_SKINNY_LAUNCH(KERNEL, 1, 4, 4);               \
+    if (M <= 32) HK_SKINNY_LAUNCH(KERNEL, 2, 4, 3);               \
+    HK_SKINNY_LAUNCH(KERNEL, 4, 4, 3)
+
+}  // namespace hk

@@ -65,7 +65,7 @@ def dispatch_fp8_gemm(A, B, C, scale_a: float = 1.0, scale_b: float = 1.0, varia
                       workspace=None) -> None:
     """C[M,N] (bf16) = (scale_a*A[M,K]) @ (scale_b*B[N,K]).T, A and B e4m3, fp32 accumulation.
 
-    `variant` -1 lets the library choose; 0..7 force a kernel (see include/hk355.h). `workspace`
+    `variant` -1 lets the library choose; 0..8 force a kernel (see include/hk355.h). `workspace`
     (uint8, fp8_gemm_workspace_bytes(M, N, K) bytes): lets the library split K for decode-like
     shapes (hk_fp8_gemm_ws)."""
     _check_tensor(A, "A", _FP8, 2)
@@ -100,7 +100,7 @@ def bf16_gemm_workspace_bytes(M: int, N: int, K: int) -> int:
 
 def dispatch_bf16_gemm(A, B, C, variant: int = -1, workspace=None) -> None:
     """C[M,N] (bf16) = A[M,K] @ B[N,K].T for bf16 operands, fp32 accumulation
-    (include/hk355.h: hk_bf16_gemm). `variant` -1 lets the library choose; 0..5 force a kernel.
+    (include/hk355.h: hk_bf16_gemm). `variant` -1 lets the library choose; 0..6 force a kernel.
     `workspace` (uint8, bf16_gemm_workspace_bytes(M, N, K) bytes): lets the library split K for
     decode-like shapes (hk_bf16_gemm_ws)."""
     _check_tensor(A, "A", _BF16, 2)

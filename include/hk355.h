@@ -41,7 +41,9 @@ int hk_version(void);
  * on the current device when the tile kernels can take it; consult_table 0: the rule alone, without the
  * generated per-shape table (what the sweep that writes the table compares against). Negative: a status.
  * Counterpart of the reference's per-shape solution selection
- * (analysis/baselines/gemm/utils/solution_selection.py, tuned.yaml). */
+ * (analysis/baselines/gemm/utils/solution_selection.py, tuned.yaml). With at most 64 rows of A the FP8 and BF16
+ * entry points may take the skinny kernel instead of a tile kernel (see hk_fp8_gemm_variant, 8); this function
+ * reports the tile they would take otherwise. */
 int hk_gemm_tile_choice(int format, int M, int N, int K, int consult_table);
 
 /*
@@ -63,7 +65,9 @@ int hk_fp8_gemm(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
  * tile, which write fp32 partial sums to the workspace, and a second kernel adds them in a fixed
  * order (deterministic) and rounds to bf16. hk_fp8_gemm_workspace_bytes returns the bytes this
  * needs, or 0 when the shape would not be split; with a NULL or too small workspace, or such a
- * shape, the call is hk_fp8_gemm. No counterpart in the reference (compile-time shapes only). */
+ * shape, the call is hk_fp8_gemm. With at most 64 rows of A most such shapes go to the skinny kernel
+ * (variant 8), which adds its partial sums inside the workgroup and leaves the workspace untouched.
+ * No counterpart in the reference (compile-time shapes only). */
 size_t hk_fp8_gemm_workspace_bytes(int M, int N, int K);
 int hk_fp8_gemm_ws(const void* A_e4m3, const void* B_e4m3, void* C_bf16, int M, int N, int K,
                    float scale_a, float scale_b, void* workspace, size_t workspace_bytes, void* stream);
@@ -87,15 +91,21 @@ int hk_fp8_gemm_static_ws(const void* A_e4m3, const void* B_e4m3, void* C_bf16, 
  * reference's second FP8 schedule, kernels/gemm/fp8fp32/README.md:3-5, schedule of
  * kernels/gemm/bf16fp32/mi325x/256_256_64_16.cpp:73-155), 4 = 256x256x128 tile, 4 waves,
  * hand-interleaved schedule over a five-slot LDS ring with the loads spread over the whole K-step
- * (what hk_fp8_gemm picks when the problem has more than 128 such tiles, or 80 to 128 of them and
- * K >= 4096, or exactly 128 and K > 2048), 5 = 128x128x128 tile, 4
+ * (what hk_fp8_gemm picks for large problems: the tile with the smallest estimated time, see
+ * hk_gemm_tile_choice), 5 = 128x128x128 tile, 4
  * waves, plain loop over three LDS stages (picked for smaller problems), 6 = the same loop with
- * 64x64 tiles and four stages, two workgroups per CU (picked when the problem has at most 128
- * tiles of 128x128), 7 = 192x256x128 tile, sixteen waves: four producers that only issue the
+ * 64x64 tiles and four stages, two workgroups per CU (picked for the smallest), 7 = 192x256x128
+ * tile, sixteen waves: four producers that only issue the
  * global->LDS loads and twelve consumers that only multiply (the wave-specialised structure of the
  * reference's kernels/gemm/bf16fp32/mi350x/micros/producer_consumer/32x16/micro_04_2stage_12c4p.cpp;
- * measured, not picked by default). 2 and 3 are not in use (HK_ERR_UNSUPPORTED). All tile kernels
- * zero-fill the last K-step of any K % 16 == 0 and give identical bits. */
+ * measured, not picked by default), 8 = the skinny kernel for M <= 64 (HK_ERR_UNSUPPORTED above): a
+ * workgroup owns 32 rows of B and all rows of A, its waves split K among themselves, stream their pieces
+ * of both operands through LDS stages of their own and add their partial sums in wave order
+ * (deterministic; one pass over B at HBM speed, no workspace; picked for decode shapes: up to 32 rows
+ * while N / 32 is at most 1.75 x the CU count, up to 64 rows while it is at most the CU count; no
+ * counterpart in the reference, whose shapes are compile-time squares). 2 and 3 are not in use
+ * (HK_ERR_UNSUPPORTED). All kernels zero-fill the last K-step of any K % 16 == 0; the tile kernels
+ * (1, 4 - 7) give identical bits, the skinny kernel adds in another order. */
 int hk_fp8_gemm_variant(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
                         int M, int N, int K, float scale_a, float scale_b,
                         int variant, void* stream);
@@ -168,7 +178,8 @@ int hk_bf16_gemm_ws(const void* A_bf16, const void* B_bf16, void* C_bf16, int M,
  * tile kernel with the reference's 8-wave ping-pong schedule
  * (kernels/gemm/bf16fp32/mi325x/256_256_64_16.cpp:73-155), 5 = 192x256x64 tile producer / consumer kernel
  * (kernels/gemm/bf16fp32/mi350x/micros/producer_consumer/32x16/micro_04_2stage_12c4p.cpp: four waves load,
- * twelve multiply). */
+ * twelve multiply), 6 = the skinny kernel for M <= 64 (see hk_fp8_gemm_variant, 8; picked by hk_bf16_gemm and
+ * hk_bf16_gemm_ws under the same conditions). */
 int hk_bf16_gemm_variant(const void* A_bf16, const void* B_bf16, void* C_bf16, int M, int N, int K,
                          int variant, void* stream);
 

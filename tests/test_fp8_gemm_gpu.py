@@ -136,7 +136,7 @@ def test_fp8_gemm_workspace_is_optional(hk):
     assert np.array_equal(C.view(torch.int16).cpu().numpy().view(np.uint16), base)
 
 
-@pytest.mark.parametrize("variant", [2, 3, 8])
+@pytest.mark.parametrize("variant", [2, 3, 9])
 def test_fp8_gemm_rejects_unknown_variants(hk, variant):
     rng = np.random.default_rng(7)
     (a, _), (b, _) = _random_codes(rng, 256, 256), _random_codes(rng, 256, 256)
