@@ -293,10 +293,11 @@ extern "C" int hk_bf16_gemm_ws(const void* A, const void* B, void* C, int M, int
     const bool can_split = splits >= 2 && workspace && workspace_bytes >= (size_t)splits * M * N * sizeof(float) &&
                            (K % 8) == 0 && (long long)2 * K * BM < (1ll << 31) && (long long)M * N < (1ll << 40);
     if (!can_split) return hk_bf16_gemm(A, B, C, M, N, K, stream);
-    if (use_skinny(M, N, (int)((2ll * K + BK - 1) / BK), true, moe_num_compute_units()))
-        return hk_bf16_gemm_variant(A, B, C, M, N, K, 6, stream);
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)workspace) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    // the skinny kernel adds its partial sums inside the workgroup and leaves the workspace alone
+    if (use_skinny(M, N, (int)((2ll * K + BK - 1) / BK), true, moe_num_compute_units()))
+        return hk_bf16_gemm_variant(A, B, C, M, N, K, 6, stream);
     const bool edge = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
     return edge ? launch_bf16_splitk<true>(A, B, C, M, N, K, splits, (float*)workspace, (hipStream_t)stream)
                 : launch_bf16_splitk<false>(A, B, C, M, N, K, splits, (float*)workspace, (hipStream_t)stream);

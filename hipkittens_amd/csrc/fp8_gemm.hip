@@ -261,11 +261,11 @@ extern "C" int hk_fp8_gemm_ws(const void* A, const void* B, void* C, int M, int 
     const bool can_split = splits >= 2 && workspace && workspace_bytes >= (size_t)splits * M * N * sizeof(float) &&
                            (K % 16) == 0 && (long long)K * BM < (1ll << 31) && (long long)M * N < (1ll << 40);
     if (!can_split) return hk_fp8_gemm(A, B, C, M, N, K, scale_a, scale_b, stream);
-    // the skinny kernel adds its partial sums inside the workgroup and needs no workspace
-    if (use_skinny(M, N, (K + BK - 1) / BK, true, moe_num_compute_units()))
-        return hk_fp8_gemm_variant(A, B, C, M, N, K, scale_a, scale_b, 8, stream);
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)workspace) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    // the skinny kernel adds its partial sums inside the workgroup and leaves the workspace alone
+    if (use_skinny(M, N, (K + BK - 1) / BK, true, moe_num_compute_units()))
+        return hk_fp8_gemm_variant(A, B, C, M, N, K, scale_a, scale_b, 8, stream);
     const bool edge = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
     const float alpha = scale_a * scale_b;
     return edge ? launch_tile128_splitk<true>(A, B, C, M, N, K, alpha, splits, (float*)workspace, (hipStream_t)stream)

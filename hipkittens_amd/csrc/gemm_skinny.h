@@ -19,14 +19,40 @@ namespace hk {
 // tile kernels spends on them).
 constexpr int kSkinnyMaxM = 64;
 // MMA: the operand type's MFMA on one 16-row x 128-byte fragment pair, `MMA::mma(acc, b, a)`. K is the operands'
-// row length in BYTES (a multiple of 16); smem: the workgroup's dynamic LDS, NW * D * (32 + 16 R) * 128 bytes.
+// row length in BYTES (a multiple of 16); smem: the workgroup's dynamic LDS, skinny_lds_bytes(R, NW, D, scaled).
+// MMA::kScaled (MXFP4): every operand row also has e8m0 block scales, 8 bytes per K-step, in rows of sa_pitch /
+// sb_pitch bytes of which `row_bytes` are scales (any pitch and alignment); `MMA::mma(acc, b, a, sb, sa)` takes,
+// per fragment, the lane's scale bytes of the K-step's two halves in bits [7:0] of .x / .y. A wave fetches the
+// scales as it fetches the operands: the 128 scale bytes of each of its rows that cover 16 K-steps form a tile of
+// the same shape as a K-step's operand bytes, loaded into one of two slots behind the stages, one such tile ahead.
+// What such a fetch brings in beyond a row's scales (the next rows' bytes, zeros past the operand's last row,
+// which ends the descriptor) belongs to K blocks past K, whose operand bytes arrive as zeros.
+// The bytes at `off` and `off + 4` of a descriptor's range (zero where outside), each in bits [7:0] of its
+// component; waits for them. The wait states in front cover a descriptor that the compiler restores from a
+// spilled register right before the statement.
+__device__ __forceinline__ v2i scale_bytes_direct(v4i srd, uint32_t off) {
+    int lo, hi;
+    asm volatile(
+        "s_nop 4\n\t"
+        "buffer_load_ubyte %0, %2, %3, 0 offen\n\t"
+        "buffer_load_ubyte %1, %2, %3, 0 offen offset:4\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(lo), "=&v"(hi)
+        : "v"(off), "s"(srd)
+        : "memory");
+    return v2i{lo, hi};
+}
+struct SkinnyScales {
+    const uint8_t* SA; const uint8_t* SB; int sa_pitch, sb_pitch, row_bytes;
+};
 template <typename MMA, int R, int NW, int D>
 __device__ __forceinline__ void gemm_skinny_body(
     uint8_t* smem, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
-    int M, int N, int K, float alpha) {
-    constexpr int kWBytes = 32 * BK, kStage = kWBytes + 16 * R * BK, kRegion = D * kStage;
-    constexpr int LPT = 4 + 2 * R;   // loads per K-step
-    static_assert(D >= 2 && (D - 1) * LPT < 64, "vmcnt range");
+    int M, int N, int K, float alpha, SkinnyScales sc = SkinnyScales{nullptr, nullptr, 0, 0, 0}) {
+    constexpr bool kScaled = MMA::kScaled;
+    constexpr int kWBytes = 32 * BK, kStage = kWBytes + 16 * R * BK, kRegion = (D + (kScaled ? 2 : 0)) * kStage;
+    constexpr int LPT = 4 + 2 * R;   // loads per K-step (and per tile of scales)
+    static_assert(D >= 2 && (D - 1 + (kScaled ? 1 : 0)) * LPT < 64, "vmcnt range");
     static_assert(NW * R * 2 * 1024 <= NW * kRegion, "the partial sums reuse the stages");
     const int lane = lane_id(), w = wave_id();
     const uint32_t r = lane & 15, g = lane >> 4;
@@ -60,6 +86,29 @@ __device__ __forceinline__ void gemm_skinny_body(
         for (int i = 0; i < 2 * R; ++i)
             dma16(srd_a, dst + kWBytes + i * 1024, (voff[i & 1] + (uint32_t)(i >> 1) * 16u * (uint32_t)K) | (last ? tail_or[i & 1] : 0u), k0);
     };
+    // scales (kScaled): tile c holds bytes [128 c, 128 c + 128) of the rows' scales, i.e. K-steps 16 c .. 16 c + 15
+    v4i srd_sb = {0, 0, 0, 0}, srd_sa = {0, 0, 0, 0};
+    uint32_t voff_sb[2] = {0, 0}, voff_sa[2] = {0, 0};
+    if constexpr (kScaled) {
+        srd_sb = make_srd(sc.SB + (size_t)n0 * sc.sb_pitch, (uint32_t)(rows_b - 1) * (uint32_t)sc.sb_pitch + (uint32_t)sc.row_bytes);
+        srd_sa = make_srd(sc.SA, (uint32_t)(M - 1) * (uint32_t)sc.sa_pitch + (uint32_t)sc.row_bytes);
+#pragma unroll
+        for (int par = 0; par < 2; ++par) {
+            const uint32_t row = 8u * par + (lane >> 3);
+            const uint32_t c = swz_chunk(row, lane & 7);
+            voff_sb[par] = row * (uint32_t)sc.sb_pitch + c * 16u;
+            voff_sa[par] = row * (uint32_t)sc.sa_pitch + c * 16u;
+        }
+    }
+    auto issue_scales = [&](int c) {
+        const uint32_t dst = region + (uint32_t)(D + (c & 1)) * kStage, off = (uint32_t)c * 128u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            dma16(srd_sb, dst + i * 1024, voff_sb[i & 1] + (uint32_t)(i >> 1) * 16u * (uint32_t)sc.sb_pitch, off);
+#pragma unroll
+        for (int i = 0; i < 2 * R; ++i)
+            dma16(srd_sa, dst + kWBytes + i * 1024, voff_sa[i & 1] + (uint32_t)(i >> 1) * 16u * (uint32_t)sc.sa_pitch, off);
+    };
     auto wait_stages = [&](int in_flight) {   // at most `in_flight` of the most recently issued K-steps still fly
         switch (in_flight) {
             case 0: wait_vmcnt<0>(); break;
@@ -78,23 +127,73 @@ __device__ __forceinline__ void gemm_skinny_body(
 #pragma unroll
     for (int i = 0; i < R; ++i) acc[i][0] = acc[i][1] = v4f{0.f, 0.f, 0.f, 0.f};
 
+    // the wave's first tile of scales goes out in front of its first K-step: it has landed when that K-step has
+    // (loads complete in order)
+    const int c_last = (s0 + n - 1) >> 4;
+    if constexpr (kScaled)
+        if (n > 0) issue_scales(s0 >> 4);
 #pragma unroll
     for (int p = 0; p < D - 1; ++p)
         if (p < n) issue(p, p);
     int st = 0;
     for (int kt = 0; kt < n; ++kt) {
-        wait_stages(min(n - 1 - kt, D - 2));   // K-step kt has landed
+        // K-step kt has landed. The count leaves the loads of scale tiles out: one of those among the loads
+        // behind K-step kt makes the wait stricter than needed, never weaker
+        wait_stages(min(n - 1 - kt, D - 2));
+        const int ks = s0 + kt;
+        if constexpr (kScaled) {
+            // entering a tile of scales: the next one goes out, 16 K-steps (or what is left of the first tile)
+            // before its first use; its slot's last reader was the K-step before this one
+            if ((kt == 0 || (ks & 15) == 0) && (ks >> 4) < c_last) issue_scales((ks >> 4) + 1);
+        }
         // the stage of K-step kt - 1 is free: its reads were waited for before its MFMAs
         if (kt + D - 1 < n) issue(st == 0 ? D - 1 : st - 1, kt + D - 1);
         const uint32_t so = (uint32_t)st * kStage;
         v8i wf[2];
 #pragma unroll
         for (int f = 0; f < 2; ++f) wf[f] = lds_frag(rd_lo + so, rd_hi + so, f * 16 * BK);
+        if constexpr (kScaled) {
+            v2i ws[2], as[R];
+            if ((sc.row_bytes & 3) != 0 && ks == nk - 1) {
+                // The range check of a descriptor works on dwords: the dword of a scale tile that reaches across
+                // the end of the operand's last row arrives as zero, and with it the last row_bytes % 4 scales of
+                // that row. They belong to the last K-step, whose scale bytes every lane therefore fetches itself,
+                // a byte at a time (the wave's loads have all landed: this is its last K-step).
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-            const v8i af = lds_frag(rd_lo + so, rd_hi + so, kWBytes + i * 16 * BK);
+                for (int f = 0; f < 2; ++f)
+                    ws[f] = scale_bytes_direct(srd_sb, (16u * f + r) * (uint32_t)sc.sb_pitch + (uint32_t)ks * 8u + g);
 #pragma unroll
-            for (int f = 0; f < 2; ++f) MMA::mma(acc[i][f], wf[f], af);
+                for (int i = 0; i < R; ++i)
+                    as[i] = scale_bytes_direct(srd_sa, (16u * i + r) * (uint32_t)sc.sa_pitch + (uint32_t)ks * 8u + g);
+            } else {
+                // the lane's scale bytes: row r of each fragment, the 8 bytes of K-step ks, byte g of each half's dword
+                const uint32_t sbase = region + (uint32_t)(D + ((ks >> 4) & 1)) * kStage + r * 128u +
+                                       swz_chunk(r, (uint32_t)(ks & 15) >> 1) * 16u + (uint32_t)(ks & 1) * 8u;
+                const uint32_t sh = 8u * g;
+#pragma unroll
+                for (int f = 0; f < 2; ++f) {
+                    ws[f] = *(lds_v2i_t*)(uintptr_t)(sbase + f * 16 * BK);
+                    ws[f].x = (int)((uint32_t)ws[f].x >> sh); ws[f].y = (int)((uint32_t)ws[f].y >> sh);
+                }
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    as[i] = *(lds_v2i_t*)(uintptr_t)(sbase + kWBytes + i * 16 * BK);
+                    as[i].x = (int)((uint32_t)as[i].x >> sh); as[i].y = (int)((uint32_t)as[i].y >> sh);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                const v8i af = lds_frag(rd_lo + so, rd_hi + so, kWBytes + i * 16 * BK);
+#pragma unroll
+                for (int f = 0; f < 2; ++f) MMA::mma(acc[i][f], wf[f], af, ws[f], as[i]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                const v8i af = lds_frag(rd_lo + so, rd_hi + so, kWBytes + i * 16 * BK);
+#pragma unroll
+                for (int f = 0; f < 2; ++f) MMA::mma(acc[i][f], wf[f], af);
+            }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this stage's reads are done before a later load may overwrite it
         st = st == D - 1 ? 0 : st + 1;
@@ -130,17 +229,20 @@ __device__ __forceinline__ void gemm_skinny_body(
     }
 }
 
-constexpr int skinny_lds_bytes(int R, int NW, int D) { return NW * D * (32 + 16 * R) * BK; }
+constexpr int skinny_lds_bytes(int R, int NW, int D, bool scaled = false) { return NW * (D + (scaled ? 2 : 0)) * (32 + 16 * R) * BK; }
 
 // Whether a GEMM entry point takes this kernel when the caller does not pin one. nk: K-steps; with_ws: the caller
 // gave a split-K workspace. From a sweep on an MI355X (M = 16 / 32 / 64, N = 512 ... 32768, K = 512 ... 16384
 // bytes per row, against the tile kernels with and without split-K): up to 32 rows it wins by 2 to 64 % while it
 // has at most 1.75 workgroups per CU (N <= 14336 on 256 CUs) and loses by 2 to 60 % from 3.5 on; with 33 to 64
 // rows it wins up to one workgroup per CU, except against split-K on few workgroups with a very long K.
-static inline bool use_skinny(int M, int N, int nk, bool with_ws, int cus) {
-    if (M > kSkinnyMaxM) return false;
+// The MXFP4 form (at most 32 rows; quarter_wgs_per_cu = 8) wins by 20 to 75 % up to two workgroups per CU
+// (N <= 16384) against the scaled tile kernels, whose scale fetches weigh more on few rows.
+static inline bool use_skinny(int M, int N, int nk, bool with_ws, int cus, int max_m = kSkinnyMaxM,
+                              int quarter_wgs_per_cu = 7) {
+    if (M > max_m) return false;
     const long long wgs = (N + 31) / 32;
-    if (M <= 32) return wgs * 4 <= 7ll * cus;
+    if (M <= 32) return wgs * 4 <= (long long)quarter_wgs_per_cu * cus;
     if (wgs > cus) return false;
     return !(with_ws && wgs * 2 <= cus && nk >= 96);
 }
@@ -163,5 +265,7 @@ static inline bool use_skinny(int M, int N, int nk, bool with_ws, int cus) {
     if (M <= 16) HK_SKINNY_LAUNCH(KERNEL, 1, 4, 4);               \
     if (M <= 32) HK_SKINNY_LAUNCH(KERNEL, 2, 4, 3);               \
     HK_SKINNY_LAUNCH(KERNEL, 4, 4, 3)
+// with block scales at most 32 rows: two slots of scales beside the stages fill the LDS of a CU at R = 2
+constexpr int kSkinnyMaxMScaled = 32;
 
 }  // namespace hk

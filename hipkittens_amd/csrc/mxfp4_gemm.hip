@@ -29,6 +29,7 @@
 #include "gemm_small_tile.h"
 #include "gemm_pingpong.h"
 #include "gemm_prodcons.h"
+#include "gemm_skinny.h"
 #include "../../include/hk355.h"
 
 namespace hk {
@@ -368,6 +369,35 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_small_tile_kernel(
         SmallTileScales{SA, SB, sa_pitch, sb_pitch, tail_pair, tail_shift, scale_row_bytes});
 }
 
+// The skinny kernel (gemm_skinny.h) with the scaled FP4 MFMA, for at most 32 rows of A. K: the operands' row
+// length in bytes; scale rows of any pitch and alignment, row_bytes scale bytes each.
+template <int R, int NW, int D>
+__global__ __launch_bounds__(64 * NW) void mxfp4_gemm_skinny_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
+    const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int sa_pitch, int sb_pitch,
+    int row_bytes) {
+    extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
+    gemm_skinny_body<Mxfp4Mma, R, NW, D>(smem, A, B, C, M, N, K, 1.0f, SkinnyScales{SA, SB, sa_pitch, sb_pitch, row_bytes});
+}
+template <int R, int NW, int D>
+static int launch_mxfp4_skinny_kernel(const void* A, const void* SA, const void* B, const void* SB, void* C, int M,
+                                      int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
+    auto kern = mxfp4_gemm_skinny_kernel<R, NW, D>;
+    constexpr int lds_bytes = skinny_lds_bytes(R, NW, D, true);
+    static_assert(lds_bytes <= 160 * 1024, "LDS of one CU");
+    static DeviceOnce configured;
+    if (!set_lds_limit_once((const void*)kern, lds_bytes, configured)) return HK_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3((N + 31) / 32), dim3(64 * NW), lds_bytes, stream, (const uint8_t*)A,
+                       (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB, (uint16_t*)C, M, N, K / 2, sa_pitch,
+                       sb_pitch, K / 32);
+    return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+}
+static int launch_mxfp4_skinny(const void* A, const void* SA, const void* B, const void* SB, void* C, int M, int N,
+                               int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
+    if (M <= 16) return launch_mxfp4_skinny_kernel<1, 4, 4>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
+    return launch_mxfp4_skinny_kernel<2, 4, 3>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
+}
+
 // What the tile kernels need to know about the scale rows (see the head of the file).
 // ok: the tile kernels can take these rows; tail_pair / tail_shift: the pair of K-steps fetched early and by how
 // many bytes (-1 / 0: none); row_bytes: what the scale descriptors cover of an operand's last row (0: its pitch).
@@ -507,7 +537,8 @@ static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, cons
 }  // namespace hk
 
 // variant: -1 = choose, 0 = portable kernel, 1 = 256x256 tile kernel (4 waves), 2 / 3 = 128x128 / 64x64 tiles,
-// 4 = 256x256 tile kernel with the 8-wave ping-pong schedule, 5 = 192x256 tile producer / consumer kernel.
+// 4 = 256x256 tile kernel with the 8-wave ping-pong schedule, 5 = 192x256 tile producer / consumer kernel,
+// 6 = the skinny kernel (at most 32 rows of A).
 // Scale rows are sa_pitch / sb_pitch bytes apart (>= K / 32).
 static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, const void* B, const void* B_scales,
                            int sb_pitch, void* C, int M, int N, int K, int variant, void* stream) {
@@ -517,7 +548,8 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
         gemm_dims_too_large(M, N, K))
         return HK_ERR_BAD_SHAPE;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) return HK_ERR_BAD_ALIGNMENT;
-    if (variant < -1 || variant > 5) return HK_ERR_UNSUPPORTED;
+    if (variant < -1 || variant > 6) return HK_ERR_UNSUPPORTED;
+    if (variant == 6 && M > kSkinnyMaxMScaled) return HK_ERR_UNSUPPORTED;
     // what the tile kernels need of the scale rows (any pitch and alignment; see mxfp4_scale_rows)
     const Mxfp4ScaleRows sr = mxfp4_scale_rows(K, sa_pitch, sb_pitch);
     const bool size_ok = (long long)(K / 2) * BM < (1ll << 31) && (long long)BM * max(sa_pitch, sb_pitch) < (1ll << 31);
@@ -525,6 +557,8 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
         // the choice of tile of hk_fp8_gemm (pick_tile); a K-step is 256 elements here
         const int tile = pick_tile(kFmtMxfp4, M, N, (K / 2 + BK - 1) / BK, kTileRuleMxfp4);
         variant = !(sr.ok && size_ok) ? 0 : tile == kTinyTile ? 3 : tile == kSmallTile ? 2 : 1;
+        // few rows: one pass over B by the skinny kernel where that is faster (use_skinny); it takes any scale rows
+        if (size_ok && use_skinny(M, N, (K / 2 + BK - 1) / BK, false, moe_num_compute_units(), kSkinnyMaxMScaled, 8)) variant = 6;
     }
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {
@@ -534,6 +568,10 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
                            (const uint8_t*)A_scales, (const uint8_t*)B, (const uint8_t*)B_scales,
                            (uint16_t*)C, M, N, K, sa_pitch, sb_pitch);
         return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
+    }
+    if (variant == 6) {
+        if (!size_ok) return HK_ERR_BAD_SHAPE;
+        return launch_mxfp4_skinny(A, A_scales, B, B_scales, C, M, N, K, sa_pitch, sb_pitch, s);
     }
     if (!size_ok || !sr.ok) return HK_ERR_BAD_SHAPE;
     if (variant == 2) {
@@ -597,6 +635,9 @@ extern "C" int hk_mxfp4_gemm_ws(const void* A, const void* A_scales, int a_scale
         return mxfp4_gemm_impl(A, A_scales, a_scale_pitch, B, B_scales, b_scale_pitch, C, M, N, K, -1, stream);
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)workspace) & 15u) return HK_ERR_BAD_ALIGNMENT;
+    // the skinny kernel adds its partial sums inside the workgroup and leaves the workspace alone
+    if (use_skinny(M, N, (K / 2 + BK - 1) / BK, true, moe_num_compute_units(), kSkinnyMaxMScaled, 8))
+        return mxfp4_gemm_impl(A, A_scales, a_scale_pitch, B, B_scales, b_scale_pitch, C, M, N, K, 6, stream);
     const bool edge = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
     return edge ? launch_mxfp4_splitk<true>(A, A_scales, B, B_scales, C, M, N, K, a_scale_pitch, b_scale_pitch, sr,
                                             splits, (float*)workspace, (hipStream_t)stream)

@@ -149,7 +149,7 @@ def dispatch_mxfp4_gemm(A, A_scales, B, B_scales, C, variant: int = -1, workspac
     (low nibble = even k), A_scales [M,K/32] e8m0, B [N,K/2], B_scales [N,K/32]. The scale tensors
     may be wider than K/32 (padded rows, e.g. quant.pad_scales: any byte but 0xFF in the padding);
     rows that are a multiple of 8 bytes keep a K that is not a multiple of 256 on the tile kernels.
-    `variant` -1 lets the library choose; 0..5 force a kernel (see include/hk355.h).
+    `variant` -1 lets the library choose; 0..6 force a kernel (see include/hk355.h).
     `workspace` (uint8, mxfp4_gemm_workspace_bytes(M, N, K) bytes): lets the library split K for
     decode-like shapes (hk_mxfp4_gemm_ws)."""
     _check_tensor(A, "A", _FP4, 2)

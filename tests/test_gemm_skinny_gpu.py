@@ -1,5 +1,5 @@
-"""The GEMM kernels for few rows of A (FP8 variant 8, BF16 variant 6; at most 64 rows) against the CPU
-oracle, through the C ABI.
+"""The GEMM kernels for few rows of A (FP8 variant 8, BF16 variant 6: at most 64 rows; MXFP4 variant 6: at most
+32) against the CPU oracle, through the C ABI.
 
 Tolerance: relative Frobenius error <= 5e-3 on the bf16 output (the north-star bound is 1e-2; accumulation
 order and the single bf16 rounding are the only differences, ~2e-3 observed). Exactly representable cases
@@ -153,3 +153,89 @@ def test_skinny_refuses_more_than_64_rows(hk):
         _fp8(hk, a, b, 1.0, 1.0, 8)
     with pytest.raises(RuntimeError):
         _bf16(hk, F.bf16_round(np.ones((65, 64), np.float32)), F.bf16_round(np.ones((64, 64), np.float32)), 6)
+
+
+# ---------------------------------------------------------------------------------------------- MXFP4
+def _rand_mx(rng, rows, K):
+    x = rng.standard_normal((rows, K)).astype(np.float32)
+    x *= np.exp2(rng.integers(-6, 7, size=(rows, K // 32))).repeat(32, axis=1).astype(np.float32)   # scales that matter
+    return F.quantize_mxfp4(x)
+
+
+def _mxfp4(hk, a, sa, b, sb, variant, misalign=0, pitches=None, workspace=False):
+    """Every operand array inside a pool of 0xFF bytes (a scale byte fetched in front of or behind an array
+    would be the e8m0 NaN), the scale arrays `misalign` bytes off a 16-byte boundary."""
+    views, pools = [], []
+    for arr, mis in ((a, 0), (sa, misalign), (b, 0), (sb, misalign)):
+        pool = torch.full((16 + mis + arr.size + 272,), 0xFF, dtype=torch.uint8, device=DEV)
+        view = pool[16 + mis:16 + mis + arr.size].view(arr.shape)
+        view.copy_(torch.from_numpy(arr).to(DEV))
+        pools.append(pool)
+        views.append(view)
+    A, SA, B, SB = views
+    C, buf = _guarded_c(a.shape[0], b.shape[0])
+    ws = None
+    if workspace:
+        ws = torch.full((max(16, hk.tk_kernel.mxfp4_gemm_workspace_bytes(a.shape[0], b.shape[0], a.shape[1] * 2)),),
+                        0xFF, dtype=torch.uint8, device=DEV)
+    hk.tk_kernel.dispatch_mxfp4_gemm(A, SA, B, SB, C, variant=variant, workspace=ws)
+    torch.cuda.synchronize()
+    _check_guards(buf, a.shape[0], b.shape[0])
+    return C.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+# K / 32 scale bytes per row: a single one, every remainder modulo 4 (the last K-step's scales are then fetched
+# byte by byte), more than one 128-byte scale tile per row (K > 4096), waves that start inside a scale tile
+MX_SHAPES = [(1, 32, 32), (16, 32, 256), (16, 64, 4096), (7, 100, 32 * 17), (16, 101, 2880), (17, 96, 2880),
+             (32, 200, 8192), (32, 72, 32 * 263), (3, 31, 96), (16, 2880, 2880), (24, 520, 32 * 47), (16, 256, 32 * 530)]
+
+
+@pytest.mark.parametrize("shape", MX_SHAPES)
+def test_mxfp4_skinny_matches_oracle(hk, shape):
+    M, N, K = shape
+    print(f"mxfp4 skinny shape={shape}", flush=True)
+    rng = np.random.default_rng(79 + M + N + K)
+    (a, sa), (b, sb) = _rand_mx(rng, M, K), _rand_mx(rng, N, K)
+    ref = G.mxfp4_gemm(a, sa, b, sb)
+    first = None
+    for mis in (0, 1, 3):
+        bits = _mxfp4(hk, a, sa, b, sb, 6, mis)
+        out = F.bf16_to_f32(bits)
+        assert np.isfinite(out).all(), mis
+        assert G.rel_fro_error(out, ref) <= 5e-3, mis
+        first = bits if first is None else first
+        assert np.array_equal(bits, first), mis
+
+
+def test_mxfp4_skinny_exact_and_scale_positions(hk):
+    """Elements in {-2..2} with scales 2^-2 .. 2^2 that differ from block to block: every partial sum is exact in
+    fp32 (below 2^18 in units of 2^-4), so the result is the exact value rounded once, whatever the order of the
+    waves' sums; a scale applied to the wrong 32-block or row would show."""
+    rng = np.random.default_rng(21)
+    codes = np.array([0, 2, 4, 10, 12], dtype=np.uint8)  # e2m1 codes of 0, 1, 2, -1, -2
+
+    def make(rows, K):
+        c = codes[rng.integers(0, 5, size=(rows, K))]
+        return ((c[:, 0::2] | (c[:, 1::2] << 4)).astype(np.uint8),
+                rng.integers(125, 130, size=(rows, K // 32)).astype(np.uint8))
+
+    for M, N, K in ((16, 96, 1024), (30, 100, 32 * 19), (9, 64, 32 * 270)):
+        (a, sa), (b, sb) = make(M, K), make(N, K)
+        exact = F.dequantize_mxfp4(a, sa).astype(np.float64) @ F.dequantize_mxfp4(b, sb).astype(np.float64).T
+        assert np.array_equal(_mxfp4(hk, a, sa, b, sb, 6, 1), F.bf16_round(exact.astype(np.float32)))
+
+
+def test_mxfp4_skinny_is_what_the_entry_points_pick_and_takes_padded_rows(hk):
+    """hk_mxfp4_gemm with and without a workspace gives the skinny kernel's bits at M = 16, N = 1024, K = 8192
+    and leaves the workspace alone; scale rows padded to a pitch give the same bits as dense rows."""
+    rng = np.random.default_rng(6)
+    M, N, K = 16, 1024, 8192
+    (a, sa), (b, sb) = _rand_mx(rng, M, K), _rand_mx(rng, N, K)
+    forced = _mxfp4(hk, a, sa, b, sb, 6)
+    assert np.array_equal(forced, _mxfp4(hk, a, sa, b, sb, -1))
+    assert np.array_equal(forced, _mxfp4(hk, a, sa, b, sb, -1, workspace=True))
+    pad = lambda s, pitch: np.concatenate([s, rng.integers(0, 255, size=(s.shape[0], pitch - s.shape[1]), dtype=np.uint8)], axis=1)
+    assert np.array_equal(forced, _mxfp4(hk, a, pad(sa, 264), b, pad(sb, 259), -1))
+    (a2, sa2), (b2, sb2) = _rand_mx(rng, 33, 256), _rand_mx(rng, 64, 256)
+    with pytest.raises(RuntimeError):
+        _mxfp4(hk, a2, sa2, b2, sb2, 6)
