@@ -236,7 +236,7 @@ constexpr int skinny_lds_bytes(int R, int NW, int D, bool scaled = false) { retu
 // bytes per row, against the tile kernels with and without split-K): up to 32 rows it wins by 2 to 64 % while it
 // has at most 1.75 workgroups per CU (N <= 14336 on 256 CUs) and loses by 2 to 60 % from 3.5 on; with 33 to 64
 // rows it wins up to one workgroup per CU, except against split-K on few workgroups with a very long K.
-// The MXFP4 form (at most 32 rows; quarter_wgs_per_cu = 8) wins by 20 to 75 % up to two workgroups per CU
+// The MXFP4 form (quarter_wgs_per_cu = 8) wins by 20 to 75 % up to two workgroups per CU
 // (N <= 16384) against the scaled tile kernels, whose scale fetches weigh more on few rows.
 static inline bool use_skinny(int M, int N, int nk, bool with_ws, int cus, int max_m = kSkinnyMaxM,
                               int quarter_wgs_per_cu = 7) {
@@ -265,7 +265,8 @@ static inline bool use_skinny(int M, int N, int nk, bool with_ws, int cus, int m
     if (M <= 16) HK_SKINNY_LAUNCH(KERNEL, 1, 4, 4);               \
     if (M <= 32) HK_SKINNY_LAUNCH(KERNEL, 2, 4, 3);               \
     HK_SKINNY_LAUNCH(KERNEL, 4, 4, 3)
-// with block scales at most 32 rows: two slots of scales beside the stages fill the LDS of a CU at R = 2
-constexpr int kSkinnyMaxMScaled = 32;
+// with block scales two slots of scales stand beside the stages: four waves with three stages fill the LDS of a CU
+// at R = 2, and R = 4 (up to 64 rows) has room for two waves with four stages
+constexpr int kSkinnyMaxMScaled = 64;
 
 }  // namespace hk

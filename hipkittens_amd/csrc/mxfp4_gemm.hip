@@ -369,7 +369,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_small_tile_kernel(
         SmallTileScales{SA, SB, sa_pitch, sb_pitch, tail_pair, tail_shift, scale_row_bytes});
 }
 
-// The skinny kernel (gemm_skinny.h) with the scaled FP4 MFMA, for at most 32 rows of A. K: the operands' row
+// The skinny kernel (gemm_skinny.h) with the scaled FP4 MFMA, for at most 64 rows of A. K: the operands' row
 // length in bytes; scale rows of any pitch and alignment, row_bytes scale bytes each.
 template <int R, int NW, int D>
 __global__ __launch_bounds__(64 * NW) void mxfp4_gemm_skinny_kernel(
@@ -395,7 +395,8 @@ static int launch_mxfp4_skinny_kernel(const void* A, const void* SA, const void*
 static int launch_mxfp4_skinny(const void* A, const void* SA, const void* B, const void* SB, void* C, int M, int N,
                                int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
     if (M <= 16) return launch_mxfp4_skinny_kernel<1, 4, 4>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
-    return launch_mxfp4_skinny_kernel<2, 4, 3>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
+    if (M <= 32) return launch_mxfp4_skinny_kernel<2, 4, 3>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
+    return launch_mxfp4_skinny_kernel<4, 2, 4>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
 }
 
 // What the tile kernels need to know about the scale rows (see the head of the file).
@@ -538,7 +539,7 @@ static int launch_mxfp4_4wave(const void* A, const void* SA, const void* B, cons
 
 // variant: -1 = choose, 0 = portable kernel, 1 = 256x256 tile kernel (4 waves), 2 / 3 = 128x128 / 64x64 tiles,
 // 4 = 256x256 tile kernel with the 8-wave ping-pong schedule, 5 = 192x256 tile producer / consumer kernel,
-// 6 = the skinny kernel (at most 32 rows of A).
+// 6 = the skinny kernel (at most 64 rows of A).
 // Scale rows are sa_pitch / sb_pitch bytes apart (>= K / 32).
 static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, const void* B, const void* B_scales,
                            int sb_pitch, void* C, int M, int N, int K, int variant, void* stream) {

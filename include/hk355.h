@@ -125,9 +125,10 @@ int hk_mxfp4_gemm(const void* A_e2m1, const void* A_scales_e8m0, const void* B_e
  * kernel (4 waves, hand-interleaved), 2 = 128x128 tiles / three LDS stages, 3 = 64x64 tiles / four
  * stages (the small-tile kernels of the FP8 GEMM with the scaled FP4 MFMA; hk_mxfp4_gemm picks by tile
  * count as hk_fp8_gemm does), 4 = 256x256x256 tile kernel with the 8-wave ping-pong schedule, 5 =
- * 192x256x256 tile producer / consumer kernel (see hk_fp8_gemm_variant, 7), 6 = the skinny kernel for M <= 32
+ * 192x256x256 tile producer / consumer kernel (see hk_fp8_gemm_variant, 7), 6 = the skinny kernel for M <= 64
  * (see hk_fp8_gemm_variant, 8; the scales travel like the operands, 128 bytes of a row at a time; picked by
- * hk_mxfp4_gemm, _pitched and _ws while N / 32 is at most twice the CU count). 1-3 take dense scale rows of
+ * hk_mxfp4_gemm, _pitched and _ws up to 32 rows while N / 32 is at most twice the CU count, up to 64 rows while
+ * it is at most the CU count). 1-3 take dense scale rows of
  * any K >= 512 (K % 32 == 0) and any alignment, 6 scale rows of any K, pitch and alignment; 4 and 5 need
  * K % 256 == 0 and 4-byte aligned scale pointers. */
 int hk_mxfp4_gemm_variant(const void* A_e2m1, const void* A_scales_e8m0, const void* B_e2m1,

@@ -1,5 +1,5 @@
-"""The GEMM kernels for few rows of A (FP8 variant 8, BF16 variant 6: at most 64 rows; MXFP4 variant 6: at most
-32) against the CPU oracle, through the C ABI.
+"""The GEMM kernels for few rows of A (at most 64; FP8 variant 8, BF16 and MXFP4 variant 6) against the CPU
+oracle, through the C ABI.
 
 Tolerance: relative Frobenius error <= 5e-3 on the bf16 output (the north-star bound is 1e-2; accumulation
 order and the single bf16 rounding are the only differences, ~2e-3 observed). Exactly representable cases
@@ -187,7 +187,8 @@ def _mxfp4(hk, a, sa, b, sb, variant, misalign=0, pitches=None, workspace=False)
 # K / 32 scale bytes per row: a single one, every remainder modulo 4 (the last K-step's scales are then fetched
 # byte by byte), more than one 128-byte scale tile per row (K > 4096), waves that start inside a scale tile
 MX_SHAPES = [(1, 32, 32), (16, 32, 256), (16, 64, 4096), (7, 100, 32 * 17), (16, 101, 2880), (17, 96, 2880),
-             (32, 200, 8192), (32, 72, 32 * 263), (3, 31, 96), (16, 2880, 2880), (24, 520, 32 * 47), (16, 256, 32 * 530)]
+             (32, 200, 8192), (32, 72, 32 * 263), (3, 31, 96), (16, 2880, 2880), (24, 520, 32 * 47), (16, 256, 32 * 530),
+             (33, 32, 256), (64, 101, 2880), (48, 200, 8192), (64, 72, 32 * 263)]
 
 
 @pytest.mark.parametrize("shape", MX_SHAPES)
@@ -219,7 +220,7 @@ def test_mxfp4_skinny_exact_and_scale_positions(hk):
         return ((c[:, 0::2] | (c[:, 1::2] << 4)).astype(np.uint8),
                 rng.integers(125, 130, size=(rows, K // 32)).astype(np.uint8))
 
-    for M, N, K in ((16, 96, 1024), (30, 100, 32 * 19), (9, 64, 32 * 270)):
+    for M, N, K in ((16, 96, 1024), (30, 100, 32 * 19), (9, 64, 32 * 270), (64, 40, 32 * 21)):
         (a, sa), (b, sb) = make(M, K), make(N, K)
         exact = F.dequantize_mxfp4(a, sa).astype(np.float64) @ F.dequantize_mxfp4(b, sb).astype(np.float64).T
         assert np.array_equal(_mxfp4(hk, a, sa, b, sb, 6, 1), F.bf16_round(exact.astype(np.float32)))
@@ -236,6 +237,6 @@ def test_mxfp4_skinny_is_what_the_entry_points_pick_and_takes_padded_rows(hk):
     assert np.array_equal(forced, _mxfp4(hk, a, sa, b, sb, -1, workspace=True))
     pad = lambda s, pitch: np.concatenate([s, rng.integers(0, 255, size=(s.shape[0], pitch - s.shape[1]), dtype=np.uint8)], axis=1)
     assert np.array_equal(forced, _mxfp4(hk, a, pad(sa, 264), b, pad(sb, 259), -1))
-    (a2, sa2), (b2, sb2) = _rand_mx(rng, 33, 256), _rand_mx(rng, 64, 256)
+    (a2, sa2), (b2, sb2) = _rand_mx(rng, 65, 256), _rand_mx(rng, 64, 256)
     with pytest.raises(RuntimeError):
         _mxfp4(hk, a2, sa2, b2, sb2, 6)

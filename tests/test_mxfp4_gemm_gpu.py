@@ -92,8 +92,9 @@ def _run_in_pool(hk, a, sa, b, sb, variant, misalign, workspace=False):
 
 
 # K / 32 scale bytes per row, dense rows: 90 (the GPT-OSS hidden size, tail fetched 2 bytes early), and one case
-# for each remainder of K / 32 modulo 4 and for rows of whole and broken groups of 16
-DENSE_RAGGED = [(512, 2880, 2880), (300, 200, 2880), (130, 520, 32 * 17), (257, 255, 32 * 19), (64, 384, 32 * 20),
+# for each remainder of K / 32 modulo 4 and for rows of whole and broken groups of 16 (more than 64 rows of A: with fewer
+# the library picks the skinny kernel, tests/test_gemm_skinny_gpu.py)
+DENSE_RAGGED = [(512, 2880, 2880), (300, 200, 2880), (130, 520, 32 * 17), (257, 255, 32 * 19), (72, 384, 32 * 20),
                 (96, 80, 32 * 47), (256, 256, 32 * 33), (200, 136, 32 * 18)]
 
 
