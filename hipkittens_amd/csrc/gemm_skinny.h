@@ -1,5 +1,5 @@
-// GEMM kernel body for few rows of A against a long weight matrix (decode shapes), shared by the FP8 and BF16
-// GEMMs (a K-step is 128 bytes per operand row in both; only the MFMA differs).
+// GEMM kernel body for few rows of A against a long weight matrix (decode shapes), shared by the FP8, BF16 and
+// MXFP4 GEMMs (a K-step is 128 bytes per operand row in all three; the MFMA differs, and MXFP4 adds its scales).
 #pragma once
 #include "gemm_tile.h"
 #include "hk_host.h"
@@ -18,15 +18,6 @@ namespace hk {
 // result does not depend on timing and no second launch or workspace is needed (what the split-K path of the
 // tile kernels spends on them).
 constexpr int kSkinnyMaxM = 64;
-// MMA: the operand type's MFMA on one 16-row x 128-byte fragment pair, `MMA::mma(acc, b, a)`. K is the operands'
-// row length in BYTES (a multiple of 16); smem: the workgroup's dynamic LDS, skinny_lds_bytes(R, NW, D, scaled).
-// MMA::kScaled (MXFP4): every operand row also has e8m0 block scales, 8 bytes per K-step, in rows of sa_pitch /
-// sb_pitch bytes of which `row_bytes` are scales (any pitch and alignment); `MMA::mma(acc, b, a, sb, sa)` takes,
-// per fragment, the lane's scale bytes of the K-step's two halves in bits [7:0] of .x / .y. A wave fetches the
-// scales as it fetches the operands: the 128 scale bytes of each of its rows that cover 16 K-steps form a tile of
-// the same shape as a K-step's operand bytes, loaded into one of two slots behind the stages, one such tile ahead.
-// What such a fetch brings in beyond a row's scales (the next rows' bytes, zeros past the operand's last row,
-// which ends the descriptor) belongs to K blocks past K, whose operand bytes arrive as zeros.
 // The bytes at `off` and `off + 4` of a descriptor's range (zero where outside), each in bits [7:0] of its
 // component; waits for them. The wait states in front cover a descriptor that the compiler restores from a
 // spilled register right before the statement.
@@ -42,6 +33,15 @@ __device__ __forceinline__ v2i scale_bytes_direct(v4i srd, uint32_t off) {
         : "memory");
     return v2i{lo, hi};
 }
+// MMA: the operand type's MFMA on one 16-row x 128-byte fragment pair, `MMA::mma(acc, b, a)`. K is the operands'
+// row length in BYTES (a multiple of 16); smem: the workgroup's dynamic LDS, skinny_lds_bytes(R, NW, D, scaled).
+// MMA::kScaled (MXFP4): every operand row also has e8m0 block scales, 8 bytes per K-step, in rows of sa_pitch /
+// sb_pitch bytes of which `row_bytes` are scales (any pitch and alignment); `MMA::mma(acc, b, a, sb, sa)` takes,
+// per fragment, the lane's scale bytes of the K-step's two halves in bits [7:0] of .x / .y. A wave fetches the
+// scales as it fetches the operands: the 128 scale bytes of each of its rows that cover 16 K-steps form a tile of
+// the same shape as a K-step's operand bytes, loaded into one of two slots behind the stages, one such tile ahead.
+// What such a fetch brings in beyond a row's scales (the next rows' bytes, zeros past the operand's last row,
+// which ends the descriptor) belongs to K blocks past K, whose operand bytes arrive as zeros.
 struct SkinnyScales {
     const uint8_t* SA; const uint8_t* SB; int sa_pitch, sb_pitch, row_bytes;
 };
