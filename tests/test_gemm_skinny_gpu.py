@@ -240,3 +240,29 @@ def test_mxfp4_skinny_is_what_the_entry_points_pick_and_takes_padded_rows(hk):
     (a2, sa2), (b2, sb2) = _rand_mx(rng, 65, 256), _rand_mx(rng, 64, 256)
     with pytest.raises(RuntimeError):
         _mxfp4(hk, a2, sa2, b2, sb2, 6)
+
+
+def test_skinny_drawn_shapes_match_oracle(hk):
+    """36 seeded random shapes (M <= 64, N < 400, K up to 150 K-steps with every kind of tail), twelve per
+    format, each against the oracle; MXFP4 scale arrays at a drawn misalignment."""
+    rng = np.random.default_rng(2024)
+    for it in range(36):
+        fmt = ("fp8", "bf16", "mxfp4")[it % 3]
+        M, N = int(rng.integers(1, 65)), int(rng.integers(1, 400))
+        if fmt == "fp8":
+            K = 16 * int(rng.integers(1, 1200))
+            (a, sa), (b, sb) = _fp8_codes(rng, M, K), _fp8_codes(rng, N, K)
+            out, ref = _fp8(hk, a, b, float(sa), float(sb), 8), G.fp8_gemm(a, b, sa, sb)
+        elif fmt == "bf16":
+            K = 8 * int(rng.integers(1, 1200))
+            a = F.bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+            b = F.bf16_round(rng.standard_normal((N, K)).astype(np.float32))
+            out, ref = _bf16(hk, a, b, 6), G.bf16_gemm(a, b)
+        else:
+            K = 32 * int(rng.integers(1, 1200))
+            (a, sa), (b, sb) = _rand_mx(rng, M, K), _rand_mx(rng, N, K)
+            out, ref = _mxfp4(hk, a, sa, b, sb, 6, int(rng.integers(0, 4))), G.mxfp4_gemm(a, sa, b, sb)
+        print(f"skinny drawn {fmt} M={M} N={N} K={K}", flush=True)
+        out = F.bf16_to_f32(out)
+        assert np.isfinite(out).all(), (fmt, M, N, K)
+        assert G.rel_fro_error(out, ref) <= 5e-3, (fmt, M, N, K)
