@@ -51,6 +51,7 @@ TRAFFIC_LEGS = {
     "fp8_gemm_8192": ("calibration", ["fp8_gemm_4wave_ring_kernel<false>"]),
     "mxfp4_gemm": ("mxfp4", ["mxfp4_gemm_4wave_kernel<false>"]),
     "bf16_gemm": ("bf16", ["bf16_gemm_4wave_ring_kernel<false, true>"]),
+    "fp8_gemm_decode_m16": ("decode", ["fp8_gemm_skinny_kernel<1, 4, 4>"]),
     "moe_mxfp4": ("moe_mxfp4", ["moe_topk_softmax_kernel<16>", "moe_sort_quantize_kernel<false>",
                                 "moe_mxfp4_stream4_kernel<0, false, false, true, true>",
                                 "moe_mxfp4_stream4_kernel<1, false, false, false, true>", "moe_unpermute_kernel<4>"]),
@@ -296,7 +297,8 @@ def bench_fp8_decode(torch, hk, warmup, iters, dev, graph=True):
         best = gms if graph else min(plain, split)
         out.append({"shape": f"M={M} N=K=8192", "us_without_workspace": round(plain * 1e3, 1),
                     "us_with_workspace": round(split * 1e3, 1), "us_from_graph": round(gms * 1e3, 1) if graph else None,
-                    "roofline": _roofline("hbm", byts / (best * 1e-3) / 1e9, PEAK_HBM, "GB/s", kernel)})
+                    "roofline": _roofline("hbm", byts / (best * 1e-3) / 1e9, PEAK_HBM, "GB/s", kernel,
+                                          _traffic("fp8_gemm_decode_m16") if M == 16 else None)})
     return out
 
 
