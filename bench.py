@@ -51,7 +51,7 @@ TRAFFIC_LEGS = {
     "fp8_gemm_8192": ("calibration", ["fp8_gemm_4wave_ring_kernel<false>"]),
     "mxfp4_gemm": ("mxfp4", ["mxfp4_gemm_4wave_kernel<false>"]),
     "bf16_gemm": ("bf16", ["bf16_gemm_4wave_ring_kernel<false, true>"]),
-    "fp8_gemm_decode_m16": ("decode", ["fp8_gemm_skinny_kernel<1, 4, 4>"]),
+    "fp8_gemm_decode_m16": ("decode", ["fp8_gemm_skinny_kernel<1, 4, 4, 2, true>"]),
     "moe_mxfp4": ("moe_mxfp4", ["moe_topk_softmax_kernel<16>", "moe_sort_quantize_kernel<false>",
                                 "moe_mxfp4_stream4_kernel<0, false, false, true, true>",
                                 "moe_mxfp4_stream4_kernel<1, false, false, false, true>", "moe_unpermute_kernel<4>"]),
@@ -275,27 +275,44 @@ def bench_bf16(torch, hk, n, warmup, iters, dev):
             "roofline": _roofline("mfma", tf, PEAK_BF16, "TFLOP/s", "bf16 256x256x64 tile kernel", _traffic("bf16_gemm"))}
 
 
+# A decode step multiplies by every weight matrix of a model once, far more bytes than the 256 MB memory-side
+# cache holds; a loop over one and the same matrix would find it there. The decode legs therefore rotate over
+# enough matrices of the shape to exceed twice that cache.
+ROTATE_BYTES = 600e6
+
+
 def bench_fp8_decode(torch, hk, warmup, iters, dev, graph=True):
-    """Decode-like shapes (few rows, N = K = 8192): HBM bound, weights read once. Per-call times include the
-    Python call path (about 9 us, which bounds them from below); `us_from_graph` is the GPU time of the same
-    call replayed from a HIP graph, and the roofline figure uses it when it was measured."""
+    """Decode-like shapes (few rows, N = K = 8192): HBM bound, weights read once, the calls rotating over
+    ROTATE_BYTES of weight matrices. Per-call times include the Python call path (about 9 us, which bounds them
+    from below); `us_from_graph` is the GPU time of the same calls replayed from a HIP graph, and the roofline
+    figure uses it when it was measured."""
     out = []
     g = torch.Generator(device=dev).manual_seed(0)
     N = K = 8192
-    B = torch.randn(N, K, device=dev, generator=g).to(torch.float8_e4m3fn)
+    nb = int(ROTATE_BYTES // (N * K)) + 1
+    Bs = [torch.randn(N, K, device=dev, generator=g).to(torch.float8_e4m3fn) for _ in range(nb)]
     for M in (16, 64, 128):
         A = torch.randn(M, K, device=dev, generator=g).to(torch.float8_e4m3fn)
-        C = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        C = torch.empty(nb, M, N, dtype=torch.bfloat16, device=dev)
         ws = torch.empty(max(16, hk.tk_kernel.fp8_gemm_workspace_bytes(M, N, K)), dtype=torch.uint8, device=dev)
-        _, plain = _timeit(torch, lambda: hk.tk_kernel.dispatch_fp8_gemm(A, B, C, 1.0, 1.0), warmup, iters)
-        _, split = _timeit(torch, lambda: hk.tk_kernel.dispatch_fp8_gemm(A, B, C, 1.0, 1.0, workspace=ws), warmup, iters)
+
+        def cycle(workspace=None):
+            for j in range(nb):
+                hk.tk_kernel.dispatch_fp8_gemm(A, Bs[j], C[j], 1.0, 1.0, workspace=workspace)
+
+        rounds = max(1, iters // nb)
+        _, plain = _timeit(torch, cycle, max(1, warmup // nb), rounds)
+        _, split = _timeit(torch, lambda: cycle(ws), max(1, warmup // nb), rounds)
+        gms = _timeit_graph(torch, lambda: cycle(ws), C, rounds) if graph else None
+        plain, split = plain / nb, split / nb
+        gms = gms / nb if graph else None
         byts = M * K + N * K + 2 * M * N
-        # up to 64 rows both calls run the skinny kernel (no workspace needed); above, the workspace enables split-K
-        kernel = ("fp8_gemm_skinny_kernel" if M <= 64 else
-                  "fp8_gemm_small_tile_kernel<64,4,SPLIT> + splitk_reduce_kernel")
-        gms = _timeit_graph(torch, lambda: hk.tk_kernel.dispatch_fp8_gemm(A, B, C, 1.0, 1.0, workspace=ws), C, iters) if graph else None
+        # up to 64 rows both calls run the skinny kernel (no workspace needed); M = 128 has a 64x64 tile for every CU
+        # and is not split either (split-K is for fewer tiles: at most one for every second CU)
+        kernel = "fp8_gemm_skinny_kernel" if M <= 64 else "fp8_gemm_small_tile_kernel<64,4>"
         best = gms if graph else min(plain, split)
-        out.append({"shape": f"M={M} N=K=8192", "us_without_workspace": round(plain * 1e3, 1),
+        out.append({"shape": f"M={M} N=K=8192, {nb} weight matrices in rotation",
+                    "us_without_workspace": round(plain * 1e3, 1),
                     "us_with_workspace": round(split * 1e3, 1), "us_from_graph": round(gms * 1e3, 1) if graph else None,
                     "roofline": _roofline("hbm", byts / (best * 1e-3) / 1e9, PEAK_HBM, "GB/s", kernel,
                                           _traffic("fp8_gemm_decode_m16") if M == 16 else None)})
@@ -303,21 +320,32 @@ def bench_fp8_decode(torch, hk, warmup, iters, dev, graph=True):
 
 
 def bench_mxfp4_decode(torch, hk, warmup, iters, dev, graph=True):
-    """MXFP4 decode-like shapes: few rows against a weight matrix that is read once (timings as in bench_fp8_decode)."""
+    """MXFP4 decode-like shapes: few rows against weight matrices that are read once (rotation and timings as in
+    bench_fp8_decode)."""
     out = []
     g = torch.Generator(device=dev).manual_seed(0)
     for M, N, K in ((16, 8192, 8192), (16, 4096, 14336)):
+        nb = int(ROTATE_BYTES // (N * (K // 2 + K // 32))) + 1
         A, SA = hk.quant.quantize_mxfp4(torch.randn(M, K, device=dev, generator=g))
-        B, SB = hk.quant.quantize_mxfp4(torch.randn(N, K, device=dev, generator=g))
-        C = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        Ws = [hk.quant.quantize_mxfp4(torch.randn(N, K, device=dev, generator=g)) for _ in range(nb)]
+        C = torch.empty(nb, M, N, dtype=torch.bfloat16, device=dev)
         ws = torch.empty(max(16, hk.tk_kernel.mxfp4_gemm_workspace_bytes(M, N, K)), dtype=torch.uint8, device=dev)
-        _, plain = _timeit(torch, lambda: hk.tk_kernel.dispatch_mxfp4_gemm(A, SA, B, SB, C), warmup, iters)
-        _, split = _timeit(torch, lambda: hk.tk_kernel.dispatch_mxfp4_gemm(A, SA, B, SB, C, workspace=ws), warmup, iters)
+
+        def cycle(workspace=None):
+            for j in range(nb):
+                hk.tk_kernel.dispatch_mxfp4_gemm(A, SA, Ws[j][0], Ws[j][1], C[j], workspace=workspace)
+
+        rounds = max(1, iters // nb)
+        _, plain = _timeit(torch, cycle, max(1, warmup // nb), rounds)
+        _, split = _timeit(torch, lambda: cycle(ws), max(1, warmup // nb), rounds)
+        gms = _timeit_graph(torch, cycle, C, rounds) if graph else None
+        plain, split = plain / nb, split / nb
+        gms = gms / nb if graph else None
         byts = (M + N) * (K // 2 + K // 32) + 2 * M * N
-        # both calls run the skinny kernel at these shapes (no workspace needed)
-        gms = _timeit_graph(torch, lambda: hk.tk_kernel.dispatch_mxfp4_gemm(A, SA, B, SB, C), C, iters) if graph else None
         best = gms if graph else min(plain, split)
-        out.append({"shape": f"M={M} N={N} K={K}", "us_without_workspace": round(plain * 1e3, 1),
+        # both calls run the skinny kernel at these shapes (no workspace needed)
+        out.append({"shape": f"M={M} N={N} K={K}, {nb} weight matrices in rotation",
+                    "us_without_workspace": round(plain * 1e3, 1),
                     "us_with_workspace": round(split * 1e3, 1), "us_from_graph": round(gms * 1e3, 1) if graph else None,
                     "roofline": _roofline("hbm", byts / (best * 1e-3) / 1e9, PEAK_HBM, "GB/s",
                                           "mxfp4_gemm_skinny_kernel")})

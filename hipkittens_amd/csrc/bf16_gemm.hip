@@ -171,12 +171,12 @@ static int launch_bf16_prodcons(const void* A, const void* B, void* C, int M, in
 }
 
 // The skinny kernel (gemm_skinny.h) with the BF16 MFMA. K: the operands' row length in bytes.
-template <int R, int NW, int D>
+template <int R, int NW, int D, int NF, bool NT>
 __global__ __launch_bounds__(64 * NW) void bf16_gemm_skinny_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
     int M, int N, int K, float alpha) {
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
-    gemm_skinny_body<Bf16Mma, R, NW, D>(smem, A, B, C, M, N, K, alpha);
+    gemm_skinny_body<Bf16Mma, R, NW, D, NF, NT>(smem, A, B, C, M, N, K, alpha);
 }
 static int launch_bf16_skinny(const void* A, const void* B, void* C, int M, int N, int K_elems, hipStream_t stream) {
     const int K = 2 * K_elems;

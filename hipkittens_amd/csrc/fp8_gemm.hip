@@ -135,12 +135,12 @@ __global__ __launch_bounds__(256) void fp8_gemm_portable_kernel(
 }
 
 // The skinny kernel (gemm_skinny.h) with the FP8 MFMA.
-template <int R, int NW, int D>
+template <int R, int NW, int D, int NF, bool NT>
 __global__ __launch_bounds__(64 * NW) void fp8_gemm_skinny_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
     int M, int N, int K, float alpha) {
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
-    gemm_skinny_body<Fp8Mma, R, NW, D>(smem, A, B, C, M, N, K, alpha);
+    gemm_skinny_body<Fp8Mma, R, NW, D, NF, NT>(smem, A, B, C, M, N, K, alpha);
 }
 static int launch_skinny(const void* A, const void* B, void* C, int M, int N, int K, float alpha, hipStream_t stream) {
     HK_SKINNY_DISPATCH(fp8_gemm_skinny_kernel);

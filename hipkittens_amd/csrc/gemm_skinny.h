@@ -45,19 +45,21 @@ __device__ __forceinline__ v2i scale_bytes_direct(v4i srd, uint32_t off) {
 struct SkinnyScales {
     const uint8_t* SA; const uint8_t* SB; int sa_pitch, sb_pitch, row_bytes;
 };
-template <typename MMA, int R, int NW, int D>
+template <typename MMA, int R, int NW, int D, int NF = 2, bool NT = false>
 __device__ __forceinline__ void gemm_skinny_body(
     uint8_t* smem, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint16_t* __restrict__ C,
     int M, int N, int K, float alpha, SkinnyScales sc = SkinnyScales{nullptr, nullptr, 0, 0, 0}) {
     constexpr bool kScaled = MMA::kScaled;
-    constexpr int kWBytes = 32 * BK, kStage = kWBytes + 16 * R * BK, kRegion = (D + (kScaled ? 2 : 0)) * kStage;
-    constexpr int LPT = 4 + 2 * R;   // loads per K-step (and per tile of scales)
+    constexpr int kRowsB = 16 * NF;   // rows of B per workgroup
+    constexpr int kWBytes = kRowsB * BK, kStage = kWBytes + 16 * R * BK, kRegion = (D + (kScaled ? 2 : 0)) * kStage;
+    constexpr int LPT = 2 * NF + 2 * R;   // loads per K-step (and per tile of scales)
     static_assert(D >= 2 && (D - 1 + (kScaled ? 1 : 0)) * LPT < 64, "vmcnt range");
-    static_assert(NW * R * 2 * 1024 <= NW * kRegion, "the partial sums reuse the stages");
+    static_assert(NF == 1 || NF == 2, "one or two fragments of B per workgroup");
+    static_assert(NW * R * NF * 1024 <= NW * kRegion, "the partial sums reuse the stages");
     const int lane = lane_id(), w = wave_id();
     const uint32_t r = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * 32;
-    const int rows_b = N - n0 < 32 ? N - n0 : 32;
+    const int n0 = blockIdx.x * kRowsB;
+    const int rows_b = N - n0 < kRowsB ? N - n0 : kRowsB;
     const v4i srd_b = make_srd(B + (size_t)n0 * K, (uint32_t)rows_b * (uint32_t)K);
     const v4i srd_a = make_srd(A, (uint32_t)M * (uint32_t)K);
     const int nk = (K + BK - 1) / BK;
@@ -80,8 +82,11 @@ __device__ __forceinline__ void gemm_skinny_body(
         const uint32_t k0 = (uint32_t)kt * BK, dst = region + (uint32_t)stage * kStage;
         const bool last = kt == nk - 1;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            dma16(srd_b, dst + i * 1024, (voff[i & 1] + (uint32_t)(i >> 1) * 16u * (uint32_t)K) | (last ? tail_or[i & 1] : 0u), k0);
+        for (int i = 0; i < 2 * NF; ++i) {
+            const uint32_t vo = (voff[i & 1] + (uint32_t)(i >> 1) * 16u * (uint32_t)K) | (last ? tail_or[i & 1] : 0u);
+            if constexpr (NT) dma16_nt(srd_b, dst + i * 1024, vo, k0);
+            else dma16(srd_b, dst + i * 1024, vo, k0);
+        }
 #pragma unroll
         for (int i = 0; i < 2 * R; ++i)
             dma16(srd_a, dst + kWBytes + i * 1024, (voff[i & 1] + (uint32_t)(i >> 1) * 16u * (uint32_t)K) | (last ? tail_or[i & 1] : 0u), k0);
@@ -103,7 +108,7 @@ __device__ __forceinline__ void gemm_skinny_body(
     auto issue_scales = [&](int c) {
         const uint32_t dst = region + (uint32_t)(D + (c & 1)) * kStage, off = (uint32_t)c * 128u;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 2 * NF; ++i)
             dma16(srd_sb, dst + i * 1024, voff_sb[i & 1] + (uint32_t)(i >> 1) * 16u * (uint32_t)sc.sb_pitch, off);
 #pragma unroll
         for (int i = 0; i < 2 * R; ++i)
@@ -123,9 +128,11 @@ __device__ __forceinline__ void gemm_skinny_body(
 
     const uint32_t rd_lo = region + r * 128u + swz_chunk(r, g) * 16u;
     const uint32_t rd_hi = region + r * 128u + swz_chunk(r, g + 4) * 16u;
-    v4f acc[R][2];
+    v4f acc[R][NF];
 #pragma unroll
-    for (int i = 0; i < R; ++i) acc[i][0] = acc[i][1] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < R; ++i)
+#pragma unroll
+        for (int f = 0; f < NF; ++f) acc[i][f] = v4f{0.f, 0.f, 0.f, 0.f};
 
     // the wave's first tile of scales goes out in front of its first K-step: it has landed when that K-step has
     // (loads complete in order)
@@ -149,18 +156,18 @@ __device__ __forceinline__ void gemm_skinny_body(
         // the stage of K-step kt - 1 is free: its reads were waited for before its MFMAs
         if (kt + D - 1 < n) issue(st == 0 ? D - 1 : st - 1, kt + D - 1);
         const uint32_t so = (uint32_t)st * kStage;
-        v8i wf[2];
+        v8i wf[NF];
 #pragma unroll
-        for (int f = 0; f < 2; ++f) wf[f] = lds_frag(rd_lo + so, rd_hi + so, f * 16 * BK);
+        for (int f = 0; f < NF; ++f) wf[f] = lds_frag(rd_lo + so, rd_hi + so, f * 16 * BK);
         if constexpr (kScaled) {
-            v2i ws[2], as[R];
+            v2i ws[NF], as[R];
             if ((sc.row_bytes & 3) != 0 && ks == nk - 1) {
                 // The range check of a descriptor works on dwords: the dword of a scale tile that reaches across
                 // the end of the operand's last row arrives as zero, and with it the last row_bytes % 4 scales of
                 // that row. They belong to the last K-step, whose scale bytes every lane therefore fetches itself,
                 // a byte at a time (the wave's loads have all landed: this is its last K-step).
 #pragma unroll
-                for (int f = 0; f < 2; ++f)
+                for (int f = 0; f < NF; ++f)
                     ws[f] = scale_bytes_direct(srd_sb, (16u * f + r) * (uint32_t)sc.sb_pitch + (uint32_t)ks * 8u + g);
 #pragma unroll
                 for (int i = 0; i < R; ++i)
@@ -171,7 +178,7 @@ __device__ __forceinline__ void gemm_skinny_body(
                                        swz_chunk(r, (uint32_t)(ks & 15) >> 1) * 16u + (uint32_t)(ks & 1) * 8u;
                 const uint32_t sh = 8u * g;
 #pragma unroll
-                for (int f = 0; f < 2; ++f) {
+                for (int f = 0; f < NF; ++f) {
                     ws[f] = *(lds_v2i_t*)(uintptr_t)(sbase + f * 16 * BK);
                     ws[f].x = (int)((uint32_t)ws[f].x >> sh); ws[f].y = (int)((uint32_t)ws[f].y >> sh);
                 }
@@ -185,14 +192,14 @@ __device__ __forceinline__ void gemm_skinny_body(
             for (int i = 0; i < R; ++i) {
                 const v8i af = lds_frag(rd_lo + so, rd_hi + so, kWBytes + i * 16 * BK);
 #pragma unroll
-                for (int f = 0; f < 2; ++f) MMA::mma(acc[i][f], wf[f], af, ws[f], as[i]);
+                for (int f = 0; f < NF; ++f) MMA::mma(acc[i][f], wf[f], af, ws[f], as[i]);
             }
         } else {
 #pragma unroll
             for (int i = 0; i < R; ++i) {
                 const v8i af = lds_frag(rd_lo + so, rd_hi + so, kWBytes + i * 16 * BK);
 #pragma unroll
-                for (int f = 0; f < 2; ++f) MMA::mma(acc[i][f], wf[f], af);
+                for (int f = 0; f < NF; ++f) MMA::mma(acc[i][f], wf[f], af);
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this stage's reads are done before a later load may overwrite it
@@ -201,19 +208,19 @@ __device__ __forceinline__ void gemm_skinny_body(
     // every wave is done with its stages (its loads have landed, its reads are complete): the partial sums take
     // their place
     __syncthreads();
-    v4f* red = (v4f*)smem;   // [NW][R][2][64]
+    v4f* red = (v4f*)smem;   // [NW][R][NF][64]
 #pragma unroll
     for (int i = 0; i < R; ++i)
 #pragma unroll
-        for (int f = 0; f < 2; ++f) red[((w * R + i) * 2 + f) * 64 + lane] = acc[i][f];
+        for (int f = 0; f < NF; ++f) red[((w * R + i) * NF + f) * 64 + lane] = acc[i][f];
     __syncthreads();
-    for (int t = threadIdx.x; t < R * 128; t += 64 * NW) {
+    for (int t = threadIdx.x; t < R * NF * 64; t += 64 * NW) {
         const int l = t & 63;
         v4f sum = red[t];
 #pragma unroll
-        for (int ww = 1; ww < NW; ++ww) sum += red[ww * R * 128 + t];
+        for (int ww = 1; ww < NW; ++ww) sum += red[ww * R * NF * 64 + t];
         sum *= alpha;
-        const int i = t >> 7, f = (t >> 6) & 1;
+        const int i = t / (NF * 64), f = (t >> 6) % NF;
         const int row = 16 * i + (l & 15), col = n0 + 16 * f + 4 * (l >> 4);
         if (row < M) {
             uint16_t* out = C + (size_t)row * N + col;
@@ -229,42 +236,67 @@ __device__ __forceinline__ void gemm_skinny_body(
     }
 }
 
-constexpr int skinny_lds_bytes(int R, int NW, int D, bool scaled = false) { return NW * (D + (scaled ? 2 : 0)) * (32 + 16 * R) * BK; }
+constexpr int skinny_lds_bytes(int R, int NW, int D, bool scaled = false, int NF = 2) {
+    return NW * (D + (scaled ? 2 : 0)) * (16 * NF + 16 * R) * BK;
+}
 
 // Whether a GEMM entry point takes this kernel when the caller does not pin one. nk: K-steps; with_ws: the caller
-// gave a split-K workspace. From a sweep on an MI355X (M = 16 / 32 / 64, N = 512 ... 32768, K = 512 ... 16384
-// bytes per row, against the tile kernels with and without split-K): up to 32 rows it wins by 2 to 64 % while it
-// has at most 1.75 workgroups per CU (N <= 14336 on 256 CUs) and loses by 2 to 60 % from 3.5 on; with 33 to 64
-// rows it wins up to one workgroup per CU, except against split-K on few workgroups with a very long K.
-// The MXFP4 form (quarter_wgs_per_cu = 8) wins by 20 to 75 % up to two workgroups per CU
-// (N <= 16384) against the scaled tile kernels, whose scale fetches weigh more on few rows.
-static inline bool use_skinny(int M, int N, int nk, bool with_ws, int cus, int max_m = kSkinnyMaxM,
-                              int quarter_wgs_per_cu = 7) {
+// gave a split-K workspace. From sweeps on an MI355X (M = 16 / 32 / 64, N = 512 ... 65536, K = 512 ... 16384
+// bytes per row, against the tile kernels with and without split-K, the calls rotating over more weight matrices
+// than the memory-side cache holds): up to 32 rows it wins by 2 to 64 % while it has at most one workgroup of 32
+// rows per CU (N <= 8192 on 256 CUs); beyond that, up to 16 rows, from 32 K-steps on (8 to 25 %; with a shorter K,
+// or with 17 to 32 rows and a long K, the 64x64-tile kernel's many tiles win by up to 20 %); with 33 to 64 rows it
+// wins up to one workgroup per CU, except against split-K on few workgroups with a very long K. The MXFP4 form (wgs_per_cu = 2) wins by 5 to 75 % up to
+// two workgroups per CU (N <= 16384) against the scaled tile kernels, whose scale fetches weigh more on few rows.
+static inline bool use_skinny(int M, int N, int nk, bool with_ws, int cus, int max_m = kSkinnyMaxM, int wgs_per_cu = 1) {
     if (M > max_m) return false;
     const long long wgs = (N + 31) / 32;
-    if (M <= 32) return wgs * 4 <= (long long)quarter_wgs_per_cu * cus;
-    if (wgs > cus) return false;
+    if (M <= 32) return wgs <= (long long)wgs_per_cu * cus || (nk >= 32 && (M <= 16 || wgs_per_cu > 1));
+    if (wgs > (long long)wgs_per_cu * cus) return false;
     return !(with_ws && wgs * 2 <= cus && nk >= 96);
 }
 
-// KERNEL<R, NW, D>: the format's __global__ instantiation of the body
-#define HK_SKINNY_LAUNCH(KERNEL, R, NW, D)                                                                     \
+// KERNEL<R, NW, D, NF, NT>: the format's __global__ instantiation of the body
+#define HK_SKINNY_LAUNCH(KERNEL, R, NW, D, NF, NT)                                                             \
     do {                                                                                                       \
-        auto kern = KERNEL<R, NW, D>;                                                                          \
-        constexpr int lds_bytes = skinny_lds_bytes(R, NW, D);                                                  \
+        auto kern = KERNEL<R, NW, D, NF, NT>;                                                                  \
+        constexpr int lds_bytes = skinny_lds_bytes(R, NW, D, false, NF);                                       \
         static_assert(lds_bytes <= 160 * 1024, "LDS of one CU");                                               \
         static DeviceOnce configured;                                                                          \
         if (!set_lds_limit_once((const void*)kern, lds_bytes, configured)) return HK_ERR_LAUNCH;               \
-        hipLaunchKernelGGL(kern, dim3((N + 31) / 32), dim3(64 * NW), lds_bytes, stream, (const uint8_t*)A,     \
-                           (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha);                                   \
+        hipLaunchKernelGGL(kern, dim3((N + 16 * NF - 1) / (16 * NF)), dim3(64 * NW), lds_bytes, stream,        \
+                           (const uint8_t*)A, (const uint8_t*)B, (uint16_t*)C, M, N, K, alpha);                \
         return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;                                        \
     } while (0)
-// waves x stages per row count: the fastest of the combinations measured on an MI355X (N, K from 1024 to 28672;
-// eight waves with three stages, two with seven and others are within 15 % of these). K in bytes per row.
-#define HK_SKINNY_DISPATCH(KERNEL)                                \
-    if (M <= 16) HK_SKINNY_LAUNCH(KERNEL, 1, 4, 4);               \
-    if (M <= 32) HK_SKINNY_LAUNCH(KERNEL, 2, 4, 3);               \
-    HK_SKINNY_LAUNCH(KERNEL, 4, 4, 3)
+// What a launch of the skinny kernel picks besides R (the rows of A):
+//  - waves x stages per row count: the fastest of the combinations measured on an MI355X (N, K from 1024 to
+//    28672; eight waves with three stages, two with seven and others are within 15 % of these);
+//  - NF, the rows of B per workgroup: 16 instead of 32 while 32 would leave half of the CUs or more without a
+//    workgroup (N <= 4096 on 256 CUs): a CU can only have so many bytes in flight, so weights that stream from
+//    HBM want every CU (M = 16, N = 4096, K = 14336: 19.6 -> 12.9 us; N = 5760, 180 workgroups of 32 rows: 7.1
+//    against 7.6 us with 16);
+//  - NT, the non-temporal hint on the loads of B, from 8 MB of B on. Measured with the calls rotating over more
+//    weight matrices than the 256 MB memory-side cache holds, which is what a model's decode step does, the hint
+//    gains 3 to 18 % (M = 16, N = K = 8192: 14.2 -> 12.0 us); a benchmark that multiplies by the same 64 MB again
+//    and again finds them in that cache and loses it with the hint, which is why small matrices, which a small
+//    model may really keep there, go without.
+// K in bytes per row.
+constexpr long long kSkinnyNtBytes = 8ll << 20;
+#define HK_SKINNY_PICK(KERNEL, R, NW, D)                                                          \
+    do {                                                                                          \
+        if (nf1) {                                                                                \
+            if (nt) HK_SKINNY_LAUNCH(KERNEL, R, NW, D, 1, true);                                  \
+            HK_SKINNY_LAUNCH(KERNEL, R, NW, D, 1, false);                                         \
+        }                                                                                         \
+        if (nt) HK_SKINNY_LAUNCH(KERNEL, R, NW, D, 2, true);                                      \
+        HK_SKINNY_LAUNCH(KERNEL, R, NW, D, 2, false);                                             \
+    } while (0)
+#define HK_SKINNY_DISPATCH(KERNEL)                                                                \
+    const bool nf1 = 2ll * ((N + 31) / 32) <= moe_num_compute_units();                            \
+    const bool nt = (long long)N * K >= kSkinnyNtBytes;                                           \
+    if (M <= 16) HK_SKINNY_PICK(KERNEL, 1, 4, 4);                                                 \
+    if (M <= 32) HK_SKINNY_PICK(KERNEL, 2, 4, 3);                                                 \
+    HK_SKINNY_PICK(KERNEL, 4, 4, 3)
 // with block scales two slots of scales stand beside the stages: four waves with three stages fill the LDS of a CU
 // at R = 2, and R = 4 (up to 64 rows) has room for two waves with four stages
 constexpr int kSkinnyMaxMScaled = 64;

@@ -257,8 +257,9 @@ static __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* 
 //     tile count cannot: 72 tiles of 256 are one round where their 288 tiles of 128 are two (the large tile
 //     wins by 4-12 % from a K of about 4096 elements on), 64 tiles of 256 are one round of four times the work
 //     of the single round of 256 small tiles (the small tile wins by 60 %). Measured against the best of the
-//     three kernels on 360 shapes per format, the rule alone is more than 5 % behind on 8 / 6 / 10 shapes
-//     (FP8 / BF16 / MXFP4; the thresholds it replaced: 13 / 18 / 19);
+//     three kernels on 360 shapes per format, every launch on another copy of B (a model's weights come from HBM, not
+//     from the memory-side cache), the rule alone is more than 5 % behind on 9 / 22 / 20 shapes (FP8 / BF16 /
+//     MXFP4), mostly by 5 to 10 % where a long B is read by several rows of small tiles;
 //  2. a generated table of the shapes on which a sweep found the rule's choice more than a few percent behind
 //     another tile (tile_table.inc, written by `python -m hipkittens_amd.tile_sweep FORMAT --emit`; the
 //     counterpart of the reference's per-shape analysis/baselines/gemm/utils/tuned.yaml). An entry is keyed by
@@ -296,7 +297,7 @@ static inline int pick_tile(int fmt, int M, int N, int nk, TileRule r, bool cons
     return pick_tile_rule(M, N, nk, r, cus);
 }
 // the formats' constants (K-steps: 128 bytes of an operand row)
-constexpr TileRule kTileRuleFp8{{7.59f, 3.08f, 2.08f}, {0.984f, 0.571f, 0.333f}};
+constexpr TileRule kTileRuleFp8{{7.43f, 3.28f, 2.02f}, {1.078f, 0.585f, 0.372f}};
 constexpr TileRule kTileRuleBf16{{7.75f, 3.15f, 2.17f}, {1.051f, 0.562f, 0.336f}};
 constexpr TileRule kTileRuleMxfp4{{7.71f, 3.13f, 1.94f}, {1.316f, 0.767f, 0.549f}};
 
@@ -309,8 +310,10 @@ static inline int splitk_ranges(int M, int N, int K, int min_nk = 48) {
     const long long tiles = (((long long)M + kTinyTile - 1) / kTinyTile) * (((long long)N + kTinyTile - 1) / kTinyTile);
     const long long nk = ((long long)K + BK - 1) / BK;
     const int cus = moe_num_compute_units();   // 256 when no device can be queried
-    // shorter K: the 64x64-tile kernel without a second launch is as fast or faster
-    if (tiles > cus || nk < min_nk) return 1;
+    // shorter K: the 64x64-tile kernel without a second launch is as fast or faster; more than one tile for every
+    // second CU: with B coming from HBM (every launch on another weight matrix) the split measured 5 to 25 % slower
+    // than the plain kernel up to 128 K-steps, and within 8 % of it at 256
+    if (tiles * 2 > cus || nk < min_nk) return 1;
     long long s = 2 * cus / tiles;
     if (s > nk / 4) s = nk / 4;
     if (s > 16) s = 16;

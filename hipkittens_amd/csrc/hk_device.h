@@ -54,6 +54,18 @@ __device__ __forceinline__ void dma16(v4i srd, uint32_t lds_base, uint32_t voff,
         : "memory", "m0");
 }
 
+// dma16 with the non-temporal hint, for data that is read once (the weights of a decode GEMM): it need not
+// displace what the caches hold for re-use.
+__device__ __forceinline__ void dma16_nt(v4i srd, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dwordx4 %1, %2, %3 offen nt lds"
+        :
+        : "s"(lds_base), "v"(voff), "s"(srd), "s"(soff)
+        : "memory", "m0");
+}
+
 // 4-byte direct global->LDS load (64 lanes -> 256 contiguous LDS bytes).
 __device__ __forceinline__ void dma4(v4i srd, uint32_t lds_base, uint32_t voff, uint32_t soff) {
     asm volatile(

@@ -371,32 +371,43 @@ __global__ __launch_bounds__(256) void mxfp4_gemm_small_tile_kernel(
 
 // The skinny kernel (gemm_skinny.h) with the scaled FP4 MFMA, for at most 64 rows of A. K: the operands' row
 // length in bytes; scale rows of any pitch and alignment, row_bytes scale bytes each.
-template <int R, int NW, int D>
+template <int R, int NW, int D, int NF, bool NT>
 __global__ __launch_bounds__(64 * NW) void mxfp4_gemm_skinny_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ SA, const uint8_t* __restrict__ B,
     const uint8_t* __restrict__ SB, uint16_t* __restrict__ C, int M, int N, int K, int sa_pitch, int sb_pitch,
     int row_bytes) {
     extern __shared__ __attribute__((aligned(2048))) uint8_t smem[];
-    gemm_skinny_body<Mxfp4Mma, R, NW, D>(smem, A, B, C, M, N, K, 1.0f, SkinnyScales{SA, SB, sa_pitch, sb_pitch, row_bytes});
+    gemm_skinny_body<Mxfp4Mma, R, NW, D, NF, NT>(smem, A, B, C, M, N, K, 1.0f, SkinnyScales{SA, SB, sa_pitch, sb_pitch, row_bytes});
 }
-template <int R, int NW, int D>
+template <int R, int NW, int D, int NF, bool NT>
 static int launch_mxfp4_skinny_kernel(const void* A, const void* SA, const void* B, const void* SB, void* C, int M,
                                       int N, int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
-    auto kern = mxfp4_gemm_skinny_kernel<R, NW, D>;
-    constexpr int lds_bytes = skinny_lds_bytes(R, NW, D, true);
+    auto kern = mxfp4_gemm_skinny_kernel<R, NW, D, NF, NT>;
+    constexpr int lds_bytes = skinny_lds_bytes(R, NW, D, true, NF);
     static_assert(lds_bytes <= 160 * 1024, "LDS of one CU");
     static DeviceOnce configured;
     if (!set_lds_limit_once((const void*)kern, lds_bytes, configured)) return HK_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3((N + 31) / 32), dim3(64 * NW), lds_bytes, stream, (const uint8_t*)A,
+    hipLaunchKernelGGL(kern, dim3((N + 16 * NF - 1) / (16 * NF)), dim3(64 * NW), lds_bytes, stream, (const uint8_t*)A,
                        (const uint8_t*)SA, (const uint8_t*)B, (const uint8_t*)SB, (uint16_t*)C, M, N, K / 2, sa_pitch,
                        sb_pitch, K / 32);
     return hipGetLastError() == hipSuccess ? HK_OK : HK_ERR_LAUNCH;
 }
+// rows of B per workgroup and the non-temporal hint as for the other formats (HK_SKINNY_DISPATCH)
+template <int R, int NW, int D>
+static int launch_mxfp4_skinny_pick(const void* A, const void* SA, const void* B, const void* SB, void* C, int M, int N,
+                                    int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
+    const bool nf1 = 2ll * ((N + 31) / 32) <= moe_num_compute_units();
+    const bool nt = (long long)N * (K / 2) >= kSkinnyNtBytes;
+    if (nf1) return nt ? launch_mxfp4_skinny_kernel<R, NW, D, 1, true>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream)
+                       : launch_mxfp4_skinny_kernel<R, NW, D, 1, false>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
+    return nt ? launch_mxfp4_skinny_kernel<R, NW, D, 2, true>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream)
+              : launch_mxfp4_skinny_kernel<R, NW, D, 2, false>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
+}
 static int launch_mxfp4_skinny(const void* A, const void* SA, const void* B, const void* SB, void* C, int M, int N,
                                int K, int sa_pitch, int sb_pitch, hipStream_t stream) {
-    if (M <= 16) return launch_mxfp4_skinny_kernel<1, 4, 4>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
-    if (M <= 32) return launch_mxfp4_skinny_kernel<2, 4, 3>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
-    return launch_mxfp4_skinny_kernel<4, 2, 4>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
+    if (M <= 16) return launch_mxfp4_skinny_pick<1, 4, 4>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
+    if (M <= 32) return launch_mxfp4_skinny_pick<2, 4, 3>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
+    return launch_mxfp4_skinny_pick<4, 2, 4>(A, SA, B, SB, C, M, N, K, sa_pitch, sb_pitch, stream);
 }
 
 // What the tile kernels need to know about the scale rows (see the head of the file).
@@ -559,7 +570,7 @@ static int mxfp4_gemm_impl(const void* A, const void* A_scales, int sa_pitch, co
         const int tile = pick_tile(kFmtMxfp4, M, N, (K / 2 + BK - 1) / BK, kTileRuleMxfp4);
         variant = !(sr.ok && size_ok) ? 0 : tile == kTinyTile ? 3 : tile == kSmallTile ? 2 : 1;
         // few rows: one pass over B by the skinny kernel where that is faster (use_skinny); it takes any scale rows
-        if (size_ok && use_skinny(M, N, (K / 2 + BK - 1) / BK, false, moe_num_compute_units(), kSkinnyMaxMScaled, 8)) variant = 6;
+        if (size_ok && use_skinny(M, N, (K / 2 + BK - 1) / BK, false, moe_num_compute_units(), kSkinnyMaxMScaled, 2)) variant = 6;
     }
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {
@@ -637,7 +648,7 @@ extern "C" int hk_mxfp4_gemm_ws(const void* A, const void* A_scales, int a_scale
     if (!A || !B || !C) return HK_ERR_NULL_POINTER;
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)workspace) & 15u) return HK_ERR_BAD_ALIGNMENT;
     // the skinny kernel adds its partial sums inside the workgroup and leaves the workspace alone
-    if (use_skinny(M, N, (K / 2 + BK - 1) / BK, true, moe_num_compute_units(), kSkinnyMaxMScaled, 8))
+    if (use_skinny(M, N, (K / 2 + BK - 1) / BK, true, moe_num_compute_units(), kSkinnyMaxMScaled, 2))
         return mxfp4_gemm_impl(A, A_scales, a_scale_pitch, B, B_scales, b_scale_pitch, C, M, N, K, 6, stream);
     const bool edge = (M % kTinyTile) != 0 || (N % kTinyTile) != 0;
     return edge ? launch_mxfp4_splitk<true>(A, A_scales, B, B_scales, C, M, N, K, a_scale_pitch, b_scale_pitch, sr,

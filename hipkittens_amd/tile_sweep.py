@@ -5,8 +5,8 @@ and writes the per-shape table that the library's choice of tile consults.
     python -m hipkittens_amd.tile_sweep fp8|bf16|mxfp4 --emit     sweep the larger grid, rewrite the format's
                                                                   entries of csrc/tile_table.inc, then rebuild
 
-For each shape it prints the GPU time (a HIP graph of 20 launches between two events, best of three
-replays, in two passes over the kernels, forwards and backwards) of the default choice (variant -1; with at
+For each shape it prints the GPU time (a HIP graph of 20 launches between two events, the launches rotating
+over copies of B that exceed the memory-side cache, as a model's weights do; best of three replays, in two passes over the kernels, forwards and backwards) of the default choice (variant -1; with at
 most 64 rows of A that can be the skinny kernel, csrc/gemm_skinny.h, instead of a tile kernel), of the 256x256,
 128x128 and 64x64 tile kernels, and of the call with a workspace where the library would split K without the
 skinny kernel, and marks the shapes where the default is more than 5 % behind the best tile kernel.
@@ -62,24 +62,49 @@ def _time_us(fn, iters=20):
     return best * 1000.0
 
 
+# B is the weight matrix of a layer: in a model it comes from HBM every time, because between two uses of it the
+# other layers' weights have passed through the 256 MB memory-side cache. Timing one and the same B again and again
+# would find it in that cache whenever it fits, and would tune the choice of tile for a case that does not occur.
+# The calls therefore rotate over copies of B that together exceed twice the cache (A, the activations, stays).
+ROTATE_BYTES = 600e6
+ROTATE_MAX = 24
+
+
+def _copies(b_bytes):
+    return 1 if b_bytes >= 256e6 else min(ROTATE_MAX, int(ROTATE_BYTES // b_bytes) + 1)
+
+
 def _problem(fmt, M, N, K, dev):
     C = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    turn = [0]
+
+    def rotating(items):
+        def nxt():
+            turn[0] = (turn[0] + 1) % len(items)
+            return items[turn[0]]
+        return nxt
+
     if fmt == "fp8":
         A = torch.randn(M, K, device=dev).to(torch.float8_e4m3fn)
-        B = torch.randn(N, K, device=dev).to(torch.float8_e4m3fn)
-        return (lambda v, ws=None: tk.dispatch_fp8_gemm(A, B, C, 1.0, 1.0, variant=v, workspace=ws),
+        B = rotating([torch.randn(N, K, device=dev).to(torch.float8_e4m3fn) for _ in range(_copies(N * K))])
+        return (lambda v, ws=None: tk.dispatch_fp8_gemm(A, B(), C, 1.0, 1.0, variant=v, workspace=ws),
                 tk.fp8_gemm_workspace_bytes(M, N, K))
     if fmt == "bf16":
         A = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
-        B = torch.randn(N, K, device=dev, dtype=torch.bfloat16)
-        return (lambda v, ws=None: tk.dispatch_bf16_gemm(A, B, C, variant=v, workspace=ws),
+        B = rotating([torch.randn(N, K, device=dev, dtype=torch.bfloat16) for _ in range(_copies(2 * N * K))])
+        return (lambda v, ws=None: tk.dispatch_bf16_gemm(A, B(), C, variant=v, workspace=ws),
                 tk.bf16_gemm_workspace_bytes(M, N, K))
     A = torch.randint(0, 256, (M, K // 2), dtype=torch.uint8, device=dev)
-    B = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, device=dev)
     As = torch.randint(120, 130, (M, K // 32), dtype=torch.uint8, device=dev)
-    Bs = torch.randint(120, 130, (N, K // 32), dtype=torch.uint8, device=dev)
-    return (lambda v, ws=None: tk.dispatch_mxfp4_gemm(A, As, B, Bs, C, variant=v, workspace=ws),
-            tk.mxfp4_gemm_workspace_bytes(M, N, K))
+    B = rotating([(torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, device=dev),
+                   torch.randint(120, 130, (N, K // 32), dtype=torch.uint8, device=dev))
+                  for _ in range(_copies(N * (K // 2 + K // 32)))])
+
+    def run(v, ws=None):
+        b, bs = B()
+        tk.dispatch_mxfp4_gemm(A, As, b, bs, C, variant=v, workspace=ws)
+
+    return run, tk.mxfp4_gemm_workspace_bytes(M, N, K)
 
 
 def _k_steps(fmt, K):

@@ -60,8 +60,8 @@ int hk_gemm_tile_choice(int format, int M, int N, int K, int consult_table);
 int hk_fp8_gemm(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
                 int M, int N, int K, float scale_a, float scale_b, void* stream);
 
-/* The same GEMM with an optional workspace, for decode-like shapes (at most one 64x64 tile of C per
- * CU and K >= 6144, e.g. M <= 128 with N = K = 8192): the K range is split over several workgroups per
+/* The same GEMM with an optional workspace, for decode-like shapes (at most one 64x64 tile of C for
+ * every second CU and K >= 6144, e.g. M = 128 with N = 4096, K = 8192): the K range is split over several workgroups per
  * tile, which write fp32 partial sums to the workspace, and a second kernel adds them in a fixed
  * order (deterministic) and rounds to bf16. hk_fp8_gemm_workspace_bytes returns the bytes this
  * needs, or 0 when the shape would not be split; with a NULL or too small workspace, or such a
