@@ -8,8 +8,8 @@
 namespace hk {
 
 // Few rows of A against a long weight matrix (M <= 16 R): the GEMM is then one pass over
-// B at HBM speed. A workgroup of NW waves owns 32 rows of B (32 columns of C, all rows of A); wave w walks
-// its share of the K-steps on its own, without workgroup barriers: it fetches the 32 x 128-byte piece of B
+// B at HBM speed. A workgroup of NW waves owns 16 NF rows of B (as many columns of C, all rows of A); wave w walks
+// its share of the K-steps on its own, without workgroup barriers: it fetches the 16 NF x 128-byte piece of B
 // and the 16 R x 128-byte piece of A of a K-step with direct global->LDS loads (a row's 128 bytes by eight
 // neighbouring lanes: whole cache lines, which a fetch straight into MFMA operand registers, a row per lane,
 // does not give) into a ring of D stages of LDS that belongs to the wave alone, D - 1 K-steps in flight,

@@ -102,8 +102,10 @@ int hk_fp8_gemm_static_ws(const void* A_e4m3, const void* B_e4m3, void* C_bf16, 
  * workgroup owns 32 rows of B and all rows of A, its waves split K among themselves, stream their pieces
  * of both operands through LDS stages of their own and add their partial sums in wave order
  * (deterministic; one pass over B at HBM speed, no workspace; picked for decode shapes: up to 32 rows
- * while N / 32 is at most 1.75 x the CU count, up to 64 rows while it is at most the CU count; no
- * counterpart in the reference, whose shapes are compile-time squares). 2 and 3 are not in use
+ * while N / 32 is at most the CU count, up to 16 rows at any N when K >= 4096, up to 64 rows while N / 32
+ * is at most the CU count; 16 rows of B per workgroup while 32 would leave half of the CUs without one, B
+ * loaded with the non-temporal hint from 8 MB of B on; no counterpart in the reference, whose shapes are
+ * compile-time squares). 2 and 3 are not in use
  * (HK_ERR_UNSUPPORTED). All kernels zero-fill the last K-step of any K % 16 == 0; the tile kernels
  * (1, 4 - 7) give identical bits, the skinny kernel adds in another order. */
 int hk_fp8_gemm_variant(const void* A_e4m3, const void* B_e4m3, void* C_bf16,
@@ -127,8 +129,8 @@ int hk_mxfp4_gemm(const void* A_e2m1, const void* A_scales_e8m0, const void* B_e
  * count as hk_fp8_gemm does), 4 = 256x256x256 tile kernel with the 8-wave ping-pong schedule, 5 =
  * 192x256x256 tile producer / consumer kernel (see hk_fp8_gemm_variant, 7), 6 = the skinny kernel for M <= 64
  * (see hk_fp8_gemm_variant, 8; the scales travel like the operands, 128 bytes of a row at a time; picked by
- * hk_mxfp4_gemm, _pitched and _ws up to 32 rows while N / 32 is at most twice the CU count, up to 64 rows while
- * it is at most the CU count). 1-3 take dense scale rows of
+ * hk_mxfp4_gemm, _pitched and _ws up to 64 rows while N / 32 is at most twice the CU count, up to 32 rows at any
+ * N when K >= 8192). 1-3 take dense scale rows of
  * any K >= 512 (K % 32 == 0) and any alignment, 6 scale rows of any K, pitch and alignment; 4 and 5 need
  * K % 256 == 0 and 4-byte aligned scale pointers. */
 int hk_mxfp4_gemm_variant(const void* A_e2m1, const void* A_scales_e8m0, const void* B_e2m1,
