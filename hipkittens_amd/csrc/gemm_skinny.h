@@ -246,13 +246,15 @@ constexpr int skinny_lds_bytes(int R, int NW, int D, bool scaled = false, int NF
 // than the memory-side cache holds): up to 32 rows it wins by 2 to 64 % while it has at most one workgroup of 32
 // rows per CU (N <= 8192 on 256 CUs); beyond that, up to 16 rows, from 32 K-steps on (8 to 25 %; with a shorter K,
 // or with 17 to 32 rows and a long K, the 64x64-tile kernel's many tiles win by up to 20 %); with 33 to 64 rows it
-// wins up to one workgroup per CU, except against split-K on few workgroups with a very long K. The MXFP4 form (wgs_per_cu = 2) wins by 5 to 75 % up to
-// two workgroups per CU (N <= 16384) against the scaled tile kernels, whose scale fetches weigh more on few rows.
+// wins up to one workgroup per CU, except against split-K on few workgroups with a very long K. The MXFP4 form
+// (wgs_per_cu = 2) wins by 5 to 75 % against the scaled tile kernels, whose scale fetches weigh more on few rows:
+// from 32 K-steps on, up to 32 rows at any N and up to 64 rows up to two workgroups per CU (N <= 16384).
 static inline bool use_skinny(int M, int N, int nk, bool with_ws, int cus, int max_m = kSkinnyMaxM, int wgs_per_cu = 1) {
     if (M > max_m) return false;
     const long long wgs = (N + 31) / 32;
-    if (M <= 32) return wgs <= (long long)wgs_per_cu * cus || (nk >= 32 && (M <= 16 || wgs_per_cu > 1));
-    if (wgs > (long long)wgs_per_cu * cus) return false;
+    const bool long_k = nk >= 32;
+    if (M <= 32) return wgs <= cus || (long_k && (M <= 16 || wgs_per_cu > 1));
+    if (wgs > cus && !(long_k && wgs <= (long long)wgs_per_cu * cus)) return false;
     return !(with_ws && wgs * 2 <= cus && nk >= 96);
 }
 

@@ -34,7 +34,8 @@ NK_GRID = ((1024, 1024), (2048, 2048), (4096, 4096), (8192, 8192), (4096, 14336)
 # the grid of --emit: the report's grid and the shapes between its points
 M_GRID_EMIT = (16, 64, 128, 192, 256, 384, 512, 640, 768, 1024, 1280, 1536, 2048, 2560, 3072, 4096, 6144, 8192)
 NK_GRID_EMIT = NK_GRID + ((1536, 1536), (3072, 3072), (6144, 6144), (5760, 2880), (2880, 5760), (4096, 7168),
-                          (7168, 4096), (1024, 8192), (8192, 1024), (2560, 10240))
+                          (7168, 4096), (1024, 8192), (8192, 1024), (2560, 10240),
+                          (28672, 4096), (32768, 8192), (65536, 2880))   # (wide outputs: vocabulary projections)
 FORMATS = {"fp8": 0, "bf16": 1, "mxfp4": 2}
 TABLE_PATH = Path(__file__).resolve().parent / "csrc" / "tile_table.inc"
 EMIT_MARGIN = 1.03
