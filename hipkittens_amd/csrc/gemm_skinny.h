@@ -77,8 +77,19 @@ __device__ __forceinline__ void gemm_skinny_body(
     }
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t region = to_sgpr(lds0 + (uint32_t)w * kRegion);
+    // Without block scales a wave walks its K-steps from a start that differs from workgroup to workgroup (and
+    // wraps around): rows whose length is a multiple of the memory channels' interleave (16 KiB: K = 8192 in bf16)
+    // would otherwise have every workgroup at the same offset into its rows at the same time, i.e. in the same few
+    // channels (M = 16, N = 8192, 16 KiB rows: 4.2 TB/s against 5.7 with rows of 18 KiB). The order is fixed by
+    // the workgroup's index, so the result still does not depend on timing. (With scales the K-steps stay in
+    // order: the scale tiles are fetched one ahead of a monotonic walk.)
+    const int rot = kScaled || n == 0 ? 0 : (int)((blockIdx.x * 5u) % (uint32_t)n);
+    auto step_of = [&](int kt_local) {
+        const int x = kt_local + rot;
+        return s0 + (x >= n ? x - n : x);
+    };
     auto issue = [&](int stage, int kt_local) {
-        const int kt = s0 + kt_local;
+        const int kt = step_of(kt_local);
         const uint32_t k0 = (uint32_t)kt * BK, dst = region + (uint32_t)stage * kStage;
         const bool last = kt == nk - 1;
 #pragma unroll
@@ -147,7 +158,7 @@ __device__ __forceinline__ void gemm_skinny_body(
         // K-step kt has landed. The count leaves the loads of scale tiles out: one of those among the loads
         // behind K-step kt makes the wait stricter than needed, never weaker
         wait_stages(min(n - 1 - kt, D - 2));
-        const int ks = s0 + kt;
+        const int ks = step_of(kt);
         if constexpr (kScaled) {
             // entering a tile of scales: the next one goes out, 16 K-steps (or what is left of the first tile)
             // before its first use; its slot's last reader was the K-step before this one
