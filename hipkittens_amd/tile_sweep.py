@@ -66,9 +66,10 @@ def _time_us(fn, iters=20):
 # B is the weight matrix of a layer: in a model it comes from HBM every time, because between two uses of it the
 # other layers' weights have passed through the 256 MB memory-side cache. Timing one and the same B again and again
 # would find it in that cache whenever it fits, and would tune the choice of tile for a case that does not occur.
-# The calls therefore rotate over copies of B that together exceed twice the cache (A, the activations, stays).
-ROTATE_BYTES = 600e6
-ROTATE_MAX = 24
+# The calls therefore rotate over copies of B that together exceed the cache more than four times (A, the
+# activations, stays).
+ROTATE_BYTES = 1.2e9
+ROTATE_MAX = 32
 
 
 def _copies(b_bytes):
