@@ -42,9 +42,10 @@ def test_fp8_gemm_in_a_graph(hk, shape):
     _replay_and_compare(lambda: hk.tk_kernel.dispatch_fp8_gemm(A, B, C, 0.5, 2.0), [C])
 
 
-def test_fp8_split_k_in_a_graph(hk):
-    M, N, K = 16, 1024, 8192
-    print("graph fp8_gemm split-k", flush=True)
+@pytest.mark.parametrize("M", [16, 128])   # the skinny kernel / split-K and its reduction
+def test_fp8_split_k_in_a_graph(hk, M):
+    N, K = 1024, 8192
+    print(f"graph fp8_gemm with workspace M={M}", flush=True)
     g = torch.Generator(device=DEV).manual_seed(1)
     A = torch.randn(M, K, device=DEV, generator=g).to(torch.float8_e4m3fn)
     B = torch.randn(N, K, device=DEV, generator=g).to(torch.float8_e4m3fn)
@@ -56,9 +57,10 @@ def test_fp8_split_k_in_a_graph(hk):
                         scratch_fn=lambda: ws.fill_(0xFF))
 
 
-def test_mxfp4_split_k_in_a_graph(hk):
-    M, N, K = 16, 1024, 8192
-    print("graph mxfp4_gemm split-k", flush=True)
+@pytest.mark.parametrize("M", [16, 128])   # the skinny kernel / split-K and its reduction
+def test_mxfp4_split_k_in_a_graph(hk, M):
+    N, K = 1024, 8192
+    print(f"graph mxfp4_gemm with workspace M={M}", flush=True)
     g = torch.Generator(device=DEV).manual_seed(5)
     Ap, As = hk.quant.quantize_mxfp4(torch.randn(M, K, device=DEV, generator=g))
     Bp, Bs = hk.quant.quantize_mxfp4(torch.randn(N, K, device=DEV, generator=g))
